@@ -1,0 +1,13 @@
+"""MI355X-native HiLS-Attention operator stack (hand-written gfx950 HIP kernels behind a C ABI).
+
+The directory name carries a hyphen, so load it by path (see ``load_package`` in the
+repository's ``__graft_entry__.py``) or put this directory on ``sys.path`` and import the
+``ops`` sub-package under the reference's own module names, e.g.
+``from ops.hils_fwd_bwd_head import HiLS_block_M_head``.
+"""
+from .ops.chunk_attn_pool_tilelang import (  # noqa: F401
+    chunk_attn_pool_tilelang, chunk_attn_pool_tilelang_shared_k, chunk_mean_pool)
+from .ops.topk_head_softmax import online_softmax_topk_head  # noqa: F401
+from .ops.hils_fwd_bwd_head import HiLS_block_M_head  # noqa: F401
+from .ops.hsa_triton import HSA  # noqa: F401
+from .ops.exact_chunk_log_z_tilelang import exact_chunk_log_z_tl  # noqa: F401

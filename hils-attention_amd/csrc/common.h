@@ -1,0 +1,106 @@
+// Shared device/host helpers for the gfx950 HiLS kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <math.h>
+
+#define HILS_OK 0
+#define HILS_ERR_ARG 1
+#define HILS_ERR_LAUNCH 2
+
+// Last-error text, readable through hils_last_error().
+void hils_set_error(const char* fmt, ...);
+
+#define HILS_REQUIRE(cond, ...)            \
+  do {                                     \
+    if (!(cond)) {                         \
+      hils_set_error(__VA_ARGS__);         \
+      return HILS_ERR_ARG;                 \
+    }                                      \
+  } while (0)
+
+#define HILS_CHECK_LAUNCH(name)                                            \
+  do {                                                                     \
+    hipError_t e__ = hipGetLastError();                                    \
+    if (e__ != hipSuccess) {                                               \
+      hils_set_error("%s: launch failed: %s", name, hipGetErrorString(e__)); \
+      return HILS_ERR_LAUNCH;                                              \
+    }                                                                      \
+  } while (0)
+
+typedef unsigned short bf16_t;  // raw bfloat16 bits
+
+#define HILS_NEG_INF (-INFINITY)
+#define HILS_LOG2E 1.4426950408889634f
+#define HILS_LN2 0.6931471805599453f
+
+__device__ __forceinline__ float bf2f(bf16_t x) { return __uint_as_float(((uint32_t)x) << 16); }
+
+// round-to-nearest-even fp32 -> bf16 (NaN stays NaN)
+__device__ __forceinline__ bf16_t f2bf(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ uint32_t pack_bf2(float lo, float hi) {
+  return (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
+}
+
+// unpack 8 bf16 held in a uint4 into 8 floats
+__device__ __forceinline__ void unpack8(const uint4& v, float* f) {
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+  f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
+  f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// block-wide reductions for blockDim.x a multiple of 64, <= 1024; `red` holds >= 17 floats
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float r = 0.f;
+  for (int i = 0; i < nw; ++i) r += red[i];
+  return r;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float r = HILS_NEG_INF;
+  for (int i = 0; i < nw; ++i) r = fmaxf(r, red[i]);
+  return r;
+}
+
+// floor division for possibly negative numerators (b > 0)
+__host__ __device__ __forceinline__ int floordiv(int a, int b) {
+  int q = a / b;
+  return (a % b != 0 && ((a < 0) != (b < 0))) ? q - 1 : q;
+}
+
+// number of chunks visible to the query at global position t: chunk c is visible iff c < limit
+__host__ __device__ __forceinline__ int visible_limit(int t_global, int window, int block) {
+  return window > 0 ? floordiv(t_global - window + 1, block) : floordiv(t_global, block);
+}
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;

@@ -1,0 +1,245 @@
+// Exact per-chunk log Z: log_z[b,t,h,c] = log sum_{j in chunk c} exp(sm_scale * <q_t, k_j>)
+// over chunks that lie fully before the query's local window.
+#include "common.h"
+#include "../../include/hils_amd.h"
+
+#define LZ_THREADS 256
+
+struct LzDims {
+  int L, HQ, H, G, D, S, W, N, mask_lmk;
+  float sm_scale;
+};
+
+// number of fully-remote chunks of query t: chunk c counts iff t >= (c+1)*S + W - 1
+__device__ __forceinline__ int lz_limit(const LzDims& dm, int t) {
+  int lm = floordiv(t - dm.W + 1, dm.S);
+  return lm < 0 ? 0 : (lm > dm.N ? dm.N : lm);
+}
+
+// One block per (b, t, hq); wavefront w takes chunks w, w+4, ...; lanes take tokens.
+__global__ void __launch_bounds__(LZ_THREADS)
+logz_fwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                float* __restrict__ log_z, LzDims dm) {
+  extern __shared__ float smem[];
+  float* q_s = smem;  // D
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const long row = blockIdx.x;  // (b*L + t)*HQ + hq
+  const int hq = (int)(row % dm.HQ);
+  const long bt = row / dm.HQ;
+  const int t = (int)(bt % dm.L);
+  const long b = bt / dm.L;
+  const int hk = hq / dm.G;
+  for (int d = tid; d < dm.D; d += LZ_THREADS) q_s[d] = bf2f(q[row * dm.D + d]);
+  __syncthreads();
+  const int lim = lz_limit(dm, t);
+  float* out = log_z + row * (long)dm.N;
+  for (int c = wave; c < dm.N; c += LZ_THREADS / 64) {
+    if (c >= lim) {
+      if (lane == 0) out[c] = HILS_NEG_INF;
+      continue;
+    }
+    float m = HILS_NEG_INF, l = 0.f;
+    for (int s = lane; s < dm.S; s += 64) {
+      const int j = c * dm.S + s;
+      if (j > t || j >= dm.L) continue;
+      if (dm.mask_lmk && ((j + 1) % dm.S) == 0) continue;
+      const bf16_t* kr = k + ((b * dm.L + j) * (long)dm.H + hk) * dm.D;
+      float a = 0.f;
+      for (int d8 = 0; d8 < dm.D / 8; ++d8) {
+        float f[8];
+        unpack8(*(const uint4*)(kr + d8 * 8), f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a = fmaf(q_s[d8 * 8 + i], f[i], a);
+      }
+      a *= dm.sm_scale;
+      const float mn = fmaxf(m, a);
+      l = l * __expf(m - mn) + __expf(a - mn);
+      m = mn;
+    }
+    const float mx = wave_max(m);
+    float part = (m > HILS_NEG_INF) ? l * __expf(m - mx) : 0.f;
+    part = wave_sum(part);
+    if (lane == 0) out[c] = (part > 0.f) ? mx + logf(part) : HILS_NEG_INF;
+  }
+}
+
+// dq[b,t,hq,:] = sum_c sum_j dlz[c] * exp(s_j - lz[c]) * scale * k_j
+__global__ void __launch_bounds__(LZ_THREADS)
+logz_bwd_dq_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                   const float* __restrict__ log_z, const float* __restrict__ d_log_z,
+                   bf16_t* __restrict__ dq, LzDims dm) {
+  extern __shared__ float smem[];
+  float* q_s = smem;          // D
+  float* ds = q_s + dm.D;     // S
+  const int tid = threadIdx.x;
+  const long row = blockIdx.x;
+  const int hq = (int)(row % dm.HQ);
+  const long bt = row / dm.HQ;
+  const int t = (int)(bt % dm.L);
+  const long b = bt / dm.L;
+  const int hk = hq / dm.G;
+  for (int d = tid; d < dm.D; d += LZ_THREADS) q_s[d] = bf2f(q[row * dm.D + d]);
+  const int lim = lz_limit(dm, t);
+  float acc = 0.f;  // thread d (< D) owns one output column
+  for (int c = 0; c < lim; ++c) {
+    const float lz = log_z[row * (long)dm.N + c];
+    const float dlz = d_log_z[row * (long)dm.N + c];
+    __syncthreads();
+    for (int s = tid; s < dm.S; s += LZ_THREADS) {
+      const int j = c * dm.S + s;
+      float val = 0.f;
+      if (j <= t && j < dm.L && lz > -1e30f) {
+        const bf16_t* kr = k + ((b * dm.L + j) * (long)dm.H + hk) * dm.D;
+        float a = 0.f;
+        for (int d8 = 0; d8 < dm.D / 8; ++d8) {
+          float f[8];
+          unpack8(*(const uint4*)(kr + d8 * 8), f);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) a = fmaf(q_s[d8 * 8 + i], f[i], a);
+        }
+        val = dlz * __expf(a * dm.sm_scale - lz) * dm.sm_scale;
+      }
+      ds[s] = val;
+    }
+    __syncthreads();
+    for (int d = tid; d < dm.D; d += LZ_THREADS) {
+      float a = 0.f;
+      for (int s = 0; s < dm.S; ++s) {
+        const int j = c * dm.S + s;
+        if (j < dm.L) a = fmaf(ds[s], bf2f(k[((b * dm.L + j) * (long)dm.H + hk) * dm.D + d]), a);
+      }
+      acc += a;  // D <= LZ_THREADS: one column per thread
+    }
+  }
+  if (tid < dm.D) dq[row * dm.D + tid] = f2bf(acc);
+}
+
+// dk[b, c*S+s, hk, :] = sum_{g} sum_{t} dlz[t,hq,c] * exp(s - lz) * scale * q[t,hq,:]
+// One block per (b, c, hk); queries are streamed in tiles of LZ_TT.
+#define LZ_TT 8
+#define LZ_MAX_ACC 32
+__global__ void __launch_bounds__(LZ_THREADS)
+logz_bwd_dk_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                   const float* __restrict__ log_z, const float* __restrict__ d_log_z,
+                   bf16_t* __restrict__ dk, LzDims dm) {
+  extern __shared__ float smem[];
+  const int G = dm.G, S = dm.S, D = dm.D, DP = dm.D + 1;
+  float* k_s = smem;                          // S*DP
+  float* q_s = k_s + (size_t)S * DP;          // TT*G*D
+  float* ds = q_s + (size_t)LZ_TT * G * D;    // TT*G*S
+  const int tid = threadIdx.x;
+  const int c = blockIdx.x, hk = blockIdx.y;
+  const long b = blockIdx.z;
+  for (int i = tid; i < S * D; i += LZ_THREADS) {
+    const int s = i / D, d = i - s * D;
+    const int j = c * S + s;
+    k_s[s * DP + d] = (j < dm.L) ? bf2f(k[((b * dm.L + j) * (long)dm.H + hk) * D + d]) : 0.f;
+  }
+  float acc[LZ_MAX_ACC];
+#pragma unroll
+  for (int i = 0; i < LZ_MAX_ACC; ++i) acc[i] = 0.f;
+  int t_first = (c + 1) * S + dm.W - 1;
+  if (t_first < 0) t_first = 0;
+  for (int t0 = t_first; t0 < dm.L; t0 += LZ_TT) {
+    __syncthreads();
+    for (int i = tid; i < LZ_TT * G * D; i += LZ_THREADS) {
+      const int tt = i / (G * D), r = i - tt * (G * D);
+      const int t = t0 + tt;
+      q_s[i] = (t < dm.L) ? bf2f(q[((b * dm.L + t) * (long)dm.HQ + hk * G) * D + r]) : 0.f;
+    }
+    __syncthreads();
+    for (int i = tid; i < LZ_TT * G * S; i += LZ_THREADS) {
+      const int tt = i / (G * S), r = i - tt * (G * S);
+      const int g = r / S, s = r - g * S;
+      const int t = t0 + tt, j = c * S + s;
+      float val = 0.f;
+      if (t < dm.L && j <= t && j < dm.L) {
+        const long zrow = ((b * dm.L + t) * (long)dm.HQ + hk * G + g) * dm.N + c;
+        const float lz = log_z[zrow];
+        if (lz > -1e30f) {
+          const float* qr = q_s + (tt * G + g) * D;
+          float a = 0.f;
+          for (int d = 0; d < D; ++d) a = fmaf(qr[d], k_s[s * DP + d], a);
+          val = d_log_z[zrow] * __expf(a * dm.sm_scale - lz) * dm.sm_scale;
+        }
+      }
+      ds[i] = val;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < LZ_MAX_ACC; ++e) {
+      const int oi = tid + e * LZ_THREADS;
+      if (oi < S * D) {
+        const int s = oi / D, d = oi - s * D;
+        float a = acc[e];
+        for (int r = 0; r < LZ_TT * G; ++r) a = fmaf(ds[r * S + s], q_s[r * D + d], a);
+        acc[e] = a;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < LZ_MAX_ACC; ++e) {
+    const int oi = tid + e * LZ_THREADS;
+    if (oi < S * D) {
+      const int s = oi / D, d = oi - s * D;
+      const int j = c * S + s;
+      if (j < dm.L) dk[((b * dm.L + j) * (long)dm.H + hk) * D + d] = f2bf(acc[e]);
+    }
+  }
+}
+
+static int lz_check(const char* name, int B, int L, int HQ, int H, int D, int S) {
+  HILS_REQUIRE(B > 0 && L > 0 && HQ > 0 && H > 0 && D > 0 && S > 0, "%s: sizes must be positive", name);
+  HILS_REQUIRE(HQ % H == 0, "%s: HQ (%d) must be a multiple of H (%d)", name, HQ, H);
+  HILS_REQUIRE(D % 8 == 0, "%s: D (%d) must be a multiple of 8", name, D);
+  HILS_REQUIRE((long)B * L * HQ <= 2147483647L, "%s: grid too large", name);
+  return HILS_OK;
+}
+
+extern "C" int hils_chunk_logz_fwd(const void* q, const void* k, float* log_z, int B, int L, int HQ,
+                                   int H, int D, int S, int window, float sm_scale, int mask_lmk,
+                                   void* stream) {
+  HILS_REQUIRE(q && k && log_z, "hils_chunk_logz_fwd: null pointer");
+  if (int rc = lz_check("hils_chunk_logz_fwd", B, L, HQ, H, D, S)) return rc;
+  LzDims dm{L, HQ, H, HQ / H, D, S, window, (L + S - 1) / S, mask_lmk, sm_scale};
+  hipLaunchKernelGGL(logz_fwd_simple, dim3((unsigned)((long)B * L * HQ)), dim3(LZ_THREADS),
+                     D * sizeof(float), (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k,
+                     log_z, dm);
+  HILS_CHECK_LAUNCH("hils_chunk_logz_fwd");
+  return HILS_OK;
+}
+
+extern "C" int hils_chunk_logz_bwd_dq(const void* q, const void* k, const float* log_z,
+                                      const float* d_log_z, void* dq, int B, int L, int HQ, int H,
+                                      int D, int S, int window, float sm_scale, void* stream) {
+  HILS_REQUIRE(q && k && log_z && d_log_z && dq, "hils_chunk_logz_bwd_dq: null pointer");
+  if (int rc = lz_check("hils_chunk_logz_bwd_dq", B, L, HQ, H, D, S)) return rc;
+  HILS_REQUIRE(D <= LZ_THREADS, "hils_chunk_logz_bwd_dq: D (%d) must be <= %d", D, LZ_THREADS);
+  LzDims dm{L, HQ, H, HQ / H, D, S, window, (L + S - 1) / S, 0, sm_scale};
+  hipLaunchKernelGGL(logz_bwd_dq_simple, dim3((unsigned)((long)B * L * HQ)), dim3(LZ_THREADS),
+                     (D + S) * sizeof(float), (hipStream_t)stream, (const bf16_t*)q,
+                     (const bf16_t*)k, log_z, d_log_z, (bf16_t*)dq, dm);
+  HILS_CHECK_LAUNCH("hils_chunk_logz_bwd_dq");
+  return HILS_OK;
+}
+
+extern "C" int hils_chunk_logz_bwd_dk(const void* q, const void* k, const float* log_z,
+                                      const float* d_log_z, void* dk, int B, int L, int HQ, int H,
+                                      int D, int S, int window, float sm_scale, void* stream) {
+  HILS_REQUIRE(q && k && log_z && d_log_z && dk, "hils_chunk_logz_bwd_dk: null pointer");
+  if (int rc = lz_check("hils_chunk_logz_bwd_dk", B, L, HQ, H, D, S)) return rc;
+  const int G = HQ / H;
+  HILS_REQUIRE(S * D <= LZ_MAX_ACC * LZ_THREADS, "hils_chunk_logz_bwd_dk: S*D (%d) too large", S * D);
+  LzDims dm{L, HQ, H, G, D, S, window, (L + S - 1) / S, 0, sm_scale};
+  size_t smem = ((size_t)S * (D + 1) + (size_t)LZ_TT * G * D + (size_t)LZ_TT * G * S) * sizeof(float);
+  HILS_REQUIRE(smem <= 160 * 1024, "hils_chunk_logz_bwd_dk: tile does not fit in LDS");
+  HILS_REQUIRE(H <= 65535 && B <= 65535, "hils_chunk_logz_bwd_dk: H/B too large for the grid");
+  if (smem > 64 * 1024)
+    (void)hipFuncSetAttribute((const void*)logz_bwd_dk_simple,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  hipLaunchKernelGGL(logz_bwd_dk_simple, dim3(dm.N, H, B), dim3(LZ_THREADS), smem,
+                     (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k, log_z, d_log_z,
+                     (bf16_t*)dk, dm);
+  HILS_CHECK_LAUNCH("hils_chunk_logz_bwd_dk");
+  return HILS_OK;
+}

@@ -1,0 +1,309 @@
+// Chunk-key pooling kernels (HBM-bandwidth-bound reductions over 64-token chunks).
+#include "common.h"
+#include "../../include/hils_amd.h"
+
+// ---------------------------------------------------------------------------
+// mean pool
+// ---------------------------------------------------------------------------
+// One block per (chunk = blockIdx.x, column group = blockIdx.y).  blockDim = (CG, TS): CG lanes
+// cover contiguous 16-byte column groups of the flattened (H*D) row, TS token slices
+// each own S/TS tokens; the slices are summed through LDS in a fixed order.
+template <int TS>
+__global__ void mean_pool_fwd_kernel(const uint4* __restrict__ k, uint4* __restrict__ out,
+                                     int S, int cols8, float inv_s) {
+  extern __shared__ float smem[];  // TS * CG * 8 floats
+  const int cg = blockIdx.y * blockDim.x + threadIdx.x;
+  const int ts = threadIdx.y;
+  const long chunk = blockIdx.x;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (cg < cols8) {
+    const uint4* base = k + (chunk * S) * (long)cols8 + cg;
+    for (int s = ts; s < S; s += TS) {
+      uint4 v = base[(long)s * cols8];
+      float f[8];
+      unpack8(v, f);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += f[i];
+    }
+  }
+  float* mine = smem + ((size_t)ts * blockDim.x + threadIdx.x) * 8;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) mine[i] = acc[i];
+  __syncthreads();
+  if (ts == 0 && cg < cols8) {
+    float r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = 0.f;
+    for (int t = 0; t < TS; ++t) {
+      const float* o = smem + ((size_t)t * blockDim.x + threadIdx.x) * 8;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) r[i] += o[i];
+    }
+    uint4 w;
+    w.x = pack_bf2(r[0] * inv_s, r[1] * inv_s);
+    w.y = pack_bf2(r[2] * inv_s, r[3] * inv_s);
+    w.z = pack_bf2(r[4] * inv_s, r[5] * inv_s);
+    w.w = pack_bf2(r[6] * inv_s, r[7] * inv_s);
+    out[chunk * cols8 + cg] = w;
+  }
+}
+
+__global__ void mean_pool_bwd_kernel(const uint4* __restrict__ g, uint4* __restrict__ dk,
+                                     int S, int cols8, float inv_s, long total8) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total8) return;
+  const long row = i / cols8;  // token row over (B*L)
+  const int cg = (int)(i - row * cols8);
+  const long chunk = row / S;
+  uint4 v = g[chunk * cols8 + cg];
+  float f[8];
+  unpack8(v, f);
+  uint4 w;
+  w.x = pack_bf2(f[0] * inv_s, f[1] * inv_s);
+  w.y = pack_bf2(f[2] * inv_s, f[3] * inv_s);
+  w.z = pack_bf2(f[4] * inv_s, f[5] * inv_s);
+  w.w = pack_bf2(f[6] * inv_s, f[7] * inv_s);
+  dk[i] = w;
+}
+
+extern "C" int hils_mean_pool_fwd(const void* k, void* lmk_k, int B, int L, int H, int D, int S,
+                                  void* stream) {
+  HILS_REQUIRE(k && lmk_k, "hils_mean_pool_fwd: null pointer");
+  HILS_REQUIRE(B > 0 && L > 0 && H > 0 && D > 0 && S > 0, "hils_mean_pool_fwd: sizes must be positive");
+  HILS_REQUIRE(L % S == 0, "hils_mean_pool_fwd: L (%d) must be a multiple of S (%d)", L, S);
+  HILS_REQUIRE((H * D) % 8 == 0, "hils_mean_pool_fwd: H*D (%d) must be a multiple of 8", H * D);
+  const int cols8 = H * D / 8;
+  const long chunks = (long)B * (L / S);
+  constexpr int TS = 8;
+  const int CG = cols8 >= 32 ? 32 : cols8;
+  dim3 block(CG, TS);
+  HILS_REQUIRE(chunks <= 2147483647L && (cols8 + CG - 1) / CG <= 65535, "hils_mean_pool_fwd: grid too large");
+  dim3 grid((unsigned)chunks, (cols8 + CG - 1) / CG);
+  size_t smem = (size_t)TS * CG * 8 * sizeof(float);
+  hipLaunchKernelGGL(mean_pool_fwd_kernel<TS>, grid, block, smem, (hipStream_t)stream,
+                     (const uint4*)k, (uint4*)lmk_k, S, cols8, 1.0f / (float)S);
+  HILS_CHECK_LAUNCH("hils_mean_pool_fwd");
+  return HILS_OK;
+}
+
+extern "C" int hils_mean_pool_bwd(const void* g_lmk, void* dk, int B, int L, int H, int D, int S,
+                                  void* stream) {
+  HILS_REQUIRE(g_lmk && dk, "hils_mean_pool_bwd: null pointer");
+  HILS_REQUIRE(B > 0 && L > 0 && H > 0 && D > 0 && S > 0, "hils_mean_pool_bwd: sizes must be positive");
+  HILS_REQUIRE(L % S == 0, "hils_mean_pool_bwd: L (%d) must be a multiple of S (%d)", L, S);
+  HILS_REQUIRE((H * D) % 8 == 0, "hils_mean_pool_bwd: H*D (%d) must be a multiple of 8", H * D);
+  const int cols8 = H * D / 8;
+  const long total8 = (long)B * L * cols8;
+  const long nblk = (total8 + 255) / 256;
+  HILS_REQUIRE(nblk <= 2147483647L, "hils_mean_pool_bwd: grid too large");
+  hipLaunchKernelGGL(mean_pool_bwd_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                     (const uint4*)g_lmk, (uint4*)dk, S, cols8, 1.0f / (float)S, total8);
+  HILS_CHECK_LAUNCH("hils_mean_pool_bwd");
+  return HILS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// attention pool: one prior query per (chunk, head) over the chunk's first S-1 keys
+// ---------------------------------------------------------------------------
+// One block of 256 threads per (chunk bn, head h).  The K tile (S x D, bf16) is staged
+// in LDS as fp32 with a padded row so that both the row-wise dot products and the
+// column-wise weighted sums are bank-conflict free.
+#define POOL_THREADS 256
+
+__global__ void __launch_bounds__(POOL_THREADS)
+attn_pool_fwd_kernel(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k,
+                     bf16_t* __restrict__ lmk_k, float* __restrict__ lmk_b, float* __restrict__ p_out,
+                     int S, int H, int D, float sm_scale, int compact, int shared_k) {
+  extern __shared__ float smem[];
+  const int DP = D + 1;
+  float* ks = smem;              // S * DP
+  float* mu = ks + (size_t)S * DP;  // D
+  float* pr = mu + D;            // S
+  float* red = pr + S;           // 32
+  const long bn = blockIdx.x;
+  const int h = blockIdx.y;
+  const int kh = shared_k ? 0 : h;
+  const int tid = threadIdx.x;
+
+  const int d8 = D / 8;
+  for (int i = tid; i < S * d8; i += POOL_THREADS) {
+    const int s = i / d8, c = i - s * d8;
+    uint4 v = *(const uint4*)(k + ((bn * S + s) * (long)H + kh) * D + c * 8);
+    float f[8];
+    unpack8(v, f);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ks[s * DP + c * 8 + j] = f[j];
+  }
+  for (int d = tid; d < D; d += POOL_THREADS) mu[d] = bf2f(mu_q[(bn * H + h) * (long)D + d]);
+  __syncthreads();
+
+  // logits, one thread per token
+  for (int s = tid; s < S; s += POOL_THREADS) {
+    float a = 0.f;
+    for (int d = 0; d < D; ++d) a += mu[d] * ks[s * DP + d];
+    a *= sm_scale;
+    if (s == S - 1) a = HILS_NEG_INF;
+    pr[s] = a;
+  }
+  __syncthreads();
+  float m = HILS_NEG_INF;
+  for (int s = tid; s < S; s += POOL_THREADS) m = fmaxf(m, pr[s]);
+  m = block_max(m, red);
+  float e_sum = 0.f;
+  for (int s = tid; s < S; s += POOL_THREADS) {
+    float e = (pr[s] == HILS_NEG_INF) ? 0.f : expf(pr[s] - m);
+    pr[s] = e;
+    e_sum += e;
+  }
+  e_sum = block_sum(e_sum, red);
+  const float inv = e_sum > 0.f ? 1.f / e_sum : 0.f;
+  float ent = 0.f;
+  for (int s = tid; s < S; s += POOL_THREADS) {
+    const float pv = pr[s] * inv;
+    pr[s] = pv;
+    p_out[(bn * S + s) * (long)H + h] = pv;
+    if (pv > 0.f) ent += pv * logf(pv);
+  }
+  ent = block_sum(ent, red);  // also orders the pr[] writes before the reads below
+  if (tid == 0) lmk_b[bn * H + h] = -ent;
+  for (int d = tid; d < D; d += POOL_THREADS) {
+    float a = 0.f;
+    if (!compact)
+      for (int s = 0; s < S; ++s) a += pr[s] * ks[s * DP + d];
+    lmk_k[(bn * H + h) * (long)D + d] = f2bf(a);
+  }
+}
+
+// Backward.  Block per (bn, h) (or per bn looping over heads when K is shared, so that
+// the per-head dK can be summed into head 0 without atomics).
+__global__ void __launch_bounds__(POOL_THREADS)
+attn_pool_bwd_kernel(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k,
+                     const float* __restrict__ p_saved, const float* __restrict__ lmk_b,
+                     const bf16_t* __restrict__ g_k, const float* __restrict__ g_b,
+                     bf16_t* __restrict__ d_mu, bf16_t* __restrict__ d_k,
+                     int S, int H, int D, float sm_scale, int compact, int shared_k) {
+  extern __shared__ float smem[];
+  const int DP = D + 1;
+  float* ks = smem;                 // S * DP
+  float* mu = ks + (size_t)S * DP;  // D
+  float* gk = mu + D;               // D
+  float* pr = gk + D;               // S
+  float* dl = pr + S;               // S  (dP, then dlogits)
+  float* red = dl + S;              // 32
+  float* dk_acc = red + 32;         // S * D, only when shared_k
+  const long bn = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int d8 = D / 8;
+  const int h_begin = shared_k ? 0 : blockIdx.y;
+  const int h_end = shared_k ? H : blockIdx.y + 1;
+
+  if (shared_k)
+    for (int i = tid; i < S * D; i += POOL_THREADS) dk_acc[i] = 0.f;
+
+  for (int h = h_begin; h < h_end; ++h) {
+    const int kh = shared_k ? 0 : h;
+    __syncthreads();
+    if (!shared_k || h == 0) {
+      for (int i = tid; i < S * d8; i += POOL_THREADS) {
+        const int s = i / d8, c = i - s * d8;
+        uint4 v = *(const uint4*)(k + ((bn * S + s) * (long)H + kh) * D + c * 8);
+        float f[8];
+        unpack8(v, f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ks[s * DP + c * 8 + j] = f[j];
+      }
+    }
+    for (int d = tid; d < D; d += POOL_THREADS) {
+      mu[d] = bf2f(mu_q[(bn * H + h) * (long)D + d]);
+      gk[d] = compact ? 0.f : bf2f(g_k[(bn * H + h) * (long)D + d]);
+    }
+    for (int s = tid; s < S; s += POOL_THREADS) pr[s] = p_saved[(bn * S + s) * (long)H + h];
+    __syncthreads();
+    float part = 0.f;
+    for (int s = tid; s < S; s += POOL_THREADS) {
+      float a = 0.f;
+      for (int d = 0; d < D; ++d) a += gk[d] * ks[s * DP + d];
+      dl[s] = a;
+      part += pr[s] * a;
+    }
+    const float delta = block_sum(part, red);
+    const float ent = lmk_b[bn * H + h];
+    const float gb = g_b[bn * H + h];
+    for (int s = tid; s < S; s += POOL_THREADS) {
+      const float pv = pr[s];
+      dl[s] = pv > 0.f ? pv * ((dl[s] - delta) - gb * (logf(pv) + ent)) : 0.f;
+    }
+    __syncthreads();
+    for (int d = tid; d < D; d += POOL_THREADS) {
+      float a = 0.f;
+      for (int s = 0; s < S; ++s) a += dl[s] * ks[s * DP + d];
+      d_mu[(bn * H + h) * (long)D + d] = f2bf(a * sm_scale);
+    }
+    if (shared_k) {
+      for (int i = tid; i < S * D; i += POOL_THREADS) {
+        const int s = i / D, d = i - s * D;
+        dk_acc[i] += sm_scale * dl[s] * mu[d] + pr[s] * gk[d];
+      }
+    } else {
+      for (int i = tid; i < S * D; i += POOL_THREADS) {
+        const int s = i / D, d = i - s * D;
+        d_k[((bn * S + s) * (long)H + h) * D + d] = f2bf(sm_scale * dl[s] * mu[d] + pr[s] * gk[d]);
+      }
+    }
+  }
+  if (shared_k) {
+    __syncthreads();
+    for (int i = tid; i < S * D; i += POOL_THREADS) {
+      const int s = i / D, d = i - s * D;
+      d_k[((bn * S + s) * (long)H + 0) * D + d] = f2bf(dk_acc[i]);
+    }
+    for (long i = tid; i < (long)S * (H - 1) * D; i += POOL_THREADS) {
+      const int s = (int)(i / ((long)(H - 1) * D));
+      const long r = i - (long)s * (H - 1) * D;
+      d_k[((bn * S + s) * (long)H + 1) * D + r] = 0;
+    }
+  }
+}
+
+static int pool_check(const char* name, int BN, int S, int H, int D) {
+  HILS_REQUIRE(BN > 0 && S > 1 && H > 0 && D > 0, "%s: sizes must be positive (S > 1)", name);
+  HILS_REQUIRE(D % 8 == 0, "%s: D (%d) must be a multiple of 8", name, D);
+  HILS_REQUIRE(H <= 65535, "%s: H (%d) too large", name, H);
+  return HILS_OK;
+}
+
+extern "C" int hils_attn_pool_fwd(const void* mu_q, const void* k, void* lmk_k, float* lmk_b,
+                                  float* p, int BN, int S, int H, int D, float sm_scale,
+                                  int compact, int shared_k, void* stream) {
+  HILS_REQUIRE(mu_q && k && lmk_k && lmk_b && p, "hils_attn_pool_fwd: null pointer");
+  if (int rc = pool_check("hils_attn_pool_fwd", BN, S, H, D)) return rc;
+  size_t smem = ((size_t)S * (D + 1) + D + S + 32) * sizeof(float);
+  HILS_REQUIRE(smem <= 160 * 1024, "hils_attn_pool_fwd: S*D (%d x %d) tile does not fit in LDS", S, D);
+  if (smem > 64 * 1024)
+    (void)hipFuncSetAttribute((const void*)attn_pool_fwd_kernel,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  hipLaunchKernelGGL(attn_pool_fwd_kernel, dim3(BN, H), dim3(POOL_THREADS), smem,
+                     (hipStream_t)stream, (const bf16_t*)mu_q, (const bf16_t*)k, (bf16_t*)lmk_k,
+                     lmk_b, p, S, H, D, sm_scale, compact, shared_k);
+  HILS_CHECK_LAUNCH("hils_attn_pool_fwd");
+  return HILS_OK;
+}
+
+extern "C" int hils_attn_pool_bwd(const void* mu_q, const void* k, const float* p,
+                                  const float* lmk_b, const void* g_k, const float* g_b,
+                                  void* d_mu, void* d_k, int BN, int S, int H, int D,
+                                  float sm_scale, int compact, int shared_k, void* stream) {
+  HILS_REQUIRE(mu_q && k && p && lmk_b && g_k && g_b && d_mu && d_k, "hils_attn_pool_bwd: null pointer");
+  if (int rc = pool_check("hils_attn_pool_bwd", BN, S, H, D)) return rc;
+  size_t smem = ((size_t)S * (D + 1) + 2 * D + 2 * S + 32 + (shared_k ? (size_t)S * D : 0)) * sizeof(float);
+  HILS_REQUIRE(smem <= 160 * 1024, "hils_attn_pool_bwd: S*D (%d x %d) tile does not fit in LDS", S, D);
+  if (smem > 64 * 1024)
+    (void)hipFuncSetAttribute((const void*)attn_pool_bwd_kernel,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  dim3 grid(BN, shared_k ? 1 : H);
+  hipLaunchKernelGGL(attn_pool_bwd_kernel, grid, dim3(POOL_THREADS), smem, (hipStream_t)stream,
+                     (const bf16_t*)mu_q, (const bf16_t*)k, p, lmk_b, (const bf16_t*)g_k, g_b,
+                     (bf16_t*)d_mu, (bf16_t*)d_k, S, H, D, sm_scale, compact, shared_k);
+  HILS_CHECK_LAUNCH("hils_attn_pool_bwd");
+  return HILS_OK;
+}

@@ -1,0 +1,299 @@
+// Sparse attention over selected chunks: shape-generic kernels (any D, Dv, G, chunk size).
+//
+// One workgroup owns one (batch, query, KV head): its G query heads share the K/V
+// chunks of the K selected slots.  These kernels do their arithmetic on the vector
+// ALU in fp32; they are the path for shapes the MFMA kernels do not cover and for
+// decode-sized query counts, and they also implement the q-block-shared index /
+// `sm_n` denominator variant of the older HSA operator.
+#include "common.h"
+#include "../../include/hils_amd.h"
+
+#define SA_THREADS 256
+#define SA_MAX_OUT 16  // outputs (g, dv) per thread
+
+struct SaDims {
+  int L, Lkv, HQ, H, G, D, Dv, K, NW, WH, q_block, S, mask_last;
+  float sm_scale, sm_n;
+};
+
+// scores of slot chunk c for all (g, s): sc[g*S+s] = (q_g . K_s - slope_g*dist_s) * sm_scale,
+// -inf for the masked last token.  q_s holds the G query rows in fp32.
+__device__ __forceinline__ void sa_scores(const SaDims& dm, const float* q_s, const bf16_t* kbase,
+                                          const float* slope_s, float* sc) {
+  const int GS = dm.G * dm.S;
+  for (int p = threadIdx.x; p < GS; p += SA_THREADS) {
+    const int g = p / dm.S, s = p - g * dm.S;
+    const bf16_t* kr = kbase + (long)s * dm.H * dm.D;
+    const float* qr = q_s + g * dm.D;
+    float a = 0.f;
+    for (int d8 = 0; d8 < dm.D / 8; ++d8) {
+      float f[8];
+      unpack8(*(const uint4*)(kr + d8 * 8), f);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) a = fmaf(qr[d8 * 8 + j], f[j], a);
+    }
+    if (slope_s) {
+      const int dist = dm.S - 2 - s;
+      a -= slope_s[g] * (float)(dist > 0 ? dist : 0);
+    }
+    a *= dm.sm_scale;
+    if (dm.mask_last && s == dm.S - 1) a = HILS_NEG_INF;
+    sc[p] = a;
+  }
+}
+
+__global__ void __launch_bounds__(SA_THREADS)
+sparse_attn_fwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                       const bf16_t* __restrict__ v, const bf16_t* __restrict__ weights,
+                       const int32_t* __restrict__ indices, const float* __restrict__ slope,
+                       bf16_t* __restrict__ o, float* __restrict__ lse, SaDims dm) {
+  extern __shared__ float smem[];
+  float* q_s = smem;                       // G*D
+  float* sc = q_s + dm.G * dm.D;           // G*S
+  float* w_s = sc + dm.G * dm.S;           // G
+  float* slope_s = w_s + dm.G;             // G
+  const int G = dm.G, S = dm.S, D = dm.D, Dv = dm.Dv;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const long row = blockIdx.x;  // (b*L + t)*H + hk
+  const int hk = (int)(row % dm.H);
+  const long bt = row / dm.H;
+  const int t = (int)(bt % dm.L);
+  const long b = bt / dm.L;
+  const long LB = dm.L / dm.q_block;
+  const long irow = (b * LB + t / dm.q_block) * dm.H + hk;
+  const int nchunk = dm.Lkv / S;
+
+  for (int i = tid; i < G * D; i += SA_THREADS)
+    q_s[i] = bf2f(q[(bt * dm.HQ + hk * G) * (long)D + i]);
+  if (tid < G) slope_s[tid] = slope ? slope[hk * G + tid] : 0.f;
+
+  float acc[SA_MAX_OUT];
+#pragma unroll
+  for (int j = 0; j < SA_MAX_OUT; ++j) acc[j] = 0.f;
+  const int nout = G * Dv;
+
+  for (int kk = 0; kk < dm.K; ++kk) {
+    const int c = indices[irow * dm.K + kk];
+    __syncthreads();
+    if (c < 0 || c >= nchunk) {
+      if (lse && c < 0)
+        for (int g = tid; g < G; g += SA_THREADS) lse[(bt * dm.HQ + hk * G + g) * (long)dm.K + kk] = HILS_NEG_INF;
+      continue;
+    }
+    if (tid < G) {
+      const long wrow = (b * LB + t / dm.q_block) * dm.WH + (dm.WH == dm.HQ ? hk * G + tid : hk);
+      w_s[tid] = bf2f(weights[wrow * dm.NW + kk]);
+    }
+    const bf16_t* kbase = k + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * D;
+    const bf16_t* vbase = v + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * Dv;
+    sa_scores(dm, q_s, kbase, slope ? slope_s : nullptr, sc);
+    __syncthreads();
+    for (int g = wave; g < G; g += SA_THREADS / 64) {
+      float m = HILS_NEG_INF;
+      for (int s = lane; s < S; s += 64) m = fmaxf(m, sc[g * S + s]);
+      m = wave_max(m);
+      float sum = 0.f;
+      for (int s = lane; s < S; s += 64) {
+        const float x = sc[g * S + s];
+        const float e = (x == HILS_NEG_INF) ? 0.f : __expf(x - m);
+        sc[g * S + s] = e;
+        sum += e;
+      }
+      sum = wave_sum(sum);
+      const float den = (m > HILS_NEG_INF) ? sum + dm.sm_n * __expf(-m) : 0.f;
+      const float f = den > 0.f ? w_s[g] / den : 0.f;
+      for (int s = lane; s < S; s += 64) sc[g * S + s] *= f;
+      if (lse && lane == 0)
+        lse[(bt * dm.HQ + hk * G + g) * (long)dm.K + kk] =
+            den > 0.f ? m * HILS_LOG2E + log2f(den) : HILS_NEG_INF;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < SA_MAX_OUT; ++j) {
+      const int oi = tid + j * SA_THREADS;
+      if (oi < nout) {
+        const int g = oi / Dv, dv = oi - g * Dv;
+        float a = acc[j];
+        for (int s = 0; s < S; ++s) a = fmaf(sc[g * S + s], bf2f(vbase[(long)s * dm.H * Dv + dv]), a);
+        acc[j] = a;
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < SA_MAX_OUT; ++j) {
+    const int oi = tid + j * SA_THREADS;
+    if (oi < nout) o[(bt * dm.HQ + hk * G) * (long)Dv + oi] = f2bf(acc[j]);
+  }
+}
+
+__global__ void __launch_bounds__(SA_THREADS)
+sparse_attn_bwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                       const bf16_t* __restrict__ v, const bf16_t* __restrict__ weights,
+                       const int32_t* __restrict__ indices, const float* __restrict__ slope,
+                       const float* __restrict__ lse, const bf16_t* __restrict__ d_o,
+                       bf16_t* __restrict__ dq, float* __restrict__ dk, float* __restrict__ dv,
+                       float* __restrict__ dw, SaDims dm) {
+  extern __shared__ float smem[];
+  const int G = dm.G, S = dm.S, D = dm.D, Dv = dm.Dv;
+  float* q_s = smem;               // G*D
+  float* do_s = q_s + G * D;       // G*Dv
+  float* p_s = do_s + G * Dv;      // G*S  probabilities
+  float* ds_s = p_s + G * S;       // G*S  dPV, then dS
+  float* w_s = ds_s + G * S;       // G
+  float* slope_s = w_s + G;        // G
+  float* dwk = slope_s + G;        // G
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const long row = blockIdx.x;
+  const int hk = (int)(row % dm.H);
+  const long bt = row / dm.H;
+  const int t = (int)(bt % dm.L);
+  const long b = bt / dm.L;
+  const long LB = dm.L / dm.q_block;
+  const long irow = (b * LB + t / dm.q_block) * dm.H + hk;
+  const int nchunk = dm.Lkv / S;
+  const bool dw_atomic = dm.q_block > 1 || dm.WH != dm.HQ;
+
+  for (int i = tid; i < G * D; i += SA_THREADS) q_s[i] = bf2f(q[(bt * dm.HQ + hk * G) * (long)D + i]);
+  for (int i = tid; i < G * Dv; i += SA_THREADS) do_s[i] = bf2f(d_o[(bt * dm.HQ + hk * G) * (long)Dv + i]);
+  if (tid < G) slope_s[tid] = slope ? slope[hk * G + tid] : 0.f;
+
+  float dq_acc[SA_MAX_OUT];
+#pragma unroll
+  for (int j = 0; j < SA_MAX_OUT; ++j) dq_acc[j] = 0.f;
+  const int nq = G * D;
+
+  for (int kk = 0; kk < dm.K; ++kk) {
+    const int c = indices[irow * dm.K + kk];
+    __syncthreads();
+    if (c < 0 || c >= nchunk) continue;
+    if (tid < G) {
+      const long wrow = (b * LB + t / dm.q_block) * dm.WH + (dm.WH == dm.HQ ? hk * G + tid : hk);
+      w_s[tid] = bf2f(weights[wrow * dm.NW + kk]);
+    }
+    const bf16_t* kbase = k + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * D;
+    const bf16_t* vbase = v + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * Dv;
+    sa_scores(dm, q_s, kbase, slope ? slope_s : nullptr, p_s);
+    // dPV[g][s] = dO_g . V_s
+    for (int p = tid; p < G * S; p += SA_THREADS) {
+      const int g = p / S, s = p - g * S;
+      const bf16_t* vr = vbase + (long)s * dm.H * Dv;
+      float a = 0.f;
+      for (int d8 = 0; d8 < Dv / 8; ++d8) {
+        float f[8];
+        unpack8(*(const uint4*)(vr + d8 * 8), f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a = fmaf(do_s[g * Dv + d8 * 8 + j], f[j], a);
+      }
+      ds_s[p] = a;
+    }
+    __syncthreads();
+    for (int g = wave; g < G; g += SA_THREADS / 64) {
+      const float l2 = lse[(bt * dm.HQ + hk * G + g) * (long)dm.K + kk];
+      float part = 0.f;
+      for (int s = lane; s < S; s += 64) {
+        const float x = p_s[g * S + s];
+        const float pv = (x == HILS_NEG_INF || l2 == HILS_NEG_INF) ? 0.f : exp2f(x * HILS_LOG2E - l2);
+        p_s[g * S + s] = pv;
+        part += pv * ds_s[g * S + s];
+      }
+      part = wave_sum(part);
+      if (lane == 0) dwk[g] = part;
+      const float wg = w_s[g];
+      for (int s = lane; s < S; s += 64)
+        ds_s[g * S + s] = dm.sm_scale * wg * p_s[g * S + s] * (ds_s[g * S + s] - part);
+    }
+    __syncthreads();
+    if (tid < G) {
+      const long wrow = (b * LB + t / dm.q_block) * dm.WH + (dm.WH == dm.HQ ? hk * G + tid : hk);
+      if (dw_atomic) atomicAdd(dw + wrow * dm.NW + kk, dwk[tid]);
+      else dw[wrow * dm.NW + kk] = dwk[tid];
+    }
+    // dV[s][dv] += sum_g w_g P[g][s] dO[g][dv]
+    float* dvb = dv + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * Dv;
+    for (int p = tid; p < S * Dv; p += SA_THREADS) {
+      const int s = p / Dv, d = p - s * Dv;
+      float a = 0.f;
+      for (int g = 0; g < G; ++g) a = fmaf(w_s[g] * p_s[g * S + s], do_s[g * Dv + d], a);
+      if (a != 0.f) atomicAdd(dvb + (long)s * dm.H * Dv + d, a);
+    }
+    // dK[s][d] += sum_g dS[g][s] q[g][d]
+    float* dkb = dk + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * D;
+    for (int p = tid; p < S * D; p += SA_THREADS) {
+      const int s = p / D, d = p - s * D;
+      float a = 0.f;
+      for (int g = 0; g < G; ++g) a = fmaf(ds_s[g * S + s], q_s[g * D + d], a);
+      if (a != 0.f) atomicAdd(dkb + (long)s * dm.H * D + d, a);
+    }
+    // dQ[g][d] += sum_s dS[g][s] K[s][d]
+#pragma unroll
+    for (int j = 0; j < SA_MAX_OUT; ++j) {
+      const int oi = tid + j * SA_THREADS;
+      if (oi < nq) {
+        const int g = oi / D, d = oi - g * D;
+        float a = dq_acc[j];
+        for (int s = 0; s < S; ++s) a = fmaf(ds_s[g * S + s], bf2f(kbase[(long)s * dm.H * D + d]), a);
+        dq_acc[j] = a;
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < SA_MAX_OUT; ++j) {
+    const int oi = tid + j * SA_THREADS;
+    if (oi < nq) dq[(bt * dm.HQ + hk * G) * (long)D + oi] = f2bf(dq_acc[j]);
+  }
+}
+
+static int sa_check(const char* name, int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K,
+                    int NW, int WH, int q_block, int S) {
+  HILS_REQUIRE(B > 0 && L > 0 && Lkv > 0 && HQ > 0 && H > 0 && D > 0 && Dv > 0 && K > 0 && S > 0,
+               "%s: sizes must be positive", name);
+  HILS_REQUIRE(HQ % H == 0, "%s: HQ (%d) must be a multiple of H (%d)", name, HQ, H);
+  HILS_REQUIRE(D % 8 == 0 && Dv % 8 == 0, "%s: D (%d) and Dv (%d) must be multiples of 8", name, D, Dv);
+  HILS_REQUIRE(NW >= K, "%s: weights hold %d columns, need at least K = %d", name, NW, K);
+  HILS_REQUIRE(WH == HQ || WH == H, "%s: weights head count %d must be HQ or H", name, WH);
+  HILS_REQUIRE(q_block >= 1 && L % q_block == 0, "%s: L (%d) must be a multiple of q_block (%d)", name, L, q_block);
+  const int G = HQ / H;
+  HILS_REQUIRE(G * Dv <= SA_MAX_OUT * SA_THREADS && G * D <= SA_MAX_OUT * SA_THREADS,
+               "%s: G*D (%d) or G*Dv (%d) too large", name, G * D, G * Dv);
+  HILS_REQUIRE((long)B * L * H <= 2147483647L, "%s: grid too large", name);
+  return HILS_OK;
+}
+
+extern "C" int hils_sparse_attn_fwd(const void* q, const void* k, const void* v,
+                                    const void* weights, const int32_t* indices,
+                                    const float* slope, void* o, float* lse, int B, int L, int Lkv,
+                                    int HQ, int H, int D, int Dv, int K, int NW, int WH,
+                                    int q_block, int S, float sm_scale, int mask_last, float sm_n,
+                                    void* stream) {
+  HILS_REQUIRE(q && k && v && weights && indices && o, "hils_sparse_attn_fwd: null pointer");
+  if (int rc = sa_check("hils_sparse_attn_fwd", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
+  SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n};
+  size_t smem = ((size_t)dm.G * D + (size_t)dm.G * S + 2 * dm.G) * sizeof(float);
+  HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_fwd: G*(D+S) too large for LDS");
+  hipLaunchKernelGGL(sparse_attn_fwd_simple, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS),
+                     smem, (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k,
+                     (const bf16_t*)v, (const bf16_t*)weights, indices, slope, (bf16_t*)o, lse, dm);
+  HILS_CHECK_LAUNCH("hils_sparse_attn_fwd");
+  return HILS_OK;
+}
+
+extern "C" int hils_sparse_attn_bwd(const void* q, const void* k, const void* v,
+                                    const void* weights, const int32_t* indices,
+                                    const float* slope, const float* lse, const void* d_o,
+                                    void* dq, float* dk, float* dv, float* dw, int B, int L,
+                                    int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int WH,
+                                    int q_block, int S, float sm_scale, int mask_last, float sm_n,
+                                    void* stream) {
+  HILS_REQUIRE(q && k && v && weights && indices && lse && d_o && dq && dk && dv && dw,
+               "hils_sparse_attn_bwd: null pointer");
+  if (int rc = sa_check("hils_sparse_attn_bwd", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
+  SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n};
+  size_t smem = ((size_t)dm.G * (D + Dv) + 2 * (size_t)dm.G * S + 3 * dm.G) * sizeof(float);
+  HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_bwd: G*(D+Dv+2S) too large for LDS");
+  hipLaunchKernelGGL(sparse_attn_bwd_simple, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS),
+                     smem, (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k,
+                     (const bf16_t*)v, (const bf16_t*)weights, indices, slope, lse,
+                     (const bf16_t*)d_o, (bf16_t*)dq, dk, dv, dw, dm);
+  HILS_CHECK_LAUNCH("hils_sparse_attn_bwd");
+  return HILS_OK;
+}

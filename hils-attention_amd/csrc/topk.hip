@@ -1,0 +1,487 @@
+// Query -> chunk-key scoring with per-(query, KV head) top-k selection.
+//
+// One workgroup (4 wavefronts) owns 16 consecutive queries of one (batch, KV head).
+// The logits of a 16-query x 16-chunk tile come from one chain of 16x16x32 bf16 MFMAs
+// per query head g (A = the 16 query rows of head g, B = 16 chunk keys).  Two passes
+// over the visible chunks: pass 1 keeps an online log-sum-exp per (query, g); pass 2
+// recomputes the logits, forms max_g(logit - lse_total), parks the pooled scores of a
+// segment of chunks in LDS and lets one wavefront per query pick the top-k with a
+// bitwise threshold search on order-preserving integer keys.  Ties: lower index wins.
+#include "common.h"
+#include "../../include/hils_amd.h"
+
+#define TOPK_THREADS 256
+#define TOPK_QT 16        // queries per workgroup
+#define TOPK_NSEG 512     // chunks per selection segment
+#define TOPK_SLOTS (TOPK_NSEG / 64)
+#define TOPK_MAXK 64
+
+__device__ __forceinline__ float logaddexp_f(float a, float b) {
+  if (a == HILS_NEG_INF) return b;
+  if (b == HILS_NEG_INF) return a;
+  const float m = fmaxf(a, b), n = fminf(a, b);
+  return m + log1pf(expf(n - m));
+}
+
+// order-preserving key: larger float <-> larger key; 0 = "not a candidate"
+__device__ __forceinline__ uint32_t score_key(float f) {
+  if (!(f > HILS_NEG_INF)) return 0u;  // -inf and NaN
+  f = f + 0.0f;                        // -0 -> +0
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_score(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// One wavefront selects the top-K of (previous candidates) U (segment scores).
+// cand_* hold the previous winners in ascending index order (ncand of them, all with
+// an index below seg_base); seg holds ns pooled scores of chunks seg_base..seg_base+ns-1.
+// The winners are written back to cand_* in ascending index order; returns the count.
+__device__ int wave_select(const float* seg, int ns, int seg_base, float* cand_s, int* cand_i,
+                           int ncand, int K) {
+  const int lane = threadIdx.x & 63;
+  uint32_t key[TOPK_SLOTS + 1];
+  int cidx = -1;
+  key[0] = 0u;
+  if (lane < ncand) {
+    key[0] = score_key(cand_s[lane]);
+    cidx = cand_i[lane];
+  }
+#pragma unroll
+  for (int s = 0; s < TOPK_SLOTS; ++s) {
+    const int i = s * 64 + lane;
+    key[s + 1] = (i < ns) ? score_key(seg[i]) : 0u;
+  }
+  const int nslot = (ns + 63) / 64 + 1;
+  int total = 0;
+#pragma unroll
+  for (int s = 0; s <= TOPK_SLOTS; ++s)
+    if (s < nslot) total += __popcll(__ballot(key[s] != 0u));
+  uint32_t T = 1u;  // every valid key is >= 1
+  if (total > K) {
+    T = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t c = T | (1u << bit);
+      int cnt = 0;
+#pragma unroll
+      for (int s = 0; s <= TOPK_SLOTS; ++s)
+        if (s < nslot) cnt += __popcll(__ballot(key[s] >= c));
+      if (cnt >= K) {
+        T = c;
+        if (cnt == K) break;
+      }
+    }
+  }
+  int gt = 0;
+#pragma unroll
+  for (int s = 0; s <= TOPK_SLOTS; ++s)
+    if (s < nslot) gt += __popcll(__ballot(key[s] > T));
+  int need = K - gt;  // ties with the threshold still to take, lowest index first
+  int pos = 0;
+  const unsigned long long lt = (1ull << lane) - 1ull;
+#pragma unroll
+  for (int s = 0; s <= TOPK_SLOTS; ++s) {
+    if (s < nslot) {
+      const unsigned long long eq = __ballot(key[s] == T && key[s] != 0u);
+      const bool take_eq = (key[s] == T && key[s] != 0u) && (__popcll(eq & lt) < need);
+      const bool sel = (key[s] > T) || take_eq;
+      const unsigned long long sm = __ballot(sel);
+      if (sel) {
+        const int o = pos + __popcll(sm & lt);
+        cand_s[o] = key_score(key[s]);
+        cand_i[o] = (s == 0) ? cidx : seg_base + (s - 1) * 64 + lane;
+      }
+      pos += __popcll(sm);
+      const int took = __popcll(eq);
+      need -= took < need ? took : need;
+    }
+  }
+  return pos;
+}
+
+template <int GMAX, int KS>
+__global__ void __launch_bounds__(TOPK_THREADS)
+topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
+                const float* __restrict__ lse_swa, const float* __restrict__ bias,
+                const float* __restrict__ gumbel, const int32_t* __restrict__ drop_mask,
+                int32_t* __restrict__ indices, bf16_t* __restrict__ scores,
+                float* __restrict__ lse_total_out, float* __restrict__ sel_logits_out,
+                int L, int N, int h_kv, int G, int topk, int block_size, int window_size,
+                int causal, int q_offset, int per_qhead, float sm_scale) {
+  constexpr int D = KS * 32;
+  __shared__ float pooled[TOPK_QT][TOPK_NSEG];
+  __shared__ float cand_s[TOPK_QT][TOPK_MAXK];
+  __shared__ int cand_i[TOPK_QT][TOPK_MAXK];
+  __shared__ float part_m[4][GMAX][TOPK_QT];
+  __shared__ float part_l[4][GMAX][TOPK_QT];
+  __shared__ float lse_tot[GMAX][TOPK_QT];
+  __shared__ int ncand_s[TOPK_QT];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int t0 = blockIdx.x * TOPK_QT;
+  const int hk = blockIdx.y;
+  const long b = blockIdx.z;
+  const int lmk_h = per_qhead ? h_kv * G : h_kv;
+
+  // visible-chunk limit of the 4 queries this lane's accumulator rows belong to
+  int lim[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int tq = t0 + grp * 4 + i;
+    int lm = causal ? visible_limit(tq + q_offset, window_size, block_size) : N;
+    lm = lm < 0 ? 0 : (lm > N ? N : lm);
+    lim[i] = (tq < L) ? lm : 0;
+  }
+  int tile_lim;
+  {
+    const int tl = (t0 + TOPK_QT - 1 < L) ? t0 + TOPK_QT - 1 : L - 1;
+    int lm = causal ? visible_limit(tl + q_offset, window_size, block_size) : N;
+    tile_lim = lm < 0 ? 0 : (lm > N ? N : lm);
+  }
+  const int nblk = (tile_lim + 15) / 16;
+
+  // A operands: row (lane & 15) = query t0 + row of head g, 8 consecutive d per k-step
+  bf16x8_t afrag[GMAX][KS];
+  {
+    const int tq = t0 + col;
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (g < G && tq < L)
+          v = *(const uint4*)(q + (((b * L + tq) * h_kv + hk) * (long)G + g) * D + ks * 32 + grp * 8);
+        afrag[g][ks] = *(bf16x8_t*)&v;
+      }
+  }
+
+  // ---------------- pass 1: online log-sum-exp per (query, g) ----------------
+  float rm[GMAX][4], rl[GMAX][4];
+#pragma unroll
+  for (int g = 0; g < GMAX; ++g)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { rm[g][i] = HILS_NEG_INF; rl[g][i] = 0.f; }
+
+  for (int blk = wave; blk < nblk; blk += 4) {
+    const int c = blk * 16 + col;
+    const bool cvalid = c < N;
+    bf16x8_t bfrag[KS];
+    if (!per_qhead) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (cvalid) v = *(const uint4*)(lmks + ((b * N + c) * (long)lmk_h + hk) * D + ks * 32 + grp * 8);
+        bfrag[ks] = *(bf16x8_t*)&v;
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+      if (g < G) {
+        if (per_qhead) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (cvalid)
+              v = *(const uint4*)(lmks + ((b * N + c) * (long)lmk_h + hk * G + g) * D + ks * 32 + grp * 8);
+            bfrag[ks] = *(bf16x8_t*)&v;
+          }
+        }
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[g][ks], bfrag[ks], acc, 0, 0, 0);
+        float add = 0.f;
+        if (cvalid) {
+          if (bias) add = bias[((b * N + c) * (long)h_kv + hk) * G + g];
+        }
+        const float gum = (cvalid && gumbel) ? gumbel[(long)(hk * G + g) * N + c] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float x = __fmul_rn(acc[i], sm_scale);
+          if (bias) x = __fadd_rn(x, add);
+          if (gumbel) x = __fadd_rn(x, gum);
+          if (!(cvalid && c < lim[i])) x = HILS_NEG_INF;
+          const float mn = fmaxf(rm[g][i], x);
+          if (mn > HILS_NEG_INF) {
+            rl[g][i] = rl[g][i] * __expf(rm[g][i] - mn) + __expf(x - mn);
+            rm[g][i] = mn;
+          }
+        }
+      }
+    }
+  }
+  // combine over the 16 columns of a lane group, then over the 4 wavefronts
+#pragma unroll
+  for (int g = 0; g < GMAX; ++g) {
+    if (g < G) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float m = rm[g][i], l = rl[g][i];
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) {
+          const float m2 = __shfl_xor(m, o, 64), l2 = __shfl_xor(l, o, 64);
+          const float mn = fmaxf(m, m2);
+          if (mn > HILS_NEG_INF) {
+            l = l * __expf(m - mn) + l2 * __expf(m2 - mn);
+            m = mn;
+          }
+        }
+        if (col == 0) {
+          part_m[wave][g][grp * 4 + i] = m;
+          part_l[wave][g][grp * 4 + i] = l;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  for (int p = tid; p < G * TOPK_QT; p += TOPK_THREADS) {
+    const int g = p / TOPK_QT, qi = p - g * TOPK_QT;
+    float m = HILS_NEG_INF, l = 0.f;
+    for (int w = 0; w < 4; ++w) {
+      const float m2 = part_m[w][g][qi], l2 = part_l[w][g][qi];
+      const float mn = fmaxf(m, m2);
+      if (mn > HILS_NEG_INF) {
+        l = l * __expf(m - mn) + l2 * __expf(m2 - mn);
+        m = mn;
+      }
+    }
+    const float lse_hils = (l > 0.f) ? m + logf(l) : HILS_NEG_INF;
+    const int tq = t0 + qi;
+    float tot = HILS_NEG_INF;
+    if (tq < L) {
+      const long o = ((b * L + tq) * (long)h_kv + hk) * G + g;
+      tot = logaddexp_f(lse_swa[o], lse_hils);
+      if (lse_total_out) lse_total_out[o] = tot;
+    }
+    lse_tot[g][qi] = tot;
+  }
+  if (tid < TOPK_QT) ncand_s[tid] = 0;
+  __syncthreads();
+
+  // ---------------- pass 2: pooled scores per segment + selection ----------------
+  float lt_reg[GMAX][4];
+#pragma unroll
+  for (int g = 0; g < GMAX; ++g)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lt_reg[g][i] = (g < G) ? lse_tot[g][grp * 4 + i] : 0.f;
+
+  const int nseg = (nblk * 16 + TOPK_NSEG - 1) / TOPK_NSEG;
+  for (int seg = 0; seg < nseg; ++seg) {
+    const int seg_base = seg * TOPK_NSEG;
+    const int blk_end = ((seg + 1) * (TOPK_NSEG / 16) < nblk) ? (seg + 1) * (TOPK_NSEG / 16) : nblk;
+    for (int blk = seg * (TOPK_NSEG / 16) + wave; blk < blk_end; blk += 4) {
+      const int c = blk * 16 + col;
+      const bool cvalid = c < N;
+      bf16x8_t bfrag[KS];
+      if (!per_qhead) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          uint4 v = make_uint4(0, 0, 0, 0);
+          if (cvalid) v = *(const uint4*)(lmks + ((b * N + c) * (long)lmk_h + hk) * D + ks * 32 + grp * 8);
+          bfrag[ks] = *(bf16x8_t*)&v;
+        }
+      }
+      float best[4] = {HILS_NEG_INF, HILS_NEG_INF, HILS_NEG_INF, HILS_NEG_INF};
+#pragma unroll
+      for (int g = 0; g < GMAX; ++g) {
+        if (g < G) {
+          if (per_qhead) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+              uint4 v = make_uint4(0, 0, 0, 0);
+              if (cvalid)
+                v = *(const uint4*)(lmks + ((b * N + c) * (long)lmk_h + hk * G + g) * D + ks * 32 + grp * 8);
+              bfrag[ks] = *(bf16x8_t*)&v;
+            }
+          }
+          f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[g][ks], bfrag[ks], acc, 0, 0, 0);
+          float add = 0.f;
+          if (cvalid && bias) add = bias[((b * N + c) * (long)h_kv + hk) * G + g];
+          const float gum = (cvalid && gumbel) ? gumbel[(long)(hk * G + g) * N + c] : 0.f;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float x = __fmul_rn(acc[i], sm_scale);
+            if (bias) x = __fadd_rn(x, add);
+            if (gumbel) x = __fadd_rn(x, gum);
+            const bool vis = cvalid && c < lim[i];
+            if (!vis) x = HILS_NEG_INF;
+            if (sel_logits_out && cvalid) {
+              const int tq = t0 + grp * 4 + i;
+              if (tq < L)
+                sel_logits_out[(((b * L + tq) * (long)h_kv + hk) * G + g) * N + c] = x;
+            }
+            const float nrm = (x == HILS_NEG_INF) ? HILS_NEG_INF : __fsub_rn(x, lt_reg[g][i]);
+            best[i] = fmaxf(best[i], nrm);  // fmaxf ignores a NaN operand
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float s = best[i];
+        if (drop_mask && s > HILS_NEG_INF) {
+          const int tq = t0 + grp * 4 + i;
+          if (tq < L && cvalid && drop_mask[(b * L + tq) * (long)N + c] != 0) s = HILS_NEG_INF;
+        }
+        pooled[grp * 4 + i][c - seg_base] = s;
+      }
+    }
+    __syncthreads();
+    const int ns = blk_end * 16 - seg_base;
+    for (int qi = wave; qi < TOPK_QT; qi += 4) {
+      if (t0 + qi < L) {
+        const int nc = wave_select(pooled[qi], ns, seg_base, cand_s[qi], cand_i[qi], ncand_s[qi], topk);
+        if (lane == 0) ncand_s[qi] = nc;
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---------------- epilogue: indices and raw scaled scores ----------------
+  for (int qi = wave; qi < TOPK_QT; qi += 4) {
+    const int tq = t0 + qi;
+    if (tq >= L) continue;
+    const int nc = ncand_s[qi];
+    int32_t* irow = indices + ((b * L + tq) * (long)h_kv + hk) * topk;
+    for (int k = lane; k < topk; k += 64) irow[k] = (k < nc) ? cand_i[qi][k] : -1;
+    for (int p = lane; p < topk * G; p += 64) {
+      const int g = p / topk, k = p - g * topk;
+      float val = HILS_NEG_INF;
+      if (k < nc) {
+        const int c = cand_i[qi][k];
+        const bf16_t* qr = q + (((b * L + tq) * h_kv + hk) * (long)G + g) * D;
+        const bf16_t* kr = lmks + ((b * N + c) * (long)lmk_h + (per_qhead ? hk * G + g : hk)) * D;
+        float a = 0.f;
+#pragma unroll
+        for (int d8 = 0; d8 < D / 8; ++d8) {
+          float fq[8], fk[8];
+          unpack8(*(const uint4*)(qr + d8 * 8), fq);
+          unpack8(*(const uint4*)(kr + d8 * 8), fk);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) a = fmaf(fq[j], fk[j], a);
+        }
+        val = a * sm_scale;
+      }
+      scores[((((b * L + tq) * (long)h_kv + hk) * G + g)) * topk + k] = f2bf(val);
+    }
+  }
+}
+
+template <int GMAX>
+static int launch_topk(int D, dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* lmks,
+                       const float* lse_swa, const float* bias, const float* gumbel,
+                       const int32_t* drop_mask, int32_t* indices, bf16_t* scores, float* lse_total,
+                       float* sel_logits, int L, int N, int h_kv, int G, int topk, int block_size,
+                       int window_size, int causal, int q_offset, int per_qhead, float sm_scale) {
+#define HILS_TOPK_LAUNCH(KS_)                                                                    \
+  hipLaunchKernelGGL((topk_fwd_kernel<GMAX, KS_>), grid, dim3(TOPK_THREADS), 0, st, q, lmks,     \
+                     lse_swa, bias, gumbel, drop_mask, indices, scores, lse_total, sel_logits, L, \
+                     N, h_kv, G, topk, block_size, window_size, causal, q_offset, per_qhead,     \
+                     sm_scale)
+  switch (D) {
+    case 64: HILS_TOPK_LAUNCH(2); break;
+    case 128: HILS_TOPK_LAUNCH(4); break;
+    default:
+      hils_set_error("hils_topk_fwd: head dim %d not supported (64 or 128)", D);
+      return HILS_ERR_ARG;
+  }
+#undef HILS_TOPK_LAUNCH
+  return HILS_OK;
+}
+
+extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_swa,
+                             const float* bias, const float* gumbel, const int32_t* drop_mask,
+                             int32_t* indices, void* scores, float* lse_total, float* sel_logits,
+                             int B, int L, int N, int h_kv, int G, int D, int topk, int block_size,
+                             int window_size, int causal, int q_offset, int per_qhead,
+                             float sm_scale, void* stream) {
+  HILS_REQUIRE(q && lmks && lse_swa && indices && scores, "hils_topk_fwd: null pointer");
+  HILS_REQUIRE(B > 0 && L > 0 && N > 0 && h_kv > 0 && G > 0 && D > 0, "hils_topk_fwd: sizes must be positive");
+  HILS_REQUIRE(topk >= 1 && topk <= TOPK_MAXK, "hils_topk_fwd: topk (%d) must be in 1..%d", topk, TOPK_MAXK);
+  HILS_REQUIRE(G <= 16, "hils_topk_fwd: group size %d not supported (max 16)", G);
+  HILS_REQUIRE(block_size > 0, "hils_topk_fwd: block_size must be positive");
+  HILS_REQUIRE(h_kv <= 65535 && B <= 65535, "hils_topk_fwd: h_kv/B too large for the grid");
+  dim3 grid((L + TOPK_QT - 1) / TOPK_QT, h_kv, B);
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+#define HILS_TOPK_ARGS                                                                             \
+  D, grid, st, (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, gumbel, drop_mask, indices,  \
+      (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk, block_size, window_size, causal, \
+      q_offset, per_qhead, sm_scale
+  if (G == 1) rc = launch_topk<1>(HILS_TOPK_ARGS);
+  else if (G == 2) rc = launch_topk<2>(HILS_TOPK_ARGS);
+  else if (G <= 4) rc = launch_topk<4>(HILS_TOPK_ARGS);
+  else if (G <= 8) rc = launch_topk<8>(HILS_TOPK_ARGS);
+  else rc = launch_topk<16>(HILS_TOPK_ARGS);
+#undef HILS_TOPK_ARGS
+  if (rc) return rc;
+  HILS_CHECK_LAUNCH("hils_topk_fwd");
+  return HILS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// backward of the score gather: scores[b,t,h,g,k] = sm_scale * <q[b,t,h,g], lmk[b,idx,h(,g)]>
+// ---------------------------------------------------------------------------
+// One block per (b, t, hk); thread d owns one feature column.
+__global__ void topk_bwd_kernel(const bf16_t* __restrict__ gs, const bf16_t* __restrict__ q,
+                                const bf16_t* __restrict__ lmks, const int32_t* __restrict__ indices,
+                                bf16_t* __restrict__ dq, float* __restrict__ dlmk, int L, int N,
+                                int h_kv, int G, int D, int topk, int per_qhead, float sm_scale) {
+  extern __shared__ float sm[];  // G*topk scaled grads, then topk indices
+  float* gsc = sm;
+  int* idx = (int*)(sm + G * topk);
+  const long row = blockIdx.x;  // (b*L + t)*h_kv + hk
+  const int hk = (int)(row % h_kv);
+  const long bt = row / h_kv;
+  const long b = bt / L;
+  const int lmk_h = per_qhead ? h_kv * G : h_kv;
+  for (int i = threadIdx.x; i < G * topk; i += blockDim.x) gsc[i] = bf2f(gs[row * G * topk + i]) * sm_scale;
+  for (int i = threadIdx.x; i < topk; i += blockDim.x) idx[i] = indices[row * topk + i];
+  __syncthreads();
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    for (int g = 0; g < G; ++g) {
+      float a = 0.f;
+      for (int k = 0; k < topk; ++k) {
+        const int c = idx[k];
+        if (c >= 0 && c < N)
+          a += gsc[g * topk + k] * bf2f(lmks[((b * N + c) * (long)lmk_h + (per_qhead ? hk * G + g : hk)) * D + d]);
+      }
+      dq[(row * G + g) * D + d] = f2bf(a);
+    }
+    for (int k = 0; k < topk; ++k) {
+      const int c = idx[k];
+      if (c < 0 || c >= N) continue;
+      if (per_qhead) {
+        for (int g = 0; g < G; ++g) {
+          const float v = gsc[g * topk + k] * bf2f(q[(row * G + g) * D + d]);
+          if (v != 0.f) atomicAdd(dlmk + ((b * N + c) * (long)lmk_h + hk * G + g) * D + d, v);
+        }
+      } else {
+        float v = 0.f;
+        for (int g = 0; g < G; ++g) v += gsc[g * topk + k] * bf2f(q[(row * G + g) * D + d]);
+        if (v != 0.f) atomicAdd(dlmk + ((b * N + c) * (long)lmk_h + hk) * D + d, v);
+      }
+    }
+  }
+}
+
+extern "C" int hils_topk_bwd(const void* g_scores, const void* q, const void* lmks,
+                             const int32_t* indices, void* dq, float* dlmk, int B, int L, int N,
+                             int h_kv, int G, int D, int topk, int per_qhead, float sm_scale,
+                             void* stream) {
+  HILS_REQUIRE(g_scores && q && lmks && indices && dq && dlmk, "hils_topk_bwd: null pointer");
+  HILS_REQUIRE(B > 0 && L > 0 && N > 0 && h_kv > 0 && G > 0 && D > 0 && topk > 0, "hils_topk_bwd: sizes must be positive");
+  const long rows = (long)B * L * h_kv;
+  HILS_REQUIRE(rows <= 2147483647L, "hils_topk_bwd: grid too large");
+  const int threads = D >= 128 ? 128 : 64;
+  size_t smem = ((size_t)G * topk + topk) * sizeof(float);
+  hipLaunchKernelGGL(topk_bwd_kernel, dim3((unsigned)rows), dim3(threads), smem, (hipStream_t)stream,
+                     (const bf16_t*)g_scores, (const bf16_t*)q, (const bf16_t*)lmks, indices,
+                     (bf16_t*)dq, dlmk, L, N, h_kv, G, D, topk, per_qhead, sm_scale);
+  HILS_CHECK_LAUNCH("hils_topk_bwd");
+  return HILS_OK;
+}

@@ -1,0 +1,87 @@
+"""ctypes binding of libhils_amd.so (the C ABI declared in include/hils_amd.h).
+
+The library is the only compute path of this package: if it is missing or a call
+fails, a RuntimeError is raised.  There is no Triton/TileLang/PyTorch fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_float, c_int, c_void_p
+
+import torch
+
+_PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG_DIR, "libhils_amd.so")
+
+_P, _I, _F = c_void_p, c_int, c_float
+
+# name -> argument types, in the order of include/hils_amd.h
+SIGNATURES = {
+    "hils_mean_pool_fwd": [_P, _P, _I, _I, _I, _I, _I, _P],
+    "hils_mean_pool_bwd": [_P, _P, _I, _I, _I, _I, _I, _P],
+    "hils_attn_pool_fwd": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
+    "hils_attn_pool_bwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
+    "hils_topk_fwd": [_P] * 10 + [_I] * 12 + [_F, _P],
+    "hils_topk_bwd": [_P] * 6 + [_I] * 8 + [_F, _P],
+    "hils_sparse_attn_fwd": [_P] * 8 + [_I] * 12 + [_F, _I, _F, _P],
+    "hils_sparse_attn_bwd": [_P] * 12 + [_I] * 12 + [_F, _I, _F, _P],
+    "hils_chunk_logz_fwd": [_P, _P, _P] + [_I] * 7 + [_F, _I, _P],
+    "hils_chunk_logz_bwd_dq": [_P] * 5 + [_I] * 7 + [_F, _P],
+    "hils_chunk_logz_bwd_dk": [_P] * 5 + [_I] * 7 + [_F, _P],
+}
+
+_lib = None
+
+
+def load():
+    """Load libhils_amd.so once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python __graft_entry__.py build` "
+            "(hipcc --offload-arch=gfx950). This package has no fallback path.")
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.hils_last_error.restype = ctypes.c_char_p
+    lib.hils_last_error.argtypes = []
+    lib.hils_version.restype = c_int
+    lib.hils_version.argtypes = []
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = c_int
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def ptr(t):
+    """Device pointer of a tensor (None -> NULL)."""
+    if t is None:
+        return None
+    return c_void_p(t.data_ptr())
+
+
+def stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def call(name, *args):
+    """Call an entry point on the current stream; raise RuntimeError on a non-zero status."""
+    lib = load()
+    rc = getattr(lib, name)(*args, stream())
+    if rc != 0:
+        msg = lib.hils_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{name} failed (status {rc}): {msg}")
+
+
+def require_gpu_bf16(name, *tensors):
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(f"{name}: tensors must live on the GPU (got {t.device}); "
+                               "this package has no CPU path")
+        if t.dtype != torch.bfloat16:
+            raise TypeError(f"{name}: expected bfloat16 tensors, got {t.dtype}")

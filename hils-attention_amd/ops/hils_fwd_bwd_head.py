@@ -1,0 +1,92 @@
+"""HiLS sparse attention over the selected chunks (drop-in for ops/hils_fwd_bwd_head.py)."""
+import math
+
+import torch
+
+from . import _cabi
+
+
+class _hils_block_M_attention_inverse(torch.autograd.Function):
+    """Mirrors _hils_block_M_attention_inverse (ops/hils_fwd_bwd_head.py:771-913)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, weights, indices, block_size, sm_scale, mask_last_token,
+                is_training, slope=None):
+        assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+        assert weights.is_contiguous() and indices.is_contiguous()
+        _cabi.require_gpu_bf16("HiLS_block_M_head", q, k, v)
+        B, L, HQ, D = q.shape
+        L_kv, H, Dk = k.shape[1], k.shape[2], k.shape[-1]
+        Dv = v.shape[-1]
+        K = indices.shape[-1]
+        num_weights = weights.shape[-1]
+        assert HQ % H == 0, f"HQ={HQ} must be divisible by H={H}"
+        assert Dk == D, f"Q head_dim ({D}) must equal K head_dim ({Dk})"
+        assert indices.shape == (B, L, H, K), f"indices shape {tuple(indices.shape)} != {(B, L, H, K)}"
+        assert weights.shape[:3] == (B, L, HQ) and num_weights >= K, (
+            f"weights shape {tuple(weights.shape)} must be ({B}, {L}, {HQ}, >= {K})")
+        if sm_scale is None:
+            sm_scale = 1.0 / math.sqrt(D)
+        slope_dev = None
+        if slope is not None:
+            assert slope.shape == (HQ,), f"slope must be 1-D with shape ({HQ},), got {tuple(slope.shape)}"
+            slope_dev = slope.to(dtype=torch.float32, device=q.device).contiguous()
+        w_in = weights.to(q.dtype).contiguous()
+        idx_in = indices.to(torch.int32).contiguous()
+        o = torch.empty((B, L, HQ, Dv), dtype=q.dtype, device=q.device)
+        lse = None
+        if is_training:
+            lse = torch.empty((B, L, HQ, K), dtype=torch.float32, device=q.device)
+        _cabi.call("hils_sparse_attn_fwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
+                   _cabi.ptr(idx_in), _cabi.ptr(slope_dev), _cabi.ptr(o), _cabi.ptr(lse),
+                   B, L, L_kv, HQ, H, D, Dv, K, num_weights, HQ, 1, int(block_size),
+                   float(sm_scale), int(bool(mask_last_token)), 0.0)
+        ctx.is_training = bool(is_training)
+        if is_training:
+            ctx.save_for_backward(q, k, v, w_in, idx_in, lse, slope_dev)
+            ctx.cfg = (B, L, L_kv, HQ, H, D, Dv, K, num_weights, int(block_size), float(sm_scale),
+                       int(bool(mask_last_token)))
+            ctx.w_dtype = weights.dtype
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        if not getattr(ctx, "is_training", True):
+            raise RuntimeError(
+                "[_hils_block_M_attention_inverse] forward ran with is_training=False: the "
+                "per-chunk LSE needed by the backward was not saved.")
+        q, k, v, w_in, idx_in, lse, slope_dev = ctx.saved_tensors
+        B, L, L_kv, HQ, H, D, Dv, K, NW, S, sm_scale, mask_last = ctx.cfg
+        do = do.to(q.dtype).contiguous()
+        dq = torch.empty_like(q)
+        dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
+        dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)
+        dw = torch.zeros((B, L, HQ, NW), dtype=torch.float32, device=q.device)
+        _cabi.call("hils_sparse_attn_bwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
+                   _cabi.ptr(idx_in), _cabi.ptr(slope_dev), _cabi.ptr(lse), _cabi.ptr(do),
+                   _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw),
+                   B, L, L_kv, HQ, H, D, Dv, K, NW, HQ, 1, S, sm_scale, mask_last, 0.0)
+        return (dq, dk.to(k.dtype), dv.to(v.dtype), dw.to(ctx.w_dtype), None,
+                None, None, None, None, None)
+
+
+def HiLS_block_M_head(q, k, v, weights, indices, block_size=64, sm_scale=None, block_M=None,
+                      mask_last_token=True, dtype="bfloat16", accum_dtype="float",
+                      num_threads=None, num_threads_fwd=None, num_threads_bwd=None,
+                      is_training=True, slope=None):
+    """o[t,h] = sum_k weights[t,h,k] * softmax_{j in chunk indices[t,k]}(sm_scale*q.K_j) V_j.
+
+    q (B,L,HQ,D), k (B,Lkv,H,D), v (B,Lkv,H,Dv) bf16 contiguous; weights (B,L,HQ,>=K) (the
+    first K columns are read); indices (B,L,H,K) int32, negative = empty slot.  Call
+    signature of ops/hils_fwd_bwd_head.py:928-934; ``block_M`` and the ``num_threads*``
+    tuning knobs are accepted and ignored (tile shapes are chosen by the HIP launcher),
+    ``dtype`` must be "bfloat16" and ``accum_dtype`` "float".
+    """
+    B, L, HQ, D = q.shape
+    _, L_kv, H, Dk = k.shape
+    assert D == Dk, f"Q head_dim ({D}) must equal K head_dim ({Dk})"
+    assert HQ % H == 0, f"HQ={HQ} must be divisible by H={H}"
+    if dtype not in ("bfloat16", torch.bfloat16) or accum_dtype not in ("float", "float32", torch.float32):
+        raise ValueError("HiLS_block_M_head: only dtype='bfloat16' with accum_dtype='float' is built")
+    return _hils_block_M_attention_inverse.apply(
+        q, k, v, weights, indices, block_size, sm_scale, mask_last_token, is_training, slope)

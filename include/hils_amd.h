@@ -1,0 +1,130 @@
+/* C ABI of libhils_amd.so: hand-written gfx950 kernels for the HiLS-Attention
+ * operator stack.  Plain pointers and sizes only; every pointer is a DEVICE
+ * pointer unless stated; `stream` is a hipStream_t passed as void*.  All tensors
+ * are contiguous, token-major (B, L, H, D), bf16 = raw bfloat16 bits.
+ * Every function returns 0 on success, 1 on an invalid argument, 2 on a launch
+ * failure; hils_last_error() then returns a message.  No function allocates or
+ * frees device memory or synchronises the stream.
+ *
+ * Each entry point cites the reference interface it replaces (paths relative to
+ * the reference repository root).
+ */
+#ifndef HILS_AMD_H
+#define HILS_AMD_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* hils_last_error(void);
+int hils_version(void);
+
+/* ---- chunk keys ------------------------------------------------------------ */
+
+/* Mean pool: lmk_k[b,n,h,:] = mean_s k[b,n*S+s,h,:].
+ * Replaces `k_chunked.mean(dim=2)` at models/FlashHiLS/hils_attention.py:398,436,446,460.
+ * k (B,L,H,D) bf16 -> lmk_k (B,L/S,H,D) bf16.  L % S == 0, D % 8 == 0. */
+int hils_mean_pool_fwd(const void* k, void* lmk_k, int B, int L, int H, int D, int S, void* stream);
+/* Its backward: dk[b,t,h,:] = g_lmk[b,t/S,h,:] / S (bf16 in, bf16 out). */
+int hils_mean_pool_bwd(const void* g_lmk, void* dk, int B, int L, int H, int D, int S, void* stream);
+
+/* Attention pool forward.  Replaces chunk_attn_pool_fwd_kernel_fallback /
+ * chunk_attn_pool_fwd_kernel behind ChunkAttnPoolFunction.forward
+ * (ops/chunk_attn_pool_tilelang.py:329-410, :31-150, :540-570).
+ * mu_q (BN,H,D) bf16, k (BN,S,H,D) bf16 -> lmk_k (BN,H,D) bf16, lmk_b (BN,H) fp32,
+ * p (BN,S,H) fp32 (saved for backward).  compact != 0: lmk_k is written as zeros.
+ * shared_k != 0: K is read from head 0 for every head. */
+int hils_attn_pool_fwd(const void* mu_q, const void* k, void* lmk_k, float* lmk_b, float* p,
+                       int BN, int S, int H, int D, float sm_scale, int compact, int shared_k,
+                       void* stream);
+/* Attention pool backward.  Replaces chunk_attn_pool_bwd_kernel_fallback /
+ * chunk_attn_pool_bwd_kernel (ops/chunk_attn_pool_tilelang.py:425-533, :165-314).
+ * g_k (BN,H,D) bf16, g_b (BN,H) fp32 -> d_mu (BN,H,D) bf16, d_k (BN,S,H,D) bf16.
+ * shared_k != 0: d_k is summed over heads into head 0 and heads 1.. are zero. */
+int hils_attn_pool_bwd(const void* mu_q, const void* k, const float* p, const float* lmk_b,
+                       const void* g_k, const float* g_b, void* d_mu, void* d_k,
+                       int BN, int S, int H, int D, float sm_scale, int compact, int shared_k,
+                       void* stream);
+
+/* ---- top-k chunk selection -------------------------------------------------- */
+
+/* Fused LSE + select + ascending sort + score gather.  Replaces hils_lse_kernel,
+ * torch.logaddexp, weighted_select_kernel, sort_topk_indices_kernel and
+ * recompute_topk_max_pooling_scores_kernel as sequenced by
+ * SoftmaxTopKMaxPoolingFusedFn.forward (ops/topk_head_softmax.py:192-400, :438-631,
+ * :870-971, :669-832, :1012-1038).
+ * q (B,L,h_kv,G,D) bf16; lmks (B,N,h_kv,D) bf16 or, per_qhead != 0, (B,N,h_kv*G,D);
+ * lse_swa (B,L,h_kv,G) fp32; bias (B,N,h_kv,G) fp32 or NULL; gumbel (h_kv*G,N) fp32 or
+ * NULL; drop_mask (B,L,N) int32 or NULL.
+ * Outputs: indices (B,L,h_kv,topk) int32 ascending, -1 padded; scores
+ * (B,L,h_kv,G,topk) bf16 = sm_scale*<q,lmk[idx]>, -inf where idx < 0.
+ * Optional outputs (NULL to skip): lse_total (B,L,h_kv,G) fp32 =
+ * logaddexp(lse_swa, lse_hils); sel_logits (B,L,h_kv,G,N) fp32 = the selection
+ * logits (scaled qk + bias + gumbel, -inf where the chunk is not visible).
+ * Chunk c is visible to query t iff !causal or c < floor((t+q_offset-window+1)/block)
+ * (window > 0) / floor((t+q_offset)/block) (window <= 0).  Ties: lower index wins. */
+int hils_topk_fwd(const void* q, const void* lmks, const float* lse_swa, const float* bias,
+                  const float* gumbel, const int32_t* drop_mask, int32_t* indices, void* scores,
+                  float* lse_total, float* sel_logits, int B, int L, int N, int h_kv, int G, int D,
+                  int topk, int block_size, int window_size, int causal, int q_offset,
+                  int per_qhead, float sm_scale, void* stream);
+
+/* Sparse backward of the score gather.  Replaces the dense scatter + two torch.bmm of
+ * SoftmaxTopKMaxPoolingFusedFn.backward (ops/topk_head_softmax.py:1040-1092).
+ * g_scores (B,L,h_kv,G,topk) bf16 -> dq (B,L,h_kv,G,D) bf16 (written),
+ * dlmk fp32 (B,N,h_kv or h_kv*G,D) (ACCUMULATED with atomics: caller zero-fills). */
+int hils_topk_bwd(const void* g_scores, const void* q, const void* lmks, const int32_t* indices,
+                  void* dq, float* dlmk, int B, int L, int N, int h_kv, int G, int D, int topk,
+                  int per_qhead, float sm_scale, void* stream);
+
+/* ---- sparse attention over the selected chunks ------------------------------ */
+
+/* Forward.  Replaces hierarchical_sparse_attention_block_M_reuseIndices behind
+ * _hils_block_M_attention_inverse.forward (ops/hils_fwd_bwd_head.py:198-496, :771-860)
+ * and, with q_block > 1 / sm_n != 0 / mask_last == 0, _attn_fwd of ops/hsa_triton.py:77-197.
+ * q (B,L,HQ,D), k (B,Lkv,H,D), v (B,Lkv,H,Dv) bf16; weights (B,L/q_block,WH,NW) bf16
+ * with WH = HQ or H (first K of NW columns are read); indices (B,L/q_block,H,K) int32,
+ * < 0 = empty slot; slope (HQ) fp32 or NULL.
+ * Outputs: o (B,L,HQ,Dv) bf16; lse (B,L,HQ,K) fp32 per-chunk log2-domain LSE or NULL
+ * (-inf for empty slots). */
+int hils_sparse_attn_fwd(const void* q, const void* k, const void* v, const void* weights,
+                         const int32_t* indices, const float* slope, void* o, float* lse,
+                         int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
+                         int WH, int q_block, int S, float sm_scale, int mask_last, float sm_n,
+                         void* stream);
+
+/* Backward.  Replaces hierarchical_sparse_attention_bwd_dqkv_block_M_inverse
+ * (ops/hils_fwd_bwd_head.py:506-766) and kernel_attn_bwd_dq / _attn_bwd_dkdv /
+ * _fill_chunk_mask of ops/hsa_triton.py:201-597.
+ * d_o (B,L,HQ,Dv) bf16, lse from the forward.
+ * dq (B,L,HQ,D) bf16 (written); dk (B,Lkv,H,D) fp32, dv (B,Lkv,H,Dv) fp32 (ACCUMULATED
+ * with atomics: caller zero-fills); dw fp32 (B,L/q_block,WH,NW) (accumulated with
+ * atomics when q_block > 1 or WH != HQ, written otherwise: caller zero-fills). */
+int hils_sparse_attn_bwd(const void* q, const void* k, const void* v, const void* weights,
+                         const int32_t* indices, const float* slope, const float* lse,
+                         const void* d_o, void* dq, float* dk, float* dv, float* dw,
+                         int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
+                         int WH, int q_block, int S, float sm_scale, int mask_last, float sm_n,
+                         void* stream);
+
+/* ---- exact per-chunk log Z ---------------------------------------------------- */
+
+/* Forward.  Replaces exact_chunk_log_z_fwd (ops/exact_chunk_log_z_tilelang.py:25-137).
+ * q (B,L,HQ,D), k (B,L,H,D) bf16 -> log_z (B,L,HQ,ceil(L/S)) fp32, every element
+ * written (-inf where the chunk is not fully remote). */
+int hils_chunk_logz_fwd(const void* q, const void* k, float* log_z, int B, int L, int HQ, int H,
+                        int D, int S, int window, float sm_scale, int mask_lmk, void* stream);
+/* Backward w.r.t. q.  Replaces exact_chunk_log_z_bwd_dq (:148-262).  dq bf16 (written). */
+int hils_chunk_logz_bwd_dq(const void* q, const void* k, const float* log_z, const float* d_log_z,
+                           void* dq, int B, int L, int HQ, int H, int D, int S, int window,
+                           float sm_scale, void* stream);
+/* Backward w.r.t. k.  Replaces exact_chunk_log_z_bwd_dk (:273-391) and the GQA sum of
+ * :472-476.  dk bf16 (B,L,H,D) (written, already summed over the G heads). */
+int hils_chunk_logz_bwd_dk(const void* q, const void* k, const float* log_z, const float* d_log_z,
+                           void* dk, int B, int L, int HQ, int H, int D, int S, int window,
+                           float sm_scale, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

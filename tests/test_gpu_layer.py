@@ -1,0 +1,38 @@
+"""Whole HiLS layer forward (config 1: B1 L2048 h4/4 D64 chunk 64 top-8, causal) on the GPU
+vs the CPU oracle: mean-pooled chunk keys -> top-k -> inter-chunk softmax -> sparse attention."""
+import pytest
+import torch
+
+from util import assert_close_bf16, note
+
+pytestmark = pytest.mark.gpu
+
+
+def test_config1_layer_forward(pkg, orc, dev):
+    note("config 1 layer forward")
+    B, L, HQ, H, D, S, K, W = 1, 2048, 4, 4, 64, 64, 8, 1
+    gen = torch.Generator().manual_seed(1001)
+    q = torch.randn(B, L, HQ, D, generator=gen).bfloat16()
+    k = torch.randn(B, L, H, D, generator=gen).bfloat16()
+    v = torch.randn(B, L, H, D, generator=gen).bfloat16()
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    lmk = pkg.chunk_mean_pool(kd, S)
+    ref = orc.hils_layer_forward(q.float(), k.float(), v.float(), chunk_size=S, topk=K, window_size=W,
+                                 lmk_k=lmk.float().cpu())
+    dbg = {}
+    lse_swa = ref["lse_swa"].bfloat16()  # the layer hands lse_swa over in bf16
+    ref = orc.hils_layer_forward(q.float(), k.float(), v.float(), chunk_size=S, topk=K, window_size=W,
+                                 lmk_k=lmk.float().cpu())
+    idx, scores = pkg.online_softmax_topk_head(qd, lmk, lse_swa.to(dev), K, S, W, _debug=dbg)
+    lim = orc.causal_chunk_limit(L, 0, W, S)
+    sel_idx = orc.topk_select(dbg["sel_logits"].cpu(), dbg["lse_total"].cpu(), lim, K)
+    assert torch.equal(idx.cpu(), sel_idx), "indices not bit-exact from identical fp32 scores"
+    w = orc.inter_chunk_softmax(scores.float().cpu(), lse_swa.float()).bfloat16()
+    o_sparse = pkg.HiLS_block_M_head(qd, kd, vd, w.to(dev), idx, block_size=S, is_training=False)
+    o = torch.addcmul(o_sparse.float().cpu(), ref["swa_o"].bfloat16().float(), w[..., K].float().unsqueeze(-1))
+    # oracle on the kernel's own indices (near-tie flips against the fp32 oracle are allowed
+    # to differ, everything downstream of the indices must agree)
+    o_ref = orc.sparse_attn(q, k, v, w, idx.cpu(), chunk_size=S) + ref["swa_o"] * w[..., K].float().unsqueeze(-1)
+    assert_close_bf16(o, o_ref, "layer output")
+    agree = (idx.cpu() == ref["indices"]).float().mean().item()
+    assert agree > 0.97, f"index agreement with the fp32 oracle {agree:.4f}"

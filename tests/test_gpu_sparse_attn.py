@@ -1,0 +1,196 @@
+"""HIP sparse attention (forward + backward) vs the CPU oracle, through the C ABI."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from util import LSE_TOL, assert_close_bf16, assert_close_f32, note, rand_indices
+
+pytestmark = pytest.mark.gpu
+
+
+def make_case(B, L, HQ, H, D, Dv, K, S, seed=42, extra_w=1, fill_prob=1.0, Lkv=None):
+    gen = torch.Generator().manual_seed(seed)
+    Lkv = Lkv or L
+    q = (torch.randn(B, L, HQ, D, generator=gen)).bfloat16()
+    k = (torch.randn(B, Lkv, H, D, generator=gen)).bfloat16()
+    v = (torch.randn(B, Lkv, H, Dv, generator=gen)).bfloat16()
+    w = torch.softmax(torch.randn(B, L, HQ, K + extra_w, generator=gen), dim=-1).bfloat16()
+    idx = rand_indices(B, L, H, K, S, gen, causal=(Lkv == L), n_chunks=Lkv // S, fill_prob=fill_prob)
+    return q, k, v, w, idx
+
+
+def fwd_check(pkg, orc, dev, q, k, v, w, idx, S, **kw):
+    o = pkg.HiLS_block_M_head(q.to(dev), k.to(dev), v.to(dev), w.to(dev), idx.to(dev),
+                              block_size=S, is_training=False, **kw)
+    torch.cuda.synchronize()
+    okw = {}
+    if "sm_scale" in kw and kw["sm_scale"] is not None:
+        okw["sm_scale"] = kw["sm_scale"]
+    if "mask_last_token" in kw:
+        okw["mask_last_token"] = kw["mask_last_token"]
+    if kw.get("slope") is not None:
+        okw["slope"] = kw["slope"]
+    ref = orc.sparse_attn(q, k, v, w, idx, chunk_size=S, **okw)
+    assert o.dtype == torch.bfloat16
+    assert_close_bf16(o, ref, "o")
+    return o
+
+
+SHAPES = [
+    # B, L, HQ, H, D, Dv, K, S
+    (1, 1024, 8, 1, 64, 64, 4, 32),   # the reference's fp32 correctness shape (hils_fwd_bwd_head.py:1045-1053)
+    (2, 512, 4, 4, 64, 64, 8, 64),    # MHA, G = 1
+    (1, 512, 8, 2, 128, 128, 8, 64),  # GQA 4:1, D = 128
+    (1, 320, 16, 1, 64, 64, 4, 64),   # G = 16
+    (1, 256, 6, 2, 64, 128, 3, 64),   # G = 3, Dv != D, K not a power of two
+    (1, 200, 4, 2, 32, 32, 4, 16),    # ragged L, small chunks
+]
+
+
+@pytest.mark.parametrize("B,L,HQ,H,D,Dv,K,S", SHAPES)
+def test_sparse_attn_fwd(pkg, orc, dev, B, L, HQ, H, D, Dv, K, S):
+    note(f"sparse_attn_fwd B{B} L{L} HQ{HQ} H{H} D{D} Dv{Dv} K{K} S{S}")
+    q, k, v, w, idx = make_case(B, L, HQ, H, D, Dv, K, S)
+    fwd_check(pkg, orc, dev, q, k, v, w, idx, S)
+
+
+def test_sparse_attn_fwd_options(pkg, orc, dev):
+    q, k, v, w, idx = make_case(1, 384, 8, 2, 64, 64, 4, 64, seed=3, fill_prob=0.5)
+    note("sparse_attn options: partial fill / no mask / scale / slope")
+    fwd_check(pkg, orc, dev, q, k, v, w, idx, 64)
+    fwd_check(pkg, orc, dev, q, k, v, w, idx, 64, mask_last_token=False)
+    fwd_check(pkg, orc, dev, q, k, v, w, idx, 64, sm_scale=0.2)
+    fwd_check(pkg, orc, dev, q, k, v, w, idx, 64, slope=torch.rand(8) * 0.1)
+
+
+def test_sparse_attn_unsorted_and_empty(pkg, orc, dev):
+    """Unsorted index rows give the same result; all-empty rows give exact zeros."""
+    q, k, v, w, idx = make_case(1, 384, 4, 2, 64, 64, 4, 64, seed=4)
+    o1 = fwd_check(pkg, orc, dev, q, k, v, w, idx, 64)
+    perm = torch.tensor([2, 0, 3, 1])
+    w2 = w.clone()
+    w2[..., :4] = w[..., :4][..., perm]
+    o2 = fwd_check(pkg, orc, dev, q, k, v, w2, idx[..., perm].contiguous(), 64)
+    assert_close_bf16(o2, o1.float().cpu(), "permuted slots", max_abs=1e-2)
+    assert torch.count_nonzero(o1[0, :64]).item() == 0  # queries of chunk 0 see no chunk
+
+
+def test_sparse_attn_textbook_k1(pkg, dev):
+    """K = 1, w = 1: softmax(q K_c[:63]^T) V_c[:63] = F.scaled_dot_product_attention."""
+    torch.manual_seed(5)
+    B, L, H, D, S = 1, 256, 2, 64, 64
+    q = torch.randn(B, L, H, D).bfloat16()
+    k = torch.randn(B, L, H, D).bfloat16()
+    v = torch.randn(B, L, H, D).bfloat16()
+    idx = torch.full((B, L, H, 1), 1, dtype=torch.int32)
+    w = torch.ones(B, L, H, 1).bfloat16()
+    o = pkg.HiLS_block_M_head(q.to(dev), k.to(dev), v.to(dev), w.to(dev), idx.to(dev), is_training=False)
+    kc = k[:, 64:127].float().permute(0, 2, 1, 3)
+    vc = v[:, 64:127].float().permute(0, 2, 1, 3)
+    ref = F.scaled_dot_product_attention(q.float().permute(0, 2, 1, 3), kc, vc).permute(0, 2, 1, 3)
+    assert_close_bf16(o, ref, "K=1 textbook")
+
+
+def test_sparse_attn_linear_in_weights(pkg, dev):
+    q, k, v, w, idx = make_case(1, 256, 4, 2, 64, 64, 4, 64, seed=6)
+    args = (q.to(dev), k.to(dev), v.to(dev))
+    w1 = w.to(dev)
+    w2 = torch.softmax(torch.randn(w.shape), -1).bfloat16().to(dev)
+    o1 = pkg.HiLS_block_M_head(*args, w1, idx.to(dev), is_training=False).float()
+    o2 = pkg.HiLS_block_M_head(*args, w2, idx.to(dev), is_training=False).float()
+    o3 = pkg.HiLS_block_M_head(*args, ((w1.float() + w2.float()) / 2).bfloat16(), idx.to(dev),
+                               is_training=False).float()
+    assert_close_bf16(o3, (o1 + o2) / 2, "linearity", max_abs=2e-2)
+
+
+def test_sparse_attn_equals_dense_when_weights_are_chunk_masses(pkg, orc, dev):
+    """Select every causal chunk with w = softmax(log Z_c, lse_swa): the factorised form must
+    equal ordinary softmax attention over the kept tokens."""
+    torch.manual_seed(7)
+    B, L, HQ, H, D, S, W = 1, 512, 4, 2, 64, 64, 1
+    N = L // S
+    q = (torch.randn(B, L, HQ, D) * 0.5).bfloat16()
+    k = (torch.randn(B, L, H, D) * 0.5).bfloat16()
+    v = torch.randn(B, L, H, D).bfloat16()
+    lim = orc.causal_chunk_limit(L, 0, W, S)
+    idx = torch.arange(N).view(1, 1, 1, N).expand(B, L, H, N).clone()
+    idx = torch.where(idx < lim.view(1, L, 1, 1), idx, torch.full_like(idx, -1)).to(torch.int32)
+    log_z = orc.exact_chunk_log_z(q, k, chunk_size=S, window_size=W, mask_lmk=True)
+    swa_o, lse_swa = orc.swa(q, k, v, window_size=W, chunk_size=S, mask_lmk=True)
+    wts = torch.softmax(torch.cat([log_z, lse_swa.unsqueeze(-1)], -1), -1)
+    o_sparse = pkg.HiLS_block_M_head(q.to(dev), k.to(dev), v.to(dev), wts.bfloat16().to(dev),
+                                     idx.to(dev), is_training=False).float().cpu()
+    o = o_sparse + swa_o * wts[..., N].bfloat16().float().unsqueeze(-1)
+    dense, _ = orc.dense_hils_attention(q, k, v, chunk_size=S, window_size=W, indices=idx)
+    assert_close_bf16(o, dense, "factorised == dense", max_abs=2e-2, rel_l2=1.5e-2)
+
+
+def run_bwd(pkg, orc, dev, B, L, HQ, H, D, Dv, K, S, seed=42, **kw):
+    q, k, v, w, idx = make_case(B, L, HQ, H, D, Dv, K, S, seed=seed)
+    gen = torch.Generator().manual_seed(seed + 1)
+    do = torch.randn(B, L, HQ, Dv, generator=gen).bfloat16()
+    qd, kd, vd, wd = (t.to(dev).requires_grad_() for t in (q, k, v, w))
+    o = pkg.HiLS_block_M_head(qd, kd, vd, wd, idx.to(dev), block_size=S, is_training=True, **kw)
+    o.backward(do.to(dev))
+    torch.cuda.synchronize()
+    qf, kf, vf, wf = (t.float().requires_grad_() for t in (q, k, v, w))
+    okw = {kk: vv for kk, vv in kw.items() if kk in ("sm_scale", "mask_last_token", "slope")}
+    ref, lse_ref = orc.sparse_attn(qf, kf, vf, wf, idx, chunk_size=S, return_lse=True, **okw)
+    ref.backward(do.float())
+    assert_close_bf16(o, ref, "o")
+    assert_close_bf16(qd.grad, qf.grad, "dq")
+    assert_close_bf16(kd.grad, kf.grad, "dk")
+    assert_close_bf16(vd.grad, vf.grad, "dv")
+    # dw is defined for the first K columns of valid slots; everything else must be zero
+    valid = (idx >= 0).repeat_interleave(HQ // H, dim=2)
+    dw_ref = torch.zeros_like(wf.grad)
+    dw_ref[..., :K] = torch.where(valid, wf.grad[..., :K], torch.zeros(()))
+    assert wd.grad.dtype == torch.bfloat16
+    assert_close_bf16(wd.grad, dw_ref, "dw")
+
+
+BWD_SHAPES = [(1, 1024, 8, 1, 64, 64, 4, 32), (1, 384, 8, 2, 128, 128, 4, 64), (2, 256, 4, 4, 64, 64, 8, 64),
+              (1, 256, 6, 2, 64, 128, 3, 64)]
+
+
+@pytest.mark.parametrize("B,L,HQ,H,D,Dv,K,S", BWD_SHAPES)
+def test_sparse_attn_bwd(pkg, orc, dev, B, L, HQ, H, D, Dv, K, S):
+    note(f"sparse_attn_bwd B{B} L{L} HQ{HQ} H{H} D{D} Dv{Dv} K{K} S{S}")
+    run_bwd(pkg, orc, dev, B, L, HQ, H, D, Dv, K, S)
+
+
+def test_sparse_attn_bwd_options(pkg, orc, dev):
+    note("sparse_attn_bwd options")
+    run_bwd(pkg, orc, dev, 1, 256, 4, 2, 64, 64, 4, 64, seed=8, mask_last_token=False)
+    run_bwd(pkg, orc, dev, 1, 256, 4, 2, 64, 64, 4, 64, seed=9, slope=torch.rand(4) * 0.1, sm_scale=0.2)
+
+
+def test_sparse_attn_per_chunk_lse(pkg, orc, dev):
+    """The saved per-chunk LSE (log2 domain) equals logsumexp of the 63 masked logits."""
+    from hils_attention_amd.ops import _cabi
+    q, k, v, w, idx = make_case(1, 256, 4, 2, 64, 64, 4, 64, seed=10)
+    B, L, HQ, D = q.shape
+    o = torch.empty(B, L, HQ, 64, dtype=torch.bfloat16, device=dev)
+    lse = torch.empty(B, L, HQ, 4, dtype=torch.float32, device=dev)
+    t = [x.to(dev) for x in (q, k, v, w, idx)]
+    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(o), _cabi.ptr(lse),
+               B, L, L, HQ, 2, D, 64, 4, w.shape[-1], HQ, 1, 64, 1 / math.sqrt(D), 1, 0.0)
+    _, lse_ref = orc.sparse_attn(q, k, v, w, idx, chunk_size=64, return_lse=True)
+    assert_close_f32(lse.cpu() / 1.4426950408889634, lse_ref, LSE_TOL, "per-chunk LSE")
+
+
+def test_sparse_attn_inference_backward_raises(pkg, dev):
+    q, k, v, w, idx = make_case(1, 128, 4, 2, 64, 64, 2, 64)
+    qd = q.to(dev).requires_grad_()
+    o = pkg.HiLS_block_M_head(qd, k.to(dev), v.to(dev), w.to(dev), idx.to(dev), is_training=False)
+    with pytest.raises(RuntimeError):
+        o.sum().backward()
+
+
+def test_sparse_attn_decode_shape(pkg, orc, dev):
+    """One query per sequence against a long KV cache (decode)."""
+    note("sparse_attn decode B4 Lq1 Lkv4096")
+    q, k, v, w, idx = make_case(4, 1, 8, 2, 128, 128, 8, 64, seed=12, Lkv=4096)
+    fwd_check(pkg, orc, dev, q, k, v, w, idx, 64)

@@ -1,0 +1,209 @@
+"""HIP top-k chunk selection vs the CPU oracle, through the C ABI.
+
+Index parity is bit-exact: the kernel exports the fp32 selection logits and lse_total it
+selected from, and the oracle's selection rule applied to those must give identical
+indices.  The logits themselves (bf16 MFMA, fp32 accumulation) are checked against the
+oracle's fp32 einsum within 1e-3.  Shapes follow the reference's in-file tests
+(ops/topk_head_softmax.py:1807-1816, :2431-2479).
+"""
+import pytest
+import torch
+
+from util import assert_close_bf16, assert_close_f32, note
+
+pytestmark = pytest.mark.gpu
+
+
+def run_case(pkg, orc, dev, B, L, N, h_kv, G, D, topk, S, W, seed=42, q_offset=0, training=True,
+             use_bias=False, use_gumbel=False, use_drop=False, per_qhead=False, lse_mode="rand",
+             dup_keys=False, is_causal=True):
+    note(f"topk B{B} L{L} N{N} hkv{h_kv} G{G} D{D} k{topk} S{S} W{W} off{q_offset} "
+         f"bias{use_bias} gum{use_gumbel} drop{use_drop} pq{per_qhead} lse={lse_mode} dup{dup_keys}")
+    gen = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, L, h_kv, G, D, generator=gen).bfloat16()
+    lmk_h = h_kv * G if per_qhead else h_kv
+    lmks = torch.randn(B, N, lmk_h, D, generator=gen).bfloat16()
+    if dup_keys:  # identical chunk keys -> exact score ties
+        lmks[:, 1::2] = lmks[:, 0::2][:, : lmks[:, 1::2].shape[1]]
+    if lse_mode == "rand":
+        lse_swa = torch.randn(B, L, h_kv * G, generator=gen) * 5 + 10
+    elif lse_mode == "neginf":
+        lse_swa = torch.full((B, L, h_kv * G), float("-inf"))
+    else:
+        lse_swa = torch.zeros(B, L, h_kv * G)
+    bias = torch.randn(B, N, h_kv * G, generator=gen) if use_bias else None
+    gumbel = None
+    if use_gumbel:
+        u = torch.rand(1, 1, h_kv * G, N, generator=gen).clamp_(1e-20, 1 - 1e-7)
+        gumbel = -torch.log(-torch.log(u))
+    drop = (torch.rand(B, L, N, generator=gen) < 0.3).to(torch.int32) if use_drop else None
+    dbg = {}
+    q_in = q if not per_qhead else q
+    idx, scores = pkg.online_softmax_topk_head(
+        q_in.to(dev), lmks.to(dev), lse_swa.to(dev), topk, S, W, is_causal=is_causal,
+        q_offset=q_offset, is_training=training,
+        drop_mask=None if drop is None else drop.to(dev),
+        bias=None if bias is None else bias.to(dev),
+        gumbel_noise=None if gumbel is None else gumbel.to(dev),
+        G=G if per_qhead else 1, _debug=dbg)
+    torch.cuda.synchronize()
+    assert idx.dtype == torch.int32 and idx.shape == (B, L, h_kv, topk)
+    assert scores.dtype == torch.bfloat16 and scores.shape == (B, L, h_kv * G, topk)
+    eff_off = 0 if training else q_offset
+    ridx, rscores, aux = orc.online_softmax_topk_head(
+        q, lmks, lse_swa, topk, S, W, is_causal=is_causal, q_offset=eff_off, drop_mask=drop,
+        bias=bias, gumbel_noise=gumbel, return_aux=True)
+    sel = dbg["sel_logits"].cpu()
+    lt = dbg["lse_total"].cpu()
+    # 1. fp32 logits and LSE against the oracle's fp32 arithmetic
+    assert_close_f32(sel, aux["sel_logits"], 2e-3, "selection logits")
+    assert_close_f32(lt, aux["lse_total"], 1e-3, "lse_total")
+    # 2. bit-exact selection from identical fp32 scores
+    lim = aux["limit"]
+    idx_from_kernel_scores = orc.topk_select(sel, lt, lim, topk, drop)
+    assert torch.equal(idx.cpu(), idx_from_kernel_scores), "indices not bit-exact"
+    # 3. invariants: ascending, -1 tail, visible only, count
+    ic = idx.cpu().long()
+    valid = ic >= 0
+    srt = torch.where(valid, ic, torch.full_like(ic, 1 << 30))
+    assert torch.all(srt[..., 1:] >= srt[..., :-1])
+    assert torch.all((srt[..., 1:] > srt[..., :-1]) | ~valid[..., 1:])
+    if lim is not None:
+        assert torch.all(~valid | (ic < lim.view(1, L, 1, 1)))
+        cnt = torch.minimum(lim.clamp_min(0), torch.tensor(topk)).view(1, L, 1)
+        if drop is None:
+            assert torch.equal(valid.sum(-1), cnt.expand(B, L, h_kv))
+    # 4. agreement with the oracle's own indices (its logits differ in the last bits, so
+    #    near-ties may flip: require >= 99 %, the reference's own bar)
+    match = (idx.cpu() == ridx).float().mean().item()
+    assert match >= 0.99, f"index agreement with the fp32 oracle only {match:.4f}"
+    # 5. scores: raw scaled qk at the kernel's indices
+    safe = ic.clamp_min(0).unsqueeze(3).expand(-1, -1, -1, G, -1)
+    want = torch.gather(aux["logits"], -1, safe).masked_fill(~valid.unsqueeze(3).expand(-1, -1, -1, G, -1),
+                                                              float("-inf"))
+    assert_close_bf16(scores.view(B, L, h_kv, G, topk), want, "scores")
+    return idx, scores
+
+
+def test_topk_reference_shape(pkg, orc, dev):
+    # (B, L, S_chunks...) of test_topk_correctness_robust, reduced L for CPU oracle time
+    run_case(pkg, orc, dev, B=2, L=1024, N=16, h_kv=2, G=8, D=64, topk=16, S=64, W=64)
+
+
+@pytest.mark.parametrize("G,D", [(1, 64), (2, 128), (4, 128), (8, 64), (16, 64), (3, 64)])
+def test_topk_group_sizes(pkg, orc, dev, G, D):
+    run_case(pkg, orc, dev, B=1, L=640, N=10, h_kv=2, G=G, D=D, topk=4, S=64, W=1)
+
+
+@pytest.mark.parametrize("L", [999, 1023, 1100, 17])
+def test_topk_ragged_lengths(pkg, orc, dev, L):
+    run_case(pkg, orc, dev, B=1, L=L, N=(L + 63) // 64, h_kv=2, G=4, D=64, topk=8, S=64, W=32)
+
+
+def test_topk_window_zero_and_noncausal(pkg, orc, dev):
+    run_case(pkg, orc, dev, B=1, L=512, N=8, h_kv=1, G=4, D=64, topk=4, S=64, W=0)
+    run_case(pkg, orc, dev, B=1, L=96, N=24, h_kv=2, G=2, D=64, topk=8, S=64, W=0, is_causal=False)
+
+
+def test_topk_bias_gumbel_drop(pkg, orc, dev):
+    run_case(pkg, orc, dev, B=2, L=512, N=8, h_kv=2, G=4, D=64, topk=4, S=64, W=16, use_bias=True)
+    run_case(pkg, orc, dev, B=1, L=512, N=8, h_kv=2, G=4, D=64, topk=4, S=64, W=16, use_gumbel=True)
+    run_case(pkg, orc, dev, B=1, L=512, N=8, h_kv=2, G=4, D=64, topk=4, S=64, W=16, use_drop=True)
+    run_case(pkg, orc, dev, B=1, L=512, N=8, h_kv=2, G=2, D=128, topk=4, S=64, W=16, use_bias=True,
+             use_gumbel=True, use_drop=True)
+
+
+def test_topk_per_qhead_lmks(pkg, orc, dev):
+    run_case(pkg, orc, dev, B=1, L=512, N=8, h_kv=2, G=4, D=64, topk=4, S=64, W=1, per_qhead=True)
+    run_case(pkg, orc, dev, B=1, L=300, N=5, h_kv=1, G=2, D=128, topk=8, S=64, W=1, per_qhead=True,
+             use_bias=True)
+
+
+def test_topk_chunked_prefill_and_decode(pkg, orc, dev):
+    # chunked prefill: q_offset=1024; decode: q_len=1, kv=2049 (reference :2431-2479)
+    run_case(pkg, orc, dev, B=1, L=256, N=20, h_kv=2, G=4, D=64, topk=8, S=64, W=64, q_offset=1024,
+             training=False)
+    run_case(pkg, orc, dev, B=2, L=1, N=32, h_kv=2, G=4, D=128, topk=8, S=64, W=64, q_offset=2048,
+             training=False)
+
+
+def test_topk_many_chunks_multi_segment(pkg, orc, dev):
+    # more chunks than one LDS selection segment (512): exercises the candidate carry-over
+    run_case(pkg, orc, dev, B=1, L=2, N=1500, h_kv=2, G=4, D=64, topk=32, S=64, W=1,
+             q_offset=1500 * 64, training=False)
+    run_case(pkg, orc, dev, B=1, L=1, N=2048, h_kv=1, G=4, D=128, topk=64, S=64, W=1,
+             q_offset=2048 * 64, training=False, dup_keys=True)
+
+
+def test_topk_tie_break_lower_index_wins(pkg, orc, dev):
+    """Duplicated chunk keys give exactly equal scores; the lower index must win."""
+    idx, _ = run_case(pkg, orc, dev, B=1, L=1024, N=16, h_kv=1, G=1, D=64, topk=3, S=64, W=1,
+                      dup_keys=True, lse_mode="neginf")
+    # with pairs (2j, 2j+1) identical and an odd k, whenever exactly one member of a pair is
+    # selected it must be the even (lower) one
+    ic = idx.cpu().long()
+    for t in range(128, 1024, 37):
+        sel = set(ic[0, t, 0][ic[0, t, 0] >= 0].tolist())
+        for c in sel:
+            if c % 2 == 1:
+                assert (c - 1) in sel, f"t={t}: chunk {c} chosen without its identical twin {c - 1}"
+
+
+def test_topk_reduces_to_torch_topk(pkg, orc, dev):
+    """lse_swa = -inf and G = 1: the selection is plain top-k of the logits."""
+    B, L, N, D, topk, S = 1, 768, 12, 64, 4, 64
+    torch.manual_seed(9)
+    q = torch.randn(B, L, 1, D).bfloat16()
+    lmks = torch.randn(B, N, 1, D).bfloat16()
+    lse = torch.full((B, L, 1), float("-inf"))
+    dbg = {}
+    idx, _ = pkg.online_softmax_topk_head(q.to(dev), lmks.to(dev), lse.to(dev), topk, S, 1, _debug=dbg)
+    sel = dbg["sel_logits"].cpu().view(B, L, N)
+    for t in range(0, L, 13):
+        nv = t // S
+        got = [c for c in idx[0, t, 0].cpu().tolist() if c >= 0]
+        assert len(got) == min(topk, nv)
+        if nv > 0:
+            want = torch.topk(sel[0, t, :nv], min(topk, nv)).indices.sort().values.tolist()
+            assert got == want
+
+
+def test_topk_backward(pkg, orc, dev):
+    B, L, N, h_kv, G, D, topk, S = 1, 512, 8, 2, 4, 64, 4, 64
+    note("topk backward")
+    torch.manual_seed(11)
+    for per_qhead in (False, True):
+        q = torch.randn(B, L, h_kv * G, D).bfloat16()
+        lmks = torch.randn(B, N, h_kv * G if per_qhead else h_kv, D).bfloat16()
+        lse = torch.randn(B, L, h_kv * G)
+        gs = torch.randn(B, L, h_kv * G, topk).bfloat16()
+        q_d = q.to(dev).requires_grad_()
+        l_d = lmks.to(dev).requires_grad_()
+        idx, scores = pkg.online_softmax_topk_head(q_d, l_d, lse.to(dev), topk, S, 1,
+                                                   G=G if per_qhead else 1)
+        valid = (idx >= 0).repeat_interleave(G, dim=2)
+        gs_d = torch.where(valid, gs.to(dev), torch.zeros_like(gs.to(dev)))
+        scores.backward(gs_d)
+        # oracle: autograd through a gather of the fp32 logits at the same indices
+        q_f = q.float().view(B, L, h_kv, G, D).requires_grad_()
+        l_f = lmks.float().requires_grad_()
+        logits = orc.topk_logits(q_f, l_f)
+        ic = idx.cpu().long()
+        safe = ic.clamp_min(0).unsqueeze(3).expand(-1, -1, -1, G, -1)
+        picked = torch.gather(logits, -1, safe)
+        g_ref = gs_d.float().cpu().view(B, L, h_kv, G, topk)
+        (picked * g_ref).sum().backward()
+        assert_close_bf16(q_d.grad.view(B, L, h_kv, G, D), q_f.grad, f"dq pq={per_qhead}")
+        assert_close_bf16(l_d.grad, l_f.grad, f"dlmk pq={per_qhead}")
+
+
+def test_topk_argument_errors(pkg, dev):
+    q = torch.randn(1, 64, 4, 64, device=dev).bfloat16()
+    lmks = torch.randn(1, 1, 3, 64, device=dev).bfloat16()
+    lse = torch.zeros(1, 64, 4, device=dev)
+    with pytest.raises(AssertionError):
+        pkg.online_softmax_topk_head(q, lmks, lse, 4, 64, 1)
+    with pytest.raises(TypeError):
+        pkg.online_softmax_topk_head(q.float(), lmks[:, :, :2].float(), lse, 4, 64, 1)
+    with pytest.raises(RuntimeError):
+        pkg.online_softmax_topk_head(q, lmks[:, :, :2], lse, 100, 64, 1)
