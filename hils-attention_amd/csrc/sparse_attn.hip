@@ -11,6 +11,14 @@
 #define SA_THREADS 256
 #define SA_MAX_OUT 16  // outputs (g, dv) per thread
 
+size_t hils_ga_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S,
+                               int q_block, int WH, float sm_n);
+int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const void* weights,
+                              const int32_t* indices, const float* slope, void* o, float* lse,
+                              void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ,
+                              int H, int D, int Dv, int K, int NW, int S, float sm_scale,
+                              int mask_last, void* stream, int* handled);
+
 struct SaDims {
   int L, Lkv, HQ, H, G, D, Dv, K, NW, WH, q_block, S, mask_last;
   float sm_scale, sm_n;
@@ -259,14 +267,31 @@ static int sa_check(const char* name, int B, int L, int Lkv, int HQ, int H, int 
   return HILS_OK;
 }
 
+extern "C" size_t hils_sparse_attn_fwd_workspace(int B, int L, int Lkv, int HQ, int H, int D,
+                                                 int Dv, int K, int WH, int q_block, int S,
+                                                 float sm_n) {
+  return hils_ga_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n);
+}
+
 extern "C" int hils_sparse_attn_fwd(const void* q, const void* k, const void* v,
                                     const void* weights, const int32_t* indices,
-                                    const float* slope, void* o, float* lse, int B, int L, int Lkv,
-                                    int HQ, int H, int D, int Dv, int K, int NW, int WH,
-                                    int q_block, int S, float sm_scale, int mask_last, float sm_n,
-                                    void* stream) {
+                                    const float* slope, void* o, float* lse, void* workspace,
+                                    int workspace_ready, int B, int L, int Lkv, int HQ, int H,
+                                    int D, int Dv, int K, int NW, int WH, int q_block, int S,
+                                    float sm_scale, int mask_last, float sm_n, void* stream) {
   HILS_REQUIRE(q && k && v && weights && indices && o, "hils_sparse_attn_fwd: null pointer");
   if (int rc = sa_check("hils_sparse_attn_fwd", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
+  if (workspace && hils_ga_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n) > 0) {
+    int handled = 0;
+    if (int rc = hils_sparse_attn_fwd_mfma(q, k, v, weights, indices, slope, o, lse, workspace,
+                                           workspace_ready, B, L, Lkv, HQ, H, D, Dv, K, NW, S,
+                                           sm_scale, mask_last, stream, &handled))
+      return rc;
+    if (handled) {
+      HILS_CHECK_LAUNCH("hils_sparse_attn_fwd");
+      return HILS_OK;
+    }
+  }
   SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n};
   size_t smem = ((size_t)dm.G * D + (size_t)dm.G * S + 2 * dm.G) * sizeof(float);
   HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_fwd: G*(D+S) too large for LDS");

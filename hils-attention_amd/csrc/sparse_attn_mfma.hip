@@ -1,0 +1,453 @@
+// Sparse attention forward on bf16 MFMA for prefill-sized query counts.
+//
+// The work is regrouped by chunk, not by query.  One workgroup owns T consecutive queries
+// of one (batch, KV head).  It sorts the T*K (query, slot) pairs by chunk index in LDS, so
+// that all queries of the block that selected chunk c sit next to each other ("a visit").
+// A wavefront takes up to 16/G queries of a visit (16 rows: queries x the G heads of the
+// KV head), loads the chunk's K rows and the gathered query rows straight into MFMA
+// operands, forms S^T = K Q^T (tokens x rows) with 16x16x32 MFMAs, does the per-chunk
+// softmax along the accumulator registers, and feeds P back as the A operand of
+// O = P V without leaving registers (the contraction order over tokens is permuted to
+// the accumulator layout; V is pre-transposed per chunk in the same order).  The
+// (rows x Dv) partial outputs are summed into an fp32 output tile in LDS with LDS
+// atomics, which is what lets rows of different visits be arbitrary subsets of the block.
+#include "common.h"
+#include "../../include/hils_amd.h"
+
+#define GA_THREADS 512
+#define GA_WAVES (GA_THREADS / 64)
+#define GA_S 64                 // chunk size this kernel is built for
+#define GA_KEY_INVALID 0xFFFFFFFFu
+#define GA_PAIR_BITS 12
+
+// ---------------------------------------------------------------------------
+// V pre-transpose: vt[b][h][c][dv][p] with token(p) = 32*(p/32) + 16*((p%8)/4) + 4*((p%32)/8) + p%4,
+// the order in which a 16x16x32 MFMA B operand wants the tokens of an accumulator-layout P.
+// Also records max|V| of every chunk (it bounds the fixed-point output accumulation).
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+transpose_v_kernel(const bf16_t* __restrict__ v, bf16_t* __restrict__ vt, float* __restrict__ vmax,
+                   int Lkv, int H, int Dv, int nchunk) {
+  extern __shared__ bf16_t tile[];  // 64 x (Dv + 2)
+  __shared__ float red[32];
+  const int c = blockIdx.x, h = blockIdx.y;
+  const long b = blockIdx.z;
+  const int DP = Dv + 2;
+  const int d8n = Dv / 8;
+  float mx = 0.f;
+  for (int i = threadIdx.x; i < GA_S * d8n; i += 256) {
+    const int s = i / d8n, d8 = i - s * d8n;
+    uint4 x = *(const uint4*)(v + ((b * Lkv + (long)c * GA_S + s) * H + h) * Dv + d8 * 8);
+    const bf16_t* xs = (const bf16_t*)&x;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      tile[s * DP + d8 * 8 + e] = xs[e];
+      mx = fmaxf(mx, fabsf(bf2f(xs[e])));
+    }
+  }
+  mx = block_max(mx, red);  // contains the barrier that orders the tile writes
+  if (threadIdx.x == 0) vmax[(b * H + h) * (long)nchunk + c] = mx;
+  bf16_t* out = vt + (((b * H + h) * (long)nchunk + c) * Dv) * GA_S;
+  for (int i = threadIdx.x; i < Dv * 8; i += 256) {
+    const int dv = i >> 3, p8 = i & 7;  // 8 positions p8*8 .. p8*8+7
+    bf16_t y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int p = p8 * 8 + e;
+      const int tok = 32 * (p >> 5) + 16 * ((p & 7) >> 2) + 4 * ((p & 31) >> 3) + (p & 3);
+      y[e] = tile[tok * DP + dv];
+    }
+    *(uint4*)(out + (long)dv * GA_S + p8 * 8) = *(uint4*)y;
+  }
+}
+
+struct GaDims {
+  int L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last;
+  float sm_scale;
+};
+
+// Output tiles are accumulated in LDS as 32-bit fixed point: integer LDS atomics run at
+// full rate on this hardware (float LDS atomics do not), and integer addition is
+// associative, so the result does not depend on the order in which wavefronts add.
+// The scale is chosen per workgroup from bound = max_row(sum_k |w|) * max_visited|V|, which
+// bounds every output element because each P row is a convex combination.
+template <int D, int DV, int G>
+__global__ void __launch_bounds__(GA_THREADS)
+sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                       const bf16_t* __restrict__ vt, const float* __restrict__ vmax,
+                       const bf16_t* __restrict__ weights, const int32_t* __restrict__ indices,
+                       const float* __restrict__ slope, bf16_t* __restrict__ o,
+                       float* __restrict__ lse, GaDims dm) {
+  constexpr int KS = D / 32;    // k-steps of S^T = K Q^T
+  constexpr int DT = DV / 16;   // 16-wide output column tiles
+  constexpr int QT = 16 / G;    // queries per 16-row tile
+  constexpr int MAXP = 8;       // pairs per thread: T*K <= MAXP * GA_THREADS
+  extern __shared__ int smem_i[];
+  const int R = dm.T * G;
+  int* o_acc = smem_i;                       // R x DV fixed point
+  int* cur = o_acc + (size_t)R * DV;         // nchunk: histogram -> running ends
+  int* pairs = cur + dm.nchunk;              // T*K pair ids grouped by chunk
+  __shared__ float red[32];
+  __shared__ int scan_s[GA_WAVES];
+  __shared__ int next_s;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  // XCD-aware order: hardware hands consecutive workgroup ids to the 8 XCDs in turn, so
+  // id -> (xcd, slot); each XCD walks one contiguous share of the (batch, head, block)
+  // list, latest query blocks first, and its L2 sees one head's K/V at a time.
+  const int total = dm.nblk * dm.H * dm.B;
+  const int per_xcd = (total + 7) / 8;
+  const int vid = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+  if (vid >= total) return;
+  const int unit = vid / dm.nblk;
+  const int blk = dm.nblk - 1 - (vid - unit * dm.nblk);
+  const int hk = unit % dm.H;
+  const long b = unit / dm.H;
+  const int t0 = blk * dm.T;
+  const int K = dm.K;
+  const int npair = dm.T * K;
+
+  for (int i = tid; i < R * DV; i += GA_THREADS) o_acc[i] = 0;
+  for (int i = tid; i < dm.nchunk; i += GA_THREADS) cur[i] = 0;
+  if (tid == 0) next_s = 0;
+  __syncthreads();
+  // histogram of the selected chunks
+  int creg[MAXP];
+#pragma unroll
+  for (int e = 0; e < MAXP; ++e) {
+    const int i = tid + e * GA_THREADS;
+    int c = -1;
+    if (i < npair) {
+      const int ql = i / K, slot = i - ql * K;
+      const int t = t0 + ql;
+      if (t < dm.L) {
+        c = indices[((b * dm.L + t) * dm.H + hk) * (long)K + slot];
+        if (c < 0 || c >= dm.nchunk) {
+          c = -1;
+          if (lse) {
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+              lse[((b * dm.L + t) * dm.HQ + hk * G + g) * (long)K + slot] = HILS_NEG_INF;
+          }
+        }
+      }
+    }
+    creg[e] = c;
+    if (c >= 0) atomicAdd(&cur[c], 1);
+  }
+  // bound for the fixed-point scale: rows' sum of |w| ...
+  float wsum = 0.f;
+  for (int row = tid; row < R; row += GA_THREADS) {
+    const int ql = row / G, g = row - ql * G;
+    const int t = t0 + ql;
+    if (t < dm.L) {
+      const bf16_t* wr = weights + ((b * dm.L + t) * (long)dm.HQ + hk * G + g) * dm.NW;
+      float a = 0.f;
+      for (int s2 = 0; s2 < K; ++s2) a += fabsf(bf2f(wr[s2]));
+      wsum = fmaxf(wsum, a);
+    }
+  }
+  wsum = block_max(wsum, red);  // barrier: histogram complete
+  // ... times max |V| over the visited chunks; exclusive scan of the histogram on the way
+  float vm = 0.f;
+  const int per_thr = (dm.nchunk + GA_THREADS - 1) / GA_THREADS;
+  const int c_lo = tid * per_thr;
+  int local = 0;
+  for (int c = c_lo; c < c_lo + per_thr && c < dm.nchunk; ++c) {
+    const int h = cur[c];
+    if (h > 0) vm = fmaxf(vm, vmax[(b * dm.H + hk) * (long)dm.nchunk + c]);
+    local += h;
+  }
+  int incl = local;
+#pragma unroll
+  for (int o2 = 1; o2 < 64; o2 <<= 1) {
+    const int x = __shfl_up(incl, o2, 64);
+    if (lane >= o2) incl += x;
+  }
+  if (lane == 63) scan_s[wave] = incl;
+  vm = block_max(vm, red);  // barrier: scan_s visible, all histogram reads done
+  int base = incl - local;
+  for (int w2 = 0; w2 < wave; ++w2) base += scan_s[w2];
+  for (int c = c_lo; c < c_lo + per_thr && c < dm.nchunk; ++c) {
+    const int h = cur[c];
+    cur[c] = base;
+    base += h;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < MAXP; ++e)
+    if (creg[e] >= 0) pairs[atomicAdd(&cur[creg[e]], 1)] = tid + e * GA_THREADS;
+  __syncthreads();  // now chunk c owns pairs[cur[c-1] .. cur[c])
+
+  const float bound = wsum * vm;
+  float fx_scale = 1.f;
+  if (bound > 0.f && bound < 3.0e38f) fx_scale = ldexpf(1.f, 28 - ilogbf(bound));
+  const float fx_inv = 1.f / fx_scale;
+  const float c2 = dm.sm_scale * HILS_LOG2E;
+  const int qs = r / G, g = r - qs * G;
+  const int hq = hk * G + g;
+  const float sl = slope ? slope[hq] : 0.f;
+
+  for (;;) {
+    int c = 0;
+    if (lane == 0) c = atomicAdd(&next_s, 1);
+    c = __shfl(c, 0, 64);
+    if (c >= dm.nchunk) break;
+    const int vs = c ? cur[c - 1] : 0, ve = cur[c];
+    if (vs == ve) continue;
+
+    // the chunk's K rows (A operands of S^T = K Q^T) and transposed V (B operands of P V)
+    bf16x8_t ka[4][KS], vb[DT][2];
+    {
+      const bf16_t* kbase = k + ((b * dm.Lkv + (long)c * GA_S + r) * dm.H + hk) * D + j * 8;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const uint4 x = *(const uint4*)(kbase + (long)mt * 16 * dm.H * D + ks * 32);
+          ka[mt][ks] = *(const bf16x8_t*)&x;
+        }
+      const bf16_t* vbase = vt + ((((b * dm.H + hk) * (long)dm.nchunk + c) * DV + r) * GA_S) + j * 8;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          const uint4 x = *(const uint4*)(vbase + (long)dt * 16 * GA_S + s * 32);
+          vb[dt][s] = *(const bf16x8_t*)&x;
+        }
+    }
+
+    for (int p = vs; p < ve; p += QT) {
+      const int n = (ve - p < QT) ? ve - p : QT;
+      // this lane's row of the tile: query slot r / G, head r % G
+      const bool rvalid = qs < n;
+      const int pid = pairs[p + (rvalid ? qs : 0)];
+      const int ql = pid / K, slot = pid - ql * K;
+      const int t = t0 + ql;
+      const int row_base = (ql * G + g) * DV;
+
+      bf16x8_t bq[KS];
+      const bf16_t* qrow = q + ((b * dm.L + t) * (long)dm.HQ + hq) * D + j * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        uint4 x = make_uint4(0, 0, 0, 0);
+        if (rvalid) x = *(const uint4*)(qrow + ks * 32);
+        bq[ks] = *(bf16x8_t*)&x;
+      }
+      float wr = 0.f;
+      if (rvalid) wr = bf2f(weights[((b * dm.L + t) * (long)dm.HQ + hq) * dm.NW + slot]);
+      f32x4_t st[4];
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        st[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          st[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[mt][ks], bq[ks], st[mt], 0, 0, 0);
+      }
+      // per-chunk softmax over the 64 tokens of row r: registers (mt, i) and lane groups j
+      float m = HILS_NEG_INF;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tok = mt * 16 + j * 4 + i;
+          float x = st[mt][i];
+          if (slope) {
+            const int dist = GA_S - 2 - tok;
+            x -= sl * (float)(dist > 0 ? dist : 0);
+          }
+          if (dm.mask_last && tok == GA_S - 1) x = HILS_NEG_INF;
+          st[mt][i] = x;
+          m = fmaxf(m, x);
+        }
+      m = fmaxf(m, __shfl_xor(m, 16, 64));
+      m = fmaxf(m, __shfl_xor(m, 32, 64));
+      const float mc = m * c2;
+      float sum = 0.f;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float e = __builtin_amdgcn_exp2f(st[mt][i] * c2 - mc);
+          st[mt][i] = e;
+          sum += e;
+        }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      if (lse && rvalid && j == 0)
+        lse[((b * dm.L + t) * (long)dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
+      const float f = wr / sum;
+      // P as the A operand of O = P V: k-step s takes tokens of accumulator tiles 2s, 2s+1
+      bf16x8_t ap[2];
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        uint4 x;
+        x.x = pack_bf2(st[2 * s][0] * f, st[2 * s][1] * f);
+        x.y = pack_bf2(st[2 * s][2] * f, st[2 * s][3] * f);
+        x.z = pack_bf2(st[2 * s + 1][0] * f, st[2 * s + 1][1] * f);
+        x.w = pack_bf2(st[2 * s + 1][2] * f, st[2 * s + 1][3] * f);
+        ap[s] = *(bf16x8_t*)&x;
+      }
+      // rows 4j+i of an output tile belong to the lanes with (lane & 15) == 4j+i
+      int rb[4];
+      bool rv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        rb[i] = __shfl(row_base, 4 * j + i, 64);
+        rv[i] = ((4 * j + i) / G) < n;
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s], vb[dt][s], acc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (rv[i]) atomicAdd(&o_acc[rb[i] + dt * 16 + r], __float2int_rn(acc[i] * fx_scale));
+      }
+    }
+  }
+  __syncthreads();
+  constexpr int C8 = DV / 8;
+  for (int i = tid; i < R * C8; i += GA_THREADS) {
+    const int row = i / C8, c8 = i - row * C8;
+    const int ql = row / G, g2 = row - ql * G;
+    const int t = t0 + ql;
+    if (t < dm.L) {
+      const int* src = o_acc + (size_t)row * DV + c8 * 8;
+      uint4 x;
+      x.x = pack_bf2((float)src[0] * fx_inv, (float)src[1] * fx_inv);
+      x.y = pack_bf2((float)src[2] * fx_inv, (float)src[3] * fx_inv);
+      x.z = pack_bf2((float)src[4] * fx_inv, (float)src[5] * fx_inv);
+      x.w = pack_bf2((float)src[6] * fx_inv, (float)src[7] * fx_inv);
+      *(uint4*)(o + ((b * dm.L + t) * (long)dm.HQ + hk * G + g2) * DV + c8 * 8) = x;
+    }
+  }
+}
+
+template <int D, int DV, int G>
+static int ga_launch(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, const bf16_t* k,
+                     const bf16_t* vt, const float* vmax, const bf16_t* w, const int32_t* idx,
+                     const float* slope, bf16_t* o, float* lse, const GaDims& dm) {
+  auto kern = sparse_attn_fwd_gather<D, DV, G>;
+  static size_t reserved = 0;  // per instantiation
+  if (smem > reserved) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem) != hipSuccess) {
+      hils_set_error("hils_sparse_attn_fwd: cannot reserve %zu bytes of LDS", smem);
+      return HILS_ERR_LAUNCH;
+    }
+    reserved = smem;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(GA_THREADS), smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
+  return HILS_OK;
+}
+
+template <int D, int DV>
+static int ga_dispatch_g(int G, dim3 grid, size_t smem, hipStream_t st, const bf16_t* q,
+                         const bf16_t* k, const bf16_t* vt, const float* vmax, const bf16_t* w,
+                         const int32_t* idx, const float* slope, bf16_t* o, float* lse,
+                         const GaDims& dm) {
+  switch (G) {
+    case 1: return ga_launch<D, DV, 1>(grid, smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
+    case 2: return ga_launch<D, DV, 2>(grid, smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
+    case 4: return ga_launch<D, DV, 4>(grid, smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
+    case 8: return ga_launch<D, DV, 8>(grid, smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
+    case 16: return ga_launch<D, DV, 16>(grid, smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
+  }
+  return -1;
+}
+
+static size_t ga_vt_bytes(int B, int H, int nchunk, int Dv) {
+  size_t n = (size_t)B * H * nchunk * Dv * GA_S * sizeof(bf16_t);
+  return (n + 255) & ~(size_t)255;
+}
+
+// Tile sizes: T queries per workgroup such that the fixed-point output tile, the chunk
+// histogram and the pair list fit in LDS.  Returns 0 when the shape does not fit.
+static int ga_pick_T(int L, int G, int Dv, int K, int nchunk, size_t* smem_out) {
+  int T = (128 * 1024) / (G * Dv * 4);
+  if (T * K > 8 * GA_THREADS) T = (8 * GA_THREADS) / K;
+  if (T > L) T = L;
+  while (T >= 1) {
+    const size_t smem = (size_t)T * G * Dv * 4 + (size_t)nchunk * 4 + (size_t)T * K * 4;
+    if (smem <= 156 * 1024) {
+      *smem_out = smem;
+      return T;
+    }
+    T /= 2;
+  }
+  return 0;
+}
+
+// Workspace the MFMA path needs (the per-chunk transposed copy of V and the per-chunk max|V|),
+// 0 if the shape is not covered by it.
+size_t hils_ga_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S,
+                               int q_block, int WH, float sm_n) {
+  if (H <= 0 || HQ % H != 0) return 0;
+  const int G = HQ / H;
+  const bool ok = S == GA_S && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) &&
+                  (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) && q_block == 1 && WH == HQ &&
+                  sm_n == 0.f && L >= 64 && Lkv >= S;
+  if (!ok) return 0;
+  size_t smem;
+  if (ga_pick_T(L, G, Dv, K, Lkv / S, &smem) == 0) return 0;
+  const int nchunk = Lkv / S;
+  return ga_vt_bytes(B, H, nchunk, Dv) + (size_t)B * H * nchunk * sizeof(float);
+}
+
+// Returns HILS_OK and sets *handled = 1 when the MFMA path ran.
+int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const void* weights,
+                              const int32_t* indices, const float* slope, void* o, float* lse,
+                              void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ,
+                              int H, int D, int Dv, int K, int NW, int S, float sm_scale,
+                              int mask_last, void* stream, int* handled) {
+  *handled = 0;
+  const int G = HQ / H;
+  const int nchunk = Lkv / S;
+  hipStream_t st = (hipStream_t)stream;
+  size_t smem;
+  const int T = ga_pick_T(L, G, Dv, K, nchunk, &smem);
+  if (T == 0 || H > 65535 || B > 65535) return HILS_OK;
+  const int nblk = (L + T - 1) / T;
+  const long total = (long)nblk * H * B;
+  if (total > (1L << 30)) return HILS_OK;
+  bf16_t* vt = (bf16_t*)workspace;
+  float* vmax = (float*)((char*)workspace + ga_vt_bytes(B, H, nchunk, Dv));
+  if (!workspace_ready)
+    hipLaunchKernelGGL(transpose_v_kernel, dim3(nchunk, H, B), dim3(256),
+                       (size_t)GA_S * (Dv + 2) * sizeof(bf16_t), st, (const bf16_t*)v, vt, vmax,
+                       Lkv, H, Dv, nchunk);
+  GaDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale};
+  const long per_xcd = (total + 7) / 8;
+  dim3 grid((unsigned)(per_xcd * 8));
+  int rc = -1;
+#define GA_CALL(D_, DV_)                                                                       \
+  rc = ga_dispatch_g<D_, DV_>(G, grid, smem, st, (const bf16_t*)q, (const bf16_t*)k, vt, vmax, \
+                              (const bf16_t*)weights, indices, slope, (bf16_t*)o, lse, dm)
+  if (D == 64 && Dv == 64) GA_CALL(64, 64);
+  else if (D == 128 && Dv == 128) GA_CALL(128, 128);
+  else if (D == 64 && Dv == 128) GA_CALL(64, 128);
+  else if (D == 128 && Dv == 64) GA_CALL(128, 64);
+#undef GA_CALL
+  if (rc != HILS_OK) return rc < 0 ? HILS_OK : rc;
+  *handled = 1;
+  return HILS_OK;
+}
+
+extern "C" int hils_transpose_v_chunks(const void* v, void* vt, int B, int Lkv, int H, int Dv,
+                                       void* stream) {
+  HILS_REQUIRE(v && vt, "hils_transpose_v_chunks: null pointer");
+  HILS_REQUIRE(B > 0 && Lkv >= GA_S && H > 0 && Dv > 0 && Dv % 8 == 0,
+               "hils_transpose_v_chunks: bad sizes (Lkv >= 64, Dv %% 8 == 0)");
+  HILS_REQUIRE(H <= 65535 && B <= 65535, "hils_transpose_v_chunks: H/B too large for the grid");
+  const int nchunk = Lkv / GA_S;
+  float* vmax = (float*)((char*)vt + ga_vt_bytes(B, H, nchunk, Dv));
+  hipLaunchKernelGGL(transpose_v_kernel, dim3(nchunk, H, B), dim3(256),
+                     (size_t)GA_S * (Dv + 2) * sizeof(bf16_t), (hipStream_t)stream,
+                     (const bf16_t*)v, (bf16_t*)vt, vmax, Lkv, H, Dv, nchunk);
+  HILS_CHECK_LAUNCH("hils_transpose_v_chunks");
+  return HILS_OK;
+}

@@ -24,7 +24,8 @@ SIGNATURES = {
     "hils_attn_pool_bwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
     "hils_topk_fwd": [_P] * 10 + [_I] * 12 + [_F, _P],
     "hils_topk_bwd": [_P] * 6 + [_I] * 8 + [_F, _P],
-    "hils_sparse_attn_fwd": [_P] * 8 + [_I] * 12 + [_F, _I, _F, _P],
+    "hils_sparse_attn_fwd": [_P] * 9 + [_I] * 13 + [_F, _I, _F, _P],
+    "hils_transpose_v_chunks": [_P, _P, _I, _I, _I, _I, _P],
     "hils_sparse_attn_bwd": [_P] * 12 + [_I] * 12 + [_F, _I, _F, _P],
     "hils_chunk_logz_fwd": [_P, _P, _P] + [_I] * 7 + [_F, _I, _P],
     "hils_chunk_logz_bwd_dq": [_P] * 5 + [_I] * 7 + [_F, _P],
@@ -48,6 +49,8 @@ def load():
     lib.hils_last_error.argtypes = []
     lib.hils_version.restype = c_int
     lib.hils_version.argtypes = []
+    lib.hils_sparse_attn_fwd_workspace.restype = ctypes.c_size_t
+    lib.hils_sparse_attn_fwd_workspace.argtypes = [_I] * 11 + [_F]
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = c_int
@@ -74,6 +77,14 @@ def call(name, *args):
     if rc != 0:
         msg = lib.hils_last_error().decode("utf-8", "replace")
         raise RuntimeError(f"{name} failed (status {rc}): {msg}")
+
+
+def sparse_attn_fwd_workspace(device, B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n):
+    """Scratch tensor for hils_sparse_attn_fwd (None when the shape needs none)."""
+    n = load().hils_sparse_attn_fwd_workspace(B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n)
+    if n == 0:
+        return None
+    return torch.empty(n, dtype=torch.uint8, device=device)
 
 
 def require_gpu_bf16(name, *tensors):

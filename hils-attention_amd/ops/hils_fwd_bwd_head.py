@@ -37,9 +37,11 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
         lse = None
         if is_training:
             lse = torch.empty((B, L, HQ, K), dtype=torch.float32, device=q.device)
+        ws = _cabi.sparse_attn_fwd_workspace(q.device, B, L, L_kv, HQ, H, D, Dv, K, HQ, 1,
+                                             int(block_size), 0.0)
         _cabi.call("hils_sparse_attn_fwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
                    _cabi.ptr(idx_in), _cabi.ptr(slope_dev), _cabi.ptr(o), _cabi.ptr(lse),
-                   B, L, L_kv, HQ, H, D, Dv, K, num_weights, HQ, 1, int(block_size),
+                   _cabi.ptr(ws), 0, B, L, L_kv, HQ, H, D, Dv, K, num_weights, HQ, 1, int(block_size),
                    float(sm_scale), int(bool(mask_last_token)), 0.0)
         ctx.is_training = bool(is_training)
         if is_training:

@@ -41,7 +41,7 @@ class _attention(torch.autograd.Function):
         o = torch.empty_like(q)
         lse = torch.empty((N, L, HQ, K), dtype=torch.float32, device=q.device)
         _cabi.call("hils_sparse_attn_fwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
-                   _cabi.ptr(idx_in), None, _cabi.ptr(o), _cabi.ptr(lse),
+                   _cabi.ptr(idx_in), None, _cabi.ptr(o), _cabi.ptr(lse), None, 0,
                    N, L, L_kv, HQ, H, D, v.shape[-1], K, K, H, q_x, int(chunk_size),
                    float(sm_scale), 0, float(sm_n))
         ctx.save_for_backward(q, k, v, w_in, idx_in, lse)

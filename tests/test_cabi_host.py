@@ -17,7 +17,7 @@ def header_functions():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     out = {}
-    for m in re.finditer(r"\bint\s+(hils_\w+)\s*\(([^)]*)\)\s*;", text):
+    for m in re.finditer(r"\b(?:int|size_t)\s+(hils_\w+)\s*\(([^)]*)\)\s*;", text):
         params = [p.strip() for p in m.group(2).split(",") if p.strip() and p.strip() != "void"]
         out[m.group(1)] = params
     return out
@@ -35,6 +35,7 @@ def test_binding_matches_header(pkg):
     from hils_attention_amd.ops import _cabi
     fns = header_functions()
     fns.pop("hils_version")
+    fns.pop("hils_sparse_attn_fwd_workspace")
     assert set(_cabi.SIGNATURES) == set(fns)
     for name, params in fns.items():
         argtypes = _cabi.SIGNATURES[name]
@@ -59,7 +60,7 @@ def test_argument_errors_are_reported_without_a_gpu(pkg):
     assert lib.hils_topk_fwd(buf, buf, buf, None, None, None, buf, buf, None, None,
                              1, 16, 4, 1, 1, 64, 1000, 64, 1, 1, 0, 0, 0.125, None) == 1
     assert b"topk" in lib.hils_last_error()
-    assert lib.hils_sparse_attn_fwd(buf, buf, buf, buf, buf, None, buf, None,
+    assert lib.hils_sparse_attn_fwd(buf, buf, buf, buf, buf, None, buf, None, None, 0,
                                     1, 16, 64, 3, 2, 64, 64, 4, 4, 3, 1, 64, 0.125, 1, 0.0, None) == 1
     assert b"multiple of H" in lib.hils_last_error()
 

@@ -175,7 +175,7 @@ def test_sparse_attn_per_chunk_lse(pkg, orc, dev):
     o = torch.empty(B, L, HQ, 64, dtype=torch.bfloat16, device=dev)
     lse = torch.empty(B, L, HQ, 4, dtype=torch.float32, device=dev)
     t = [x.to(dev) for x in (q, k, v, w, idx)]
-    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(o), _cabi.ptr(lse),
+    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(o), _cabi.ptr(lse), None, 0,
                B, L, L, HQ, 2, D, 64, 4, w.shape[-1], HQ, 1, 64, 1 / math.sqrt(D), 1, 0.0)
     _, lse_ref = orc.sparse_attn(q, k, v, w, idx, chunk_size=64, return_lse=True)
     assert_close_f32(lse.cpu() / 1.4426950408889634, lse_ref, LSE_TOL, "per-chunk LSE")
@@ -194,3 +194,31 @@ def test_sparse_attn_decode_shape(pkg, orc, dev):
     note("sparse_attn decode B4 Lq1 Lkv4096")
     q, k, v, w, idx = make_case(4, 1, 8, 2, 128, 128, 8, 64, seed=12, Lkv=4096)
     fwd_check(pkg, orc, dev, q, k, v, w, idx, 64)
+
+
+@pytest.mark.parametrize("B,L,HQ,H,D,Dv,K", [(1, 1024, 8, 2, 128, 128, 8), (2, 512, 4, 4, 64, 64, 16),
+                                              (1, 700, 16, 1, 64, 128, 4), (1, 512, 8, 4, 128, 64, 32),
+                                              (1, 300, 16, 2, 64, 64, 8)])
+def test_sparse_attn_mfma_path_matches_generic_path(pkg, orc, dev, B, L, HQ, H, D, Dv, K):
+    """The chunk-regrouped MFMA kernel (workspace given) against the shape-generic kernel
+    (workspace NULL) and the oracle, output and per-chunk LSE, through the C ABI."""
+    from hils_attention_amd.ops import _cabi
+    note(f"sparse_attn mfma-vs-generic B{B} L{L} HQ{HQ} H{H} D{D} Dv{Dv} K{K}")
+    q, k, v, w, idx = make_case(B, L, HQ, H, D, Dv, K, 64, seed=21, fill_prob=0.8)
+    t = [x.to(dev) for x in (q, k, v, w, idx)]
+    outs = []
+    ws = _cabi.sparse_attn_fwd_workspace(dev, B, L, L, HQ, H, D, Dv, K, HQ, 1, 64, 0.0)
+    assert ws is not None, "this shape must be covered by the MFMA path"
+    for use_ws in (False, True):
+        o = torch.empty(B, L, HQ, Dv, dtype=torch.bfloat16, device=dev)
+        lse = torch.empty(B, L, HQ, K, dtype=torch.float32, device=dev)
+        _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(o), _cabi.ptr(lse),
+                   _cabi.ptr(ws) if use_ws else None, 0,
+                   B, L, L, HQ, H, D, Dv, K, w.shape[-1], HQ, 1, 64, 1 / math.sqrt(D), 1, 0.0)
+        torch.cuda.synchronize()
+        outs.append((o.cpu(), lse.cpu()))
+    ref, lse_ref = orc.sparse_attn(q, k, v, w, idx, chunk_size=64, return_lse=True)
+    for name, (o, lse) in zip(("generic", "mfma"), outs):
+        assert_close_bf16(o, ref, f"{name} o")
+        assert_close_f32(lse / 1.4426950408889634, lse_ref, LSE_TOL, f"{name} lse")
+    assert_close_bf16(outs[1][0], outs[0][0].float(), "mfma vs generic", max_abs=1e-2, rel_l2=5e-3)
