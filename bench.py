@@ -1,0 +1,241 @@
+"""Benchmark of the HiLS attention forward hot path on one MI355X.
+
+`python bench.py --gpus 1 --steps K --warmup W` prints ONE JSON line.
+
+Workload at N=1 (`config.workload`): the 7B-shaped 32K-token prefill layer forward
+(B1 L32768, 32 query heads / 8 KV heads, head_dim 128, chunk 64 -> 512 chunks, top-32).
+One step = mean-pool chunk keys -> fused top-k -> inter-chunk softmax -> sparse
+attention, inputs resident in HBM.  `value` is tokens/s of that step.  The same line
+carries the 128K-context decode step (batch 32, 2048 pooled chunk keys per KV head) as
+`decode_us_per_step`, a roofline object for the dominant kernel of each, and the CPU
+oracle timed on a bounded query slice as `cpu_baseline`.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+
+
+def gpu_randn(shape, gen, dev, scale=None, chunk=1 << 26):
+    """bf16 N(0,1) tensor generated on the GPU in slices (no fp32 copy of the whole tensor)."""
+    out = torch.empty(shape, dtype=torch.bfloat16, device=dev)
+    flat = out.view(-1)
+    for s in range(0, flat.numel(), chunk):
+        e = min(flat.numel(), s + chunk)
+        flat[s:e] = torch.randn(e - s, device=dev, generator=gen).bfloat16()
+    if scale is not None:
+        out.mul_(scale.to(torch.bfloat16))
+    return out
+
+
+def swa_lse_current_chunk(q, k, S):
+    """Exact lse of the local branch for window 1: keys of the query's own chunk up to the
+    query, landmark (last token of the chunk) masked.  (B,L,HQ) fp32, computed with torch."""
+    B, L, HQ, D = q.shape
+    H = k.shape[2]
+    G = HQ // H
+    N = L // S
+    qc = q.view(B, N, S, H, G, D).float()
+    kc = k.view(B, N, S, H, D).float()
+    s = torch.einsum("bnihgd,bnjhd->bnhgij", qc, kc) / math.sqrt(D)
+    i = torch.arange(S, device=q.device).view(S, 1)
+    j = torch.arange(S, device=q.device).view(1, S)
+    s = s.masked_fill((j > i) | (j == S - 1), float("-inf"))
+    lse = torch.logsumexp(s, dim=-1)  # (B,N,H,G,S)
+    return lse.permute(0, 1, 4, 2, 3).reshape(B, L, HQ).contiguous()
+
+
+def time_steps(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def bench_prefill(pkg, dev, steps, warmup):
+    from hils_attention_amd.ops import hils_fwd_bwd_head as attn_mod
+    B, L, HQ, H, D, S, K, W = 1, 32768, 32, 8, 128, 64, 32, 1
+    G = HQ // H
+    gen = torch.Generator(device=dev).manual_seed(1003)
+    hs = torch.rand(HQ, device=dev, generator=gen) * 1.5 + 0.5
+    q = gpu_randn((B, L, HQ, D), gen, dev, hs.view(1, 1, HQ, 1))
+    k = gpu_randn((B, L, H, D), gen, dev, hs[::G].view(1, 1, H, 1))
+    v = gpu_randn((B, L, H, D), gen, dev)
+    lse_swa = swa_lse_current_chunk(q, k, S).bfloat16()  # the layer hands it over in bf16
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
+    state = {}
+    acc = {"pool": 0.0, "topk": 0.0, "glue": 0.0, "vt": 0.0, "attn": 0.0, "n": 0}
+
+    def step(record=False):
+        if record:
+            ev[0].record()
+        lmk = pkg.chunk_mean_pool(k, S)
+        if record:
+            ev[1].record()
+        idx, scores = pkg.online_softmax_topk_head(q, lmk, lse_swa, K, S, W, is_training=False)
+        if record:
+            ev[2].record()
+        w = torch.softmax(torch.cat([scores, lse_swa.unsqueeze(-1)], dim=-1).float(), dim=-1).to(q.dtype)
+        if record:
+            ev[3].record()
+        ws = attn_mod.prepare_v_workspace(L, v, HQ, D, K, S)
+        if record:
+            ev[4].record()
+        o = pkg.HiLS_block_M_head(q, k, v, w, idx, block_size=S, is_training=False, v_workspace=ws)
+        if record:
+            ev[5].record()
+            torch.cuda.synchronize()
+            for name, a, b in (("pool", 0, 1), ("topk", 1, 2), ("glue", 2, 3), ("vt", 3, 4), ("attn", 4, 5)):
+                acc[name] += ev[a].elapsed_time(ev[b])
+            acc["n"] += 1
+        state["idx"], state["o"] = idx, o
+
+    sec = time_steps(step, steps, warmup)
+    for _ in range(min(steps, 5)):  # per-kernel durations with events on the launch stream
+        step(record=True)
+    per = {kk: vv / acc["n"] for kk, vv in acc.items() if kk != "n"}
+    n_sel = int((state["idx"] >= 0).sum().item())
+    flops = 4.0 * D * S * G * n_sel
+    attn_ms = per["attn"]
+    roof = {"kernel": "sparse_attn_fwd_gather", "bound": "mfma",
+            "achieved": flops / (attn_ms * 1e-3) / 1e12, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": flops / (attn_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, "traffic": None,
+            "flops_per_launch": flops, "ms_per_launch": attn_ms}
+    cfg = {"workload": "prefill_fwd B1 L32768 hq32/hkv8 D128 chunk64 top32 causal (7B-shaped, config 3)",
+           "global_batch": B, "seq_len": L, "n_sel": n_sel}
+    data = {"q": q, "k": k, "v": v, "lse_swa": lse_swa}
+    return sec, per, roof, cfg, data
+
+
+def bench_decode(pkg, dev, steps, warmup):
+    B, Lkv, HQ, H, D, S, K, W = 32, 131072, 32, 8, 128, 64, 32, 1
+    N = Lkv // S
+    gen = torch.Generator(device=dev).manual_seed(1004)
+    q = gpu_randn((B, 1, HQ, D), gen, dev)
+    kc = gpu_randn((B, Lkv, H, D), gen, dev)
+    vc = gpu_randn((B, Lkv, H, D), gen, dev)
+    lmk = pkg.chunk_mean_pool(kc, S)  # precomputed pooled keys (untimed)
+    lse_swa = (torch.randn(B, 1, HQ, device=dev, generator=gen) * 5 + 10).bfloat16()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    acc = {"topk": 0.0, "glue": 0.0, "attn": 0.0, "n": 0}
+
+    def step(record=False):
+        if record:
+            ev[0].record()
+        idx, scores = pkg.online_softmax_topk_head(q, lmk, lse_swa, K, S, W, q_offset=Lkv - 1,
+                                                   is_training=False)
+        if record:
+            ev[1].record()
+        w = torch.softmax(torch.cat([scores, lse_swa.unsqueeze(-1)], dim=-1).float(), dim=-1).to(q.dtype)
+        if record:
+            ev[2].record()
+        pkg.HiLS_block_M_head(q, kc, vc, w, idx, block_size=S, is_training=False)
+        if record:
+            ev[3].record()
+            torch.cuda.synchronize()
+            for name, a, b in (("topk", 0, 1), ("glue", 1, 2), ("attn", 2, 3)):
+                acc[name] += ev[a].elapsed_time(ev[b])
+            acc["n"] += 1
+
+    sec = time_steps(step, steps, warmup)
+    for _ in range(min(steps, 5)):
+        step(record=True)
+    per = {kk: vv / acc["n"] for kk, vv in acc.items() if kk != "n"}
+    lmk_bytes = B * N * H * D * 2
+    kv_bytes = B * H * K * S * D * 2 * 2
+    small = B * HQ * D * 2 * 2
+    total = lmk_bytes + kv_bytes + small
+    roof = {"kernel": "topk_fwd + sparse_attn_fwd (decode step)", "bound": "hbm",
+            "achieved": total / sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": total / sec / 1e9 / HBM_PEAK_GBS, "traffic": None, "bytes_per_step": total,
+            "topk_gbs": lmk_bytes / (per["topk"] * 1e-3) / 1e9,
+            "attn_gbs": kv_bytes / (per["attn"] * 1e-3) / 1e9}
+    del kc, vc
+    torch.cuda.empty_cache()
+    return sec, per, roof
+
+
+def cpu_baseline(data, n_queries=256):
+    """The CPU oracle on a bounded slice of the prefill workload: n_queries consecutive
+    queries around the middle of the sequence (top-k + inter-chunk softmax + sparse attention)."""
+    orc = entry.load_oracle()
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    S, K, W = 64, 32, 1
+    q, k, v, lse = (data[n].cpu() for n in ("q", "k", "v", "lse_swa"))
+    B, L, HQ, D = q.shape
+    H = k.shape[2]
+    t0q = L // 2 - n_queries // 2
+    qs = q[:, t0q:t0q + n_queries]
+    ls = lse[:, t0q:t0q + n_queries].float()
+    t0 = time.perf_counter()
+    lmk = orc.mean_pool(k, S)
+    idx, scores = orc.online_softmax_topk_head(qs.view(B, n_queries, H, HQ // H, D), lmk.bfloat16(), ls, K, S,
+                                               W, q_offset=t0q)
+    w = orc.inter_chunk_softmax(scores.reshape(B, n_queries, HQ, K), ls)
+    orc.sparse_attn(qs, k, v, w, idx, chunk_size=S)
+    dt = time.perf_counter() - t0
+    return {"value": n_queries * B / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"{n_queries} consecutive queries at t={t0q} of the same 32K prefill inputs "
+                      f"(pure-torch fp32 oracle: mean pool of all K, top-k, softmax, sparse attention), "
+                      f"{dt:.2f} s", "seconds": dt}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (no collectives are part of the hot "
+                 "path); run with --gpus 1")
+    entry.ensure_built()
+    pkg = entry.load_package()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    sec, per, roof, cfg, data = bench_prefill(pkg, dev, args.steps, args.warmup)
+    tokens = cfg["global_batch"] * cfg["seq_len"]
+    line = {
+        "metric": "hils_attn_fwd_tokens_per_s_32k_prefill", "value": tokens / sec, "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (seeded N(0,1), per-head scale U[0.5,2] on q/k; lse_swa of the local chunk)",
+        "config": cfg, "kernel_ms": per, "roofline": roof,
+    }
+    cpu = None if args.no_cpu else cpu_baseline(data)
+    del data
+    torch.cuda.empty_cache()
+    if not args.no_decode:
+        dsec, dper, droof = bench_decode(pkg, dev, max(args.steps, 20), args.warmup)
+        line["decode_us_per_step"] = dsec * 1e6
+        line["decode_config"] = {"workload": "decode step B32 Lq1 Lkv131072 (2048 pooled keys) hq32/hkv8 D128 top32 "
+                                             "(config 4)"}
+        line["decode_kernel_ms"] = dper
+        line["roofline_decode"] = droof
+    if cpu is not None:
+        line["cpu_baseline"] = cpu
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
