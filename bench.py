@@ -152,10 +152,22 @@ def bench_decode(pkg, dev, steps, warmup):
                 acc[name] += ev[a].elapsed_time(ev[b])
             acc["n"] += 1
 
-    sec = time_steps(step, steps, warmup)
+    eager_sec = time_steps(step, steps, warmup)
     for _ in range(min(steps, 5)):
         step(record=True)
     per = {kk: vv / acc["n"] for kk, vv in acc.items() if kk != "n"}
+    # the serving loop replays the step as one HIP graph (no host work between kernels)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    sec = time_steps(graph.replay, steps, warmup)
+    per["eager_step"] = eager_sec * 1e3
     lmk_bytes = B * N * H * D * 2
     kv_bytes = B * H * K * S * D * 2 * 2
     small = B * HQ * D * 2 * 2
@@ -170,7 +182,7 @@ def bench_decode(pkg, dev, steps, warmup):
     return sec, per, roof
 
 
-def cpu_baseline(data, n_queries=256):
+def cpu_baseline(data, n_queries=4096):
     """The CPU oracle on a bounded slice of the prefill workload: n_queries consecutive
     queries around the middle of the sequence (top-k + inter-chunk softmax + sparse attention)."""
     orc = entry.load_oracle()
@@ -203,6 +215,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true", help="profiling aid: decode step only")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives are part of the hot "
@@ -213,6 +226,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.no_prefill:
+        dsec, dper, droof = bench_decode(pkg, dev, max(args.steps, 20), args.warmup)
+        print(json.dumps({"decode_us_per_step": dsec * 1e6, "decode_kernel_ms": dper, "roofline_decode": droof}))
+        return
     sec, per, roof, cfg, data = bench_prefill(pkg, dev, args.steps, args.warmup)
     tokens = cfg["global_batch"] * cfg["seq_len"]
     line = {

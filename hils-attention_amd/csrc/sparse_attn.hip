@@ -19,6 +19,14 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
                               int H, int D, int Dv, int K, int NW, int S, float sm_scale,
                               int mask_last, void* stream, int* handled);
 
+bool hils_decode_covers(int L, int HQ, int H, int D, int Dv, int S, int q_block, int WH, float sm_n,
+                        const float* slope, const float* lse);
+size_t hils_decode_workspace_bytes(int B, int L, int HQ, int H, int Dv, int K);
+int hils_sparse_attn_decode(const void* q, const void* k, const void* v, const void* weights,
+                            const int32_t* indices, void* o, void* workspace, int B, int L, int Lkv,
+                            int HQ, int H, int D, int Dv, int K, int NW, float sm_scale,
+                            int mask_last, void* stream);
+
 struct SaDims {
   int L, Lkv, HQ, H, G, D, Dv, K, NW, WH, q_block, S, mask_last;
   float sm_scale, sm_n;
@@ -270,6 +278,8 @@ static int sa_check(const char* name, int B, int L, int Lkv, int HQ, int H, int 
 extern "C" size_t hils_sparse_attn_fwd_workspace(int B, int L, int Lkv, int HQ, int H, int D,
                                                  int Dv, int K, int WH, int q_block, int S,
                                                  float sm_n) {
+  if (hils_decode_covers(L, HQ, H, D, Dv, S, q_block, WH, sm_n, nullptr, nullptr))
+    return hils_decode_workspace_bytes(B, L, HQ, H, Dv, K);
   return hils_ga_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n);
 }
 
@@ -281,6 +291,13 @@ extern "C" int hils_sparse_attn_fwd(const void* q, const void* k, const void* v,
                                     float sm_scale, int mask_last, float sm_n, void* stream) {
   HILS_REQUIRE(q && k && v && weights && indices && o, "hils_sparse_attn_fwd: null pointer");
   if (int rc = sa_check("hils_sparse_attn_fwd", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
+  if (hils_decode_covers(L, HQ, H, D, Dv, S, q_block, WH, sm_n, slope, lse) && Lkv >= S) {
+    if (int rc = hils_sparse_attn_decode(q, k, v, weights, indices, o, workspace, B, L, Lkv, HQ, H, D,
+                                         Dv, K, NW, sm_scale, mask_last, stream))
+      return rc;
+    HILS_CHECK_LAUNCH("hils_sparse_attn_fwd");
+    return HILS_OK;
+  }
   if (workspace && hils_ga_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n) > 0) {
     int handled = 0;
     if (int rc = hils_sparse_attn_fwd_mfma(q, k, v, weights, indices, slope, o, lse, workspace,

@@ -1,0 +1,175 @@
+// Decode sparse attention, row-streaming variant (D == Dv, G <= 4).
+//
+// Every K and V load is a fully coalesced 16-byte lane load: LR = D/8 neighbouring lanes
+// read one 2*D-byte token row, 64/LR token rows per instruction.  q.K uses packed bf16
+// dot2 instructions plus a DPP reduction over the LR lanes of a row; because K and V rows
+// are mapped to lanes the same way, the softmax probabilities of a token already sit in
+// the lanes that hold that token's V row, so P V needs no data movement at all.
+#include "decode_rows.h"
+#include "../../include/hils_amd.h"
+
+#define DR_THREADS 256
+#define DR_WAVES (DR_THREADS / 64)
+#define DR_S 64
+
+struct DrDims {
+  int L, Lkv, HQ, H, G, K, NW, nchunk, nsplit, mask_last;
+  float sm_scale;
+};
+
+template <int D, int GMAX>
+__global__ void __launch_bounds__(DR_THREADS, 4)
+sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                               const bf16_t* __restrict__ v, const bf16_t* __restrict__ weights,
+                               const int32_t* __restrict__ indices, bf16_t* __restrict__ o,
+                               float* __restrict__ partial, DrDims dm) {
+  constexpr int LR = D / 8;        // lanes per token row
+  constexpr int TPI = 64 / LR;     // token rows per load instruction
+  constexpr int NI = DR_S / TPI;   // load instructions per chunk
+  constexpr int GI = 4;            // load instructions per pipelined group
+  constexpr int NG = NI / GI;      // groups per chunk
+  extern __shared__ float o_s[];   // [wave][G][D] partial outputs
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int piece = lane % LR, tsub = lane / LR;
+  const int split = blockIdx.x, hk = blockIdx.y;
+  const long bt = blockIdx.z;
+  const long b = bt / dm.L;
+  const int G = dm.G, K = dm.K;
+
+  uint4 qp[GMAX];  // this lane's 8 features of each query head, packed bf16
+#pragma unroll
+  for (int g = 0; g < GMAX; ++g) {
+    qp[g] = make_uint4(0, 0, 0, 0);
+    if (g < G) qp[g] = *(const uint4*)(q + (bt * dm.HQ + hk * G + g) * (long)D + piece * 8);
+  }
+  const float c2 = dm.sm_scale * HILS_LOG2E;
+  // running output of this wavefront, kept in its private slice of LDS (lanes < LR own it)
+  for (int i = lane; i < G * D; i += 64) o_s[(size_t)wave * G * D + i] = 0.f;
+
+  const int per_split = (K + dm.nsplit - 1) / dm.nsplit;
+  const int s_begin = split * per_split;
+  const int s_end = (s_begin + per_split < K) ? s_begin + per_split : K;
+  for (int slot = s_begin + wave; slot < s_end; slot += DR_WAVES) {
+    const int c = indices[(bt * dm.H + hk) * (long)K + slot];
+    if (c < 0 || c >= dm.nchunk) continue;
+    const long row0 = (b * dm.Lkv + (long)c * DR_S + tsub) * dm.H + hk;
+    const bf16_t* kp = k + row0 * D + piece * 8;
+    const bf16_t* vp = v + row0 * D + piece * 8;
+    const long step = (long)TPI * dm.H * D;
+    // flash-style pass over the chunk in NG groups of GI*TPI tokens; every token sub-group
+    // (lanes with the same tsub) keeps its own running max / sum / accumulator
+    float mrun[GMAX], lrun[GMAX], acc[GMAX][8];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+      mrun[g] = HILS_NEG_INF;
+      lrun[g] = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+    }
+#pragma unroll 1
+    for (int grp = 0; grp < NG; ++grp) {
+      constexpr int cur = 0;
+      uint4 kr[1][GI], vr[1][GI];
+#pragma unroll
+      for (int i = 0; i < GI; ++i) {
+        kr[0][i] = *(const uint4*)(kp + (grp * GI + i) * step);
+        vr[0][i] = *(const uint4*)(vp + (grp * GI + i) * step);
+      }
+      float sc[GMAX][GI];
+#pragma unroll
+      for (int i = 0; i < GI; ++i)
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g)
+          if (g < G) {
+            float s = row_sum<LR>(dot8_bf16(qp[g], kr[cur][i], 0.f));
+            if (dm.mask_last && grp == NG - 1 && i == GI - 1 && tsub == TPI - 1) s = HILS_NEG_INF;
+            sc[g][i] = s;
+          }
+#pragma unroll
+      for (int g = 0; g < GMAX; ++g)
+        if (g < G) {
+          float mn = mrun[g];
+#pragma unroll
+          for (int i = 0; i < GI; ++i) mn = fmaxf(mn, sc[g][i]);
+          if (mn > HILS_NEG_INF) {
+            const float corr = __builtin_amdgcn_exp2f((mrun[g] - mn) * c2);
+            lrun[g] *= corr;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[g][e] *= corr;
+#pragma unroll
+            for (int i = 0; i < GI; ++i) {
+              sc[g][i] = __builtin_amdgcn_exp2f((sc[g][i] - mn) * c2);
+              lrun[g] += sc[g][i];
+            }
+            mrun[g] = mn;
+          } else {
+#pragma unroll
+            for (int i = 0; i < GI; ++i) sc[g][i] = 0.f;
+          }
+        }
+#pragma unroll
+      for (int i = 0; i < GI; ++i) {
+        float vf[8];
+        unpack8(vr[cur][i], vf);
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g)
+          if (g < G) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(sc[g][i], vf[e], acc[g][e]);
+          }
+      }
+    }
+    // merge the token sub-groups, normalise, weight and add to the running output
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g)
+      if (g < G) {
+        float m = mrun[g];
+#pragma unroll
+        for (int off = LR; off < 64; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+        const float sc2 = (mrun[g] > HILS_NEG_INF) ? __builtin_amdgcn_exp2f((mrun[g] - m) * c2) : 0.f;
+        float l = lrun[g] * sc2;
+#pragma unroll
+        for (int off = LR; off < 64; off <<= 1) l += __shfl_xor(l, off, 64);
+        const float wr = bf2f(weights[(bt * dm.HQ + hk * G + g) * (long)dm.NW + slot]);
+        const float f = (l > 0.f) ? sc2 * wr / l : 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float x = acc[g][e] * f;
+#pragma unroll
+          for (int off = LR; off < 64; off <<= 1) x += __shfl_xor(x, off, 64);
+          if (lane < LR) o_s[((size_t)wave * G + g) * D + lane * 8 + e] += x;
+        }
+      }
+  }
+  __syncthreads();
+  for (int i = tid; i < G * D; i += DR_THREADS) {
+    const int g = i / D, dv = i - g * D;
+    float x = 0.f;
+#pragma unroll
+    for (int w2 = 0; w2 < DR_WAVES; ++w2) x += o_s[((size_t)w2 * G + g) * D + dv];
+    if (dm.nsplit == 1) o[(bt * dm.HQ + hk * G + g) * (long)D + dv] = f2bf(x);
+    else partial[((bt * dm.HQ + hk * G + g) * (long)dm.nsplit + split) * D + dv] = x;
+  }
+}
+
+bool hils_decode_rows_covers(int D, int Dv, int G) { return D == Dv && (D == 64 || D == 128) && G <= 4; }
+
+void hils_sparse_attn_decode_rows(const void* q, const void* k, const void* v, const void* weights,
+                                  const int32_t* indices, void* o, void* workspace, int nsplit,
+                                  int B, int L, int Lkv, int HQ, int H, int D, int K, int NW,
+                                  float sm_scale, int mask_last, hipStream_t st) {
+  const int G = HQ / H;
+  DrDims dm{L, Lkv, HQ, H, G, K, NW, Lkv / DR_S, nsplit, mask_last, sm_scale};
+  dim3 grid(nsplit, H, (unsigned)((long)B * L));
+  const size_t smem = (size_t)DR_WAVES * G * D * sizeof(float);
+#define DR_CALL(D_, G_)                                                                         \
+  hipLaunchKernelGGL((sparse_attn_decode_rows_kernel<D_, G_>), grid, dim3(DR_THREADS), smem, st, \
+                     (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)weights, \
+                     indices, (bf16_t*)o, (float*)workspace, dm)
+  if (D == 64) {
+    if (G == 1) DR_CALL(64, 1); else if (G == 2) DR_CALL(64, 2); else DR_CALL(64, 4);
+  } else {
+    if (G == 1) DR_CALL(128, 1); else if (G == 2) DR_CALL(128, 2); else DR_CALL(128, 4);
+  }
+#undef DR_CALL
+}

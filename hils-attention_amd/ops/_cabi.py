@@ -22,7 +22,7 @@ SIGNATURES = {
     "hils_mean_pool_bwd": [_P, _P, _I, _I, _I, _I, _I, _P],
     "hils_attn_pool_fwd": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
     "hils_attn_pool_bwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
-    "hils_topk_fwd": [_P] * 10 + [_I] * 12 + [_F, _P],
+    "hils_topk_fwd": [_P] * 11 + [_I] * 12 + [_F, _P],
     "hils_topk_bwd": [_P] * 6 + [_I] * 8 + [_F, _P],
     "hils_sparse_attn_fwd": [_P] * 9 + [_I] * 13 + [_F, _I, _F, _P],
     "hils_transpose_v_chunks": [_P, _P, _I, _I, _I, _I, _P],
@@ -49,6 +49,8 @@ def load():
     lib.hils_last_error.argtypes = []
     lib.hils_version.restype = c_int
     lib.hils_version.argtypes = []
+    lib.hils_topk_fwd_workspace.restype = ctypes.c_size_t
+    lib.hils_topk_fwd_workspace.argtypes = [_I] * 5
     lib.hils_sparse_attn_fwd_workspace.restype = ctypes.c_size_t
     lib.hils_sparse_attn_fwd_workspace.argtypes = [_I] * 11 + [_F]
     for name, argtypes in SIGNATURES.items():
@@ -77,6 +79,14 @@ def call(name, *args):
     if rc != 0:
         msg = lib.hils_last_error().decode("utf-8", "replace")
         raise RuntimeError(f"{name} failed (status {rc}): {msg}")
+
+
+def topk_fwd_workspace(device, B, L, N, h_kv, G):
+    """Scratch tensor for hils_topk_fwd (None when the fused kernel needs none)."""
+    n = load().hils_topk_fwd_workspace(B, L, N, h_kv, G)
+    if n == 0:
+        return None
+    return torch.empty(n, dtype=torch.uint8, device=device)
 
 
 def sparse_attn_fwd_workspace(device, B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n):

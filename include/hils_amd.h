@@ -63,12 +63,16 @@ int hils_attn_pool_bwd(const void* mu_q, const void* k, const float* p, const fl
  * logaddexp(lse_swa, lse_hils); sel_logits (B,L,h_kv,G,N) fp32 = the selection
  * logits (scaled qk + bias + gumbel, -inf where the chunk is not visible).
  * Chunk c is visible to query t iff !causal or c < floor((t+q_offset-window+1)/block)
- * (window > 0) / floor((t+q_offset)/block) (window <= 0).  Ties: lower index wins. */
+ * (window > 0) / floor((t+q_offset)/block) (window <= 0).  Ties: lower index wins.
+ * workspace: device scratch of hils_topk_fwd_workspace(...) bytes or NULL.  With few queries
+ * (decode) and a workspace, the logits are spread over many workgroups and parked there
+ * before a separate selection kernel; otherwise one fused kernel runs. */
+size_t hils_topk_fwd_workspace(int B, int L, int N, int h_kv, int G);
 int hils_topk_fwd(const void* q, const void* lmks, const float* lse_swa, const float* bias,
                   const float* gumbel, const int32_t* drop_mask, int32_t* indices, void* scores,
-                  float* lse_total, float* sel_logits, int B, int L, int N, int h_kv, int G, int D,
-                  int topk, int block_size, int window_size, int causal, int q_offset,
-                  int per_qhead, float sm_scale, void* stream);
+                  float* lse_total, float* sel_logits, void* workspace, int B, int L, int N,
+                  int h_kv, int G, int D, int topk, int block_size, int window_size, int causal,
+                  int q_offset, int per_qhead, float sm_scale, void* stream);
 
 /* Sparse backward of the score gather.  Replaces the dense scatter + two torch.bmm of
  * SoftmaxTopKMaxPoolingFusedFn.backward (ops/topk_head_softmax.py:1040-1092).

@@ -36,6 +36,7 @@ def test_binding_matches_header(pkg):
     fns = header_functions()
     fns.pop("hils_version")
     fns.pop("hils_sparse_attn_fwd_workspace")
+    fns.pop("hils_topk_fwd_workspace")
     assert set(_cabi.SIGNATURES) == set(fns)
     for name, params in fns.items():
         argtypes = _cabi.SIGNATURES[name]
@@ -57,7 +58,7 @@ def test_argument_errors_are_reported_without_a_gpu(pkg):
     buf = ctypes.c_void_p(16)
     assert lib.hils_mean_pool_fwd(buf, buf, 1, 100, 1, 64, 64, None) == 1
     assert b"multiple" in lib.hils_last_error()
-    assert lib.hils_topk_fwd(buf, buf, buf, None, None, None, buf, buf, None, None,
+    assert lib.hils_topk_fwd(buf, buf, buf, None, None, None, buf, buf, None, None, None,
                              1, 16, 4, 1, 1, 64, 1000, 64, 1, 1, 0, 0, 0.125, None) == 1
     assert b"topk" in lib.hils_last_error()
     assert lib.hils_sparse_attn_fwd(buf, buf, buf, buf, buf, None, buf, None, None, 0,

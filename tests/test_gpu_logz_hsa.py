@@ -100,4 +100,5 @@ def test_hsa_sm_n_zero_equals_hils_without_mask(pkg, dev):
     a = pkg.HSA(q, k, v, w, idx, 0.0, S, None)
     b = pkg.HiLS_block_M_head(q, k, v, w.repeat_interleave(HQ // H, 2).contiguous(), idx, block_size=S,
                               mask_last_token=False, is_training=False)
-    assert torch.equal(a, b)
+    # the two entry points may run on different kernels (shape-generic vs MFMA): same math
+    assert_close_bf16(a, b.float(), "hsa(sm_n=0) vs hils(no mask)", max_abs=1e-2, rel_l2=5e-3)

@@ -207,3 +207,38 @@ def test_topk_argument_errors(pkg, dev):
         pkg.online_softmax_topk_head(q.float(), lmks[:, :, :2].float(), lse, 4, 64, 1)
     with pytest.raises(RuntimeError):
         pkg.online_softmax_topk_head(q, lmks[:, :, :2], lse, 100, 64, 1)
+
+
+def test_topk_split_path_options(pkg, orc, dev):
+    """Few queries and many chunks take the two-kernel path (logits spread over workgroups,
+    then selection); cover bias / Gumbel / drop mask / per-q-head keys / ragged N there."""
+    run_case(pkg, orc, dev, B=2, L=3, N=600, h_kv=2, G=4, D=64, topk=16, S=64, W=64, q_offset=600 * 64,
+             training=False, use_bias=True, use_drop=True)
+    run_case(pkg, orc, dev, B=1, L=1, N=1000, h_kv=2, G=2, D=128, topk=8, S=64, W=1, q_offset=70000,
+             training=False, per_qhead=True)
+    run_case(pkg, orc, dev, B=1, L=20, N=700, h_kv=1, G=3, D=64, topk=32, S=64, W=1, q_offset=700 * 64 - 20,
+             training=False, use_bias=True)
+    run_case(pkg, orc, dev, B=1, L=2, N=513, h_kv=1, G=1, D=64, topk=4, S=64, W=0, is_causal=False,
+             training=True, use_gumbel=True)
+
+
+def test_topk_split_and_fused_paths_agree(pkg, dev):
+    from hils_attention_amd.ops import _cabi
+    B, L, N, h_kv, G, D, topk = 2, 4, 1024, 2, 4, 128, 32
+    gen = torch.Generator().manual_seed(5)
+    q = torch.randn(B, L, h_kv, G, D, generator=gen).bfloat16().to(dev)
+    lmks = torch.randn(B, N, h_kv, D, generator=gen).bfloat16().to(dev)
+    lse = (torch.randn(B, L, h_kv, G, generator=gen) * 5 + 10).to(dev)
+    ws = _cabi.topk_fwd_workspace(dev, B, L, N, h_kv, G)
+    assert ws is not None
+    outs = []
+    for w in (None, ws):
+        idx = torch.empty(B, L, h_kv, topk, dtype=torch.int32, device=dev)
+        sc = torch.empty(B, L, h_kv, G, topk, dtype=torch.bfloat16, device=dev)
+        _cabi.call("hils_topk_fwd", _cabi.ptr(q), _cabi.ptr(lmks), _cabi.ptr(lse), None, None, None,
+                   _cabi.ptr(idx), _cabi.ptr(sc), None, None, _cabi.ptr(w), B, L, N, h_kv, G, D, topk, 64, 1, 1,
+                   N * 64, 0, D ** -0.5)
+        torch.cuda.synchronize()
+        outs.append((idx.cpu(), sc.float().cpu()))
+    assert torch.equal(outs[0][0], outs[1][0])
+    assert (outs[0][1] - outs[1][1]).abs().max().item() <= 2e-2
