@@ -93,10 +93,10 @@ def bench_prefill(pkg, dev, steps, warmup):
         w = torch.softmax(torch.cat([scores, lse_swa.unsqueeze(-1)], dim=-1).float(), dim=-1).to(q.dtype)
         if record:
             ev[3].record()
-        ws = attn_mod.prepare_v_workspace(L, v, HQ, D, K, S)
+        ws = attn_mod.prepare_kv_workspace(L, k, v, HQ, K, S)
         if record:
             ev[4].record()
-        o = pkg.HiLS_block_M_head(q, k, v, w, idx, block_size=S, is_training=False, v_workspace=ws)
+        o = pkg.HiLS_block_M_head(q, k, v, w, idx, block_size=S, is_training=False, kv_workspace=ws)
         if record:
             ev[5].record()
             torch.cuda.synchronize()

@@ -21,17 +21,40 @@
 #define GA_PAIR_BITS 12
 
 // ---------------------------------------------------------------------------
-// V pre-transpose: vt[b][h][c][dv][p] with token(p) = 32*(p/32) + 16*((p%8)/4) + 4*((p%32)/8) + p%4,
-// the order in which a 16x16x32 MFMA B operand wants the tokens of an accumulator-layout P.
+// Operand packing.  Each 64-token chunk of K and V of a (batch, KV head) is rewritten once
+// into the exact register order of the 16x16x32 MFMA operands the forward kernel needs, so
+// that every operand load of a wavefront is one contiguous 1 KiB burst (8 full cache lines)
+// instead of 16 half-used lines at a 2*H*D-byte stride:
+//   kp[chunk][mt][ks][lane][8] = K[token mt*16 + (lane&15)][d = ks*32 + (lane>>4)*8 + e]
+//   vp[chunk][dt][s][lane][8]  = V[token tok(s, lane>>4, e)][dv = dt*16 + (lane&15)]
+// with tok(s, j, e) = 32*s + 16*(e/4) + 4*j + e%4, the order in which an accumulator-layout
+// P supplies tokens when it is fed back as the A operand of O = P V.
 // Also records max|V| of every chunk (it bounds the fixed-point output accumulation).
 // ---------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)
-transpose_v_kernel(const bf16_t* __restrict__ v, bf16_t* __restrict__ vt, float* __restrict__ vmax,
-                   int Lkv, int H, int Dv, int nchunk) {
-  extern __shared__ bf16_t tile[];  // 64 x (Dv + 2)
+pack_kv_kernel(const bf16_t* __restrict__ k, const bf16_t* __restrict__ v, bf16_t* __restrict__ kp,
+               bf16_t* __restrict__ vp, float* __restrict__ vmax, int Lkv, int H, int D, int Dv,
+               int nchunk) {
+  extern __shared__ bf16_t tile[];  // 64 x (max(D, Dv) + 2)
   __shared__ float red[32];
   const int c = blockIdx.x, h = blockIdx.y;
   const long b = blockIdx.z;
+  const long chunk = (b * H + h) * (long)nchunk + c;
+  // ---- K: rows are already contiguous along d; only the order of 16-byte pieces changes
+  {
+    const int pieces = D / 8;  // 16-byte pieces per token row
+    bf16_t* out = kp + chunk * (long)GA_S * D;
+    for (int i = threadIdx.x; i < GA_S * pieces; i += 256) {
+      // destination order: ((mt * KS + ks) * 64 + lane)
+      const int lane = i & 63, blk = i >> 6;
+      const int KS = D / 32;
+      const int mt = blk / KS, ks = blk - mt * KS;
+      const int tok = mt * 16 + (lane & 15), d = ks * 32 + (lane >> 4) * 8;
+      const uint4 x = *(const uint4*)(k + ((b * Lkv + (long)c * GA_S + tok) * H + h) * D + d);
+      *(uint4*)(out + (long)i * 8) = x;
+    }
+  }
+  // ---- V: transposed through LDS
   const int DP = Dv + 2;
   const int d8n = Dv / 8;
   float mx = 0.f;
@@ -46,18 +69,20 @@ transpose_v_kernel(const bf16_t* __restrict__ v, bf16_t* __restrict__ vt, float*
     }
   }
   mx = block_max(mx, red);  // contains the barrier that orders the tile writes
-  if (threadIdx.x == 0) vmax[(b * H + h) * (long)nchunk + c] = mx;
-  bf16_t* out = vt + (((b * H + h) * (long)nchunk + c) * Dv) * GA_S;
+  if (threadIdx.x == 0) vmax[chunk] = mx;
+  bf16_t* out = vp + chunk * (long)GA_S * Dv;
   for (int i = threadIdx.x; i < Dv * 8; i += 256) {
-    const int dv = i >> 3, p8 = i & 7;  // 8 positions p8*8 .. p8*8+7
+    // destination order: ((dt * 2 + s) * 64 + lane)
+    const int lane = i & 63, blk = i >> 6;
+    const int dt = blk >> 1, s = blk & 1;
+    const int dv = dt * 16 + (lane & 15), j = lane >> 4;
     bf16_t y[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int p = p8 * 8 + e;
-      const int tok = 32 * (p >> 5) + 16 * ((p & 7) >> 2) + 4 * ((p & 31) >> 3) + (p & 3);
+      const int tok = 32 * s + 16 * (e >> 2) + 4 * j + (e & 3);
       y[e] = tile[tok * DP + dv];
     }
-    *(uint4*)(out + (long)dv * GA_S + p8 * 8) = *(uint4*)y;
+    *(uint4*)(out + (long)i * 8) = *(uint4*)y;
   }
 }
 
@@ -73,8 +98,8 @@ struct GaDims {
 // bounds every output element because each P row is a convex combination.
 template <int D, int DV, int G>
 __global__ void __launch_bounds__(GA_THREADS)
-sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
-                       const bf16_t* __restrict__ vt, const float* __restrict__ vmax,
+sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kp,
+                       const bf16_t* __restrict__ vp, const float* __restrict__ vmax,
                        const bf16_t* __restrict__ weights, const int32_t* __restrict__ indices,
                        const float* __restrict__ slope, bf16_t* __restrict__ o,
                        float* __restrict__ lse, GaDims dm) {
@@ -200,43 +225,58 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
     // the chunk's K rows (A operands of S^T = K Q^T) and transposed V (B operands of P V)
     bf16x8_t ka[4][KS], vb[DT][2];
     {
-      const bf16_t* kbase = k + ((b * dm.Lkv + (long)c * GA_S + r) * dm.H + hk) * D + j * 8;
+      const long chunk = (b * dm.H + hk) * (long)dm.nchunk + c;
+      const bf16_t* kbase = kp + chunk * (long)GA_S * D + lane * 8;
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          const uint4 x = *(const uint4*)(kbase + (long)mt * 16 * dm.H * D + ks * 32);
+          const uint4 x = *(const uint4*)(kbase + (mt * KS + ks) * 512);
           ka[mt][ks] = *(const bf16x8_t*)&x;
         }
-      const bf16_t* vbase = vt + ((((b * dm.H + hk) * (long)dm.nchunk + c) * DV + r) * GA_S) + j * 8;
+      const bf16_t* vbase = vp + chunk * (long)GA_S * DV + lane * 8;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-          const uint4 x = *(const uint4*)(vbase + (long)dt * 16 * GA_S + s * 32);
+          const uint4 x = *(const uint4*)(vbase + (dt * 2 + s) * 512);
           vb[dt][s] = *(const bf16x8_t*)&x;
         }
     }
 
+    // gathered query rows (B operands) and weights are loaded one tile ahead
+    auto load_tile = [&](int p, int& pid_o, uint4* bq_o, bf16_t& w_o) {
+      const int n = (ve - p < QT) ? ve - p : QT;
+      const bool rvalid = qs < n;
+      pid_o = pairs[p + (rvalid ? qs : 0)];
+      const int ql = pid_o / K, slot = pid_o - ql * K;
+      const long t = t0 + ql;
+      const bf16_t* qrow = q + ((b * dm.L + t) * (long)dm.HQ + hq) * D + j * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        bq_o[ks] = make_uint4(0, 0, 0, 0);
+        if (rvalid) bq_o[ks] = *(const uint4*)(qrow + ks * 32);
+      }
+      w_o = 0;
+      if (rvalid) w_o = weights[((b * dm.L + t) * (long)dm.HQ + hq) * dm.NW + slot];
+    };
+    int pid_n;
+    uint4 bq_n[KS];
+    bf16_t w_n;
+    load_tile(vs, pid_n, bq_n, w_n);
     for (int p = vs; p < ve; p += QT) {
       const int n = (ve - p < QT) ? ve - p : QT;
       // this lane's row of the tile: query slot r / G, head r % G
       const bool rvalid = qs < n;
-      const int pid = pairs[p + (rvalid ? qs : 0)];
+      const int pid = pid_n;
       const int ql = pid / K, slot = pid - ql * K;
       const int t = t0 + ql;
       const int row_base = (ql * G + g) * DV;
-
       bf16x8_t bq[KS];
-      const bf16_t* qrow = q + ((b * dm.L + t) * (long)dm.HQ + hq) * D + j * 8;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        uint4 x = make_uint4(0, 0, 0, 0);
-        if (rvalid) x = *(const uint4*)(qrow + ks * 32);
-        bq[ks] = *(bf16x8_t*)&x;
-      }
-      float wr = 0.f;
-      if (rvalid) wr = bf2f(weights[((b * dm.L + t) * (long)dm.HQ + hq) * dm.NW + slot]);
+      for (int ks = 0; ks < KS; ++ks) bq[ks] = *(bf16x8_t*)&bq_n[ks];
+      const float wr = bf2f(w_n);
+      if (p + QT < ve) load_tile(p + QT, pid_n, bq_n, w_n);
       f32x4_t st[4];
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) {
@@ -360,7 +400,7 @@ static int ga_dispatch_g(int G, dim3 grid, size_t smem, hipStream_t st, const bf
   return -1;
 }
 
-static size_t ga_vt_bytes(int B, int H, int nchunk, int Dv) {
+static size_t ga_vt_bytes(int B, int H, int nchunk, int Dv) {  // one packed tensor (K or V)
   size_t n = (size_t)B * H * nchunk * Dv * GA_S * sizeof(bf16_t);
   return (n + 255) & ~(size_t)255;
 }
@@ -395,7 +435,7 @@ size_t hils_ga_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int 
   size_t smem;
   if (ga_pick_T(L, G, Dv, K, Lkv / S, &smem) == 0) return 0;
   const int nchunk = Lkv / S;
-  return ga_vt_bytes(B, H, nchunk, Dv) + (size_t)B * H * nchunk * sizeof(float);
+  return ga_vt_bytes(B, H, nchunk, Dv) + ga_vt_bytes(B, H, nchunk, D) + (size_t)B * H * nchunk * sizeof(float);
 }
 
 // Returns HILS_OK and sets *handled = 1 when the MFMA path ran.
@@ -414,18 +454,21 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
   const int nblk = (L + T - 1) / T;
   const long total = (long)nblk * H * B;
   if (total > (1L << 30)) return HILS_OK;
-  bf16_t* vt = (bf16_t*)workspace;
-  float* vmax = (float*)((char*)workspace + ga_vt_bytes(B, H, nchunk, Dv));
-  if (!workspace_ready)
-    hipLaunchKernelGGL(transpose_v_kernel, dim3(nchunk, H, B), dim3(256),
-                       (size_t)GA_S * (Dv + 2) * sizeof(bf16_t), st, (const bf16_t*)v, vt, vmax,
-                       Lkv, H, Dv, nchunk);
+  bf16_t* vpk = (bf16_t*)workspace;
+  bf16_t* kpk = (bf16_t*)((char*)workspace + ga_vt_bytes(B, H, nchunk, Dv));
+  float* vmax = (float*)((char*)kpk + ga_vt_bytes(B, H, nchunk, D));
+  if (!workspace_ready) {
+    const int dmax = D > Dv ? D : Dv;
+    hipLaunchKernelGGL(pack_kv_kernel, dim3(nchunk, H, B), dim3(256),
+                       (size_t)GA_S * (dmax + 2) * sizeof(bf16_t), st, (const bf16_t*)k,
+                       (const bf16_t*)v, kpk, vpk, vmax, Lkv, H, D, Dv, nchunk);
+  }
   GaDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale};
   const long per_xcd = (total + 7) / 8;
   dim3 grid((unsigned)(per_xcd * 8));
   int rc = -1;
 #define GA_CALL(D_, DV_)                                                                       \
-  rc = ga_dispatch_g<D_, DV_>(G, grid, smem, st, (const bf16_t*)q, (const bf16_t*)k, vt, vmax, \
+  rc = ga_dispatch_g<D_, DV_>(G, grid, smem, st, (const bf16_t*)q, kpk, vpk, vmax,             \
                               (const bf16_t*)weights, indices, slope, (bf16_t*)o, lse, dm)
   if (D == 64 && Dv == 64) GA_CALL(64, 64);
   else if (D == 128 && Dv == 128) GA_CALL(128, 128);
@@ -437,17 +480,20 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
   return HILS_OK;
 }
 
-extern "C" int hils_transpose_v_chunks(const void* v, void* vt, int B, int Lkv, int H, int Dv,
-                                       void* stream) {
-  HILS_REQUIRE(v && vt, "hils_transpose_v_chunks: null pointer");
-  HILS_REQUIRE(B > 0 && Lkv >= GA_S && H > 0 && Dv > 0 && Dv % 8 == 0,
-               "hils_transpose_v_chunks: bad sizes (Lkv >= 64, Dv %% 8 == 0)");
-  HILS_REQUIRE(H <= 65535 && B <= 65535, "hils_transpose_v_chunks: H/B too large for the grid");
+extern "C" int hils_pack_kv_chunks(const void* k, const void* v, void* workspace, int B, int Lkv,
+                                   int H, int D, int Dv, void* stream) {
+  HILS_REQUIRE(k && v && workspace, "hils_pack_kv_chunks: null pointer");
+  HILS_REQUIRE(B > 0 && Lkv >= GA_S && H > 0 && (D == 64 || D == 128) && (Dv == 64 || Dv == 128),
+               "hils_pack_kv_chunks: bad sizes (Lkv >= 64, D and Dv in {64, 128})");
+  HILS_REQUIRE(H <= 65535 && B <= 65535, "hils_pack_kv_chunks: H/B too large for the grid");
   const int nchunk = Lkv / GA_S;
-  float* vmax = (float*)((char*)vt + ga_vt_bytes(B, H, nchunk, Dv));
-  hipLaunchKernelGGL(transpose_v_kernel, dim3(nchunk, H, B), dim3(256),
-                     (size_t)GA_S * (Dv + 2) * sizeof(bf16_t), (hipStream_t)stream,
-                     (const bf16_t*)v, (bf16_t*)vt, vmax, Lkv, H, Dv, nchunk);
-  HILS_CHECK_LAUNCH("hils_transpose_v_chunks");
+  bf16_t* vpk = (bf16_t*)workspace;
+  bf16_t* kpk = (bf16_t*)((char*)workspace + ga_vt_bytes(B, H, nchunk, Dv));
+  float* vmax = (float*)((char*)kpk + ga_vt_bytes(B, H, nchunk, D));
+  const int dmax = D > Dv ? D : Dv;
+  hipLaunchKernelGGL(pack_kv_kernel, dim3(nchunk, H, B), dim3(256),
+                     (size_t)GA_S * (dmax + 2) * sizeof(bf16_t), (hipStream_t)stream,
+                     (const bf16_t*)k, (const bf16_t*)v, kpk, vpk, vmax, Lkv, H, D, Dv, nchunk);
+  HILS_CHECK_LAUNCH("hils_pack_kv_chunks");
   return HILS_OK;
 }

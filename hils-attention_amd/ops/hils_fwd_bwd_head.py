@@ -11,7 +11,7 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, weights, indices, block_size, sm_scale, mask_last_token,
-                is_training, slope=None, v_workspace=None):
+                is_training, slope=None, kv_workspace=None):
         assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
         assert weights.is_contiguous() and indices.is_contiguous()
         _cabi.require_gpu_bf16("HiLS_block_M_head", q, k, v)
@@ -38,8 +38,8 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
         if is_training:
             lse = torch.empty((B, L, HQ, K), dtype=torch.float32, device=q.device)
         ws_ready = 0
-        if v_workspace is not None:
-            ws, ws_ready = v_workspace, 1
+        if kv_workspace is not None:
+            ws, ws_ready = kv_workspace, 1
         else:
             ws = _cabi.sparse_attn_fwd_workspace(q.device, B, L, L_kv, HQ, H, D, Dv, K, HQ, 1,
                                                  int(block_size), 0.0)
@@ -79,16 +79,16 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
 def HiLS_block_M_head(q, k, v, weights, indices, block_size=64, sm_scale=None, block_M=None,
                       mask_last_token=True, dtype="bfloat16", accum_dtype="float",
                       num_threads=None, num_threads_fwd=None, num_threads_bwd=None,
-                      is_training=True, slope=None, v_workspace=None):
+                      is_training=True, slope=None, kv_workspace=None):
     """o[t,h] = sum_k weights[t,h,k] * softmax_{j in chunk indices[t,k]}(sm_scale*q.K_j) V_j.
 
     q (B,L,HQ,D), k (B,Lkv,H,D), v (B,Lkv,H,Dv) bf16 contiguous; weights (B,L,HQ,>=K) (the
     first K columns are read); indices (B,L,H,K) int32, negative = empty slot.  Call
     signature of ops/hils_fwd_bwd_head.py:928-934; ``block_M`` and the ``num_threads*``
     tuning knobs are accepted and ignored (tile shapes are chosen by the HIP launcher),
-    ``dtype`` must be "bfloat16" and ``accum_dtype`` "float".  ``v_workspace`` (not in the
-    reference) is an optional tensor from ``prepare_v_workspace`` for the same ``v``: the
-    per-chunk transposed copy of V the MFMA kernel reads, reusable across calls.
+    ``dtype`` must be "bfloat16" and ``accum_dtype`` "float".  ``kv_workspace`` (not in the
+    reference) is an optional tensor from ``prepare_kv_workspace`` for the same ``v``: the
+    MFMA-operand-ordered copies of K and V the prefill kernel reads, reusable across calls.
     """
     B, L, HQ, D = q.shape
     _, L_kv, H, Dk = k.shape
@@ -98,16 +98,18 @@ def HiLS_block_M_head(q, k, v, weights, indices, block_size=64, sm_scale=None, b
         raise ValueError("HiLS_block_M_head: only dtype='bfloat16' with accum_dtype='float' is built")
     return _hils_block_M_attention_inverse.apply(
         q, k, v, weights, indices, block_size, sm_scale, mask_last_token, is_training, slope,
-        v_workspace)
+        kv_workspace)
 
 
-def prepare_v_workspace(q_len, v, num_q_heads, head_dim, topk, block_size=64):
-    """Build the transposed-V workspace ``HiLS_block_M_head(..., v_workspace=...)`` accepts
-    (None when the shape runs on the shape-generic kernels, which need none)."""
-    _cabi.require_gpu_bf16("prepare_v_workspace", v)
+def prepare_kv_workspace(q_len, k, v, num_q_heads, topk, block_size=64):
+    """Build the packed K/V workspace ``HiLS_block_M_head(..., kv_workspace=...)`` accepts
+    (None when the shape runs on kernels that need none)."""
+    _cabi.require_gpu_bf16("prepare_kv_workspace", k, v)
     B, L_kv, H, Dv = v.shape
-    ws = _cabi.sparse_attn_fwd_workspace(v.device, B, q_len, L_kv, num_q_heads, H, head_dim, Dv,
+    D = k.shape[-1]
+    ws = _cabi.sparse_attn_fwd_workspace(v.device, B, q_len, L_kv, num_q_heads, H, D, Dv,
                                          topk, num_q_heads, 1, int(block_size), 0.0)
-    if ws is not None:
-        _cabi.call("hils_transpose_v_chunks", _cabi.ptr(v.contiguous()), _cabi.ptr(ws), B, L_kv, H, Dv)
+    if ws is not None and q_len >= 64:
+        _cabi.call("hils_pack_kv_chunks", _cabi.ptr(k.contiguous()), _cabi.ptr(v.contiguous()),
+                   _cabi.ptr(ws), B, L_kv, H, D, Dv)
     return ws

@@ -93,8 +93,8 @@ int hils_topk_bwd(const void* g_scores, const void* q, const void* lmks, const i
  * Outputs: o (B,L,HQ,Dv) bf16; lse (B,L,HQ,K) fp32 per-chunk log2-domain LSE or NULL
  * (-inf for empty slots).
  * workspace: device scratch of hils_sparse_attn_fwd_workspace(...) bytes; the MFMA path
- * keeps a per-chunk transposed copy of V there.  workspace_ready != 0 says the copy from an
- * earlier call (or from hils_transpose_v_chunks) on the same v is still valid and is not
+ * keeps MFMA-operand-ordered copies of K and V there.  workspace_ready != 0 says the copies from
+ * an earlier call (or from hils_pack_kv_chunks) on the same k and v are still valid and is not
  * rebuilt.  With workspace == NULL, or a size of 0 from the query, the shape-generic path
  * runs. */
 size_t hils_sparse_attn_fwd_workspace(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K,
@@ -104,11 +104,13 @@ int hils_sparse_attn_fwd(const void* q, const void* k, const void* v, const void
                          void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ, int H,
                          int D, int Dv, int K, int NW, int WH, int q_block, int S, float sm_scale,
                          int mask_last, float sm_n, void* stream);
-/* Fills a workspace of hils_sparse_attn_fwd_workspace(...) bytes on its own: v (B,Lkv,H,Dv)
- * bf16 -> (B,H,Lkv/64,Dv,64) bf16 with the 64 tokens of a chunk in MFMA operand order,
- * followed by max|V| of every chunk (fp32).  No counterpart in the reference (TileLang
- * stages V through shared memory on every use). */
-int hils_transpose_v_chunks(const void* v, void* vt, int B, int Lkv, int H, int Dv, void* stream);
+/* Fills a workspace of hils_sparse_attn_fwd_workspace(...) bytes on its own: per 64-token
+ * chunk of a (batch, KV head), K and V rewritten in the register order of the MFMA operands
+ * the prefill kernel loads (every operand load becomes one contiguous 1 KiB burst), followed
+ * by max|V| of every chunk (fp32).  No counterpart in the reference (TileLang stages K/V
+ * through shared memory on every use). */
+int hils_pack_kv_chunks(const void* k, const void* v, void* workspace, int B, int Lkv, int H, int D,
+                        int Dv, void* stream);
 
 /* Backward.  Replaces hierarchical_sparse_attention_bwd_dqkv_block_M_inverse
  * (ops/hils_fwd_bwd_head.py:506-766) and kernel_attn_bwd_dq / _attn_bwd_dkdv /
