@@ -90,7 +90,7 @@ def bench_prefill(pkg, dev, steps, warmup):
         idx, scores = pkg.online_softmax_topk_head(q, lmk, lse_swa, K, S, W, is_training=False)
         if record:
             ev[2].record()
-        w = torch.softmax(torch.cat([scores, lse_swa.unsqueeze(-1)], dim=-1).float(), dim=-1).to(q.dtype)
+        w = pkg.chunk_weights(scores, lse_swa)
         if record:
             ev[3].record()
         ws = attn_mod.prepare_kv_workspace(L, k, v, HQ, K, S)
@@ -141,7 +141,7 @@ def bench_decode(pkg, dev, steps, warmup):
                                                    is_training=False)
         if record:
             ev[1].record()
-        w = torch.softmax(torch.cat([scores, lse_swa.unsqueeze(-1)], dim=-1).float(), dim=-1).to(q.dtype)
+        w = pkg.chunk_weights(scores, lse_swa)
         if record:
             ev[2].record()
         pkg.HiLS_block_M_head(q, kc, vc, w, idx, block_size=S, is_training=False)

@@ -37,17 +37,17 @@ typedef unsigned short bf16_t;  // raw bfloat16 bits
 
 __device__ __forceinline__ float bf2f(bf16_t x) { return __uint_as_float(((uint32_t)x) << 16); }
 
-// round-to-nearest-even fp32 -> bf16 (NaN stays NaN)
-__device__ __forceinline__ bf16_t f2bf(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
-}
+// round-to-nearest-even fp32 -> bf16 on the hardware converter (v_cvt_pk_bf16_f32)
+typedef __attribute__((ext_vector_type(2))) __bf16 hils_bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) float hils_f32x2_t;
 
 __device__ __forceinline__ uint32_t pack_bf2(float lo, float hi) {
-  return (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
+  const hils_f32x2_t x = {lo, hi};
+  const hils_bf16x2_t y = __builtin_convertvector(x, hils_bf16x2_t);
+  return *(const uint32_t*)&y;
 }
+
+__device__ __forceinline__ bf16_t f2bf(float f) { return (bf16_t)(pack_bf2(f, 0.f) & 0xffffu); }
 
 // unpack 8 bf16 held in a uint4 into 8 floats
 __device__ __forceinline__ void unpack8(const uint4& v, float* f) {

@@ -1,0 +1,161 @@
+// Inter-chunk softmax of the HiLS layer, fused: prior-bias gather + concatenation with the
+// local-branch LSE (+ the optional "softmax-1" zero logit) + softmax, one pass, bf16 out.
+#include "common.h"
+#include "../../include/hils_amd.h"
+
+#define GL_MAXK 64
+
+// One thread per (batch, query, query head) row.
+__global__ void __launch_bounds__(256)
+chunk_weights_kernel(const bf16_t* __restrict__ scores, const void* __restrict__ lse_ptr,
+                     int lse_bf16, const float* __restrict__ prior_b, const int32_t* __restrict__ indices,
+                     bf16_t* __restrict__ weights, long rows, int L, int HQ, int H, int N, int K,
+                     int softmax1) {
+  const long row = (long)blockIdx.x * blockDim.x + threadIdx.x;  // (b*L + t)*HQ + hq
+  if (row >= rows) return;
+  const int hq = (int)(row % HQ);
+  const long bt = row / HQ;
+  const long b = bt / L;
+  const int G = HQ / H;
+  const bf16_t* srow = scores + row * K;
+  float x[GL_MAXK];
+  const float lse_v = lse_bf16 ? bf2f(((const bf16_t*)lse_ptr)[row]) : ((const float*)lse_ptr)[row];
+  float m = lse_v;
+  if (softmax1) m = fmaxf(m, 0.f);
+#pragma unroll
+  for (int k = 0; k < GL_MAXK; ++k) {
+    if (k < K) {
+      float s = bf2f(srow[k]);
+      if (prior_b) {
+        int c = indices[(bt * H + hq / G) * (long)K + k];
+        c = c < 0 ? 0 : c;
+        // the layer adds the gathered bias after casting it to the scores' dtype
+        s = bf2f(f2bf(s + bf2f(f2bf(prior_b[(b * N + c) * (long)HQ + hq]))));
+      }
+      x[k] = s;
+      m = fmaxf(m, s);
+    }
+  }
+  const int NW = K + 1 + (softmax1 ? 1 : 0);
+  bf16_t* wrow = weights + row * NW;
+  if (m == HILS_NEG_INF) {  // every logit is -inf: softmax of that row is NaN in the reference
+    for (int k = 0; k < NW; ++k) wrow[k] = 0x7fc0;
+    return;
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < GL_MAXK; ++k)
+    if (k < K) { x[k] = __expf(x[k] - m); sum += x[k]; }
+  const float el = __expf(lse_v - m);
+  sum += el;
+  const float e0 = softmax1 ? __expf(0.f - m) : 0.f;
+  sum += e0;
+  const float inv = 1.f / sum;
+#pragma unroll
+  for (int k = 0; k < GL_MAXK; ++k)
+    if (k < K) wrow[k] = f2bf(x[k] * inv);
+  wrow[K] = f2bf(el * inv);
+  if (softmax1) wrow[K + 1] = f2bf(e0 * inv);
+}
+
+// Cooperative variant for K in {8, 16, 32, 64}: K/8 neighbouring lanes own one row (one
+// 16-byte load each), reductions run over those lanes with DPP, and the (K+1(+1))-wide output
+// rows of a wavefront, contiguous in memory, are staged in LDS and stored coalesced.
+template <int LPR>
+__global__ void __launch_bounds__(256)
+chunk_weights_rows_kernel(const bf16_t* __restrict__ scores, const void* __restrict__ lse_swa,
+                          int lse_bf16, const float* __restrict__ prior_b,
+                          const int32_t* __restrict__ indices, bf16_t* __restrict__ weights, long rows,
+                          int L, int HQ, int H, int N, int softmax1) {
+  constexpr int K = LPR * 8, RPW = 64 / LPR;
+  __shared__ bf16_t stage[4][RPW * (K + 2)];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane % LPR, rl = lane / LPR;
+  const long row0 = ((long)blockIdx.x * 4 + wave) * RPW;
+  const long row = row0 + rl;
+  const int NW = K + 1 + (softmax1 ? 1 : 0);
+  const bool valid = row < rows;
+  float x[8];
+  float lse = HILS_NEG_INF;
+  if (valid) {
+    const uint4 v = *(const uint4*)(scores + row * K + sub * 8);
+    unpack8(v, x);
+    lse = lse_bf16 ? bf2f(((const bf16_t*)lse_swa)[row]) : ((const float*)lse_swa)[row];
+    if (prior_b) {
+      const int hq = (int)(row % HQ);
+      const long bt = row / HQ;
+      const long b = bt / L;
+      const int G = HQ / H;
+      const int32_t* ip = indices + (bt * H + hq / G) * (long)K + sub * 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        int c = ip[e];
+        c = c < 0 ? 0 : c;
+        x[e] = bf2f(f2bf(x[e] + bf2f(f2bf(prior_b[(b * N + c) * (long)HQ + hq]))));
+      }
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = HILS_NEG_INF;
+  }
+  float m = softmax1 ? fmaxf(lse, 0.f) : lse;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) m = fmaxf(m, x[e]);
+  if (LPR >= 2) m = fmaxf(m, __shfl_xor(m, 1, 64));
+  if (LPR >= 4) m = fmaxf(m, __shfl_xor(m, 2, 64));
+  if (LPR >= 8) m = fmaxf(m, __shfl_xor(m, 4, 64));
+  const bool dead = !(m > HILS_NEG_INF);  // all logits -inf: the reference's softmax gives NaN
+  float sum = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) { x[e] = dead ? 0.f : __expf(x[e] - m); sum += x[e]; }
+  if (LPR >= 2) sum += __shfl_xor(sum, 1, 64);
+  if (LPR >= 4) sum += __shfl_xor(sum, 2, 64);
+  if (LPR >= 8) sum += __shfl_xor(sum, 4, 64);
+  const float el = dead ? 0.f : __expf(lse - m);
+  const float e0 = (softmax1 && !dead) ? __expf(0.f - m) : 0.f;
+  const float inv = dead ? __uint_as_float(0x7fc00000u) : 1.f / (sum + el + e0);
+  bf16_t* st = stage[wave] + rl * NW;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) st[sub * 8 + e] = f2bf(dead ? inv : x[e] * inv);
+  if (sub == 0) {
+    st[K] = f2bf(dead ? inv : el * inv);
+    if (softmax1) st[K + 1] = f2bf(dead ? inv : e0 * inv);
+  }
+  // same wavefront wrote the slice: stores and loads of one wavefront stay in program order
+  long nrow = rows - row0;
+  if (nrow > RPW) nrow = RPW;
+  if (nrow <= 0) return;
+  const int total = (int)nrow * NW;
+  bf16_t* dst = weights + row0 * NW;
+  for (int i = lane; i < total; i += 64) dst[i] = stage[wave][i];
+}
+
+extern "C" int hils_chunk_weights(const void* scores, const void* lse_swa, int lse_bf16,
+                                  const float* prior_b, const int32_t* indices, void* weights, int B,
+                                  int L, int HQ, int H, int N, int K, int softmax1, void* stream) {
+  HILS_REQUIRE(scores && lse_swa && weights, "hils_chunk_weights: null pointer");
+  HILS_REQUIRE(!prior_b || indices, "hils_chunk_weights: prior_b needs indices");
+  HILS_REQUIRE(B > 0 && L > 0 && HQ > 0 && H > 0 && HQ % H == 0, "hils_chunk_weights: bad head counts");
+  HILS_REQUIRE(K >= 1 && K <= GL_MAXK, "hils_chunk_weights: K (%d) must be in 1..%d", K, GL_MAXK);
+  const long rows = (long)B * L * HQ;
+  const long nblk = (rows + 255) / 256;
+  HILS_REQUIRE(nblk <= 2147483647L, "hils_chunk_weights: grid too large");
+  if (K == 8 || K == 16 || K == 32 || K == 64) {
+    const int rpw = 64 / (K / 8);
+    const long nb = (rows + 4 * rpw - 1) / (4 * rpw);
+    HILS_REQUIRE(nb <= 2147483647L, "hils_chunk_weights: grid too large");
+#define GL_CALL(LPR_)                                                                              \
+  hipLaunchKernelGGL(chunk_weights_rows_kernel<LPR_>, dim3((unsigned)nb), dim3(256), 0,            \
+                     (hipStream_t)stream, (const bf16_t*)scores, lse_swa, lse_bf16, prior_b, indices, \
+                     (bf16_t*)weights, rows, L, HQ, H, N, softmax1)
+    if (K == 8) GL_CALL(1); else if (K == 16) GL_CALL(2); else if (K == 32) GL_CALL(4); else GL_CALL(8);
+#undef GL_CALL
+    HILS_CHECK_LAUNCH("hils_chunk_weights");
+    return HILS_OK;
+  }
+  hipLaunchKernelGGL(chunk_weights_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16_t*)scores, lse_swa, lse_bf16, prior_b, indices, (bf16_t*)weights, rows, L, HQ, H,
+                     N, K, softmax1);
+  HILS_CHECK_LAUNCH("hils_chunk_weights");
+  return HILS_OK;
+}

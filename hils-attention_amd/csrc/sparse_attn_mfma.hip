@@ -207,7 +207,11 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
 
   const float bound = wsum * vm;
   float fx_scale = 1.f;
-  if (bound > 0.f && bound < 3.0e38f) fx_scale = ldexpf(1.f, 28 - ilogbf(bound));
+  if (bound > 0.f && bound < 3.0e38f) {
+    int e2 = 28 - ilogbf(bound);
+    e2 = e2 > 90 ? 90 : (e2 < -90 ? -90 : e2);
+    fx_scale = ldexpf(1.f, e2);
+  }
   const float fx_inv = 1.f / fx_scale;
   const float c2 = dm.sm_scale * HILS_LOG2E;
   const int qs = r / G, g = r - qs * G;
@@ -317,7 +321,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
       sum += __shfl_xor(sum, 32, 64);
       if (lse && rvalid && j == 0)
         lse[((b * dm.L + t) * (long)dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
-      const float f = wr / sum;
+      const float f = wr * fx_scale / sum;  // fixed-point scale (a power of two) folded into P
       // P as the A operand of O = P V: k-step s takes tokens of accumulator tiles 2s, 2s+1
       bf16x8_t ap[2];
 #pragma unroll
@@ -345,7 +349,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s], vb[dt][s], acc, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (rv[i]) atomicAdd(&o_acc[rb[i] + dt * 16 + r], __float2int_rn(acc[i] * fx_scale));
+          if (rv[i]) atomicAdd(&o_acc[rb[i] + dt * 16 + r], __float2int_rn(acc[i]));
       }
     }
   }

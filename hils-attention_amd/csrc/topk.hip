@@ -7,6 +7,7 @@
 // recomputes the logits, forms max_g(logit - lse_total), parks the pooled scores of a
 // segment of chunks in LDS and lets one wavefront per query pick the top-k with a
 // bitwise threshold search on order-preserving integer keys.  Ties: lower index wins.
+#include <stdlib.h>
 #include "decode_rows.h"
 #include "../../include/hils_amd.h"
 
@@ -122,7 +123,7 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                 int32_t* __restrict__ indices, bf16_t* __restrict__ scores,
                 float* __restrict__ lse_total_out, float* __restrict__ sel_logits_out,
                 int L, int N, int h_kv, int G, int topk, int block_size, int window_size,
-                int causal, int q_offset, int per_qhead, float sm_scale) {
+                int causal, int q_offset, int per_qhead, float sm_scale, int dbg) {
   constexpr int D = KS * 32;
   __shared__ float pooled[TOPK_QT][TOPK_NSEG];
   __shared__ float cand_s[TOPK_QT][TOPK_MAXK];
@@ -226,6 +227,7 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       }
     }
   }
+  if (dbg == 1) return;
   // combine over the 16 columns of a lane group, then over the 4 wavefronts
 #pragma unroll
   for (int g = 0; g < GMAX; ++g) {
@@ -345,6 +347,7 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       }
     }
     __syncthreads();
+    if (dbg == 2) return;
     const int ns = blk_end * 16 - seg_base;
     for (int qi = wave; qi < TOPK_QT; qi += 4) {
       if (t0 + qi < L) {
@@ -355,6 +358,7 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     __syncthreads();
   }
 
+  if (dbg == 3) return;
   // ---------------- epilogue: indices and raw scaled scores ----------------
   for (int qi = wave; qi < TOPK_QT; qi += 4) {
     const int tq = t0 + qi;
@@ -362,25 +366,40 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     const int nc = ncand_s[qi];
     int32_t* irow = indices + ((b * L + tq) * (long)h_kv + hk) * topk;
     for (int k = lane; k < topk; k += 64) irow[k] = (k < nc) ? cand_i[qi][k] : -1;
-    for (int p = lane; p < topk * G; p += 64) {
-      const int g = p / topk, k = p - g * topk;
-      float val = HILS_NEG_INF;
-      if (k < nc) {
-        const int c = cand_i[qi][k];
-        const bf16_t* qr = q + (((b * L + tq) * h_kv + hk) * (long)G + g) * D;
-        const bf16_t* kr = lmks + ((b * N + c) * (long)lmk_h + (per_qhead ? hk * G + g : hk)) * D;
-        float a = 0.f;
+    // raw scaled scores at the selected chunks: one MFMA chain per 16 slots with the
+    // selected chunk keys as rows and the G query heads as columns
+    bf16x8_t bq[KS];
 #pragma unroll
-        for (int d8 = 0; d8 < D / 8; ++d8) {
-          float fq[8], fk[8];
-          unpack8(*(const uint4*)(qr + d8 * 8), fq);
-          unpack8(*(const uint4*)(kr + d8 * 8), fk);
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (col < G) v = *(const uint4*)(q + (((b * L + tq) * h_kv + hk) * (long)G + col) * D + ks * 32 + grp * 8);
+      bq[ks] = *(bf16x8_t*)&v;
+    }
+    const int ntile = (topk + 15) / 16;
+    const int g_loops = per_qhead ? G : 1;
+    const long srow = ((b * L + tq) * (long)h_kv + hk) * G;
+    for (int gq = 0; gq < g_loops; ++gq) {
+      for (int tile = 0; tile < ntile; ++tile) {
+        const int slot_r = tile * 16 + col;
+        const int c = (slot_r < nc) ? cand_i[qi][slot_r] : -1;
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int j = 0; j < 8; ++j) a = fmaf(fq[j], fk[j], a);
+        for (int ks = 0; ks < KS; ++ks) {
+          uint4 v = make_uint4(0, 0, 0, 0);
+          if (c >= 0)
+            v = *(const uint4*)(lmks + ((b * N + c) * (long)lmk_h + (per_qhead ? hk * G + gq : hk)) * D + ks * 32 + grp * 8);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8_t*)&v, bq[ks], acc, 0, 0, 0);
         }
-        val = a * sm_scale;
+        const bool mine = per_qhead ? (col == gq) : (col < G);
+        if (mine) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int slot = tile * 16 + grp * 4 + i;
+            if (slot < topk)
+              scores[(srow + col) * topk + slot] = f2bf(slot < nc ? __fmul_rn(acc[i], sm_scale) : HILS_NEG_INF);
+          }
+        }
       }
-      scores[((((b * L + tq) * (long)h_kv + hk) * G + g)) * topk + k] = f2bf(val);
     }
   }
 }
@@ -395,7 +414,7 @@ static int launch_topk(int D, dim3 grid, hipStream_t st, const bf16_t* q, const 
   hipLaunchKernelGGL((topk_fwd_kernel<GMAX, KS_>), grid, dim3(TOPK_THREADS), 0, st, q, lmks,     \
                      lse_swa, bias, gumbel, drop_mask, indices, scores, lse_total, sel_logits, L, \
                      N, h_kv, G, topk, block_size, window_size, causal, q_offset, per_qhead,     \
-                     sm_scale)
+                     sm_scale, getenv("HILS_DBG") ? atoi(getenv("HILS_DBG")) : 0)
   switch (D) {
     case 64: HILS_TOPK_LAUNCH(2); break;
     case 128: HILS_TOPK_LAUNCH(4); break;

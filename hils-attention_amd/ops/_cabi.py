@@ -27,6 +27,7 @@ SIGNATURES = {
     "hils_sparse_attn_fwd": [_P] * 9 + [_I] * 13 + [_F, _I, _F, _P],
     "hils_pack_kv_chunks": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
     "hils_sparse_attn_bwd": [_P] * 12 + [_I] * 12 + [_F, _I, _F, _P],
+    "hils_chunk_weights": [_P, _P, _I, _P, _P, _P] + [_I] * 7 + [_P],
     "hils_chunk_logz_fwd": [_P, _P, _P] + [_I] * 7 + [_F, _I, _P],
     "hils_chunk_logz_bwd_dq": [_P] * 5 + [_I] * 7 + [_F, _P],
     "hils_chunk_logz_bwd_dk": [_P] * 5 + [_I] * 7 + [_F, _P],

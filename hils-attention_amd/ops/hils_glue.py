@@ -1,0 +1,40 @@
+"""Fused inter-chunk softmax of the HiLS layer (forward / inference).
+
+The reference computes it with torch ops inside the layer
+(models/FlashHiLS/hils_attention.py:585-610): gather the prior bias at the selected chunks,
+add it to the scores, concatenate the local-branch LSE (and a zero logit when
+``enable_softmax1``), softmax, cast to the hidden dtype.  ``chunk_weights`` does that in one
+kernel; column K is the weight of the local (sliding-window) branch.
+"""
+import torch
+
+from . import _cabi
+
+
+def chunk_weights(scores, lse_swa, prior_b=None, indices=None, enable_softmax1=False):
+    """scores (B,L,HQ,K) bf16, lse_swa (B,L,HQ) -> weights (B,L,HQ,K+1(+1)) bf16.
+    ``prior_b`` (B,N,HQ) with ``indices`` (B,L,H,K) adds the gathered prior bias first.
+    Forward only: inputs that require grad are rejected."""
+    _cabi.require_gpu_bf16("chunk_weights", scores)
+    if torch.is_grad_enabled() and (scores.requires_grad or lse_swa.requires_grad):
+        raise RuntimeError("chunk_weights is forward-only; use the torch ops of the layer for training")
+    B, L, HQ, K = scores.shape
+    lse = lse_swa.reshape(B, L, HQ).contiguous()
+    if lse.dtype not in (torch.bfloat16, torch.float32):
+        lse = lse.float()
+    H, N = HQ, 1
+    pb = idx = None
+    if prior_b is not None:
+        assert indices is not None, "prior_b needs the selected indices"
+        H = indices.shape[2]
+        N = prior_b.shape[1]
+        assert prior_b.shape == (B, N, HQ), f"prior_b shape {tuple(prior_b.shape)} != {(B, N, HQ)}"
+        assert indices.shape == (B, L, H, K)
+        pb = prior_b.float().contiguous()
+        idx = indices.to(torch.int32).contiguous()
+    out = torch.empty((B, L, HQ, K + 1 + (1 if enable_softmax1 else 0)), dtype=scores.dtype,
+                      device=scores.device)
+    _cabi.call("hils_chunk_weights", _cabi.ptr(scores.contiguous()), _cabi.ptr(lse),
+               int(lse.dtype == torch.bfloat16), _cabi.ptr(pb),
+               _cabi.ptr(idx), _cabi.ptr(out), B, L, HQ, H, N, K, int(bool(enable_softmax1)))
+    return out

@@ -82,6 +82,18 @@ int hils_topk_bwd(const void* g_scores, const void* q, const void* lmks, const i
                   void* dq, float* dlmk, int B, int L, int N, int h_kv, int G, int D, int topk,
                   int per_qhead, float sm_scale, void* stream);
 
+/* ---- inter-chunk softmax (layer glue) ------------------------------------------ */
+
+/* chunk_weights = softmax([scores_1..K (+ prior_b gathered at the indices), lse_swa (, 0)]).
+ * Replaces the gather / cat / F.softmax glue of models/FlashHiLS/hils_attention.py:585-610
+ * (forward only).  scores (B,L,HQ,K) bf16; lse_swa (B,L,HQ) fp32, or bf16 when lse_bf16 != 0;
+ * prior_b (B,N,HQ) fp32 or
+ * NULL; indices (B,L,H,K) int32 (needed with prior_b) -> weights (B,L,HQ,K+1(+1)) bf16, the
+ * local-branch weight in column K, the softmax-1 sink (softmax1 != 0) in column K+1. */
+int hils_chunk_weights(const void* scores, const void* lse_swa, int lse_bf16, const float* prior_b,
+                       const int32_t* indices, void* weights, int B, int L, int HQ, int H, int N,
+                       int K, int softmax1, void* stream);
+
 /* ---- sparse attention over the selected chunks ------------------------------ */
 
 /* Forward.  Replaces hierarchical_sparse_attention_block_M_reuseIndices behind

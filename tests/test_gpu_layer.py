@@ -36,3 +36,31 @@ def test_config1_layer_forward(pkg, orc, dev):
     assert_close_bf16(o, o_ref, "layer output")
     agree = (idx.cpu() == ref["indices"]).float().mean().item()
     assert agree > 0.97, f"index agreement with the fp32 oracle {agree:.4f}"
+
+
+def test_chunk_weights_kernel(pkg, orc, dev):
+    """Fused inter-chunk softmax against the layer's torch glue restated in the oracle."""
+    note("chunk_weights")
+    torch.manual_seed(3)
+    for K in (16, 32, 12):
+        _chunk_weights_case(pkg, orc, dev, K)
+
+
+def _chunk_weights_case(pkg, orc, dev, K):
+    B, L, HQ, H, N = 2, 301, 8, 2, 40
+    scores = torch.randn(B, L, HQ, K).bfloat16()
+    scores[:, :5, :, 7:] = float("-inf")
+    lse = torch.randn(B, L, HQ).bfloat16()
+    idx = torch.randint(-1, N, (B, L, H, K), dtype=torch.int32)
+    pb = torch.randn(B, N, HQ)
+    for prior, s1 in ((False, False), (True, False), (False, True), (True, True)):
+        w = pkg.chunk_weights(scores.to(dev), lse.to(dev), pb.to(dev) if prior else None,
+                              idx.to(dev) if prior else None, enable_softmax1=s1)
+        ref = orc.inter_chunk_softmax(scores, lse, pb.bfloat16() if prior else None, idx if prior else None,
+                                      softmax1=s1)
+        assert w.dtype == torch.bfloat16 and w.shape == ref.shape
+        assert_close_bf16(w, ref, f"chunk_weights prior={prior} softmax1={s1}", max_abs=8e-3)
+    w32 = pkg.chunk_weights(scores.to(dev), lse.float().to(dev))
+    assert torch.equal(w32, pkg.chunk_weights(scores.to(dev), lse.to(dev)))
+    with pytest.raises(RuntimeError):
+        pkg.chunk_weights(scores.to(dev).requires_grad_(), lse.to(dev))
