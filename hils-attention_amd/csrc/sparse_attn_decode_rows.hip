@@ -9,6 +9,9 @@
 #include "../../include/hils_amd.h"
 
 #define DR_THREADS 256
+#ifndef DR_MINW
+#define DR_MINW 4
+#endif
 #define DR_WAVES (DR_THREADS / 64)
 #define DR_S 64
 
@@ -18,7 +21,7 @@ struct DrDims {
 };
 
 template <int D, int GMAX>
-__global__ void __launch_bounds__(DR_THREADS, 4)
+__global__ void __launch_bounds__(DR_THREADS, DR_MINW)
 sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                const bf16_t* __restrict__ v, const bf16_t* __restrict__ weights,
                                const int32_t* __restrict__ indices, bf16_t* __restrict__ o,
@@ -26,7 +29,10 @@ sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   constexpr int LR = D / 8;        // lanes per token row
   constexpr int TPI = 64 / LR;     // token rows per load instruction
   constexpr int NI = DR_S / TPI;   // load instructions per chunk
-  constexpr int GI = 4;            // load instructions per pipelined group
+#ifndef DR_GI
+#define DR_GI 4
+#endif
+  constexpr int GI = DR_GI;        // load instructions per pipelined group
   constexpr int NG = NI / GI;      // groups per chunk
   extern __shared__ float o_s[];   // [wave][G][D] partial outputs
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;

@@ -7,7 +7,6 @@
 // recomputes the logits, forms max_g(logit - lse_total), parks the pooled scores of a
 // segment of chunks in LDS and lets one wavefront per query pick the top-k with a
 // bitwise threshold search on order-preserving integer keys.  Ties: lower index wins.
-#include <stdlib.h>
 #include "decode_rows.h"
 #include "../../include/hils_amd.h"
 
@@ -38,10 +37,12 @@ __device__ __forceinline__ float key_score(uint32_t k) {
 // One wavefront selects the top-K of (previous candidates) U (segment scores).
 // cand_* hold the previous winners in ascending index order (ncand of them, all with
 // an index below seg_base); seg holds ns pooled scores of chunks seg_base..seg_base+ns-1.
+// With KEYS the segment already holds order-preserving keys instead of floats.
 // With seg_idx the chunk index of seg[i] is seg_idx[i] (ascending in i) instead of seg_base + i.
 // The winners are written back to cand_* in ascending index order; returns the count.
 // The K-th largest key is found bit by bit; the bits all valid keys share are skipped, and
 // every count is a per-lane tally plus one DPP reduction (no scalar dependency per slot).
+template <bool KEYS = false>
 __device__ int wave_select(const float* seg, int ns, int seg_base, float* cand_s, int* cand_i,
                            int ncand, int K, const int* seg_idx = nullptr) {
   const int lane = threadIdx.x & 63;
@@ -55,7 +56,7 @@ __device__ int wave_select(const float* seg, int ns, int seg_base, float* cand_s
 #pragma unroll
   for (int s = 0; s < TOPK_SLOTS; ++s) {
     const int i = s * 64 + lane;
-    key[s + 1] = (i < ns) ? score_key(seg[i]) : 0u;
+    key[s + 1] = (i < ns) ? (KEYS ? ((const uint32_t*)seg)[i] : score_key(seg[i])) : 0u;
   }
   const int nslot = (ns + 63) / 64 + 1;
   int tl = 0;
@@ -123,7 +124,7 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                 int32_t* __restrict__ indices, bf16_t* __restrict__ scores,
                 float* __restrict__ lse_total_out, float* __restrict__ sel_logits_out,
                 int L, int N, int h_kv, int G, int topk, int block_size, int window_size,
-                int causal, int q_offset, int per_qhead, float sm_scale, int dbg) {
+                int causal, int q_offset, int per_qhead, float sm_scale) {
   constexpr int D = KS * 32;
   __shared__ float pooled[TOPK_QT][TOPK_NSEG];
   __shared__ float cand_s[TOPK_QT][TOPK_MAXK];
@@ -157,6 +158,165 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   }
   const int nblk = (tile_lim + 15) / 16;
 
+  // ---------------- register path: G <= 4 and at most 512 visible chunks ----------------
+  // One MFMA pass: wavefront w takes chunk blocks w, w+4, ... (at most 8), the query tile
+  // is read from LDS as the A operand, and the 16x16 logit tiles of all G heads stay in
+  // registers until the pooled score max_g(logit - lse_total) is written.
+  bool use_reg = false;
+  if constexpr (GMAX <= 4) {
+    use_reg = nblk <= 32;
+    if (use_reg) {
+      constexpr int QROW = D + 8;  // padded row (bf16 elements) of the staged query tile
+      __shared__ bf16_t q_lds[TOPK_QT * GMAX * QROW];
+      for (int i = tid; i < TOPK_QT * G * (D / 8); i += TOPK_THREADS) {
+        const int rowi = i / (D / 8), d8 = i - rowi * (D / 8);
+        const int qi = rowi / G, g = rowi - qi * G;
+        const int tq = t0 + qi;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (tq < L) v = *(const uint4*)(q + (((b * L + tq) * h_kv + hk) * (long)G + g) * D + d8 * 8);
+        *(uint4*)(q_lds + (qi * GMAX + g) * QROW + d8 * 8) = v;
+      }
+      if (tid < TOPK_QT) ncand_s[tid] = 0;
+      __syncthreads();
+      auto load_b = [&](int blk, int g, uint4* dst) {
+        const int c = blk * 16 + col;
+        const int lh = per_qhead ? hk * G + g : hk;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          dst[ks] = make_uint4(0, 0, 0, 0);
+          if (c < N) dst[ks] = *(const uint4*)(lmks + ((b * N + c) * (long)lmk_h + lh) * D + ks * 32 + grp * 8);
+        }
+      };
+      float xs[8][GMAX][4];
+      float m4[GMAX][4];
+#pragma unroll
+      for (int g = 0; g < GMAX; ++g)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) m4[g][i] = HILS_NEG_INF;
+      uint4 bcur[KS], bnext[KS];
+      if (!per_qhead && wave < nblk) load_b(wave, 0, bcur);
+#pragma unroll
+      for (int bi = 0; bi < 8; ++bi) {
+        const int blk = wave + bi * 4;
+        if (blk >= nblk) break;
+        if (!per_qhead && blk + 4 < nblk) load_b(blk + 4, 0, bnext);
+        const int c = blk * 16 + col;
+        const bool cvalid = c < N;
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g) {
+          if (g < G) {
+            if (per_qhead) load_b(blk, g, bcur);
+            f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+              const uint4 av = *(const uint4*)(q_lds + (col * GMAX + g) * QROW + ks * 32 + grp * 8);
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&av, *(bf16x8_t*)&bcur[ks], acc, 0, 0, 0);
+            }
+            float add = 0.f, gum = 0.f;
+            if (cvalid && bias) add = bias[((b * N + c) * (long)h_kv + hk) * G + g];
+            if (cvalid && gumbel) gum = gumbel[(long)(hk * G + g) * N + c];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              float x = __fmul_rn(acc[i], sm_scale);
+              if (bias) x = __fadd_rn(x, add);
+              if (gumbel) x = __fadd_rn(x, gum);
+              if (!(cvalid && c < lim[i])) x = HILS_NEG_INF;
+              xs[bi][g][i] = x;
+              m4[g][i] = fmaxf(m4[g][i], x);
+            }
+          }
+        }
+        if (!per_qhead) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) bcur[ks] = bnext[ks];
+        }
+      }
+      // log-sum-exp per (query, g): this lane's blocks, the 16 columns of the lane group
+      // (one DPP row), then the 4 wavefronts through LDS
+#pragma unroll
+      for (int g = 0; g < GMAX; ++g) {
+        if (g < G) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float m = m4[g][i];
+            m = fmaxf(m, __shfl_xor(m, 1, 64));
+            m = fmaxf(m, __shfl_xor(m, 2, 64));
+            m = fmaxf(m, __shfl_xor(m, 4, 64));
+            m = fmaxf(m, __shfl_xor(m, 8, 64));
+            float l = 0.f;
+            if (m > HILS_NEG_INF) {
+#pragma unroll
+              for (int bi = 0; bi < 8; ++bi)
+                if (wave + bi * 4 < nblk) l += __expf(xs[bi][g][i] - m);
+            }
+            l = row_sum<16>(l);
+            if (col == 0) {
+              part_m[wave][g][grp * 4 + i] = m;
+              part_l[wave][g][grp * 4 + i] = l;
+            }
+          }
+        }
+      }
+      __syncthreads();
+      for (int p = tid; p < G * TOPK_QT; p += TOPK_THREADS) {
+        const int g = p / TOPK_QT, qi = p - g * TOPK_QT;
+        float m = HILS_NEG_INF, l = 0.f;
+        for (int w = 0; w < 4; ++w) {
+          const float m2 = part_m[w][g][qi], l2 = part_l[w][g][qi];
+          const float mn = fmaxf(m, m2);
+          if (mn > HILS_NEG_INF) {
+            l = l * __expf(m - mn) + l2 * __expf(m2 - mn);
+            m = mn;
+          }
+        }
+        const float lse_hils = (l > 0.f) ? m + logf(l) : HILS_NEG_INF;
+        const int tq = t0 + qi;
+        float tot = HILS_NEG_INF;
+        if (tq < L) {
+          const long o = ((b * L + tq) * (long)h_kv + hk) * G + g;
+          tot = logaddexp_f(lse_swa[o], lse_hils);
+          if (lse_total_out) lse_total_out[o] = tot;
+        }
+        lse_tot[g][qi] = tot;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int bi = 0; bi < 8; ++bi) {
+        const int blk = wave + bi * 4;
+        if (blk >= nblk) break;
+        const int c = blk * 16 + col;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tq = t0 + grp * 4 + i;
+          float best = HILS_NEG_INF;
+#pragma unroll
+          for (int g = 0; g < GMAX; ++g) {
+            if (g < G) {
+              const float x = xs[bi][g][i];
+              if (sel_logits_out && c < N && tq < L)
+                sel_logits_out[(((b * L + tq) * (long)h_kv + hk) * G + g) * N + c] = x;
+              const float nrm = (x == HILS_NEG_INF) ? HILS_NEG_INF : __fsub_rn(x, lse_tot[g][grp * 4 + i]);
+              best = fmaxf(best, nrm);
+            }
+          }
+          if (drop_mask && best > HILS_NEG_INF && tq < L && c < N &&
+              drop_mask[(b * L + tq) * (long)N + c] != 0)
+            best = HILS_NEG_INF;
+          pooled[grp * 4 + i][c] = best;
+        }
+      }
+      __syncthreads();
+      const int ns = nblk * 16;
+      for (int qi = wave; qi < TOPK_QT; qi += 4) {
+        if (t0 + qi < L) {
+          const int nc = wave_select(pooled[qi], ns, 0, cand_s[qi], cand_i[qi], 0, topk);
+          if (lane == 0) ncand_s[qi] = nc;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  if (!use_reg) {
   // A operands: row (lane & 15) = query t0 + row of head g, 8 consecutive d per k-step
   bf16x8_t afrag[GMAX][KS];
   {
@@ -227,7 +387,6 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       }
     }
   }
-  if (dbg == 1) return;
   // combine over the 16 columns of a lane group, then over the 4 wavefronts
 #pragma unroll
   for (int g = 0; g < GMAX; ++g) {
@@ -347,7 +506,6 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       }
     }
     __syncthreads();
-    if (dbg == 2) return;
     const int ns = blk_end * 16 - seg_base;
     for (int qi = wave; qi < TOPK_QT; qi += 4) {
       if (t0 + qi < L) {
@@ -358,7 +516,8 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     __syncthreads();
   }
 
-  if (dbg == 3) return;
+  }
+
   // ---------------- epilogue: indices and raw scaled scores ----------------
   for (int qi = wave; qi < TOPK_QT; qi += 4) {
     const int tq = t0 + qi;
@@ -414,7 +573,7 @@ static int launch_topk(int D, dim3 grid, hipStream_t st, const bf16_t* q, const 
   hipLaunchKernelGGL((topk_fwd_kernel<GMAX, KS_>), grid, dim3(TOPK_THREADS), 0, st, q, lmks,     \
                      lse_swa, bias, gumbel, drop_mask, indices, scores, lse_total, sel_logits, L, \
                      N, h_kv, G, topk, block_size, window_size, causal, q_offset, per_qhead,     \
-                     sm_scale, getenv("HILS_DBG") ? atoi(getenv("HILS_DBG")) : 0)
+                     sm_scale)
   switch (D) {
     case 64: HILS_TOPK_LAUNCH(2); break;
     case 128: HILS_TOPK_LAUNCH(4); break;
