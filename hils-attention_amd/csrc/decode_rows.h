@@ -42,6 +42,19 @@ __device__ __forceinline__ int wave_sum_i(int x) {
          __builtin_amdgcn_readlane(x, 32) + __builtin_amdgcn_readlane(x, 48);
 }
 
+// wavefront-wide unsigned maximum, result uniform
+__device__ __forceinline__ uint32_t wave_max_u(uint32_t v) {
+  uint32_t x = v, y;
+  y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, true);  x = x > y ? x : y;
+  y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true);  x = x > y ? x : y;
+  y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x141, 0xF, 0xF, true); x = x > y ? x : y;
+  y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x140, 0xF, 0xF, true); x = x > y ? x : y;
+  const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)x, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)x, 16);
+  const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)x, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)x, 48);
+  const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+  return ab > cd ? ab : cd;
+}
+
 // wavefront-wide bitwise AND / OR, result uniform
 __device__ __forceinline__ uint32_t wave_and_u(uint32_t v) {
   int x = (int)v;

@@ -7,6 +7,7 @@
 // recomputes the logits, forms max_g(logit - lse_total), parks the pooled scores of a
 // segment of chunks in LDS and lets one wavefront per query pick the top-k with a
 // bitwise threshold search on order-preserving integer keys.  Ties: lower index wins.
+#include <type_traits>
 #include "decode_rows.h"
 #include "../../include/hils_amd.h"
 
@@ -34,18 +35,46 @@ __device__ __forceinline__ float key_score(uint32_t k) {
   return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
+// K-th largest of one value per lane by a bitwise threshold search.  Every non-zero x lies in
+// [lo, hi] and at least K lanes hold a non-zero x; the leading bits lo and hi share are
+// skipped.  Counting is one ballot + scalar popcount per bit.  Returns T with
+// count(x >= T) >= K and count(x > T) < K (T need not be one of the values when exactly K
+// values are >= T).
+__device__ __forceinline__ uint32_t lane_kth_largest(uint32_t x, uint32_t lo, uint32_t hi, int K) {
+  const uint32_t diff = lo ^ hi;
+  if (diff == 0u) return lo;
+  const int top = 31 - __clz((int)diff);
+  uint32_t T = (top == 31) ? 0u : (lo & ~((2u << top) - 1u));
+  for (int bit = top; bit >= 0; --bit) {
+    const uint32_t c = T | (1u << bit);
+    const int cnt = __popcll(__ballot(x >= c));
+    if (cnt >= K) {
+      T = c;
+      if (cnt == K) break;
+    }
+  }
+  return T;
+}
+
 // One wavefront selects the top-K of (previous candidates) U (segment scores).
 // cand_* hold the previous winners in ascending index order (ncand of them, all with
 // an index below seg_base); seg holds ns pooled scores of chunks seg_base..seg_base+ns-1.
 // With KEYS the segment already holds order-preserving keys instead of floats.
 // With seg_idx the chunk index of seg[i] is seg_idx[i] (ascending in i) instead of seg_base + i.
 // The winners are written back to cand_* in ascending index order; returns the count.
-// The K-th largest key is found bit by bit; the bits all valid keys share are skipped, and
-// every count is a per-lane tally plus one DPP reduction (no scalar dependency per slot).
+//
+// Fast path: the K-th largest of the 64 per-lane maxima is a lower bound of the K-th largest
+// key with at least K keys above it; the keys that reach it (about 1.3 K for K = 32 of 512)
+// are compacted to one per lane through a 64-entry scratch (scr_*, by default cand_*, which
+// must then hold 64 entries) and the exact threshold is searched on those with ballots.
+// If more than 64 keys reach the bound, the K-th largest key is found bit by bit over all
+// slots (per-lane tallies plus one DPP reduction per bit).
 template <bool KEYS = false>
-__device__ int wave_select(const float* seg, int ns, int seg_base, float* cand_s, int* cand_i,
-                           int ncand, int K, const int* seg_idx = nullptr) {
+__device__ __forceinline__ int wave_select(const float* seg, int ns, int seg_base, float* cand_s,
+                                           int* cand_i, int ncand, int K, const int* seg_idx = nullptr,
+                                           float* scr_s = nullptr, int* scr_i = nullptr) {
   const int lane = threadIdx.x & 63;
+  if (!scr_s) { scr_s = cand_s; scr_i = cand_i; }
   uint32_t key[TOPK_SLOTS + 1];
   int cidx = -1;
   key[0] = 0u;
@@ -59,20 +88,76 @@ __device__ int wave_select(const float* seg, int ns, int seg_base, float* cand_s
     key[s + 1] = (i < ns) ? (KEYS ? ((const uint32_t*)seg)[i] : score_key(seg[i])) : 0u;
   }
   const int nslot = (ns + 63) / 64 + 1;
-  int tl = 0;
-  uint32_t ka = 0xffffffffu, ko = 0u;
+  auto index_of = [&](int s) -> int {
+    return (s == 0) ? cidx : (seg_idx ? seg_idx[(s - 1) * 64 + lane] : seg_base + (s - 1) * 64 + lane);
+  };
+  const unsigned long long lt = (1ull << lane) - 1ull;
+  uint32_t lm = 0u;  // largest key of this lane
 #pragma unroll
-  for (int s = 0; s <= TOPK_SLOTS; ++s)
-    if (key[s] != 0u) { ++tl; ka &= key[s]; ko |= key[s]; }
-  const int total = wave_sum_i(tl);
-  uint32_t T = 1u;  // every valid key is >= 1
-  if (total > K) {
+  for (int s = 0; s <= TOPK_SLOTS; ++s) lm = key[s] > lm ? key[s] : lm;
+  const bool many = __popcll(__ballot(lm != 0u)) >= K;  // at least K lanes hold a valid key
+  uint32_t thr = 1u, hi = 0u;  // every valid key is >= 1
+  if (many) {
+    hi = wave_max_u(lm);
+    const uint32_t lo = ~wave_max_u(lm ? ~lm : 0u);  // smallest non-zero lane maximum
+    thr = lane_kth_largest(lm, lo, hi, K);
+  }
+  // compact the keys >= thr, in index order, to one per lane
+  uint32_t* cs_u = (uint32_t*)scr_s;
+  int pos = 0;
+#pragma unroll
+  for (int s = 0; s <= TOPK_SLOTS; ++s) {
+    if (s < nslot) {
+      const bool pred = key[s] >= thr;
+      const unsigned long long m = __ballot(pred);
+      if (pred) {
+        const int o = pos + __popcll(m & lt);
+        if (o < 64) {
+          cs_u[o] = key[s];
+          scr_i[o] = index_of(s);
+        }
+      }
+      pos += __popcll(m);
+    }
+  }
+  if (pos <= 64) {
+    __builtin_amdgcn_wave_barrier();
+    uint32_t ck = 0u;
+    int ci = -1;
+    if (lane < pos) {
+      ck = cs_u[lane];
+      ci = scr_i[lane];
+    }
+    bool sel = lane < pos;  // pos <= K: every valid key wins
+    if (pos > K) {
+      if (!many) hi = wave_max_u(ck);
+      const uint32_t T = lane_kth_largest(ck, thr, hi, K);
+      const int need = K - __popcll(__ballot(ck > T));  // ties with the threshold to take, lowest index first
+      const unsigned long long eq = __ballot(ck == T);
+      sel = (ck > T) || (ck == T && __popcll(eq & lt) < need);
+    }
+    const unsigned long long sm = __ballot(sel);
+    __builtin_amdgcn_wave_barrier();
+    if (sel) {
+      const int o = __popcll(sm & lt);
+      cand_s[o] = key_score(ck);
+      cand_i[o] = ci;
+    }
+    return __popcll(sm);
+  }
+  // general search over all slots (more than 64 > K keys reach the bound); the bits all
+  // valid keys share are skipped
+  uint32_t T;
+  {
+    uint32_t ka = 0xffffffffu, ko = 0u;
+#pragma unroll
+    for (int s = 0; s <= TOPK_SLOTS; ++s)
+      if (key[s] != 0u) { ka &= key[s]; ko |= key[s]; }
     ka = wave_and_u(ka);
     ko = wave_or_u(ko);
     const uint32_t diff = ka ^ ko;  // bits in which the valid keys differ
-    if (diff == 0u) {
-      T = ka;
-    } else {
+    T = ka;
+    if (diff != 0u) {
       const int top = 31 - __clz((int)diff);
       T = (top == 31) ? 0u : (ka & ~((2u << top) - 1u));  // the shared leading bits
       for (int bit = top; bit >= 0; --bit) {
@@ -93,8 +178,7 @@ __device__ int wave_select(const float* seg, int ns, int seg_base, float* cand_s
   for (int s = 0; s <= TOPK_SLOTS; ++s) gl += (key[s] > T) ? 1 : 0;
   const int gt = wave_sum_i(gl);
   int need = K - gt;  // ties with the threshold still to take, lowest index first
-  int pos = 0;
-  const unsigned long long lt = (1ull << lane) - 1ull;
+  pos = 0;
 #pragma unroll
   for (int s = 0; s <= TOPK_SLOTS; ++s) {
     if (s < nslot) {
@@ -105,8 +189,7 @@ __device__ int wave_select(const float* seg, int ns, int seg_base, float* cand_s
       if (sel) {
         const int o = pos + __popcll(sm & lt);
         cand_s[o] = key_score(key[s]);
-        cand_i[o] = (s == 0) ? cidx
-                             : (seg_idx ? seg_idx[(s - 1) * 64 + lane] : seg_base + (s - 1) * 64 + lane);
+        cand_i[o] = index_of(s);
       }
       pos += __popcll(sm);
       const int took = __popcll(eq);
@@ -158,165 +241,6 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   }
   const int nblk = (tile_lim + 15) / 16;
 
-  // ---------------- register path: G <= 4 and at most 512 visible chunks ----------------
-  // One MFMA pass: wavefront w takes chunk blocks w, w+4, ... (at most 8), the query tile
-  // is read from LDS as the A operand, and the 16x16 logit tiles of all G heads stay in
-  // registers until the pooled score max_g(logit - lse_total) is written.
-  bool use_reg = false;
-  if constexpr (GMAX <= 4) {
-    use_reg = nblk <= 32;
-    if (use_reg) {
-      constexpr int QROW = D + 8;  // padded row (bf16 elements) of the staged query tile
-      __shared__ bf16_t q_lds[TOPK_QT * GMAX * QROW];
-      for (int i = tid; i < TOPK_QT * G * (D / 8); i += TOPK_THREADS) {
-        const int rowi = i / (D / 8), d8 = i - rowi * (D / 8);
-        const int qi = rowi / G, g = rowi - qi * G;
-        const int tq = t0 + qi;
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (tq < L) v = *(const uint4*)(q + (((b * L + tq) * h_kv + hk) * (long)G + g) * D + d8 * 8);
-        *(uint4*)(q_lds + (qi * GMAX + g) * QROW + d8 * 8) = v;
-      }
-      if (tid < TOPK_QT) ncand_s[tid] = 0;
-      __syncthreads();
-      auto load_b = [&](int blk, int g, uint4* dst) {
-        const int c = blk * 16 + col;
-        const int lh = per_qhead ? hk * G + g : hk;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          dst[ks] = make_uint4(0, 0, 0, 0);
-          if (c < N) dst[ks] = *(const uint4*)(lmks + ((b * N + c) * (long)lmk_h + lh) * D + ks * 32 + grp * 8);
-        }
-      };
-      float xs[8][GMAX][4];
-      float m4[GMAX][4];
-#pragma unroll
-      for (int g = 0; g < GMAX; ++g)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) m4[g][i] = HILS_NEG_INF;
-      uint4 bcur[KS], bnext[KS];
-      if (!per_qhead && wave < nblk) load_b(wave, 0, bcur);
-#pragma unroll
-      for (int bi = 0; bi < 8; ++bi) {
-        const int blk = wave + bi * 4;
-        if (blk >= nblk) break;
-        if (!per_qhead && blk + 4 < nblk) load_b(blk + 4, 0, bnext);
-        const int c = blk * 16 + col;
-        const bool cvalid = c < N;
-#pragma unroll
-        for (int g = 0; g < GMAX; ++g) {
-          if (g < G) {
-            if (per_qhead) load_b(blk, g, bcur);
-            f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-              const uint4 av = *(const uint4*)(q_lds + (col * GMAX + g) * QROW + ks * 32 + grp * 8);
-              acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&av, *(bf16x8_t*)&bcur[ks], acc, 0, 0, 0);
-            }
-            float add = 0.f, gum = 0.f;
-            if (cvalid && bias) add = bias[((b * N + c) * (long)h_kv + hk) * G + g];
-            if (cvalid && gumbel) gum = gumbel[(long)(hk * G + g) * N + c];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              float x = __fmul_rn(acc[i], sm_scale);
-              if (bias) x = __fadd_rn(x, add);
-              if (gumbel) x = __fadd_rn(x, gum);
-              if (!(cvalid && c < lim[i])) x = HILS_NEG_INF;
-              xs[bi][g][i] = x;
-              m4[g][i] = fmaxf(m4[g][i], x);
-            }
-          }
-        }
-        if (!per_qhead) {
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks) bcur[ks] = bnext[ks];
-        }
-      }
-      // log-sum-exp per (query, g): this lane's blocks, the 16 columns of the lane group
-      // (one DPP row), then the 4 wavefronts through LDS
-#pragma unroll
-      for (int g = 0; g < GMAX; ++g) {
-        if (g < G) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            float m = m4[g][i];
-            m = fmaxf(m, __shfl_xor(m, 1, 64));
-            m = fmaxf(m, __shfl_xor(m, 2, 64));
-            m = fmaxf(m, __shfl_xor(m, 4, 64));
-            m = fmaxf(m, __shfl_xor(m, 8, 64));
-            float l = 0.f;
-            if (m > HILS_NEG_INF) {
-#pragma unroll
-              for (int bi = 0; bi < 8; ++bi)
-                if (wave + bi * 4 < nblk) l += __expf(xs[bi][g][i] - m);
-            }
-            l = row_sum<16>(l);
-            if (col == 0) {
-              part_m[wave][g][grp * 4 + i] = m;
-              part_l[wave][g][grp * 4 + i] = l;
-            }
-          }
-        }
-      }
-      __syncthreads();
-      for (int p = tid; p < G * TOPK_QT; p += TOPK_THREADS) {
-        const int g = p / TOPK_QT, qi = p - g * TOPK_QT;
-        float m = HILS_NEG_INF, l = 0.f;
-        for (int w = 0; w < 4; ++w) {
-          const float m2 = part_m[w][g][qi], l2 = part_l[w][g][qi];
-          const float mn = fmaxf(m, m2);
-          if (mn > HILS_NEG_INF) {
-            l = l * __expf(m - mn) + l2 * __expf(m2 - mn);
-            m = mn;
-          }
-        }
-        const float lse_hils = (l > 0.f) ? m + logf(l) : HILS_NEG_INF;
-        const int tq = t0 + qi;
-        float tot = HILS_NEG_INF;
-        if (tq < L) {
-          const long o = ((b * L + tq) * (long)h_kv + hk) * G + g;
-          tot = logaddexp_f(lse_swa[o], lse_hils);
-          if (lse_total_out) lse_total_out[o] = tot;
-        }
-        lse_tot[g][qi] = tot;
-      }
-      __syncthreads();
-#pragma unroll
-      for (int bi = 0; bi < 8; ++bi) {
-        const int blk = wave + bi * 4;
-        if (blk >= nblk) break;
-        const int c = blk * 16 + col;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int tq = t0 + grp * 4 + i;
-          float best = HILS_NEG_INF;
-#pragma unroll
-          for (int g = 0; g < GMAX; ++g) {
-            if (g < G) {
-              const float x = xs[bi][g][i];
-              if (sel_logits_out && c < N && tq < L)
-                sel_logits_out[(((b * L + tq) * (long)h_kv + hk) * G + g) * N + c] = x;
-              const float nrm = (x == HILS_NEG_INF) ? HILS_NEG_INF : __fsub_rn(x, lse_tot[g][grp * 4 + i]);
-              best = fmaxf(best, nrm);
-            }
-          }
-          if (drop_mask && best > HILS_NEG_INF && tq < L && c < N &&
-              drop_mask[(b * L + tq) * (long)N + c] != 0)
-            best = HILS_NEG_INF;
-          pooled[grp * 4 + i][c] = best;
-        }
-      }
-      __syncthreads();
-      const int ns = nblk * 16;
-      for (int qi = wave; qi < TOPK_QT; qi += 4) {
-        if (t0 + qi < L) {
-          const int nc = wave_select(pooled[qi], ns, 0, cand_s[qi], cand_i[qi], 0, topk);
-          if (lane == 0) ncand_s[qi] = nc;
-        }
-      }
-      __syncthreads();
-    }
-  }
-  if (!use_reg) {
   // A operands: row (lane & 15) = query t0 + row of head g, 8 consecutive d per k-step
   bf16x8_t afrag[GMAX][KS];
   {
@@ -516,8 +440,6 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     __syncthreads();
   }
 
-  }
-
   // ---------------- epilogue: indices and raw scaled scores ----------------
   for (int qi = wave; qi < TOPK_QT; qi += 4) {
     const int tq = t0 + qi;
@@ -561,6 +483,323 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       }
     }
   }
+}
+
+// ---------------------------------------------------------------------------
+// Row-packed variant for 2 <= G <= 4 with one chunk key per KV head: the 16 rows of an MFMA
+// tile are (16/GMAX queries) x (GMAX query heads), so the max over the heads of a query is
+// a max over accumulator registers of one lane, and a wavefront needs nobody else: one
+// wavefront per workgroup owns 8 consecutive queries of a (batch, KV head), keeps their
+// query rows in registers as A operands and streams the chunk keys as B operands.
+// Pass 1 accumulates sum exp2(y - ref) per lane against a reference that is only moved when
+// a logit exceeds it by 2^40 (one exp2 per logit); pass 2 recomputes the logits, writes the
+// pooled scores of a segment of chunks to LDS and selects per query.
+// ---------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float x) {
+  const int v = __builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), CTRL, 0xF, 0xF, false);
+  return fmaxf(x, __int_as_float(v));
+}
+__device__ __forceinline__ float row_max16(float x) {
+  x = dpp_max<0xB1>(x);
+  x = dpp_max<0x4E>(x);
+  x = dpp_max<0x141>(x);
+  x = dpp_max<0x140>(x);
+  return x;
+}
+
+template <int GMAX, int KS, bool PLAIN>
+__global__ void __launch_bounds__(64)
+topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
+                     const float* __restrict__ lse_swa, const float* __restrict__ bias,
+                     const float* __restrict__ gumbel, const int32_t* __restrict__ drop_mask,
+                     int32_t* __restrict__ indices, bf16_t* __restrict__ scores,
+                     float* __restrict__ lse_total_out, float* __restrict__ sel_logits_out,
+                     int L, int N, int h_kv, int G, int topk, int block_size, int window_size,
+                     int causal, int q_offset, float sm_scale, int segw) {
+  // PLAIN: no bias, Gumbel noise, drop mask or logit export (the inference path)
+  constexpr int D = KS * 32;
+  constexpr int QPT = 16 / GMAX;            // queries per 16-row tile
+  constexpr int NT = (GMAX == 4) ? 2 : 1;   // tiles per wavefront
+  constexpr int NQ = NT * QPT;              // queries per wavefront (8)
+  constexpr int GPL = 4 / GMAX;             // queries per lane and tile
+  extern __shared__ float tr_smem[];
+  const int stride = segw + 16;             // row stride: lane groups on disjoint banks
+  float* pooled = tr_smem;                  // NQ x stride
+  float* scr_s = pooled + NQ * stride;      // 64-entry compaction scratch of the selection
+  int* scr_i = (int*)(scr_s + 64);
+  float* car_s = (float*)(scr_i + 64);      // NQ x topk winners carried across segments
+  int* car_i = (int*)(car_s + NQ * topk);
+
+  const int lane = threadIdx.x, col = lane & 15, j = lane >> 4;
+  const int t0 = blockIdx.x * NQ;
+  const int hk = blockIdx.y;
+  const long b = blockIdx.z;
+
+  auto limit_of = [&](int tq) -> int {
+    int lm = causal ? visible_limit(tq + q_offset, window_size, block_size) : N;
+    return lm < 0 ? 0 : (lm > N ? N : lm);
+  };
+  // accumulator row 4j+i of tile nt <-> (query t0 + nt*QPT + (4j+i)/GMAX, head (4j+i)%GMAX)
+  int lim[NT][4];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 4 * j + i;
+      const int tq = t0 + nt * QPT + r / GMAX;
+      lim[nt][i] = (tq < L && (r % GMAX) < G) ? limit_of(tq) : 0;
+    }
+  const int t_last = (t0 + NQ - 1 < L) ? t0 + NQ - 1 : L - 1;
+  const int nblk = (limit_of(t_last) + 15) / 16;
+  // blocks below nfull are visible to every row: no masking there
+  const int nfull = (G == GMAX && t0 + NQ <= L) ? limit_of(t0) / 16 : 0;
+
+  bf16x8_t afrag[NT][KS];
+  {
+    const int r = lane & 15;
+    const int g = r % GMAX;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int tq = t0 + nt * QPT + r / GMAX;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (tq < L && g < G)
+          v = *(const uint4*)(q + (((b * L + tq) * h_kv + hk) * (long)G + g) * D + ks * 32 + j * 8);
+        afrag[nt][ks] = *(bf16x8_t*)&v;
+      }
+    }
+  }
+  // chunk keys as B operands; rows beyond N are read from row N-1 and masked by the caller
+  const long bstride = (long)h_kv * D;  // elements between consecutive chunk keys
+  const bf16_t* bbase = lmks + (b * N * (long)h_kv + hk) * D + j * 8;
+  auto load_b = [&](int blk, uint4* dst) {
+    int c = blk * 16 + col;
+    c = c < N ? c : N - 1;
+    const bf16_t* p = bbase + c * bstride;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) dst[ks] = *(const uint4*)(p + ks * 32);
+  };
+  auto scores_of = [&](const uint4* bb, f32x4_t* acc) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      acc[nt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[nt][ks], *(const bf16x8_t*)&bb[ks], acc[nt], 0, 0, 0);
+    }
+  };
+  // exact fp32 logit of accumulator element i of chunk c (before masking)
+  auto logit = [&](float acc, int c, int i) -> float {
+    float x = __fmul_rn(acc, sm_scale);
+    if (!PLAIN) {
+      const int g = (4 * j + i) % GMAX;
+      if (c < N && g < G) {
+        if (bias) x = __fadd_rn(x, bias[((b * N + c) * (long)h_kv + hk) * G + g]);
+        if (gumbel) x = __fadd_rn(x, gumbel[(long)(hk * G + g) * N + c]);
+      }
+    }
+    return x;
+  };
+  // run body(bb, blk, masked) over blocks [lo, hi): two operand buffers in turn, the next
+  // block's keys always in flight (a load past hi reads a clamped row and is never used)
+  auto for_range = [&](int lo, int hi, auto masked_t, auto& body) {
+    if (lo >= hi) return;
+    uint4 b0[KS], b1[KS];
+    load_b(lo, b0);
+    int blk = lo;
+    for (; blk + 1 < hi; blk += 2) {
+      load_b(blk + 1, b1);
+      body(b0, blk, masked_t);
+      load_b(blk + 2, b0);
+      body(b1, blk + 1, masked_t);
+    }
+    if (blk < hi) body(b0, blk, masked_t);
+  };
+  auto for_blocks = [&](int lo, int hi, auto body) {
+    const int mid = nfull < hi ? (nfull > lo ? nfull : lo) : hi;  // masking starts here
+    for_range(lo, mid, std::false_type{}, body);
+    for_range(mid, hi, std::true_type{}, body);
+  };
+
+  // ---------------- pass 1: sum of exp2(y - ref) per lane and row ----------------
+  const float c2 = sm_scale * HILS_LOG2E;
+  float ref[NT][4], l[NT][4];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { ref[nt][i] = -1e30f; l[nt][i] = 0.f; }
+  for_blocks(0, nblk, [&](const uint4* bb, int blk, auto masked_t) {
+    constexpr bool MASKED = decltype(masked_t)::value;
+    const int c = blk * 16 + col;
+    f32x4_t acc[NT];
+    scores_of(bb, acc);
+    float y[NT][4], d[NT][4];
+    float dmax = HILS_NEG_INF;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float yy = PLAIN ? acc[nt][i] * c2 : logit(acc[nt][i], c, i) * HILS_LOG2E;
+        if (MASKED && !(c < lim[nt][i])) yy = HILS_NEG_INF;
+        y[nt][i] = yy;
+        d[nt][i] = yy - ref[nt][i];
+        dmax = fmaxf(dmax, d[nt][i]);
+      }
+    if (__any(dmax > 40.f)) {  // move the reference of the rows that outgrew it
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (d[nt][i] > 40.f) {
+            l[nt][i] *= __builtin_amdgcn_exp2f(ref[nt][i] - y[nt][i]);
+            ref[nt][i] = y[nt][i];
+            d[nt][i] = 0.f;
+          }
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) l[nt][i] += __builtin_amdgcn_exp2f(d[nt][i]);
+  });
+  // combine the 16 lanes (chunk columns) of each row; lse_total per row
+  float lse_tot[NT][4];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float M = row_max16(ref[nt][i]);
+      const float ls = row_sum<16>(l[nt][i] * __builtin_amdgcn_exp2f(ref[nt][i] - M));
+      const float lse_hils = (ls > 0.f) ? (M + __builtin_amdgcn_logf(ls)) * HILS_LN2 : HILS_NEG_INF;
+      const int r = 4 * j + i;
+      const int tq = t0 + nt * QPT + r / GMAX, g = r % GMAX;
+      float tot = HILS_NEG_INF;
+      if (tq < L && g < G) {
+        const long o = ((b * L + tq) * (long)h_kv + hk) * G + g;
+        tot = logaddexp_f(lse_swa[o], lse_hils);
+        if (lse_total_out && col == 0) lse_total_out[o] = tot;
+      }
+      lse_tot[nt][i] = tot;
+    }
+
+  // ---------------- pass 2: pooled scores per segment + selection ----------------
+  int ncand_v = 0;  // lane qi holds the number of winners of query qi so far
+  const int bps = segw / 16;
+  const int nseg = (nblk + bps - 1) / bps;
+  for (int seg = 0; seg < nseg; ++seg) {
+    const int seg_base = seg * segw;
+    const int blk_end = ((seg + 1) * bps < nblk) ? (seg + 1) * bps : nblk;
+    for_blocks(seg * bps, blk_end, [&](const uint4* bb, int blk, auto masked_t) {
+      constexpr bool MASKED = decltype(masked_t)::value;
+      const int c = blk * 16 + col;
+      f32x4_t acc[NT];
+      scores_of(bb, acc);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        float nrm[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float x = logit(acc[nt][i], c, i);
+          if (MASKED && !(c < lim[nt][i])) x = HILS_NEG_INF;
+          if (!PLAIN) {
+            if (sel_logits_out && c < N) {
+              const int r = 4 * j + i;
+              const int tq = t0 + nt * QPT + r / GMAX, g = r % GMAX;
+              if (tq < L && g < G) sel_logits_out[(((b * L + tq) * (long)h_kv + hk) * G + g) * N + c] = x;
+            }
+          }
+          nrm[i] = __fsub_rn(x, lse_tot[nt][i]);
+          if (MASKED || !PLAIN) nrm[i] = (x == HILS_NEG_INF) ? HILS_NEG_INF : nrm[i];
+        }
+#pragma unroll
+        for (int u = 0; u < GPL; ++u) {
+          float best = nrm[u * GMAX];
+#pragma unroll
+          for (int e = 1; e < GMAX; ++e) best = fmaxf(best, nrm[u * GMAX + e]);  // fmaxf ignores a NaN operand
+          const int ql = nt * QPT + (4 * j) / GMAX + u;
+          if (!PLAIN) {
+            if (drop_mask && best > HILS_NEG_INF && t0 + ql < L && c < N &&
+                drop_mask[(b * L + t0 + ql) * (long)N + c] != 0)
+              best = HILS_NEG_INF;
+          }
+          pooled[ql * stride + (c - seg_base)] = best;
+        }
+      }
+    });
+    __builtin_amdgcn_wave_barrier();
+    const int ns = blk_end * 16 - seg_base;
+#pragma unroll 1
+    for (int qi = 0; qi < NQ; ++qi) {
+      if (t0 + qi < L) {
+        const int prev = __builtin_amdgcn_readlane(ncand_v, qi);
+        const int nc = wave_select(pooled + qi * stride, ns, seg_base, car_s + qi * topk, car_i + qi * topk,
+                                   prev, topk, nullptr, scr_s, scr_i);
+        if (lane == qi) ncand_v = nc;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+
+  // ---------------- epilogue: indices and raw scaled scores ----------------
+#pragma unroll 1
+  for (int qi = 0; qi < NQ; ++qi) {
+    const int tq = t0 + qi;
+    if (tq >= L) break;
+    const int nc = __builtin_amdgcn_readlane(ncand_v, qi);
+    int32_t* irow = indices + ((b * L + tq) * (long)h_kv + hk) * topk;
+    for (int k = lane; k < topk; k += 64) irow[k] = (k < nc) ? car_i[qi * topk + k] : -1;
+  }
+  // Raw scaled scores at the winners: the query rows are still the A operands; the B operand
+  // gathers 16 winning chunk keys of one query, and the rows of that query are kept.
+  // Four queries (gathers) are in flight at a time.
+  const int ntile = (topk + 15) / 16;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+    for (int qq = 0; qq < QPT; qq += 4) {
+#pragma unroll 1
+      for (int tile = 0; tile < ntile; ++tile) {
+        uint4 bg[4][KS];
+        int ncs[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int qi = nt * QPT + qq + u;
+          ncs[u] = __builtin_amdgcn_readlane(ncand_v, qi);
+          const int slot = tile * 16 + col;
+          int c = (slot < ncs[u]) ? car_i[qi * topk + slot] : 0;  // chunk 0 stands in; masked at the store
+          const bf16_t* p = bbase + c * bstride;
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) bg[u][ks] = *(const uint4*)(p + ks * 32);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int qi = nt * QPT + qq + u;
+          const int tq = t0 + qi;
+          f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[nt][ks], *(const bf16x8_t*)&bg[u][ks], acc, 0, 0, 0);
+          const int slot = tile * 16 + col;
+          if (tq < L && slot < topk) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int r = 4 * j + i;
+              const int g = r % GMAX;
+              if (r / GMAX == qq + u && g < G)
+                scores[(((b * L + tq) * (long)h_kv + hk) * G + g) * topk + slot] =
+                    f2bf(slot < ncs[u] ? __fmul_rn(acc[i], sm_scale) : HILS_NEG_INF);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+static int topk_rows_segw(int N) {
+  const int n16 = (N + 15) / 16 * 16;
+  return n16 < TOPK_NSEG ? n16 : TOPK_NSEG;
 }
 
 template <int GMAX>
@@ -971,6 +1210,33 @@ extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_s
                                  sel_logits, (float*)workspace, B, L, N, h_kv, G, D, topk, block_size,
                                  window_size, causal, q_offset, per_qhead, sm_scale, st))
       return rc2;
+    HILS_CHECK_LAUNCH("hils_topk_fwd");
+    return HILS_OK;
+  }
+  if (!per_qhead && G >= 2 && G <= 4 && (D == 64 || D == 128)) {
+    const int segw = topk_rows_segw(N);
+    const size_t smem = sizeof(float) * ((size_t)8 * (segw + 16) + 128 + (size_t)2 * 8 * topk);
+    dim3 grid_r((L + 7) / 8, h_kv, B);
+#define HILS_TOPK_ROWS(G_, KS_)                                                                     \
+  do {                                                                                             \
+    if (plain)                                                                                     \
+      hipLaunchKernelGGL((topk_fwd_rows_kernel<G_, KS_, true>), grid_r, dim3(64), smem, st,        \
+                         (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, gumbel, drop_mask,  \
+                         indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,     \
+                         block_size, window_size, causal, q_offset, sm_scale, segw);               \
+    else                                                                                           \
+      hipLaunchKernelGGL((topk_fwd_rows_kernel<G_, KS_, false>), grid_r, dim3(64), smem, st,       \
+                         (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, gumbel, drop_mask,  \
+                         indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,     \
+                         block_size, window_size, causal, q_offset, sm_scale, segw);               \
+  } while (0)
+    const bool plain = !bias && !gumbel && !drop_mask && !sel_logits;
+    if (G == 2) {
+      if (D == 64) HILS_TOPK_ROWS(2, 2); else HILS_TOPK_ROWS(2, 4);
+    } else {
+      if (D == 64) HILS_TOPK_ROWS(4, 2); else HILS_TOPK_ROWS(4, 4);
+    }
+#undef HILS_TOPK_ROWS
     HILS_CHECK_LAUNCH("hils_topk_fwd");
     return HILS_OK;
   }

@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 
 def run_case(pkg, orc, dev, B, L, N, h_kv, G, D, topk, S, W, seed=42, q_offset=0, training=True,
              use_bias=False, use_gumbel=False, use_drop=False, per_qhead=False, lse_mode="rand",
-             dup_keys=False, is_causal=True):
+             dup_keys=False, is_causal=True, one_kernel=False):
     note(f"topk B{B} L{L} N{N} hkv{h_kv} G{G} D{D} k{topk} S{S} W{W} off{q_offset} "
          f"bias{use_bias} gum{use_gumbel} drop{use_drop} pq{per_qhead} lse={lse_mode} dup{dup_keys}")
     gen = torch.Generator().manual_seed(seed)
@@ -37,7 +37,7 @@ def run_case(pkg, orc, dev, B, L, N, h_kv, G, D, topk, S, W, seed=42, q_offset=0
         u = torch.rand(1, 1, h_kv * G, N, generator=gen).clamp_(1e-20, 1 - 1e-7)
         gumbel = -torch.log(-torch.log(u))
     drop = (torch.rand(B, L, N, generator=gen) < 0.3).to(torch.int32) if use_drop else None
-    dbg = {}
+    dbg = {"no_workspace": True} if one_kernel else {}
     q_in = q if not per_qhead else q
     idx, scores = pkg.online_softmax_topk_head(
         q_in.to(dev), lmks.to(dev), lse_swa.to(dev), topk, S, W, is_causal=is_causal,
@@ -133,6 +133,50 @@ def test_topk_many_chunks_multi_segment(pkg, orc, dev):
              q_offset=1500 * 64, training=False)
     run_case(pkg, orc, dev, B=1, L=1, N=2048, h_kv=1, G=4, D=128, topk=64, S=64, W=1,
              q_offset=2048 * 64, training=False, dup_keys=True)
+
+
+def test_topk_one_kernel_path_many_chunks(pkg, orc, dev):
+    """The one-kernel path with more chunks than a selection segment, ragged query count,
+    exact ties, and every optional input (winners carried across segments)."""
+    run_case(pkg, orc, dev, B=1, L=21, N=1100, h_kv=2, G=4, D=128, topk=32, S=64, W=1,
+             q_offset=1100 * 64 - 21, training=False, dup_keys=True, one_kernel=True)
+    run_case(pkg, orc, dev, B=2, L=13, N=700, h_kv=1, G=2, D=64, topk=64, S=64, W=0, is_causal=False,
+             training=True, use_bias=True, use_gumbel=True, use_drop=True, one_kernel=True)
+    run_case(pkg, orc, dev, B=1, L=9, N=530, h_kv=1, G=3, D=64, topk=16, S=64, W=0, is_causal=False,
+             one_kernel=True)
+
+
+@pytest.mark.parametrize("G,D,L,N,topk,W", [(4, 128, 2050, 33, 32, 1), (2, 64, 777, 13, 8, 64),
+                                            (3, 128, 300, 5, 4, 1), (4, 64, 40, 600, 16, 1)])
+def test_topk_inference_variant_matches_export_variant(pkg, dev, G, D, L, N, topk, W):
+    """The kernel variant without logit export / bias / noise / drop mask (the one inference
+    runs) must give the same indices and scores as the exporting variant checked above."""
+    note(f"topk plain-vs-export G{G} D{D} L{L} N{N} k{topk} W{W}")
+    gen = torch.Generator().manual_seed(123)
+    h_kv = 2
+    q = torch.randn(1, L, h_kv, G, D, generator=gen).bfloat16().to(dev)
+    lmks = torch.randn(1, N, h_kv, D, generator=gen).bfloat16()
+    lmks[:, 1::2] = lmks[:, 0::2][:, : lmks[:, 1::2].shape[1]]  # exact ties
+    lmks = lmks.to(dev)
+    lse = (torch.randn(1, L, h_kv * G, generator=gen) * 3 + 5).to(dev)
+    off = max(0, N * 64 - L)
+    outs = []
+    for dbg in ({"no_workspace": True}, None):
+        if dbg is None:
+            from hils_attention_amd.ops import _cabi
+            idx = torch.empty(1, L, h_kv, topk, dtype=torch.int32, device=dev)
+            sc = torch.empty(1, L, h_kv, G, topk, dtype=torch.bfloat16, device=dev)
+            _cabi.call("hils_topk_fwd", _cabi.ptr(q), _cabi.ptr(lmks), _cabi.ptr(lse.view(1, L, h_kv, G).contiguous()),
+                       None, None, None, _cabi.ptr(idx), _cabi.ptr(sc), None, None, None, 1, L, N, h_kv, G, D,
+                       topk, 64, W, 1, off, 0, D ** -0.5)
+        else:
+            idx, sc = pkg.online_softmax_topk_head(q, lmks, lse, topk, 64, W, q_offset=off,
+                                                   is_training=False, _debug=dbg)
+            sc = sc.view(1, L, h_kv, G, topk)
+        torch.cuda.synchronize()
+        outs.append((idx.cpu(), sc.float().cpu()))
+    assert torch.equal(outs[0][0], outs[1][0]), "indices differ between kernel variants"
+    assert torch.equal(outs[0][1], outs[1][1]), "scores differ between kernel variants"
 
 
 def test_topk_tie_break_lower_index_wins(pkg, orc, dev):
