@@ -516,7 +516,7 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
                      int32_t* __restrict__ indices, bf16_t* __restrict__ scores,
                      float* __restrict__ lse_total_out, float* __restrict__ sel_logits_out,
                      int L, int N, int h_kv, int G, int topk, int block_size, int window_size,
-                     int causal, int q_offset, float sm_scale, int segw) {
+                     int causal, int q_offset, float sm_scale, int segw, int pool_floats) {
   // PLAIN: no bias, Gumbel noise, drop mask or logit export (the inference path)
   constexpr int D = KS * 32;
   constexpr int QPT = 16 / GMAX;            // queries per 16-row tile
@@ -525,8 +525,8 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
   constexpr int GPL = 4 / GMAX;             // queries per lane and tile
   extern __shared__ float tr_smem[];
   const int stride = segw + 16;             // row stride: lane groups on disjoint banks
-  float* pooled = tr_smem;                  // NQ x stride
-  float* scr_s = pooled + NQ * stride;      // 64-entry compaction scratch of the selection
+  float* pooled = tr_smem;                  // NQ x stride (pool_floats >= that, and >= the score staging)
+  float* scr_s = pooled + pool_floats;      // 64-entry compaction scratch of the selection
   int* scr_i = (int*)(scr_s + 64);
   float* car_s = (float*)(scr_i + 64);      // NQ x topk winners carried across segments
   int* car_i = (int*)(car_s + NQ * topk);
@@ -602,17 +602,30 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
     }
     return x;
   };
+  // blocks that lie wholly inside [0, N): uniform block address + a 32-bit lane offset
+  const char* ubase = (const char*)lmks + ((b * N * (long)h_kv + hk) * D) * 2;
+  const uint32_t lane_off = (uint32_t)((col * bstride + j * 8) * 2);
+  auto load_b_full = [&](int blk, uint4* dst) {
+    const char* p = ubase + (long)blk * (32 * bstride);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) dst[ks] = *(const uint4*)(p + lane_off + ks * 64);
+  };
   // run body(bb, blk, masked) over blocks [lo, hi): two operand buffers in turn, the next
-  // block's keys always in flight (a load past hi reads a clamped row and is never used)
+  // block's keys always in flight (a load past hi re-reads an earlier row and is never used)
   auto for_range = [&](int lo, int hi, auto masked_t, auto& body) {
+    constexpr bool MASKED = decltype(masked_t)::value;
     if (lo >= hi) return;
+    auto ld = [&](int blk, uint4* dst) {
+      if (MASKED) load_b(blk, dst);
+      else load_b_full(blk < hi ? blk : hi - 1, dst);
+    };
     uint4 b0[KS], b1[KS];
-    load_b(lo, b0);
+    ld(lo, b0);
     int blk = lo;
     for (; blk + 1 < hi; blk += 2) {
-      load_b(blk + 1, b1);
+      ld(blk + 1, b1);
       body(b0, blk, masked_t);
-      load_b(blk + 2, b0);
+      ld(blk + 2, b0);
       body(b1, blk + 1, masked_t);
     }
     if (blk < hi) body(b0, blk, masked_t);
@@ -625,6 +638,15 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
 
   // ---------------- pass 1: sum of exp2(y - ref) per lane and row ----------------
   const float c2 = sm_scale * HILS_LOG2E;
+  float swa[NT][4];  // lse_swa of this lane's rows (-inf for padding rows)
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 4 * j + i;
+      const int tq = t0 + nt * QPT + r / GMAX, g = r % GMAX;
+      swa[nt][i] = (tq < L && g < G) ? lse_swa[((b * L + tq) * (long)h_kv + hk) * G + g] : HILS_NEG_INF;
+    }
   float ref[NT][4], l[NT][4];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
@@ -663,7 +685,8 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
 #pragma unroll
       for (int i = 0; i < 4; ++i) l[nt][i] += __builtin_amdgcn_exp2f(d[nt][i]);
   });
-  // combine the 16 lanes (chunk columns) of each row; lse_total per row
+  // combine the 16 lanes (chunk columns) of each row; lse_total per row, in the log2 domain
+  // with the hardware exp2/log2 (absolute error ~1e-6, far inside the 1e-4 the LSE needs)
   float lse_tot[NT][4];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
@@ -671,15 +694,16 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
     for (int i = 0; i < 4; ++i) {
       const float M = row_max16(ref[nt][i]);
       const float ls = row_sum<16>(l[nt][i] * __builtin_amdgcn_exp2f(ref[nt][i] - M));
-      const float lse_hils = (ls > 0.f) ? (M + __builtin_amdgcn_logf(ls)) * HILS_LN2 : HILS_NEG_INF;
+      const float hils2 = (ls > 0.f) ? M + __builtin_amdgcn_logf(ls) : HILS_NEG_INF;
+      const float swa2 = swa[nt][i] * HILS_LOG2E;
+      const float mx = fmaxf(swa2, hils2), mn = fminf(swa2, hils2);
+      float tot2 = mx;
+      if (mn > HILS_NEG_INF) tot2 = mx + __builtin_amdgcn_logf(1.f + __builtin_amdgcn_exp2f(mn - mx));
+      const float tot = tot2 * HILS_LN2;
       const int r = 4 * j + i;
       const int tq = t0 + nt * QPT + r / GMAX, g = r % GMAX;
-      float tot = HILS_NEG_INF;
-      if (tq < L && g < G) {
-        const long o = ((b * L + tq) * (long)h_kv + hk) * G + g;
-        tot = logaddexp_f(lse_swa[o], lse_hils);
-        if (lse_total_out && col == 0) lse_total_out[o] = tot;
-      }
+      if (lse_total_out && col == 0 && tq < L && g < G)
+        lse_total_out[((b * L + tq) * (long)h_kv + hk) * G + g] = tot;
       lse_tot[nt][i] = tot;
     }
 
@@ -742,17 +766,31 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
   }
 
   // ---------------- epilogue: indices and raw scaled scores ----------------
-#pragma unroll 1
-  for (int qi = 0; qi < NQ; ++qi) {
-    const int tq = t0 + qi;
-    if (tq >= L) break;
-    const int nc = __builtin_amdgcn_readlane(ncand_v, qi);
-    int32_t* irow = indices + ((b * L + tq) * (long)h_kv + hk) * topk;
-    for (int k = lane; k < topk; k += 64) irow[k] = (k < nc) ? car_i[qi * topk + k] : -1;
+  // Indices: the winners sit in LDS as [query][topk]; 16-byte lane stores when rows allow it.
+  if ((topk & 3) == 0) {
+    const int per_q = topk / 4;
+    for (int e = lane; e < NQ * per_q; e += 64) {
+      const int qi = e / per_q, k0 = (e - qi * per_q) * 4;
+      const int nc = __shfl(ncand_v, qi, 64);
+      int4 v = *(const int4*)(car_i + qi * topk + k0);
+      v.x = (k0 + 0 < nc) ? v.x : -1;
+      v.y = (k0 + 1 < nc) ? v.y : -1;
+      v.z = (k0 + 2 < nc) ? v.z : -1;
+      v.w = (k0 + 3 < nc) ? v.w : -1;
+      if (t0 + qi < L) *(int4*)(indices + ((b * L + t0 + qi) * (long)h_kv + hk) * topk + k0) = v;
+    }
+  } else {
+    for (int e = lane; e < NQ * topk; e += 64) {
+      const int qi = e / topk, k = e - qi * topk;
+      const int nc = __shfl(ncand_v, qi, 64);
+      if (t0 + qi < L) indices[((b * L + t0 + qi) * (long)h_kv + hk) * topk + k] = (k < nc) ? car_i[e] : -1;
+    }
   }
   // Raw scaled scores at the winners: the query rows are still the A operands; the B operand
-  // gathers 16 winning chunk keys of one query, and the rows of that query are kept.
-  // Four queries (gathers) are in flight at a time.
+  // gathers 16 winning chunk keys of one query, and the rows of that query are kept.  Four
+  // queries (gathers) are in flight at a time.  The scores are staged in LDS (over the dead
+  // pooled rows) as [query][head][slot], the layout of the output, and stored in 16-byte pieces.
+  bf16_t* stage = (bf16_t*)pooled;
   const int ntile = (topk + 15) / 16;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
@@ -762,12 +800,12 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
       for (int tile = 0; tile < ntile; ++tile) {
         uint4 bg[4][KS];
         int ncs[4];
+        const int slot = tile * 16 + col;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
           const int qi = nt * QPT + qq + u;
           ncs[u] = __builtin_amdgcn_readlane(ncand_v, qi);
-          const int slot = tile * 16 + col;
-          int c = (slot < ncs[u]) ? car_i[qi * topk + slot] : 0;  // chunk 0 stands in; masked at the store
+          const int c = (slot < ncs[u]) ? car_i[qi * topk + slot] : 0;  // chunk 0 stands in; masked below
           const bf16_t* p = bbase + c * bstride;
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) bg[u][ks] = *(const uint4*)(p + ks * 32);
@@ -775,24 +813,37 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
           const int qi = nt * QPT + qq + u;
-          const int tq = t0 + qi;
           f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks)
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[nt][ks], *(const bf16x8_t*)&bg[u][ks], acc, 0, 0, 0);
-          const int slot = tile * 16 + col;
-          if (tq < L && slot < topk) {
+          if (slot < topk) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const int r = 4 * j + i;
               const int g = r % GMAX;
               if (r / GMAX == qq + u && g < G)
-                scores[(((b * L + tq) * (long)h_kv + hk) * G + g) * topk + slot] =
-                    f2bf(slot < ncs[u] ? __fmul_rn(acc[i], sm_scale) : HILS_NEG_INF);
+                stage[(qi * G + g) * topk + slot] = f2bf(slot < ncs[u] ? __fmul_rn(acc[i], sm_scale) : HILS_NEG_INF);
             }
           }
         }
       }
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+  const int row_e = G * topk;  // bf16 elements per query
+  if ((row_e & 7) == 0) {
+    const int per_q = row_e / 8;
+    for (int e = lane; e < NQ * per_q; e += 64) {
+      const int qi = e / per_q, part = e - qi * per_q;
+      if (t0 + qi < L)
+        *(uint4*)(scores + ((b * L + t0 + qi) * (long)h_kv + hk) * row_e + part * 8) =
+            *(const uint4*)(stage + qi * row_e + part * 8);
+    }
+  } else {
+    for (int e = lane; e < NQ * row_e; e += 64) {
+      const int qi = e / row_e;
+      if (t0 + qi < L) scores[((b * L + t0 + qi) * (long)h_kv + hk) * row_e + (e - qi * row_e)] = stage[e];
     }
   }
 }
@@ -1215,7 +1266,9 @@ extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_s
   }
   if (!per_qhead && G >= 2 && G <= 4 && (D == 64 || D == 128)) {
     const int segw = topk_rows_segw(N);
-    const size_t smem = sizeof(float) * ((size_t)8 * (segw + 16) + 128 + (size_t)2 * 8 * topk);
+    int pool_floats = 8 * (segw + 16);                              // pooled scores of 8 queries
+    if (pool_floats < 8 * 4 * topk / 2) pool_floats = 8 * 4 * topk / 2;  // bf16 score staging
+    const size_t smem = sizeof(float) * ((size_t)pool_floats + 128 + (size_t)2 * 8 * topk);
     dim3 grid_r((L + 7) / 8, h_kv, B);
 #define HILS_TOPK_ROWS(G_, KS_)                                                                     \
   do {                                                                                             \
@@ -1223,12 +1276,12 @@ extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_s
       hipLaunchKernelGGL((topk_fwd_rows_kernel<G_, KS_, true>), grid_r, dim3(64), smem, st,        \
                          (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, gumbel, drop_mask,  \
                          indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,     \
-                         block_size, window_size, causal, q_offset, sm_scale, segw);               \
+                         block_size, window_size, causal, q_offset, sm_scale, segw, pool_floats);  \
     else                                                                                           \
       hipLaunchKernelGGL((topk_fwd_rows_kernel<G_, KS_, false>), grid_r, dim3(64), smem, st,       \
                          (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, gumbel, drop_mask,  \
                          indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,     \
-                         block_size, window_size, causal, q_offset, sm_scale, segw);               \
+                         block_size, window_size, causal, q_offset, sm_scale, segw, pool_floats);  \
   } while (0)
     const bool plain = !bias && !gumbel && !drop_mask && !sel_logits;
     if (G == 2) {
