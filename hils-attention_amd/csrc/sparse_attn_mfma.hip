@@ -96,9 +96,9 @@ struct GaDims {
 // associative, so the result does not depend on the order in which wavefronts add.
 // The scale is chosen per workgroup from bound = max_row(sum_k |w|) * max_visited|V|, which
 // bounds every output element because each P row is a convex combination.
-template <int D, int DV, int G>
+template <int D, int DV, int G, bool SLOPE>
 __global__ void __launch_bounds__(GA_THREADS)
-sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kp,
+sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* __restrict__ kp,
                        const bf16_t* __restrict__ vp, const float* __restrict__ vmax,
                        const bf16_t* __restrict__ weights, const int32_t* __restrict__ indices,
                        const float* __restrict__ slope, bf16_t* __restrict__ o,
@@ -109,9 +109,9 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
   constexpr int MAXP = 8;       // pairs per thread: T*K <= MAXP * GA_THREADS
   extern __shared__ int smem_i[];
   const int R = dm.T * G;
-  int* o_acc = smem_i;                       // R x DV fixed point
-  int* cur = o_acc + (size_t)R * DV;         // nchunk: histogram -> running ends
-  int* pairs = cur + dm.nchunk;              // T*K pair ids grouped by chunk
+  int* o_acc = smem_i;                       // (R + 1) x DV fixed point; row R takes the padding rows of a tile
+  int* cur = o_acc + (size_t)(R + 1) * DV;   // nchunk: histogram -> running ends
+  int* pairs = cur + dm.nchunk;              // T*K pairs (query << 8 | slot) grouped by chunk
   __shared__ float red[32];
   __shared__ int scan_s[GA_WAVES];
   __shared__ int next_s;
@@ -136,15 +136,32 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
   for (int i = tid; i < R * DV; i += GA_THREADS) o_acc[i] = 0;
   for (int i = tid; i < dm.nchunk; i += GA_THREADS) cur[i] = 0;
   if (tid == 0) next_s = 0;
+  // Packed copy of this block's query rows: within the G heads of a (query, KV head) the
+  // 16-byte pieces are interleaved head-minor, [piece][head][8], so that the B-operand loads
+  // of the G lanes that hold the heads of one query are contiguous.  Only this workgroup
+  // reads what it writes here (made visible by the barriers below).
+  {
+    constexpr int PPR = D / 8;
+    for (int i = tid; i < dm.T * G * PPR; i += GA_THREADS) {
+      const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
+      const int g2 = rem / PPR, pc = rem - g2 * PPR;
+      if (t0 + ql < dm.L) {
+        const long blk_e = ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G) * D;
+        *(uint4*)(qp + blk_e + (pc * G + g2) * 8) = *(const uint4*)(q + blk_e + g2 * D + pc * 8);
+      }
+    }
+  }
   __syncthreads();
   // histogram of the selected chunks
-  int creg[MAXP];
+  int creg[MAXP], preg[MAXP];
 #pragma unroll
   for (int e = 0; e < MAXP; ++e) {
     const int i = tid + e * GA_THREADS;
     int c = -1;
+    preg[e] = 0;
     if (i < npair) {
       const int ql = i / K, slot = i - ql * K;
+      preg[e] = (ql << 8) | slot;
       const int t = t0 + ql;
       if (t < dm.L) {
         c = indices[((b * dm.L + t) * dm.H + hk) * (long)K + slot];
@@ -202,7 +219,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
   __syncthreads();
 #pragma unroll
   for (int e = 0; e < MAXP; ++e)
-    if (creg[e] >= 0) pairs[atomicAdd(&cur[creg[e]], 1)] = tid + e * GA_THREADS;
+    if (creg[e] >= 0) pairs[atomicAdd(&cur[creg[e]], 1)] = preg[e];
   __syncthreads();  // now chunk c owns pairs[cur[c-1] .. cur[c])
 
   const float bound = wsum * vm;
@@ -214,14 +231,19 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
   }
   const float fx_inv = 1.f / fx_scale;
   const float c2 = dm.sm_scale * HILS_LOG2E;
-  const int qs = r / G, g = r - qs * G;
+  const int qs = r / G, g = r - qs * G;  // this lane's row of a tile: query slot, head
   const int hq = hk * G + g;
-  const float sl = slope ? slope[hq] : 0.f;
+  const float sl = SLOPE ? slope[hq] : 0.f;
+  // rows of a tile are addressed from the block's first query with 32-bit element offsets
+  const bf16_t* qb = qp + ((b * dm.L + t0) * (long)dm.HQ + hk * G) * D;
+  const bf16_t* wb = weights + ((b * dm.L + t0) * (long)dm.HQ + hk * G) * dm.NW;
+  const int q_lane = (j * G + g) * 8, w_lane = g * dm.NW;
+  const int q_step = dm.HQ * D, w_step = dm.HQ * dm.NW;  // per query of the block
 
   for (;;) {
     int c = 0;
     if (lane == 0) c = atomicAdd(&next_s, 1);
-    c = __shfl(c, 0, 64);
+    c = __builtin_amdgcn_readfirstlane(c);
     if (c >= dm.nchunk) break;
     const int vs = c ? cur[c - 1] : 0, ve = cur[c];
     if (vs == ve) continue;
@@ -248,39 +270,43 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
         }
     }
 
-    // gathered query rows (B operands) and weights are loaded one tile ahead
-    auto load_tile = [&](int p, int& pid_o, uint4* bq_o, bf16_t& w_o) {
-      const int n = (ve - p < QT) ? ve - p : QT;
-      const bool rvalid = qs < n;
-      pid_o = pairs[p + (rvalid ? qs : 0)];
-      const int ql = pid_o / K, slot = pid_o - ql * K;
-      const long t = t0 + ql;
-      const bf16_t* qrow = q + ((b * dm.L + t) * (long)dm.HQ + hq) * D + j * 8;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        bq_o[ks] = make_uint4(0, 0, 0, 0);
-        if (rvalid) bq_o[ks] = *(const uint4*)(qrow + ks * 32);
-      }
-      w_o = 0;
-      if (rvalid) w_o = weights[((b * dm.L + t) * (long)dm.HQ + hq) * dm.NW + slot];
-    };
-    int pid_n;
+    // A tile is up to QT pairs of the visit.  Its gathered query rows (B operands), weights
+    // and output rows are fetched one tile ahead.  Padding rows of the last tile repeat the
+    // visit's first pair (finite arithmetic) and are accumulated into the spare row R.
+    // Query rows come from the packed copy, in which the G heads of a query are interleaved
+    // per 16-byte piece: the lanes of the G heads of one query read contiguous bytes.
     uint4 bq_n[KS];
-    bf16_t w_n;
-    load_tile(vs, pid_n, bq_n, w_n);
+    int w_n, pk_n;     // weight bits (loaded by lane group j == 0) and pair of this lane's row
+    int orow_n[4];     // o_acc element offsets of accumulator rows 4j..4j+3 (column r included)
+    auto load_tile = [&](int p) {
+      const int n = (ve - p < QT) ? ve - p : QT;
+      pk_n = pairs[p + (qs < n ? qs : 0)];
+      const bf16_t* qrow = qb + ((pk_n >> 8) * q_step + q_lane);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) bq_n[ks] = *(const uint4*)(qrow + ks * (4 * G * 8));
+      w_n = 0;
+      if (j == 0) w_n = wb[(pk_n >> 8) * w_step + w_lane + (pk_n & 255)];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int rr = 4 * j + i;
+        const int qsl = rr / G;
+        const int pk2 = pairs[p + (qsl < n ? qsl : 0)];
+        const int row = (qsl < n) ? (pk2 >> 8) * G + (rr - qsl * G) : R;
+        orow_n[i] = row * DV + r;
+      }
+    };
+    load_tile(vs);
     for (int p = vs; p < ve; p += QT) {
       const int n = (ve - p < QT) ? ve - p : QT;
-      // this lane's row of the tile: query slot r / G, head r % G
-      const bool rvalid = qs < n;
-      const int pid = pid_n;
-      const int ql = pid / K, slot = pid - ql * K;
-      const int t = t0 + ql;
-      const int row_base = (ql * G + g) * DV;
       bf16x8_t bq[KS];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) bq[ks] = *(bf16x8_t*)&bq_n[ks];
-      const float wr = bf2f(w_n);
-      if (p + QT < ve) load_tile(p + QT, pid_n, bq_n, w_n);
+      const int pk_c = pk_n, w_c = w_n;
+      int orow_c[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) orow_c[i] = orow_n[i];
+      if (p + QT < ve) load_tile(p + QT);
+      const float w_row = bf2f((bf16_t)__shfl(w_c, r, 64));
       f32x4_t st[4];
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) {
@@ -290,21 +316,19 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
           st[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[mt][ks], bq[ks], st[mt], 0, 0, 0);
       }
       // per-chunk softmax over the 64 tokens of row r: registers (mt, i) and lane groups j
-      float m = HILS_NEG_INF;
+      if (SLOPE) {
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
+        for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int tok = mt * 16 + j * 4 + i;
-          float x = st[mt][i];
-          if (slope) {
-            const int dist = GA_S - 2 - tok;
-            x -= sl * (float)(dist > 0 ? dist : 0);
+          for (int i = 0; i < 4; ++i) {
+            const int dist = GA_S - 2 - (mt * 16 + j * 4 + i);
+            st[mt][i] -= sl * (float)(dist > 0 ? dist : 0);
           }
-          if (dm.mask_last && tok == GA_S - 1) x = HILS_NEG_INF;
-          st[mt][i] = x;
-          m = fmaxf(m, x);
-        }
+      }
+      if (dm.mask_last && j == 3) st[3][3] = HILS_NEG_INF;  // token 63 = tile 3, lane group 3, register 3
+      float m = fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3]));
+#pragma unroll
+      for (int mt = 1; mt < 4; ++mt) m = fmaxf(fmaxf(m, fmaxf(st[mt][0], st[mt][1])), fmaxf(st[mt][2], st[mt][3]));
       m = fmaxf(m, __shfl_xor(m, 16, 64));
       m = fmaxf(m, __shfl_xor(m, 32, 64));
       const float mc = m * c2;
@@ -319,9 +343,11 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
         }
       sum += __shfl_xor(sum, 16, 64);
       sum += __shfl_xor(sum, 32, 64);
-      if (lse && rvalid && j == 0)
-        lse[((b * dm.L + t) * (long)dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
-      const float f = wr * fx_scale / sum;  // fixed-point scale (a power of two) folded into P
+      if (lse && qs < n && j == 0) {
+        const int ql = pk_c >> 8, slot = pk_c & 255;
+        lse[((b * dm.L + t0 + ql) * (long)dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
+      }
+      const float f = w_row * fx_scale / sum;  // fixed-point scale (a power of two) folded into P
       // P as the A operand of O = P V: k-step s takes tokens of accumulator tiles 2s, 2s+1
       bf16x8_t ap[2];
 #pragma unroll
@@ -333,14 +359,6 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
         x.w = pack_bf2(st[2 * s + 1][2] * f, st[2 * s + 1][3] * f);
         ap[s] = *(bf16x8_t*)&x;
       }
-      // rows 4j+i of an output tile belong to the lanes with (lane & 15) == 4j+i
-      int rb[4];
-      bool rv[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        rb[i] = __shfl(row_base, 4 * j + i, 64);
-        rv[i] = ((4 * j + i) / G) < n;
-      }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
@@ -348,8 +366,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
         for (int s = 0; s < 2; ++s)
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s], vb[dt][s], acc, 0, 0, 0);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (rv[i]) atomicAdd(&o_acc[rb[i] + dt * 16 + r], __float2int_rn(acc[i]));
+        for (int i = 0; i < 4; ++i) atomicAdd(&o_acc[orow_c[i] + dt * 16], __float2int_rn(acc[i]));
       }
     }
   }
@@ -371,11 +388,11 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
   }
 }
 
-template <int D, int DV, int G>
-static int ga_launch(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, const bf16_t* k,
-                     const bf16_t* vt, const float* vmax, const bf16_t* w, const int32_t* idx,
-                     const float* slope, bf16_t* o, float* lse, const GaDims& dm) {
-  auto kern = sparse_attn_fwd_gather<D, DV, G>;
+template <int D, int DV, int G, bool SLOPE>
+static int ga_launch_s(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, bf16_t* qp, const bf16_t* k,
+                       const bf16_t* vt, const float* vmax, const bf16_t* w, const int32_t* idx,
+                       const float* slope, bf16_t* o, float* lse, const GaDims& dm) {
+  auto kern = sparse_attn_fwd_gather<D, DV, G, SLOPE>;
   static size_t reserved = 0;  // per instantiation
   if (smem > reserved) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -385,21 +402,29 @@ static int ga_launch(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, co
     }
     reserved = smem;
   }
-  hipLaunchKernelGGL(kern, grid, dim3(GA_THREADS), smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
+  hipLaunchKernelGGL(kern, grid, dim3(GA_THREADS), smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
   return HILS_OK;
 }
 
+template <int D, int DV, int G>
+static int ga_launch(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, bf16_t* qp, const bf16_t* k,
+                     const bf16_t* vt, const float* vmax, const bf16_t* w, const int32_t* idx,
+                     const float* slope, bf16_t* o, float* lse, const GaDims& dm) {
+  if (slope) return ga_launch_s<D, DV, G, true>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
+  return ga_launch_s<D, DV, G, false>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
+}
+
 template <int D, int DV>
-static int ga_dispatch_g(int G, dim3 grid, size_t smem, hipStream_t st, const bf16_t* q,
+static int ga_dispatch_g(int G, dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, bf16_t* qp,
                          const bf16_t* k, const bf16_t* vt, const float* vmax, const bf16_t* w,
                          const int32_t* idx, const float* slope, bf16_t* o, float* lse,
                          const GaDims& dm) {
   switch (G) {
-    case 1: return ga_launch<D, DV, 1>(grid, smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
-    case 2: return ga_launch<D, DV, 2>(grid, smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
-    case 4: return ga_launch<D, DV, 4>(grid, smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
-    case 8: return ga_launch<D, DV, 8>(grid, smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
-    case 16: return ga_launch<D, DV, 16>(grid, smem, st, q, k, vt, vmax, w, idx, slope, o, lse, dm);
+    case 1: return ga_launch<D, DV, 1>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
+    case 2: return ga_launch<D, DV, 2>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
+    case 4: return ga_launch<D, DV, 4>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
+    case 8: return ga_launch<D, DV, 8>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
+    case 16: return ga_launch<D, DV, 16>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
   }
   return -1;
 }
@@ -409,6 +434,10 @@ static size_t ga_vt_bytes(int B, int H, int nchunk, int Dv) {  // one packed ten
   return (n + 255) & ~(size_t)255;
 }
 
+static size_t ga_vmax_bytes(int B, int H, int nchunk) {
+  return ((size_t)B * H * nchunk * sizeof(float) + 255) & ~(size_t)255;
+}
+
 // Tile sizes: T queries per workgroup such that the fixed-point output tile, the chunk
 // histogram and the pair list fit in LDS.  Returns 0 when the shape does not fit.
 static int ga_pick_T(int L, int G, int Dv, int K, int nchunk, size_t* smem_out) {
@@ -416,7 +445,7 @@ static int ga_pick_T(int L, int G, int Dv, int K, int nchunk, size_t* smem_out) 
   if (T * K > 8 * GA_THREADS) T = (8 * GA_THREADS) / K;
   if (T > L) T = L;
   while (T >= 1) {
-    const size_t smem = (size_t)T * G * Dv * 4 + (size_t)nchunk * 4 + (size_t)T * K * 4;
+    const size_t smem = (size_t)(T * G + 1) * Dv * 4 + (size_t)nchunk * 4 + (size_t)T * K * 4;
     if (smem <= 156 * 1024) {
       *smem_out = smem;
       return T;
@@ -434,12 +463,13 @@ size_t hils_ga_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int 
   const int G = HQ / H;
   const bool ok = S == GA_S && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) &&
                   (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) && q_block == 1 && WH == HQ &&
-                  sm_n == 0.f && L >= 64 && Lkv >= S;
+                  sm_n == 0.f && L >= 64 && Lkv >= S && K >= 1 && K <= 256;
   if (!ok) return 0;
   size_t smem;
   if (ga_pick_T(L, G, Dv, K, Lkv / S, &smem) == 0) return 0;
   const int nchunk = Lkv / S;
-  return ga_vt_bytes(B, H, nchunk, Dv) + ga_vt_bytes(B, H, nchunk, D) + (size_t)B * H * nchunk * sizeof(float);
+  return ga_vt_bytes(B, H, nchunk, Dv) + ga_vt_bytes(B, H, nchunk, D) + ga_vmax_bytes(B, H, nchunk) +
+         (size_t)B * L * HQ * D * sizeof(bf16_t);  // packed K, packed V, per-chunk max|V|, packed Q
 }
 
 // Returns HILS_OK and sets *handled = 1 when the MFMA path ran.
@@ -461,6 +491,7 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
   bf16_t* vpk = (bf16_t*)workspace;
   bf16_t* kpk = (bf16_t*)((char*)workspace + ga_vt_bytes(B, H, nchunk, Dv));
   float* vmax = (float*)((char*)kpk + ga_vt_bytes(B, H, nchunk, D));
+  bf16_t* qpk = (bf16_t*)((char*)vmax + ga_vmax_bytes(B, H, nchunk));
   if (!workspace_ready) {
     const int dmax = D > Dv ? D : Dv;
     hipLaunchKernelGGL(pack_kv_kernel, dim3(nchunk, H, B), dim3(256),
@@ -472,7 +503,7 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
   dim3 grid((unsigned)(per_xcd * 8));
   int rc = -1;
 #define GA_CALL(D_, DV_)                                                                       \
-  rc = ga_dispatch_g<D_, DV_>(G, grid, smem, st, (const bf16_t*)q, kpk, vpk, vmax,             \
+  rc = ga_dispatch_g<D_, DV_>(G, grid, smem, st, (const bf16_t*)q, qpk, kpk, vpk, vmax,        \
                               (const bf16_t*)weights, indices, slope, (bf16_t*)o, lse, dm)
   if (D == 64 && Dv == 64) GA_CALL(64, 64);
   else if (D == 128 && Dv == 128) GA_CALL(128, 128);
