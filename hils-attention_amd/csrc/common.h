@@ -68,6 +68,30 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Reductions / broadcast across the four 16-lane rows of a wavefront, per column (lane & 15),
+// with the gfx950 row-swap instructions: vector-ALU only, no LDS queue involved.
+//   permlane16_swap(x, x) = { [r0, r0, r2, r2], [r1, r1, r3, r3] }   (rows of x)
+//   permlane32_swap(x, x) = { [lo, lo], [hi, hi] }                   (halves of x)
+typedef unsigned hils_uint2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float rows_max(float x) {
+  hils_uint2v a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(a.x), __uint_as_float(a.y));
+  hils_uint2v b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(b.x), __uint_as_float(b.y));
+}
+__device__ __forceinline__ float rows_sum(float x) {
+  hils_uint2v a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(a.x) + __uint_as_float(a.y);
+  hils_uint2v b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(b.x) + __uint_as_float(b.y);
+}
+// value of row 0 (lanes 0..15) in every row
+__device__ __forceinline__ unsigned rows_bcast0(unsigned x) {
+  hils_uint2v a = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+  hils_uint2v b = __builtin_amdgcn_permlane32_swap(a.x, a.x, false, false);
+  return b.x;
+}
+
 // block-wide reductions for blockDim.x a multiple of 64, <= 1024; `red` holds >= 17 floats
 __device__ __forceinline__ float block_sum(float v, float* red) {
   v = wave_sum(v);

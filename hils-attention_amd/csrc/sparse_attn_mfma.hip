@@ -240,135 +240,192 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   const int q_lane = (j * G + g) * 8, w_lane = g * dm.NW;
   const int q_step = dm.HQ * D, w_step = dm.HQ * dm.NW;  // per query of the block
 
-  for (;;) {
-    int c = 0;
-    if (lane == 0) c = atomicAdd(&next_s, 1);
-    c = __builtin_amdgcn_readfirstlane(c);
-    if (c >= dm.nchunk) break;
-    const int vs = c ? cur[c - 1] : 0, ve = cur[c];
-    if (vs == ve) continue;
-
-    // the chunk's K rows (A operands of S^T = K Q^T) and transposed V (B operands of P V)
-    bf16x8_t ka[4][KS], vb[DT][2];
-    {
-      const long chunk = (b * dm.H + hk) * (long)dm.nchunk + c;
-      const bf16_t* kbase = kp + chunk * (long)GA_S * D + lane * 8;
+  // ---- visits: a wavefront takes chunks from a shared counter; a visit is all pairs of the
+  // block on one chunk, processed as tiles of up to QT pairs.  The tile stream of a wavefront
+  // is software-pipelined so that no operand load is waited for right after it is issued:
+  //   iteration i:  issue Q(i+1);  O += P(i-1) V  [then V(chunk i) replaces V in place];
+  //                 S(i) = K Q(i)^T  [then K(chunk i+1) replaces K in place];  softmax -> P(i).
+  // K and V of a chunk are reloaded only when the next tile belongs to another chunk.
+  bf16x8_t ka[4][KS], vb[DT][2];
+  auto load_k = [&](int c, int mt) {
+    const bf16_t* kbase = kp + ((b * dm.H + hk) * (long)dm.nchunk + c) * (long)GA_S * D + lane * 8;
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const uint4 x = *(const uint4*)(kbase + (mt * KS + ks) * 512);
-          ka[mt][ks] = *(const bf16x8_t*)&x;
-        }
-      const bf16_t* vbase = vp + chunk * (long)GA_S * DV + lane * 8;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-          const uint4 x = *(const uint4*)(vbase + (dt * 2 + s) * 512);
-          vb[dt][s] = *(const bf16x8_t*)&x;
-        }
+    for (int ks = 0; ks < KS; ++ks) {
+      const uint4 x = *(const uint4*)(kbase + (mt * KS + ks) * 512);
+      ka[mt][ks] = *(const bf16x8_t*)&x;
     }
-
-    // A tile is up to QT pairs of the visit.  Its gathered query rows (B operands), weights
-    // and output rows are fetched one tile ahead.  Padding rows of the last tile repeat the
-    // visit's first pair (finite arithmetic) and are accumulated into the spare row R.
-    // Query rows come from the packed copy, in which the G heads of a query are interleaved
-    // per 16-byte piece: the lanes of the G heads of one query read contiguous bytes.
-    uint4 bq_n[KS];
-    int w_n, pk_n;     // weight bits (loaded by lane group j == 0) and pair of this lane's row
-    int orow_n[4];     // o_acc element offsets of accumulator rows 4j..4j+3 (column r included)
-    auto load_tile = [&](int p) {
-      const int n = (ve - p < QT) ? ve - p : QT;
-      pk_n = pairs[p + (qs < n ? qs : 0)];
-      const bf16_t* qrow = qb + ((pk_n >> 8) * q_step + q_lane);
+  };
+  auto load_v = [&](int c, int dt) {
+    const bf16_t* vbase = vp + ((b * dm.H + hk) * (long)dm.nchunk + c) * (long)GA_S * DV + lane * 8;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) bq_n[ks] = *(const uint4*)(qrow + ks * (4 * G * 8));
-      w_n = 0;
-      if (j == 0) w_n = wb[(pk_n >> 8) * w_step + w_lane + (pk_n & 255)];
+    for (int s = 0; s < 2; ++s) {
+      const uint4 x = *(const uint4*)(vbase + (dt * 2 + s) * 512);
+      vb[dt][s] = *(const bf16x8_t*)&x;
+    }
+  };
+  // next non-empty visit: chunk id (or -1) and its pair range
+  auto grab = [&](int& vs_o, int& ve_o) -> int {
+    for (;;) {
+      int c = 0;
+      if (lane == 0) c = atomicAdd(&next_s, 1);
+      c = __builtin_amdgcn_readfirstlane(c);
+      if (c >= dm.nchunk) return -1;
+      vs_o = c ? cur[c - 1] : 0;
+      ve_o = cur[c];
+      if (vs_o != ve_o) return c;
+    }
+  };
+  // tile after (c, p, ve)
+  auto advance = [&](int& c, int& p, int& ve) {
+    if (p + QT < ve) { p += QT; return; }
+    int vs2, ve2;
+    c = grab(vs2, ve2);
+    p = vs2;
+    ve = ve2;
+  };
+  // A tile's gathered query rows (B operands), weight and output rows.  Padding rows of a
+  // visit's last tile repeat the visit's first pair (finite arithmetic) and are accumulated
+  // into the spare row R.  Query rows come from the packed copy, in which the G heads of a
+  // query are interleaved per 16-byte piece: the lanes of one query read contiguous bytes.
+  uint4 bq_n[KS];
+  int w_n, pk_n, orow_n[4];
+  auto load_tile = [&](int p, int ve) {
+    const int last = ((ve - p < QT) ? ve - p : QT) - 1;  // padding rows repeat the tile's last pair
+    // all pair reads first, one wait
+    pk_n = pairs[p + (qs < last ? qs : last)];
+    int pk_o[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int rr = 4 * j + i;
-        const int qsl = rr / G;
-        const int pk2 = pairs[p + (qsl < n ? qsl : 0)];
-        const int row = (qsl < n) ? (pk2 >> 8) * G + (rr - qsl * G) : R;
-        orow_n[i] = row * DV + r;
-      }
-    };
-    load_tile(vs);
-    for (int p = vs; p < ve; p += QT) {
-      const int n = (ve - p < QT) ? ve - p : QT;
-      bf16x8_t bq[KS];
+    for (int i = 0; i < 4; ++i) {
+      const int qsl = (4 * j + i) / G;
+      pk_o[i] = pairs[p + (qsl < last ? qsl : last)];
+    }
+    const bf16_t* qrow = qb + ((pk_n >> 8) * q_step + q_lane);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) bq[ks] = *(bf16x8_t*)&bq_n[ks];
-      const int pk_c = pk_n, w_c = w_n;
-      int orow_c[4];
+    for (int ks = 0; ks < KS; ++ks) bq_n[ks] = *(const uint4*)(qrow + ks * (4 * G * 8));
+    w_n = 0;
+    if (j == 0) w_n = wb[(pk_n >> 8) * w_step + w_lane + (pk_n & 255)];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) orow_c[i] = orow_n[i];
-      if (p + QT < ve) load_tile(p + QT);
-      const float w_row = bf2f((bf16_t)__shfl(w_c, r, 64));
-      f32x4_t st[4];
+    for (int i = 0; i < 4; ++i) {
+      const int rr = 4 * j + i;
+      const int qsl = rr / G;
+      const int row = (qsl <= last) ? (pk_o[i] >> 8) * G + (rr - qsl * G) : R;
+      orow_n[i] = row * DV + r;
+    }
+  };
+  bf16x8_t ap[2];   // P of the previous tile (A operand of O = P V)
+  int orow_p[4];    // its output rows
+  // S = K Q^T of the tile in (bq_c, w_c, pk_c), softmax, P -> ap; K(c_next) replaces K when asked
+  auto score_stage = [&](const uint4* bq_c, int w_c, int pk_c, int n, bool reload, int c_next) {
+    const float w_row = bf2f((bf16_t)rows_bcast0((unsigned)w_c));
+    f32x4_t st[4];
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt) {
-        st[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < 4; ++mt) {
+      st[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-          st[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[mt][ks], bq[ks], st[mt], 0, 0, 0);
-      }
-      // per-chunk softmax over the 64 tokens of row r: registers (mt, i) and lane groups j
-      if (SLOPE) {
+      for (int ks = 0; ks < KS; ++ks)
+        st[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[mt][ks], *(const bf16x8_t*)&bq_c[ks], st[mt], 0, 0, 0);
+    }
+    if (reload) {
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int dist = GA_S - 2 - (mt * 16 + j * 4 + i);
-            st[mt][i] -= sl * (float)(dist > 0 ? dist : 0);
-          }
-      }
-      if (dm.mask_last && j == 3) st[3][3] = HILS_NEG_INF;  // token 63 = tile 3, lane group 3, register 3
-      float m = fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3]));
-#pragma unroll
-      for (int mt = 1; mt < 4; ++mt) m = fmaxf(fmaxf(m, fmaxf(st[mt][0], st[mt][1])), fmaxf(st[mt][2], st[mt][3]));
-      m = fmaxf(m, __shfl_xor(m, 16, 64));
-      m = fmaxf(m, __shfl_xor(m, 32, 64));
-      const float mc = m * c2;
-      float sum = 0.f;
+      for (int mt = 0; mt < 4; ++mt) load_k(c_next, mt);
+    }
+    if (SLOPE) {
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float e = __builtin_amdgcn_exp2f(st[mt][i] * c2 - mc);
-          st[mt][i] = e;
-          sum += e;
+          const int dist = GA_S - 2 - (mt * 16 + j * 4 + i);
+          st[mt][i] -= sl * (float)(dist > 0 ? dist : 0);
         }
-      sum += __shfl_xor(sum, 16, 64);
-      sum += __shfl_xor(sum, 32, 64);
-      if (lse && qs < n && j == 0) {
-        const int ql = pk_c >> 8, slot = pk_c & 255;
-        lse[((b * dm.L + t0 + ql) * (long)dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
-      }
-      const float f = w_row * fx_scale / sum;  // fixed-point scale (a power of two) folded into P
-      // P as the A operand of O = P V: k-step s takes tokens of accumulator tiles 2s, 2s+1
-      bf16x8_t ap[2];
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        uint4 x;
-        x.x = pack_bf2(st[2 * s][0] * f, st[2 * s][1] * f);
-        x.y = pack_bf2(st[2 * s][2] * f, st[2 * s][3] * f);
-        x.z = pack_bf2(st[2 * s + 1][0] * f, st[2 * s + 1][1] * f);
-        x.w = pack_bf2(st[2 * s + 1][2] * f, st[2 * s + 1][3] * f);
-        ap[s] = *(bf16x8_t*)&x;
-      }
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s], vb[dt][s], acc, 0, 0, 0);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) atomicAdd(&o_acc[orow_c[i] + dt * 16], __float2int_rn(acc[i]));
-      }
     }
+    if (dm.mask_last && j == 3) st[3][3] = HILS_NEG_INF;  // token 63 = tile 3, lane group 3, register 3
+    float m = fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3]));
+#pragma unroll
+    for (int mt = 1; mt < 4; ++mt) m = fmaxf(fmaxf(m, fmaxf(st[mt][0], st[mt][1])), fmaxf(st[mt][2], st[mt][3]));
+    m = rows_max(m);
+    const float mc = m * c2;
+    float sum = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float e = __builtin_amdgcn_exp2f(st[mt][i] * c2 - mc);
+        st[mt][i] = e;
+        sum += e;
+      }
+    sum = rows_sum(sum);
+    if (lse && qs < n && j == 0) {
+      const int ql = pk_c >> 8, slot = pk_c & 255;
+      lse[((b * dm.L + t0 + ql) * (long)dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
+    }
+    const float f = w_row * fx_scale / sum;  // fixed-point scale (a power of two) folded into P
+    // P as the A operand of O = P V: k-step s takes tokens of accumulator tiles 2s, 2s+1
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      uint4 x;
+      x.x = pack_bf2(st[2 * s][0] * f, st[2 * s][1] * f);
+      x.y = pack_bf2(st[2 * s][2] * f, st[2 * s][3] * f);
+      x.z = pack_bf2(st[2 * s + 1][0] * f, st[2 * s + 1][1] * f);
+      x.w = pack_bf2(st[2 * s + 1][2] * f, st[2 * s + 1][3] * f);
+      ap[s] = *(bf16x8_t*)&x;
+    }
+  };
+  // O += P V for the tile in (ap, orow_p); V(c_next) replaces V when asked
+  auto output_stage = [&](bool reload, int c_next) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s], vb[dt][s], acc, 0, 0, 0);
+      if (reload) load_v(c_next, dt);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) atomicAdd(&o_acc[orow_p[i] + dt * 16], __float2int_rn(acc[i]));
+    }
+  };
+
+  int c_cur, p_cur = 0, ve_cur = 0;
+  c_cur = grab(p_cur, ve_cur);
+  if (c_cur >= 0) {
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) load_k(c_cur, mt);
+    load_tile(p_cur, ve_cur);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) load_v(c_cur, dt);
+    int c_nxt = c_cur, p_nxt = p_cur, ve_nxt = ve_cur;
+    advance(c_nxt, p_nxt, ve_nxt);
+    // first tile: scores only
+    {
+      uint4 bq_c[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) bq_c[ks] = bq_n[ks];
+      const int w_c = w_n, pk_c = pk_n;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) orow_p[i] = orow_n[i];
+      const int n = (ve_cur - p_cur < QT) ? ve_cur - p_cur : QT;
+      if (c_nxt >= 0) load_tile(p_nxt, ve_nxt);
+      score_stage(bq_c, w_c, pk_c, n, c_nxt >= 0 && c_nxt != c_cur, c_nxt);
+    }
+    int c_prev = c_cur;
+    while (c_nxt >= 0) {
+      c_cur = c_nxt; p_cur = p_nxt; ve_cur = ve_nxt;
+      advance(c_nxt, p_nxt, ve_nxt);
+      uint4 bq_c[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) bq_c[ks] = bq_n[ks];
+      const int w_c = w_n, pk_c = pk_n;
+      int orow_c[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) orow_c[i] = orow_n[i];
+      const int n = (ve_cur - p_cur < QT) ? ve_cur - p_cur : QT;
+      if (c_nxt >= 0) load_tile(p_nxt, ve_nxt);
+      output_stage(c_cur != c_prev, c_cur);
+      score_stage(bq_c, w_c, pk_c, n, c_nxt >= 0 && c_nxt != c_cur, c_nxt);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) orow_p[i] = orow_c[i];
+      c_prev = c_cur;
+    }
+    output_stage(false, 0);
   }
   __syncthreads();
   constexpr int C8 = DV / 8;
