@@ -133,26 +133,30 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   const int K = dm.K;
   const int npair = dm.T * K;
 
-  for (int i = tid; i < R * DV; i += GA_THREADS) o_acc[i] = 0;
-  for (int i = tid; i < dm.nchunk; i += GA_THREADS) cur[i] = 0;
-  if (tid == 0) next_s = 0;
-  // Packed copy of this block's query rows: within the G heads of a (query, KV head) the
+  // ---- prologue.  All global loads of the block set-up are issued before anything waits:
+  // the query rows to repack, the selected chunk indices, and the weight rows.
+  // (1) Packed copy of this block's query rows: within the G heads of a (query, KV head) the
   // 16-byte pieces are interleaved head-minor, [piece][head][8], so that the B-operand loads
   // of the G lanes that hold the heads of one query are contiguous.  Only this workgroup
   // reads what it writes here (made visible by the barriers below).
-  {
-    constexpr int PPR = D / 8;
-    for (int i = tid; i < dm.T * G * PPR; i += GA_THREADS) {
-      const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
-      const int g2 = rem / PPR, pc = rem - g2 * PPR;
-      if (t0 + ql < dm.L) {
-        const long blk_e = ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G) * D;
-        *(uint4*)(qp + blk_e + (pc * G + g2) * 8) = *(const uint4*)(q + blk_e + g2 * D + pc * 8);
-      }
-    }
+  constexpr int PPR = D / 8;
+  constexpr int QPK = 8;  // pieces per thread and round
+  const int npiece = dm.T * G * PPR;
+  uint4 qtmp[QPK];
+  auto piece_src_dst = [&](int i, long& src, long& dst) -> bool {
+    const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
+    const int g2 = rem / PPR, pc = rem - g2 * PPR;
+    const long blk_e = ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G) * D;
+    src = blk_e + g2 * D + pc * 8;
+    dst = blk_e + (pc * G + g2) * 8;
+    return i < npiece && t0 + ql < dm.L;
+  };
+#pragma unroll
+  for (int e = 0; e < QPK; ++e) {
+    long src, dst;
+    if (piece_src_dst(tid + e * GA_THREADS, src, dst)) qtmp[e] = *(const uint4*)(q + src);
   }
-  __syncthreads();
-  // histogram of the selected chunks
+  // (2) selected chunk of every (query, slot) pair of the block
   int creg[MAXP], preg[MAXP];
 #pragma unroll
   for (int e = 0; e < MAXP; ++e) {
@@ -162,33 +166,68 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     if (i < npair) {
       const int ql = i / K, slot = i - ql * K;
       preg[e] = (ql << 8) | slot;
-      const int t = t0 + ql;
-      if (t < dm.L) {
-        c = indices[((b * dm.L + t) * dm.H + hk) * (long)K + slot];
-        if (c < 0 || c >= dm.nchunk) {
-          c = -1;
-          if (lse) {
+      if (t0 + ql < dm.L) c = indices[((b * dm.L + t0 + ql) * dm.H + hk) * (long)K + slot];
+    }
+    creg[e] = c;
+  }
+  // (3) weight rows, for the bound of the fixed-point scale: rows' sum of |w| over the K slots.
+  // A row is read as aligned dwords (rows start on any bf16), all loads in flight together.
+  constexpr int WDW = 17;  // dwords per round: 32 slots + alignment slack
+  float wsum = 0.f;
+  for (int row = tid; row < R; row += GA_THREADS) {
+    const int ql = row / G, g = row - ql * G;
+    if (t0 + ql < dm.L) {
+      const long e0 = ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G + g) * dm.NW;  // first element
+      const long e_end = e0 + K;
+      const long tot_e = (long)dm.B * dm.L * dm.HQ * dm.NW;
+      float a = 0.f;
+      for (long eb = e0 & ~1L; eb < e_end; eb += 2 * WDW) {
+        uint32_t wd[WDW];
 #pragma unroll
-            for (int g = 0; g < G; ++g)
-              lse[((b * dm.L + t) * dm.HQ + hk * G + g) * (long)K + slot] = HILS_NEG_INF;
-          }
+        for (int u = 0; u < WDW; ++u) {
+          const long ee = eb + 2 * u;
+          wd[u] = 0u;
+          if (ee < e_end) wd[u] = (ee + 1 < tot_e) ? *(const uint32_t*)(weights + ee) : (uint32_t)weights[ee];
         }
+#pragma unroll
+        for (int u = 0; u < WDW; ++u) {
+          const long ee = eb + 2 * u;
+          if (ee >= e0 && ee < e_end) a += fabsf(__uint_as_float(wd[u] << 16));
+          if (ee + 1 >= e0 && ee + 1 < e_end) a += fabsf(__uint_as_float(wd[u] & 0xffff0000u));
+        }
+      }
+      wsum = fmaxf(wsum, a);
+    }
+  }
+  for (int i = tid; i < R * DV; i += GA_THREADS) o_acc[i] = 0;
+  for (int i = tid; i < dm.nchunk; i += GA_THREADS) cur[i] = 0;
+  if (tid == 0) next_s = 0;
+#pragma unroll
+  for (int e = 0; e < QPK; ++e) {
+    long src, dst;
+    if (piece_src_dst(tid + e * GA_THREADS, src, dst)) *(uint4*)(qp + dst) = qtmp[e];
+  }
+  for (int i0 = QPK * GA_THREADS; i0 < npiece; i0 += GA_THREADS) {  // blocks with more pieces (rare shapes)
+    long src, dst;
+    if (piece_src_dst(i0 + tid, src, dst)) *(uint4*)(qp + dst) = *(const uint4*)(q + src);
+  }
+  __syncthreads();
+  // histogram of the selected chunks
+#pragma unroll
+  for (int e = 0; e < MAXP; ++e) {
+    int c = creg[e];
+    if (c < -1 || c >= dm.nchunk) c = -1;
+    if (c < 0 && lse) {
+      const int i = tid + e * GA_THREADS;
+      const int ql = i / K, slot = i - ql * K;
+      if (i < npair && t0 + ql < dm.L) {
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+          lse[((b * dm.L + t0 + ql) * dm.HQ + hk * G + g) * (long)K + slot] = HILS_NEG_INF;
       }
     }
     creg[e] = c;
     if (c >= 0) atomicAdd(&cur[c], 1);
-  }
-  // bound for the fixed-point scale: rows' sum of |w| ...
-  float wsum = 0.f;
-  for (int row = tid; row < R; row += GA_THREADS) {
-    const int ql = row / G, g = row - ql * G;
-    const int t = t0 + ql;
-    if (t < dm.L) {
-      const bf16_t* wr = weights + ((b * dm.L + t) * (long)dm.HQ + hk * G + g) * dm.NW;
-      float a = 0.f;
-      for (int s2 = 0; s2 < K; ++s2) a += fabsf(bf2f(wr[s2]));
-      wsum = fmaxf(wsum, a);
-    }
   }
   wsum = block_max(wsum, red);  // barrier: histogram complete
   // ... times max |V| over the visited chunks; exclusive scan of the histogram on the way
@@ -263,6 +302,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       vb[dt][s] = *(const bf16x8_t*)&x;
     }
   };
+  const int npair_valid = cur[dm.nchunk - 1];  // pairs with a valid chunk
   // next non-empty visit: chunk id (or -1) and its pair range
   auto grab = [&](int& vs_o, int& ve_o) -> int {
     for (;;) {
@@ -271,6 +311,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       c = __builtin_amdgcn_readfirstlane(c);
       if (c >= dm.nchunk) return -1;
       vs_o = c ? cur[c - 1] : 0;
+      if (vs_o >= npair_valid) return -1;  // every pair lies in an earlier chunk
       ve_o = cur[c];
       if (vs_o != ve_o) return c;
     }
