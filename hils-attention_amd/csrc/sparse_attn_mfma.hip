@@ -143,18 +143,14 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   constexpr int QPK = 8;  // pieces per thread and round
   const int npiece = dm.T * G * PPR;
   uint4 qtmp[QPK];
-  auto piece_src_dst = [&](int i, long& src, long& dst) -> bool {
-    const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
-    const int g2 = rem / PPR, pc = rem - g2 * PPR;
-    const long blk_e = ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G) * D;
-    src = blk_e + g2 * D + pc * 8;
-    dst = blk_e + (pc * G + g2) * 8;
-    return i < npiece && t0 + ql < dm.L;
-  };
 #pragma unroll
   for (int e = 0; e < QPK; ++e) {
-    long src, dst;
-    if (piece_src_dst(tid + e * GA_THREADS, src, dst)) qtmp[e] = *(const uint4*)(q + src);
+    const int i = tid + e * GA_THREADS;
+    const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
+    const int g2 = rem / PPR, pc = rem - g2 * PPR;
+    const bool ok = i < npiece && t0 + ql < dm.L;
+    const long blk_e = ((b * dm.L + (ok ? t0 + ql : t0)) * (long)dm.HQ + hk * G) * D;  // t0 < L always
+    qtmp[e] = *(const uint4*)(q + blk_e + g2 * D + pc * 8);
   }
   // (2) selected chunk of every (query, slot) pair of the block
   int creg[MAXP], preg[MAXP];
@@ -204,12 +200,19 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   if (tid == 0) next_s = 0;
 #pragma unroll
   for (int e = 0; e < QPK; ++e) {
-    long src, dst;
-    if (piece_src_dst(tid + e * GA_THREADS, src, dst)) *(uint4*)(qp + dst) = qtmp[e];
+    const int i = tid + e * GA_THREADS;
+    const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
+    const int g2 = rem / PPR, pc = rem - g2 * PPR;
+    if (i < npiece && t0 + ql < dm.L)
+      *(uint4*)(qp + ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G) * D + (pc * G + g2) * 8) = qtmp[e];
   }
-  for (int i0 = QPK * GA_THREADS; i0 < npiece; i0 += GA_THREADS) {  // blocks with more pieces (rare shapes)
-    long src, dst;
-    if (piece_src_dst(i0 + tid, src, dst)) *(uint4*)(qp + dst) = *(const uint4*)(q + src);
+  for (int i = QPK * GA_THREADS + tid; i < npiece; i += GA_THREADS) {  // blocks with more pieces (rare shapes)
+    const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
+    const int g2 = rem / PPR, pc = rem - g2 * PPR;
+    if (t0 + ql < dm.L) {
+      const long blk_e = ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G) * D;
+      *(uint4*)(qp + blk_e + (pc * G + g2) * 8) = *(const uint4*)(q + blk_e + g2 * D + pc * 8);
+    }
   }
   __syncthreads();
   // histogram of the selected chunks
@@ -358,14 +361,16 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   // S = K Q^T of the tile in (bq_c, w_c, pk_c), softmax, P -> ap; K(c_next) replaces K when asked
   auto score_stage = [&](const uint4* bq_c, int w_c, int pk_c, int n, bool reload, int c_next) {
     const float w_row = bf2f((bf16_t)rows_bcast0((unsigned)w_c));
+    // four independent accumulation chains (token tiles), interleaved so that a chain's next
+    // MFMA is issued only after three others
     f32x4_t st[4];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-      st[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < 4; ++mt) st[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
         st[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[mt][ks], *(const bf16x8_t*)&bq_c[ks], st[mt], 0, 0, 0);
-    }
     if (reload) {
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) load_k(c_next, mt);
@@ -413,15 +418,26 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   };
   // O += P V for the tile in (ap, orow_p); V(c_next) replaces V when asked
   auto output_stage = [&](bool reload, int c_next) {
+    // four column tiles at a time: their eight MFMAs interleaved (two-deep chains), then the
+    // operand reload, then the fixed-point adds
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int d0 = 0; d0 < DT; d0 += 4) {
+      f32x4_t acc[4];
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s], vb[dt][s], acc, 0, 0, 0);
-      if (reload) load_v(c_next, dt);
+      for (int u = 0; u < 4; ++u) acc[u] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < 4; ++i) atomicAdd(&o_acc[orow_p[i] + dt * 16], __float2int_rn(acc[i]));
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s2], vb[d0 + u][s2], acc[u], 0, 0, 0);
+      if (reload) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) load_v(c_next, d0 + u);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) atomicAdd(&o_acc[orow_p[i] + (d0 + u) * 16], __float2int_rn(acc[u][i]));
     }
   };
 
