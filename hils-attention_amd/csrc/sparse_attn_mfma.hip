@@ -404,7 +404,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       const int ql = pk_c >> 8, slot = pk_c & 255;
       lse[((b * dm.L + t0 + ql) * (long)dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
     }
-    const float f = w_row * fx_scale / sum;  // fixed-point scale (a power of two) folded into P
+    const float f = w_row * fx_scale * __builtin_amdgcn_rcpf(sum);  // fixed-point scale (a power of two) folded into P
     // P as the A operand of O = P V: k-step s takes tokens of accumulator tiles 2s, 2s+1
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
