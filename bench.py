@@ -216,6 +216,9 @@ def main():
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="profiling aid: decode step only")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="profiling aid: run only a 512 MiB device copy (reference reading for the "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives are part of the hot "
@@ -226,6 +229,14 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.copy_calibration:
+        src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes": int(src.numel())}))
+        return
     if args.no_prefill:
         dsec, dper, droof = bench_decode(pkg, dev, max(args.steps, 20), args.warmup)
         print(json.dumps({"decode_us_per_step": dsec * 1e6, "decode_kernel_ms": dper, "roofline_decode": droof}))
