@@ -25,6 +25,10 @@ import __graft_entry__ as entry  # noqa: E402
 
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the readings of
+# a 512 MiB copy: x2.0 and x1.0), see profiles/hbm_traffic_fetch_write_size.md
+TRAFFIC_PREFILL_ATTN_BYTES = 3.04e9
+TRAFFIC_DECODE_STEP_BYTES = 4.28e8
 
 
 def gpu_randn(shape, gen, dev, scale=None, chunk=1 << 26):
@@ -114,7 +118,7 @@ def bench_prefill(pkg, dev, steps, warmup):
     attn_ms = per["attn"]
     roof = {"kernel": "sparse_attn_fwd_gather", "bound": "mfma",
             "achieved": flops / (attn_ms * 1e-3) / 1e12, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": flops / (attn_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, "traffic": None,
+            "frac": flops / (attn_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, "traffic": TRAFFIC_PREFILL_ATTN_BYTES,
             "flops_per_launch": flops, "ms_per_launch": attn_ms}
     cfg = {"workload": "prefill_fwd B1 L32768 hq32/hkv8 D128 chunk64 top32 causal (7B-shaped, config 3)",
            "global_batch": B, "seq_len": L, "n_sel": n_sel}
@@ -174,7 +178,7 @@ def bench_decode(pkg, dev, steps, warmup):
     total = lmk_bytes + kv_bytes + small
     roof = {"kernel": "topk_fwd + sparse_attn_fwd (decode step)", "bound": "hbm",
             "achieved": total / sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": total / sec / 1e9 / HBM_PEAK_GBS, "traffic": None, "bytes_per_step": total,
+            "frac": total / sec / 1e9 / HBM_PEAK_GBS, "traffic": TRAFFIC_DECODE_STEP_BYTES, "bytes_per_step": total,
             "topk_gbs": lmk_bytes / (per["topk"] * 1e-3) / 1e9,
             "attn_gbs": kv_bytes / (per["attn"] * 1e-3) / 1e9}
     del kc, vc
