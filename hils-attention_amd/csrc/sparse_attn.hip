@@ -30,6 +30,7 @@ int hils_sparse_attn_decode(const void* q, const void* k, const void* v, const v
 struct SaDims {
   int L, Lkv, HQ, H, G, D, Dv, K, NW, WH, q_block, S, mask_last;
   float sm_scale, sm_n;
+  int skip_dkdv;  // backward: dK and dV come from the chunk-major kernel
 };
 
 // scores of slot chunk c for all (g, s): sc[g*S+s] = (q_g . K_s - slope_g*dist_s) * sm_scale,
@@ -226,7 +227,7 @@ sparse_attn_bwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
     }
     // dV[s][dv] += sum_g w_g P[g][s] dO[g][dv]
     float* dvb = dv + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * Dv;
-    for (int p = tid; p < S * Dv; p += SA_THREADS) {
+    for (int p = tid; p < (dm.skip_dkdv ? 0 : S * Dv); p += SA_THREADS) {
       const int s = p / Dv, d = p - s * Dv;
       float a = 0.f;
       for (int g = 0; g < G; ++g) a = fmaf(w_s[g] * p_s[g * S + s], do_s[g * Dv + d], a);
@@ -234,7 +235,7 @@ sparse_attn_bwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
     }
     // dK[s][d] += sum_g dS[g][s] q[g][d]
     float* dkb = dk + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * D;
-    for (int p = tid; p < S * D; p += SA_THREADS) {
+    for (int p = tid; p < (dm.skip_dkdv ? 0 : S * D); p += SA_THREADS) {
       const int s = p / D, d = p - s * D;
       float a = 0.f;
       for (int g = 0; g < G; ++g) a = fmaf(ds_s[g * S + s], q_s[g * D + d], a);
@@ -309,7 +310,7 @@ extern "C" int hils_sparse_attn_fwd(const void* q, const void* k, const void* v,
       return HILS_OK;
     }
   }
-  SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n};
+  SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n, 0};
   size_t smem = ((size_t)dm.G * D + (size_t)dm.G * S + 2 * dm.G) * sizeof(float);
   HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_fwd: G*(D+S) too large for LDS");
   hipLaunchKernelGGL(sparse_attn_fwd_simple, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS),
@@ -319,23 +320,43 @@ extern "C" int hils_sparse_attn_fwd(const void* q, const void* k, const void* v,
   return HILS_OK;
 }
 
+bool hils_bw_covers(int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S, int q_block, int WH,
+                    float sm_n, const float* slope);
+size_t hils_bw_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S,
+                               int q_block, int WH, float sm_n);
+int hils_bw_dkdv(const void* q, const void* k, const void* v, const void* weights, const int32_t* indices,
+                 const float* lse, const void* d_o, float* dk, float* dv, void* workspace, int B, int L,
+                 int Lkv, int HQ, int H, int D, int Dv, int K, int NW, float sm_scale, int mask_last,
+                 void* stream);
+
+extern "C" size_t hils_sparse_attn_bwd_workspace(int B, int L, int Lkv, int HQ, int H, int D, int Dv,
+                                                 int K, int WH, int q_block, int S, float sm_n) {
+  return hils_bw_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n);
+}
+
 extern "C" int hils_sparse_attn_bwd(const void* q, const void* k, const void* v,
                                     const void* weights, const int32_t* indices,
                                     const float* slope, const float* lse, const void* d_o,
-                                    void* dq, float* dk, float* dv, float* dw, int B, int L,
-                                    int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int WH,
+                                    void* dq, float* dk, float* dv, float* dw, void* workspace, int B,
+                                    int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int WH,
                                     int q_block, int S, float sm_scale, int mask_last, float sm_n,
                                     void* stream) {
   HILS_REQUIRE(q && k && v && weights && indices && lse && d_o && dq && dk && dv && dw,
                "hils_sparse_attn_bwd: null pointer");
   if (int rc = sa_check("hils_sparse_attn_bwd", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
-  SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n};
+  const bool fast = workspace && hils_bw_covers(L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n, slope);
+  SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n, fast ? 1 : 0};
   size_t smem = ((size_t)dm.G * (D + Dv) + 2 * (size_t)dm.G * S + 3 * dm.G) * sizeof(float);
   HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_bwd: G*(D+Dv+2S) too large for LDS");
   hipLaunchKernelGGL(sparse_attn_bwd_simple, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS),
                      smem, (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k,
                      (const bf16_t*)v, (const bf16_t*)weights, indices, slope, lse,
                      (const bf16_t*)d_o, (bf16_t*)dq, dk, dv, dw, dm);
+  if (fast) {
+    const int rc = hils_bw_dkdv(q, k, v, weights, indices, lse, d_o, dk, dv, workspace, B, L, Lkv, HQ, H, D,
+                                Dv, K, NW, sm_scale, mask_last, stream);
+    HILS_REQUIRE(rc == HILS_OK, "hils_sparse_attn_bwd: no dK/dV kernel for this shape");
+  }
   HILS_CHECK_LAUNCH("hils_sparse_attn_bwd");
   return HILS_OK;
 }

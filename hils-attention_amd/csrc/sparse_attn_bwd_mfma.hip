@@ -1,0 +1,362 @@
+// Sparse attention backward on bf16 MFMA (chunk size 64, D and Dv in {64, 128}).
+//
+// dK and dV of a chunk are sums over every (query, head) row that selected the chunk, so
+// that side is computed chunk-major: an inverse index (for each (batch, KV head, chunk) the
+// list of (query, slot) pairs that hold it) is built by a counting sort, then one workgroup
+// per chunk streams its rows in tiles of 16, recomputes P and dS with the scores in the
+// orientation rows x tokens, and keeps dK, dV of the chunk in MFMA accumulators: no atomics,
+// one write per element.
+//
+//   S  = Q K^T            (16 rows x 16 tokens per wavefront, 16x16x32 MFMA over d)
+//   dP = dO V^T           (same shape, 16x16x32 MFMA over dv)
+//   P  = exp2(S c2 - lse2),  delta = sum_tokens P dP,  dS = w P (dP - delta)
+//   dV += (w P)^T dO      (16 tokens x Dv, 16x16x16 MFMA over the 16 rows)
+//   dK += scale dS^T Q    (16 tokens x D,  16x16x16 MFMA over the 16 rows)
+//
+// An accumulator-layout tile (lane: column = token, registers = rows 4j..4j+3) is exactly the A
+// operand of the 16x16x16 MFMA with the roles (row m = token, k = rows), so P and dS feed the
+// second pair of products without leaving registers.  Their B operands (k = rows, n = feature)
+// are read from a transposed copy of the gathered Q and dO rows that the workgroup stages in
+// LDS once per tile and all four wavefronts (16 tokens each) share.
+#include "decode_rows.h"
+#include "../../include/hils_amd.h"
+
+#define BW_S 64
+typedef short bw_s4 __attribute__((ext_vector_type(4)));
+
+__global__ void bw_fill_int_kernel(int* p, int value, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = value;
+}
+
+// ---------------------------------------------------------------------------
+// Inverse index: pairs (query << 8 | slot) grouped by (batch, KV head, chunk).
+// ---------------------------------------------------------------------------
+// counts[(b*H + h) * nchunk + c] = number of valid entries equal to c; one workgroup per
+// (batch, KV head, segment of queries), LDS histogram first.
+__global__ void __launch_bounds__(1024)
+bw_count_kernel(const int32_t* __restrict__ indices, int* __restrict__ counts, int L, int H, int K,
+                int nchunk, int seg_len) {
+  extern __shared__ int hist[];
+  const int h = blockIdx.y;
+  const long b = blockIdx.z;
+  const int t_lo = blockIdx.x * seg_len;
+  const int t_hi = (t_lo + seg_len < L) ? t_lo + seg_len : L;
+  for (int i = threadIdx.x; i < nchunk; i += 1024) hist[i] = 0;
+  __syncthreads();
+  const long n = (long)(t_hi - t_lo) * K;
+  for (long i = threadIdx.x; i < n; i += 1024) {
+    const int t = t_lo + (int)(i / K), slot = (int)(i % K);
+    const int c = indices[((b * L + t) * H + h) * (long)K + slot];
+    if (c >= 0 && c < nchunk) atomicAdd(&hist[c], 1);
+  }
+  __syncthreads();
+  int* out = counts + (b * H + h) * (long)nchunk;
+  for (int i = threadIdx.x; i < nchunk; i += 1024)
+    if (hist[i]) atomicAdd(&out[i], hist[i]);
+}
+
+// exclusive scan of n counts into offsets[0..n] (offsets[n] = total); one workgroup
+__global__ void __launch_bounds__(1024)
+bw_scan_kernel(const int* __restrict__ counts, int* __restrict__ offsets, int* __restrict__ cursor, long n) {
+  __shared__ int wsum[16];
+  __shared__ int carry_s;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) carry_s = 0;
+  __syncthreads();
+  for (long base = 0; base < n; base += 1024) {
+    const long i = base + tid;
+    const int x = (i < n) ? counts[i] : 0;
+    int incl = x;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int y = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += y;
+    }
+    if (lane == 63) wsum[wave] = incl;
+    __syncthreads();
+    int pre = carry_s;
+    for (int w = 0; w < wave; ++w) pre += wsum[w];
+    if (i < n) {
+      offsets[i] = pre + incl - x;
+      cursor[i] = pre + incl - x;
+    }
+    __syncthreads();
+    if (tid == 1023) carry_s = pre + incl;
+    __syncthreads();
+  }
+  if (tid == 0) offsets[n] = carry_s;
+}
+
+// pairs[cursor[(b,h,c)]++] = (t << 8 | slot)
+__global__ void __launch_bounds__(1024)
+bw_scatter_kernel(const int32_t* __restrict__ indices, int* __restrict__ cursor,
+                  uint32_t* __restrict__ pairs, int L, int H, int K, int nchunk, int seg_len) {
+  const int h = blockIdx.y;
+  const long b = blockIdx.z;
+  const int t_lo = blockIdx.x * seg_len;
+  const int t_hi = (t_lo + seg_len < L) ? t_lo + seg_len : L;
+  int* cur = cursor + (b * H + h) * (long)nchunk;
+  const long n = (long)(t_hi - t_lo) * K;
+  for (long i = threadIdx.x; i < n; i += 1024) {
+    const int t = t_lo + (int)(i / K), slot = (int)(i % K);
+    const int c = indices[((b * L + t) * H + h) * (long)K + slot];
+    if (c >= 0 && c < nchunk) pairs[atomicAdd(&cur[c], 1)] = ((uint32_t)t << 8) | (uint32_t)slot;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// dK, dV: one workgroup of four wavefronts per (batch, KV head, chunk)
+// ---------------------------------------------------------------------------
+struct BwDims {
+  int L, Lkv, HQ, H, K, NW, nchunk, mask_last;
+  float sm_scale;
+};
+
+template <int D, int DV, int G>
+__global__ void __launch_bounds__(256)
+bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+               const bf16_t* __restrict__ weights, const float* __restrict__ lse,
+               const bf16_t* __restrict__ d_o, const int* __restrict__ offsets,
+               const uint32_t* __restrict__ pairs, float* __restrict__ dk, float* __restrict__ dv,
+               BwDims dm) {
+  constexpr int KS = D / 32, VS = DV / 32;    // k-steps of the two 16x16x32 products
+  constexpr int DT = D / 16, VT = DV / 16;    // 16-wide column tiles of dK, dV
+  constexpr int QT = 16 / G;                  // pairs per 16-row tile
+  constexpr int QROW = D * 2 + 16;            // row-major staging: padded row (bytes)
+  constexpr int OROW = DV * 2 + 16;
+  constexpr int CS = 40;                      // transposed staging: bytes per feature column (16 rows + pad)
+  __shared__ __attribute__((aligned(16))) char q_rm[16 * QROW];
+  __shared__ __attribute__((aligned(16))) char o_rm[16 * OROW];
+  __shared__ __attribute__((aligned(16))) char q_tr[D * CS];
+  __shared__ __attribute__((aligned(16))) char o_tr[DV * CS];
+  __shared__ float row_lse[16], row_w[16];
+  __shared__ float red[4][16];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, j = lane >> 4;
+  const int c = blockIdx.x, hk = blockIdx.y;
+  const long b = blockIdx.z;
+  const long cell = (b * dm.H + hk) * (long)dm.nchunk + c;
+  const int p_lo = offsets[cell], p_hi = offsets[cell + 1];
+  if (p_lo == p_hi) return;
+
+  // this wavefront's 16 tokens of the chunk as B operands (k = feature, n = token)
+  const long tok = (long)c * BW_S + wave * 16 + col;
+  uint4 kb[KS], vb[VS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    kb[ks] = *(const uint4*)(k + ((b * dm.Lkv + tok) * dm.H + hk) * D + ks * 32 + j * 8);
+#pragma unroll
+  for (int ks = 0; ks < VS; ++ks)
+    vb[ks] = *(const uint4*)(v + ((b * dm.Lkv + tok) * dm.H + hk) * DV + ks * 32 + j * 8);
+  const bool masked_col = dm.mask_last && wave == 3 && col == 15;  // token 63 of the chunk
+
+  f32x4_t acc_k[DT], acc_v[VT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t) acc_k[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int t = 0; t < VT; ++t) acc_v[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  const float c2 = dm.sm_scale * HILS_LOG2E;
+
+  // staging roles: thread -> (row, 16-byte piece) of the Q tile and of the dO tile
+  constexpr int QPP = D / 8, OPP = DV / 8;
+  const int q_row = tid / QPP, q_pc = tid % QPP;
+  const int o_row = tid / OPP, o_pc = tid % OPP;
+  const int npair = p_hi - p_lo;
+
+  for (int p0 = 0; p0 < npair; p0 += QT) {
+    const int n = (npair - p0 < QT) ? npair - p0 : QT;  // pairs in this tile
+    __syncthreads();  // the previous tile's staging is no longer read
+    // ---- stage the gathered rows: row-major (A operands) and transposed (B operands)
+    if (q_row < 16) {
+      uint4 x = make_uint4(0, 0, 0, 0);
+      const int pr = q_row / G, g = q_row - pr * G;
+      if (pr < n) {
+        const uint32_t pk = pairs[p_lo + p0 + pr];
+        x = *(const uint4*)(q + ((b * dm.L + (pk >> 8)) * (long)dm.HQ + hk * G + g) * D + q_pc * 8);
+      }
+      *(uint4*)(q_rm + q_row * QROW + q_pc * 16) = x;
+      const bf16_t* xe = (const bf16_t*)&x;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) *(bf16_t*)(q_tr + (q_pc * 8 + e) * CS + q_row * 2) = xe[e];
+    }
+    if (o_row < 16) {
+      uint4 x = make_uint4(0, 0, 0, 0);
+      const int pr = o_row / G, g = o_row - pr * G;
+      if (pr < n) {
+        const uint32_t pk = pairs[p_lo + p0 + pr];
+        x = *(const uint4*)(d_o + ((b * dm.L + (pk >> 8)) * (long)dm.HQ + hk * G + g) * DV + o_pc * 8);
+      }
+      *(uint4*)(o_rm + o_row * OROW + o_pc * 16) = x;
+      const bf16_t* xe = (const bf16_t*)&x;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) *(bf16_t*)(o_tr + (o_pc * 8 + e) * CS + o_row * 2) = xe[e];
+    }
+    if (tid < 16) {
+      const int pr = tid / G, g = tid - pr * G;
+      float l2 = INFINITY, w = 0.f;  // padding rows: P = 0
+      if (pr < n) {
+        const uint32_t pk = pairs[p_lo + p0 + pr];
+        const long rowi = (b * dm.L + (pk >> 8)) * (long)dm.HQ + hk * G + g;
+        l2 = lse[rowi * dm.K + (pk & 255)];
+        if (l2 == HILS_NEG_INF) l2 = INFINITY;
+        w = bf2f(weights[rowi * dm.NW + (pk & 255)]);
+      }
+      row_lse[tid] = l2;
+      row_w[tid] = w;
+    }
+    __syncthreads();
+    // ---- S and dP for this wavefront's 16 tokens
+    f32x4_t s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const uint4 a = *(const uint4*)(q_rm + col * QROW + (ks * 32 + j * 8) * 2);
+      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&kb[ks], s, 0, 0, 0);
+    }
+#pragma unroll
+    for (int ks = 0; ks < VS; ++ks) {
+      const uint4 a = *(const uint4*)(o_rm + col * OROW + (ks * 32 + j * 8) * 2);
+      dp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&vb[ks], dp, 0, 0, 0);
+    }
+    // accumulator layout: column = token `col`, registers = rows 4j..4j+3
+    float pr4[4], part[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float pv = __builtin_amdgcn_exp2f(s[i] * c2 - row_lse[4 * j + i]);
+      if (masked_col) pv = 0.f;
+      pr4[i] = pv;
+      part[i] = pv * dp[i];
+    }
+    // delta of a row = sum over the 64 tokens: 16 lanes of the row group, then 4 wavefronts
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      part[i] = row_sum<16>(part[i]);
+    }
+    if (col == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][4 * j + i] = part[i];
+    }
+    __syncthreads();
+    bw_s4 a_p, a_ds;
+    {
+      float pw[4], ds[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 4 * j + i;
+        const float delta = red[0][r] + red[1][r] + red[2][r] + red[3][r];
+        const float w = row_w[r];
+        pw[i] = w * pr4[i];
+        ds[i] = pw[i] * (dp[i] - delta);
+      }
+      uint2 x;
+      x.x = pack_bf2(pw[0], pw[1]);
+      x.y = pack_bf2(pw[2], pw[3]);
+      a_p = *(bw_s4*)&x;
+      x.x = pack_bf2(ds[0], ds[1]);
+      x.y = pack_bf2(ds[2], ds[3]);
+      a_ds = *(bw_s4*)&x;
+    }
+    // ---- dK += dS^T Q, dV += (wP)^T dO: contraction over the 16 rows
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+      const uint2 bq = *(const uint2*)(q_tr + (t * 16 + col) * CS + j * 8);
+      acc_k[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_ds, *(const bw_s4*)&bq, acc_k[t], 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < VT; ++t) {
+      const uint2 bo = *(const uint2*)(o_tr + (t * 16 + col) * CS + j * 8);
+      acc_v[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_p, *(const bw_s4*)&bo, acc_v[t], 0, 0, 0);
+    }
+  }
+  // accumulators: column = feature t*16 + col, rows = tokens wave*16 + 4j + i
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const long tk = (long)c * BW_S + wave * 16 + 4 * j + i;
+    float* dkr = dk + ((b * dm.Lkv + tk) * dm.H + hk) * D;
+    float* dvr = dv + ((b * dm.Lkv + tk) * dm.H + hk) * DV;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) dkr[t * 16 + col] += acc_k[t][i] * dm.sm_scale;
+#pragma unroll
+    for (int t = 0; t < VT; ++t) dvr[t * 16 + col] += acc_v[t][i];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+static size_t bw_round(size_t n) { return (n + 255) & ~(size_t)255; }
+
+bool hils_bw_covers(int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S, int q_block, int WH,
+                    float sm_n, const float* slope) {
+  if (H <= 0 || HQ % H != 0) return false;
+  const int G = HQ / H;
+  return S == BW_S && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) &&
+         (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) && q_block == 1 && WH == HQ && sm_n == 0.f &&
+         slope == nullptr && Lkv % S == 0 && K <= 256 && L < (1 << 24) && Lkv / S <= 12288;
+}
+
+size_t hils_bw_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S,
+                               int q_block, int WH, float sm_n) {
+  if (!hils_bw_covers(L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n, nullptr)) return 0;
+  const size_t cells = (size_t)B * H * (Lkv / S);
+  return bw_round((cells + 1) * 4) * 3 + bw_round((size_t)B * L * H * K * 4);  // counts, offsets, cursor, pairs
+}
+
+template <int D, int DV>
+static int bw_launch_dkdv(int G, dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* k,
+                          const bf16_t* v, const bf16_t* w, const float* lse, const bf16_t* d_o,
+                          const int* offsets, const uint32_t* pairs, float* dk, float* dv,
+                          const BwDims& dm) {
+#define BW_CALL(G_)                                                                                 \
+  hipLaunchKernelGGL((bw_dkdv_kernel<D, DV, G_>), grid, dim3(256), 0, st, q, k, v, w, lse, d_o, offsets, \
+                     pairs, dk, dv, dm)
+  switch (G) {
+    case 1: BW_CALL(1); break;
+    case 2: BW_CALL(2); break;
+    case 4: BW_CALL(4); break;
+    case 8: BW_CALL(8); break;
+    case 16: BW_CALL(16); break;
+    default: return -1;
+  }
+#undef BW_CALL
+  return HILS_OK;
+}
+
+// dK and dV (accumulated into the caller's fp32 buffers) through the inverse index.
+int hils_bw_dkdv(const void* q, const void* k, const void* v, const void* weights, const int32_t* indices,
+                 const float* lse, const void* d_o, float* dk, float* dv, void* workspace, int B, int L,
+                 int Lkv, int HQ, int H, int D, int Dv, int K, int NW, float sm_scale, int mask_last,
+                 void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  const int nchunk = Lkv / BW_S;
+  const size_t cells = (size_t)B * H * nchunk;
+  int* counts = (int*)workspace;
+  int* offsets = (int*)((char*)counts + bw_round((cells + 1) * 4));
+  int* cursor = (int*)((char*)offsets + bw_round((cells + 1) * 4));
+  uint32_t* pairs = (uint32_t*)((char*)cursor + bw_round((cells + 1) * 4));
+  const int G = HQ / H;
+  // zero the counts with a kernel (keeps the call capturable in a HIP graph)
+  {
+    const long n = (long)cells + 1;
+    hipLaunchKernelGGL(bw_fill_int_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, counts, 0, n);
+  }
+  int seg_len = L;
+  while ((long)B * H * ((L + seg_len - 1) / seg_len) < 512 && seg_len > 256) seg_len = (seg_len + 1) / 2;
+  dim3 gs((L + seg_len - 1) / seg_len, H, B);
+  hipLaunchKernelGGL(bw_count_kernel, gs, dim3(1024), (size_t)nchunk * 4, st, indices, counts, L, H, K, nchunk, seg_len);
+  hipLaunchKernelGGL(bw_scan_kernel, dim3(1), dim3(1024), 0, st, counts, offsets, cursor, (long)cells);
+  hipLaunchKernelGGL(bw_scatter_kernel, gs, dim3(1024), 0, st, indices, cursor, pairs, L, H, K, nchunk, seg_len);
+  BwDims dm{L, Lkv, HQ, H, K, NW, nchunk, mask_last, sm_scale};
+  dim3 grid(nchunk, H, B);
+  int rc = -1;
+#define BW_D(D_, DV_)                                                                              \
+  rc = bw_launch_dkdv<D_, DV_>(G, grid, st, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v,   \
+                               (const bf16_t*)weights, lse, (const bf16_t*)d_o, offsets, pairs, dk, dv, dm)
+  if (D == 64 && Dv == 64) BW_D(64, 64);
+  else if (D == 128 && Dv == 128) BW_D(128, 128);
+  else if (D == 64 && Dv == 128) BW_D(64, 128);
+  else if (D == 128 && Dv == 64) BW_D(128, 64);
+#undef BW_D
+  return rc;
+}

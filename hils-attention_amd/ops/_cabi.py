@@ -26,7 +26,7 @@ SIGNATURES = {
     "hils_topk_bwd": [_P] * 6 + [_I] * 8 + [_F, _P],
     "hils_sparse_attn_fwd": [_P] * 9 + [_I] * 13 + [_F, _I, _F, _P],
     "hils_pack_kv_chunks": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
-    "hils_sparse_attn_bwd": [_P] * 12 + [_I] * 12 + [_F, _I, _F, _P],
+    "hils_sparse_attn_bwd": [_P] * 13 + [_I] * 12 + [_F, _I, _F, _P],
     "hils_chunk_weights": [_P, _P, _I, _P, _P, _P] + [_I] * 7 + [_P],
     "hils_chunk_logz_fwd": [_P, _P, _P] + [_I] * 7 + [_F, _I, _P],
     "hils_chunk_logz_bwd_dq": [_P] * 5 + [_I] * 7 + [_F, _P],
@@ -54,6 +54,8 @@ def load():
     lib.hils_topk_fwd_workspace.argtypes = [_I] * 5
     lib.hils_sparse_attn_fwd_workspace.restype = ctypes.c_size_t
     lib.hils_sparse_attn_fwd_workspace.argtypes = [_I] * 11 + [_F]
+    lib.hils_sparse_attn_bwd_workspace.restype = ctypes.c_size_t
+    lib.hils_sparse_attn_bwd_workspace.argtypes = [_I] * 11 + [_F]
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = c_int
@@ -93,6 +95,14 @@ def topk_fwd_workspace(device, B, L, N, h_kv, G):
 def sparse_attn_fwd_workspace(device, B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n):
     """Scratch tensor for hils_sparse_attn_fwd (None when the shape needs none)."""
     n = load().hils_sparse_attn_fwd_workspace(B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n)
+    if n == 0:
+        return None
+    return torch.empty(n, dtype=torch.uint8, device=device)
+
+
+def sparse_attn_bwd_workspace(device, B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n):
+    """Scratch tensor for hils_sparse_attn_bwd (None when the shape needs none)."""
+    n = load().hils_sparse_attn_bwd_workspace(B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n)
     if n == 0:
         return None
     return torch.empty(n, dtype=torch.uint8, device=device)

@@ -61,7 +61,7 @@ class _attention(torch.autograd.Function):
         dw = torch.zeros(w_in.shape, dtype=torch.float32, device=q.device)
         _cabi.call("hils_sparse_attn_bwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
                    _cabi.ptr(idx_in), None, _cabi.ptr(lse), _cabi.ptr(do),
-                   _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw),
+                   _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), None,
                    N, L, L_kv, HQ, H, D, Dv, K, K, H, q_x, S, sm_scale, 0, sm_n)
         return (dq, dk.to(k.dtype), dv.to(v.dtype), dw.to(ctx.w_dtype),
                 None, None, None, None, None, None)

@@ -130,10 +130,16 @@ int hils_pack_kv_chunks(const void* k, const void* v, void* workspace, int B, in
  * d_o (B,L,HQ,Dv) bf16, lse from the forward.
  * dq (B,L,HQ,D) bf16 (written); dk (B,Lkv,H,D) fp32, dv (B,Lkv,H,Dv) fp32 (ACCUMULATED
  * with atomics: caller zero-fills); dw fp32 (B,L/q_block,WH,NW) (accumulated with
- * atomics when q_block > 1 or WH != HQ, written otherwise: caller zero-fills). */
+ * atomics when q_block > 1 or WH != HQ, written otherwise: caller zero-fills).
+ * workspace: device scratch of hils_sparse_attn_bwd_workspace(...) bytes (0 = shape not covered)
+ * for the MFMA kernels: an inverse index (pairs of (query, slot) grouped by chunk) is built there
+ * and dK, dV are then computed chunk-major without atomics.  NULL selects the shape-generic
+ * kernel for everything. */
+size_t hils_sparse_attn_bwd_workspace(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K,
+                                      int WH, int q_block, int S, float sm_n);
 int hils_sparse_attn_bwd(const void* q, const void* k, const void* v, const void* weights,
                          const int32_t* indices, const float* slope, const float* lse,
-                         const void* d_o, void* dq, float* dk, float* dv, float* dw,
+                         const void* d_o, void* dq, float* dk, float* dv, float* dw, void* workspace,
                          int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
                          int WH, int q_block, int S, float sm_scale, int mask_last, float sm_n,
                          void* stream);
