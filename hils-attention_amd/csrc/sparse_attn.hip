@@ -324,10 +324,10 @@ bool hils_bw_covers(int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S, 
                     float sm_n, const float* slope);
 size_t hils_bw_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S,
                                int q_block, int WH, float sm_n);
-int hils_bw_dkdv(const void* q, const void* k, const void* v, const void* weights, const int32_t* indices,
-                 const float* lse, const void* d_o, float* dk, float* dv, void* workspace, int B, int L,
-                 int Lkv, int HQ, int H, int D, int Dv, int K, int NW, float sm_scale, int mask_last,
-                 void* stream);
+int hils_bw_run(const void* q, const void* k, const void* v, const void* weights, const int32_t* indices,
+                const float* lse, const void* d_o, void* dq, float* dk, float* dv, float* dw,
+                void* workspace, int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
+                float sm_scale, int mask_last, void* stream);
 
 extern "C" size_t hils_sparse_attn_bwd_workspace(int B, int L, int Lkv, int HQ, int H, int D, int Dv,
                                                  int K, int WH, int q_block, int S, float sm_n) {
@@ -344,19 +344,23 @@ extern "C" int hils_sparse_attn_bwd(const void* q, const void* k, const void* v,
   HILS_REQUIRE(q && k && v && weights && indices && lse && d_o && dq && dk && dv && dw,
                "hils_sparse_attn_bwd: null pointer");
   if (int rc = sa_check("hils_sparse_attn_bwd", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
-  const bool fast = workspace && hils_bw_covers(L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n, slope);
-  SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n, fast ? 1 : 0};
+  if (workspace && hils_bw_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n) > 0 &&
+      hils_bw_covers(L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n, slope)) {
+    const int rc = hils_bw_run(q, k, v, weights, indices, lse, d_o, dq, dk, dv, dw, workspace, B, L, Lkv, HQ,
+                               H, D, Dv, K, NW, sm_scale, mask_last, stream);
+    if (rc > 0) return rc;
+    if (rc == HILS_OK) {
+      HILS_CHECK_LAUNCH("hils_sparse_attn_bwd");
+      return HILS_OK;
+    }
+  }
+  SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n, 0};
   size_t smem = ((size_t)dm.G * (D + Dv) + 2 * (size_t)dm.G * S + 3 * dm.G) * sizeof(float);
   HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_bwd: G*(D+Dv+2S) too large for LDS");
   hipLaunchKernelGGL(sparse_attn_bwd_simple, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS),
                      smem, (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k,
                      (const bf16_t*)v, (const bf16_t*)weights, indices, slope, lse,
                      (const bf16_t*)d_o, (bf16_t*)dq, dk, dv, dw, dm);
-  if (fast) {
-    const int rc = hils_bw_dkdv(q, k, v, weights, indices, lse, d_o, dk, dv, workspace, B, L, Lkv, HQ, H, D,
-                                Dv, K, NW, sm_scale, mask_last, stream);
-    HILS_REQUIRE(rc == HILS_OK, "hils_sparse_attn_bwd: no dK/dV kernel for this shape");
-  }
   HILS_CHECK_LAUNCH("hils_sparse_attn_bwd");
   return HILS_OK;
 }

@@ -283,6 +283,279 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
 }
 
 // ---------------------------------------------------------------------------
+// dQ, dW: query-block-major, like the forward kernel.  One workgroup owns T consecutive
+// queries of a (batch, KV head), sorts the T*K (query, slot) pairs by chunk in LDS, and its
+// wavefronts take chunks from a shared counter.  Per 16-row tile of a visit, with the scores
+// in the orientation tokens x rows:
+//   S^T  = K Q^T,  dP^T = V dO^T      (16x16x32 MFMAs, K and V of the chunk as A operands)
+//   P = exp2(S c2 - lse2), delta = sum_tokens P dP (= dW of the pair), dS = w P (dP - delta)
+//   dQ  += scale dS K                 (dS^T in accumulator layout is the A operand; K of the chunk
+//                                      pre-transposed as B operand)
+// dQ tiles are added into an LDS tile of the block as 32-bit fixed point (integer LDS atomics),
+// scaled by a power of two from the bound  scale * 2 * max_row(sum_k|w| * |dO|_1) * max|V| * max|K|.
+// ---------------------------------------------------------------------------
+#define BQ_THREADS 512
+#define BQ_WAVES (BQ_THREADS / 64)
+
+struct BqDims {
+  int L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last;
+  float sm_scale;
+};
+
+template <int D, int DV, int G>
+__global__ void __launch_bounds__(BQ_THREADS)
+bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const bf16_t* __restrict__ ka,
+             const bf16_t* __restrict__ va, const bf16_t* __restrict__ kt, const float* __restrict__ vmax,
+             const float* __restrict__ kmax, const bf16_t* __restrict__ weights,
+             const int32_t* __restrict__ indices, const float* __restrict__ lse, bf16_t* __restrict__ dq,
+             float* __restrict__ dw, BqDims dm) {
+  constexpr int KS = D / 32, VS = DV / 32;
+  constexpr int DT = D / 16;
+  constexpr int QT = 16 / G;
+  constexpr int MAXP = 8;
+  extern __shared__ int smem_i[];
+  const int R = dm.T * G;
+  int* q_acc = smem_i;                       // (R + 1) x D fixed point; row R takes padding rows
+  int* cur = q_acc + (size_t)(R + 1) * D;    // nchunk: histogram -> running ends
+  int* pairs = cur + dm.nchunk;              // T*K pairs (query << 8 | slot) grouped by chunk
+  __shared__ float red[32];
+  __shared__ int scan_s[BQ_WAVES];
+  __shared__ int next_s;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  const int total = dm.nblk * dm.H * dm.B;
+  const int per_xcd = (total + 7) / 8;
+  const int vid = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+  if (vid >= total) return;
+  const int unit = vid / dm.nblk;
+  const int blk = dm.nblk - 1 - (vid - unit * dm.nblk);
+  const int hk = unit % dm.H;
+  const long b = unit / dm.H;
+  const int t0 = blk * dm.T;
+  const int K = dm.K;
+  const int npair = dm.T * K;
+
+  // selected chunk of every (query, slot) pair of the block
+  int creg[MAXP], preg[MAXP];
+#pragma unroll
+  for (int e = 0; e < MAXP; ++e) {
+    const int i = tid + e * BQ_THREADS;
+    int c = -1;
+    preg[e] = 0;
+    if (i < npair) {
+      const int ql = i / K, slot = i - ql * K;
+      preg[e] = (ql << 8) | slot;
+      if (t0 + ql < dm.L) c = indices[((b * dm.L + t0 + ql) * dm.H + hk) * (long)K + slot];
+    }
+    if (c < 0 || c >= dm.nchunk) c = -1;
+    creg[e] = c;
+  }
+  // row bound: sum_k |w| * |dO|_1
+  float rb = 0.f;
+  for (int row = tid; row < R; row += BQ_THREADS) {
+    const int ql = row / G, g = row - ql * G;
+    if (t0 + ql < dm.L) {
+      const long rowi = (b * dm.L + t0 + ql) * (long)dm.HQ + hk * G + g;
+      float a = 0.f;
+      for (int s2 = 0; s2 < K; ++s2) a += fabsf(bf2f(weights[rowi * dm.NW + s2]));
+      float l1 = 0.f;
+#pragma unroll
+      for (int p8 = 0; p8 < DV / 8; ++p8) {
+        float f[8];
+        unpack8(*(const uint4*)(d_o + rowi * DV + p8 * 8), f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) l1 += fabsf(f[e]);
+      }
+      rb = fmaxf(rb, a * l1);
+    }
+  }
+  for (int i = tid; i < (R + 1) * D; i += BQ_THREADS) q_acc[i] = 0;
+  for (int i = tid; i < dm.nchunk; i += BQ_THREADS) cur[i] = 0;
+  if (tid == 0) next_s = 0;
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < MAXP; ++e)
+    if (creg[e] >= 0) atomicAdd(&cur[creg[e]], 1);
+  rb = block_max(rb, red);  // barrier: histogram complete
+  float vm = 0.f, km = 0.f;
+  const int per_thr = (dm.nchunk + BQ_THREADS - 1) / BQ_THREADS;
+  const int c_lo = tid * per_thr;
+  int local = 0;
+  for (int c = c_lo; c < c_lo + per_thr && c < dm.nchunk; ++c) {
+    const int h = cur[c];
+    if (h > 0) {
+      vm = fmaxf(vm, vmax[(b * dm.H + hk) * (long)dm.nchunk + c]);
+      km = fmaxf(km, kmax[(b * dm.H + hk) * (long)dm.nchunk + c]);
+    }
+    local += h;
+  }
+  int incl = local;
+#pragma unroll
+  for (int o2 = 1; o2 < 64; o2 <<= 1) {
+    const int x = __shfl_up(incl, o2, 64);
+    if (lane >= o2) incl += x;
+  }
+  if (lane == 63) scan_s[wave] = incl;
+  vm = block_max(vm, red);  // barrier: scan_s visible, all histogram reads done
+  km = block_max(km, red);
+  int base = incl - local;
+  for (int w2 = 0; w2 < wave; ++w2) base += scan_s[w2];
+  for (int c = c_lo; c < c_lo + per_thr && c < dm.nchunk; ++c) {
+    const int h = cur[c];
+    cur[c] = base;
+    base += h;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < MAXP; ++e)
+    if (creg[e] >= 0) pairs[atomicAdd(&cur[creg[e]], 1)] = preg[e];
+  __syncthreads();  // now chunk c owns pairs[cur[c-1] .. cur[c])
+
+  const float bound = 2.f * dm.sm_scale * rb * vm * km;
+  float fx_scale = 1.f;
+  if (bound > 0.f && bound < 3.0e38f) {
+    int e2 = 28 - ilogbf(bound);
+    e2 = e2 > 90 ? 90 : (e2 < -90 ? -90 : e2);
+    fx_scale = ldexpf(1.f, e2);
+  }
+  const float fx_inv = 1.f / fx_scale;
+  const float c2 = dm.sm_scale * HILS_LOG2E;
+  const float out_scale = dm.sm_scale * fx_scale;
+  const int qs = r / G, g = r - qs * G;  // this lane's row of a tile: query slot, head
+  const int hq = hk * G + g;
+  const int npair_valid = cur[dm.nchunk - 1];
+
+  for (;;) {
+    int c = 0;
+    if (lane == 0) c = atomicAdd(&next_s, 1);
+    c = __builtin_amdgcn_readfirstlane(c);
+    if (c >= dm.nchunk) break;
+    const int vs = c ? cur[c - 1] : 0;
+    if (vs >= npair_valid) break;
+    const int ve = cur[c];
+    if (vs == ve) continue;
+    const long chunk = (b * dm.H + hk) * (long)dm.nchunk + c;
+    const bf16_t* ka_c = ka + chunk * (long)BW_S * D + lane * 8;
+    const bf16_t* va_c = va + chunk * (long)BW_S * DV + lane * 8;
+    const bf16_t* kt_c = kt + chunk * (long)BW_S * D + lane * 8;
+    for (int p = vs; p < ve; p += QT) {
+      const int last = ((ve - p < QT) ? ve - p : QT) - 1;  // padding rows repeat the tile's last pair
+      // ---- operands of the two score products and the tile's rows
+      uint4 xa[4 * KS], ya[4 * VS];
+#pragma unroll
+      for (int u = 0; u < 4 * KS; ++u) xa[u] = *(const uint4*)(ka_c + u * 512);
+#pragma unroll
+      for (int u = 0; u < 4 * VS; ++u) ya[u] = *(const uint4*)(va_c + u * 512);
+      const int pk = pairs[p + (qs < last ? qs : last)];
+      int pk_o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int qsl = (4 * j + i) / G;
+        pk_o[i] = pairs[p + (qsl < last ? qsl : last)];
+      }
+      const int ql = pk >> 8, slot = pk & 255;
+      const long rowi = (b * dm.L + t0 + ql) * (long)dm.HQ + hq;
+      uint4 bq[KS], bdo[VS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) bq[ks] = *(const uint4*)(q + rowi * D + ks * 32 + j * 8);
+#pragma unroll
+      for (int ks = 0; ks < VS; ++ks) bdo[ks] = *(const uint4*)(d_o + rowi * DV + ks * 32 + j * 8);
+      float l2 = lse[rowi * K + slot];
+      if (l2 == HILS_NEG_INF) l2 = INFINITY;
+      const float w_row = bf2f(weights[rowi * dm.NW + slot]);
+      int orow[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int rr = 4 * j + i;
+        const int qsl = rr / G;
+        const int row = (qsl <= last) ? (pk_o[i] >> 8) * G + (rr - qsl * G) : R;
+        orow[i] = row * D + r;
+      }
+      // ---- S^T and dP^T: tokens x rows, four token tiles each
+      f32x4_t st[4], dpt[4];
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        st[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+        dpt[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+          st[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&xa[mt * KS + ks], *(const bf16x8_t*)&bq[ks], st[mt], 0, 0, 0);
+#pragma unroll
+      for (int ks = 0; ks < VS; ++ks)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+          dpt[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&ya[mt * VS + ks], *(const bf16x8_t*)&bdo[ks], dpt[mt], 0, 0, 0);
+      // K of the chunk as B operand of dQ = dS K replaces the first operand set
+#pragma unroll
+      for (int u = 0; u < 2 * DT; ++u) xa[u] = *(const uint4*)(kt_c + u * 512);
+      // ---- P, delta, dS (this lane: row r of the tile, tokens mt*16 + 4j + i)
+      float delta = 0.f;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float pv = __builtin_amdgcn_exp2f(st[mt][i] * c2 - l2);
+          st[mt][i] = pv;
+          delta += pv * dpt[mt][i];
+        }
+      if (dm.mask_last && j == 3) {  // token 63 = tile 3, lane group 3, register 3
+        delta -= st[3][3] * dpt[3][3];
+        st[3][3] = 0.f;
+      }
+      delta = rows_sum(delta);
+      if (j == 0 && qs <= last) dw[rowi * dm.NW + slot] = delta;
+      const float f = w_row * out_scale;
+      bf16x8_t ap[2];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        uint4 x;
+        x.x = pack_bf2(f * st[2 * s2][0] * (dpt[2 * s2][0] - delta), f * st[2 * s2][1] * (dpt[2 * s2][1] - delta));
+        x.y = pack_bf2(f * st[2 * s2][2] * (dpt[2 * s2][2] - delta), f * st[2 * s2][3] * (dpt[2 * s2][3] - delta));
+        x.z = pack_bf2(f * st[2 * s2 + 1][0] * (dpt[2 * s2 + 1][0] - delta), f * st[2 * s2 + 1][1] * (dpt[2 * s2 + 1][1] - delta));
+        x.w = pack_bf2(f * st[2 * s2 + 1][2] * (dpt[2 * s2 + 1][2] - delta), f * st[2 * s2 + 1][3] * (dpt[2 * s2 + 1][3] - delta));
+        ap[s2] = *(bf16x8_t*)&x;
+      }
+      // ---- dQ tile += dS K: four column tiles at a time
+#pragma unroll
+      for (int d0 = 0; d0 < DT; d0 += 4) {
+        f32x4_t acc[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc[u] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s2], *(const bf16x8_t*)&xa[(d0 + u) * 2 + s2], acc[u], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) atomicAdd(&q_acc[orow[i] + (d0 + u) * 16], __float2int_rn(acc[u][i]));
+      }
+    }
+  }
+  __syncthreads();
+  constexpr int C8 = D / 8;
+  for (int i = tid; i < R * C8; i += BQ_THREADS) {
+    const int row = i / C8, c8 = i - row * C8;
+    const int ql = row / G, g2 = row - ql * G;
+    const int t = t0 + ql;
+    if (t < dm.L) {
+      const int* src = q_acc + (size_t)row * D + c8 * 8;
+      uint4 x;
+      x.x = pack_bf2((float)src[0] * fx_inv, (float)src[1] * fx_inv);
+      x.y = pack_bf2((float)src[2] * fx_inv, (float)src[3] * fx_inv);
+      x.z = pack_bf2((float)src[4] * fx_inv, (float)src[5] * fx_inv);
+      x.w = pack_bf2((float)src[6] * fx_inv, (float)src[7] * fx_inv);
+      *(uint4*)(dq + ((b * dm.L + t) * (long)dm.HQ + hk * G + g2) * D + c8 * 8) = x;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 static size_t bw_round(size_t n) { return (n + 255) & ~(size_t)255; }
@@ -296,11 +569,52 @@ bool hils_bw_covers(int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S, 
          slope == nullptr && Lkv % S == 0 && K <= 256 && L < (1 << 24) && Lkv / S <= 12288;
 }
 
+void hils_ga_pack_launch(const void* a, const void* b, void* ap, void* bp, float* bmax, int B, int Lkv,
+                         int H, int Da, int Db, void* stream);
+
+// T queries per workgroup of the dQ kernel such that the fixed-point tile, the chunk histogram
+// and the pair list fit in LDS; 0 when the shape does not fit.
+static int bq_pick_T(int L, int G, int D, int K, int nchunk, size_t* smem_out) {
+  int T = (128 * 1024) / (G * D * 4);
+  if (T * K > 8 * BQ_THREADS) T = (8 * BQ_THREADS) / K;
+  if (T > L) T = L;
+  while (T >= 1) {
+    const size_t smem = (size_t)(T * G + 1) * D * 4 + (size_t)nchunk * 4 + (size_t)T * K * 4;
+    if (smem <= 156 * 1024) {
+      *smem_out = smem;
+      return T;
+    }
+    T /= 2;
+  }
+  return 0;
+}
+
+struct BwLayout {
+  size_t counts, offsets, cursor, pairs, ka, va, kt, vmax, kmax, total;
+};
+static BwLayout bw_layout(int B, int L, int Lkv, int H, int D, int Dv, int K) {
+  const size_t cells = (size_t)B * H * (Lkv / BW_S);
+  BwLayout lo;
+  size_t o = 0;
+  lo.counts = o; o += bw_round((cells + 1) * 4);
+  lo.offsets = o; o += bw_round((cells + 1) * 4);
+  lo.cursor = o; o += bw_round((cells + 1) * 4);
+  lo.pairs = o; o += bw_round((size_t)B * L * H * K * 4);
+  lo.ka = o; o += bw_round(cells * BW_S * D * 2);
+  lo.va = o; o += bw_round(cells * BW_S * Dv * 2);
+  lo.kt = o; o += bw_round(cells * BW_S * D * 2);
+  lo.vmax = o; o += bw_round(cells * 4);
+  lo.kmax = o; o += bw_round(cells * 4);
+  lo.total = o;
+  return lo;
+}
+
 size_t hils_bw_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S,
                                int q_block, int WH, float sm_n) {
   if (!hils_bw_covers(L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n, nullptr)) return 0;
-  const size_t cells = (size_t)B * H * (Lkv / S);
-  return bw_round((cells + 1) * 4) * 3 + bw_round((size_t)B * L * H * K * 4);  // counts, offsets, cursor, pairs
+  size_t smem;
+  if (bq_pick_T(L, HQ / H, D, K, Lkv / S, &smem) == 0) return 0;
+  return bw_layout(B, L, Lkv, H, D, Dv, K).total;
 }
 
 template <int D, int DV>
@@ -323,20 +637,86 @@ static int bw_launch_dkdv(int G, dim3 grid, hipStream_t st, const bf16_t* q, con
   return HILS_OK;
 }
 
-// dK and dV (accumulated into the caller's fp32 buffers) through the inverse index.
-int hils_bw_dkdv(const void* q, const void* k, const void* v, const void* weights, const int32_t* indices,
-                 const float* lse, const void* d_o, float* dk, float* dv, void* workspace, int B, int L,
-                 int Lkv, int HQ, int H, int D, int Dv, int K, int NW, float sm_scale, int mask_last,
-                 void* stream) {
+template <int D, int DV, int G>
+static int bq_launch(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, const bf16_t* d_o,
+                     const bf16_t* ka, const bf16_t* va, const bf16_t* kt, const float* vmax,
+                     const float* kmax, const bf16_t* w, const int32_t* idx, const float* lse, bf16_t* dq,
+                     float* dw, const BqDims& dm) {
+  auto kern = bw_dq_kernel<D, DV, G>;
+  static size_t reserved = 0;  // per instantiation
+  if (smem > reserved) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+      hils_set_error("hils_sparse_attn_bwd: cannot reserve %zu bytes of LDS", smem);
+      return HILS_ERR_LAUNCH;
+    }
+    reserved = smem;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(BQ_THREADS), smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
+  return HILS_OK;
+}
+
+template <int D, int DV>
+static int bq_dispatch_g(int G, dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, const bf16_t* d_o,
+                         const bf16_t* ka, const bf16_t* va, const bf16_t* kt, const float* vmax,
+                         const float* kmax, const bf16_t* w, const int32_t* idx, const float* lse,
+                         bf16_t* dq, float* dw, const BqDims& dm) {
+  switch (G) {
+    case 1: return bq_launch<D, DV, 1>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
+    case 2: return bq_launch<D, DV, 2>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
+    case 4: return bq_launch<D, DV, 4>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
+    case 8: return bq_launch<D, DV, 8>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
+    case 16: return bq_launch<D, DV, 16>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
+  }
+  return -1;
+}
+
+// Whole backward on the MFMA kernels: dq (bf16, written), dw (fp32, written at the valid slots),
+// dk / dv (fp32, accumulated into the caller's buffers).
+int hils_bw_run(const void* q, const void* k, const void* v, const void* weights, const int32_t* indices,
+                const float* lse, const void* d_o, void* dq, float* dk, float* dv, float* dw,
+                void* workspace, int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
+                float sm_scale, int mask_last, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   const int nchunk = Lkv / BW_S;
   const size_t cells = (size_t)B * H * nchunk;
-  int* counts = (int*)workspace;
-  int* offsets = (int*)((char*)counts + bw_round((cells + 1) * 4));
-  int* cursor = (int*)((char*)offsets + bw_round((cells + 1) * 4));
-  uint32_t* pairs = (uint32_t*)((char*)cursor + bw_round((cells + 1) * 4));
+  const BwLayout lo = bw_layout(B, L, Lkv, H, D, Dv, K);
+  char* ws = (char*)workspace;
+  int* counts = (int*)(ws + lo.counts);
+  int* offsets = (int*)(ws + lo.offsets);
+  int* cursor = (int*)(ws + lo.cursor);
+  uint32_t* pairs = (uint32_t*)(ws + lo.pairs);
+  bf16_t* ka = (bf16_t*)(ws + lo.ka);
+  bf16_t* va = (bf16_t*)(ws + lo.va);
+  bf16_t* kt = (bf16_t*)(ws + lo.kt);
+  float* vmax = (float*)(ws + lo.vmax);
+  float* kmax = (float*)(ws + lo.kmax);
   const int G = HQ / H;
-  // zero the counts with a kernel (keeps the call capturable in a HIP graph)
+  if (H > 65535 || B > 65535) return -1;
+  // ---- operand packing: K as A operand (+ max|V|), V as A operand + K transposed (+ max|K|)
+  hils_ga_pack_launch(k, v, ka, nullptr, vmax, B, Lkv, H, D, Dv, stream);
+  hils_ga_pack_launch(v, k, va, kt, kmax, B, Lkv, H, Dv, D, stream);
+  // ---- dQ, dW
+  {
+    size_t smem;
+    const int T = bq_pick_T(L, G, D, K, nchunk, &smem);
+    if (T == 0) return -1;
+    const int nblk = (L + T - 1) / T;
+    const long total = (long)nblk * H * B;
+    if (total > (1L << 30)) return -1;
+    BqDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale};
+    dim3 grid((unsigned)(((total + 7) / 8) * 8));
+    int rc = -1;
+#define BQ_D(D_, DV_)                                                                                 \
+  rc = bq_dispatch_g<D_, DV_>(G, grid, smem, st, (const bf16_t*)q, (const bf16_t*)d_o, ka, va, kt, vmax, \
+                              kmax, (const bf16_t*)weights, indices, lse, (bf16_t*)dq, dw, dm)
+    if (D == 64 && Dv == 64) BQ_D(64, 64);
+    else if (D == 128 && Dv == 128) BQ_D(128, 128);
+    else if (D == 64 && Dv == 128) BQ_D(64, 128);
+    else if (D == 128 && Dv == 64) BQ_D(128, 64);
+#undef BQ_D
+    if (rc != HILS_OK) return rc;
+  }
+  // ---- inverse index, then dK, dV
   {
     const long n = (long)cells + 1;
     hipLaunchKernelGGL(bw_fill_int_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, counts, 0, n);

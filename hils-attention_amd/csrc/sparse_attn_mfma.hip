@@ -70,6 +70,7 @@ pack_kv_kernel(const bf16_t* __restrict__ k, const bf16_t* __restrict__ v, bf16_
   }
   mx = block_max(mx, red);  // contains the barrier that orders the tile writes
   if (threadIdx.x == 0) vmax[chunk] = mx;
+  if (!vp) return;  // only max|V| wanted
   bf16_t* out = vp + chunk * (long)GA_S * Dv;
   for (int i = threadIdx.x; i < Dv * 8; i += 256) {
     // destination order: ((dt * 2 + s) * 64 + lane)
@@ -627,6 +628,17 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
   if (rc != HILS_OK) return rc < 0 ? HILS_OK : rc;
   *handled = 1;
   return HILS_OK;
+}
+
+// Launches the packing kernel on explicit buffers: ap = a in A-operand order, bp = b in the
+// transposed B-operand order, bmax = max|b| per chunk (also used by the backward kernels).
+void hils_ga_pack_launch(const void* a, const void* b, void* ap, void* bp, float* bmax, int B, int Lkv,
+                         int H, int Da, int Db, void* stream) {
+  const int nchunk = Lkv / GA_S;
+  const int dmax = Da > Db ? Da : Db;
+  hipLaunchKernelGGL(pack_kv_kernel, dim3(nchunk, H, B), dim3(256),
+                     (size_t)GA_S * (dmax + 2) * sizeof(bf16_t), (hipStream_t)stream, (const bf16_t*)a,
+                     (const bf16_t*)b, (bf16_t*)ap, (bf16_t*)bp, bmax, Lkv, H, Da, Db, nchunk);
 }
 
 extern "C" int hils_pack_kv_chunks(const void* k, const void* v, void* workspace, int B, int Lkv,
