@@ -88,20 +88,35 @@ bw_scan_kernel(const int* __restrict__ counts, int* __restrict__ offsets, int* _
   if (tid == 0) offsets[n] = carry_s;
 }
 
-// pairs[cursor[(b,h,c)]++] = (t << 8 | slot)
+// pairs grouped by (b,h,c): a workgroup histograms its segment of queries in LDS, reserves one
+// range per chunk with a single global atomic, and scatters (t << 8 | slot) inside its ranges
 __global__ void __launch_bounds__(1024)
 bw_scatter_kernel(const int32_t* __restrict__ indices, int* __restrict__ cursor,
                   uint32_t* __restrict__ pairs, int L, int H, int K, int nchunk, int seg_len) {
+  extern __shared__ int pos[];  // nchunk: count -> next free position
   const int h = blockIdx.y;
   const long b = blockIdx.z;
   const int t_lo = blockIdx.x * seg_len;
   const int t_hi = (t_lo + seg_len < L) ? t_lo + seg_len : L;
   int* cur = cursor + (b * H + h) * (long)nchunk;
+  for (int i = threadIdx.x; i < nchunk; i += 1024) pos[i] = 0;
+  __syncthreads();
   const long n = (long)(t_hi - t_lo) * K;
   for (long i = threadIdx.x; i < n; i += 1024) {
     const int t = t_lo + (int)(i / K), slot = (int)(i % K);
     const int c = indices[((b * L + t) * H + h) * (long)K + slot];
-    if (c >= 0 && c < nchunk) pairs[atomicAdd(&cur[c], 1)] = ((uint32_t)t << 8) | (uint32_t)slot;
+    if (c >= 0 && c < nchunk) atomicAdd(&pos[c], 1);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < nchunk; i += 1024) {
+    const int cnt = pos[i];
+    pos[i] = cnt ? atomicAdd(&cur[i], cnt) : 0;
+  }
+  __syncthreads();
+  for (long i = threadIdx.x; i < n; i += 1024) {
+    const int t = t_lo + (int)(i / K), slot = (int)(i % K);
+    const int c = indices[((b * L + t) * H + h) * (long)K + slot];
+    if (c >= 0 && c < nchunk) pairs[atomicAdd(&pos[c], 1)] = ((uint32_t)t << 8) | (uint32_t)slot;
   }
 }
 
@@ -117,9 +132,10 @@ template <int D, int DV, int G>
 __global__ void __launch_bounds__(256)
 bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
                const bf16_t* __restrict__ weights, const float* __restrict__ lse,
-               const bf16_t* __restrict__ d_o, const int* __restrict__ offsets,
-               const uint32_t* __restrict__ pairs, float* __restrict__ dk, float* __restrict__ dv,
-               BwDims dm) {
+               const float* __restrict__ delta, const bf16_t* __restrict__ d_o,
+               const int* __restrict__ offsets, const uint32_t* __restrict__ pairs,
+               float* __restrict__ dk, float* __restrict__ dv, BwDims dm) {
+  // delta (B,L,HQ,NW) fp32: sum_tokens P dP of every (row, slot), written by the dQ kernel
   constexpr int KS = D / 32, VS = DV / 32;    // k-steps of the two 16x16x32 products
   constexpr int DT = D / 16, VT = DV / 16;    // 16-wide column tiles of dK, dV
   constexpr int QT = 16 / G;                  // pairs per 16-row tile
@@ -130,8 +146,7 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
   __shared__ __attribute__((aligned(16))) char o_rm[16 * OROW];
   __shared__ __attribute__((aligned(16))) char q_tr[D * CS];
   __shared__ __attribute__((aligned(16))) char o_tr[DV * CS];
-  __shared__ float row_lse[16], row_w[16];
-  __shared__ float red[4][16];
+  __shared__ float row_lse[16], row_w[16], row_delta[16];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, j = lane >> 4;
@@ -159,52 +174,98 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
   for (int t = 0; t < VT; ++t) acc_v[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   const float c2 = dm.sm_scale * HILS_LOG2E;
 
-  // staging roles: thread -> (row, 16-byte piece) of the Q tile and of the dO tile
+  // Staging roles.  Threads are paired over two neighbouring rows of a tile: thread -> (row,
+  // 16-byte piece); the partner (row ^ 1, same piece) sits QPP (OPP) lanes away, so a pair can
+  // assemble dwords of (row 2a, row 2a+1) for the transposed copy.
   constexpr int QPP = D / 8, OPP = DV / 8;
   const int q_row = tid / QPP, q_pc = tid % QPP;
   const int o_row = tid / OPP, o_pc = tid % OPP;
   const int npair = p_hi - p_lo;
+  const int ntile = (npair + QT - 1) / QT;
 
-  for (int p0 = 0; p0 < npair; p0 += QT) {
-    const int n = (npair - p0 < QT) ? npair - p0 : QT;  // pairs in this tile
+  // gathered data of the next tile, fetched one tile ahead
+  auto pair_of = [&](int tile, int row) -> uint32_t {  // pair of a tile row; ~0u for padding rows
+    const int pi = tile * QT + row / G;
+    return (row < 16 && pi < npair) ? pairs[p_lo + pi] : 0xffffffffu;
+  };
+  uint32_t pk_q = pair_of(0, q_row), pk_o = pair_of(0, o_row), pk_r = pair_of(0, tid);
+  uint4 xq = make_uint4(0, 0, 0, 0), xo = make_uint4(0, 0, 0, 0);
+  float r_l2 = INFINITY, r_w = 0.f, r_dl = 0.f;
+  auto fetch = [&]() {
+    xq = make_uint4(0, 0, 0, 0);
+    xo = make_uint4(0, 0, 0, 0);
+    if (pk_q != 0xffffffffu)
+      xq = *(const uint4*)(q + ((b * dm.L + (pk_q >> 8)) * (long)dm.HQ + hk * G + q_row % G) * D + q_pc * 8);
+    if (pk_o != 0xffffffffu)
+      xo = *(const uint4*)(d_o + ((b * dm.L + (pk_o >> 8)) * (long)dm.HQ + hk * G + o_row % G) * DV + o_pc * 8);
+    r_l2 = INFINITY;  // padding rows: P = 0
+    r_w = 0.f;
+    r_dl = 0.f;
+    if (tid < 16 && pk_r != 0xffffffffu) {
+      const long rowi = (b * dm.L + (pk_r >> 8)) * (long)dm.HQ + hk * G + tid % G;
+      r_l2 = lse[rowi * dm.K + (pk_r & 255)];
+      if (r_l2 == HILS_NEG_INF) r_l2 = INFINITY;
+      r_w = bf2f(weights[rowi * dm.NW + (pk_r & 255)]);
+      r_dl = delta[rowi * dm.NW + (pk_r & 255)];
+    }
+  };
+  fetch();
+  pk_q = pair_of(1, q_row);
+  pk_o = pair_of(1, o_row);
+  pk_r = pair_of(1, tid);
+
+  for (int tile = 0; tile < ntile; ++tile) {
     __syncthreads();  // the previous tile's staging is no longer read
     // ---- stage the gathered rows: row-major (A operands) and transposed (B operands)
     if (q_row < 16) {
-      uint4 x = make_uint4(0, 0, 0, 0);
-      const int pr = q_row / G, g = q_row - pr * G;
-      if (pr < n) {
-        const uint32_t pk = pairs[p_lo + p0 + pr];
-        x = *(const uint4*)(q + ((b * dm.L + (pk >> 8)) * (long)dm.HQ + hk * G + g) * D + q_pc * 8);
-      }
-      *(uint4*)(q_rm + q_row * QROW + q_pc * 16) = x;
-      const bf16_t* xe = (const bf16_t*)&x;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) *(bf16_t*)(q_tr + (q_pc * 8 + e) * CS + q_row * 2) = xe[e];
+      *(uint4*)(q_rm + q_row * QROW + q_pc * 16) = xq;
+      // partner row's piece: even rows write features 0..3 of the piece, odd rows 4..7
+      uint4 y;
+      y.x = __shfl_xor((int)xq.x, QPP, 64);
+      y.y = __shfl_xor((int)xq.y, QPP, 64);
+      y.z = __shfl_xor((int)xq.z, QPP, 64);
+      y.w = __shfl_xor((int)xq.w, QPP, 64);
+      const bool odd = q_row & 1;
+      const uint32_t me0 = odd ? xq.z : xq.x, me1 = odd ? xq.w : xq.y;
+      const uint32_t ot0 = odd ? y.z : y.x, ot1 = odd ? y.w : y.y;
+      // dword = (even row value, odd row value) of one feature
+      const uint32_t ev0 = odd ? ot0 : me0, od0 = odd ? me0 : ot0;
+      const uint32_t ev1 = odd ? ot1 : me1, od1 = odd ? me1 : ot1;
+      char* dst = q_tr + (q_pc * 8 + (odd ? 4 : 0)) * CS + (q_row & ~1) * 2;
+      *(uint32_t*)(dst + 0 * CS) = (ev0 & 0xffffu) | (od0 << 16);
+      *(uint32_t*)(dst + 1 * CS) = (ev0 >> 16) | (od0 & 0xffff0000u);
+      *(uint32_t*)(dst + 2 * CS) = (ev1 & 0xffffu) | (od1 << 16);
+      *(uint32_t*)(dst + 3 * CS) = (ev1 >> 16) | (od1 & 0xffff0000u);
     }
     if (o_row < 16) {
-      uint4 x = make_uint4(0, 0, 0, 0);
-      const int pr = o_row / G, g = o_row - pr * G;
-      if (pr < n) {
-        const uint32_t pk = pairs[p_lo + p0 + pr];
-        x = *(const uint4*)(d_o + ((b * dm.L + (pk >> 8)) * (long)dm.HQ + hk * G + g) * DV + o_pc * 8);
-      }
-      *(uint4*)(o_rm + o_row * OROW + o_pc * 16) = x;
-      const bf16_t* xe = (const bf16_t*)&x;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) *(bf16_t*)(o_tr + (o_pc * 8 + e) * CS + o_row * 2) = xe[e];
+      *(uint4*)(o_rm + o_row * OROW + o_pc * 16) = xo;
+      uint4 y;
+      y.x = __shfl_xor((int)xo.x, OPP, 64);
+      y.y = __shfl_xor((int)xo.y, OPP, 64);
+      y.z = __shfl_xor((int)xo.z, OPP, 64);
+      y.w = __shfl_xor((int)xo.w, OPP, 64);
+      const bool odd = o_row & 1;
+      const uint32_t me0 = odd ? xo.z : xo.x, me1 = odd ? xo.w : xo.y;
+      const uint32_t ot0 = odd ? y.z : y.x, ot1 = odd ? y.w : y.y;
+      const uint32_t ev0 = odd ? ot0 : me0, od0 = odd ? me0 : ot0;
+      const uint32_t ev1 = odd ? ot1 : me1, od1 = odd ? me1 : ot1;
+      char* dst = o_tr + (o_pc * 8 + (odd ? 4 : 0)) * CS + (o_row & ~1) * 2;
+      *(uint32_t*)(dst + 0 * CS) = (ev0 & 0xffffu) | (od0 << 16);
+      *(uint32_t*)(dst + 1 * CS) = (ev0 >> 16) | (od0 & 0xffff0000u);
+      *(uint32_t*)(dst + 2 * CS) = (ev1 & 0xffffu) | (od1 << 16);
+      *(uint32_t*)(dst + 3 * CS) = (ev1 >> 16) | (od1 & 0xffff0000u);
     }
     if (tid < 16) {
-      const int pr = tid / G, g = tid - pr * G;
-      float l2 = INFINITY, w = 0.f;  // padding rows: P = 0
-      if (pr < n) {
-        const uint32_t pk = pairs[p_lo + p0 + pr];
-        const long rowi = (b * dm.L + (pk >> 8)) * (long)dm.HQ + hk * G + g;
-        l2 = lse[rowi * dm.K + (pk & 255)];
-        if (l2 == HILS_NEG_INF) l2 = INFINITY;
-        w = bf2f(weights[rowi * dm.NW + (pk & 255)]);
-      }
-      row_lse[tid] = l2;
-      row_w[tid] = w;
+      row_lse[tid] = r_l2;
+      row_w[tid] = r_w;
+      row_delta[tid] = r_dl;
+    }
+    // next tile's gathers fly during this tile's arithmetic
+    if (tile + 1 < ntile) {
+      fetch();
+      pk_q = pair_of(tile + 2, q_row);
+      pk_o = pair_of(tile + 2, o_row);
+      pk_r = pair_of(tile + 2, tid);
     }
     __syncthreads();
     // ---- S and dP for this wavefront's 16 tokens
@@ -220,34 +281,16 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
       dp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&vb[ks], dp, 0, 0, 0);
     }
     // accumulator layout: column = token `col`, registers = rows 4j..4j+3
-    float pr4[4], part[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float pv = __builtin_amdgcn_exp2f(s[i] * c2 - row_lse[4 * j + i]);
-      if (masked_col) pv = 0.f;
-      pr4[i] = pv;
-      part[i] = pv * dp[i];
-    }
-    // delta of a row = sum over the 64 tokens: 16 lanes of the row group, then 4 wavefronts
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      part[i] = row_sum<16>(part[i]);
-    }
-    if (col == 0) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) red[wave][4 * j + i] = part[i];
-    }
-    __syncthreads();
     bw_s4 a_p, a_ds;
     {
       float pw[4], ds[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = 4 * j + i;
-        const float delta = red[0][r] + red[1][r] + red[2][r] + red[3][r];
-        const float w = row_w[r];
-        pw[i] = w * pr4[i];
-        ds[i] = pw[i] * (dp[i] - delta);
+        float pv = __builtin_amdgcn_exp2f(s[i] * c2 - row_lse[r]);
+        if (masked_col) pv = 0.f;
+        pw[i] = row_w[r] * pv;
+        ds[i] = pw[i] * (dp[i] - row_delta[r]);
       }
       uint2 x;
       x.x = pack_bf2(pw[0], pw[1]);
@@ -619,12 +662,12 @@ size_t hils_bw_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int 
 
 template <int D, int DV>
 static int bw_launch_dkdv(int G, dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* k,
-                          const bf16_t* v, const bf16_t* w, const float* lse, const bf16_t* d_o,
-                          const int* offsets, const uint32_t* pairs, float* dk, float* dv,
+                          const bf16_t* v, const bf16_t* w, const float* lse, const float* delta,
+                          const bf16_t* d_o, const int* offsets, const uint32_t* pairs, float* dk, float* dv,
                           const BwDims& dm) {
 #define BW_CALL(G_)                                                                                 \
-  hipLaunchKernelGGL((bw_dkdv_kernel<D, DV, G_>), grid, dim3(256), 0, st, q, k, v, w, lse, d_o, offsets, \
-                     pairs, dk, dv, dm)
+  hipLaunchKernelGGL((bw_dkdv_kernel<D, DV, G_>), grid, dim3(256), 0, st, q, k, v, w, lse, delta, d_o,  \
+                     offsets, pairs, dk, dv, dm)
   switch (G) {
     case 1: BW_CALL(1); break;
     case 2: BW_CALL(2); break;
@@ -726,13 +769,13 @@ int hils_bw_run(const void* q, const void* k, const void* v, const void* weights
   dim3 gs((L + seg_len - 1) / seg_len, H, B);
   hipLaunchKernelGGL(bw_count_kernel, gs, dim3(1024), (size_t)nchunk * 4, st, indices, counts, L, H, K, nchunk, seg_len);
   hipLaunchKernelGGL(bw_scan_kernel, dim3(1), dim3(1024), 0, st, counts, offsets, cursor, (long)cells);
-  hipLaunchKernelGGL(bw_scatter_kernel, gs, dim3(1024), 0, st, indices, cursor, pairs, L, H, K, nchunk, seg_len);
+  hipLaunchKernelGGL(bw_scatter_kernel, gs, dim3(1024), (size_t)nchunk * 4, st, indices, cursor, pairs, L, H, K, nchunk, seg_len);
   BwDims dm{L, Lkv, HQ, H, K, NW, nchunk, mask_last, sm_scale};
   dim3 grid(nchunk, H, B);
   int rc = -1;
 #define BW_D(D_, DV_)                                                                              \
   rc = bw_launch_dkdv<D_, DV_>(G, grid, st, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v,   \
-                               (const bf16_t*)weights, lse, (const bf16_t*)d_o, offsets, pairs, dk, dv, dm)
+                               (const bf16_t*)weights, lse, dw, (const bf16_t*)d_o, offsets, pairs, dk, dv, dm)
   if (D == 64 && Dv == 64) BW_D(64, 64);
   else if (D == 128 && Dv == 128) BW_D(128, 128);
   else if (D == 64 && Dv == 128) BW_D(64, 128);
