@@ -138,15 +138,21 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
   // delta (B,L,HQ,NW) fp32: sum_tokens P dP of every (row, slot), written by the dQ kernel
   constexpr int KS = D / 32, VS = DV / 32;    // k-steps of the two 16x16x32 products
   constexpr int DT = D / 16, VT = DV / 16;    // 16-wide column tiles of dK, dV
-  constexpr int QT = 16 / G;                  // pairs per 16-row tile
+  constexpr int DMAX = D > DV ? D : DV;
+  constexpr int NSUB = 256 / DMAX;            // 16-row tiles staged per round (4 or 2)
+  constexpr int ROWS = 16 * NSUB;             // rows per round
+  constexpr int PPR = ROWS / G;               // pairs per round
   constexpr int QROW = D * 2 + 16;            // row-major staging: padded row (bytes)
   constexpr int OROW = DV * 2 + 16;
   constexpr int CS = 40;                      // transposed staging: bytes per feature column (16 rows + pad)
-  __shared__ __attribute__((aligned(16))) char q_rm[16 * QROW];
-  __shared__ __attribute__((aligned(16))) char o_rm[16 * OROW];
-  __shared__ __attribute__((aligned(16))) char q_tr[D * CS];
-  __shared__ __attribute__((aligned(16))) char o_tr[DV * CS];
-  __shared__ float row_lse[16], row_w[16], row_delta[16];
+  extern __shared__ __attribute__((aligned(16))) char bw_smem[];
+  char* q_rm = bw_smem;                       // ROWS x QROW
+  char* o_rm = q_rm + ROWS * QROW;            // ROWS x OROW
+  char* q_tr = o_rm + ROWS * OROW;            // NSUB x D x CS
+  char* o_tr = q_tr + NSUB * D * CS;          // NSUB x DV x CS
+  float* row_lse = (float*)(o_tr + NSUB * DV * CS);
+  float* row_w = row_lse + ROWS;
+  float* row_delta = row_w + ROWS;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, j = lane >> 4;
@@ -174,34 +180,48 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
   for (int t = 0; t < VT; ++t) acc_v[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   const float c2 = dm.sm_scale * HILS_LOG2E;
 
-  // Staging roles.  Threads are paired over two neighbouring rows of a tile: thread -> (row,
-  // 16-byte piece); the partner (row ^ 1, same piece) sits QPP (OPP) lanes away, so a pair can
-  // assemble dwords of (row 2a, row 2a+1) for the transposed copy.
+  // Staging roles: thread -> (row, 16-byte piece), NQ (NO) items per thread and round.  The
+  // thread of the neighbouring row (row ^ 1, same piece) sits QPP (OPP) lanes away, so a pair of
+  // threads can assemble dwords of (row 2a, row 2a+1) for the transposed copy.
   constexpr int QPP = D / 8, OPP = DV / 8;
-  const int q_row = tid / QPP, q_pc = tid % QPP;
-  const int o_row = tid / OPP, o_pc = tid % OPP;
+  constexpr int NQ = ROWS * QPP / 256, NO = ROWS * OPP / 256;
+  constexpr int QRS = 256 / QPP, ORS = 256 / OPP;  // row step between a thread's items
+  const int q_row0 = tid / QPP, q_pc = tid % QPP;
+  const int o_row0 = tid / OPP, o_pc = tid % OPP;
   const int npair = p_hi - p_lo;
-  const int ntile = (npair + QT - 1) / QT;
+  const int nround = (npair + PPR - 1) / PPR;
 
-  // gathered data of the next tile, fetched one tile ahead
-  auto pair_of = [&](int tile, int row) -> uint32_t {  // pair of a tile row; ~0u for padding rows
-    const int pi = tile * QT + row / G;
-    return (row < 16 && pi < npair) ? pairs[p_lo + pi] : 0xffffffffu;
+  auto pair_of = [&](int round, int row) -> uint32_t {  // pair of a round's row; ~0u for padding rows
+    const int pi = round * PPR + row / G;
+    return (row < ROWS && pi < npair) ? pairs[p_lo + pi] : 0xffffffffu;
   };
-  uint32_t pk_q = pair_of(0, q_row), pk_o = pair_of(0, o_row), pk_r = pair_of(0, tid);
-  uint4 xq = make_uint4(0, 0, 0, 0), xo = make_uint4(0, 0, 0, 0);
+  uint32_t pk_q[NQ], pk_o[NO], pk_r;
+  uint4 xq[NQ], xo[NO];
   float r_l2 = INFINITY, r_w = 0.f, r_dl = 0.f;
+  auto load_pairs = [&](int round) {
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) pk_q[u] = pair_of(round, q_row0 + u * QRS);
+#pragma unroll
+    for (int u = 0; u < NO; ++u) pk_o[u] = pair_of(round, o_row0 + u * ORS);
+    pk_r = pair_of(round, tid);
+  };
   auto fetch = [&]() {
-    xq = make_uint4(0, 0, 0, 0);
-    xo = make_uint4(0, 0, 0, 0);
-    if (pk_q != 0xffffffffu)
-      xq = *(const uint4*)(q + ((b * dm.L + (pk_q >> 8)) * (long)dm.HQ + hk * G + q_row % G) * D + q_pc * 8);
-    if (pk_o != 0xffffffffu)
-      xo = *(const uint4*)(d_o + ((b * dm.L + (pk_o >> 8)) * (long)dm.HQ + hk * G + o_row % G) * DV + o_pc * 8);
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) {
+      xq[u] = make_uint4(0, 0, 0, 0);
+      if (pk_q[u] != 0xffffffffu)
+        xq[u] = *(const uint4*)(q + ((b * dm.L + (pk_q[u] >> 8)) * (long)dm.HQ + hk * G + (q_row0 + u * QRS) % G) * D + q_pc * 8);
+    }
+#pragma unroll
+    for (int u = 0; u < NO; ++u) {
+      xo[u] = make_uint4(0, 0, 0, 0);
+      if (pk_o[u] != 0xffffffffu)
+        xo[u] = *(const uint4*)(d_o + ((b * dm.L + (pk_o[u] >> 8)) * (long)dm.HQ + hk * G + (o_row0 + u * ORS) % G) * DV + o_pc * 8);
+    }
     r_l2 = INFINITY;  // padding rows: P = 0
     r_w = 0.f;
     r_dl = 0.f;
-    if (tid < 16 && pk_r != 0xffffffffu) {
+    if (pk_r != 0xffffffffu) {
       const long rowi = (b * dm.L + (pk_r >> 8)) * (long)dm.HQ + hk * G + tid % G;
       r_l2 = lse[rowi * dm.K + (pk_r & 255)];
       if (r_l2 == HILS_NEG_INF) r_l2 = INFINITY;
@@ -209,107 +229,94 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
       r_dl = delta[rowi * dm.NW + (pk_r & 255)];
     }
   };
+  // row-major copy + transposed copy (dwords of two neighbouring rows) of one 16-byte piece
+  auto stage_piece = [&](const uint4& x, int row, int pc, int lanes_apart, char* rm, int rowb, char* tr, int feat) {
+    *(uint4*)(rm + row * rowb + pc * 16) = x;
+    uint4 y;
+    y.x = __shfl_xor((int)x.x, lanes_apart, 64);
+    y.y = __shfl_xor((int)x.y, lanes_apart, 64);
+    y.z = __shfl_xor((int)x.z, lanes_apart, 64);
+    y.w = __shfl_xor((int)x.w, lanes_apart, 64);
+    const bool odd = row & 1;  // even rows write features 0..3 of the piece, odd rows 4..7
+    const uint32_t me0 = odd ? x.z : x.x, me1 = odd ? x.w : x.y;
+    const uint32_t ot0 = odd ? y.z : y.x, ot1 = odd ? y.w : y.y;
+    const uint32_t ev0 = odd ? ot0 : me0, od0 = odd ? me0 : ot0;
+    const uint32_t ev1 = odd ? ot1 : me1, od1 = odd ? me1 : ot1;
+    char* dst = tr + ((row >> 4) * feat + pc * 8 + (odd ? 4 : 0)) * CS + ((row & 15) & ~1) * 2;
+    *(uint32_t*)(dst + 0 * CS) = (ev0 & 0xffffu) | (od0 << 16);
+    *(uint32_t*)(dst + 1 * CS) = (ev0 >> 16) | (od0 & 0xffff0000u);
+    *(uint32_t*)(dst + 2 * CS) = (ev1 & 0xffffu) | (od1 << 16);
+    *(uint32_t*)(dst + 3 * CS) = (ev1 >> 16) | (od1 & 0xffff0000u);
+  };
+  load_pairs(0);
   fetch();
-  pk_q = pair_of(1, q_row);
-  pk_o = pair_of(1, o_row);
-  pk_r = pair_of(1, tid);
+  load_pairs(1);
 
-  for (int tile = 0; tile < ntile; ++tile) {
-    __syncthreads();  // the previous tile's staging is no longer read
-    // ---- stage the gathered rows: row-major (A operands) and transposed (B operands)
-    if (q_row < 16) {
-      *(uint4*)(q_rm + q_row * QROW + q_pc * 16) = xq;
-      // partner row's piece: even rows write features 0..3 of the piece, odd rows 4..7
-      uint4 y;
-      y.x = __shfl_xor((int)xq.x, QPP, 64);
-      y.y = __shfl_xor((int)xq.y, QPP, 64);
-      y.z = __shfl_xor((int)xq.z, QPP, 64);
-      y.w = __shfl_xor((int)xq.w, QPP, 64);
-      const bool odd = q_row & 1;
-      const uint32_t me0 = odd ? xq.z : xq.x, me1 = odd ? xq.w : xq.y;
-      const uint32_t ot0 = odd ? y.z : y.x, ot1 = odd ? y.w : y.y;
-      // dword = (even row value, odd row value) of one feature
-      const uint32_t ev0 = odd ? ot0 : me0, od0 = odd ? me0 : ot0;
-      const uint32_t ev1 = odd ? ot1 : me1, od1 = odd ? me1 : ot1;
-      char* dst = q_tr + (q_pc * 8 + (odd ? 4 : 0)) * CS + (q_row & ~1) * 2;
-      *(uint32_t*)(dst + 0 * CS) = (ev0 & 0xffffu) | (od0 << 16);
-      *(uint32_t*)(dst + 1 * CS) = (ev0 >> 16) | (od0 & 0xffff0000u);
-      *(uint32_t*)(dst + 2 * CS) = (ev1 & 0xffffu) | (od1 << 16);
-      *(uint32_t*)(dst + 3 * CS) = (ev1 >> 16) | (od1 & 0xffff0000u);
-    }
-    if (o_row < 16) {
-      *(uint4*)(o_rm + o_row * OROW + o_pc * 16) = xo;
-      uint4 y;
-      y.x = __shfl_xor((int)xo.x, OPP, 64);
-      y.y = __shfl_xor((int)xo.y, OPP, 64);
-      y.z = __shfl_xor((int)xo.z, OPP, 64);
-      y.w = __shfl_xor((int)xo.w, OPP, 64);
-      const bool odd = o_row & 1;
-      const uint32_t me0 = odd ? xo.z : xo.x, me1 = odd ? xo.w : xo.y;
-      const uint32_t ot0 = odd ? y.z : y.x, ot1 = odd ? y.w : y.y;
-      const uint32_t ev0 = odd ? ot0 : me0, od0 = odd ? me0 : ot0;
-      const uint32_t ev1 = odd ? ot1 : me1, od1 = odd ? me1 : ot1;
-      char* dst = o_tr + (o_pc * 8 + (odd ? 4 : 0)) * CS + (o_row & ~1) * 2;
-      *(uint32_t*)(dst + 0 * CS) = (ev0 & 0xffffu) | (od0 << 16);
-      *(uint32_t*)(dst + 1 * CS) = (ev0 >> 16) | (od0 & 0xffff0000u);
-      *(uint32_t*)(dst + 2 * CS) = (ev1 & 0xffffu) | (od1 << 16);
-      *(uint32_t*)(dst + 3 * CS) = (ev1 >> 16) | (od1 & 0xffff0000u);
-    }
-    if (tid < 16) {
+  for (int round = 0; round < nround; ++round) {
+    __syncthreads();  // the previous round's staging is no longer read
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) stage_piece(xq[u], q_row0 + u * QRS, q_pc, QPP, q_rm, QROW, q_tr, D);
+#pragma unroll
+    for (int u = 0; u < NO; ++u) stage_piece(xo[u], o_row0 + u * ORS, o_pc, OPP, o_rm, OROW, o_tr, DV);
+    if (tid < ROWS) {
       row_lse[tid] = r_l2;
       row_w[tid] = r_w;
       row_delta[tid] = r_dl;
     }
-    // next tile's gathers fly during this tile's arithmetic
-    if (tile + 1 < ntile) {
+    // next round's gathers fly during this round's arithmetic
+    if (round + 1 < nround) {
       fetch();
-      pk_q = pair_of(tile + 2, q_row);
-      pk_o = pair_of(tile + 2, o_row);
-      pk_r = pair_of(tile + 2, tid);
+      load_pairs(round + 2);
     }
     __syncthreads();
-    // ---- S and dP for this wavefront's 16 tokens
-    f32x4_t s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+    const int rows_here = ((npair - round * PPR < PPR) ? npair - round * PPR : PPR) * G;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const uint4 a = *(const uint4*)(q_rm + col * QROW + (ks * 32 + j * 8) * 2);
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&kb[ks], s, 0, 0, 0);
-    }
+    for (int sub = 0; sub < NSUB; ++sub) {
+      if (sub * 16 < rows_here) {
+        // ---- S and dP of 16 rows x this wavefront's 16 tokens
+        f32x4_t s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ks = 0; ks < VS; ++ks) {
-      const uint4 a = *(const uint4*)(o_rm + col * OROW + (ks * 32 + j * 8) * 2);
-      dp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&vb[ks], dp, 0, 0, 0);
-    }
-    // accumulator layout: column = token `col`, registers = rows 4j..4j+3
-    bw_s4 a_p, a_ds;
-    {
-      float pw[4], ds[4];
+        for (int ks = 0; ks < KS; ++ks) {
+          const uint4 a = *(const uint4*)(q_rm + (sub * 16 + col) * QROW + (ks * 32 + j * 8) * 2);
+          s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&kb[ks], s, 0, 0, 0);
+        }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int r = 4 * j + i;
-        float pv = __builtin_amdgcn_exp2f(s[i] * c2 - row_lse[r]);
-        if (masked_col) pv = 0.f;
-        pw[i] = row_w[r] * pv;
-        ds[i] = pw[i] * (dp[i] - row_delta[r]);
+        for (int ks = 0; ks < VS; ++ks) {
+          const uint4 a = *(const uint4*)(o_rm + (sub * 16 + col) * OROW + (ks * 32 + j * 8) * 2);
+          dp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&vb[ks], dp, 0, 0, 0);
+        }
+        // accumulator layout: column = token `col`, registers = rows 4j..4j+3
+        bw_s4 a_p, a_ds;
+        {
+          float pw[4], ds[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int r = sub * 16 + 4 * j + i;
+            float pv = __builtin_amdgcn_exp2f(s[i] * c2 - row_lse[r]);
+            if (masked_col) pv = 0.f;
+            pw[i] = row_w[r] * pv;
+            ds[i] = pw[i] * (dp[i] - row_delta[r]);
+          }
+          uint2 x;
+          x.x = pack_bf2(pw[0], pw[1]);
+          x.y = pack_bf2(pw[2], pw[3]);
+          a_p = *(bw_s4*)&x;
+          x.x = pack_bf2(ds[0], ds[1]);
+          x.y = pack_bf2(ds[2], ds[3]);
+          a_ds = *(bw_s4*)&x;
+        }
+        // ---- dK += dS^T Q, dV += (wP)^T dO: contraction over the 16 rows
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+          const uint2 bq = *(const uint2*)(q_tr + (sub * D + t * 16 + col) * CS + j * 8);
+          acc_k[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_ds, *(const bw_s4*)&bq, acc_k[t], 0, 0, 0);
+        }
+#pragma unroll
+        for (int t = 0; t < VT; ++t) {
+          const uint2 bo = *(const uint2*)(o_tr + (sub * DV + t * 16 + col) * CS + j * 8);
+          acc_v[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_p, *(const bw_s4*)&bo, acc_v[t], 0, 0, 0);
+        }
       }
-      uint2 x;
-      x.x = pack_bf2(pw[0], pw[1]);
-      x.y = pack_bf2(pw[2], pw[3]);
-      a_p = *(bw_s4*)&x;
-      x.x = pack_bf2(ds[0], ds[1]);
-      x.y = pack_bf2(ds[2], ds[3]);
-      a_ds = *(bw_s4*)&x;
-    }
-    // ---- dK += dS^T Q, dV += (wP)^T dO: contraction over the 16 rows
-#pragma unroll
-    for (int t = 0; t < DT; ++t) {
-      const uint2 bq = *(const uint2*)(q_tr + (t * 16 + col) * CS + j * 8);
-      acc_k[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_ds, *(const bw_s4*)&bq, acc_k[t], 0, 0, 0);
-    }
-#pragma unroll
-    for (int t = 0; t < VT; ++t) {
-      const uint2 bo = *(const uint2*)(o_tr + (t * 16 + col) * CS + j * 8);
-      acc_v[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_p, *(const bw_s4*)&bo, acc_v[t], 0, 0, 0);
     }
   }
   // accumulators: column = feature t*16 + col, rows = tokens wave*16 + 4j + i
@@ -666,8 +673,12 @@ static int bw_launch_dkdv(int G, dim3 grid, hipStream_t st, const bf16_t* q, con
                           const bf16_t* d_o, const int* offsets, const uint32_t* pairs, float* dk, float* dv,
                           const BwDims& dm) {
 #define BW_CALL(G_)                                                                                 \
-  hipLaunchKernelGGL((bw_dkdv_kernel<D, DV, G_>), grid, dim3(256), 0, st, q, k, v, w, lse, delta, d_o,  \
+  hipLaunchKernelGGL((bw_dkdv_kernel<D, DV, G_>), grid, dim3(256), smem, st, q, k, v, w, lse, delta, d_o, \
                      offsets, pairs, dk, dv, dm)
+  constexpr int DMAX = D > DV ? D : DV;
+  constexpr int NSUB = 256 / DMAX;
+  const size_t smem = (size_t)16 * NSUB * (D * 2 + 16) + (size_t)16 * NSUB * (DV * 2 + 16) +
+                      (size_t)NSUB * (D + DV) * 40 + (size_t)3 * 16 * NSUB * sizeof(float);
   switch (G) {
     case 1: BW_CALL(1); break;
     case 2: BW_CALL(2); break;
