@@ -616,7 +616,7 @@ bool hils_bw_covers(int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S, 
   const int G = HQ / H;
   return S == BW_S && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) &&
          (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) && q_block == 1 && WH == HQ && sm_n == 0.f &&
-         slope == nullptr && Lkv % S == 0 && K <= 256 && L < (1 << 24) && Lkv / S <= 12288;
+         slope == nullptr && Lkv >= S && K <= 256 && L < (1 << 24) && Lkv / S <= 12288;
 }
 
 void hils_ga_pack_launch(const void* a, const void* b, void* ap, void* bp, float* bmax, int B, int Lkv,

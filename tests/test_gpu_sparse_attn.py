@@ -222,3 +222,39 @@ def test_sparse_attn_mfma_path_matches_generic_path(pkg, orc, dev, B, L, HQ, H, 
         assert_close_bf16(o, ref, f"{name} o")
         assert_close_f32(lse / 1.4426950408889634, lse_ref, LSE_TOL, f"{name} lse")
     assert_close_bf16(outs[1][0], outs[0][0].float(), "mfma vs generic", max_abs=1e-2, rel_l2=5e-3)
+
+
+@pytest.mark.parametrize("B,L,HQ,H,D,Dv,K,mask_last", [(1, 1100, 8, 2, 128, 128, 6, 1), (2, 640, 4, 4, 64, 64, 16, 1),
+                                                        (1, 700, 16, 1, 64, 128, 4, 0), (1, 2048, 8, 4, 128, 64, 32, 1)])
+def test_sparse_attn_bwd_mfma_path_matches_generic_path(pkg, dev, B, L, HQ, H, D, Dv, K, mask_last):
+    """The MFMA backward (inverse index + chunk-major dK/dV kernel + query-block-major dQ/dW
+    kernel; workspace given) against the shape-generic backward (workspace NULL), through the
+    C ABI: ragged lengths, partly filled index rows, extra weight columns, many rows per chunk."""
+    from hils_attention_amd.ops import _cabi
+    note(f"sparse_attn bwd mfma-vs-generic B{B} L{L} HQ{HQ} H{H} D{D} Dv{Dv} K{K} mask{mask_last}")
+    q, k, v, w, idx = make_case(B, L, HQ, H, D, Dv, K, 64, seed=31, fill_prob=0.8)
+    gen = torch.Generator().manual_seed(32)
+    do = torch.randn(B, L, HQ, Dv, generator=gen).bfloat16()
+    NW = w.shape[-1]
+    t = [x.to(dev) for x in (q, k, v, w, idx)]
+    o = torch.empty(B, L, HQ, Dv, dtype=torch.bfloat16, device=dev)
+    lse = torch.empty(B, L, HQ, K, dtype=torch.float32, device=dev)
+    scale = 1 / math.sqrt(D)
+    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(o), _cabi.ptr(lse), None, 0,
+               B, L, L, HQ, H, D, Dv, K, NW, HQ, 1, 64, scale, mask_last, 0.0)
+    ws = _cabi.sparse_attn_bwd_workspace(dev, B, L, L, HQ, H, D, Dv, K, HQ, 1, 64, 0.0)
+    assert ws is not None, "this shape must be covered by the MFMA backward"
+    res = []
+    for use_ws in (False, True):
+        dq = torch.empty_like(t[0])
+        dk = torch.zeros(t[1].shape, dtype=torch.float32, device=dev)
+        dv = torch.zeros(t[2].shape, dtype=torch.float32, device=dev)
+        dw = torch.zeros(B, L, HQ, NW, dtype=torch.float32, device=dev)
+        _cabi.call("hils_sparse_attn_bwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(lse), _cabi.ptr(do.to(dev)),
+                   _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), _cabi.ptr(ws) if use_ws else None,
+                   B, L, L, HQ, H, D, Dv, K, NW, HQ, 1, 64, scale, mask_last, 0.0)
+        torch.cuda.synchronize()
+        res.append([x.float().cpu() for x in (dq, dk, dv, dw)])
+    for name, a, b in zip(("dq", "dk", "dv", "dw"), res[1], res[0]):
+        assert_close_bf16(a, b, f"{name} mfma vs generic")
+    assert torch.count_nonzero(res[1][3][..., K:]).item() == 0  # weight columns beyond K get no gradient
