@@ -486,7 +486,7 @@ topk_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
 }
 
 // ---------------------------------------------------------------------------
-// Row-packed variant for 2 <= G <= 4 with one chunk key per KV head: the 16 rows of an MFMA
+// Row-packed variant for G <= 4 with one chunk key per KV head: the 16 rows of an MFMA
 // tile are (16/GMAX queries) x (GMAX query heads), so the max over the heads of a query is
 // a max over accumulator registers of one lane, and a wavefront needs nobody else: one
 // wavefront per workgroup owns 8 consecutive queries of a (batch, KV head), keeps their
@@ -1264,12 +1264,15 @@ extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_s
     HILS_CHECK_LAUNCH("hils_topk_fwd");
     return HILS_OK;
   }
-  if (!per_qhead && G >= 2 && G <= 4 && (D == 64 || D == 128)) {
+  if (!per_qhead && G <= 4 && (D == 64 || D == 128)) {
     const int segw = topk_rows_segw(N);
-    int pool_floats = 8 * (segw + 16);                              // pooled scores of 8 queries
-    if (pool_floats < 8 * 4 * topk / 2) pool_floats = 8 * 4 * topk / 2;  // bf16 score staging
-    const size_t smem = sizeof(float) * ((size_t)pool_floats + 128 + (size_t)2 * 8 * topk);
-    dim3 grid_r((L + 7) / 8, h_kv, B);
+    const int NQ = (G == 1) ? 16 : 8;                                 // queries per wavefront
+    const int GM = (G == 1) ? 1 : (G == 2 ? 2 : 4);
+    int pool_floats = NQ * (segw + 16);                               // pooled scores of NQ queries
+    if (pool_floats < NQ * GM * topk / 2) pool_floats = NQ * GM * topk / 2;  // bf16 score staging
+    pool_floats = (pool_floats + 3) & ~3;
+    const size_t smem = sizeof(float) * ((size_t)pool_floats + 128 + (size_t)2 * NQ * topk);
+    dim3 grid_r((L + NQ - 1) / NQ, h_kv, B);
 #define HILS_TOPK_ROWS(G_, KS_)                                                                     \
   do {                                                                                             \
     if (plain)                                                                                     \
@@ -1284,7 +1287,9 @@ extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_s
                          block_size, window_size, causal, q_offset, sm_scale, segw, pool_floats);  \
   } while (0)
     const bool plain = !bias && !gumbel && !drop_mask && !sel_logits;
-    if (G == 2) {
+    if (G == 1) {
+      if (D == 64) HILS_TOPK_ROWS(1, 2); else HILS_TOPK_ROWS(1, 4);
+    } else if (G == 2) {
       if (D == 64) HILS_TOPK_ROWS(2, 2); else HILS_TOPK_ROWS(2, 4);
     } else {
       if (D == 64) HILS_TOPK_ROWS(4, 2); else HILS_TOPK_ROWS(4, 4);
