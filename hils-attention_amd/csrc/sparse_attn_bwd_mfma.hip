@@ -724,6 +724,25 @@ static int bq_dispatch_g(int G, dim3 grid, size_t smem, hipStream_t st, const bf
   return -1;
 }
 
+// Inverse index of an index tensor (B, L, H, K) with values in [0, nchunk) or < 0: counts,
+// offsets (cells + 1 ints, cells = B*H*nchunk), cursor (scratch) and the pairs (t << 8 | slot)
+// grouped by (b, h, chunk).  Also used by the top-k backward.
+void hils_build_chunk_index(const int32_t* indices, int* counts, int* offsets, int* cursor, uint32_t* pairs,
+                            int B, int L, int H, int K, int nchunk, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  const long cells = (long)B * H * nchunk;
+  {
+    const long n = cells + 1;
+    hipLaunchKernelGGL(bw_fill_int_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, counts, 0, n);
+  }
+  int seg_len = L;
+  while ((long)B * H * ((L + seg_len - 1) / seg_len) < 512 && seg_len > 256) seg_len = (seg_len + 1) / 2;
+  dim3 gs((L + seg_len - 1) / seg_len, H, B);
+  hipLaunchKernelGGL(bw_count_kernel, gs, dim3(1024), (size_t)nchunk * 4, st, indices, counts, L, H, K, nchunk, seg_len);
+  hipLaunchKernelGGL(bw_scan_kernel, dim3(1), dim3(1024), 0, st, counts, offsets, cursor, cells);
+  hipLaunchKernelGGL(bw_scatter_kernel, gs, dim3(1024), (size_t)nchunk * 4, st, indices, cursor, pairs, L, H, K, nchunk, seg_len);
+}
+
 // Whole backward on the MFMA kernels: dq (bf16, written), dw (fp32, written at the valid slots),
 // dk / dv (fp32, accumulated into the caller's buffers).
 int hils_bw_run(const void* q, const void* k, const void* v, const void* weights, const int32_t* indices,
@@ -771,16 +790,7 @@ int hils_bw_run(const void* q, const void* k, const void* v, const void* weights
     if (rc != HILS_OK) return rc;
   }
   // ---- inverse index, then dK, dV
-  {
-    const long n = (long)cells + 1;
-    hipLaunchKernelGGL(bw_fill_int_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, counts, 0, n);
-  }
-  int seg_len = L;
-  while ((long)B * H * ((L + seg_len - 1) / seg_len) < 512 && seg_len > 256) seg_len = (seg_len + 1) / 2;
-  dim3 gs((L + seg_len - 1) / seg_len, H, B);
-  hipLaunchKernelGGL(bw_count_kernel, gs, dim3(1024), (size_t)nchunk * 4, st, indices, counts, L, H, K, nchunk, seg_len);
-  hipLaunchKernelGGL(bw_scan_kernel, dim3(1), dim3(1024), 0, st, counts, offsets, cursor, (long)cells);
-  hipLaunchKernelGGL(bw_scatter_kernel, gs, dim3(1024), (size_t)nchunk * 4, st, indices, cursor, pairs, L, H, K, nchunk, seg_len);
+  hils_build_chunk_index(indices, counts, offsets, cursor, pairs, B, L, H, K, nchunk, stream);
   BwDims dm{L, Lkv, HQ, H, K, NW, nchunk, mask_last, sm_scale};
   dim3 grid(nchunk, H, B);
   int rc = -1;

@@ -1361,17 +1361,128 @@ __global__ void topk_bwd_kernel(const bf16_t* __restrict__ gs, const bf16_t* __r
   }
 }
 
+// ---- backward without atomics (workspace given) ----
+// dq: a thread owns 8 consecutive features of one (query, head): sum over the K slots of
+// grad * chunk key (chunk keys stay in L2).
+__global__ void __launch_bounds__(256)
+topk_bwd_dq_kernel(const bf16_t* __restrict__ gs, const bf16_t* __restrict__ lmks,
+                   const int32_t* __restrict__ indices, bf16_t* __restrict__ dq, long rows_g, int L, int N,
+                   int h_kv, int G, int D, int topk, int per_qhead, float sm_scale) {
+  const int pieces = D / 8;
+  const long item = (long)blockIdx.x * 256 + threadIdx.x;  // (row, g, piece)
+  if (item >= rows_g * pieces) return;
+  const int pc = (int)(item % pieces);
+  const long rg = item / pieces;      // (b*L + t)*h_kv + hk)*G + g
+  const int g = (int)(rg % G);
+  const long row = rg / G;
+  const int hk = (int)(row % h_kv);
+  const long b = row / h_kv / L;
+  const int lmk_h = per_qhead ? h_kv * G : h_kv;
+  const int lh = per_qhead ? hk * G + g : hk;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  for (int k = 0; k < topk; ++k) {
+    const int c = indices[row * topk + k];
+    if (c < 0 || c >= N) continue;
+    const float gv = bf2f(gs[rg * topk + k]) * sm_scale;
+    float f[8];
+    unpack8(*(const uint4*)(lmks + ((b * N + c) * (long)lmk_h + lh) * D + pc * 8), f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = fmaf(gv, f[e], acc[e]);
+  }
+  uint4 o;
+  o.x = pack_bf2(acc[0], acc[1]);
+  o.y = pack_bf2(acc[2], acc[3]);
+  o.z = pack_bf2(acc[4], acc[5]);
+  o.w = pack_bf2(acc[6], acc[7]);
+  *(uint4*)(dq + rg * D + pc * 8) = o;
+}
+
+// dlmk: one workgroup per (batch, chunk-key head, chunk) sums grad * q over the (query, slot)
+// pairs of the chunk from the inverse index; 16-byte pieces across lanes, pairs across lane groups.
+__global__ void __launch_bounds__(256)
+topk_bwd_dlmk_kernel(const bf16_t* __restrict__ gs, const bf16_t* __restrict__ q,
+                     const int* __restrict__ offsets, const uint32_t* __restrict__ pairs,
+                     float* __restrict__ dlmk, int L, int N, int h_kv, int G, int D, int topk,
+                     int per_qhead, float sm_scale) {
+  __shared__ float red[256 * 8];
+  const int c = blockIdx.x, lh = blockIdx.y;  // chunk-key head
+  const long b = blockIdx.z;
+  const int lmk_h = per_qhead ? h_kv * G : h_kv;
+  const int hk = per_qhead ? lh / G : lh;
+  const int g_lo = per_qhead ? lh % G : 0, g_n = per_qhead ? 1 : G;
+  const long cell = (b * h_kv + hk) * (long)N + c;
+  const int p_lo = offsets[cell], p_hi = offsets[cell + 1];
+  const int pieces = D / 8;
+  const int pc = threadIdx.x % pieces, grp = threadIdx.x / pieces, ngrp = 256 / pieces;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  const long n_items = (long)(p_hi - p_lo) * g_n;
+  for (long it = grp; it < n_items; it += ngrp) {
+    const uint32_t pk = pairs[p_lo + it / g_n];
+    const int g = g_lo + (int)(it % g_n);
+    const long rg = (((b * L + (pk >> 8)) * h_kv + hk) * (long)G + g);
+    const float gv = bf2f(gs[rg * topk + (pk & 255)]) * sm_scale;
+    float f[8];
+    unpack8(*(const uint4*)(q + rg * D + pc * 8), f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = fmaf(gv, f[e], acc[e]);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) red[(grp * pieces + pc) * 8 + e] = acc[e];
+  __syncthreads();
+  for (int i = threadIdx.x; i < D; i += 256) {
+    const int p2 = i / 8, e = i % 8;
+    float x = 0.f;
+    for (int g2 = 0; g2 < ngrp; ++g2) x += red[(g2 * pieces + p2) * 8 + e];
+    if (p_hi > p_lo) dlmk[((b * N + c) * (long)lmk_h + lh) * D + i] += x;
+  }
+}
+
+void hils_build_chunk_index(const int32_t* indices, int* counts, int* offsets, int* cursor, uint32_t* pairs,
+                            int B, int L, int H, int K, int nchunk, void* stream);
+
+static size_t topk_bwd_round(size_t n) { return (n + 255) & ~(size_t)255; }
+
+extern "C" size_t hils_topk_bwd_workspace(int B, int L, int N, int h_kv, int G, int D, int topk) {
+  if (D % 8 != 0 || D > 2048 || topk > 256 || N > 12288 || L >= (1 << 24)) return 0;
+  const size_t cells = (size_t)B * h_kv * N;
+  return 3 * topk_bwd_round((cells + 1) * 4) + topk_bwd_round((size_t)B * L * h_kv * topk * 4);
+}
+
 extern "C" int hils_topk_bwd(const void* g_scores, const void* q, const void* lmks,
-                             const int32_t* indices, void* dq, float* dlmk, int B, int L, int N,
-                             int h_kv, int G, int D, int topk, int per_qhead, float sm_scale,
-                             void* stream) {
+                             const int32_t* indices, void* dq, float* dlmk, void* workspace, int B,
+                             int L, int N, int h_kv, int G, int D, int topk, int per_qhead,
+                             float sm_scale, void* stream) {
   HILS_REQUIRE(g_scores && q && lmks && indices && dq && dlmk, "hils_topk_bwd: null pointer");
   HILS_REQUIRE(B > 0 && L > 0 && N > 0 && h_kv > 0 && G > 0 && D > 0 && topk > 0, "hils_topk_bwd: sizes must be positive");
   const long rows = (long)B * L * h_kv;
   HILS_REQUIRE(rows <= 2147483647L, "hils_topk_bwd: grid too large");
+  hipStream_t st = (hipStream_t)stream;
+  if (workspace && hils_topk_bwd_workspace(B, L, N, h_kv, G, D, topk) > 0 && h_kv * G <= 65535 && B <= 65535) {
+    const size_t cells = (size_t)B * h_kv * N;
+    char* ws = (char*)workspace;
+    int* counts = (int*)ws;
+    int* offsets = (int*)(ws + topk_bwd_round((cells + 1) * 4));
+    int* cursor = (int*)(ws + 2 * topk_bwd_round((cells + 1) * 4));
+    uint32_t* pairs = (uint32_t*)(ws + 3 * topk_bwd_round((cells + 1) * 4));
+    const long rows_g = rows * G;
+    const long items = rows_g * (D / 8);
+    hipLaunchKernelGGL(topk_bwd_dq_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st,
+                       (const bf16_t*)g_scores, (const bf16_t*)lmks, indices, (bf16_t*)dq, rows_g, L, N, h_kv,
+                       G, D, topk, per_qhead, sm_scale);
+    hils_build_chunk_index(indices, counts, offsets, cursor, pairs, B, L, h_kv, topk, N, stream);
+    const int lmk_h = per_qhead ? h_kv * G : h_kv;
+    hipLaunchKernelGGL(topk_bwd_dlmk_kernel, dim3(N, lmk_h, B), dim3(256), 0, st, (const bf16_t*)g_scores,
+                       (const bf16_t*)q, offsets, pairs, dlmk, L, N, h_kv, G, D, topk, per_qhead, sm_scale);
+    HILS_CHECK_LAUNCH("hils_topk_bwd");
+    return HILS_OK;
+  }
   const int threads = D >= 128 ? 128 : 64;
   size_t smem = ((size_t)G * topk + topk) * sizeof(float);
-  hipLaunchKernelGGL(topk_bwd_kernel, dim3((unsigned)rows), dim3(threads), smem, (hipStream_t)stream,
+  hipLaunchKernelGGL(topk_bwd_kernel, dim3((unsigned)rows), dim3(threads), smem, st,
                      (const bf16_t*)g_scores, (const bf16_t*)q, (const bf16_t*)lmks, indices,
                      (bf16_t*)dq, dlmk, L, N, h_kv, G, D, topk, per_qhead, sm_scale);
   HILS_CHECK_LAUNCH("hils_topk_bwd");

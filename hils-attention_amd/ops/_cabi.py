@@ -23,7 +23,7 @@ SIGNATURES = {
     "hils_attn_pool_fwd": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
     "hils_attn_pool_bwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
     "hils_topk_fwd": [_P] * 11 + [_I] * 12 + [_F, _P],
-    "hils_topk_bwd": [_P] * 6 + [_I] * 8 + [_F, _P],
+    "hils_topk_bwd": [_P] * 7 + [_I] * 8 + [_F, _P],
     "hils_sparse_attn_fwd": [_P] * 9 + [_I] * 13 + [_F, _I, _F, _P],
     "hils_pack_kv_chunks": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
     "hils_sparse_attn_bwd": [_P] * 13 + [_I] * 12 + [_F, _I, _F, _P],
@@ -54,6 +54,8 @@ def load():
     lib.hils_topk_fwd_workspace.argtypes = [_I] * 5
     lib.hils_sparse_attn_fwd_workspace.restype = ctypes.c_size_t
     lib.hils_sparse_attn_fwd_workspace.argtypes = [_I] * 11 + [_F]
+    lib.hils_topk_bwd_workspace.restype = ctypes.c_size_t
+    lib.hils_topk_bwd_workspace.argtypes = [_I] * 7
     lib.hils_sparse_attn_bwd_workspace.restype = ctypes.c_size_t
     lib.hils_sparse_attn_bwd_workspace.argtypes = [_I] * 11 + [_F]
     for name, argtypes in SIGNATURES.items():
@@ -95,6 +97,14 @@ def topk_fwd_workspace(device, B, L, N, h_kv, G):
 def sparse_attn_fwd_workspace(device, B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n):
     """Scratch tensor for hils_sparse_attn_fwd (None when the shape needs none)."""
     n = load().hils_sparse_attn_fwd_workspace(B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n)
+    if n == 0:
+        return None
+    return torch.empty(n, dtype=torch.uint8, device=device)
+
+
+def topk_bwd_workspace(device, B, L, N, h_kv, G, D, topk):
+    """Scratch tensor for hils_topk_bwd (None when the shape needs none)."""
+    n = load().hils_topk_bwd_workspace(B, L, N, h_kv, G, D, topk)
     if n == 0:
         return None
     return torch.empty(n, dtype=torch.uint8, device=device)

@@ -66,8 +66,9 @@ class SoftmaxTopKMaxPoolingFusedFn(torch.autograd.Function):
         gs = grad_scores.to(q_in.dtype).contiguous()
         dq = torch.empty_like(q_in)
         dlmk = torch.zeros(k_in.shape, dtype=torch.float32, device=k_in.device)
+        ws = _cabi.topk_bwd_workspace(q_in.device, B, L, N, h_kv, G, D, topk)
         _cabi.call("hils_topk_bwd", _cabi.ptr(gs), _cabi.ptr(q_in), _cabi.ptr(k_in),
-                   _cabi.ptr(indices), _cabi.ptr(dq), _cabi.ptr(dlmk), B, L, N, h_kv, G, D, topk,
+                   _cabi.ptr(indices), _cabi.ptr(dq), _cabi.ptr(dlmk), _cabi.ptr(ws), B, L, N, h_kv, G, D, topk,
                    int(per_qhead), scale)
         return (dq, dlmk.to(k_in.dtype)) + (None,) * 12
 

@@ -77,10 +77,13 @@ int hils_topk_fwd(const void* q, const void* lmks, const float* lse_swa, const f
 /* Sparse backward of the score gather.  Replaces the dense scatter + two torch.bmm of
  * SoftmaxTopKMaxPoolingFusedFn.backward (ops/topk_head_softmax.py:1040-1092).
  * g_scores (B,L,h_kv,G,topk) bf16 -> dq (B,L,h_kv,G,D) bf16 (written),
- * dlmk fp32 (B,N,h_kv or h_kv*G,D) (ACCUMULATED with atomics: caller zero-fills). */
+ * dlmk fp32 (B,N,h_kv or h_kv*G,D) (ACCUMULATED: caller zero-fills).
+ * workspace: device scratch of hils_topk_bwd_workspace(...) bytes; with it the chunk-key gradient
+ * is summed chunk by chunk over an inverse index (no atomics); NULL selects the atomic kernel. */
+size_t hils_topk_bwd_workspace(int B, int L, int N, int h_kv, int G, int D, int topk);
 int hils_topk_bwd(const void* g_scores, const void* q, const void* lmks, const int32_t* indices,
-                  void* dq, float* dlmk, int B, int L, int N, int h_kv, int G, int D, int topk,
-                  int per_qhead, float sm_scale, void* stream);
+                  void* dq, float* dlmk, void* workspace, int B, int L, int N, int h_kv, int G, int D,
+                  int topk, int per_qhead, float sm_scale, void* stream);
 
 /* ---- inter-chunk softmax (layer glue) ------------------------------------------ */
 
