@@ -186,6 +186,52 @@ def bench_decode(pkg, dev, steps, warmup):
     return sec, per, roof
 
 
+def bench_train(pkg, dev, iters=3):
+    """Config 5: 345M-shaped training layer, forward + backward (B8 L8192, 16 heads MHA, D64, top-32):
+    mean pool -> top-k scores -> softmax over [scores, lse_swa] (torch autograd) -> sparse attention,
+    gradients to q, k, v through every op."""
+    B, L, HQ, H, D, S, K, W = 8, 8192, 16, 16, 64, 64, 32, 1
+    gen = torch.Generator(device=dev).manual_seed(1005)
+    q = gpu_randn((B, L, HQ, D), gen, dev).requires_grad_()
+    k = gpu_randn((B, L, H, D), gen, dev).requires_grad_()
+    v = gpu_randn((B, L, H, D), gen, dev).requires_grad_()
+    d_o = gpu_randn((B, L, HQ, D), gen, dev)
+    lse_swa = swa_lse_current_chunk(q.detach(), k.detach(), S)
+
+    def fwd():
+        lmk = pkg.chunk_mean_pool(k, S)
+        idx, scores = pkg.online_softmax_topk_head(q, lmk, lse_swa, K, S, W, is_training=True)
+        w = torch.softmax(torch.cat([scores.float(), lse_swa.unsqueeze(-1)], -1), -1).to(q.dtype)
+        return pkg.HiLS_block_M_head(q, k, v, w, idx, block_size=S, is_training=True), idx
+
+    def fwd_bwd():
+        for t in (q, k, v):
+            t.grad = None
+        o, _ = fwd()
+        o.backward(d_o)
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    with torch.no_grad():
+        t_fwd = timed(lambda: fwd())
+        n_sel = int((fwd()[1] >= 0).sum().item())
+    t_all = timed(fwd_bwd)
+    flops_fwd = 4.0 * D * S * (HQ // H) * n_sel
+    return {"workload": "train layer fwd+bwd B8 L8192 h16/16 D64 chunk64 top32 (config 5)",
+            "fwd_ms": t_fwd, "fwd_bwd_ms": t_all, "tokens_per_s_fwd_bwd": B * L / (t_all * 1e-3),
+            "attn_flops_fwd": flops_fwd, "attn_flops_bwd": 2.5 * flops_fwd,
+            "layer_tflops_fwd_bwd": 3.5 * flops_fwd / (t_all * 1e-3) / 1e12}
+
+
 def cpu_baseline(data, n_queries=4096):
     """The CPU oracle on a bounded slice of the prefill workload: n_queries consecutive
     queries around the middle of the sequence (top-k + inter-chunk softmax + sparse attention)."""
@@ -219,6 +265,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-train", action="store_true", help="skip the config-5 forward+backward timing")
     ap.add_argument("--no-prefill", action="store_true", help="profiling aid: decode step only")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: run only a 512 MiB device copy (reference reading for the "
@@ -264,6 +311,8 @@ def main():
                                              "(config 4)"}
         line["decode_kernel_ms"] = dper
         line["roofline_decode"] = droof
+    if not args.no_train:
+        line["train_fwd_bwd"] = bench_train(pkg, dev)
     if cpu is not None:
         line["cpu_baseline"] = cpu
     print(json.dumps(line))
