@@ -63,6 +63,130 @@ logz_fwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
   }
 }
 
+// Matrix-core forward for 64-token chunks.  A workgroup of four wavefronts owns 128/G consecutive
+// queries of one KV head (128 score rows: query x head of the group) and walks the chunks that are
+// remote for its last query.  The chunk's keys pass through LDS once per workgroup (double
+// buffered); each wavefront multiplies them with its 32 rows, computing the TRANSPOSED scores
+// K Q^T so that the 64 tokens of one row lie in 16 registers of 4 lanes: the log-sum-exp is an
+// in-lane reduction plus one row-swap reduction.
+#define LZM_RT 2  // 16-row tiles per wavefront
+template <int D, int G>
+__global__ void __launch_bounds__(256)
+logz_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+              float* __restrict__ log_z, LzDims dm, int n_qt) {
+  constexpr int KS = D / 32;
+  constexpr int QW = 16 * LZM_RT / G;  // queries per wavefront
+  constexpr int QB = 4 * QW;           // queries per workgroup
+  constexpr int PITCH = D * 2 + 16;    // bytes per staged key row
+  constexpr int NP = D / 32;           // 16-byte pieces of a chunk per thread
+  __shared__ __align__(16) unsigned char k_s[2][64 * PITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, j = lane >> 4;
+  const int qt = n_qt - 1 - (int)blockIdx.x;  // longest rows first
+  const int hk = blockIdx.y;
+  const long b = blockIdx.z;
+  const int t0 = qt * QB + wave * QW;
+
+  bf16x8_t qa[LZM_RT][KS];
+  int lim[LZM_RT];
+  long orow[LZM_RT];
+  bool live[LZM_RT];
+#pragma unroll
+  for (int rt = 0; rt < LZM_RT; ++rt) {
+    const int row = rt * 16 + col;
+    const int t = t0 + row / G, g = row % G;
+    live[rt] = t < dm.L;
+    const int tc = live[rt] ? t : dm.L - 1;
+    lim[rt] = live[rt] ? lz_limit(dm, t) : 0;
+    orow[rt] = ((b * dm.L + tc) * (long)dm.HQ + hk * G + g);
+    const bf16_t* qp = q + orow[rt] * D + j * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qa[rt][ks] = *(const bf16x8_t*)(qp + ks * 32);
+  }
+  int t_last = qt * QB + QB - 1;
+  if (t_last > dm.L - 1) t_last = dm.L - 1;
+  const int nc = lz_limit(dm, t_last);  // chunks the workgroup walks
+  const float sc2 = dm.sm_scale * HILS_LOG2E;
+
+  uint4 kr[NP];
+  auto fetch = [&](int c) {
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = tid + 256 * i;
+      const int tok = p / (D / 8), seg = p % (D / 8);
+      kr[i] = *(const uint4*)(k + ((b * dm.L + c * 64 + tok) * (long)dm.H + hk) * D + seg * 8);
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = tid + 256 * i;
+      const int tok = p / (D / 8), seg = p % (D / 8);
+      *(uint4*)(&k_s[buf][tok * PITCH + seg * 16]) = kr[i];
+    }
+  };
+  if (nc > 0) {
+    fetch(0);
+    stash(0);
+  }
+  __syncthreads();
+  float keep[LZM_RT];
+#pragma unroll
+  for (int rt = 0; rt < LZM_RT; ++rt) keep[rt] = HILS_NEG_INF;
+  for (int c = 0; c < nc; ++c) {
+    fetch(c + 1 < nc ? c + 1 : c);
+    const unsigned char* kb = k_s[c & 1];
+    f32x4_t acc[LZM_RT][4];
+#pragma unroll
+    for (int rt = 0; rt < LZM_RT; ++rt)
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) acc[rt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8_t a = *(const bf16x8_t*)(kb + (tt * 16 + col) * PITCH + ks * 64 + j * 16);
+#pragma unroll
+        for (int rt = 0; rt < LZM_RT; ++rt)
+          acc[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qa[rt][ks], acc[rt][tt], 0, 0, 0);
+      }
+#pragma unroll
+    for (int rt = 0; rt < LZM_RT; ++rt) {
+      float x[16];
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[tt * 4 + i] = acc[rt][tt][i] * sc2;
+      if (dm.mask_lmk && j == 3) x[15] = HILS_NEG_INF;  // token 63 = tile 3, lane row 3, register 3
+      float m = x[0];
+#pragma unroll
+      for (int i = 1; i < 16; ++i) m = fmaxf(m, x[i]);
+      m = rows_max(m);
+      float s = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s += __builtin_amdgcn_exp2f(x[i] - m);
+      s = rows_sum(s);
+      const float val = (c < lim[rt]) ? (m + __builtin_amdgcn_logf(s)) * HILS_LN2 : HILS_NEG_INF;
+      if (j == (c & 3)) keep[rt] = val;
+    }
+    if ((c & 3) == 3 || c == nc - 1) {
+      const int cc = (c & ~3) + j;
+#pragma unroll
+      for (int rt = 0; rt < LZM_RT; ++rt)
+        if (live[rt] && cc <= c) log_z[orow[rt] * dm.N + cc] = keep[rt];
+    }
+    stash((c + 1) & 1);
+    __syncthreads();
+  }
+  // chunks past the workgroup's walk are not remote for any of its rows
+  for (int r = 0; r < 16 * LZM_RT; ++r) {
+    const int t = t0 + r / G, g = r % G;
+    if (t >= dm.L) break;
+    float* out = log_z + ((b * dm.L + t) * (long)dm.HQ + hk * G + g) * dm.N;
+    for (int c = nc + lane; c < dm.N; c += 64) out[c] = HILS_NEG_INF;
+  }
+}
+
 // dq[b,t,hq,:] = sum_c sum_j dlz[c] * exp(s_j - lz[c]) * scale * k_j
 __global__ void __launch_bounds__(LZ_THREADS)
 logz_bwd_dq_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
@@ -202,6 +326,29 @@ extern "C" int hils_chunk_logz_fwd(const void* q, const void* k, float* log_z, i
   HILS_REQUIRE(q && k && log_z, "hils_chunk_logz_fwd: null pointer");
   if (int rc = lz_check("hils_chunk_logz_fwd", B, L, HQ, H, D, S)) return rc;
   LzDims dm{L, HQ, H, HQ / H, D, S, window, (L + S - 1) / S, mask_lmk, sm_scale};
+  const int G = HQ / H;
+  if (S == 64 && (D == 64 || D == 128) && (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) &&
+      H <= 65535 && B <= 65535) {
+    const int QB = 4 * 16 * LZM_RT / G;
+    const int n_qt = (L + QB - 1) / QB;
+    const dim3 grid((unsigned)n_qt, (unsigned)H, (unsigned)B);
+#define LZ_LAUNCH(DD, GG)                                                                      \
+  hipLaunchKernelGGL((logz_fwd_mfma<DD, GG>), grid, dim3(256), 0, (hipStream_t)stream,         \
+                     (const bf16_t*)q, (const bf16_t*)k, log_z, dm, n_qt)
+#define LZ_LAUNCH_G(DD)                                                                        \
+  switch (G) {                                                                                 \
+    case 1: LZ_LAUNCH(DD, 1); break;                                                           \
+    case 2: LZ_LAUNCH(DD, 2); break;                                                           \
+    case 4: LZ_LAUNCH(DD, 4); break;                                                           \
+    case 8: LZ_LAUNCH(DD, 8); break;                                                           \
+    default: LZ_LAUNCH(DD, 16); break;                                                         \
+  }
+    if (D == 64) { LZ_LAUNCH_G(64); } else { LZ_LAUNCH_G(128); }
+#undef LZ_LAUNCH_G
+#undef LZ_LAUNCH
+    HILS_CHECK_LAUNCH("hils_chunk_logz_fwd");
+    return HILS_OK;
+  }
   hipLaunchKernelGGL(logz_fwd_simple, dim3((unsigned)((long)B * L * HQ)), dim3(LZ_THREADS),
                      D * sizeof(float), (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k,
                      log_z, dm);

@@ -11,7 +11,9 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("B,L,HQ,H,D,S,W,mask_lmk", [
     (1, 512, 4, 2, 64, 64, 64, False), (2, 300, 4, 4, 64, 32, 16, False),
-    (1, 512, 8, 2, 128, 64, 1, True), (1, 256, 2, 1, 64, 64, 0, False), (1, 100, 2, 2, 64, 64, 8, False)])
+    (1, 512, 8, 2, 128, 64, 1, True), (1, 256, 2, 1, 64, 64, 0, False), (1, 100, 2, 2, 64, 64, 8, False),
+    (1, 1100, 8, 2, 128, 64, 33, True), (2, 700, 16, 1, 64, 64, 1, False), (1, 650, 2, 2, 128, 64, 64, False),
+    (1, 330, 16, 2, 64, 64, 64, True), (1, 200, 3, 1, 64, 64, 16, False)])
 def test_logz_fwd(pkg, orc, dev, B, L, HQ, H, D, S, W, mask_lmk):
     note(f"logz_fwd B{B} L{L} HQ{HQ} H{H} D{D} S{S} W{W} lmk{mask_lmk}")
     torch.manual_seed(42)
