@@ -187,6 +187,321 @@ logz_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
   }
 }
 
+// ---- matrix-core backward -------------------------------------------------------------------
+// Both gradients are a pair of products around the same element-wise step
+//   dS[row, tok] = d_log_z[row, c(tok)] * exp(s[row, tok] - log_z[row, c(tok)]) * sm_scale
+//   dQ = dS K,   dK = dS^T Q.
+// One side of the product is OWNED by a wavefront (32 rows, held in registers as matrix operands,
+// with the fp32 gradient accumulators), the other side STREAMS through LDS in 64-row tiles, stored
+// twice: row-major (operand of the score product) and transposed (operand of the gradient
+// product, whose contraction runs over the streamed rows).  The scores are computed with the
+// owned side as matrix columns, so their accumulator registers are already the left operand of
+// the gradient product.
+#define LZM_PT 136  // bytes per row of the transposed tile: 64 bf16 + 8 pad
+
+// Two adjacent rows of the streamed tile (8 elements each): row-major and element-paired stores.
+template <int PITCH>
+__device__ __forceinline__ void lzm_stash_pair(unsigned char* rm, unsigned char* tr, int row0,
+                                               int seg, const uint4& a, const uint4& b) {
+  *(uint4*)(rm + row0 * PITCH + seg * 16) = a;
+  *(uint4*)(rm + (row0 + 1) * PITCH + seg * 16) = b;
+  const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const uint32_t lo = __builtin_amdgcn_perm(bw[w], aw[w], 0x05040100u);
+    const uint32_t hi = __builtin_amdgcn_perm(bw[w], aw[w], 0x07060302u);
+    *(uint32_t*)(tr + (seg * 8 + 2 * w) * LZM_PT + row0 * 2) = lo;
+    *(uint32_t*)(tr + (seg * 8 + 2 * w + 1) * LZM_PT + row0 * 2) = hi;
+  }
+}
+
+// Gradient product of one wavefront: acc[rt][dt] += P[rt] (16 owned x 64 streamed) * T (64 x D).
+// p[rt][tt] are score-accumulator tiles (lane: owned row = lane & 15, streamed rows 4*(lane>>4)+i
+// of tile tt); two tiles form one 32-deep operand, and the transposed tile is read in the same order.
+template <int D, int NT>
+__device__ __forceinline__ void lzm_grad_product(const unsigned char* tr, const float (&p)[NT][4][4],
+                                                 f32x4_t (&acc)[NT][D / 16], int col, int j) {
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    bf16x8_t a[NT];
+#pragma unroll
+    for (int rt = 0; rt < NT; ++rt) {
+      uint4 u;
+      u.x = pack_bf2(p[rt][2 * h][0], p[rt][2 * h][1]);
+      u.y = pack_bf2(p[rt][2 * h][2], p[rt][2 * h][3]);
+      u.z = pack_bf2(p[rt][2 * h + 1][0], p[rt][2 * h + 1][1]);
+      u.w = pack_bf2(p[rt][2 * h + 1][2], p[rt][2 * h + 1][3]);
+      a[rt] = *(const bf16x8_t*)&u;
+    }
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt) {
+      const unsigned char* base = tr + (dt * 16 + col) * LZM_PT + (2 * h * 16 + 4 * j) * 2;
+      const uint2 b0 = *(const uint2*)base, b1 = *(const uint2*)(base + 32);
+      const uint4 bu = {b0.x, b0.y, b1.x, b1.y};
+#pragma unroll
+      for (int rt = 0; rt < NT; ++rt)
+        acc[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt], *(const bf16x8_t*)&bu, acc[rt][dt], 0, 0, 0);
+    }
+  }
+}
+
+// dQ: a wavefront owns 32 score rows (query x head), the chunks' keys stream.
+template <int D, int G>
+__global__ void __launch_bounds__(256)
+logz_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                 const float* __restrict__ log_z, const float* __restrict__ d_log_z,
+                 bf16_t* __restrict__ dq, LzDims dm, int n_qt) {
+  constexpr int KS = D / 32, DT = D / 16;
+  constexpr int QW = 16 * LZM_RT / G, QB = 4 * QW;
+  constexpr int PITCH = D * 2 + 16;
+  constexpr int SEGS = D / 8;            // 16-byte pieces per row
+  constexpr int PPP = 256 / SEGS;        // row pairs per pass of the workgroup
+  constexpr int NPASS = 32 / PPP;
+  __shared__ __align__(16) unsigned char k_s[64 * PITCH];
+  __shared__ __align__(16) unsigned char kt_s[D * LZM_PT];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, j = lane >> 4;
+  const int qt = n_qt - 1 - (int)blockIdx.x;
+  const int hk = blockIdx.y;
+  const long b = blockIdx.z;
+  const int t0 = qt * QB + wave * QW;
+
+  bf16x8_t qa[LZM_RT][KS];
+  int lim[LZM_RT];
+  long orow[LZM_RT];
+#pragma unroll
+  for (int rt = 0; rt < LZM_RT; ++rt) {
+    const int row = rt * 16 + col;
+    const int t = t0 + row / G, g = row % G;
+    const int tc = t < dm.L ? t : dm.L - 1;
+    lim[rt] = t < dm.L ? lz_limit(dm, t) : 0;
+    orow[rt] = ((b * dm.L + tc) * (long)dm.HQ + hk * G + g);
+    const bf16_t* qp = q + orow[rt] * D + j * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qa[rt][ks] = *(const bf16x8_t*)(qp + ks * 32);
+  }
+  int t_last = qt * QB + QB - 1;
+  if (t_last > dm.L - 1) t_last = dm.L - 1;
+  const int nc = lz_limit(dm, t_last);
+  const float sc2 = dm.sm_scale * HILS_LOG2E;
+
+  const int seg = tid % SEGS, rp0 = tid / SEGS;
+  uint4 kr[NPASS][2];
+  auto fetch = [&](int c) {
+#pragma unroll
+    for (int i = 0; i < NPASS; ++i)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int tok = 2 * (rp0 + PPP * i) + h;
+        kr[i][h] = *(const uint4*)(k + ((b * dm.L + c * 64 + tok) * (long)dm.H + hk) * D + seg * 8);
+      }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < NPASS; ++i)
+      lzm_stash_pair<PITCH>(k_s, kt_s, 2 * (rp0 + PPP * i), seg, kr[i][0], kr[i][1]);
+  };
+  f32x4_t acc[LZM_RT][DT];
+#pragma unroll
+  for (int rt = 0; rt < LZM_RT; ++rt)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float lzn[LZM_RT], dln[LZM_RT];
+  auto fetch_z = [&](int c) {
+#pragma unroll
+    for (int rt = 0; rt < LZM_RT; ++rt) {
+      lzn[rt] = log_z[orow[rt] * dm.N + c];
+      dln[rt] = d_log_z[orow[rt] * dm.N + c];
+    }
+  };
+  if (nc > 0) {
+    fetch(0);
+    fetch_z(0);
+    stash();
+  }
+  __syncthreads();
+  for (int c = 0; c < nc; ++c) {
+    float off[LZM_RT], coef[LZM_RT];
+#pragma unroll
+    for (int rt = 0; rt < LZM_RT; ++rt) {
+      const bool ok = c < lim[rt] && lzn[rt] > -1e30f;
+      off[rt] = ok ? lzn[rt] * HILS_LOG2E : 0.f;
+      coef[rt] = ok ? dln[rt] * dm.sm_scale : 0.f;
+    }
+    const int cn = c + 1 < nc ? c + 1 : c;
+    fetch(cn);
+    fetch_z(cn);
+    float p[LZM_RT][4][4];
+    {
+      f32x4_t st[LZM_RT][4];
+#pragma unroll
+      for (int rt = 0; rt < LZM_RT; ++rt)
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) st[rt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8_t a = *(const bf16x8_t*)(k_s + (tt * 16 + col) * PITCH + ks * 64 + j * 16);
+#pragma unroll
+          for (int rt = 0; rt < LZM_RT; ++rt)
+            st[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qa[rt][ks], st[rt][tt], 0, 0, 0);
+        }
+#pragma unroll
+      for (int rt = 0; rt < LZM_RT; ++rt)
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            p[rt][tt][i] = __builtin_amdgcn_exp2f(st[rt][tt][i] * sc2 - off[rt]) * coef[rt];
+    }
+    lzm_grad_product<D, LZM_RT>(kt_s, p, acc, col, j);
+    __syncthreads();
+    stash();
+    __syncthreads();
+  }
+#pragma unroll
+  for (int rt = 0; rt < LZM_RT; ++rt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = rt * 16 + 4 * j + i;
+      const int t = t0 + row / G, g = row % G;
+      if (t >= dm.L) continue;
+      bf16_t* out = dq + ((b * dm.L + t) * (long)dm.HQ + hk * G + g) * D + col;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) out[dt * 16] = f2bf(acc[rt][dt][i]);
+    }
+}
+
+// dK: a workgroup owns two chunks (wavefront: 32 tokens of one chunk), the score rows of the
+// queries behind them stream in tiles of 64 rows (64/G queries x G heads).
+template <int D, int G>
+__global__ void __launch_bounds__(256)
+logz_bwd_dk_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                 const float* __restrict__ log_z, const float* __restrict__ d_log_z,
+                 bf16_t* __restrict__ dk, LzDims dm) {
+  constexpr int KS = D / 32, DT = D / 16;
+  constexpr int QT = 64 / G;  // queries per streamed tile
+  constexpr int PITCH = D * 2 + 16;
+  constexpr int SEGS = D / 8, PPP = 256 / SEGS, NPASS = 32 / PPP;
+  __shared__ __align__(16) unsigned char q_s[64 * PITCH];
+  __shared__ __align__(16) unsigned char qt_s[D * LZM_PT];
+  __shared__ __align__(16) float off_s[2][64];
+  __shared__ __align__(16) float coef_s[2][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, j = lane >> 4;
+  const int c0 = 2 * (int)blockIdx.x, ch = wave >> 1;
+  const int hk = blockIdx.y;
+  const long b = blockIdx.z;
+  const int tok0 = (c0 + ch) * 64 + (wave & 1) * 32;  // first owned token
+
+  bf16x8_t ka[2][KS];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+    int tok = tok0 + tt * 16 + col;
+    if (tok > dm.L - 1) tok = dm.L - 1;  // such tokens get no gradient: every coefficient is 0
+    const bf16_t* kp = k + ((b * dm.L + tok) * (long)dm.H + hk) * D + j * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ka[tt][ks] = *(const bf16x8_t*)(kp + ks * 32);
+  }
+  // first query with chunk c0 fully behind its window, rounded down to a tile
+  int t_first = (c0 + 1) * 64 + dm.W - 1;
+  if (t_first < 0) t_first = 0;
+  const int tile0 = t_first / QT;
+  const int n_tiles = (dm.L + QT - 1) / QT;
+  const float sc2 = dm.sm_scale * HILS_LOG2E;
+
+  const int seg = tid % SEGS, rp0 = tid / SEGS;
+  uint4 qr[NPASS][2];
+  float zo = 0.f, zc = 0.f;
+  auto fetch = [&](int tile) {
+#pragma unroll
+    for (int i = 0; i < NPASS; ++i)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int row = 2 * (rp0 + PPP * i) + h;
+        int t = tile * QT + row / G;
+        if (t > dm.L - 1) t = dm.L - 1;
+        qr[i][h] = *(const uint4*)(q + ((b * dm.L + t) * (long)dm.HQ + hk * G + row % G) * D + seg * 8);
+      }
+    if (tid < 128) {
+      const int row = tid & 63, cc = c0 + (tid >> 6);
+      const int t = tile * QT + row / G;
+      const bool in = t < dm.L && cc < dm.N && cc < lz_limit(dm, t < dm.L ? t : 0);
+      const long zi = ((b * dm.L + (t < dm.L ? t : dm.L - 1)) * (long)dm.HQ + hk * G + row % G) * dm.N +
+                      (cc < dm.N ? cc : dm.N - 1);
+      const float lz = log_z[zi], dl = d_log_z[zi];
+      const bool ok = in && lz > -1e30f;
+      zo = ok ? lz * HILS_LOG2E : 0.f;
+      zc = ok ? dl * dm.sm_scale : 0.f;
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < NPASS; ++i)
+      lzm_stash_pair<PITCH>(q_s, qt_s, 2 * (rp0 + PPP * i), seg, qr[i][0], qr[i][1]);
+    if (tid < 128) {
+      off_s[tid >> 6][tid & 63] = zo;
+      coef_s[tid >> 6][tid & 63] = zc;
+    }
+  };
+  f32x4_t acc[2][DT];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[tt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  if (tile0 < n_tiles) {
+    fetch(tile0);
+    stash();
+  }
+  __syncthreads();
+  for (int tile = tile0; tile < n_tiles; ++tile) {
+    fetch(tile + 1 < n_tiles ? tile + 1 : tile);
+    float p[2][4][4];  // [owned token tile][streamed row tile][row 4j+i]
+    {
+      f32x4_t st[2][4];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) st[tt][rr] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8_t a = *(const bf16x8_t*)(q_s + (rr * 16 + col) * PITCH + ks * 64 + j * 16);
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt)
+            st[tt][rr] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ka[tt][ks], st[tt][rr], 0, 0, 0);
+        }
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const float4 o4 = *(const float4*)&off_s[ch][rr * 16 + 4 * j];
+        const float4 c4 = *(const float4*)&coef_s[ch][rr * 16 + 4 * j];
+        const float o[4] = {o4.x, o4.y, o4.z, o4.w}, cf[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            p[tt][rr][i] = __builtin_amdgcn_exp2f(st[tt][rr][i] * sc2 - o[i]) * cf[i];
+      }
+    }
+    lzm_grad_product<D, 2>(qt_s, p, acc, col, j);
+    __syncthreads();
+    stash();
+    __syncthreads();
+  }
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int tok = tok0 + tt * 16 + 4 * j + i;
+      if (tok >= dm.L) continue;
+      bf16_t* out = dk + ((b * dm.L + tok) * (long)dm.H + hk) * D + col;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) out[dt * 16] = f2bf(acc[tt][dt][i]);
+    }
+}
+
 // dq[b,t,hq,:] = sum_c sum_j dlz[c] * exp(s_j - lz[c]) * scale * k_j
 __global__ void __launch_bounds__(LZ_THREADS)
 logz_bwd_dq_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
@@ -312,6 +627,23 @@ logz_bwd_dk_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
   }
 }
 
+// shapes of the matrix-core kernels: 64-token chunks, head dim 64/128, group size dividing 16
+static bool lz_mfma_covers(int G, int D, int S, int H, int B) {
+  return S == 64 && (D == 64 || D == 128) && (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) &&
+         H <= 65535 && B <= 65535;
+}
+// expands LZ_LAUNCH(D, G) for the covered (D, G)
+#define LZ_DISPATCH_G(DD, G_)                                                                  \
+  switch (G_) {                                                                                \
+    case 1: LZ_LAUNCH(DD, 1); break;                                                           \
+    case 2: LZ_LAUNCH(DD, 2); break;                                                           \
+    case 4: LZ_LAUNCH(DD, 4); break;                                                           \
+    case 8: LZ_LAUNCH(DD, 8); break;                                                           \
+    default: LZ_LAUNCH(DD, 16); break;                                                         \
+  }
+#define LZ_DISPATCH(D_, G_)                                                                    \
+  if ((D_) == 64) { LZ_DISPATCH_G(64, G_) } else { LZ_DISPATCH_G(128, G_) }
+
 static int lz_check(const char* name, int B, int L, int HQ, int H, int D, int S) {
   HILS_REQUIRE(B > 0 && L > 0 && HQ > 0 && H > 0 && D > 0 && S > 0, "%s: sizes must be positive", name);
   HILS_REQUIRE(HQ % H == 0, "%s: HQ (%d) must be a multiple of H (%d)", name, HQ, H);
@@ -327,24 +659,14 @@ extern "C" int hils_chunk_logz_fwd(const void* q, const void* k, float* log_z, i
   if (int rc = lz_check("hils_chunk_logz_fwd", B, L, HQ, H, D, S)) return rc;
   LzDims dm{L, HQ, H, HQ / H, D, S, window, (L + S - 1) / S, mask_lmk, sm_scale};
   const int G = HQ / H;
-  if (S == 64 && (D == 64 || D == 128) && (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) &&
-      H <= 65535 && B <= 65535) {
+  if (lz_mfma_covers(G, D, S, H, B)) {
     const int QB = 4 * 16 * LZM_RT / G;
     const int n_qt = (L + QB - 1) / QB;
     const dim3 grid((unsigned)n_qt, (unsigned)H, (unsigned)B);
 #define LZ_LAUNCH(DD, GG)                                                                      \
   hipLaunchKernelGGL((logz_fwd_mfma<DD, GG>), grid, dim3(256), 0, (hipStream_t)stream,         \
                      (const bf16_t*)q, (const bf16_t*)k, log_z, dm, n_qt)
-#define LZ_LAUNCH_G(DD)                                                                        \
-  switch (G) {                                                                                 \
-    case 1: LZ_LAUNCH(DD, 1); break;                                                           \
-    case 2: LZ_LAUNCH(DD, 2); break;                                                           \
-    case 4: LZ_LAUNCH(DD, 4); break;                                                           \
-    case 8: LZ_LAUNCH(DD, 8); break;                                                           \
-    default: LZ_LAUNCH(DD, 16); break;                                                         \
-  }
-    if (D == 64) { LZ_LAUNCH_G(64); } else { LZ_LAUNCH_G(128); }
-#undef LZ_LAUNCH_G
+    LZ_DISPATCH(D, G);
 #undef LZ_LAUNCH
     HILS_CHECK_LAUNCH("hils_chunk_logz_fwd");
     return HILS_OK;
@@ -363,6 +685,19 @@ extern "C" int hils_chunk_logz_bwd_dq(const void* q, const void* k, const float*
   if (int rc = lz_check("hils_chunk_logz_bwd_dq", B, L, HQ, H, D, S)) return rc;
   HILS_REQUIRE(D <= LZ_THREADS, "hils_chunk_logz_bwd_dq: D (%d) must be <= %d", D, LZ_THREADS);
   LzDims dm{L, HQ, H, HQ / H, D, S, window, (L + S - 1) / S, 0, sm_scale};
+  if (lz_mfma_covers(HQ / H, D, S, H, B)) {
+    const int G = HQ / H;
+    const int QB = 4 * 16 * LZM_RT / G;
+    const int n_qt = (L + QB - 1) / QB;
+    const dim3 grid((unsigned)n_qt, (unsigned)H, (unsigned)B);
+#define LZ_LAUNCH(DD, GG)                                                                      \
+  hipLaunchKernelGGL((logz_bwd_dq_mfma<DD, GG>), grid, dim3(256), 0, (hipStream_t)stream,      \
+                     (const bf16_t*)q, (const bf16_t*)k, log_z, d_log_z, (bf16_t*)dq, dm, n_qt)
+    LZ_DISPATCH(D, G);
+#undef LZ_LAUNCH
+    HILS_CHECK_LAUNCH("hils_chunk_logz_bwd_dq");
+    return HILS_OK;
+  }
   hipLaunchKernelGGL(logz_bwd_dq_simple, dim3((unsigned)((long)B * L * HQ)), dim3(LZ_THREADS),
                      (D + S) * sizeof(float), (hipStream_t)stream, (const bf16_t*)q,
                      (const bf16_t*)k, log_z, d_log_z, (bf16_t*)dq, dm);
@@ -378,6 +713,16 @@ extern "C" int hils_chunk_logz_bwd_dk(const void* q, const void* k, const float*
   const int G = HQ / H;
   HILS_REQUIRE(S * D <= LZ_MAX_ACC * LZ_THREADS, "hils_chunk_logz_bwd_dk: S*D (%d) too large", S * D);
   LzDims dm{L, HQ, H, G, D, S, window, (L + S - 1) / S, 0, sm_scale};
+  if (lz_mfma_covers(G, D, S, H, B)) {
+    const dim3 grid((unsigned)((dm.N + 1) / 2), (unsigned)H, (unsigned)B);
+#define LZ_LAUNCH(DD, GG)                                                                      \
+  hipLaunchKernelGGL((logz_bwd_dk_mfma<DD, GG>), grid, dim3(256), 0, (hipStream_t)stream,      \
+                     (const bf16_t*)q, (const bf16_t*)k, log_z, d_log_z, (bf16_t*)dk, dm)
+    LZ_DISPATCH(D, G);
+#undef LZ_LAUNCH
+    HILS_CHECK_LAUNCH("hils_chunk_logz_bwd_dk");
+    return HILS_OK;
+  }
   size_t smem = ((size_t)S * (D + 1) + (size_t)LZ_TT * G * D + (size_t)LZ_TT * G * S) * sizeof(float);
   HILS_REQUIRE(smem <= 160 * 1024, "hils_chunk_logz_bwd_dk: tile does not fit in LDS");
   HILS_REQUIRE(H <= 65535 && B <= 65535, "hils_chunk_logz_bwd_dk: H/B too large for the grid");

@@ -28,7 +28,9 @@ def test_logz_fwd(pkg, orc, dev, B, L, HQ, H, D, S, W, mask_lmk):
 def test_logz_bwd(pkg, orc, dev):
     note("logz_bwd")
     torch.manual_seed(43)
-    for (B, L, HQ, H, D, S, W) in [(1, 384, 4, 2, 64, 64, 32), (1, 200, 2, 2, 128, 32, 1)]:
+    for (B, L, HQ, H, D, S, W) in [(1, 384, 4, 2, 64, 64, 32), (1, 200, 2, 2, 128, 32, 1),
+                                   (1, 700, 8, 2, 128, 64, 64), (2, 330, 16, 1, 64, 64, 1),
+                                   (1, 450, 2, 2, 128, 64, 17), (1, 300, 3, 1, 64, 64, 8)]:
         q = torch.randn(B, L, HQ, D).bfloat16()
         k = torch.randn(B, L, H, D).bfloat16()
         qd, kd = q.to(dev).requires_grad_(), k.to(dev).requires_grad_()
