@@ -134,7 +134,8 @@ def bench_decode(pkg, dev, steps, warmup):
     kc = gpu_randn((B, Lkv, H, D), gen, dev)
     vc = gpu_randn((B, Lkv, H, D), gen, dev)
     lmk = pkg.chunk_mean_pool(kc, S)  # precomputed pooled keys (untimed)
-    lse_swa = (torch.randn(B, 1, HQ, device=dev, generator=gen) * 5 + 10).bfloat16()
+    # fp32, as the sliding-window attention kernel hands its log-sum-exp over
+    lse_swa = torch.randn(B, 1, HQ, device=dev, generator=gen) * 5 + 10
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
     acc = {"topk": 0.0, "glue": 0.0, "attn": 0.0, "n": 0}
 

@@ -172,6 +172,8 @@ static int de_pick_nsplit(int B, int L, int H, int K) {
       cus = v;
   }
   const long rows = (long)B * L * H;
+  // whole waves of one 16-wavefront workgroup per compute unit: no split, no partial sums
+  if (K >= 16 && rows >= cus && (rows % cus == 0 || rows >= 8L * cus)) return 1;
   int nsplit = 1;
   // aim for >= 4 workgroups per CU, at least one slot per wavefront
   while (rows * nsplit < 4L * cus && (K + nsplit * 2 - 1) / (nsplit * 2) >= DE_WAVES / 2 && nsplit < 16) nsplit *= 2;

@@ -20,8 +20,8 @@ struct DrDims {
   float sm_scale;
 };
 
-template <int D, int GMAX>
-__global__ void __launch_bounds__(DR_THREADS, DR_MINW)
+template <int D, int GMAX, int NWAVE>
+__global__ void __launch_bounds__(NWAVE * 64, (NWAVE == 4 ? DR_MINW : 1))
 sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                const bf16_t* __restrict__ v, const bf16_t* __restrict__ weights,
                                const int32_t* __restrict__ indices, bf16_t* __restrict__ o,
@@ -55,7 +55,7 @@ sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   const int per_split = (K + dm.nsplit - 1) / dm.nsplit;
   const int s_begin = split * per_split;
   const int s_end = (s_begin + per_split < K) ? s_begin + per_split : K;
-  for (int slot = s_begin + wave; slot < s_end; slot += DR_WAVES) {
+  for (int slot = s_begin + wave; slot < s_end; slot += NWAVE) {
     const int c = indices[(bt * dm.H + hk) * (long)K + slot];
     if (c < 0 || c >= dm.nchunk) continue;
     const long row0 = (b * dm.Lkv + (long)c * DR_S + tsub) * dm.H + hk;
@@ -148,11 +148,11 @@ sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
       }
   }
   __syncthreads();
-  for (int i = tid; i < G * D; i += DR_THREADS) {
+  for (int i = tid; i < G * D; i += NWAVE * 64) {
     const int g = i / D, dv = i - g * D;
     float x = 0.f;
 #pragma unroll
-    for (int w2 = 0; w2 < DR_WAVES; ++w2) x += o_s[((size_t)w2 * G + g) * D + dv];
+    for (int w2 = 0; w2 < NWAVE; ++w2) x += o_s[((size_t)w2 * G + g) * D + dv];
     if (dm.nsplit == 1) o[(bt * dm.HQ + hk * G + g) * (long)D + dv] = f2bf(x);
     else partial[((bt * dm.HQ + hk * G + g) * (long)dm.nsplit + split) * D + dv] = x;
   }
@@ -167,15 +167,22 @@ void hils_sparse_attn_decode_rows(const void* q, const void* k, const void* v, c
   const int G = HQ / H;
   DrDims dm{L, Lkv, HQ, H, G, K, NW, Lkv / DR_S, nsplit, mask_last, sm_scale};
   dim3 grid(nsplit, H, (unsigned)((long)B * L));
-  const size_t smem = (size_t)DR_WAVES * G * D * sizeof(float);
-#define DR_CALL(D_, G_)                                                                         \
-  hipLaunchKernelGGL((sparse_attn_decode_rows_kernel<D_, G_>), grid, dim3(DR_THREADS), smem, st, \
+  // nsplit == 1 with many slots: one workgroup of 16 wavefronts per (query, KV head), no partial sums
+  const int nwave = (nsplit == 1 && K >= 16) ? 16 : DR_WAVES;
+  const size_t smem = (size_t)nwave * G * D * sizeof(float);
+#define DR_CALL_W(D_, G_, W_)                                                                    \
+  hipLaunchKernelGGL((sparse_attn_decode_rows_kernel<D_, G_, W_>), grid, dim3(W_ * 64), smem, st, \
                      (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)weights, \
                      indices, (bf16_t*)o, (float*)workspace, dm)
+#define DR_CALL(D_, G_)                                                                          \
+  do {                                                                                           \
+    if (nwave == 16) DR_CALL_W(D_, G_, 16); else DR_CALL_W(D_, G_, DR_WAVES);                    \
+  } while (0)
   if (D == 64) {
     if (G == 1) DR_CALL(64, 1); else if (G == 2) DR_CALL(64, 2); else DR_CALL(64, 4);
   } else {
     if (G == 1) DR_CALL(128, 1); else if (G == 2) DR_CALL(128, 2); else DR_CALL(128, 4);
   }
+#undef DR_CALL_W
 #undef DR_CALL
 }

@@ -1181,6 +1181,289 @@ topk_select_kernel(const float* __restrict__ raw, const float* __restrict__ lse_
   topk_tail(tail_sh, pooled, lim, rrow, row, N, G, topk, indices, scores);
 }
 
+// ---------------------------------------------------------------------------
+// Few queries, about one (query, KV head) row per compute unit: one workgroup of 16 wavefronts
+// per row does everything.  The row's chunk keys are streamed once with coalesced 16-byte lane
+// loads (two register buffers in flight per wavefront), the raw scaled logits stay in LDS, and
+// LSE, pooling, the 16 per-wavefront selections and their merge follow without leaving the
+// workgroup: no scratch in HBM and no second launch.
+// ---------------------------------------------------------------------------
+#define TOPK_R_THREADS 1024
+#define TOPK_R_WAVES 16
+#define TOPK_R_MAXN 4096
+#define TOPK_R_EPT (TOPK_R_MAXN / TOPK_R_THREADS)
+
+__device__ __forceinline__ float wave_max_f(float x) {
+  x = fmaxf(x, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), 0xB1, 0xF, 0xF, false)));
+  x = fmaxf(x, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), 0x4E, 0xF, 0xF, false)));
+  x = fmaxf(x, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), 0x141, 0xF, 0xF, false)));
+  x = fmaxf(x, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), 0x140, 0xF, 0xF, false)));
+  const int xi = __float_as_int(x);
+  return fmaxf(fmaxf(__int_as_float(__builtin_amdgcn_readlane(xi, 0)), __int_as_float(__builtin_amdgcn_readlane(xi, 16))),
+               fmaxf(__int_as_float(__builtin_amdgcn_readlane(xi, 32)), __int_as_float(__builtin_amdgcn_readlane(xi, 48))));
+}
+__device__ __forceinline__ float wave_sum_f(float x) {
+  x = row_sum<16>(x);
+  const int xi = __float_as_int(x);
+  return (__int_as_float(__builtin_amdgcn_readlane(xi, 0)) + __int_as_float(__builtin_amdgcn_readlane(xi, 16))) +
+         (__int_as_float(__builtin_amdgcn_readlane(xi, 32)) + __int_as_float(__builtin_amdgcn_readlane(xi, 48)));
+}
+
+struct TopkRowShared {
+  float cand_s[TOPK_R_WAVES][64];
+  int cand_i[TOPK_R_WAVES][64];
+  float merge_s[TOPK_R_WAVES * TOPK_MAXK];
+  int merge_i[TOPK_R_WAVES * TOPK_MAXK];
+  int ncand[TOPK_R_WAVES];
+  float4 red_m[TOPK_R_WAVES];  // per wavefront, one component per head
+  float4 red_l[TOPK_R_WAVES];
+  int next_group;
+};
+
+template <int D, int GMAX>
+__global__ void __launch_bounds__(TOPK_R_THREADS)
+topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
+                const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
+                bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
+                float* __restrict__ sel_logits_out, int L, int N, int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
+                float sm_scale) {
+  constexpr int LR = D / 8, TPI = 64 / LR;
+  constexpr int GI = 8;          // load instructions per register buffer
+  constexpr int KG = GI * TPI;   // chunk keys per buffer
+  extern __shared__ float dyn[];
+  float* logit_s = dyn;                       // [GMAX][NP] raw scaled logits
+  float* pooled = dyn + (size_t)GMAX * NP;    // [NP]
+  __shared__ TopkRowShared sh;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int piece = lane % LR, tsub = lane / LR;
+  const long row = blockIdx.x;  // (b*L + t)*h_kv + hk
+  const int hk = (int)(row % h_kv);
+  const long bt = row / h_kv;
+  const int t = (int)(bt % L);
+  const long b = bt / L;
+  int lim = causal ? visible_limit(t + q_offset, window_size, block_size) : N;
+  lim = lim < 0 ? 0 : (lim > N ? N : lim);
+  float swa[GMAX];
+#pragma unroll
+  for (int g = 0; g < GMAX; ++g) swa[g] = (g < G) ? lse_swa[row * G + g] : 0.f;
+  if (tid == 0) sh.next_group = 2 * TOPK_R_WAVES;
+  __syncthreads();
+
+  // ---- phase 1: logits of the visible chunks ----
+  {
+    uint4 qp[GMAX];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+      qp[g] = make_uint4(0, 0, 0, 0);
+      if (g < G) qp[g] = *(const uint4*)(q + (row * (long)G + g) * D + piece * 8);
+    }
+    const int ngroups = (lim + KG - 1) / KG;
+    const bf16_t* base = lmks + (b * N * (long)h_kv + hk) * D + piece * 8;
+    const long cstride = (long)h_kv * D;
+    auto fetch = [&](uint4 (&kr)[GI], int grp) {
+#pragma unroll
+      for (int it = 0; it < GI; ++it) {
+        int c = grp * KG + it * TPI + tsub;
+        c = c < N ? c : N - 1;
+        kr[it] = *(const uint4*)(base + c * cstride);
+      }
+    };
+    auto consume = [&](const uint4 (&kr)[GI], int grp) {
+#pragma unroll
+      for (int it = 0; it < GI; ++it) {
+        const int c = grp * KG + it * TPI + tsub;
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g)
+          if (g < G) {
+            const float sdot = row_sum<LR>(dot8_bf16(qp[g], kr[it], 0.f));
+            if (piece == 0 && c < N) logit_s[g * NP + c] = __fmul_rn(sdot, sm_scale);
+          }
+      }
+    };
+    // Groups of KG keys are handed out through a counter in LDS: the wavefronts of a workgroup
+    // are served unevenly by the memory system, a fixed share would wait for the slowest.
+    // The first two groups of every wavefront are fixed (wave, wave + 16), the rest drawn.
+    auto draw = [&]() -> int {
+      int v = 0;
+      if (lane == 0) v = atomicAdd(&sh.next_group, 1);
+      return __builtin_amdgcn_readfirstlane(v);
+    };
+    // drawn group numbers only grow, so the first one past the end ends the wavefront's walk
+    const int last = ngroups - 1;
+    uint4 ka[GI], kb[GI];
+    int ga = wave, gb = wave + TOPK_R_WAVES;
+    if (ngroups > 0) {
+      fetch(ka, ga < last ? ga : last);
+      fetch(kb, gb < last ? gb : last);
+    }
+    while (ga < ngroups) {
+      consume(ka, ga);
+      ga = draw();
+      fetch(ka, ga < last ? ga : last);
+      if (gb >= ngroups) break;
+      consume(kb, gb);
+      gb = draw();
+      fetch(kb, gb < last ? gb : last);
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 2: LSE per head, pooled scores ----
+  static_assert(GMAX == 4, "the cross-wavefront reductions carry four heads per float4");
+  float x[GMAX][TOPK_R_EPT];
+  {
+    float m[GMAX];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+      m[g] = HILS_NEG_INF;
+#pragma unroll
+      for (int e = 0; e < TOPK_R_EPT; ++e) {
+        const int c = tid + e * TOPK_R_THREADS;
+        x[g][e] = (g < G && c < lim) ? logit_s[g * NP + c] : HILS_NEG_INF;
+        m[g] = fmaxf(m[g], x[g][e]);
+      }
+      m[g] = wave_max_f(m[g]);
+    }
+    if (lane == 0) sh.red_m[wave] = make_float4(m[0], m[1], m[2], m[3]);
+  }
+  __syncthreads();
+  float gmax[GMAX];
+  {
+    float4 mm = sh.red_m[0];
+#pragma unroll
+    for (int w = 1; w < TOPK_R_WAVES; ++w) {
+      const float4 r = sh.red_m[w];
+      mm.x = fmaxf(mm.x, r.x); mm.y = fmaxf(mm.y, r.y); mm.z = fmaxf(mm.z, r.z); mm.w = fmaxf(mm.w, r.w);
+    }
+    gmax[0] = mm.x; gmax[1] = mm.y; gmax[2] = mm.z; gmax[3] = mm.w;
+    float l[GMAX];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+      l[g] = 0.f;
+      if (gmax[g] > HILS_NEG_INF) {
+#pragma unroll
+        for (int e = 0; e < TOPK_R_EPT; ++e) l[g] += __expf(x[g][e] - gmax[g]);
+      }
+      l[g] = wave_sum_f(l[g]);
+    }
+    if (lane == 0) sh.red_l[wave] = make_float4(l[0], l[1], l[2], l[3]);
+  }
+  __syncthreads();
+  float tot[GMAX];
+  {
+    float4 ll = sh.red_l[0];
+#pragma unroll
+    for (int w = 1; w < TOPK_R_WAVES; ++w) {
+      const float4 r = sh.red_l[w];
+      ll.x += r.x; ll.y += r.y; ll.z += r.z; ll.w += r.w;
+    }
+    const float lsum[GMAX] = {ll.x, ll.y, ll.z, ll.w};
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+      const float lse_hils = (lsum[g] > 0.f) ? gmax[g] + __logf(lsum[g]) : HILS_NEG_INF;
+      // logaddexp on the hardware exp2/log2 (every thread computes the same value)
+      const float hi = fmaxf(swa[g], lse_hils), lo = fminf(swa[g], lse_hils);
+      tot[g] = (lo == HILS_NEG_INF) ? hi : hi + __logf(1.f + __expf(lo - hi));
+      if (lse_total_out && tid == 0 && g < G) lse_total_out[row * G + g] = tot[g];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < TOPK_R_EPT; ++e) {
+    const int c = tid + e * TOPK_R_THREADS;
+    float best = HILS_NEG_INF;
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g)
+      if (g < G) {
+        const float nrm = (x[g][e] == HILS_NEG_INF) ? HILS_NEG_INF : __fsub_rn(x[g][e], tot[g]);
+        best = fmaxf(best, nrm);
+        if (sel_logits_out && c < N) sel_logits_out[(row * G + g) * (long)N + c] = x[g][e];
+      }
+    if (c < lim) pooled[c] = best;
+  }
+  __syncthreads();
+
+  // ---- phase 3: every wavefront selects from its share, then the shares are merged ----
+  {
+    int per = (lim + TOPK_R_WAVES - 1) / TOPK_R_WAVES;
+    per = (per + 63) & ~63;  // at most TOPK_R_MAXN / 16 = 256 <= TOPK_NSEG
+    const int base = wave * per;
+    int nc = 0;
+    if (base < lim) {
+      const int ns = (lim - base < per) ? lim - base : per;
+      nc = wave_select(pooled + base, ns, base, sh.cand_s[wave], sh.cand_i[wave], 0, topk);
+    }
+    if (lane == 0) sh.ncand[wave] = nc;
+  }
+  __syncthreads();
+  {
+    int off = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < TOPK_R_WAVES; ++w) {
+      const int n = sh.ncand[w];
+      off += (w < wave) ? n : 0;
+      total += n;
+    }
+    const int n = sh.ncand[wave];
+    if (lane < n) {
+      sh.merge_s[off + lane] = sh.cand_s[wave][lane];
+      sh.merge_i[off + lane] = sh.cand_i[wave][lane];
+    }
+    __syncthreads();
+    if (wave == 0) {
+      int nc = 0;
+      for (int p0 = 0; p0 < total; p0 += TOPK_NSEG) {
+        const int ns = (total - p0 < TOPK_NSEG) ? total - p0 : TOPK_NSEG;
+        nc = wave_select(sh.merge_s + p0, ns, 0, sh.cand_s[0], sh.cand_i[0], nc, topk, sh.merge_i + p0);
+      }
+      if (lane == 0) sh.ncand[0] = nc;
+    }
+  }
+  __syncthreads();
+  // ---- phase 4: indices (ascending) and the raw scaled scores of the winners ----
+  const int nc = sh.ncand[0];
+  for (int kk = tid; kk < topk; kk += TOPK_R_THREADS) indices[row * topk + kk] = (kk < nc) ? sh.cand_i[0][kk] : -1;
+  for (int p = tid; p < topk * G; p += TOPK_R_THREADS) {
+    const int g = p / topk, kk = p - g * topk;
+    const float val = (kk < nc) ? logit_s[g * NP + sh.cand_i[0][kk]] : HILS_NEG_INF;
+    scores[(row * G + g) * (long)topk + kk] = f2bf(val);
+  }
+}
+
+// rows = (query, KV head) pairs; the row kernel wants about one row per compute unit
+static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool plain) {
+  return plain && !per_qhead && G <= 4 && (D == 64 || D == 128) && N >= 256 && N <= TOPK_R_MAXN &&
+         rows >= 96 && rows <= 2147483647L;
+}
+
+static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, int32_t* indices,
+                        void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv, int G, int D,
+                        int topk, int block_size, int window_size, int causal, int q_offset,
+                        float sm_scale, hipStream_t st) {
+  const long rows = (long)B * L * h_kv;
+  const int NP = (N + 63) & ~63;
+  const size_t smem = (size_t)5 * NP * sizeof(float);
+#define TOPK_ROW_CALL(D_)                                                                         \
+  do {                                                                                           \
+    auto kern = topk_row_kernel<D_, 4>;                                                          \
+    static size_t reserved = 48 * 1024;                                                          \
+    if (smem > reserved) {                                                                       \
+      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,     \
+                              (int)smem) != hipSuccess) {                                        \
+        hils_set_error("hils_topk_fwd: cannot reserve %zu bytes of LDS", smem);                  \
+        return HILS_ERR_LAUNCH;                                                                  \
+      }                                                                                          \
+      reserved = smem;                                                                           \
+    }                                                                                            \
+    hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(TOPK_R_THREADS), smem, st,               \
+                       (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, indices, (bf16_t*)scores, \
+                       lse_total, sel_logits, L, N, NP, h_kv, G, topk, block_size, window_size,  \
+                       causal, q_offset, sm_scale);                                                    \
+  } while (0)
+  if (D == 64) TOPK_ROW_CALL(64); else TOPK_ROW_CALL(128);
+#undef TOPK_ROW_CALL
+  return HILS_OK;
+}
+
 static bool topk_use_split(int B, int L, int N, int h_kv) {
   static int cus = 0;  // looked up once (keeps the query out of HIP graph capture)
   if (cus == 0) {
@@ -1255,6 +1538,14 @@ extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_s
   HILS_REQUIRE(block_size > 0, "hils_topk_fwd: block_size must be positive");
   HILS_REQUIRE(h_kv <= 65535 && B <= 65535, "hils_topk_fwd: h_kv/B too large for the grid");
   hipStream_t st = (hipStream_t)stream;
+  if (topk_use_split(B, L, N, h_kv) &&
+      topk_use_row((long)B * L * h_kv, N, G, D, per_qhead, !bias && !gumbel && !drop_mask)) {
+    if (int rc2 = topk_fwd_row(q, lmks, lse_swa, indices, scores, lse_total, sel_logits, B, L, N, h_kv, G, D, topk,
+                               block_size, window_size, causal, q_offset, sm_scale, st))
+      return rc2;
+    HILS_CHECK_LAUNCH("hils_topk_fwd");
+    return HILS_OK;
+  }
   if (workspace && (D == 64 || D == 128) && topk_use_split(B, L, N, h_kv) &&
       (long)B * L <= 2147483647L / h_kv) {
     if (int rc2 = topk_fwd_split(q, lmks, lse_swa, bias, gumbel, drop_mask, indices, scores, lse_total,
