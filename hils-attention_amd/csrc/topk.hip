@@ -45,13 +45,21 @@ __device__ __forceinline__ uint32_t lane_kth_largest(uint32_t x, uint32_t lo, ui
   if (diff == 0u) return lo;
   const int top = 31 - __clz((int)diff);
   uint32_t T = (top == 31) ? 0u : (lo & ~((2u << top) - 1u));
-  for (int bit = top; bit >= 0; --bit) {
-    const uint32_t c = T | (1u << bit);
-    const int cnt = __popcll(__ballot(x >= c));
-    if (cnt >= K) {
-      T = c;
-      if (cnt == K) break;
-    }
+  // two bits per step: the three counts are independent, so one step costs about one count's latency
+  int bit = top;
+  for (; bit >= 1; bit -= 2) {
+    const uint32_t c2 = T | (2u << (bit - 1)), c1 = T | (1u << (bit - 1)), c3 = c2 | c1;
+    const int n3 = __popcll(__ballot(x >= c3)), n2 = __popcll(__ballot(x >= c2)),
+              n1 = __popcll(__ballot(x >= c1));
+    int cnt = 0;
+    if (n3 >= K) { T = c3; cnt = n3; }
+    else if (n2 >= K) { T = c2; cnt = n2; }
+    else if (n1 >= K) { T = c1; cnt = n1; }
+    if (cnt == K) return T;
+  }
+  if (bit == 0) {
+    const uint32_t c = T | 1u;
+    if (__popcll(__ballot(x >= c)) >= K) T = c;
   }
   return T;
 }
@@ -69,13 +77,13 @@ __device__ __forceinline__ uint32_t lane_kth_largest(uint32_t x, uint32_t lo, ui
 // must then hold 64 entries) and the exact threshold is searched on those with ballots.
 // If more than 64 keys reach the bound, the K-th largest key is found bit by bit over all
 // slots (per-lane tallies plus one DPP reduction per bit).
-template <bool KEYS = false>
+template <bool KEYS = false, int SLOTS = TOPK_SLOTS>
 __device__ __forceinline__ int wave_select(const float* seg, int ns, int seg_base, float* cand_s,
                                            int* cand_i, int ncand, int K, const int* seg_idx = nullptr,
                                            float* scr_s = nullptr, int* scr_i = nullptr) {
   const int lane = threadIdx.x & 63;
   if (!scr_s) { scr_s = cand_s; scr_i = cand_i; }
-  uint32_t key[TOPK_SLOTS + 1];
+  uint32_t key[SLOTS + 1];
   int cidx = -1;
   key[0] = 0u;
   if (lane < ncand) {
@@ -83,7 +91,7 @@ __device__ __forceinline__ int wave_select(const float* seg, int ns, int seg_bas
     cidx = cand_i[lane];
   }
 #pragma unroll
-  for (int s = 0; s < TOPK_SLOTS; ++s) {
+  for (int s = 0; s < SLOTS; ++s) {
     const int i = s * 64 + lane;
     key[s + 1] = (i < ns) ? (KEYS ? ((const uint32_t*)seg)[i] : score_key(seg[i])) : 0u;
   }
@@ -94,7 +102,7 @@ __device__ __forceinline__ int wave_select(const float* seg, int ns, int seg_bas
   const unsigned long long lt = (1ull << lane) - 1ull;
   uint32_t lm = 0u;  // largest key of this lane
 #pragma unroll
-  for (int s = 0; s <= TOPK_SLOTS; ++s) lm = key[s] > lm ? key[s] : lm;
+  for (int s = 0; s <= SLOTS; ++s) lm = key[s] > lm ? key[s] : lm;
   const bool many = __popcll(__ballot(lm != 0u)) >= K;  // at least K lanes hold a valid key
   uint32_t thr = 1u, hi = 0u;  // every valid key is >= 1
   if (many) {
@@ -106,7 +114,7 @@ __device__ __forceinline__ int wave_select(const float* seg, int ns, int seg_bas
   uint32_t* cs_u = (uint32_t*)scr_s;
   int pos = 0;
 #pragma unroll
-  for (int s = 0; s <= TOPK_SLOTS; ++s) {
+  for (int s = 0; s <= SLOTS; ++s) {
     if (s < nslot) {
       const bool pred = key[s] >= thr;
       const unsigned long long m = __ballot(pred);
@@ -151,7 +159,7 @@ __device__ __forceinline__ int wave_select(const float* seg, int ns, int seg_bas
   {
     uint32_t ka = 0xffffffffu, ko = 0u;
 #pragma unroll
-    for (int s = 0; s <= TOPK_SLOTS; ++s)
+    for (int s = 0; s <= SLOTS; ++s)
       if (key[s] != 0u) { ka &= key[s]; ko |= key[s]; }
     ka = wave_and_u(ka);
     ko = wave_or_u(ko);
@@ -164,7 +172,7 @@ __device__ __forceinline__ int wave_select(const float* seg, int ns, int seg_bas
         const uint32_t c = T | (1u << bit);
         int cl = 0;  // keys of unused slots are 0 and never count
 #pragma unroll
-        for (int s = 0; s <= TOPK_SLOTS; ++s) cl += (key[s] >= c) ? 1 : 0;
+        for (int s = 0; s <= SLOTS; ++s) cl += (key[s] >= c) ? 1 : 0;
         const int cnt = wave_sum_i(cl);
         if (cnt >= K) {
           T = c;
@@ -175,12 +183,12 @@ __device__ __forceinline__ int wave_select(const float* seg, int ns, int seg_bas
   }
   int gl = 0;
 #pragma unroll
-  for (int s = 0; s <= TOPK_SLOTS; ++s) gl += (key[s] > T) ? 1 : 0;
+  for (int s = 0; s <= SLOTS; ++s) gl += (key[s] > T) ? 1 : 0;
   const int gt = wave_sum_i(gl);
   int need = K - gt;  // ties with the threshold still to take, lowest index first
   pos = 0;
 #pragma unroll
-  for (int s = 0; s <= TOPK_SLOTS; ++s) {
+  for (int s = 0; s <= SLOTS; ++s) {
     if (s < nslot) {
       const unsigned long long eq = __ballot(key[s] == T && key[s] != 0u);
       const bool take_eq = (key[s] == T && key[s] != 0u) && (__popcll(eq & lt) < need);
@@ -1308,115 +1316,92 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   }
   __syncthreads();
 
-  // ---- phase 2: LSE per head, pooled scores ----
+  // ---- phase 2: LSE per head.  Wavefront w owns the chunks [w*per, (w+1)*per): the same chunks it
+  // selects from later, so its pooled scores never leave the wavefront before the selection. ----
   static_assert(GMAX == 4, "the cross-wavefront reductions carry four heads per float4");
+  const int per = ((N + TOPK_R_WAVES - 1) / TOPK_R_WAVES + 63) & ~63;  // <= 256 = 64 * TOPK_R_EPT
+  const int cbase = wave * per;
   float x[GMAX][TOPK_R_EPT];
   {
-    float m[GMAX];
+    float m[GMAX], l[GMAX];
 #pragma unroll
     for (int g = 0; g < GMAX; ++g) {
       m[g] = HILS_NEG_INF;
 #pragma unroll
       for (int e = 0; e < TOPK_R_EPT; ++e) {
-        const int c = tid + e * TOPK_R_THREADS;
-        x[g][e] = (g < G && c < lim) ? logit_s[g * NP + c] : HILS_NEG_INF;
+        const int c = cbase + e * 64 + lane;
+        x[g][e] = (g < G && e * 64 < per && c < lim) ? logit_s[g * NP + c] : HILS_NEG_INF;
         m[g] = fmaxf(m[g], x[g][e]);
       }
       m[g] = wave_max_f(m[g]);
-    }
-    if (lane == 0) sh.red_m[wave] = make_float4(m[0], m[1], m[2], m[3]);
-  }
-  __syncthreads();
-  float gmax[GMAX];
-  {
-    float4 mm = sh.red_m[0];
-#pragma unroll
-    for (int w = 1; w < TOPK_R_WAVES; ++w) {
-      const float4 r = sh.red_m[w];
-      mm.x = fmaxf(mm.x, r.x); mm.y = fmaxf(mm.y, r.y); mm.z = fmaxf(mm.z, r.z); mm.w = fmaxf(mm.w, r.w);
-    }
-    gmax[0] = mm.x; gmax[1] = mm.y; gmax[2] = mm.z; gmax[3] = mm.w;
-    float l[GMAX];
-#pragma unroll
-    for (int g = 0; g < GMAX; ++g) {
       l[g] = 0.f;
-      if (gmax[g] > HILS_NEG_INF) {
+      if (m[g] > HILS_NEG_INF) {
 #pragma unroll
-        for (int e = 0; e < TOPK_R_EPT; ++e) l[g] += __expf(x[g][e] - gmax[g]);
+        for (int e = 0; e < TOPK_R_EPT; ++e) l[g] += __expf(x[g][e] - m[g]);
       }
       l[g] = wave_sum_f(l[g]);
     }
-    if (lane == 0) sh.red_l[wave] = make_float4(l[0], l[1], l[2], l[3]);
+    if (lane == 0) {
+      sh.red_m[wave] = make_float4(m[0], m[1], m[2], m[3]);
+      sh.red_l[wave] = make_float4(l[0], l[1], l[2], l[3]);
+    }
   }
   __syncthreads();
   float tot[GMAX];
   {
-    float4 ll = sh.red_l[0];
-#pragma unroll
-    for (int w = 1; w < TOPK_R_WAVES; ++w) {
-      const float4 r = sh.red_l[w];
-      ll.x += r.x; ll.y += r.y; ll.z += r.z; ll.w += r.w;
-    }
-    const float lsum[GMAX] = {ll.x, ll.y, ll.z, ll.w};
+    // every row of 16 lanes combines the 16 (max, sum) pairs: the result is uniform without a broadcast
+    const float4 m4 = sh.red_m[lane & 15], l4 = sh.red_l[lane & 15];
+    const float mw[GMAX] = {m4.x, m4.y, m4.z, m4.w}, lw[GMAX] = {l4.x, l4.y, l4.z, l4.w};
 #pragma unroll
     for (int g = 0; g < GMAX; ++g) {
-      const float lse_hils = (lsum[g] > 0.f) ? gmax[g] + __logf(lsum[g]) : HILS_NEG_INF;
-      // logaddexp on the hardware exp2/log2 (every thread computes the same value)
+      const float mx = row_max16(mw[g]);
+      const float part = (mw[g] > HILS_NEG_INF) ? lw[g] * __expf(mw[g] - mx) : 0.f;
+      const float lsum = row_sum<16>(part);
+      const float lse_hils = (lsum > 0.f) ? mx + __logf(lsum) : HILS_NEG_INF;
+      // logaddexp on the hardware exp2/log2
       const float hi = fmaxf(swa[g], lse_hils), lo = fminf(swa[g], lse_hils);
       tot[g] = (lo == HILS_NEG_INF) ? hi : hi + __logf(1.f + __expf(lo - hi));
       if (lse_total_out && tid == 0 && g < G) lse_total_out[row * G + g] = tot[g];
     }
   }
+  // ---- phase 3: pooled scores of the own chunks, selection among them, winners (padded to topk
+  // entries with -inf) straight into this wavefront's slice of the merge list ----
 #pragma unroll
   for (int e = 0; e < TOPK_R_EPT; ++e) {
-    const int c = tid + e * TOPK_R_THREADS;
+    const int c = cbase + e * 64 + lane;
     float best = HILS_NEG_INF;
 #pragma unroll
     for (int g = 0; g < GMAX; ++g)
       if (g < G) {
         const float nrm = (x[g][e] == HILS_NEG_INF) ? HILS_NEG_INF : __fsub_rn(x[g][e], tot[g]);
         best = fmaxf(best, nrm);
-        if (sel_logits_out && c < N) sel_logits_out[(row * G + g) * (long)N + c] = x[g][e];
+        if (sel_logits_out && e * 64 < per && c < N) sel_logits_out[(row * G + g) * (long)N + c] = x[g][e];
       }
-    if (c < lim) pooled[c] = best;
+    if (e * 64 < per && c < lim) pooled[c] = best;
   }
-  __syncthreads();
-
-  // ---- phase 3: every wavefront selects from its share, then the shares are merged ----
+  __builtin_amdgcn_wave_barrier();
   {
-    int per = (lim + TOPK_R_WAVES - 1) / TOPK_R_WAVES;
-    per = (per + 63) & ~63;  // at most TOPK_R_MAXN / 16 = 256 <= TOPK_NSEG
-    const int base = wave * per;
     int nc = 0;
-    if (base < lim) {
-      const int ns = (lim - base < per) ? lim - base : per;
-      nc = wave_select(pooled + base, ns, base, sh.cand_s[wave], sh.cand_i[wave], 0, topk);
+    if (cbase < lim) {
+      const int ns = (lim - cbase < per) ? lim - cbase : per;
+      nc = wave_select<false, TOPK_R_EPT>(pooled + cbase, ns, cbase, sh.merge_s + wave * topk,
+                                          sh.merge_i + wave * topk, 0, topk, nullptr, sh.cand_s[wave],
+                                          sh.cand_i[wave]);
     }
-    if (lane == 0) sh.ncand[wave] = nc;
+    if (lane >= nc && lane < topk) {
+      sh.merge_s[wave * topk + lane] = HILS_NEG_INF;
+      sh.merge_i[wave * topk + lane] = 0;
+    }
   }
   __syncthreads();
-  {
-    int off = 0, total = 0;
-#pragma unroll
-    for (int w = 0; w < TOPK_R_WAVES; ++w) {
-      const int n = sh.ncand[w];
-      off += (w < wave) ? n : 0;
-      total += n;
+  if (wave == 0) {
+    const int total = TOPK_R_WAVES * topk;
+    int nc = 0;
+    for (int p0 = 0; p0 < total; p0 += TOPK_NSEG) {
+      const int ns = (total - p0 < TOPK_NSEG) ? total - p0 : TOPK_NSEG;
+      nc = wave_select(sh.merge_s + p0, ns, 0, sh.cand_s[0], sh.cand_i[0], nc, topk, sh.merge_i + p0);
     }
-    const int n = sh.ncand[wave];
-    if (lane < n) {
-      sh.merge_s[off + lane] = sh.cand_s[wave][lane];
-      sh.merge_i[off + lane] = sh.cand_i[wave][lane];
-    }
-    __syncthreads();
-    if (wave == 0) {
-      int nc = 0;
-      for (int p0 = 0; p0 < total; p0 += TOPK_NSEG) {
-        const int ns = (total - p0 < TOPK_NSEG) ? total - p0 : TOPK_NSEG;
-        nc = wave_select(sh.merge_s + p0, ns, 0, sh.cand_s[0], sh.cand_i[0], nc, topk, sh.merge_i + p0);
-      }
-      if (lane == 0) sh.ncand[0] = nc;
-    }
+    if (lane == 0) sh.ncand[0] = nc;
   }
   __syncthreads();
   // ---- phase 4: indices (ascending) and the raw scaled scores of the winners ----
