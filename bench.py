@@ -233,6 +233,79 @@ def bench_train(pkg, dev, iters=3):
             "layer_tflops_fwd_bwd": 3.5 * flops_fwd / (t_all * 1e-3) / 1e12}
 
 
+def bench_ops(pkg, dev, iters=3):
+    """The operators of the path that the prefill / decode steps above do not exercise, each at a
+    config-3-shaped size: attention pooling of the chunk keys, exact chunk log-Z (forward and
+    forward+backward), and the older HSA operator."""
+    gen = torch.Generator(device=dev).manual_seed(1006)
+
+    def timed(fn, n=iters):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    out = {}
+    # attention pool: B1, 512 chunks of 64 tokens, 32 heads, D128 (one K tile per head)
+    N, S, H, D = 512, 64, 32, 128
+    mu = gpu_randn((1, N, H, D), gen, dev)
+    kc = gpu_randn((1, N, S, H, D), gen, dev)
+    with torch.no_grad():
+        t = timed(lambda: pkg.chunk_attn_pool_tilelang(mu, kc))
+    out["attn_pool_fwd"] = {"workload": "B1 N512 S64 H32 D128", "us": t * 1e3,
+                            "hbm_gbs": kc.numel() * 2 / (t * 1e-3) / 1e9}
+    mu_g, kc_g = mu.clone().requires_grad_(), kc.clone().requires_grad_()
+
+    def pool_fb():
+        mu_g.grad = None
+        kc_g.grad = None
+        a, b = pkg.chunk_attn_pool_tilelang(mu_g, kc_g)
+        (a.float().sum() + b.sum()).backward()
+
+    out["attn_pool_fwd_bwd"] = {"workload": "B1 N512 S64 H32 D128 (includes the torch glue of the loss)",
+                                "us": timed(pool_fb) * 1e3}
+    del kc, kc_g, mu, mu_g
+    # exact chunk log-Z: B1 L8192 hq32/hkv8 D128, window 64
+    L, HQ, HK = 8192, 32, 8
+    q = gpu_randn((1, L, HQ, D), gen, dev)
+    k = gpu_randn((1, L, HK, D), gen, dev)
+    with torch.no_grad():
+        t = timed(lambda: pkg.exact_chunk_log_z_tl(q, k, chunk_size=64, window_size=64))
+    flops = 2.0 * D * HQ * L * (L / 2)
+    out["log_z_fwd"] = {"workload": "B1 L8192 hq32/hkv8 D128 chunk64 window64", "ms": t,
+                        "mfma_tflops": flops / (t * 1e-3) / 1e12}
+    qg, kg = q.clone().requires_grad_(), k.clone().requires_grad_()
+
+    def lz_fb():
+        qg.grad = None
+        kg.grad = None
+        z = pkg.exact_chunk_log_z_tl(qg, kg, chunk_size=64, window_size=64)
+        torch.where(torch.isfinite(z), z, torch.zeros_like(z)).sum().backward()
+
+    t = timed(lz_fb)
+    out["log_z_fwd_bwd"] = {"workload": "same (includes the torch glue of the loss)", "ms": t,
+                            "mfma_tflops": 5.0 * flops / (t * 1e-3) / 1e12}
+    del q, k, qg, kg
+    # HSA: N2 L4096 hq16/hkv4 D64, 16 chunks per block of 16 queries
+    Nb, L, HQ, HK, D, K, QX = 2, 4096, 16, 4, 64, 16, 16
+    q = gpu_randn((Nb, L, HQ, D), gen, dev)
+    k = gpu_randn((Nb, L, HK, D), gen, dev)
+    v = gpu_randn((Nb, L, HK, D), gen, dev)
+    idx = torch.rand(Nb, L // QX, HK, L // 64, device=dev, generator=gen).topk(K, dim=-1).indices
+    idx = idx.sort(-1).values.to(torch.int32)
+    w = torch.softmax(torch.randn(Nb, L // QX, HK, K, device=dev, generator=gen), -1).bfloat16()
+    with torch.no_grad():
+        t = timed(lambda: pkg.HSA(q, k, v, w, idx, 1.0, 64, 1 / 8.0))
+    out["hsa_fwd"] = {"workload": "N2 L4096 hq16/hkv4 D64 top16 q_block16", "ms": t,
+                      "tflops": 4.0 * D * 64 * HQ * Nb * L * K / (t * 1e-3) / 1e12}
+    return out
+
+
 def cpu_baseline(data, n_queries=4096):
     """The CPU oracle on a bounded slice of the prefill workload: n_queries consecutive
     queries around the middle of the sequence (top-k + inter-chunk softmax + sparse attention)."""
@@ -267,6 +340,7 @@ def main():
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-train", action="store_true", help="skip the config-5 forward+backward timing")
+    ap.add_argument("--no-ops", action="store_true", help="skip the timings of the secondary operators")
     ap.add_argument("--no-prefill", action="store_true", help="profiling aid: decode step only")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: run only a 512 MiB device copy (reference reading for the "
@@ -314,6 +388,8 @@ def main():
         line["roofline_decode"] = droof
     if not args.no_train:
         line["train_fwd_bwd"] = bench_train(pkg, dev)
+    if not args.no_ops:
+        line["ops"] = bench_ops(pkg, dev)
     if cpu is not None:
         line["cpu_baseline"] = cpu
     print(json.dumps(line))

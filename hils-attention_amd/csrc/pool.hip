@@ -1,5 +1,5 @@
 // Chunk-key pooling kernels (HBM-bandwidth-bound reductions over 64-token chunks).
-#include "common.h"
+#include "decode_rows.h"
 #include "../../include/hils_amd.h"
 
 // ---------------------------------------------------------------------------
@@ -174,6 +174,209 @@ attn_pool_fwd_kernel(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__
   }
 }
 
+// Row-streaming variant for 64-token chunks and D = 64 / 128: one wavefront per (chunk, head), the
+// K tile is read once with coalesced 16-byte lane loads (LR = D/8 lanes per token row, 64/LR rows
+// per instruction) and stays in registers; logits by packed bf16 dot2 + DPP row reduction, the
+// softmax over tokens and the weighted sum by in-lane loops plus a reduction over the lanes that
+// hold the same 8 columns of different rows.  The four wavefronts of a workgroup take four
+// neighbouring heads, i.e. neighbouring 2*D-byte pieces of the same token rows.
+template <int LR>
+__device__ __forceinline__ float pool_groups_max(float x) {  // over lanes with the same lane % LR
+  if (LR == 8) x = fmaxf(x, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), 0x128, 0xF, 0xF, false)));
+  return rows_max(x);
+}
+template <int LR>
+__device__ __forceinline__ float pool_groups_sum(float x) {
+  if (LR == 8) x += __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), 0x128, 0xF, 0xF, false));
+  return rows_sum(x);
+}
+
+template <int D>
+__global__ void __launch_bounds__(256)
+attn_pool_fwd_rows(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k,
+                   bf16_t* __restrict__ lmk_k, float* __restrict__ lmk_b, float* __restrict__ p_out,
+                   int H, float sm_scale, int compact, int shared_k) {
+  constexpr int S = 64, LR = D / 8, TPI = 64 / LR, NI = S / TPI;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int piece = lane % LR, tsub = lane / LR;
+  const int hgroups = (H + 3) / 4;  // neighbouring workgroups: neighbouring heads of one chunk
+  const long bn = blockIdx.x / hgroups;
+  const int h = (int)(blockIdx.x % hgroups) * 4 + wave;
+  if (h >= H) return;
+  const int kh = shared_k ? 0 : h;
+  const bf16_t* kp = k + ((bn * S + tsub) * (long)H + kh) * D + piece * 8;
+  const long step = (long)TPI * H * D;
+  uint4 kr[NI];
+#pragma unroll
+  for (int it = 0; it < NI; ++it) kr[it] = *(const uint4*)(kp + it * step);
+  const uint4 mq = *(const uint4*)(mu_q + (bn * H + h) * (long)D + piece * 8);
+  float a[NI];
+  float m = HILS_NEG_INF;
+#pragma unroll
+  for (int it = 0; it < NI; ++it) {
+    a[it] = row_sum<LR>(dot8_bf16(mq, kr[it], 0.f)) * sm_scale;
+    if (it == NI - 1 && tsub == TPI - 1) a[it] = HILS_NEG_INF;  // the chunk's last token is never pooled
+    m = fmaxf(m, a[it]);
+  }
+  m = pool_groups_max<LR>(m);
+  float e_sum = 0.f;
+#pragma unroll
+  for (int it = 0; it < NI; ++it) {
+    a[it] = (a[it] == HILS_NEG_INF) ? 0.f : __expf(a[it] - m);
+    e_sum += a[it];
+  }
+  e_sum = pool_groups_sum<LR>(e_sum);
+  const float inv = e_sum > 0.f ? 1.f / e_sum : 0.f;
+  float ent = 0.f;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int it = 0; it < NI; ++it) {
+    const float pv = a[it] * inv;
+    if (piece == 0) p_out[(bn * S + it * TPI + tsub) * (long)H + h] = pv;
+    if (pv > 0.f) ent += pv * __logf(pv);
+    float f[8];
+    unpack8(kr[it], f);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = fmaf(pv, f[i], acc[i]);
+  }
+  ent = pool_groups_sum<LR>(ent);
+  if (lane == 0) lmk_b[bn * H + h] = -ent;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = compact ? 0.f : pool_groups_sum<LR>(acc[i]);
+  if (tsub == 0) {
+    uint4 w;
+    w.x = pack_bf2(acc[0], acc[1]);
+    w.y = pack_bf2(acc[2], acc[3]);
+    w.z = pack_bf2(acc[4], acc[5]);
+    w.w = pack_bf2(acc[6], acc[7]);
+    *(uint4*)(lmk_k + (bn * H + h) * (long)D + piece * 8) = w;
+  }
+}
+
+// Row-streaming backward, same lane layout.  Per (chunk, head):
+//   dP_s = <g_k, K_s>,  delta = sum_s p_s dP_s,  dl_s = p_s (dP_s - delta - g_b (log p_s + H)),
+//   d_mu = scale * sum_s dl_s K_s,  dK_s = scale * dl_s * mu + p_s * g_k.
+// SHARED: K is head 0's tile for every head; a workgroup owns a chunk, its wavefronts walk the
+// heads h = wave, wave + 4, ... with the dK sum in registers, the four sums meet in LDS (two
+// rounds), head 0 receives the total and heads 1..H-1 are zeroed.
+template <int D, bool SHARED>
+__global__ void __launch_bounds__(256)
+attn_pool_bwd_rows(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k,
+                   const float* __restrict__ p_saved, const float* __restrict__ lmk_b,
+                   const bf16_t* __restrict__ g_k, const float* __restrict__ g_b,
+                   bf16_t* __restrict__ d_mu, bf16_t* __restrict__ d_k, int H, float sm_scale,
+                   int compact) {
+  constexpr int S = 64, LR = D / 8, TPI = 64 / LR, NI = S / TPI;
+  extern __shared__ float xch[];  // SHARED: 2 * NI * 8 * 64 floats
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int piece = lane % LR, tsub = lane / LR;
+  const int hgroups = SHARED ? 1 : (H + 3) / 4;
+  const long bn = blockIdx.x / hgroups;
+  const int h_first = SHARED ? wave : (int)(blockIdx.x % hgroups) * 4 + wave;
+  const int h_step = SHARED ? 4 : H;  // not SHARED: a single head
+  const int kh = SHARED ? 0 : h_first;
+  uint4 kr[NI];
+  if (SHARED || h_first < H) {
+    const bf16_t* kp = k + ((bn * S + tsub) * (long)H + kh) * D + piece * 8;
+    const long step = (long)TPI * H * D;
+#pragma unroll
+    for (int it = 0; it < NI; ++it) kr[it] = *(const uint4*)(kp + it * step);
+  }
+  float dk_acc[SHARED ? NI : 1][8];
+  if (SHARED) {
+#pragma unroll
+    for (int it = 0; it < NI; ++it)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dk_acc[it][i] = 0.f;
+  }
+  for (int h = h_first; h < H; h += h_step) {
+    const uint4 mq = *(const uint4*)(mu_q + (bn * H + h) * (long)D + piece * 8);
+    uint4 gq = make_uint4(0, 0, 0, 0);
+    if (!compact) gq = *(const uint4*)(g_k + (bn * H + h) * (long)D + piece * 8);
+    const float ent = lmk_b[bn * H + h], gb = g_b[bn * H + h];
+    float pv[NI], dl[NI];
+    float part = 0.f;
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      pv[it] = p_saved[(bn * S + it * TPI + tsub) * (long)H + h];
+      dl[it] = row_sum<LR>(dot8_bf16(gq, kr[it], 0.f));
+      part += pv[it] * dl[it];
+    }
+    const float delta = pool_groups_sum<LR>(part);
+    float muf[8], gkf[8];
+    unpack8(mq, muf);
+    unpack8(gq, gkf);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      const float x = pv[it] > 0.f ? pv[it] * ((dl[it] - delta) - gb * (__logf(pv[it]) + ent)) : 0.f;
+      float f[8];
+      unpack8(kr[it], f);
+      float o[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        acc[i] = fmaf(x, f[i], acc[i]);
+        o[i] = sm_scale * x * muf[i] + pv[it] * gkf[i];
+      }
+      if (SHARED) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dk_acc[it][i] += o[i];
+      } else {
+        uint4 w;
+        w.x = pack_bf2(o[0], o[1]); w.y = pack_bf2(o[2], o[3]);
+        w.z = pack_bf2(o[4], o[5]); w.w = pack_bf2(o[6], o[7]);
+        *(uint4*)(d_k + ((bn * S + it * TPI + tsub) * (long)H + h) * D + piece * 8) = w;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = pool_groups_sum<LR>(acc[i]) * sm_scale;
+    if (tsub == 0) {
+      uint4 w;
+      w.x = pack_bf2(acc[0], acc[1]); w.y = pack_bf2(acc[2], acc[3]);
+      w.z = pack_bf2(acc[4], acc[5]); w.w = pack_bf2(acc[6], acc[7]);
+      *(uint4*)(d_mu + (bn * H + h) * (long)D + piece * 8) = w;
+    }
+  }
+  if (SHARED) {
+    // waves 2,3 -> LDS; waves 0,1 add; wave 1 -> LDS; wave 0 adds and writes head 0
+    float* slot = xch + (size_t)(wave & 1) * NI * 8 * 64;
+    auto put = [&]() {
+#pragma unroll
+      for (int it = 0; it < NI; ++it)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) slot[(it * 8 + i) * 64 + lane] = dk_acc[it][i];
+    };
+    auto add = [&]() {
+#pragma unroll
+      for (int it = 0; it < NI; ++it)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dk_acc[it][i] += slot[(it * 8 + i) * 64 + lane];
+    };
+    if (wave >= 2) put();
+    __syncthreads();
+    if (wave < 2) add();
+    __syncthreads();
+    if (wave == 1) { slot = xch; put(); }
+    __syncthreads();
+    if (wave == 0) {
+      add();
+#pragma unroll
+      for (int it = 0; it < NI; ++it) {
+        uint4 w;
+        w.x = pack_bf2(dk_acc[it][0], dk_acc[it][1]); w.y = pack_bf2(dk_acc[it][2], dk_acc[it][3]);
+        w.z = pack_bf2(dk_acc[it][4], dk_acc[it][5]); w.w = pack_bf2(dk_acc[it][6], dk_acc[it][7]);
+        *(uint4*)(d_k + ((bn * S + it * TPI + tsub) * (long)H) * D + piece * 8) = w;
+      }
+    }
+    // heads 1..H-1 of every token row: (H-1)*D/8 zero pieces per row
+    const int zp = (H - 1) * (D / 8);
+    for (int i = threadIdx.x; i < S * zp; i += 256) {
+      const int srow = i / zp, c = i - srow * zp;
+      *(uint4*)(d_k + ((bn * S + srow) * (long)H + 1) * D + (long)c * 8) = make_uint4(0, 0, 0, 0);
+    }
+  }
+}
+
 // Backward.  Block per (bn, h) (or per bn looping over heads when K is shared, so that
 // the per-head dK can be summed into head 0 without atomics).
 __global__ void __launch_bounds__(POOL_THREADS)
@@ -277,6 +480,19 @@ extern "C" int hils_attn_pool_fwd(const void* mu_q, const void* k, void* lmk_k, 
                                   int compact, int shared_k, void* stream) {
   HILS_REQUIRE(mu_q && k && lmk_k && lmk_b && p, "hils_attn_pool_fwd: null pointer");
   if (int rc = pool_check("hils_attn_pool_fwd", BN, S, H, D)) return rc;
+  if (S == 64 && (D == 64 || D == 128) && (long)BN * ((H + 3) / 4) <= 2147483647L) {
+    const dim3 grid((unsigned)((long)BN * ((H + 3) / 4)));
+    if (D == 64)
+      hipLaunchKernelGGL(attn_pool_fwd_rows<64>, grid, dim3(256), 0, (hipStream_t)stream,
+                         (const bf16_t*)mu_q, (const bf16_t*)k, (bf16_t*)lmk_k, lmk_b, p, H, sm_scale,
+                         compact, shared_k);
+    else
+      hipLaunchKernelGGL(attn_pool_fwd_rows<128>, grid, dim3(256), 0, (hipStream_t)stream,
+                         (const bf16_t*)mu_q, (const bf16_t*)k, (bf16_t*)lmk_k, lmk_b, p, H, sm_scale,
+                         compact, shared_k);
+    HILS_CHECK_LAUNCH("hils_attn_pool_fwd");
+    return HILS_OK;
+  }
   size_t smem = ((size_t)S * (D + 1) + D + S + 32) * sizeof(float);
   HILS_REQUIRE(smem <= 160 * 1024, "hils_attn_pool_fwd: S*D (%d x %d) tile does not fit in LDS", S, D);
   if (smem > 64 * 1024)
@@ -295,6 +511,22 @@ extern "C" int hils_attn_pool_bwd(const void* mu_q, const void* k, const float* 
                                   float sm_scale, int compact, int shared_k, void* stream) {
   HILS_REQUIRE(mu_q && k && p && lmk_b && g_k && g_b && d_mu && d_k, "hils_attn_pool_bwd: null pointer");
   if (int rc = pool_check("hils_attn_pool_bwd", BN, S, H, D)) return rc;
+  if (S == 64 && (D == 64 || D == 128) && (long)BN * ((H + 3) / 4) <= 2147483647L) {
+    const dim3 grid((unsigned)((long)BN * (shared_k ? 1 : (H + 3) / 4)));
+    const size_t xch = shared_k ? (size_t)2 * S * D * sizeof(float) : 0;
+#define POOL_BWD_ROWS(D_, SH_)                                                                      \
+  hipLaunchKernelGGL((attn_pool_bwd_rows<D_, SH_>), grid, dim3(256), xch, (hipStream_t)stream,      \
+                     (const bf16_t*)mu_q, (const bf16_t*)k, p, lmk_b, (const bf16_t*)g_k, g_b,      \
+                     (bf16_t*)d_mu, (bf16_t*)d_k, H, sm_scale, compact)
+    if (D == 64) {
+      if (shared_k) POOL_BWD_ROWS(64, true); else POOL_BWD_ROWS(64, false);
+    } else {
+      if (shared_k) POOL_BWD_ROWS(128, true); else POOL_BWD_ROWS(128, false);
+    }
+#undef POOL_BWD_ROWS
+    HILS_CHECK_LAUNCH("hils_attn_pool_bwd");
+    return HILS_OK;
+  }
   size_t smem = ((size_t)S * (D + 1) + 2 * D + 2 * S + 32 + (shared_k ? (size_t)S * D : 0)) * sizeof(float);
   HILS_REQUIRE(smem <= 160 * 1024, "hils_attn_pool_bwd: S*D (%d x %d) tile does not fit in LDS", S, D);
   if (smem > 64 * 1024)
