@@ -17,7 +17,8 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
                               const int32_t* indices, const float* slope, void* o, float* lse,
                               void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ,
                               int H, int D, int Dv, int K, int NW, int S, float sm_scale,
-                              int mask_last, void* stream, int* handled);
+                              int mask_last, int q_block, int WH, float sm_n, void* stream,
+                              int* handled);
 
 bool hils_decode_covers(int L, int HQ, int H, int D, int Dv, int S, int q_block, int WH, float sm_n,
                         const float* slope, const float* lse);
@@ -303,7 +304,7 @@ extern "C" int hils_sparse_attn_fwd(const void* q, const void* k, const void* v,
     int handled = 0;
     if (int rc = hils_sparse_attn_fwd_mfma(q, k, v, weights, indices, slope, o, lse, workspace,
                                            workspace_ready, B, L, Lkv, HQ, H, D, Dv, K, NW, S,
-                                           sm_scale, mask_last, stream, &handled))
+                                           sm_scale, mask_last, q_block, WH, sm_n, stream, &handled))
       return rc;
     if (handled) {
       HILS_CHECK_LAUNCH("hils_sparse_attn_fwd");

@@ -90,6 +90,10 @@ pack_kv_kernel(const bf16_t* __restrict__ k, const bf16_t* __restrict__ v, bf16_
 struct GaDims {
   int L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last;
   float sm_scale;
+  // indices (and weights) are shared by q_block consecutive queries (T % q_block == 0); weights
+  // have WH = HQ or H heads; sm_n * exp(-max) joins every chunk's softmax denominator
+  int q_block, WH;
+  float sm_n;
 };
 
 // Output tiles are accumulated in LDS as 32-bit fixed point: integer LDS atomics run at
@@ -133,6 +137,8 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   const int t0 = blk * dm.T;
   const int K = dm.K;
   const int npair = dm.T * K;
+  const long LB = dm.L / dm.q_block;          // rows of indices / weights per batch element
+  const bool w_per_q = dm.WH == dm.HQ;        // weights per query head (else per KV head)
 
   // ---- prologue.  All global loads of the block set-up are issued before anything waits:
   // the query rows to repack, the selected chunk indices, and the weight rows.
@@ -163,7 +169,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     if (i < npair) {
       const int ql = i / K, slot = i - ql * K;
       preg[e] = (ql << 8) | slot;
-      if (t0 + ql < dm.L) c = indices[((b * dm.L + t0 + ql) * dm.H + hk) * (long)K + slot];
+      if (t0 + ql < dm.L) c = indices[((b * LB + (t0 + ql) / dm.q_block) * dm.H + hk) * (long)K + slot];
     }
     creg[e] = c;
   }
@@ -174,9 +180,10 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   for (int row = tid; row < R; row += GA_THREADS) {
     const int ql = row / G, g = row - ql * G;
     if (t0 + ql < dm.L) {
-      const long e0 = ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G + g) * dm.NW;  // first element
+      const long e0 = ((b * LB + (t0 + ql) / dm.q_block) * (long)dm.WH + (w_per_q ? hk * G + g : hk)) *
+                      dm.NW;  // first element
       const long e_end = e0 + K;
-      const long tot_e = (long)dm.B * dm.L * dm.HQ * dm.NW;
+      const long tot_e = (long)dm.B * LB * dm.WH * dm.NW;
       float a = 0.f;
       for (long eb = e0 & ~1L; eb < e_end; eb += 2 * WDW) {
         uint32_t wd[WDW];
@@ -279,9 +286,10 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   const float sl = SLOPE ? slope[hq] : 0.f;
   // rows of a tile are addressed from the block's first query with 32-bit element offsets
   const bf16_t* qb = qp + ((b * dm.L + t0) * (long)dm.HQ + hk * G) * D;
-  const bf16_t* wb = weights + ((b * dm.L + t0) * (long)dm.HQ + hk * G) * dm.NW;
-  const int q_lane = (j * G + g) * 8, w_lane = g * dm.NW;
-  const int q_step = dm.HQ * D, w_step = dm.HQ * dm.NW;  // per query of the block
+  const bf16_t* wb = weights + ((b * LB + t0 / dm.q_block) * (long)dm.WH + (w_per_q ? hk * G : hk)) * dm.NW;
+  const int q_lane = (j * G + g) * 8, w_lane = w_per_q ? g * dm.NW : 0;
+  const int q_step = dm.HQ * D;          // per query of the block
+  const int w_step = dm.WH * dm.NW;      // per group of q_block queries
 
   // ---- visits: a wavefront takes chunks from a shared counter; a visit is all pairs of the
   // block on one chunk, processed as tiles of up to QT pairs.  The tile stream of a wavefront
@@ -348,7 +356,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) bq_n[ks] = *(const uint4*)(qrow + ks * (4 * G * 8));
     w_n = 0;
-    if (j == 0) w_n = wb[(pk_n >> 8) * w_step + w_lane + (pk_n & 255)];
+    if (j == 0) w_n = wb[((pk_n >> 8) / dm.q_block) * w_step + w_lane + (pk_n & 255)];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int rr = 4 * j + i;
@@ -401,6 +409,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
         sum += e;
       }
     sum = rows_sum(sum);
+    if (dm.sm_n != 0.f) sum += dm.sm_n * __builtin_amdgcn_exp2f(-mc);
     if (lse && qs < n && j == 0) {
       const int ql = pk_c >> 8, slot = pk_c & 255;
       lse[((b * dm.L + t0 + ql) * (long)dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
@@ -577,11 +586,13 @@ size_t hils_ga_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int 
   if (H <= 0 || HQ % H != 0) return 0;
   const int G = HQ / H;
   const bool ok = S == GA_S && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) &&
-                  (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) && q_block == 1 && WH == HQ &&
-                  sm_n == 0.f && L >= 64 && Lkv >= S && K >= 1 && K <= 256;
+                  (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) && q_block >= 1 &&
+                  L % q_block == 0 && (WH == HQ || WH == H) && sm_n >= 0.f && L >= 64 && Lkv >= S &&
+                  K >= 1 && K <= 256;
   if (!ok) return 0;
   size_t smem;
-  if (ga_pick_T(L, G, Dv, K, Lkv / S, &smem) == 0) return 0;
+  const int T = ga_pick_T(L, G, Dv, K, Lkv / S, &smem);
+  if (T == 0 || T % q_block != 0) return 0;  // a query block holds whole index-sharing groups
   const int nchunk = Lkv / S;
   return ga_vt_bytes(B, H, nchunk, Dv) + ga_vt_bytes(B, H, nchunk, D) + ga_vmax_bytes(B, H, nchunk) +
          (size_t)B * L * HQ * D * sizeof(bf16_t);  // packed K, packed V, per-chunk max|V|, packed Q
@@ -592,14 +603,15 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
                               const int32_t* indices, const float* slope, void* o, float* lse,
                               void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ,
                               int H, int D, int Dv, int K, int NW, int S, float sm_scale,
-                              int mask_last, void* stream, int* handled) {
+                              int mask_last, int q_block, int WH, float sm_n, void* stream,
+                              int* handled) {
   *handled = 0;
   const int G = HQ / H;
   const int nchunk = Lkv / S;
   hipStream_t st = (hipStream_t)stream;
   size_t smem;
   const int T = ga_pick_T(L, G, Dv, K, nchunk, &smem);
-  if (T == 0 || H > 65535 || B > 65535) return HILS_OK;
+  if (T == 0 || T % q_block != 0 || H > 65535 || B > 65535) return HILS_OK;
   const int nblk = (L + T - 1) / T;
   const long total = (long)nblk * H * B;
   if (total > (1L << 30)) return HILS_OK;
@@ -613,7 +625,7 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
                        (size_t)GA_S * (dmax + 2) * sizeof(bf16_t), st, (const bf16_t*)k,
                        (const bf16_t*)v, kpk, vpk, vmax, Lkv, H, D, Dv, nchunk);
   }
-  GaDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale};
+  GaDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale, q_block, WH, sm_n};
   const long per_xcd = (total + 7) / 8;
   dim3 grid((unsigned)(per_xcd * 8));
   int rc = -1;

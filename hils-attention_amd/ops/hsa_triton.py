@@ -40,8 +40,10 @@ class _attention(torch.autograd.Function):
         idx_in = indices.to(torch.int32).contiguous()
         o = torch.empty_like(q)
         lse = torch.empty((N, L, HQ, K), dtype=torch.float32, device=q.device)
+        ws = _cabi.sparse_attn_fwd_workspace(q.device, N, L, L_kv, HQ, H, D, v.shape[-1], K, H, q_x,
+                                             int(chunk_size), float(sm_n))
         _cabi.call("hils_sparse_attn_fwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
-                   _cabi.ptr(idx_in), None, _cabi.ptr(o), _cabi.ptr(lse), None, 0,
+                   _cabi.ptr(idx_in), None, _cabi.ptr(o), _cabi.ptr(lse), _cabi.ptr(ws), 0,
                    N, L, L_kv, HQ, H, D, v.shape[-1], K, K, H, q_x, int(chunk_size),
                    float(sm_scale), 0, float(sm_n))
         ctx.save_for_backward(q, k, v, w_in, idx_in, lse)

@@ -71,7 +71,8 @@ def test_logz_total_mass_invariant(pkg, orc, dev):
 
 @pytest.mark.parametrize("Z,HQ,H,N_CTX,D,K,S,Q_X,sm_n", [
     (1, 16, 1, 32, 16, 2, 16, 1, 1.0),    # the reference's own test shape (hsa_triton.py:818)
-    (2, 16, 4, 256, 64, 4, 64, 16, 1.0), (2, 16, 1, 256, 64, 4, 64, 1, 0.0), (1, 8, 2, 128, 32, 4, 32, 4, 0.5)])
+    (2, 16, 4, 256, 64, 4, 64, 16, 1.0), (2, 16, 1, 256, 64, 4, 64, 1, 0.0), (1, 8, 2, 128, 32, 4, 32, 4, 0.5),
+    (1, 8, 2, 512, 128, 8, 64, 32, 2.0), (1, 4, 4, 320, 64, 3, 64, 8, 0.25)])
 def test_hsa(pkg, orc, dev, Z, HQ, H, N_CTX, D, K, S, Q_X, sm_n):
     note(f"HSA Z{Z} HQ{HQ} H{H} L{N_CTX} D{D} K{K} S{S} QX{Q_X} sm_n{sm_n}")
     torch.manual_seed(22)
