@@ -1,0 +1,277 @@
+// Sliding-window attention of the local branch: every query attends causally to the keys from
+// the start of the chunk that holds (query - window + 1) up to itself (or from query - window + 1
+// exactly), optionally without the landmark key of every chunk; outputs o and the natural-log LSE.
+//
+// A workgroup of four wavefronts owns 128/G consecutive queries of one KV head (32 score rows per
+// wavefront: query x head of the group, held as matrix B operands).  The keys and values of the
+// window stream through LDS in 64-token tiles: K row-major (A operand of the transposed scores
+// K Q^T), V transposed (B operand of O += P V, whose contraction runs over the tokens).  With the
+// rows as matrix columns a row's 64 scores lie in 16 registers of 4 lanes (in-lane softmax plus
+// one row-swap reduction) and the probabilities are already the A operand of the second product.
+#include "stream_tiles.h"
+#include "../../include/hils_amd.h"
+
+#define SWA_RT 2  // 16-row tiles per wavefront
+
+struct SwaDims {
+  int Lq, Lk, HQ, H, window, chunk, mask_lmk, expand, kv_start, chunk_pow2;
+  float sm_scale;
+};
+
+template <int D, int DV, int G>
+__global__ void __launch_bounds__(256)
+swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+             bf16_t* __restrict__ o, float* __restrict__ lse, SwaDims dm, int n_qt) {
+  constexpr int KS = D / 32, DT = DV / 16;
+  constexpr int QW = 16 * SWA_RT / G, QB = 4 * QW;
+  constexpr int PITCH = D * 2 + 16;
+  constexpr int KSEG = D / 8, KPASS = 64 * KSEG / 256;        // K tile: 16-byte pieces per thread
+  constexpr int VSEG = DV / 8, VPPP = 256 / VSEG, VPASS = 32 / VPPP;  // V tile: row pairs per pass
+  __shared__ __align__(16) unsigned char k_s[64 * PITCH];
+  __shared__ __align__(16) unsigned char vt_s[DV * LZM_PT];
+  __shared__ __align__(16) float bc_s[4][SWA_RT][16];  // per wavefront: per-row factors, transposed read
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, j = lane >> 4;
+  const int qt = n_qt - 1 - (int)blockIdx.x;
+  const int hk = blockIdx.y;
+  const long b = blockIdx.z;
+  const int t0 = qt * QB + wave * QW;
+  const int q_off = dm.kv_start + dm.Lk - dm.Lq;  // absolute position of query 0
+
+  bf16x8_t qa[SWA_RT][KS];
+  int qabs[SWA_RT], cstart[SWA_RT];
+#pragma unroll
+  for (int rt = 0; rt < SWA_RT; ++rt) {
+    const int row = rt * 16 + col;
+    const int t = t0 + row / G, g = row % G;
+    const int tc = t < dm.Lq ? t : dm.Lq - 1;
+    qabs[rt] = t < dm.Lq ? q_off + t : -2147483647;  // dead rows see nothing
+    const int left = q_off + tc - dm.window + 1;
+    cstart[rt] = dm.expand ? floordiv(left, dm.chunk) * dm.chunk : left;
+    const bf16_t* qp = q + ((b * dm.Lq + tc) * (long)dm.HQ + hk * G + g) * D + j * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qa[rt][ks] = *(const bf16x8_t*)(qp + ks * 32);
+  }
+  // key range of the workgroup (raw indices into k / v)
+  int tile_lo, tile_hi;
+  {
+    const int tq0 = qt * QB;
+    int tq1 = tq0 + QB - 1;
+    if (tq1 > dm.Lq - 1) tq1 = dm.Lq - 1;
+    const int left_abs = q_off + tq0 - dm.window + 1;
+    int lo = (dm.expand ? floordiv(left_abs, dm.chunk) * dm.chunk : left_abs) - dm.kv_start;
+    int hi = q_off + tq1 - dm.kv_start + 1;
+    lo = lo < 0 ? 0 : lo;
+    hi = hi > dm.Lk ? dm.Lk : hi;
+    tile_lo = lo / 64;
+    tile_hi = (hi + 63) / 64;  // may be <= tile_lo: nothing visible
+  }
+  const float c2 = dm.sm_scale * HILS_LOG2E;
+
+  uint4 kr[KPASS], vr[VPASS][2];
+  auto fetch = [&](int tile) {
+#pragma unroll
+    for (int i = 0; i < KPASS; ++i) {
+      const int p = tid + 256 * i;
+      const int tok = tile * 64 + p / KSEG, seg = p % KSEG;
+      kr[i] = make_uint4(0, 0, 0, 0);
+      if (tok < dm.Lk) kr[i] = *(const uint4*)(k + ((b * dm.Lk + tok) * (long)dm.H + hk) * D + seg * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < VPASS; ++i)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int tok = tile * 64 + 2 * (tid / VSEG + VPPP * i) + h;
+        vr[i][h] = make_uint4(0, 0, 0, 0);
+        if (tok < dm.Lk) vr[i][h] = *(const uint4*)(v + ((b * dm.Lk + tok) * (long)dm.H + hk) * DV + (tid % VSEG) * 8);
+      }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < KPASS; ++i) {
+      const int p = tid + 256 * i;
+      *(uint4*)(k_s + (p / KSEG) * PITCH + (p % KSEG) * 16) = kr[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VPASS; ++i) {
+      const int row0 = 2 * (tid / VSEG + VPPP * i), seg = tid % VSEG;
+      const uint32_t aw[4] = {vr[i][0].x, vr[i][0].y, vr[i][0].z, vr[i][0].w};
+      const uint32_t bw[4] = {vr[i][1].x, vr[i][1].y, vr[i][1].z, vr[i][1].w};
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        *(uint32_t*)(vt_s + (seg * 8 + 2 * w) * LZM_PT + row0 * 2) = __builtin_amdgcn_perm(bw[w], aw[w], 0x05040100u);
+        *(uint32_t*)(vt_s + (seg * 8 + 2 * w + 1) * LZM_PT + row0 * 2) = __builtin_amdgcn_perm(bw[w], aw[w], 0x07060302u);
+      }
+    }
+  };
+  f32x4_t acc[SWA_RT][DT];
+#pragma unroll
+  for (int rt = 0; rt < SWA_RT; ++rt)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m_run[SWA_RT], l_run[SWA_RT];  // running max (raw score units) and sum, per row (lane & 15)
+#pragma unroll
+  for (int rt = 0; rt < SWA_RT; ++rt) {
+    m_run[rt] = HILS_NEG_INF;
+    l_run[rt] = 0.f;
+  }
+  if (tile_lo < tile_hi) {
+    fetch(tile_lo);
+    stash();
+  }
+  __syncthreads();
+  for (int tile = tile_lo; tile < tile_hi; ++tile) {
+    fetch(tile + 1 < tile_hi ? tile + 1 : tile);
+    float p[SWA_RT][4][4];
+    {
+      f32x4_t st[SWA_RT][4];
+#pragma unroll
+      for (int rt = 0; rt < SWA_RT; ++rt)
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) st[rt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8_t a = *(const bf16x8_t*)(k_s + (tt * 16 + col) * PITCH + ks * 64 + j * 16);
+#pragma unroll
+          for (int rt = 0; rt < SWA_RT; ++rt)
+            st[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qa[rt][ks], st[rt][tt], 0, 0, 0);
+        }
+      // visibility of this lane's 16 tokens: bit tt*4+i; the landmark test does not depend on the row
+      unsigned lmk_ok = 0xffffu;
+      if (dm.mask_lmk) {
+        lmk_ok = 0u;
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int ta = dm.kv_start + tile * 64 + tt * 16 + 4 * j + i + 1;
+            const bool lm = dm.chunk_pow2 ? ((ta & (dm.chunk - 1)) == 0) : (ta % dm.chunk == 0);
+            lmk_ok |= lm ? 0u : (1u << (tt * 4 + i));
+          }
+      }
+      const int tok_abs0 = dm.kv_start + tile * 64 + 4 * j;
+      const int raw_left = dm.Lk - tile * 64 - 4 * j;  // tokens tt*16+i < raw_left exist
+#pragma unroll
+      for (int rt = 0; rt < SWA_RT; ++rt) {
+        float mx = HILS_NEG_INF;
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int ta = tok_abs0 + tt * 16 + i;
+            const bool vis = ta >= cstart[rt] && ta <= qabs[rt] && (tt * 16 + i) < raw_left &&
+                             ((lmk_ok >> (tt * 4 + i)) & 1u);
+            const float sv = vis ? st[rt][tt][i] : HILS_NEG_INF;
+            p[rt][tt][i] = sv;
+            mx = fmaxf(mx, sv);
+          }
+        mx = rows_max(mx);
+        const float m_new = fmaxf(m_run[rt], mx);
+        const bool any = m_new > HILS_NEG_INF;
+        const float corr = any ? __builtin_amdgcn_exp2f((m_run[rt] - m_new) * c2) : 1.f;  // exp2(-inf) = 0
+        const float mc = any ? m_new * c2 : 0.f;
+        float sum = 0.f;
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float e = __builtin_amdgcn_exp2f(p[rt][tt][i] * c2 - mc);  // masked: exp2(-inf) = 0
+            p[rt][tt][i] = e;
+            sum += e;
+          }
+        sum = rows_sum(sum);
+        l_run[rt] = l_run[rt] * corr + sum;
+        m_run[rt] = m_new;
+        if (j == 0) bc_s[wave][rt][col] = corr;
+      }
+    }
+    // rescale the output accumulators: their rows are 4j+i, the factors live per lane & 15
+#pragma unroll
+    for (int rt = 0; rt < SWA_RT; ++rt) {
+      const float4 c4 = *(const float4*)&bc_s[wave][rt][4 * j];
+      const float cf[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[rt][dt][i] *= cf[i];
+    }
+    lzm_grad_product<DV, SWA_RT>(vt_s, p, acc, col, j);
+    __syncthreads();
+    stash();
+    __syncthreads();
+  }
+  // ---- finalize: o = acc / l, lse = ln(l) + max * scale ----
+#pragma unroll
+  for (int rt = 0; rt < SWA_RT; ++rt) {
+    const float inv = l_run[rt] > 0.f ? 1.f / l_run[rt] : 0.f;
+    if (j == 0) bc_s[wave][rt][col] = inv;
+    const int row = rt * 16 + col;
+    const int t = t0 + row / G, g = row % G;
+    if (j == 0 && t < dm.Lq)
+      lse[(b * dm.Lq + t) * (long)dm.HQ + hk * G + g] =
+          l_run[rt] > 0.f ? (m_run[rt] * c2 + __builtin_amdgcn_logf(l_run[rt])) * HILS_LN2 : HILS_NEG_INF;
+  }
+#pragma unroll
+  for (int rt = 0; rt < SWA_RT; ++rt) {
+    const float4 c4 = *(const float4*)&bc_s[wave][rt][4 * j];
+    const float cf[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = rt * 16 + 4 * j + i;
+      const int t = t0 + row / G, g = row % G;
+      if (t >= dm.Lq) continue;
+      bf16_t* out = o + ((b * dm.Lq + t) * (long)dm.HQ + hk * G + g) * DV + col;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) out[dt * 16] = f2bf(acc[rt][dt][i] * cf[i]);
+    }
+  }
+}
+
+template <int D, int DV>
+static void swa_launch_g(int G, dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* k,
+                         const bf16_t* v, bf16_t* o, float* lse, const SwaDims& dm, int n_qt) {
+#define SWA_CALL(G_) \
+  hipLaunchKernelGGL((swa_fwd_mfma<D, DV, G_>), grid, dim3(256), 0, st, q, k, v, o, lse, dm, n_qt)
+  switch (G) {
+    case 1: SWA_CALL(1); break;
+    case 2: SWA_CALL(2); break;
+    case 4: SWA_CALL(4); break;
+    case 8: SWA_CALL(8); break;
+    default: SWA_CALL(16); break;
+  }
+#undef SWA_CALL
+}
+
+extern "C" int hils_swa_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B,
+                            int Lq, int Lk, int HQ, int H, int D, int Dv, int window, int chunk,
+                            int mask_lmk, int expand_to_chunk, int kv_start, float sm_scale,
+                            void* stream) {
+  HILS_REQUIRE(q && k && v && o && lse, "hils_swa_fwd: null pointer");
+  HILS_REQUIRE(B > 0 && Lq > 0 && Lk > 0 && HQ > 0 && H > 0, "hils_swa_fwd: sizes must be positive");
+  HILS_REQUIRE(Lq <= Lk, "hils_swa_fwd: Lq (%d) must not exceed Lk (%d)", Lq, Lk);
+  HILS_REQUIRE(HQ % H == 0, "hils_swa_fwd: HQ (%d) must be a multiple of H (%d)", HQ, H);
+  HILS_REQUIRE(window >= 1 && chunk >= 1, "hils_swa_fwd: window and chunk must be positive");
+  HILS_REQUIRE(kv_start >= 0, "hils_swa_fwd: kv_start must not be negative");
+  const int G = HQ / H;
+  HILS_REQUIRE((D == 64 || D == 128) && (Dv == 64 || Dv == 128),
+               "hils_swa_fwd: head dims (%d, %d) must be 64 or 128", D, Dv);
+  HILS_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8 || G == 16,
+               "hils_swa_fwd: group size %d must be 1, 2, 4, 8 or 16", G);
+  HILS_REQUIRE(H <= 65535 && B <= 65535, "hils_swa_fwd: H/B too large for the grid");
+  HILS_REQUIRE((long)kv_start + Lk < 2147483647L / 2, "hils_swa_fwd: positions overflow 32 bits");
+  SwaDims dm{Lq, Lk, HQ, H, window, chunk, mask_lmk, expand_to_chunk, kv_start,
+             (chunk & (chunk - 1)) == 0, sm_scale};
+  const int QB = 4 * 16 * SWA_RT / G;
+  const int n_qt = (Lq + QB - 1) / QB;
+  const dim3 grid((unsigned)n_qt, (unsigned)H, (unsigned)B);
+  hipStream_t st = (hipStream_t)stream;
+  const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k, *vv = (const bf16_t*)v;
+  if (D == 64 && Dv == 64) swa_launch_g<64, 64>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
+  else if (D == 128 && Dv == 128) swa_launch_g<128, 128>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
+  else if (D == 64) swa_launch_g<64, 128>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
+  else swa_launch_g<128, 64>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
+  HILS_CHECK_LAUNCH("hils_swa_fwd");
+  return HILS_OK;
+}

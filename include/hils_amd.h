@@ -164,6 +164,20 @@ int hils_chunk_logz_bwd_dk(const void* q, const void* k, const float* log_z, con
                            void* dk, int B, int L, int HQ, int H, int D, int S, int window,
                            float sm_scale, void* stream);
 
+/* ---- sliding-window attention of the local branch ------------------------------- */
+
+/* Forward.  Replaces flex_attn_fwd (ops/flex_attn_tilelang.py:26-267) behind flex_attn_tl
+ * (:1261-1310).  q (B,Lq,HQ,D), k (B,Lk,H,D), v (B,Lk,H,Dv) bf16, Lq <= Lk; query t sits at the
+ * absolute position kv_start + Lk - Lq + t, key j at kv_start + j.  A query sees the keys from
+ * chunk_start to itself, chunk_start = floor((pos - window + 1) / chunk) * chunk when
+ * expand_to_chunk, else pos - window + 1; with mask_lmk the keys with (pos + 1) % chunk == 0 are
+ * excluded.  Writes o (B,Lq,HQ,Dv) bf16 and lse (B,Lq,HQ) fp32 in natural-log units (the
+ * reference's kernel writes log2 units and converts at :1307-1309); rows that see no key get
+ * o = 0, lse = -inf.  D, Dv in {64,128}; HQ/H in {1,2,4,8,16}. */
+int hils_swa_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B, int Lq,
+                 int Lk, int HQ, int H, int D, int Dv, int window, int chunk, int mask_lmk,
+                 int expand_to_chunk, int kv_start, float sm_scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,7 +24,8 @@ reference repository root):
                              :171-193 (the ``sm_n`` denominator term)
 * ``exact_chunk_log_z``    - models/NaiveBSA/naive_bsa_kernel.py:39-118 and the
                              mask of ops/exact_chunk_log_z_tilelang.py:89-107
-* ``swa``                  - ops/flex_attn_tilelang.py:1355-1386 (mask definition)
+* ``swa``                  - ops/flex_attn_tilelang.py:1355-1386 (mask definition) and
+                             :108-121,155-171 (absolute positions with a cache offset)
 * ``hils_layer_forward``   - models/FlashHiLS/hils_attention.py:536-623 (op order,
                              dtypes of the glue)
 * ``dense_hils_attention`` - models/NaiveBSA/naive_bsa_ref.py:111-187 (dense
@@ -318,26 +319,35 @@ def exact_chunk_log_z(q, k, *, chunk_size: int, window_size: int, sm_scale: Opti
 # the sliding-window branch (only to synthesise a self-consistent lse_swa)
 # ----------------------------------------------------------------------------
 def swa(q, k, v, *, window_size: int, chunk_size: int, mask_lmk: bool = True,
-        sm_scale: Optional[float] = None, q_offset: int = 0):
-    """Causal window whose left edge is expanded to the chunk start; landmark keys
-    masked.  Returns (o fp32 (B,L,hq,Dv), lse fp32 (B,L,hq), natural log)."""
+        sm_scale: Optional[float] = None, q_offset: Optional[int] = None, expand_to_chunk: bool = True,
+        kv_start: int = 0):
+    """Causal window whose left edge is expanded to the chunk start (``expand_to_chunk``);
+    landmark keys masked (``mask_lmk``).  Query t sits at the absolute position
+    kv_start + q_offset + t with q_offset = Lk - Lq by default, key j at kv_start + j
+    (ops/flex_attn_tilelang.py:108-121,155-171).  Returns (o fp32 (B,Lq,hq,Dv), lse fp32
+    (B,Lq,hq), natural log); rows that see no key get o = 0, lse = -inf."""
     B, L, HQ, D = q.shape
     Lk, H = k.shape[1], k.shape[2]
     G = HQ // H
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D)
+    if q_offset is None:
+        q_offset = Lk - L
     kf = k.float().repeat_interleave(G, dim=2)
     vf = v.float().repeat_interleave(G, dim=2)
     s = torch.einsum("bihd,bjhd->bhij", q.float(), kf) * sm_scale
-    real_q = torch.arange(L).view(L, 1) + q_offset
-    kv = torch.arange(Lk).view(1, Lk)
-    start = torch.div(real_q - window_size + 1, chunk_size, rounding_mode="floor") * chunk_size
+    real_q = torch.arange(L).view(L, 1) + q_offset + kv_start
+    kv = torch.arange(Lk).view(1, Lk) + kv_start
+    start = real_q - window_size + 1
+    if expand_to_chunk:
+        start = torch.div(start, chunk_size, rounding_mode="floor") * chunk_size
     keep = (kv >= start) & (kv <= real_q)
     if mask_lmk:
         keep = keep & (((kv + 1) % chunk_size) != 0)
     s = s.masked_fill(~keep.view(1, 1, L, Lk), NEG_INF)
     lse = torch.logsumexp(s, dim=-1)
     p = torch.exp(s - torch.where(torch.isfinite(lse), lse, torch.zeros_like(lse)).unsqueeze(-1))
+    p = torch.where(keep.view(1, 1, L, Lk), p, torch.zeros_like(p))
     o = torch.einsum("bhij,bjhd->bihd", p, vf)
     return o, lse.permute(0, 2, 1).contiguous()
 

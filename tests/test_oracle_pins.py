@@ -313,6 +313,32 @@ def test_swa_brute_force(orc):
         assert torch.allclose(o[0, t, 0], torch.softmax(s, 0) @ v[0, toks, 0], atol=1e-5)
 
 
+def test_swa_reduces_to_sdpa_and_positions(orc):
+    """Without chunk expansion and landmark mask the window is a plain banded causal mask
+    (F.scaled_dot_product_attention); with a cache, the queries are the last Lq positions and
+    a truncated cache only shifts absolute positions (brute force)."""
+    import torch.nn.functional as F
+    torch.manual_seed(13)
+    B, L, HQ, H, D, W = 1, 50, 2, 2, 8, 7
+    q, k, v = torch.randn(B, L, HQ, D), torch.randn(B, L, H, D), torch.randn(B, L, H, D)
+    o, lse = orc.swa(q, k, v, window_size=W, chunk_size=16, mask_lmk=False, expand_to_chunk=False)
+    i, j = torch.arange(L).view(L, 1), torch.arange(L).view(1, L)
+    band = (j <= i) & (j >= i - W + 1)
+    ref = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
+                                         attn_mask=band).transpose(1, 2)
+    assert torch.allclose(o, ref, atol=1e-5)
+    # inference: 5 queries at the end of a cache of 50 keys whose first key is position 11
+    S, kv0, Lq = 8, 11, 5
+    o2, lse2 = orc.swa(q[:, -Lq:], k, v, window_size=W, chunk_size=S, kv_start=kv0)
+    for t in range(Lq):
+        pos = kv0 + L - Lq + t
+        start = ((pos - W + 1) // S) * S
+        toks = [jj for jj in range(L) if start <= kv0 + jj <= pos and (kv0 + jj + 1) % S != 0]
+        sc = torch.stack([torch.dot(q[0, L - Lq + t, 1], k[0, jj, 1]) for jj in toks]) / math.sqrt(D)
+        assert lse2[0, t, 1].item() == pytest.approx(torch.logsumexp(sc, 0).item(), abs=1e-5)
+        assert torch.allclose(o2[0, t, 1], torch.softmax(sc, 0) @ v[0, toks, 1], atol=1e-5)
+
+
 def test_inter_chunk_softmax(orc):
     torch.manual_seed(12)
     B, L, HQ, H, K, N = 1, 6, 4, 2, 3, 5
