@@ -229,6 +229,379 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
   }
 }
 
+// ---- backward (training: Lq == Lk, kv_start == 0) -------------------------------------------
+//   P = exp(s - lse),  dP = dO V^T,  delta = sum_d o*dO - d_lse,  dS = P (dP - delta) * scale
+//   dQ = dS K,  dK = dS^T Q,  dV = P^T dO.
+// Same split as the forward: one side owned by a wavefront in registers, the other streamed
+// through LDS in 64-row tiles (row-major for the score-like products, transposed for the
+// gradient products).
+
+// visibility bits of this lane's landmark test for the 16 tokens tt*16 + 4j + i of a 64-token tile
+__device__ __forceinline__ unsigned swa_lmk_bits(const SwaDims& dm, int tok0) {
+  if (!dm.mask_lmk) return 0xffffu;
+  unsigned ok = 0u;
+#pragma unroll
+  for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ta = tok0 + tt * 16 + i + 1;
+      const bool lm = dm.chunk_pow2 ? ((ta & (dm.chunk - 1)) == 0) : (ta % dm.chunk == 0);
+      ok |= lm ? 0u : (1u << (tt * 4 + i));
+    }
+  return ok;
+}
+
+// dQ (and delta): a wavefront owns 32 score rows; K (row-major and transposed) and V stream.
+template <int D, int DV, int G>
+__global__ void __launch_bounds__(256)
+swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+                const bf16_t* __restrict__ o, const float* __restrict__ lse,
+                const bf16_t* __restrict__ d_o, const float* __restrict__ d_lse,
+                bf16_t* __restrict__ dq, float* __restrict__ delta_out, SwaDims dm, int n_qt) {
+  constexpr int KS = D / 32, VS = DV / 32, DT = D / 16;
+  constexpr int QW = 16 * SWA_RT / G, QB = 4 * QW;
+  constexpr int PITCH = D * 2 + 16, VPITCH = DV * 2 + 16;
+  constexpr int KSEG = D / 8, KPPP = 256 / KSEG, KPASS = 32 / KPPP;
+  constexpr int VSEG = DV / 8, VPASS = 64 * VSEG / 256;
+  __shared__ __align__(16) unsigned char k_s[64 * PITCH];
+  __shared__ __align__(16) unsigned char kt_s[D * LZM_PT];
+  __shared__ __align__(16) unsigned char v_s[64 * VPITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, j = lane >> 4;
+  const int qt = n_qt - 1 - (int)blockIdx.x;
+  const int hk = blockIdx.y;
+  const long b = blockIdx.z;
+  const int t0 = qt * QB + wave * QW;
+  const int L = dm.Lq;
+
+  bf16x8_t qa[SWA_RT][KS], doa[SWA_RT][VS];
+  int qabs[SWA_RT], cstart[SWA_RT];
+  float lse2[SWA_RT], delta[SWA_RT];
+#pragma unroll
+  for (int rt = 0; rt < SWA_RT; ++rt) {
+    const int row = rt * 16 + col;
+    const int t = t0 + row / G, g = row % G;
+    const int tc = t < L ? t : L - 1;
+    const long rix = (b * L + tc) * (long)dm.HQ + hk * G + g;
+    const float ls = lse[rix];
+    const bool live = t < L && ls > -1e30f;  // rows that saw no key have no gradient
+    qabs[rt] = live ? t : -2147483647;
+    const int left = tc - dm.window + 1;
+    cstart[rt] = dm.expand ? floordiv(left, dm.chunk) * dm.chunk : left;
+    lse2[rt] = live ? ls * HILS_LOG2E : 0.f;
+    const bf16_t* qp = q + rix * D + j * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qa[rt][ks] = *(const bf16x8_t*)(qp + ks * 32);
+    float part = 0.f;
+#pragma unroll
+    for (int vs = 0; vs < VS; ++vs) {
+      const uint4 dv4 = *(const uint4*)(d_o + rix * DV + vs * 32 + j * 8);
+      const uint4 ov4 = *(const uint4*)(o + rix * DV + vs * 32 + j * 8);
+      doa[rt][vs] = *(const bf16x8_t*)&dv4;
+      float a[8], c[8];
+      unpack8(dv4, a);
+      unpack8(ov4, c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) part = fmaf(a[e], c[e], part);
+    }
+    part = rows_sum(part);
+    delta[rt] = part - (d_lse ? d_lse[rix] : 0.f);
+    if (j == 0 && t < L) delta_out[rix] = delta[rt];
+  }
+  int tile_lo, tile_hi;
+  {
+    const int tq0 = qt * QB;
+    int tq1 = tq0 + QB - 1;
+    if (tq1 > L - 1) tq1 = L - 1;
+    const int left_abs = tq0 - dm.window + 1;
+    int lo = dm.expand ? floordiv(left_abs, dm.chunk) * dm.chunk : left_abs;
+    lo = lo < 0 ? 0 : lo;
+    tile_lo = lo / 64;
+    tile_hi = tq1 / 64 + 1;
+  }
+  const float c2 = dm.sm_scale * HILS_LOG2E;
+
+  uint4 kr[KPASS][2], vr[VPASS];
+  auto fetch = [&](int tile) {
+#pragma unroll
+    for (int i = 0; i < KPASS; ++i)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int tok = tile * 64 + 2 * (tid / KSEG + KPPP * i) + h;
+        kr[i][h] = make_uint4(0, 0, 0, 0);
+        if (tok < L) kr[i][h] = *(const uint4*)(k + ((b * L + tok) * (long)dm.H + hk) * D + (tid % KSEG) * 8);
+      }
+#pragma unroll
+    for (int i = 0; i < VPASS; ++i) {
+      const int p = tid + 256 * i;
+      const int tok = tile * 64 + p / VSEG;
+      vr[i] = make_uint4(0, 0, 0, 0);
+      if (tok < L) vr[i] = *(const uint4*)(v + ((b * L + tok) * (long)dm.H + hk) * DV + (p % VSEG) * 8);
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < KPASS; ++i)
+      lzm_stash_pair<PITCH>(k_s, kt_s, 2 * (tid / KSEG + KPPP * i), tid % KSEG, kr[i][0], kr[i][1]);
+#pragma unroll
+    for (int i = 0; i < VPASS; ++i) {
+      const int p = tid + 256 * i;
+      *(uint4*)(v_s + (p / VSEG) * VPITCH + (p % VSEG) * 16) = vr[i];
+    }
+  };
+  f32x4_t acc[SWA_RT][DT];
+#pragma unroll
+  for (int rt = 0; rt < SWA_RT; ++rt)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  fetch(tile_lo);
+  stash();
+  __syncthreads();
+  for (int tile = tile_lo; tile < tile_hi; ++tile) {
+    fetch(tile + 1 < tile_hi ? tile + 1 : tile);
+    float ds[SWA_RT][4][4];
+    {
+      f32x4_t st[SWA_RT][4], dp[SWA_RT][4];
+#pragma unroll
+      for (int rt = 0; rt < SWA_RT; ++rt)
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+          st[rt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+          dp[rt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8_t a = *(const bf16x8_t*)(k_s + (tt * 16 + col) * PITCH + ks * 64 + j * 16);
+#pragma unroll
+          for (int rt = 0; rt < SWA_RT; ++rt)
+            st[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qa[rt][ks], st[rt][tt], 0, 0, 0);
+        }
+#pragma unroll
+        for (int vs = 0; vs < VS; ++vs) {
+          const bf16x8_t a = *(const bf16x8_t*)(v_s + (tt * 16 + col) * VPITCH + vs * 64 + j * 16);
+#pragma unroll
+          for (int rt = 0; rt < SWA_RT; ++rt)
+            dp[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, doa[rt][vs], dp[rt][tt], 0, 0, 0);
+        }
+      }
+      const int tok0 = tile * 64 + 4 * j;
+      const unsigned lmk_ok = swa_lmk_bits(dm, tok0);
+#pragma unroll
+      for (int rt = 0; rt < SWA_RT; ++rt)
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int ta = tok0 + tt * 16 + i;
+            const bool vis = ta >= cstart[rt] && ta <= qabs[rt] && ((lmk_ok >> (tt * 4 + i)) & 1u);
+            const float pv = vis ? __builtin_amdgcn_exp2f(st[rt][tt][i] * c2 - lse2[rt]) : 0.f;
+            ds[rt][tt][i] = pv * (dp[rt][tt][i] - delta[rt]) * dm.sm_scale;
+          }
+    }
+    lzm_grad_product<D, SWA_RT>(kt_s, ds, acc, col, j);
+    __syncthreads();
+    stash();
+    __syncthreads();
+  }
+#pragma unroll
+  for (int rt = 0; rt < SWA_RT; ++rt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = rt * 16 + 4 * j + i;
+      const int t = t0 + row / G, g = row % G;
+      if (t >= L) continue;
+      bf16_t* out = dq + ((b * L + t) * (long)dm.HQ + hk * G + g) * D + col;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) out[dt * 16] = f2bf(acc[rt][dt][i]);
+    }
+}
+
+// dK, dV: a workgroup owns 128 tokens of one KV head (32 per wavefront, as matrix B operands); the
+// score rows (query x head) that can see them stream in tiles of 64 rows, Q and dO both row-major
+// and transposed, with the rows' lse, delta and window start beside them.
+template <int D, int DV, int G>
+__global__ void __launch_bounds__(256)
+swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                  const bf16_t* __restrict__ v, const float* __restrict__ lse,
+                  const bf16_t* __restrict__ d_o, const float* __restrict__ delta_in,
+                  bf16_t* __restrict__ dk, bf16_t* __restrict__ dv, SwaDims dm) {
+  constexpr int KS = D / 32, VS = DV / 32, DT = D / 16, DVT = DV / 16;
+  constexpr int QT = 64 / G;
+  constexpr int PITCH = D * 2 + 16, VPITCH = DV * 2 + 16;
+  constexpr int QSEG = D / 8, QPPP = 256 / QSEG, QPASS = 32 / QPPP;
+  constexpr int OSEG = DV / 8, OPPP = 256 / OSEG, OPASS = 32 / OPPP;
+  extern __shared__ __align__(16) unsigned char dyn[];
+  unsigned char* q_s = dyn;                       // 64 * PITCH
+  unsigned char* qt_s = q_s + 64 * PITCH;         // D * LZM_PT
+  unsigned char* do_s = qt_s + D * LZM_PT;        // 64 * VPITCH
+  unsigned char* dot_s = do_s + 64 * VPITCH;      // DV * LZM_PT
+  float* lse_s = (float*)(dot_s + DV * LZM_PT);   // 64
+  float* del_s = lse_s + 64;                      // 64
+  int* cs_s = (int*)(del_s + 64);                 // 64: window start of the row (INT_MAX: dead row)
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, j = lane >> 4;
+  const int hk = blockIdx.y;
+  const long b = blockIdx.z;
+  const int L = dm.Lq;
+  const int j0 = (int)blockIdx.x * 128;
+  const int tok_w = j0 + wave * 32;  // first owned token of the wavefront
+
+  bf16x8_t ka[2][KS], va[2][VS];
+  unsigned lmk_ok = 0u;  // bit tt: owned token tt*16 + col is not a landmark
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+    const int tok = tok_w + tt * 16 + col;
+    const int tc = tok < L ? tok : L - 1;  // tokens past the end are never visible
+    const bf16_t* kp = k + ((b * L + tc) * (long)dm.H + hk) * D + j * 8;
+    const bf16_t* vp = v + ((b * L + tc) * (long)dm.H + hk) * DV + j * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ka[tt][ks] = *(const bf16x8_t*)(kp + ks * 32);
+#pragma unroll
+    for (int vs = 0; vs < VS; ++vs) va[tt][vs] = *(const bf16x8_t*)(vp + vs * 32);
+    const bool lm = dm.mask_lmk && (dm.chunk_pow2 ? (((tok + 1) & (dm.chunk - 1)) == 0) : ((tok + 1) % dm.chunk == 0));
+    if (!lm && tok < L) lmk_ok |= 1u << tt;
+  }
+  // queries that can see a token of [j0, j1]: j0 <= t <= (last window that starts at or before j1)
+  int j1 = j0 + 127;
+  if (j1 > L - 1) j1 = L - 1;
+  long t_hi = dm.expand ? ((long)(j1 / dm.chunk) + 1) * dm.chunk + dm.window - 2 : (long)j1 + dm.window - 1;
+  if (t_hi > L - 1) t_hi = L - 1;
+  const int tile0 = j0 / QT;
+  const int n_tiles = (int)(t_hi / QT) + 1;
+  const float c2 = dm.sm_scale * HILS_LOG2E;
+
+  uint4 qr[QPASS][2], dor[OPASS][2];
+  float r_lse = 0.f, r_del = 0.f;
+  int r_cs = 2147483647;
+  auto fetch = [&](int tile) {
+#pragma unroll
+    for (int i = 0; i < QPASS; ++i)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int row = 2 * (tid / QSEG + QPPP * i) + h;
+        int t = tile * QT + row / G;
+        if (t > L - 1) t = L - 1;
+        qr[i][h] = *(const uint4*)(q + ((b * L + t) * (long)dm.HQ + hk * G + row % G) * D + (tid % QSEG) * 8);
+      }
+#pragma unroll
+    for (int i = 0; i < OPASS; ++i)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int row = 2 * (tid / OSEG + OPPP * i) + h;
+        int t = tile * QT + row / G;
+        if (t > L - 1) t = L - 1;
+        dor[i][h] = *(const uint4*)(d_o + ((b * L + t) * (long)dm.HQ + hk * G + row % G) * DV + (tid % OSEG) * 8);
+      }
+    if (tid < 64) {
+      const int t = tile * QT + tid / G;
+      const int tc = t < L ? t : L - 1;
+      const long rix = (b * L + tc) * (long)dm.HQ + hk * G + tid % G;
+      const float ls = lse[rix];
+      const bool live = t < L && ls > -1e30f;
+      r_lse = live ? ls * HILS_LOG2E : 0.f;
+      r_del = delta_in[rix];
+      const int left = tc - dm.window + 1;
+      r_cs = live ? (dm.expand ? floordiv(left, dm.chunk) * dm.chunk : left) : 2147483647;
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < QPASS; ++i)
+      lzm_stash_pair<PITCH>(q_s, qt_s, 2 * (tid / QSEG + QPPP * i), tid % QSEG, qr[i][0], qr[i][1]);
+#pragma unroll
+    for (int i = 0; i < OPASS; ++i)
+      lzm_stash_pair<VPITCH>(do_s, dot_s, 2 * (tid / OSEG + OPPP * i), tid % OSEG, dor[i][0], dor[i][1]);
+    if (tid < 64) {
+      lse_s[tid] = r_lse;
+      del_s[tid] = r_del;
+      cs_s[tid] = r_cs;
+    }
+  };
+  f32x4_t acck[2][DT], accv[2][DVT];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acck[tt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt) accv[tt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  fetch(tile0);
+  stash();
+  __syncthreads();
+  for (int tile = tile0; tile < n_tiles; ++tile) {
+    fetch(tile + 1 < n_tiles ? tile + 1 : tile);
+    float p[2][4][4], ds[2][4][4];  // [owned token tile][streamed row tile][row 4j+i]
+    {
+      f32x4_t st[2][4], dp[2][4];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          st[tt][rr] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+          dp[tt][rr] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8_t a = *(const bf16x8_t*)(q_s + (rr * 16 + col) * PITCH + ks * 64 + j * 16);
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt)
+            st[tt][rr] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ka[tt][ks], st[tt][rr], 0, 0, 0);
+        }
+#pragma unroll
+        for (int vs = 0; vs < VS; ++vs) {
+          const bf16x8_t a = *(const bf16x8_t*)(do_s + (rr * 16 + col) * VPITCH + vs * 64 + j * 16);
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt)
+            dp[tt][rr] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, va[tt][vs], dp[tt][rr], 0, 0, 0);
+        }
+      }
+      const int tq0 = tile * QT;
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const float4 l4 = *(const float4*)&lse_s[rr * 16 + 4 * j];
+        const float4 d4 = *(const float4*)&del_s[rr * 16 + 4 * j];
+        const int4 c4 = *(const int4*)&cs_s[rr * 16 + 4 * j];
+        const float ls[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
+        const int cs[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int t = tq0 + (rr * 16 + 4 * j + i) / G;
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt) {
+            const int tok = tok_w + tt * 16 + col;
+            const bool vis = tok >= cs[i] && tok <= t && ((lmk_ok >> tt) & 1u);
+            const float pv = vis ? __builtin_amdgcn_exp2f(st[tt][rr][i] * c2 - ls[i]) : 0.f;
+            p[tt][rr][i] = pv;
+            ds[tt][rr][i] = pv * (dp[tt][rr][i] - dl[i]) * dm.sm_scale;
+          }
+        }
+      }
+    }
+    lzm_grad_product<DV, 2>(dot_s, p, accv, col, j);
+    lzm_grad_product<D, 2>(qt_s, ds, acck, col, j);
+    __syncthreads();
+    stash();
+    __syncthreads();
+  }
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int tok = tok_w + tt * 16 + 4 * j + i;
+      if (tok >= L) continue;
+      bf16_t* outk = dk + ((b * L + tok) * (long)dm.H + hk) * D + col;
+      bf16_t* outv = dv + ((b * L + tok) * (long)dm.H + hk) * DV + col;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) outk[dt * 16] = f2bf(acck[tt][dt][i]);
+#pragma unroll
+      for (int dt = 0; dt < DVT; ++dt) outv[dt * 16] = f2bf(accv[tt][dt][i]);
+    }
+}
+
 template <int D, int DV>
 static void swa_launch_g(int G, dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* k,
                          const bf16_t* v, bf16_t* o, float* lse, const SwaDims& dm, int n_qt) {
@@ -273,5 +646,76 @@ extern "C" int hils_swa_fwd(const void* q, const void* k, const void* v, void* o
   else if (D == 64) swa_launch_g<64, 128>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
   else swa_launch_g<128, 64>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
   HILS_CHECK_LAUNCH("hils_swa_fwd");
+  return HILS_OK;
+}
+
+template <int D, int DV, int G>
+static int swa_bwd_launch(const bf16_t* q, const bf16_t* k, const bf16_t* v, const bf16_t* o,
+                          const float* lse, const bf16_t* d_o, const float* d_lse, bf16_t* dq, bf16_t* dk,
+                          bf16_t* dv, float* delta, int B, const SwaDims& dm, hipStream_t st) {
+  const int QB = 4 * 16 * SWA_RT / G;
+  const int n_qt = (dm.Lq + QB - 1) / QB;
+  hipLaunchKernelGGL((swa_bwd_dq_mfma<D, DV, G>), dim3((unsigned)n_qt, (unsigned)dm.H, (unsigned)B),
+                     dim3(256), 0, st, q, k, v, o, lse, d_o, d_lse, dq, delta, dm, n_qt);
+  const size_t smem = (size_t)64 * (D * 2 + 16) + (size_t)D * LZM_PT + (size_t)64 * (DV * 2 + 16) +
+                      (size_t)DV * LZM_PT + 3 * 64 * sizeof(float);
+  auto kern = swa_bwd_dkdv_mfma<D, DV, G>;
+  static size_t reserved = 48 * 1024;  // per instantiation
+  if (smem > reserved) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) !=
+        hipSuccess) {
+      hils_set_error("hils_swa_bwd: cannot reserve %zu bytes of LDS", smem);
+      return HILS_ERR_LAUNCH;
+    }
+    reserved = smem;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)((dm.Lq + 127) / 128), (unsigned)dm.H, (unsigned)B), dim3(256),
+                     smem, st, q, k, v, lse, d_o, delta, dk, dv, dm);
+  return HILS_OK;
+}
+
+template <int D, int DV>
+static int swa_bwd_launch_g(int G, const bf16_t* q, const bf16_t* k, const bf16_t* v, const bf16_t* o,
+                            const float* lse, const bf16_t* d_o, const float* d_lse, bf16_t* dq,
+                            bf16_t* dk, bf16_t* dv, float* delta, int B, const SwaDims& dm, hipStream_t st) {
+  switch (G) {
+    case 1: return swa_bwd_launch<D, DV, 1>(q, k, v, o, lse, d_o, d_lse, dq, dk, dv, delta, B, dm, st);
+    case 2: return swa_bwd_launch<D, DV, 2>(q, k, v, o, lse, d_o, d_lse, dq, dk, dv, delta, B, dm, st);
+    case 4: return swa_bwd_launch<D, DV, 4>(q, k, v, o, lse, d_o, d_lse, dq, dk, dv, delta, B, dm, st);
+    case 8: return swa_bwd_launch<D, DV, 8>(q, k, v, o, lse, d_o, d_lse, dq, dk, dv, delta, B, dm, st);
+    default: return swa_bwd_launch<D, DV, 16>(q, k, v, o, lse, d_o, d_lse, dq, dk, dv, delta, B, dm, st);
+  }
+}
+
+extern "C" int hils_swa_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse,
+                            const void* d_o, const float* d_lse, void* dq, void* dk, void* dv,
+                            float* delta, int B, int L, int HQ, int H, int D, int Dv, int window,
+                            int chunk, int mask_lmk, int expand_to_chunk, float sm_scale, void* stream) {
+  HILS_REQUIRE(q && k && v && o && lse && d_o && dq && dk && dv && delta, "hils_swa_bwd: null pointer");
+  HILS_REQUIRE(B > 0 && L > 0 && HQ > 0 && H > 0, "hils_swa_bwd: sizes must be positive");
+  HILS_REQUIRE(HQ % H == 0, "hils_swa_bwd: HQ (%d) must be a multiple of H (%d)", HQ, H);
+  HILS_REQUIRE(window >= 1 && chunk >= 1, "hils_swa_bwd: window and chunk must be positive");
+  const int G = HQ / H;
+  HILS_REQUIRE((D == 64 || D == 128) && (Dv == 64 || Dv == 128),
+               "hils_swa_bwd: head dims (%d, %d) must be 64 or 128", D, Dv);
+  HILS_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8 || G == 16,
+               "hils_swa_bwd: group size %d must be 1, 2, 4, 8 or 16", G);
+  HILS_REQUIRE(H <= 65535 && B <= 65535, "hils_swa_bwd: H/B too large for the grid");
+  HILS_REQUIRE((long)L + window < 2147483647L / 2, "hils_swa_bwd: positions overflow 32 bits");
+  SwaDims dm{L, L, HQ, H, window, chunk, mask_lmk, expand_to_chunk, 0, (chunk & (chunk - 1)) == 0, sm_scale};
+  hipStream_t st = (hipStream_t)stream;
+  const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k, *vv = (const bf16_t*)v,
+               *oo = (const bf16_t*)o, *dd = (const bf16_t*)d_o;
+  int rc;
+  if (D == 64 && Dv == 64)
+    rc = swa_bwd_launch_g<64, 64>(G, qq, kk, vv, oo, lse, dd, d_lse, (bf16_t*)dq, (bf16_t*)dk, (bf16_t*)dv, delta, B, dm, st);
+  else if (D == 128 && Dv == 128)
+    rc = swa_bwd_launch_g<128, 128>(G, qq, kk, vv, oo, lse, dd, d_lse, (bf16_t*)dq, (bf16_t*)dk, (bf16_t*)dv, delta, B, dm, st);
+  else if (D == 64)
+    rc = swa_bwd_launch_g<64, 128>(G, qq, kk, vv, oo, lse, dd, d_lse, (bf16_t*)dq, (bf16_t*)dk, (bf16_t*)dv, delta, B, dm, st);
+  else
+    rc = swa_bwd_launch_g<128, 64>(G, qq, kk, vv, oo, lse, dd, d_lse, (bf16_t*)dq, (bf16_t*)dk, (bf16_t*)dv, delta, B, dm, st);
+  if (rc) return rc;
+  HILS_CHECK_LAUNCH("hils_swa_bwd");
   return HILS_OK;
 }

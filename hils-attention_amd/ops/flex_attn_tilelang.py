@@ -1,4 +1,4 @@
-"""Sliding-window attention of the local branch (drop-in for the forward of the reference's
+"""Sliding-window attention of the local branch (drop-in for flex_attn_tl of the reference's
 ops/flex_attn_tilelang.py)."""
 import math
 
@@ -8,8 +8,8 @@ from . import _cabi
 
 
 class _FlexAttnTL(torch.autograd.Function):
-    """Mirrors the forward of _FlexAttnTL (ops/flex_attn_tilelang.py:1261-1310 and the kernel at
-    :26-267).  The backward kernels are not built: backward raises."""
+    """Mirrors _FlexAttnTL (ops/flex_attn_tilelang.py:1156-1255; kernels :26-267 forward,
+    :270-1153 backward).  lse is kept in natural-log units throughout."""
 
     @staticmethod
     def forward(ctx, q, k, v, window_size, chunk_size, mask_lmk, expand_to_chunk, use_cache, sm_scale,
@@ -33,13 +33,28 @@ class _FlexAttnTL(torch.autograd.Function):
         _cabi.call("hils_swa_fwd", _cabi.ptr(q_c), _cabi.ptr(k_c), _cabi.ptr(v_c), _cabi.ptr(o),
                    _cabi.ptr(lse), B, Lq, Lk, HQ, H, D, Dv, int(window_size), int(chunk_size),
                    int(bool(mask_lmk)), int(bool(expand_to_chunk)), int(kv_start), float(sm_scale))
+        ctx.save_for_backward(q_c, k_c, v_c, o, lse)
+        ctx.cfg = (int(window_size), int(chunk_size), bool(mask_lmk), bool(expand_to_chunk),
+                   bool(use_cache), float(sm_scale))
         return o, lse
 
     @staticmethod
     def backward(ctx, do, dlse):
-        raise NotImplementedError(
-            "flex_attn_tl: only the forward runs on this library; the backward kernels "
-            "(flex_attn_bwd_dq / flex_attn_bwd_dkdv of the reference) are not built yet")
+        q, k, v, o, lse = ctx.saved_tensors
+        window_size, chunk_size, mask_lmk, expand_to_chunk, use_cache, sm_scale = ctx.cfg
+        if use_cache:
+            raise RuntimeError("flex_attn_tl backward is not supported in inference (training=False) mode")
+        B, L, HQ, D = q.shape
+        H, Dv = k.shape[2], v.shape[-1]
+        do = do.to(torch.bfloat16).contiguous()
+        d_lse = None if dlse is None else dlse.float().contiguous()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        delta = torch.empty((B, L, HQ), dtype=torch.float32, device=q.device)
+        _cabi.call("hils_swa_bwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(o), _cabi.ptr(lse),
+                   _cabi.ptr(do), _cabi.ptr(d_lse), _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv),
+                   _cabi.ptr(delta), B, L, HQ, H, D, Dv, window_size, chunk_size, int(mask_lmk),
+                   int(expand_to_chunk), sm_scale)
+        return dq, dk, dv, None, None, None, None, None, None, None
 
 
 def flex_attn_tl(q, k, v, window_size: int, chunk_size: int, training: bool = True,

@@ -178,6 +178,17 @@ int hils_swa_fwd(const void* q, const void* k, const void* v, void* o, float* ls
                  int Lk, int HQ, int H, int D, int Dv, int window, int chunk, int mask_lmk,
                  int expand_to_chunk, int kv_start, float sm_scale, void* stream);
 
+/* Backward (training: Lq == Lk = L, kv_start = 0).  Replaces flex_attn_bwd_preprocess,
+ * flex_attn_bwd_dq and flex_attn_bwd_dkdv (ops/flex_attn_tilelang.py:270-1153) as driven by
+ * _FlexAttnTL.backward.  o, lse: the forward's outputs (lse in natural-log units); d_o bf16;
+ * d_lse (B,L,HQ) fp32 gradient of lse, may be NULL (= 0).  Writes dq (B,L,HQ,D), dk (B,L,H,D),
+ * dv (B,L,H,Dv) bf16 (every element, dk/dv already summed over the heads of a group) and uses
+ * delta (B,L,HQ) fp32 as scratch (sum_d o*d_o - d_lse). */
+int hils_swa_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse,
+                 const void* d_o, const float* d_lse, void* dq, void* dk, void* dv, float* delta,
+                 int B, int L, int HQ, int H, int D, int Dv, int window, int chunk, int mask_lmk,
+                 int expand_to_chunk, float sm_scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

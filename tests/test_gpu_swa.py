@@ -62,10 +62,51 @@ def test_swa_landmark_query_row_sees_no_key(pkg, dev):
     assert torch.isfinite(lse[0, 62]).all()
 
 
-def test_swa_backward_raises_and_argument_errors(pkg, dev):
+@pytest.mark.parametrize("B,L,HQ,H,D,Dv,W,S,mask_lmk,expand", [
+    (1, 384, 4, 2, 64, 64, 64, 64, True, True), (2, 200, 8, 2, 128, 128, 48, 64, True, True),
+    (1, 300, 2, 2, 64, 128, 100, 32, False, True), (1, 260, 16, 1, 64, 64, 33, 48, True, False),
+    (1, 513, 4, 4, 128, 64, 1, 64, False, False)])
+def test_swa_backward(pkg, orc, dev, B, L, HQ, H, D, Dv, W, S, mask_lmk, expand):
+    """dq, dk, dv with gradients arriving through both outputs (o and lse)."""
+    note(f"swa_bwd B{B} L{L} HQ{HQ} H{H} D{D} Dv{Dv} W{W} S{S} lmk{mask_lmk} exp{expand}")
+    gen = torch.Generator().manual_seed(7)
+    q = torch.randn(B, L, HQ, D, generator=gen).bfloat16()
+    k = torch.randn(B, L, H, D, generator=gen).bfloat16()
+    v = torch.randn(B, L, H, Dv, generator=gen).bfloat16()
+    do = torch.randn(B, L, HQ, Dv, generator=gen).bfloat16()
+    dl = torch.randn(B, L, HQ, generator=gen)
+    qd, kd, vd = (t.to(dev).requires_grad_() for t in (q, k, v))
+    o, lse = pkg.flex_attn_tl(qd, kd, vd, W, S, mask_lmk=mask_lmk, expand_to_chunk=expand)
+    fin = torch.isfinite(lse)
+    ((o.float() * do.to(dev).float()).sum() + torch.where(fin, lse, torch.zeros_like(lse)).mul(dl.to(dev)).sum()).backward()
+    qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
+    ro, rlse = orc.swa(qf, kf, vf, window_size=W, chunk_size=S, mask_lmk=mask_lmk, expand_to_chunk=expand)
+    rfin = torch.isfinite(rlse)
+    assert torch.equal(fin.cpu(), rfin)
+    ((ro * do.float()).sum() + torch.where(rfin, rlse, torch.zeros_like(rlse)).mul(dl).sum()).backward()
+    assert_close_bf16(qd.grad, qf.grad, "swa dq")
+    assert_close_bf16(kd.grad, kf.grad, "swa dk")
+    assert_close_bf16(vd.grad, vf.grad, "swa dv")
+
+
+def test_swa_backward_only_through_o(pkg, orc, dev):
+    torch.manual_seed(8)
+    q, k, v = (torch.randn(1, 192, h, 64).bfloat16() for h in (4, 2, 2))
+    qd, kd, vd = (t.to(dev).requires_grad_() for t in (q, k, v))
+    o, _ = pkg.flex_attn_tl(qd, kd, vd, 64, 64)
+    o.float().pow(2).sum().backward()
+    qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
+    ro, _ = orc.swa(qf, kf, vf, window_size=64, chunk_size=64)
+    ro.pow(2).sum().backward()
+    assert_close_bf16(qd.grad, qf.grad, "swa dq (o only)")
+    assert_close_bf16(kd.grad, kf.grad, "swa dk (o only)")
+    assert_close_bf16(vd.grad, vf.grad, "swa dv (o only)")
+
+
+def test_swa_inference_backward_raises_and_argument_errors(pkg, dev):
     q = torch.randn(1, 64, 2, 64, device=dev).bfloat16().requires_grad_()
-    o, lse = pkg.flex_attn_tl(q, q.detach(), q.detach(), 16, 64)
-    with pytest.raises(NotImplementedError):
+    o, lse = pkg.flex_attn_tl(q, q.detach(), q.detach(), 16, 64, training=False)
+    with pytest.raises(RuntimeError):
         o.sum().backward()
     with pytest.raises(ValueError):
         pkg.flex_attn_tl(q, q, q, 16, 64, training=True, kv_start=5)
