@@ -291,6 +291,32 @@ def bench_ops(pkg, dev, iters=3):
     out["log_z_fwd_bwd"] = {"workload": "same (includes the torch glue of the loss)", "ms": t,
                             "mfma_tflops": 5.0 * flops / (t * 1e-3) / 1e12}
     del q, k, qg, kg
+    # sliding-window attention of the local branch: B1 L32768 hq32/hkv8 D128, window 64, chunk 64
+    L, HQ, HK, D = 32768, 32, 8, 128
+    q = gpu_randn((1, L, HQ, D), gen, dev)
+    k = gpu_randn((1, L, HK, D), gen, dev)
+    v = gpu_randn((1, L, HK, D), gen, dev)
+    with torch.no_grad():
+        t = timed(lambda: pkg.flex_attn_tl(q, k, v, 64, 64))
+        _, lse_w = pkg.flex_attn_tl(q, k, v, 64, 64)
+    # visible keys per query: from the chunk start of (t - 63) to t, landmarks excluded
+    tt = torch.arange(L, device=dev)
+    start = torch.div(tt - 63, 64, rounding_mode="floor").clamp_min(0) * 64
+    n_vis = float((tt - start + 1 - (tt // 64 - start // 64) - ((tt + 1) % 64 == 0).long()).sum().item())
+    out["swa_fwd"] = {"workload": "B1 L32768 hq32/hkv8 D128 window64 chunk64", "us": t * 1e3,
+                      "visible_tflops": 4.0 * D * HQ * n_vis / (t * 1e-3) / 1e12,
+                      "hbm_gbs": (2 * q.numel() + k.numel() + v.numel()) * 2 / (t * 1e-3) / 1e9}
+    qg, kg, vg = (x.clone().requires_grad_() for x in (q, k, v))
+    d_o = gpu_randn((1, L, HQ, D), gen, dev)
+
+    def swa_fb():
+        for x in (qg, kg, vg):
+            x.grad = None
+        o, lse = pkg.flex_attn_tl(qg, kg, vg, 64, 64)
+        torch.autograd.backward([o, lse], [d_o, torch.ones_like(lse)])
+
+    out["swa_fwd_bwd"] = {"workload": "same", "us": timed(swa_fb) * 1e3}
+    del q, k, v, qg, kg, vg, d_o
     # HSA: N2 L4096 hq16/hkv4 D64, 16 chunks per block of 16 queries
     Nb, L, HQ, HK, D, K, QX = 2, 4096, 16, 4, 64, 16, 16
     q = gpu_randn((Nb, L, HQ, D), gen, dev)

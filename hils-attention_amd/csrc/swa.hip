@@ -18,18 +18,20 @@ struct SwaDims {
   float sm_scale;
 };
 
-template <int D, int DV, int G>
-__global__ void __launch_bounds__(256)
+template <int D, int DV, int G, int RT>
+__global__ void __launch_bounds__(256, (RT == 1 ? 3 : 2))
 swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
              bf16_t* __restrict__ o, float* __restrict__ lse, SwaDims dm, int n_qt) {
   constexpr int KS = D / 32, DT = DV / 16;
-  constexpr int QW = 16 * SWA_RT / G, QB = 4 * QW;
+  constexpr int QW = 16 * RT / G, QB = 4 * QW;
   constexpr int PITCH = D * 2 + 16;
   constexpr int KSEG = D / 8, KPASS = 64 * KSEG / 256;        // K tile: 16-byte pieces per thread
   constexpr int VSEG = DV / 8, VPPP = 256 / VSEG, VPASS = 32 / VPPP;  // V tile: row pairs per pass
-  __shared__ __align__(16) unsigned char k_s[64 * PITCH];
+  constexpr int OP = DV * 2 + 16;  // bytes per staged output row
+  constexpr int KBYTES = 64 * PITCH > 64 * RT * OP ? 64 * PITCH : 64 * RT * OP;
+  __shared__ __align__(16) unsigned char k_s[KBYTES];  // K tile; the output tile at the end
   __shared__ __align__(16) unsigned char vt_s[DV * LZM_PT];
-  __shared__ __align__(16) float bc_s[4][SWA_RT][16];  // per wavefront: per-row factors, transposed read
+  __shared__ __align__(16) float bc_s[4][RT][16];  // per wavefront: per-row factors, transposed read
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, j = lane >> 4;
   const int qt = n_qt - 1 - (int)blockIdx.x;
@@ -38,10 +40,10 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
   const int t0 = qt * QB + wave * QW;
   const int q_off = dm.kv_start + dm.Lk - dm.Lq;  // absolute position of query 0
 
-  bf16x8_t qa[SWA_RT][KS];
-  int qabs[SWA_RT], cstart[SWA_RT];
+  bf16x8_t qa[RT][KS];
+  int qabs[RT], cstart[RT];
 #pragma unroll
-  for (int rt = 0; rt < SWA_RT; ++rt) {
+  for (int rt = 0; rt < RT; ++rt) {
     const int row = rt * 16 + col;
     const int t = t0 + row / G, g = row % G;
     const int tc = t < dm.Lq ? t : dm.Lq - 1;
@@ -104,14 +106,14 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
       }
     }
   };
-  f32x4_t acc[SWA_RT][DT];
+  f32x4_t acc[RT][DT];
 #pragma unroll
-  for (int rt = 0; rt < SWA_RT; ++rt)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  float m_run[SWA_RT], l_run[SWA_RT];  // running max (raw score units) and sum, per row (lane & 15)
+  float m_run[RT], l_run[RT];  // running max (raw score units) and sum, per row (lane & 15)
 #pragma unroll
-  for (int rt = 0; rt < SWA_RT; ++rt) {
+  for (int rt = 0; rt < RT; ++rt) {
     m_run[rt] = HILS_NEG_INF;
     l_run[rt] = 0.f;
   }
@@ -122,11 +124,11 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
   __syncthreads();
   for (int tile = tile_lo; tile < tile_hi; ++tile) {
     fetch(tile + 1 < tile_hi ? tile + 1 : tile);
-    float p[SWA_RT][4][4];
+    float p[RT][4][4];
     {
-      f32x4_t st[SWA_RT][4];
+      f32x4_t st[RT][4];
 #pragma unroll
-      for (int rt = 0; rt < SWA_RT; ++rt)
+      for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) st[rt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -135,7 +137,7 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
         for (int ks = 0; ks < KS; ++ks) {
           const bf16x8_t a = *(const bf16x8_t*)(k_s + (tt * 16 + col) * PITCH + ks * 64 + j * 16);
 #pragma unroll
-          for (int rt = 0; rt < SWA_RT; ++rt)
+          for (int rt = 0; rt < RT; ++rt)
             st[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qa[rt][ks], st[rt][tt], 0, 0, 0);
         }
       // visibility of this lane's 16 tokens: bit tt*4+i; the landmark test does not depend on the row
@@ -154,7 +156,7 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
       const int tok_abs0 = dm.kv_start + tile * 64 + 4 * j;
       const int raw_left = dm.Lk - tile * 64 - 4 * j;  // tokens tt*16+i < raw_left exist
 #pragma unroll
-      for (int rt = 0; rt < SWA_RT; ++rt) {
+      for (int rt = 0; rt < RT; ++rt) {
         float mx = HILS_NEG_INF;
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
@@ -189,7 +191,7 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
     }
     // rescale the output accumulators: their rows are 4j+i, the factors live per lane & 15
 #pragma unroll
-    for (int rt = 0; rt < SWA_RT; ++rt) {
+    for (int rt = 0; rt < RT; ++rt) {
       const float4 c4 = *(const float4*)&bc_s[wave][rt][4 * j];
       const float cf[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
@@ -197,14 +199,14 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[rt][dt][i] *= cf[i];
     }
-    lzm_grad_product<DV, SWA_RT>(vt_s, p, acc, col, j);
+    lzm_grad_product<DV, RT>(vt_s, p, acc, col, j);
     __syncthreads();
     stash();
     __syncthreads();
   }
   // ---- finalize: o = acc / l, lse = ln(l) + max * scale ----
 #pragma unroll
-  for (int rt = 0; rt < SWA_RT; ++rt) {
+  for (int rt = 0; rt < RT; ++rt) {
     const float inv = l_run[rt] > 0.f ? 1.f / l_run[rt] : 0.f;
     if (j == 0) bc_s[wave][rt][col] = inv;
     const int row = rt * 16 + col;
@@ -213,19 +215,28 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
       lse[(b * dm.Lq + t) * (long)dm.HQ + hk * G + g] =
           l_run[rt] > 0.f ? (m_run[rt] * c2 + __builtin_amdgcn_logf(l_run[rt])) * HILS_LN2 : HILS_NEG_INF;
   }
+  // the loop's last barrier has passed: the K buffer is free.  Each wavefront parks its normalised
+  // rows there as bf16 and writes them out as 16-byte pieces (a query's heads are contiguous).
+  unsigned char* ob = k_s + wave * (16 * RT) * OP;
 #pragma unroll
-  for (int rt = 0; rt < SWA_RT; ++rt) {
+  for (int rt = 0; rt < RT; ++rt) {
     const float4 c4 = *(const float4*)&bc_s[wave][rt][4 * j];
     const float cf[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = rt * 16 + 4 * j + i;
-      const int t = t0 + row / G, g = row % G;
-      if (t >= dm.Lq) continue;
-      bf16_t* out = o + ((b * dm.Lq + t) * (long)dm.HQ + hk * G + g) * DV + col;
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) out[dt * 16] = f2bf(acc[rt][dt][i] * cf[i]);
-    }
+      for (int dt = 0; dt < DT; ++dt)
+        *(bf16_t*)(ob + (rt * 16 + 4 * j + i) * OP + (dt * 16 + col) * 2) = f2bf(acc[rt][dt][i] * cf[i]);
+  }
+  __builtin_amdgcn_wave_barrier();
+  constexpr int OSEG = DV / 8;
+#pragma unroll
+  for (int p = 0; p < 16 * RT * OSEG / 64; ++p) {
+    const int pc = p * 64 + lane;
+    const int row = pc / OSEG, seg = pc % OSEG;
+    const int t = t0 + row / G, g = row % G;
+    if (t < dm.Lq)
+      *(uint4*)(o + ((b * dm.Lq + t) * (long)dm.HQ + hk * G + g) * DV + seg * 8) = *(const uint4*)(ob + row * OP + seg * 16);
   }
 }
 
@@ -602,11 +613,14 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     }
 }
 
+// rows per wavefront of the forward kernel: 16 * SWA_FWD_RT(D, DV)
+#define SWA_FWD_RT(D_, DV_) (((D_) + (DV_) > 128) ? 1 : 2)
 template <int D, int DV>
 static void swa_launch_g(int G, dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* k,
                          const bf16_t* v, bf16_t* o, float* lse, const SwaDims& dm, int n_qt) {
-#define SWA_CALL(G_) \
-  hipLaunchKernelGGL((swa_fwd_mfma<D, DV, G_>), grid, dim3(256), 0, st, q, k, v, o, lse, dm, n_qt)
+#define SWA_CALL(G_)                                                                             \
+  hipLaunchKernelGGL((swa_fwd_mfma<D, DV, G_, SWA_FWD_RT(D, DV)>), grid, dim3(256), 0, st, q, k, v, \
+                     o, lse, dm, n_qt)
   switch (G) {
     case 1: SWA_CALL(1); break;
     case 2: SWA_CALL(2); break;
@@ -636,7 +650,7 @@ extern "C" int hils_swa_fwd(const void* q, const void* k, const void* v, void* o
   HILS_REQUIRE((long)kv_start + Lk < 2147483647L / 2, "hils_swa_fwd: positions overflow 32 bits");
   SwaDims dm{Lq, Lk, HQ, H, window, chunk, mask_lmk, expand_to_chunk, kv_start,
              (chunk & (chunk - 1)) == 0, sm_scale};
-  const int QB = 4 * 16 * SWA_RT / G;
+  const int QB = 4 * 16 * SWA_FWD_RT(D, Dv) / G;  // rows of a workgroup / group size (>= 1: G <= 16)
   const int n_qt = (Lq + QB - 1) / QB;
   const dim3 grid((unsigned)n_qt, (unsigned)H, (unsigned)B);
   hipStream_t st = (hipStream_t)stream;
