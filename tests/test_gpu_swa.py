@@ -113,3 +113,39 @@ def test_swa_inference_backward_raises_and_argument_errors(pkg, dev):
     with pytest.raises(RuntimeError):  # head dim the kernels do not cover
         x = torch.randn(1, 64, 2, 32, device=dev).bfloat16()
         pkg.flex_attn_tl(x, x, x, 16, 64)
+
+
+@pytest.mark.parametrize("L,HQ,H,D,W", [(512, 4, 2, 64, 64), (448, 8, 2, 128, 1)])
+def test_local_and_remote_branch_sum_to_dense_attention(pkg, dev, L, HQ, H, D, W):
+    """Every piece on the GPU: local branch (o, lse) + every remote chunk selected with the weights
+    softmax([log Z_c, lse_swa]) must equal ordinary causal attention over the non-landmark tokens
+    (torch scaled_dot_product_attention); the log-sum-exps must add up to the dense one."""
+    import torch.nn.functional as F
+    torch.manual_seed(17)
+    B, S = 1, 64
+    N = L // S
+    q = (torch.randn(B, L, HQ, D, device=dev) * 0.5).bfloat16()
+    k = (torch.randn(B, L, H, D, device=dev) * 0.5).bfloat16()
+    v = torch.randn(B, L, H, D, device=dev).bfloat16()
+    swa_o, lse_swa = pkg.flex_attn_tl(q, k, v, W, S, mask_lmk=True)
+    log_z = pkg.exact_chunk_log_z_tl(q, k, chunk_size=S, window_size=W, mask_lmk=True)
+    t = torch.arange(L, device=dev)
+    lim = torch.div(t - W + 1, S, rounding_mode="floor").clamp_min(0)  # fully remote chunks per query
+    idx = torch.arange(N, device=dev).view(1, 1, 1, N).expand(B, L, H, N)
+    idx = torch.where(idx < lim.view(1, L, 1, 1), idx, torch.full_like(idx, -1)).to(torch.int32).contiguous()
+    wts = torch.softmax(torch.cat([log_z, lse_swa.unsqueeze(-1)], -1), -1)
+    o_sparse = pkg.HiLS_block_M_head(q, k, v, wts.bfloat16(), idx, block_size=S, is_training=False)
+    o = o_sparse.float() + swa_o.float() * wts[..., N].bfloat16().float().unsqueeze(-1)
+    keep = (t.view(1, L) <= t.view(L, 1)) & (((t + 1) % S) != 0).view(1, L)
+    G = HQ // H
+    qf, kf, vf = q.float().transpose(1, 2), k.float().repeat_interleave(G, 2).transpose(1, 2), \
+        v.float().repeat_interleave(G, 2).transpose(1, 2)
+    dense = F.scaled_dot_product_attention(qf, kf, vf, attn_mask=keep).transpose(1, 2)
+    row_ok = keep.any(-1)  # query 63 with window 1 ... sees nothing but earlier chunks: still fine
+    assert_close_bf16(o[:, row_ok].cpu(), dense[:, row_ok].cpu(), "local + remote == dense", max_abs=2e-2,
+                      rel_l2=1.5e-2)
+    s = torch.einsum("bhid,bhjd->bhij", qf, kf) / D ** 0.5
+    full_lse = torch.logsumexp(s.masked_fill(~keep, float("-inf")), -1).transpose(1, 2)
+    total = torch.logaddexp(torch.logsumexp(log_z, -1), lse_swa)
+    fin = torch.isfinite(full_lse)
+    assert (total[fin] - full_lse[fin]).abs().max().item() < 2e-3
