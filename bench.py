@@ -329,6 +329,15 @@ def bench_ops(pkg, dev, iters=3):
         t = timed(lambda: pkg.HSA(q, k, v, w, idx, 1.0, 64, 1 / 8.0))
     out["hsa_fwd"] = {"workload": "N2 L4096 hq16/hkv4 D64 top16 q_block16", "ms": t,
                       "tflops": 4.0 * D * 64 * HQ * Nb * L * K / (t * 1e-3) / 1e12}
+    qg, kg, vg, wg = (x.clone().requires_grad_() for x in (q, k, v, w))
+    d_o = gpu_randn((Nb, L, HQ, D), gen, dev)
+
+    def hsa_fb():
+        for x in (qg, kg, vg, wg):
+            x.grad = None
+        pkg.HSA(qg, kg, vg, wg, idx, 1.0, 64, 1 / 8.0).backward(d_o)
+
+    out["hsa_fwd_bwd"] = {"workload": "same", "ms": timed(hsa_fb)}
     return out
 
 

@@ -610,12 +610,14 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
 // ---------------------------------------------------------------------------
 static size_t bw_round(size_t n) { return (n + 255) & ~(size_t)255; }
 
+// sm_n (an extra term in every chunk's softmax denominator) reaches the backward only through
+// the saved per-chunk LSE, so any sm_n >= 0 is covered.
 bool hils_bw_covers(int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S, int q_block, int WH,
                     float sm_n, const float* slope) {
   if (H <= 0 || HQ % H != 0) return false;
   const int G = HQ / H;
   return S == BW_S && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) &&
-         (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) && q_block == 1 && WH == HQ && sm_n == 0.f &&
+         (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) && q_block == 1 && WH == HQ && sm_n >= 0.f &&
          slope == nullptr && Lkv >= S && K <= 256 && L < (1 << 24) && Lkv / S <= 12288;
 }
 
