@@ -1233,7 +1233,8 @@ __global__ void __launch_bounds__(TOPK_R_THREADS)
 topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                 const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
                 bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
-                float* __restrict__ sel_logits_out, int L, int N, int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
+                float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
+                int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
                 float sm_scale) {
   constexpr int LR = D / 8, TPI = 64 / LR;
   constexpr int GI = 8;          // load instructions per register buffer
@@ -1412,6 +1413,26 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     const float val = (kk < nc) ? logit_s[g * NP + sh.cand_i[0][kk]] : HILS_NEG_INF;
     scores[(row * G + g) * (long)topk + kk] = f2bf(val);
   }
+  // optional: the layer's inter-chunk softmax over [scores (as bf16), lse_swa], one wavefront per head
+  if (weights_out && wave < G) {
+    const int g = wave;
+    float lse_g = swa[0];
+#pragma unroll
+    for (int g2 = 1; g2 < GMAX; ++g2) lse_g = (g == g2) ? swa[g2] : lse_g;
+    float x = HILS_NEG_INF;
+    if (lane < topk && lane < nc) x = bf2f(f2bf(logit_s[g * NP + sh.cand_i[0][lane]]));
+    const float m = fmaxf(wave_max_f(x), lse_g);
+    bf16_t* wrow = weights_out + (row * G + g) * (long)(topk + 1);
+    if (m == HILS_NEG_INF) {  // every logit -inf: NaN row, as a softmax gives
+      if (lane <= topk) wrow[lane] = 0x7fc0;
+    } else {
+      const float e = (x == HILS_NEG_INF) ? 0.f : __expf(x - m);
+      const float el = __expf(lse_g - m);
+      const float inv = 1.f / (wave_sum_f(e) + el);
+      if (lane < topk) wrow[lane] = f2bf(e * inv);
+      if (lane == 0) wrow[topk] = f2bf(el * inv);
+    }
+  }
 }
 
 // rows = (query, KV head) pairs; the row kernel wants about one row per compute unit
@@ -1421,7 +1442,7 @@ static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool pla
 }
 
 static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, int32_t* indices,
-                        void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv, int G, int D,
+                        void* scores, float* lse_total, float* sel_logits, void* weights, int B, int L, int N, int h_kv, int G, int D,
                         int topk, int block_size, int window_size, int causal, int q_offset,
                         float sm_scale, hipStream_t st) {
   const long rows = (long)B * L * h_kv;
@@ -1441,8 +1462,8 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, i
     }                                                                                            \
     hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(TOPK_R_THREADS), smem, st,               \
                        (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, indices, (bf16_t*)scores, \
-                       lse_total, sel_logits, L, N, NP, h_kv, G, topk, block_size, window_size,  \
-                       causal, q_offset, sm_scale);                                                    \
+                       lse_total, sel_logits, (bf16_t*)weights, L, N, NP, h_kv, G, topk,         \
+                       block_size, window_size, causal, q_offset, sm_scale);                                                    \
   } while (0)
   if (D == 64) TOPK_ROW_CALL(64); else TOPK_ROW_CALL(128);
 #undef TOPK_ROW_CALL
@@ -1510,12 +1531,13 @@ static int topk_fwd_split(const void* q, const void* lmks, const float* lse_swa,
   return HILS_OK;
 }
 
-extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_swa,
-                             const float* bias, const float* gumbel, const int32_t* drop_mask,
-                             int32_t* indices, void* scores, float* lse_total, float* sel_logits,
-                             void* workspace, int B, int L, int N, int h_kv, int G, int D, int topk,
-                             int block_size, int window_size, int causal, int q_offset,
-                             int per_qhead, float sm_scale, void* stream) {
+// weights_fused: the row kernel also writes the inter-chunk softmax (set to 1 when it did)
+static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
+                         const float* bias, const float* gumbel, const int32_t* drop_mask,
+                         int32_t* indices, void* scores, float* lse_total, float* sel_logits,
+                         void* workspace, void* weights, int* weights_fused, int B, int L, int N,
+                         int h_kv, int G, int D, int topk, int block_size, int window_size,
+                         int causal, int q_offset, int per_qhead, float sm_scale, void* stream) {
   HILS_REQUIRE(q && lmks && lse_swa && indices && scores, "hils_topk_fwd: null pointer");
   HILS_REQUIRE(B > 0 && L > 0 && N > 0 && h_kv > 0 && G > 0 && D > 0, "hils_topk_fwd: sizes must be positive");
   HILS_REQUIRE(topk >= 1 && topk <= TOPK_MAXK, "hils_topk_fwd: topk (%d) must be in 1..%d", topk, TOPK_MAXK);
@@ -1525,7 +1547,8 @@ extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_s
   hipStream_t st = (hipStream_t)stream;
   if (topk_use_split(B, L, N, h_kv) &&
       topk_use_row((long)B * L * h_kv, N, G, D, per_qhead, !bias && !gumbel && !drop_mask)) {
-    if (int rc2 = topk_fwd_row(q, lmks, lse_swa, indices, scores, lse_total, sel_logits, B, L, N, h_kv, G, D, topk,
+    *weights_fused = weights != nullptr;
+    if (int rc2 = topk_fwd_row(q, lmks, lse_swa, indices, scores, lse_total, sel_logits, weights, B, L, N, h_kv, G, D, topk,
                                block_size, window_size, causal, q_offset, sm_scale, st))
       return rc2;
     HILS_CHECK_LAUNCH("hils_topk_fwd");
@@ -1589,6 +1612,35 @@ extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_s
   if (rc) return rc;
   HILS_CHECK_LAUNCH("hils_topk_fwd");
   return HILS_OK;
+}
+
+extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_swa,
+                             const float* bias, const float* gumbel, const int32_t* drop_mask,
+                             int32_t* indices, void* scores, float* lse_total, float* sel_logits,
+                             void* workspace, int B, int L, int N, int h_kv, int G, int D, int topk,
+                             int block_size, int window_size, int causal, int q_offset,
+                             int per_qhead, float sm_scale, void* stream) {
+  int fused = 0;
+  return topk_fwd_impl(q, lmks, lse_swa, bias, gumbel, drop_mask, indices, scores, lse_total, sel_logits,
+                       workspace, nullptr, &fused, B, L, N, h_kv, G, D, topk, block_size, window_size,
+                       causal, q_offset, per_qhead, sm_scale, stream);
+}
+
+extern "C" int hils_topk_fwd_weights(const void* q, const void* lmks, const float* lse_swa,
+                                     const float* bias, const float* gumbel, const int32_t* drop_mask,
+                                     int32_t* indices, void* scores, void* weights, void* workspace,
+                                     int B, int L, int N, int h_kv, int G, int D, int topk,
+                                     int block_size, int window_size, int causal, int q_offset,
+                                     int per_qhead, float sm_scale, void* stream) {
+  HILS_REQUIRE(weights, "hils_topk_fwd_weights: null pointer");
+  int fused = 0;
+  if (int rc = topk_fwd_impl(q, lmks, lse_swa, bias, gumbel, drop_mask, indices, scores, nullptr, nullptr,
+                             workspace, weights, &fused, B, L, N, h_kv, G, D, topk, block_size,
+                             window_size, causal, q_offset, per_qhead, sm_scale, stream))
+    return rc;
+  if (fused) return HILS_OK;
+  return hils_chunk_weights(scores, lse_swa, 0, nullptr, nullptr, weights, B, L, h_kv * G, h_kv, N, topk, 0,
+                            stream);
 }
 
 // ---------------------------------------------------------------------------

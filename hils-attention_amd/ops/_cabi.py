@@ -23,6 +23,7 @@ SIGNATURES = {
     "hils_attn_pool_fwd": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
     "hils_attn_pool_bwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
     "hils_topk_fwd": [_P] * 11 + [_I] * 12 + [_F, _P],
+    "hils_topk_fwd_weights": [_P] * 10 + [_I] * 12 + [_F, _P],
     "hils_topk_bwd": [_P] * 7 + [_I] * 8 + [_F, _P],
     "hils_sparse_attn_fwd": [_P] * 9 + [_I] * 13 + [_F, _I, _F, _P],
     "hils_pack_kv_chunks": [_P, _P, _P, _I, _I, _I, _I, _I, _P],

@@ -38,3 +38,33 @@ def chunk_weights(scores, lse_swa, prior_b=None, indices=None, enable_softmax1=F
                int(lse.dtype == torch.bfloat16), _cabi.ptr(pb),
                _cabi.ptr(idx), _cabi.ptr(out), B, L, HQ, H, N, K, int(bool(enable_softmax1)))
     return out
+
+
+def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causal=True, q_offset=0,
+                       sm_scale=None):
+    """Inference: ``online_softmax_topk_head`` (shared chunk keys, no bias / Gumbel / drop mask)
+    followed by ``chunk_weights`` in one call, for the serving loop.  q (B,L,h_q,D) bf16, lmks
+    (B,N,h_kv,D) bf16, lse_swa (B,L,h_q) -> indices (B,L,h_kv,topk) int32, scores (B,L,h_q,topk)
+    bf16, weights (B,L,h_q,topk+1) bf16.  With about one (query, KV head) row per compute unit
+    the selection kernel writes the weights itself; otherwise two kernels run."""
+    import math
+    _cabi.require_gpu_bf16("topk_chunk_weights", q, lmks)
+    if torch.is_grad_enabled() and (q.requires_grad or lmks.requires_grad or lse_swa.requires_grad):
+        raise RuntimeError("topk_chunk_weights is forward-only")
+    B, L, h_q, D = q.shape
+    N, h_kv = lmks.shape[1], lmks.shape[2]
+    assert lmks.shape[0] == B and lmks.shape[3] == D
+    assert h_q % h_kv == 0, f"h_q ({h_q}) must be divisible by h_kv ({h_kv})"
+    G = h_q // h_kv
+    scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(D)
+    dev = q.device
+    lse = lse_swa.reshape(B, L, h_q).float().contiguous()
+    indices = torch.empty((B, L, h_kv, topk), dtype=torch.int32, device=dev)
+    scores = torch.empty((B, L, h_q, topk), dtype=q.dtype, device=dev)
+    weights = torch.empty((B, L, h_q, topk + 1), dtype=q.dtype, device=dev)
+    ws = _cabi.topk_fwd_workspace(dev, B, L, N, h_kv, G)
+    _cabi.call("hils_topk_fwd_weights", _cabi.ptr(q.contiguous()), _cabi.ptr(lmks.contiguous()),
+               _cabi.ptr(lse), None, None, None, _cabi.ptr(indices), _cabi.ptr(scores),
+               _cabi.ptr(weights), _cabi.ptr(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),
+               int(window_size), int(bool(is_causal)), int(q_offset), 0, scale)
+    return indices, scores, weights

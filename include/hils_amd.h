@@ -74,6 +74,18 @@ int hils_topk_fwd(const void* q, const void* lmks, const float* lse_swa, const f
                   int h_kv, int G, int D, int topk, int block_size, int window_size, int causal,
                   int q_offset, int per_qhead, float sm_scale, void* stream);
 
+/* hils_topk_fwd plus the layer's inter-chunk softmax in the same call (inference): also writes
+ * weights (B,L,h_kv*G,topk+1) bf16 = softmax over [scores (as bf16), lse_swa], the K+1-way
+ * softmax of models/FlashHiLS/hils_attention.py:604-610 without prior bias (what
+ * hils_chunk_weights computes from these scores).  With about one (query, KV head) row per
+ * compute unit the selection kernel writes them itself; otherwise hils_chunk_weights runs on the
+ * same stream.  No lse_total / sel_logits outputs. */
+int hils_topk_fwd_weights(const void* q, const void* lmks, const float* lse_swa, const float* bias,
+                          const float* gumbel, const int32_t* drop_mask, int32_t* indices,
+                          void* scores, void* weights, void* workspace, int B, int L, int N, int h_kv,
+                          int G, int D, int topk, int block_size, int window_size, int causal,
+                          int q_offset, int per_qhead, float sm_scale, void* stream);
+
 /* Sparse backward of the score gather.  Replaces the dense scatter + two torch.bmm of
  * SoftmaxTopKMaxPoolingFusedFn.backward (ops/topk_head_softmax.py:1040-1092).
  * g_scores (B,L,h_kv,G,topk) bf16 -> dq (B,L,h_kv,G,D) bf16 (written),

@@ -64,3 +64,23 @@ def _chunk_weights_case(pkg, orc, dev, K):
     assert torch.equal(w32, pkg.chunk_weights(scores.to(dev), lse.to(dev)))
     with pytest.raises(RuntimeError):
         pkg.chunk_weights(scores.to(dev).requires_grad_(), lse.to(dev))
+
+
+@pytest.mark.parametrize("B,L,N,HQ,H,D,K,off", [(32, 1, 2048, 32, 8, 128, 32, 2048 * 64 - 1),
+                                                (13, 1, 500, 8, 8, 64, 16, 300 * 64),
+                                                (2, 3, 700, 8, 2, 128, 8, 700 * 64 - 3)])
+def test_topk_with_fused_weights_matches_two_calls(pkg, dev, B, L, N, HQ, H, D, K, off):
+    """One call for selection + inter-chunk softmax (the selection kernel writes the weights when
+    it runs one workgroup per row, else a second kernel) against the two separate operators."""
+    note(f"topk+weights B{B} L{L} N{N} HQ{HQ} H{H} D{D} K{K}")
+    gen = torch.Generator().manual_seed(77)
+    q = torch.randn(B, L, HQ, D, generator=gen).bfloat16().to(dev)
+    lmk = torch.randn(B, N, H, D, generator=gen).bfloat16().to(dev)
+    lse = (torch.randn(B, L, HQ, generator=gen) * 5 + 10).to(dev)
+    idx0, sc0 = pkg.online_softmax_topk_head(q, lmk, lse, K, 64, 1, q_offset=off, is_training=False)
+    w0 = pkg.chunk_weights(sc0, lse)
+    idx1, sc1, w1 = pkg.topk_chunk_weights(q, lmk, lse, K, 64, 1, q_offset=off)
+    assert torch.equal(idx0, idx1) and torch.equal(sc0, sc1)
+    assert w1.shape == w0.shape and w1.dtype == torch.bfloat16
+    assert (w1.float() - w0.float()).abs().max().item() <= 4e-3  # one bf16 step at weights below 1
+    assert (w1.float().sum(-1) - 1).abs().max().item() < 2e-2
