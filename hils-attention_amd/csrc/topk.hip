@@ -516,7 +516,32 @@ __device__ __forceinline__ float row_max16(float x) {
   return x;
 }
 
-template <int GMAX, int KS, bool PLAIN>
+// Chunk keys of a (batch, KV head) in the register order of the MFMA B operand: block of 16
+// chunks x k-step x lane (chunk = lane & 15, 8 features from 8 * (lane >> 4)) x 8 bf16, so that a
+// wavefront's operand load is one contiguous 1 KiB burst (from the token-major tensor the 16
+// chunk rows of a block lie 2*h_kv*D bytes apart and every lane touches its own 64-byte segment).
+// Chunks past N are zero.  One thread per 16-byte piece.
+__global__ void __launch_bounds__(256)
+topk_pack_lmk_kernel(const bf16_t* __restrict__ lmks, uint4* __restrict__ packed, int N, int h_kv,
+                     int D, int nblk16, long total) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int KS = D / 32;
+  const int lane = (int)(i & 63);
+  long r = i >> 6;
+  const int ks = (int)(r % KS);
+  r /= KS;
+  const int blk = (int)(r % nblk16);
+  r /= nblk16;
+  const int hk = (int)(r % h_kv);
+  const long b = r / h_kv;
+  const int c = blk * 16 + (lane & 15);
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (c < N) v = *(const uint4*)(lmks + ((b * N + c) * (long)h_kv + hk) * D + ks * 32 + (lane >> 4) * 8);
+  packed[i] = v;
+}
+
+template <int GMAX, int KS, bool PLAIN, bool PACKED>
 __global__ void __launch_bounds__(64)
 topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                      const float* __restrict__ lse_swa, const float* __restrict__ bias,
@@ -524,8 +549,10 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
                      int32_t* __restrict__ indices, bf16_t* __restrict__ scores,
                      float* __restrict__ lse_total_out, float* __restrict__ sel_logits_out,
                      int L, int N, int h_kv, int G, int topk, int block_size, int window_size,
-                     int causal, int q_offset, float sm_scale, int segw, int pool_floats) {
+                     int causal, int q_offset, float sm_scale, int segw, int pool_floats,
+                     const uint4* __restrict__ lmk_packed) {
   // PLAIN: no bias, Gumbel noise, drop mask or logit export (the inference path)
+  // PACKED: the chunk keys of the two passes come from lmk_packed (topk_pack_lmk_kernel's order)
   constexpr int D = KS * 32;
   constexpr int QPT = 16 / GMAX;            // queries per 16-row tile
   constexpr int NT = (GMAX == 4) ? 2 : 1;   // tiles per wavefront
@@ -582,7 +609,14 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
   // chunk keys as B operands; rows beyond N are read from row N-1 and masked by the caller
   const long bstride = (long)h_kv * D;  // elements between consecutive chunk keys
   const bf16_t* bbase = lmks + (b * N * (long)h_kv + hk) * D + j * 8;
+  const uint4* pbase = PACKED ? lmk_packed + ((b * h_kv + hk) * (long)((N + 15) / 16) * KS) * 64 + lane : nullptr;
   auto load_b = [&](int blk, uint4* dst) {
+    if (PACKED) {
+      const int bc = blk < (N + 15) / 16 ? blk : (N + 15) / 16 - 1;  // a prefetch may run past the end
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) dst[ks] = pbase[((long)bc * KS + ks) * 64];
+      return;
+    }
     int c = blk * 16 + col;
     c = c < N ? c : N - 1;
     const bf16_t* p = bbase + c * bstride;
@@ -614,6 +648,11 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
   const char* ubase = (const char*)lmks + ((b * N * (long)h_kv + hk) * D) * 2;
   const uint32_t lane_off = (uint32_t)((col * bstride + j * 8) * 2);
   auto load_b_full = [&](int blk, uint4* dst) {
+    if (PACKED) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) dst[ks] = pbase[((long)blk * KS + ks) * 64];
+      return;
+    }
     const char* p = ubase + (long)blk * (32 * bstride);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) dst[ks] = *(const uint4*)(p + lane_off + ks * 64);
@@ -1484,7 +1523,9 @@ static bool topk_use_split(int B, int L, int N, int h_kv) {
 }
 
 extern "C" size_t hils_topk_fwd_workspace(int B, int L, int N, int h_kv, int G) {
-  if (!topk_use_split(B, L, N, h_kv)) return 0;
+  // many queries: room for the chunk keys repacked into MFMA operand order (head dim up to 128)
+  if (!topk_use_split(B, L, N, h_kv))
+    return G <= 4 ? (size_t)B * h_kv * ((N + 15) / 16) * 16 * 128 * sizeof(bf16_t) : 0;
   return (size_t)B * L * h_kv * G * N * sizeof(float);
 }
 
@@ -1572,18 +1613,27 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
     pool_floats = (pool_floats + 3) & ~3;
     const size_t smem = sizeof(float) * ((size_t)pool_floats + 128 + (size_t)2 * NQ * topk);
     dim3 grid_r((L + NQ - 1) / NQ, h_kv, B);
+    // with a workspace the chunk keys are first repacked into MFMA operand order
+    const uint4* packed = nullptr;
+    if (workspace) {
+      const int nblk16 = (N + 15) / 16;
+      const long total = (long)B * h_kv * nblk16 * (D / 32) * 64;
+      hipLaunchKernelGGL(topk_pack_lmk_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                         (const bf16_t*)lmks, (uint4*)workspace, N, h_kv, D, nblk16, total);
+      packed = (const uint4*)workspace;
+    }
+#define HILS_TOPK_ROWS_P(G_, KS_, PL_, PK_)                                                         \
+  hipLaunchKernelGGL((topk_fwd_rows_kernel<G_, KS_, PL_, PK_>), grid_r, dim3(64), smem, st,         \
+                     (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, gumbel, drop_mask,       \
+                     indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,          \
+                     block_size, window_size, causal, q_offset, sm_scale, segw, pool_floats, packed)
 #define HILS_TOPK_ROWS(G_, KS_)                                                                     \
   do {                                                                                             \
-    if (plain)                                                                                     \
-      hipLaunchKernelGGL((topk_fwd_rows_kernel<G_, KS_, true>), grid_r, dim3(64), smem, st,        \
-                         (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, gumbel, drop_mask,  \
-                         indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,     \
-                         block_size, window_size, causal, q_offset, sm_scale, segw, pool_floats);  \
-    else                                                                                           \
-      hipLaunchKernelGGL((topk_fwd_rows_kernel<G_, KS_, false>), grid_r, dim3(64), smem, st,       \
-                         (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, gumbel, drop_mask,  \
-                         indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,     \
-                         block_size, window_size, causal, q_offset, sm_scale, segw, pool_floats);  \
+    if (plain) {                                                                                   \
+      if (packed) HILS_TOPK_ROWS_P(G_, KS_, true, true); else HILS_TOPK_ROWS_P(G_, KS_, true, false);   \
+    } else {                                                                                       \
+      if (packed) HILS_TOPK_ROWS_P(G_, KS_, false, true); else HILS_TOPK_ROWS_P(G_, KS_, false, false); \
+    }                                                                                              \
   } while (0)
     const bool plain = !bias && !gumbel && !drop_mask && !sel_logits;
     if (G == 1) {
@@ -1593,6 +1643,7 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
     } else {
       if (D == 64) HILS_TOPK_ROWS(4, 2); else HILS_TOPK_ROWS(4, 4);
     }
+#undef HILS_TOPK_ROWS_P
 #undef HILS_TOPK_ROWS
     HILS_CHECK_LAUNCH("hils_topk_fwd");
     return HILS_OK;

@@ -66,7 +66,9 @@ int hils_attn_pool_bwd(const void* mu_q, const void* k, const float* p, const fl
  * (window > 0) / floor((t+q_offset)/block) (window <= 0).  Ties: lower index wins.
  * workspace: device scratch of hils_topk_fwd_workspace(...) bytes or NULL.  With few queries
  * (decode) and a workspace, the logits are spread over many workgroups and parked there
- * before a separate selection kernel; otherwise one fused kernel runs. */
+ * before a separate selection kernel (or one workgroup per (query, KV head) keeps them in LDS
+ * and needs no scratch); with many queries the chunk keys are first repacked there into MFMA
+ * operand order.  Without a workspace one fused kernel reads the chunk keys as they are. */
 size_t hils_topk_fwd_workspace(int B, int L, int N, int h_kv, int G);
 int hils_topk_fwd(const void* q, const void* lmks, const float* lse_swa, const float* bias,
                   const float* gumbel, const int32_t* drop_mask, int32_t* indices, void* scores,
