@@ -542,7 +542,7 @@ topk_pack_lmk_kernel(const bf16_t* __restrict__ lmks, uint4* __restrict__ packed
 }
 
 template <int GMAX, int KS, bool PLAIN, bool PACKED>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4)))
 topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                      const float* __restrict__ lse_swa, const float* __restrict__ bias,
                      const float* __restrict__ gumbel, const int32_t* __restrict__ drop_mask,
@@ -897,7 +897,7 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
 
 static int topk_rows_segw(int N) {
   const int n16 = (N + 15) / 16 * 16;
-  return n16 < TOPK_NSEG ? n16 : TOPK_NSEG;
+  return n16 < 256 ? n16 : 256;
 }
 
 template <int GMAX>
