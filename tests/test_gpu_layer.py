@@ -84,3 +84,44 @@ def test_topk_with_fused_weights_matches_two_calls(pkg, dev, B, L, N, HQ, H, D, 
     assert w1.shape == w0.shape and w1.dtype == torch.bfloat16
     assert (w1.float() - w0.float()).abs().max().item() <= 4e-3  # one bf16 step at weights below 1
     assert (w1.float().sum(-1) - 1).abs().max().item() < 2e-2
+
+
+def test_decode_step_replays_as_hip_graph(pkg, orc, dev):
+    """The decode step (selection + inter-chunk softmax, then sparse attention) captured as one HIP
+    graph: every replay, with eager work and synchronisations in between and with new inputs
+    copied into the captured buffers, must reproduce the eager result bit for bit."""
+    note("decode step as a HIP graph")
+    B, Lkv, HQ, H, D, S, K = 32, 4096, 32, 8, 128, 64, 16
+    gen = torch.Generator().manual_seed(91)
+    q = torch.randn(B, 1, HQ, D, generator=gen).bfloat16().to(dev)
+    kc = torch.randn(B, Lkv, H, D, generator=gen).bfloat16().to(dev)
+    vc = torch.randn(B, Lkv, H, D, generator=gen).bfloat16().to(dev)
+    lse = (torch.randn(B, 1, HQ, generator=gen) * 2 + 3).to(dev)
+    lmk = pkg.chunk_mean_pool(kc, S)
+
+    def step():
+        idx, scores, w = pkg.topk_chunk_weights(q, lmk, lse, K, S, 1, q_offset=Lkv - 1)
+        return idx, w, pkg.HiLS_block_M_head(q, kc, vc, w, idx, block_size=S, is_training=False)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_idx, g_w, g_o = step()
+    for it in range(4):
+        if it:
+            q.copy_(torch.randn(B, 1, HQ, D, generator=gen).bfloat16())  # new query, same buffers
+        e_idx, e_w, e_o = step()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_idx, e_idx), f"replay {it}: indices differ"
+        assert torch.equal(g_w, e_w), f"replay {it}: weights differ"
+        assert torch.equal(g_o, e_o), f"replay {it}: outputs differ"
+    # and the eager result itself against the oracle
+    ref = orc.sparse_attn(q.cpu(), kc.cpu(), vc.cpu(), e_w.cpu(), e_idx.cpu(), chunk_size=S)
+    assert_close_bf16(e_o, ref, "decode step output")
