@@ -126,6 +126,41 @@ def bench_prefill(pkg, dev, steps, warmup):
     return sec, per, roof, cfg, data
 
 
+def bench_config2(pkg, dev, iters=5):
+    """Config 2: B4 L8192, 16 heads MHA, D64, top-32: the same forward step as the headline
+    (mean pool -> top-k -> inter-chunk softmax -> K/V packing -> sparse attention)."""
+    from hils_attention_amd.ops import hils_fwd_bwd_head as attn_mod
+    B, L, HQ, H, D, S, K, W = 4, 8192, 16, 16, 64, 64, 32, 1
+    gen = torch.Generator(device=dev).manual_seed(1002)
+    q = gpu_randn((B, L, HQ, D), gen, dev)
+    k = gpu_randn((B, L, H, D), gen, dev)
+    v = gpu_randn((B, L, H, D), gen, dev)
+    lse_swa = swa_lse_current_chunk(q, k, S).bfloat16()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    t_all = t_attn = 0.0
+    n_sel = 0
+    for it in range(iters + 1):
+        ev[0].record()
+        lmk = pkg.chunk_mean_pool(k, S)
+        idx, scores = pkg.online_softmax_topk_head(q, lmk, lse_swa, K, S, W, is_training=False)
+        w = pkg.chunk_weights(scores, lse_swa)
+        ws = attn_mod.prepare_kv_workspace(L, k, v, HQ, K, S)
+        ev[1].record()
+        pkg.HiLS_block_M_head(q, k, v, w, idx, block_size=S, is_training=False, kv_workspace=ws)
+        ev[2].record()
+        torch.cuda.synchronize()
+        if it:  # the first pass warms up
+            t_all += ev[0].elapsed_time(ev[2])
+            t_attn += ev[1].elapsed_time(ev[2])
+        n_sel = int((idx >= 0).sum().item())
+    t_all /= iters
+    t_attn /= iters
+    flops = 4.0 * D * S * (HQ // H) * n_sel
+    return {"workload": "prefill_fwd B4 L8192 h16/16 D64 chunk64 top32 causal (config 2)",
+            "ms_per_step": t_all, "tokens_per_s": B * L / (t_all * 1e-3), "attn_ms": t_attn,
+            "attn_mfma_frac": flops / (t_attn * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS}
+
+
 def bench_decode(pkg, dev, steps, warmup):
     B, Lkv, HQ, H, D, S, K, W = 32, 131072, 32, 8, 128, 64, 32, 1
     N = Lkv // S
@@ -423,6 +458,7 @@ def main():
         line["decode_kernel_ms"] = dper
         line["roofline_decode"] = droof
     if not args.no_train:
+        line["config2_fwd"] = bench_config2(pkg, dev)
         line["train_fwd_bwd"] = bench_train(pkg, dev)
     if not args.no_ops:
         line["ops"] = bench_ops(pkg, dev)
