@@ -68,7 +68,8 @@ def _chunk_weights_case(pkg, orc, dev, K):
 
 @pytest.mark.parametrize("B,L,N,HQ,H,D,K,off", [(32, 1, 2048, 32, 8, 128, 32, 2048 * 64 - 1),
                                                 (13, 1, 500, 8, 8, 64, 16, 300 * 64),
-                                                (2, 3, 700, 8, 2, 128, 8, 700 * 64 - 3)])
+                                                (2, 3, 700, 8, 2, 128, 8, 700 * 64 - 3),
+                                                (128, 1, 256, 4, 1, 64, 8, 64 * 2 + 1)])
 def test_topk_with_fused_weights_matches_two_calls(pkg, dev, B, L, N, HQ, H, D, K, off):
     """One call for selection + inter-chunk softmax (the selection kernel writes the weights when
     it runs one workgroup per row, else a second kernel) against the two separate operators."""
@@ -84,6 +85,7 @@ def test_topk_with_fused_weights_matches_two_calls(pkg, dev, B, L, N, HQ, H, D, 
     assert w1.shape == w0.shape and w1.dtype == torch.bfloat16
     assert (w1.float() - w0.float()).abs().max().item() <= 4e-3  # one bf16 step at weights below 1
     assert (w1.float().sum(-1) - 1).abs().max().item() < 2e-2
+    assert torch.equal(w1[..., :K] == 0, w0[..., :K] == 0)  # empty slots carry exactly zero weight
 
 
 def test_decode_step_replays_as_hip_graph(pkg, orc, dev):
