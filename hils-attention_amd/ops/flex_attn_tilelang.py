@@ -69,3 +69,16 @@ def flex_attn_tl(q, k, v, window_size: int, chunk_size: int, training: bool = Tr
         raise ValueError("flex_attn_tl only supports non-zero kv_start in inference (training=False)")
     return _FlexAttnTL.apply(q, k, v, int(window_size), int(chunk_size), bool(mask_lmk),
                              bool(expand_to_chunk), not training, sm_scale, int(kv_start))
+
+
+def flex_attn_tl_two_phase(q, k, v, window_size: int, chunk_size: int, training: bool = True,
+                           mask_lmk: bool = True, expand_to_chunk: bool = True, sm_scale: float = None,
+                           kv_start: int = 0):
+    """Same as ``flex_attn_tl`` (ops/flex_attn_tilelang.py:1313-1349 of the reference): the
+    reference's variant with an atomic-free backward of two kernels (dQ over query blocks, dK/dV
+    over key blocks, bf16 outputs written directly), which is how the backward here always works."""
+    if training and int(kv_start) != 0:
+        raise ValueError(
+            "flex_attn_tl_two_phase only supports non-zero kv_start in inference (training=False)")
+    return flex_attn_tl(q, k, v, window_size, chunk_size, training=training, mask_lmk=mask_lmk,
+                        expand_to_chunk=expand_to_chunk, sm_scale=sm_scale, kv_start=kv_start)

@@ -103,6 +103,16 @@ def test_swa_backward_only_through_o(pkg, orc, dev):
     assert_close_bf16(vd.grad, vf.grad, "swa dv (o only)")
 
 
+def test_swa_two_phase_name_is_the_same_operator(pkg, dev):
+    q = torch.randn(1, 130, 4, 64, device=dev).bfloat16()
+    k = torch.randn(1, 130, 2, 64, device=dev).bfloat16()
+    a = pkg.flex_attn_tl(q, k, k, 40, 64)
+    b = pkg.flex_attn_tl_two_phase(q, k, k, 40, 64)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    with pytest.raises(ValueError):
+        pkg.flex_attn_tl_two_phase(q, k, k, 40, 64, training=True, kv_start=3)
+
+
 def test_swa_inference_backward_raises_and_argument_errors(pkg, dev):
     q = torch.randn(1, 64, 2, 64, device=dev).bfloat16().requires_grad_()
     o, lse = pkg.flex_attn_tl(q, q.detach(), q.detach(), 16, 64, training=False)
