@@ -350,6 +350,18 @@ def bench_ops(pkg, dev, iters=3):
 
     out["swa_fwd_bwd"] = {"workload": "same", "us": timed(swa_fb) * 1e3}
     del q, k, v, qg, kg, vg, d_o
+    # rotary embedding of q and k: B1 L32768 hq32/hkv8 D128
+    L, HQ, HK, D = 32768, 32, 8, 128
+    q = gpu_randn((1, L, HQ, D), gen, dev)
+    k = gpu_randn((1, L, HK, D), gen, dev)
+    ang = torch.rand(1, L, D // 2, device=dev, generator=gen) * 6.283
+    cos = torch.cat([ang.cos(), ang.cos()], -1).bfloat16()
+    sin = torch.cat([ang.sin(), ang.sin()], -1).bfloat16()
+    with torch.no_grad():
+        t = timed(lambda: pkg.rope_rotary_pos_emb(q, k, cos, sin))
+    out["rope_qk"] = {"workload": "B1 L32768 hq32/hkv8 D128", "us": t * 1e3,
+                      "hbm_gbs": 2 * (q.numel() + k.numel()) * 2 / (t * 1e-3) / 1e9}
+    del q, k, cos, sin, ang
     # HSA: N2 L4096 hq16/hkv4 D64, 16 chunks per block of 16 queries
     Nb, L, HQ, HK, D, K, QX = 2, 4096, 16, 4, 64, 16, 16
     q = gpu_randn((Nb, L, HQ, D), gen, dev)

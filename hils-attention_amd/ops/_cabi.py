@@ -32,6 +32,7 @@ SIGNATURES = {
     "hils_chunk_logz_fwd": [_P, _P, _P] + [_I] * 7 + [_F, _I, _P],
     "hils_chunk_logz_bwd_dq": [_P] * 5 + [_I] * 7 + [_F, _P],
     "hils_chunk_logz_bwd_dk": [_P] * 5 + [_I] * 7 + [_F, _P],
+    "hils_rope": [_P] * 4 + [_I] * 7 + [_F, _P],
     "hils_swa_fwd": [_P] * 5 + [_I] * 12 + [_F, _P],
     "hils_swa_bwd": [_P] * 11 + [_I] * 10 + [_F, _P],
 }

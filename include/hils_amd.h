@@ -203,6 +203,17 @@ int hils_swa_bwd(const void* q, const void* k, const void* v, const void* o, con
                  int B, int L, int HQ, int H, int D, int Dv, int window, int chunk, int mask_lmk,
                  int expand_to_chunk, float sm_scale, void* stream);
 
+/* ---- rotary position embedding ---------------------------------------------------- */
+
+/* Replaces rope_fwd_kernel and single_tensor_rope_kernel (ops/rope_tilelang_fp32.py:19-81,
+ * :96-137).  x, out (B,L,H,D) bf16, D a multiple of 16; with x = (x1, x2) the two halves of a
+ * head vector: out1 = x1*cos[d] - x2*sin[d]*sin_sign, out2 = x2*cos[d'] + x1*sin[d']*sin_sign,
+ * d' = d (lo_only != 0, the two-tensor kernel) or d + D/2 (the single-tensor kernel).  Tables
+ * cos_t, sin_t: (L,D), or (B,L,D) when table_per_batch != 0; fp32 when table_f32 != 0, else bf16.
+ * sin_sign = -1 gives the backward (rotation by the opposite angle). */
+int hils_rope(const void* x, const void* cos_t, const void* sin_t, void* out, int B, int L, int H,
+              int D, int table_per_batch, int table_f32, int lo_only, float sin_sign, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,6 +24,8 @@ reference repository root):
                              :171-193 (the ``sm_n`` denominator term)
 * ``exact_chunk_log_z``    - models/NaiveBSA/naive_bsa_kernel.py:39-118 and the
                              mask of ops/exact_chunk_log_z_tilelang.py:89-107
+* ``rope``                 - ops/rope_tilelang_fp32.py:48-62,125-134 (kernel arithmetic) and
+                             :185-189 (the rotate-half torch formula its tests compare with)
 * ``swa``                  - ops/flex_attn_tilelang.py:1355-1386 (mask definition) and
                              :108-121,155-171 (absolute positions with a cache offset)
 * ``hils_layer_forward``   - models/FlashHiLS/hils_attention.py:536-623 (op order,
@@ -313,6 +315,25 @@ def exact_chunk_log_z(q, k, *, chunk_size: int, window_size: int, sm_scale: Opti
         s = s.masked_fill(masked.view(1, t1 - t0, 1, 1, N, S), NEG_INF)
         out[:, t0:t1] = torch.logsumexp(s, dim=-1).reshape(B, t1 - t0, HQ, N)
     return out
+
+
+# ----------------------------------------------------------------------------
+# rotary position embedding
+# ----------------------------------------------------------------------------
+def rope(x, cos, sin, *, lo_only: bool = False):
+    """Rotate-half RoPE in fp32.  x (B,L,H,D); cos, sin (L,D), (1,L,D) or (B,L,D).
+    out1 = x1*cos[d] - x2*sin[d], out2 = x2*cos[d'] + x1*sin[d'] with d' = d + D/2, or d when
+    ``lo_only`` (ops/rope_tilelang_fp32.py:48-62 two-tensor kernel; :125-134 single-tensor kernel)."""
+    B, L, H, D = x.shape
+    half = D // 2
+    cos, sin = cos.float(), sin.float()
+    if cos.dim() == 2:
+        cos, sin = cos.unsqueeze(0), sin.unsqueeze(0)
+    cos, sin = cos.unsqueeze(2), sin.unsqueeze(2)  # (B or 1, L, 1, D)
+    x1, x2 = x.float()[..., :half], x.float()[..., half:]
+    c1, s1 = cos[..., :half], sin[..., :half]
+    c2, s2 = (c1, s1) if lo_only else (cos[..., half:], sin[..., half:])
+    return torch.cat([x1 * c1 - x2 * s1, x2 * c2 + x1 * s2], dim=-1)
 
 
 # ----------------------------------------------------------------------------

@@ -352,3 +352,32 @@ def test_inter_chunk_softmax(orc):
     assert torch.allclose(w[0, t, hq], torch.softmax(row, 0), atol=1e-6)
     w1 = orc.inter_chunk_softmax(scores, lse, softmax1=True)
     assert w1.shape[-1] == K + 2 and torch.allclose(w1.sum(-1), torch.ones(B, L, HQ))
+
+
+def test_rope_is_a_rotation(orc):
+    """rope == x*cos + rotate_half(x)*sin for tables with equal halves; angle 0 is the identity,
+    90 degrees maps (x1, x2) to (-x2, x1), angles add, pair norms are preserved."""
+    torch.manual_seed(21)
+    B, L, H, D = 2, 5, 3, 8
+    x = torch.randn(B, L, H, D)
+    ang = torch.rand(L, D // 2) * 6.0
+    ang2 = torch.rand(L, D // 2) * 6.0
+    full = lambda a: (torch.cat([a.cos(), a.cos()], -1), torch.cat([a.sin(), a.sin()], -1))
+    cos, sin = full(ang)
+    out = orc.rope(x, cos, sin)
+    rot_half = torch.cat([-x[..., D // 2:], x[..., :D // 2]], -1)
+    assert torch.allclose(out, x * cos.view(1, L, 1, D) + rot_half * sin.view(1, L, 1, D), atol=1e-6)
+    assert torch.allclose(out, orc.rope(x, cos, sin, lo_only=True), atol=0)  # equal halves: same thing
+    z = torch.zeros(L, D // 2)
+    assert torch.equal(orc.rope(x, *full(z)), x)
+    assert torch.allclose(orc.rope(x, *full(z + math.pi / 2)), rot_half, atol=1e-6)
+    assert torch.allclose(orc.rope(out, *full(ang2)), orc.rope(x, *full(ang + ang2)), atol=1e-5)
+    n_in = x[..., :D // 2] ** 2 + x[..., D // 2:] ** 2
+    n_out = out[..., :D // 2] ** 2 + out[..., D // 2:] ** 2
+    assert torch.allclose(n_in, n_out, atol=1e-5)
+    # tables whose halves differ: the single-tensor form uses each half for its own output
+    c, s_ = torch.randn(L, D), torch.randn(L, D)
+    o2 = orc.rope(x, c, s_)
+    t, h, d = 3, 1, 2
+    assert o2[1, t, h, d].item() == pytest.approx((x[1, t, h, d] * c[t, d] - x[1, t, h, d + 4] * s_[t, d]).item(), abs=1e-6)
+    assert o2[1, t, h, d + 4].item() == pytest.approx((x[1, t, h, d + 4] * c[t, d + 4] + x[1, t, h, d] * s_[t, d + 4]).item(), abs=1e-6)
