@@ -1235,10 +1235,8 @@ topk_select_kernel(const float* __restrict__ raw, const float* __restrict__ lse_
 // LSE, pooling, the 16 per-wavefront selections and their merge follow without leaving the
 // workgroup: no scratch in HBM and no second launch.
 // ---------------------------------------------------------------------------
-#define TOPK_R_THREADS 1024
-#define TOPK_R_WAVES 16
+#define TOPK_R_WAVES 16  // most wavefronts of a row workgroup (sizes the shared arrays)
 #define TOPK_R_MAXN 4096
-#define TOPK_R_EPT (TOPK_R_MAXN / TOPK_R_THREADS)
 
 __device__ __forceinline__ float wave_max_f(float x) {
   x = fmaxf(x, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), 0xB1, 0xF, 0xF, false)));
@@ -1267,8 +1265,8 @@ struct TopkRowShared {
   int next_group;
 };
 
-template <int D, int GMAX>
-__global__ void __launch_bounds__(TOPK_R_THREADS)
+template <int D, int GMAX, int NW>
+__global__ void __launch_bounds__(NW * 64)
 topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                 const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
                 bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
@@ -1276,6 +1274,8 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                 int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
                 float sm_scale) {
   constexpr int LR = D / 8, TPI = 64 / LR;
+  constexpr int THREADS = NW * 64;       // NW = 8 or 16 wavefronts
+  constexpr int EPT = TOPK_R_MAXN / THREADS;  // 64-chunk slots of a wavefront's share
   constexpr int GI = 8;          // load instructions per register buffer
   constexpr int KG = GI * TPI;   // chunk keys per buffer
   extern __shared__ float dyn[];
@@ -1294,7 +1294,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   float swa[GMAX];
 #pragma unroll
   for (int g = 0; g < GMAX; ++g) swa[g] = (g < G) ? lse_swa[row * G + g] : 0.f;
-  if (tid == 0) sh.next_group = 2 * TOPK_R_WAVES;
+  if (tid == 0) sh.next_group = 2 * NW;
   __syncthreads();
 
   // ---- phase 1: logits of the visible chunks ----
@@ -1339,7 +1339,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     // drawn group numbers only grow, so the first one past the end ends the wavefront's walk
     const int last = ngroups - 1;
     uint4 ka[GI], kb[GI];
-    int ga = wave, gb = wave + TOPK_R_WAVES;
+    int ga = wave, gb = wave + NW;
     if (ngroups > 0) {
       fetch(ka, ga < last ? ga : last);
       fetch(kb, gb < last ? gb : last);
@@ -1359,16 +1359,16 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   // ---- phase 2: LSE per head.  Wavefront w owns the chunks [w*per, (w+1)*per): the same chunks it
   // selects from later, so its pooled scores never leave the wavefront before the selection. ----
   static_assert(GMAX == 4, "the cross-wavefront reductions carry four heads per float4");
-  const int per = ((N + TOPK_R_WAVES - 1) / TOPK_R_WAVES + 63) & ~63;  // <= 256 = 64 * TOPK_R_EPT
+  const int per = ((N + NW - 1) / NW + 63) & ~63;  // <= 256 = 64 * EPT
   const int cbase = wave * per;
-  float x[GMAX][TOPK_R_EPT];
+  float x[GMAX][EPT];
   {
     float m[GMAX], l[GMAX];
 #pragma unroll
     for (int g = 0; g < GMAX; ++g) {
       m[g] = HILS_NEG_INF;
 #pragma unroll
-      for (int e = 0; e < TOPK_R_EPT; ++e) {
+      for (int e = 0; e < EPT; ++e) {
         const int c = cbase + e * 64 + lane;
         x[g][e] = (g < G && e * 64 < per && c < lim) ? logit_s[g * NP + c] : HILS_NEG_INF;
         m[g] = fmaxf(m[g], x[g][e]);
@@ -1377,7 +1377,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       l[g] = 0.f;
       if (m[g] > HILS_NEG_INF) {
 #pragma unroll
-        for (int e = 0; e < TOPK_R_EPT; ++e) l[g] += __expf(x[g][e] - m[g]);
+        for (int e = 0; e < EPT; ++e) l[g] += __expf(x[g][e] - m[g]);
       }
       l[g] = wave_sum_f(l[g]);
     }
@@ -1390,7 +1390,9 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   float tot[GMAX];
   {
     // every row of 16 lanes combines the 16 (max, sum) pairs: the result is uniform without a broadcast
-    const float4 m4 = sh.red_m[lane & 15], l4 = sh.red_l[lane & 15];
+    const bool has = (lane & 15) < NW;
+    const float4 m4 = has ? sh.red_m[lane & 15] : make_float4(HILS_NEG_INF, HILS_NEG_INF, HILS_NEG_INF, HILS_NEG_INF);
+    const float4 l4 = has ? sh.red_l[lane & 15] : make_float4(0.f, 0.f, 0.f, 0.f);
     const float mw[GMAX] = {m4.x, m4.y, m4.z, m4.w}, lw[GMAX] = {l4.x, l4.y, l4.z, l4.w};
 #pragma unroll
     for (int g = 0; g < GMAX; ++g) {
@@ -1407,7 +1409,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   // ---- phase 3: pooled scores of the own chunks, selection among them, winners (padded to topk
   // entries with -inf) straight into this wavefront's slice of the merge list ----
 #pragma unroll
-  for (int e = 0; e < TOPK_R_EPT; ++e) {
+  for (int e = 0; e < EPT; ++e) {
     const int c = cbase + e * 64 + lane;
     float best = HILS_NEG_INF;
 #pragma unroll
@@ -1424,7 +1426,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     int nc = 0;
     if (cbase < lim) {
       const int ns = (lim - cbase < per) ? lim - cbase : per;
-      nc = wave_select<false, TOPK_R_EPT>(pooled + cbase, ns, cbase, sh.merge_s + wave * topk,
+      nc = wave_select<false, EPT>(pooled + cbase, ns, cbase, sh.merge_s + wave * topk,
                                           sh.merge_i + wave * topk, 0, topk, nullptr, sh.cand_s[wave],
                                           sh.cand_i[wave]);
     }
@@ -1435,7 +1437,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   }
   __syncthreads();
   if (wave == 0) {
-    const int total = TOPK_R_WAVES * topk;
+    const int total = NW * topk;
     int nc = 0;
     for (int p0 = 0; p0 < total; p0 += TOPK_NSEG) {
       const int ns = (total - p0 < TOPK_NSEG) ? total - p0 : TOPK_NSEG;
@@ -1446,8 +1448,8 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   __syncthreads();
   // ---- phase 4: indices (ascending) and the raw scaled scores of the winners ----
   const int nc = sh.ncand[0];
-  for (int kk = tid; kk < topk; kk += TOPK_R_THREADS) indices[row * topk + kk] = (kk < nc) ? sh.cand_i[0][kk] : -1;
-  for (int p = tid; p < topk * G; p += TOPK_R_THREADS) {
+  for (int kk = tid; kk < topk; kk += THREADS) indices[row * topk + kk] = (kk < nc) ? sh.cand_i[0][kk] : -1;
+  for (int p = tid; p < topk * G; p += THREADS) {
     const int g = p / topk, kk = p - g * topk;
     const float val = (kk < nc) ? logit_s[g * NP + sh.cand_i[0][kk]] : HILS_NEG_INF;
     scores[(row * G + g) * (long)topk + kk] = f2bf(val);
@@ -1474,6 +1476,19 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   }
 }
 
+// compute units of the current device, looked up once (keeps the query out of HIP graph capture)
+static int topk_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, v = 0;
+    cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      cus = v;
+  }
+  return cus;
+}
+
 // rows = (query, KV head) pairs; the row kernel wants about one row per compute unit
 static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool plain) {
   return plain && !per_qhead && G <= 4 && (D == 64 || D == 128) && N >= 256 && N <= TOPK_R_MAXN &&
@@ -1487,9 +1502,13 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, i
   const long rows = (long)B * L * h_kv;
   const int NP = (N + 63) & ~63;
   const size_t smem = (size_t)5 * NP * sizeof(float);
-#define TOPK_ROW_CALL(D_)                                                                         \
+  // one round of rows or less: 16 wavefronts per row (the whole compute unit streams one row);
+  // more rows than compute units: 8, so that two workgroups share a unit and one row's selection
+  // overlaps the other row's streaming
+  const bool wide = rows <= topk_cus();
+#define TOPK_ROW_CALL_W(D_, W_)                                                                   \
   do {                                                                                           \
-    auto kern = topk_row_kernel<D_, 4>;                                                          \
+    auto kern = topk_row_kernel<D_, 4, W_>;                                                      \
     static size_t reserved = 48 * 1024;                                                          \
     if (smem > reserved) {                                                                       \
       if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,     \
@@ -1499,27 +1518,24 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, i
       }                                                                                          \
       reserved = smem;                                                                           \
     }                                                                                            \
-    hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(TOPK_R_THREADS), smem, st,               \
+    hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(W_ * 64), smem, st,                      \
                        (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, indices, (bf16_t*)scores, \
                        lse_total, sel_logits, (bf16_t*)weights, L, N, NP, h_kv, G, topk,         \
-                       block_size, window_size, causal, q_offset, sm_scale);                                                    \
+                       block_size, window_size, causal, q_offset, sm_scale);                     \
+  } while (0)
+#define TOPK_ROW_CALL(D_)                                                                        \
+  do {                                                                                           \
+    if (wide) TOPK_ROW_CALL_W(D_, 16); else TOPK_ROW_CALL_W(D_, 8);                              \
   } while (0)
   if (D == 64) TOPK_ROW_CALL(64); else TOPK_ROW_CALL(128);
 #undef TOPK_ROW_CALL
+#undef TOPK_ROW_CALL_W
   return HILS_OK;
 }
 
 static bool topk_use_split(int B, int L, int N, int h_kv) {
-  static int cus = 0;  // looked up once (keeps the query out of HIP graph capture)
-  if (cus == 0) {
-    int dev = 0, v = 0;
-    cus = 256;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      cus = v;
-  }
   const long fused_wgs = (long)B * ((L + TOPK_QT - 1) / TOPK_QT) * h_kv;
-  return fused_wgs < 2L * cus && N >= 256 && N <= 16384;
+  return fused_wgs < 2L * topk_cus() && N >= 256 && N <= 16384;
 }
 
 extern "C" size_t hils_topk_fwd_workspace(int B, int L, int N, int h_kv, int G) {
@@ -1586,7 +1602,9 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
   HILS_REQUIRE(block_size > 0, "hils_topk_fwd: block_size must be positive");
   HILS_REQUIRE(h_kv <= 65535 && B <= 65535, "hils_topk_fwd: h_kv/B too large for the grid");
   hipStream_t st = (hipStream_t)stream;
-  if (topk_use_split(B, L, N, h_kv) &&
+  // few queries per (batch, KV head) (decode, short continuations): one workgroup per row whenever
+  // there are enough rows to occupy the machine, however many more there are
+  if ((topk_use_split(B, L, N, h_kv) || L <= 4) &&
       topk_use_row((long)B * L * h_kv, N, G, D, per_qhead, !bias && !gumbel && !drop_mask)) {
     *weights_fused = weights != nullptr;
     if (int rc2 = topk_fwd_row(q, lmks, lse_swa, indices, scores, lse_total, sel_logits, weights, B, L, N, h_kv, G, D, topk,

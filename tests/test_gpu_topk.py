@@ -270,6 +270,7 @@ def test_topk_split_path_options(pkg, orc, dev):
     (16, 1, 2048, 8, 4, 128, 32, 2048 * 64), (12, 1, 1000, 8, 2, 64, 64, 1000 * 64 - 1),
     (100, 1, 300, 1, 1, 128, 8, 200 * 64), (3, 5, 4096, 8, 4, 64, 16, 4096 * 64 - 5),
     (24, 1, 777, 4, 3, 128, 32, 500 * 64 + 7),
+    (40, 2, 1536, 8, 4, 128, 32, 1536 * 64 - 2),  # more rows than compute units: 8-wavefront workgroups
     (128, 1, 256, 1, 4, 64, 8, 10),           # no chunk visible yet: all -1
     (64, 2, 300, 2, 2, 128, 8, 64 * 3 + 5)])  # fewer visible chunks than topk
 def test_topk_workgroup_per_row_path(pkg, orc, dev, B, L, N, h_kv, G, D, topk, off):
