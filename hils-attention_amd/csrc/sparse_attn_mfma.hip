@@ -87,6 +87,13 @@ pack_kv_kernel(const bf16_t* __restrict__ k, const bf16_t* __restrict__ v, bf16_
   }
 }
 
+// Fixed point by accumulator bias: a product accumulated onto GA_FX_BIAS = 1.5 * 2^23 comes out
+// as a float whose unit in the last place is 1, so (bits - bits of the bias) is the sum rounded
+// to an integer, for |sum| < 2^22.
+#define GA_FX_BIAS 12582912.0f
+#define GA_FX_BIAS_BITS 0x4B400000
+#define GA_FX_LOG2_MAX 21  // sums are scaled below 2^21: one bit of head room for the rounding of P
+
 struct GaDims {
   int L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last;
   float sm_scale;
@@ -111,14 +118,15 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   constexpr int KS = D / 32;    // k-steps of S^T = K Q^T
   constexpr int DT = DV / 16;   // 16-wide output column tiles
   constexpr int QT = 16 / G;    // queries per 16-row tile
+  constexpr int NT = GA_THREADS;
   constexpr int MAXP = 8;       // pairs per thread: T*K <= MAXP * GA_THREADS
-  extern __shared__ int smem_i[];
+  extern __shared__ __align__(16) int smem_i[];
   const int R = dm.T * G;
-  int* o_acc = smem_i;                       // (R + 1) x DV fixed point; row R takes the padding rows of a tile
-  int* cur = o_acc + (size_t)(R + 1) * DV;   // nchunk: histogram -> running ends
+  int* o_acc = smem_i;                       // R x DV fixed point
+  int* cur = o_acc + (size_t)R * DV;         // nchunk: histogram -> running ends
   int* pairs = cur + dm.nchunk;              // T*K pairs (query << 8 | slot) grouped by chunk
   __shared__ float red[32];
-  __shared__ int scan_s[GA_WAVES];
+  __shared__ int scan_s[NT / 64];
   __shared__ int next_s;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -152,7 +160,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   uint4 qtmp[QPK];
 #pragma unroll
   for (int e = 0; e < QPK; ++e) {
-    const int i = tid + e * GA_THREADS;
+    const int i = tid + e * NT;
     const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
     const int g2 = rem / PPR, pc = rem - g2 * PPR;
     const bool ok = i < npiece && t0 + ql < dm.L;
@@ -163,7 +171,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   int creg[MAXP], preg[MAXP];
 #pragma unroll
   for (int e = 0; e < MAXP; ++e) {
-    const int i = tid + e * GA_THREADS;
+    const int i = tid + e * NT;
     int c = -1;
     preg[e] = 0;
     if (i < npair) {
@@ -177,7 +185,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   // A row is read as aligned dwords (rows start on any bf16), all loads in flight together.
   constexpr int WDW = 17;  // dwords per round: 32 slots + alignment slack
   float wsum = 0.f;
-  for (int row = tid; row < R; row += GA_THREADS) {
+  for (int row = tid; row < R; row += NT) {
     const int ql = row / G, g = row - ql * G;
     if (t0 + ql < dm.L) {
       const long e0 = ((b * LB + (t0 + ql) / dm.q_block) * (long)dm.WH + (w_per_q ? hk * G + g : hk)) *
@@ -203,18 +211,18 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       wsum = fmaxf(wsum, a);
     }
   }
-  for (int i = tid; i < R * DV; i += GA_THREADS) o_acc[i] = 0;
-  for (int i = tid; i < dm.nchunk; i += GA_THREADS) cur[i] = 0;
+  for (int i = tid; i < R * DV; i += NT) o_acc[i] = 0;
+  for (int i = tid; i < dm.nchunk; i += NT) cur[i] = 0;
   if (tid == 0) next_s = 0;
 #pragma unroll
   for (int e = 0; e < QPK; ++e) {
-    const int i = tid + e * GA_THREADS;
+    const int i = tid + e * NT;
     const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
     const int g2 = rem / PPR, pc = rem - g2 * PPR;
     if (i < npiece && t0 + ql < dm.L)
       *(uint4*)(qp + ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G) * D + (pc * G + g2) * 8) = qtmp[e];
   }
-  for (int i = QPK * GA_THREADS + tid; i < npiece; i += GA_THREADS) {  // blocks with more pieces (rare shapes)
+  for (int i = QPK * NT + tid; i < npiece; i += NT) {  // blocks with more pieces (rare shapes)
     const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
     const int g2 = rem / PPR, pc = rem - g2 * PPR;
     if (t0 + ql < dm.L) {
@@ -229,7 +237,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     int c = creg[e];
     if (c < -1 || c >= dm.nchunk) c = -1;
     if (c < 0 && lse) {
-      const int i = tid + e * GA_THREADS;
+      const int i = tid + e * NT;
       const int ql = i / K, slot = i - ql * K;
       if (i < npair && t0 + ql < dm.L) {
 #pragma unroll
@@ -243,7 +251,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   wsum = block_max(wsum, red);  // barrier: histogram complete
   // ... times max |V| over the visited chunks; exclusive scan of the histogram on the way
   float vm = 0.f;
-  const int per_thr = (dm.nchunk + GA_THREADS - 1) / GA_THREADS;
+  const int per_thr = (dm.nchunk + NT - 1) / NT;
   const int c_lo = tid * per_thr;
   int local = 0;
   for (int c = c_lo; c < c_lo + per_thr && c < dm.nchunk; ++c) {
@@ -275,7 +283,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   const float bound = wsum * vm;
   float fx_scale = 1.f;
   if (bound > 0.f && bound < 3.0e38f) {
-    int e2 = 28 - ilogbf(bound);
+    int e2 = GA_FX_LOG2_MAX - 1 - ilogbf(bound);  // bound * 2^e2 < 2^GA_FX_LOG2_MAX
     e2 = e2 > 90 ? 90 : (e2 < -90 ? -90 : e2);
     fx_scale = ldexpf(1.f, e2);
   }
@@ -287,6 +295,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   // rows of a tile are addressed from the block's first query with 32-bit element offsets
   const bf16_t* qb = qp + ((b * dm.L + t0) * (long)dm.HQ + hk * G) * D;
   const bf16_t* wb = weights + ((b * LB + t0 / dm.q_block) * (long)dm.WH + (w_per_q ? hk * G : hk)) * dm.NW;
+  float* lse_blk = lse ? lse + (b * dm.L + t0) * (long)dm.HQ * K : nullptr;  // the block's first row
   const int q_lane = (j * G + g) * 8, w_lane = w_per_q ? g * dm.NW : 0;
   const int q_step = dm.HQ * D;          // per query of the block
   const int w_step = dm.WH * dm.NW;      // per group of q_block queries
@@ -298,19 +307,21 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   //                 S(i) = K Q(i)^T  [then K(chunk i+1) replaces K in place];  softmax -> P(i).
   // K and V of a chunk are reloaded only when the next tile belongs to another chunk.
   bf16x8_t ka[4][KS], vb[DT][2];
+  // operand loads: a wavefront-uniform 64-bit base plus this lane's 32-bit byte offset
+  const unsigned lane_b = lane * 16;
   auto load_k = [&](int c, int mt) {
-    const bf16_t* kbase = kp + ((b * dm.H + hk) * (long)dm.nchunk + c) * (long)GA_S * D + lane * 8;
+    const char* kbase = (const char*)(kp + ((b * dm.H + hk) * (long)dm.nchunk + c) * (long)GA_S * D);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const uint4 x = *(const uint4*)(kbase + (mt * KS + ks) * 512);
+      const uint4 x = *(const uint4*)(kbase + (mt * KS + ks) * 1024 + lane_b);
       ka[mt][ks] = *(const bf16x8_t*)&x;
     }
   };
   auto load_v = [&](int c, int dt) {
-    const bf16_t* vbase = vp + ((b * dm.H + hk) * (long)dm.nchunk + c) * (long)GA_S * DV + lane * 8;
+    const char* vbase = (const char*)(vp + ((b * dm.H + hk) * (long)dm.nchunk + c) * (long)GA_S * DV);
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const uint4 x = *(const uint4*)(vbase + (dt * 2 + s) * 512);
+      const uint4 x = *(const uint4*)(vbase + (dt * 2 + s) * 1024 + lane_b);
       vb[dt][s] = *(const bf16x8_t*)&x;
     }
   };
@@ -337,32 +348,45 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     ve = ve2;
   };
   // A tile's gathered query rows (B operands), weight and output rows.  Padding rows of a
-  // visit's last tile repeat the visit's first pair (finite arithmetic) and are accumulated
-  // into the spare row R.  Query rows come from the packed copy, in which the G heads of a
-  // query are interleaved per 16-byte piece: the lanes of one query read contiguous bytes.
+  // visit's last tile repeat the tile's last pair with weight 0: their P is exactly 0 and is
+  // added to that pair's output rows.  Query rows come from the packed copy, in which the G
+  // heads of a query are interleaved per 16-byte piece: the lanes of one query read contiguous
+  // bytes.
   uint4 bq_n[KS];
   int w_n, pk_n, orow_n[4];
-  auto load_tile = [&](int p, int ve) {
-    const int last = ((ve - p < QT) ? ve - p : QT) - 1;  // padding rows repeat the tile's last pair
-    // all pair reads first, one wait
-    pk_n = pairs[p + (qs < last ? qs : last)];
-    int pk_o[4];
+  // output rows 4j .. 4j+3 of a tile starting at pair p (element offsets of this lane's column)
+  auto tile_rows = [&](int p, int last, int* orow) {
+    if constexpr (G >= 4) {  // the four rows are consecutive heads of one query
+      const int qsl = (4 * j) / G;
+      const int pk = pairs[p + (qsl < last ? qsl : last)];
+      const int base = ((pk >> 8) * G + (4 * j) % G) * DV + r;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int qsl = (4 * j + i) / G;
-      pk_o[i] = pairs[p + (qsl < last ? qsl : last)];
+      for (int i = 0; i < 4; ++i) orow[i] = base + i * DV;
+    } else {
+      int pk_o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int qsl = (4 * j + i) / G;
+        pk_o[i] = pairs[p + (qsl < last ? qsl : last)];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int rr = 4 * j + i;
+        orow[i] = ((pk_o[i] >> 8) * G + rr % G) * DV + r;
+      }
     }
+  };
+  auto load_tile = [&](int p, int ve) {
+    const int last = ((ve - p < QT) ? ve - p : QT) - 1;
+    pk_n = pairs[p + (qs < last ? qs : last)];
+    tile_rows(p, last, orow_n);
     const bf16_t* qrow = qb + ((pk_n >> 8) * q_step + q_lane);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) bq_n[ks] = *(const uint4*)(qrow + ks * (4 * G * 8));
     w_n = 0;
-    if (j == 0) w_n = wb[((pk_n >> 8) / dm.q_block) * w_step + w_lane + (pk_n & 255)];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int rr = 4 * j + i;
-      const int qsl = rr / G;
-      const int row = (qsl <= last) ? (pk_o[i] >> 8) * G + (rr - qsl * G) : R;
-      orow_n[i] = row * DV + r;
+    if (j == 0 && qs <= last) {
+      const int ql = pk_n >> 8;
+      w_n = wb[(dm.q_block == 1 ? ql : ql / dm.q_block) * w_step + w_lane + (pk_n & 255)];
     }
   };
   bf16x8_t ap[2];   // P of the previous tile (A operand of O = P V)
@@ -394,10 +418,15 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
         }
     }
     if (dm.mask_last && j == 3) st[3][3] = HILS_NEG_INF;  // token 63 = tile 3, lane group 3, register 3
-    float m = fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3]));
-#pragma unroll
-    for (int mt = 1; mt < 4; ++mt) m = fmaxf(fmaxf(m, fmaxf(st[mt][0], st[mt][1])), fmaxf(st[mt][2], st[mt][3]));
-    m = rows_max(m);
+    // (this file is compiled without NaN handling: the maxima are bare v_max3 instructions)
+    float m = fmaxf(fmaxf(st[0][0], st[0][1]), st[0][2]);
+    m = fmaxf(fmaxf(m, st[0][3]), st[1][0]);
+    m = fmaxf(fmaxf(m, st[1][1]), st[1][2]);
+    m = fmaxf(fmaxf(m, st[1][3]), st[2][0]);
+    m = fmaxf(fmaxf(m, st[2][1]), st[2][2]);
+    m = fmaxf(fmaxf(m, st[2][3]), st[3][0]);
+    m = fmaxf(fmaxf(m, st[3][1]), st[3][2]);
+    m = rows_max(fmaxf(m, st[3][3]));
     const float mc = m * c2;
     float sum = 0.f;
 #pragma unroll
@@ -412,7 +441,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     if (dm.sm_n != 0.f) sum += dm.sm_n * __builtin_amdgcn_exp2f(-mc);
     if (lse && qs < n && j == 0) {
       const int ql = pk_c >> 8, slot = pk_c & 255;
-      lse[((b * dm.L + t0 + ql) * (long)dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
+      lse_blk[(ql * dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
     }
     const float f = w_row * fx_scale * __builtin_amdgcn_rcpf(sum);  // fixed-point scale (a power of two) folded into P
     // P as the A operand of O = P V: k-step s takes tokens of accumulator tiles 2s, 2s+1
@@ -427,6 +456,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     }
   };
   // O += P V for the tile in (ap, orow_p); V(c_next) replaces V when asked
+  const f32x4_t fx_bias = {GA_FX_BIAS, GA_FX_BIAS, GA_FX_BIAS, GA_FX_BIAS};
   auto output_stage = [&](bool reload, int c_next) {
     // four column tiles at a time: their eight MFMAs interleaved (two-deep chains), then the
     // operand reload, then the fixed-point adds
@@ -434,7 +464,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     for (int d0 = 0; d0 < DT; d0 += 4) {
       f32x4_t acc[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) acc[u] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+      for (int u = 0; u < 4; ++u) acc[u] = fx_bias;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
@@ -447,7 +477,8 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
 #pragma unroll
       for (int u = 0; u < 4; ++u)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) atomicAdd(&o_acc[orow_p[i] + (d0 + u) * 16], __float2int_rn(acc[u][i]));
+        for (int i = 0; i < 4; ++i)
+          atomicAdd(&o_acc[orow_p[i] + (d0 + u) * 16], __float_as_int(acc[u][i]) - GA_FX_BIAS_BITS);
     }
   };
 
@@ -496,17 +527,20 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   }
   __syncthreads();
   constexpr int C8 = DV / 8;
-  for (int i = tid; i < R * C8; i += GA_THREADS) {
+  for (int i = tid; i < R * C8; i += NT) {
     const int row = i / C8, c8 = i - row * C8;
     const int ql = row / G, g2 = row - ql * G;
     const int t = t0 + ql;
     if (t < dm.L) {
       const int* src = o_acc + (size_t)row * DV + c8 * 8;
+      float f[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = (float)src[e] * fx_inv;
       uint4 x;
-      x.x = pack_bf2((float)src[0] * fx_inv, (float)src[1] * fx_inv);
-      x.y = pack_bf2((float)src[2] * fx_inv, (float)src[3] * fx_inv);
-      x.z = pack_bf2((float)src[4] * fx_inv, (float)src[5] * fx_inv);
-      x.w = pack_bf2((float)src[6] * fx_inv, (float)src[7] * fx_inv);
+      x.x = pack_bf2(f[0], f[1]);
+      x.y = pack_bf2(f[2], f[3]);
+      x.z = pack_bf2(f[4], f[5]);
+      x.w = pack_bf2(f[6], f[7]);
       *(uint4*)(o + ((b * dm.L + t) * (long)dm.HQ + hk * G + g2) * DV + c8 * 8) = x;
     }
   }
@@ -569,7 +603,7 @@ static int ga_pick_T(int L, int G, int Dv, int K, int nchunk, size_t* smem_out) 
   if (T * K > 8 * GA_THREADS) T = (8 * GA_THREADS) / K;
   if (T > L) T = L;
   while (T >= 1) {
-    const size_t smem = (size_t)(T * G + 1) * Dv * 4 + (size_t)nchunk * 4 + (size_t)T * K * 4;
+    const size_t smem = (size_t)T * G * Dv * 4 + (size_t)nchunk * 4 + (size_t)T * K * 4;
     if (smem <= 156 * 1024) {
       *smem_out = smem;
       return T;
