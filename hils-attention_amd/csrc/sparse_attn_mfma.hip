@@ -89,7 +89,8 @@ pack_kv_kernel(const bf16_t* __restrict__ k, const bf16_t* __restrict__ v, bf16_
 
 // Fixed point by accumulator bias: a product accumulated onto GA_FX_BIAS = 1.5 * 2^23 comes out
 // as a float whose unit in the last place is 1, so (bits - bits of the bias) is the sum rounded
-// to an integer, for |sum| < 2^22.
+// to an integer, for |sum| < 2^22.  The kernel adds the raw bits and counts the adds of every
+// output row; the biases leave in the epilogue (all of it modulo 2^32).
 #define GA_FX_BIAS 12582912.0f
 #define GA_FX_BIAS_BITS 0x4B400000
 #define GA_FX_LOG2_MAX 21  // sums are scaled below 2^21: one bit of head room for the rounding of P
@@ -125,6 +126,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   int* o_acc = smem_i;                       // R x DV fixed point
   int* cur = o_acc + (size_t)R * DV;         // nchunk: histogram -> running ends
   int* pairs = cur + dm.nchunk;              // T*K pairs (query << 8 | slot) grouped by chunk
+  int* nadd = pairs + dm.T * dm.K;           // R: tiles added to each output row
   __shared__ float red[32];
   __shared__ int scan_s[NT / 64];
   __shared__ int next_s;
@@ -213,6 +215,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   }
   for (int i = tid; i < R * DV; i += NT) o_acc[i] = 0;
   for (int i = tid; i < dm.nchunk; i += NT) cur[i] = 0;
+  for (int i = tid; i < R; i += NT) nadd[i] = 0;
   if (tid == 0) next_s = 0;
 #pragma unroll
   for (int e = 0; e < QPK; ++e) {
@@ -443,6 +446,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       const int ql = pk_c >> 8, slot = pk_c & 255;
       lse_blk[(ql * dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
     }
+    if (j == 0) atomicAdd(&nadd[(pk_c >> 8) * G + g], 1);  // padding rows count on the row they are added to
     const float f = w_row * fx_scale * __builtin_amdgcn_rcpf(sum);  // fixed-point scale (a power of two) folded into P
     // P as the A operand of O = P V: k-step s takes tokens of accumulator tiles 2s, 2s+1
 #pragma unroll
@@ -478,7 +482,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       for (int u = 0; u < 4; ++u)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          atomicAdd(&o_acc[orow_p[i] + (d0 + u) * 16], __float_as_int(acc[u][i]) - GA_FX_BIAS_BITS);
+          atomicAdd(&o_acc[orow_p[i] + (d0 + u) * 16], __float_as_int(acc[u][i]));
     }
   };
 
@@ -533,9 +537,10 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     const int t = t0 + ql;
     if (t < dm.L) {
       const int* src = o_acc + (size_t)row * DV + c8 * 8;
+      const unsigned bias = (unsigned)nadd[row] * (unsigned)GA_FX_BIAS_BITS;  // wraps like the sums did
       float f[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] = (float)src[e] * fx_inv;
+      for (int e = 0; e < 8; ++e) f[e] = (float)(int)((unsigned)src[e] - bias) * fx_inv;
       uint4 x;
       x.x = pack_bf2(f[0], f[1]);
       x.y = pack_bf2(f[2], f[3]);
@@ -603,7 +608,7 @@ static int ga_pick_T(int L, int G, int Dv, int K, int nchunk, size_t* smem_out) 
   if (T * K > 8 * GA_THREADS) T = (8 * GA_THREADS) / K;
   if (T > L) T = L;
   while (T >= 1) {
-    const size_t smem = (size_t)T * G * Dv * 4 + (size_t)nchunk * 4 + (size_t)T * K * 4;
+    const size_t smem = (size_t)T * G * Dv * 4 + (size_t)nchunk * 4 + (size_t)T * K * 4 + (size_t)T * G * 4;
     if (smem <= 156 * 1024) {
       *smem_out = smem;
       return T;
