@@ -101,11 +101,9 @@ def bench_prefill(pkg, dev, steps, warmup):
         lmk = pkg.chunk_mean_pool(k, S)
         if record:
             ev[1].record()
-        idx, scores = pkg.online_softmax_topk_head(q, lmk, lse_swa, K, S, W, is_training=False)
+        idx, scores, w = pkg.topk_chunk_weights(q, lmk, lse_swa, K, S, W)  # selection + inter-chunk softmax, one call
         if record:
             ev[2].record()
-        w = pkg.chunk_weights(scores, lse_swa)
-        if record:
             ev[3].record()
             ws = attn_mod.prepare_kv_workspace(L, k, v, HQ, K, S)  # serial here: per-kernel durations
             ev[4].record()
@@ -153,8 +151,7 @@ def bench_config2(pkg, dev, iters=5):
     for it in range(iters + 1):
         ev[0].record()
         lmk = pkg.chunk_mean_pool(k, S)
-        idx, scores = pkg.online_softmax_topk_head(q, lmk, lse_swa, K, S, W, is_training=False)
-        w = pkg.chunk_weights(scores, lse_swa)
+        idx, scores, w = pkg.topk_chunk_weights(q, lmk, lse_swa, K, S, W)
         ws = attn_mod.prepare_kv_workspace(L, k, v, HQ, K, S)
         ev[1].record()
         pkg.HiLS_block_M_head(q, k, v, w, idx, block_size=S, is_training=False, kv_workspace=ws)

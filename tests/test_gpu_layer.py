@@ -69,7 +69,12 @@ def _chunk_weights_case(pkg, orc, dev, K):
 @pytest.mark.parametrize("B,L,N,HQ,H,D,K,off", [(32, 1, 2048, 32, 8, 128, 32, 2048 * 64 - 1),
                                                 (13, 1, 500, 8, 8, 64, 16, 300 * 64),
                                                 (2, 3, 700, 8, 2, 128, 8, 700 * 64 - 3),
-                                                (128, 1, 256, 4, 1, 64, 8, 64 * 2 + 1)])
+                                                (128, 1, 256, 4, 1, 64, 8, 64 * 2 + 1),
+                                                # prefill shapes: two kernels behind the one call
+                                                (1, 1024, 16, 8, 2, 128, 8, 0),
+                                                (2, 1000, 16, 4, 4, 64, 16, 24),
+                                                (1, 2048, 32, 4, 2, 128, 32, 0),
+                                                (1, 512, 8, 8, 2, 64, 12, 0)])
 def test_topk_with_fused_weights_matches_two_calls(pkg, dev, B, L, N, HQ, H, D, K, off):
     """One call for selection + inter-chunk softmax (the selection kernel writes the weights when
     it runs one workgroup per row, else a second kernel) against the two separate operators."""
