@@ -601,21 +601,23 @@ static size_t ga_vmax_bytes(int B, int H, int nchunk) {
   return ((size_t)B * H * nchunk * sizeof(float) + 255) & ~(size_t)255;
 }
 
-// Tile sizes: T queries per workgroup such that the fixed-point output tile, the chunk
-// histogram and the pair list fit in LDS.  Returns 0 when the shape does not fit.
-static int ga_pick_T(int L, int G, int Dv, int K, int nchunk, size_t* smem_out) {
-  int T = (128 * 1024) / (G * Dv * 4);
+// Tile sizes: the largest T (queries per workgroup, a multiple of q_block and of 8 when it can be)
+// such that the fixed-point output tile, the chunk histogram, the pair list and the add counts
+// fit in the LDS of a compute unit, with at most 8 pairs per thread.  The more rows share a
+// visit, the fewer bytes of K and V the block pulls per row.  Returns 0 when nothing fits.
+#define GA_SMEM_MAX (160 * 1024 - 512)  // dynamic LDS beside the kernel's static arrays
+static int ga_pick_T(int L, int G, int Dv, int K, int nchunk, int q_block, size_t* smem_out) {
+  const size_t per_q = (size_t)G * Dv * 4 + (size_t)K * 4 + (size_t)G * 4;
+  const size_t fixed = (size_t)nchunk * 4;
+  if (fixed + per_q > GA_SMEM_MAX) return 0;
+  long T = (long)((GA_SMEM_MAX - fixed) / per_q);
   if (T * K > 8 * GA_THREADS) T = (8 * GA_THREADS) / K;
   if (T > L) T = L;
-  while (T >= 1) {
-    const size_t smem = (size_t)T * G * Dv * 4 + (size_t)nchunk * 4 + (size_t)T * K * 4 + (size_t)T * G * 4;
-    if (smem <= 156 * 1024) {
-      *smem_out = smem;
-      return T;
-    }
-    T /= 2;
-  }
-  return 0;
+  if (T >= 8 && q_block <= 8 && 8 % q_block == 0) T &= ~7L;
+  else T -= T % q_block;
+  if (T < 1) return 0;
+  *smem_out = fixed + (size_t)T * per_q;
+  return (int)T;
 }
 
 // Workspace the MFMA path needs (the per-chunk transposed copy of V and the per-chunk max|V|),
@@ -630,7 +632,7 @@ size_t hils_ga_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int 
                   K >= 1 && K <= 256;
   if (!ok) return 0;
   size_t smem;
-  const int T = ga_pick_T(L, G, Dv, K, Lkv / S, &smem);
+  const int T = ga_pick_T(L, G, Dv, K, Lkv / S, q_block, &smem);
   if (T == 0 || T % q_block != 0) return 0;  // a query block holds whole index-sharing groups
   const int nchunk = Lkv / S;
   return ga_vt_bytes(B, H, nchunk, Dv) + ga_vt_bytes(B, H, nchunk, D) + ga_vmax_bytes(B, H, nchunk) +
@@ -649,7 +651,7 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
   const int nchunk = Lkv / S;
   hipStream_t st = (hipStream_t)stream;
   size_t smem;
-  const int T = ga_pick_T(L, G, Dv, K, nchunk, &smem);
+  const int T = ga_pick_T(L, G, Dv, K, nchunk, q_block, &smem);
   if (T == 0 || T % q_block != 0 || H > 65535 || B > 65535) return HILS_OK;
   const int nblk = (L + T - 1) / T;
   const long total = (long)nblk * H * B;
