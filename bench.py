@@ -27,7 +27,7 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the readings of
 # a 512 MiB copy: x2.0 and x1.0), see profiles/hbm_traffic_fetch_write_size.md
-TRAFFIC_PREFILL_ATTN_BYTES = 3.09e9
+TRAFFIC_PREFILL_ATTN_BYTES = 4.53e9
 TRAFFIC_DECODE_STEP_BYTES = 4.05e8
 
 
