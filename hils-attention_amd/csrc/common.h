@@ -103,6 +103,25 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   for (int i = 0; i < nw; ++i) r += red[i];
   return r;
 }
+// Workgroup barrier that orders LDS accesses only: global stores issued before it stay in
+// flight (a __syncthreads() waits for them too).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+// block_max with LDS-only barriers
+__device__ __forceinline__ float block_max_lds(float v, float* red) {
+  v = wave_max(v);
+  const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  lds_barrier();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  lds_barrier();
+  float r = HILS_NEG_INF;
+  for (int i = 0; i < nw; ++i) r = fmaxf(r, red[i]);
+  return r;
+}
+
 __device__ __forceinline__ float block_max(float v, float* red) {
   v = wave_max(v);
   const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;

@@ -157,7 +157,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   // of the G lanes that hold the heads of one query are contiguous.  Only this workgroup
   // reads what it writes here (made visible by the barriers below).
   constexpr int PPR = D / 8;
-  constexpr int QPK = 8;  // pieces per thread and round
+  constexpr int QPK = 10;  // pieces per thread in flight (a 72-query block of 4 heads, D = 128, has 9)
   const int npiece = dm.T * G * PPR;
   uint4 qtmp[QPK];
 #pragma unroll
@@ -213,27 +213,38 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       wsum = fmaxf(wsum, a);
     }
   }
-  for (int i = tid; i < R * DV; i += NT) o_acc[i] = 0;
-  for (int i = tid; i < dm.nchunk; i += NT) cur[i] = 0;
-  for (int i = tid; i < R; i += NT) nadd[i] = 0;
-  if (tid == 0) next_s = 0;
+  // The packed copy goes through LDS (the output tile is not in use yet): pieces arrive in the
+  // order of the source rows and leave in packed order, so that loads and stores are both
+  // contiguous 1 KiB per wavefront instruction.
+  uint4* stage = (uint4*)o_acc;  // npiece * 16 bytes <= R * DV * 4
 #pragma unroll
   for (int e = 0; e < QPK; ++e) {
     const int i = tid + e * NT;
     const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
     const int g2 = rem / PPR, pc = rem - g2 * PPR;
-    if (i < npiece && t0 + ql < dm.L)
-      *(uint4*)(qp + ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G) * D + (pc * G + g2) * 8) = qtmp[e];
+    if (i < npiece) stage[ql * (G * PPR) + pc * G + g2] = qtmp[e];
   }
   for (int i = QPK * NT + tid; i < npiece; i += NT) {  // blocks with more pieces (rare shapes)
     const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
     const int g2 = rem / PPR, pc = rem - g2 * PPR;
-    if (t0 + ql < dm.L) {
-      const long blk_e = ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G) * D;
-      *(uint4*)(qp + blk_e + (pc * G + g2) * 8) = *(const uint4*)(q + blk_e + g2 * D + pc * 8);
-    }
+    const long blk_e = ((b * dm.L + (t0 + ql < dm.L ? t0 + ql : t0)) * (long)dm.HQ + hk * G) * D;
+    stage[ql * (G * PPR) + pc * G + g2] = *(const uint4*)(q + blk_e + g2 * D + pc * 8);
   }
-  __syncthreads();
+  for (int i = tid; i < dm.nchunk; i += NT) cur[i] = 0;
+  for (int i = tid; i < R; i += NT) nadd[i] = 0;
+  if (tid == 0) next_s = 0;
+  lds_barrier();
+  for (int i = tid; i < npiece; i += NT) {
+    const int ql = i / (G * PPR);
+    const uint4 x = stage[i];
+    stage[i] = make_uint4(0, 0, 0, 0);  // this thread's share of clearing the output tile
+    if (t0 + ql < dm.L)
+      *(uint4*)(qp + ((b * dm.L + t0 + ql) * (long)dm.HQ + hk * G) * D + (i - ql * (G * PPR)) * 8) = x;
+  }
+  for (int i = npiece * 4 + tid; i < R * DV; i += NT) o_acc[i] = 0;  // the rest of the tile
+  // (LDS-only barriers up to the last one of the prologue: the packed-query stores above stay in
+  // flight behind the sort instead of being waited for here)
+  lds_barrier();
   // histogram of the selected chunks
 #pragma unroll
   for (int e = 0; e < MAXP; ++e) {
@@ -251,7 +262,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     creg[e] = c;
     if (c >= 0) atomicAdd(&cur[c], 1);
   }
-  wsum = block_max(wsum, red);  // barrier: histogram complete
+  wsum = block_max_lds(wsum, red);  // barrier: histogram complete
   // ... times max |V| over the visited chunks; exclusive scan of the histogram on the way
   float vm = 0.f;
   const int per_thr = (dm.nchunk + NT - 1) / NT;
@@ -269,7 +280,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     if (lane >= o2) incl += x;
   }
   if (lane == 63) scan_s[wave] = incl;
-  vm = block_max(vm, red);  // barrier: scan_s visible, all histogram reads done
+  vm = block_max_lds(vm, red);  // barrier: scan_s visible, all histogram reads done
   int base = incl - local;
   for (int w2 = 0; w2 < wave; ++w2) base += scan_s[w2];
   for (int c = c_lo; c < c_lo + per_thr && c < dm.nchunk; ++c) {
@@ -277,7 +288,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     cur[c] = base;
     base += h;
   }
-  __syncthreads();
+  lds_barrier();
 #pragma unroll
   for (int e = 0; e < MAXP; ++e)
     if (creg[e] >= 0) pairs[atomicAdd(&cur[creg[e]], 1)] = preg[e];
