@@ -167,7 +167,12 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     const int g2 = rem / PPR, pc = rem - g2 * PPR;
     const bool ok = i < npiece && t0 + ql < dm.L;
     const long blk_e = ((b * dm.L + (ok ? t0 + ql : t0)) * (long)dm.HQ + hk * G) * D;  // t0 < L always
-    qtmp[e] = *(const uint4*)(q + blk_e + g2 * D + pc * 8);
+    // relaxed atomic loads: the compiler keeps them here, ahead of the loads below, instead of
+    // moving them next to their use behind the weight loop (a second exposed latency)
+    const unsigned long long* src = (const unsigned long long*)(q + blk_e + g2 * D + pc * 8);
+    const unsigned long long lo = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const unsigned long long hi = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    qtmp[e] = make_uint4((unsigned)lo, (unsigned)(lo >> 32), (unsigned)hi, (unsigned)(hi >> 32));
   }
   // (2) selected chunk of every (query, slot) pair of the block
   int creg[MAXP], preg[MAXP];
@@ -222,7 +227,8 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     const int i = tid + e * NT;
     const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
     const int g2 = rem / PPR, pc = rem - g2 * PPR;
-    if (i < npiece) stage[ql * (G * PPR) + pc * G + g2] = qtmp[e];
+    // (unconditional: pieces past the end land behind the staged ones, in bytes cleared below)
+    stage[i < npiece ? ql * (G * PPR) + pc * G + g2 : npiece + lane] = qtmp[e];
   }
   for (int i = QPK * NT + tid; i < npiece; i += NT) {  // blocks with more pieces (rare shapes)
     const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
