@@ -599,9 +599,9 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
       const int tq = t0 + nt * QPT + r / GMAX;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (tq < L && g < G)
-          v = *(const uint4*)(q + (((b * L + tq) * h_kv + hk) * (long)G + g) * D + ks * 32 + j * 8);
+        const bool ok = tq < L && g < G;
+        uint4 v = *(const uint4*)(q + (((b * L + (ok ? tq : t0)) * h_kv + hk) * (long)G + (ok ? g : 0)) * D + ks * 32 + j * 8);
+        if (!ok) v = make_uint4(0, 0, 0, 0);
         afrag[nt][ks] = *(bf16x8_t*)&v;
       }
     }
@@ -692,7 +692,11 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
     for (int i = 0; i < 4; ++i) {
       const int r = 4 * j + i;
       const int tq = t0 + nt * QPT + r / GMAX, g = r % GMAX;
-      swa[nt][i] = (tq < L && g < G) ? lse_swa[((b * L + tq) * (long)h_kv + hk) * G + g] : HILS_NEG_INF;
+      // unconditional loads from a clamped address: all eight are in flight together (a load
+      // inside a branch is waited for inside it, one memory latency after the other)
+      const bool ok = tq < L && g < G;
+      const float x = lse_swa[((b * L + (ok ? tq : t0)) * (long)h_kv + hk) * G + (ok ? g : 0)];
+      swa[nt][i] = ok ? x : HILS_NEG_INF;
     }
   float ref[NT][4], l[NT][4];
 #pragma unroll
