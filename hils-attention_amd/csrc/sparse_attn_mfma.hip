@@ -9,8 +9,8 @@
 // softmax along the accumulator registers, and feeds P back as the A operand of
 // O = P V without leaving registers (the contraction order over tokens is permuted to
 // the accumulator layout; V is pre-transposed per chunk in the same order).  The
-// (rows x Dv) partial outputs are summed into an fp32 output tile in LDS with LDS
-// atomics, which is what lets rows of different visits be arbitrary subsets of the block.
+// (rows x Dv) partial outputs are summed into a fixed-point output tile in LDS with integer
+// LDS atomics, which is what lets rows of different visits be arbitrary subsets of the block.
 #include "common.h"
 #include "../../include/hils_amd.h"
 
