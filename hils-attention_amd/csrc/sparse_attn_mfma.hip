@@ -227,8 +227,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     const int i = tid + e * NT;
     const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
     const int g2 = rem / PPR, pc = rem - g2 * PPR;
-    // (unconditional: pieces past the end land behind the staged ones, in bytes cleared below)
-    stage[i < npiece ? ql * (G * PPR) + pc * G + g2 : npiece + lane] = qtmp[e];
+    if (i < npiece) stage[ql * (G * PPR) + pc * G + g2] = qtmp[e];
   }
   for (int i = QPK * NT + tid; i < npiece; i += NT) {  // blocks with more pieces (rare shapes)
     const int ql = i / (G * PPR), rem = i - ql * (G * PPR);
