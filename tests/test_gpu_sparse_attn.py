@@ -208,7 +208,12 @@ def test_sparse_attn_decode_one_workgroup_per_row(pkg, orc, dev, B, HQ, H, D, K,
 
 @pytest.mark.parametrize("B,L,HQ,H,D,Dv,K", [(1, 1024, 8, 2, 128, 128, 8), (2, 512, 4, 4, 64, 64, 16),
                                               (1, 700, 16, 1, 64, 128, 4), (1, 512, 8, 4, 128, 64, 32),
-                                              (1, 300, 16, 2, 64, 64, 8)])
+                                              (1, 300, 16, 2, 64, 64, 8),
+                                              # query blocks with fewer 16-byte query pieces than the workgroup
+                                              # stages per round, D = 128 with Dv = 64 (the staged queries fill
+                                              # the output tile exactly) and the other head-dim pairs
+                                              (2, 128, 4, 2, 128, 64, 8), (1, 256, 8, 4, 128, 64, 16),
+                                              (3, 192, 8, 8, 128, 64, 4), (1, 128, 16, 4, 64, 128, 8)])
 def test_sparse_attn_mfma_path_matches_generic_path(pkg, orc, dev, B, L, HQ, H, D, Dv, K):
     """The chunk-regrouped MFMA kernel (workspace given) against the shape-generic kernel
     (workspace NULL) and the oracle, output and per-chunk LSE, through the C ABI."""
