@@ -17,6 +17,7 @@
 #define GA_THREADS 512
 #define GA_WAVES (GA_THREADS / 64)
 #define GA_S 64                 // chunk size this kernel is built for
+#define GA_MAXP 16              // (query, slot) pairs of a block per thread
 #define GA_KEY_INVALID 0xFFFFFFFFu
 #define GA_PAIR_BITS 12
 
@@ -120,7 +121,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   constexpr int DT = DV / 16;   // 16-wide output column tiles
   constexpr int QT = 16 / G;    // queries per 16-row tile
   constexpr int NT = GA_THREADS;
-  constexpr int MAXP = 8;       // pairs per thread: T*K <= MAXP * GA_THREADS
+  constexpr int MAXP = GA_MAXP;  // pairs per thread: T*K <= MAXP * GA_THREADS
   extern __shared__ __align__(16) int smem_i[];
   const int R = dm.T * G;
   int* o_acc = smem_i;                       // R x DV fixed point
@@ -619,7 +620,7 @@ static size_t ga_vmax_bytes(int B, int H, int nchunk) {
 
 // Tile sizes: the largest T (queries per workgroup, a multiple of q_block and of 8 when it can be)
 // such that the fixed-point output tile, the chunk histogram, the pair list and the add counts
-// fit in the LDS of a compute unit, with at most 8 pairs per thread.  The more rows share a
+// fit in the LDS of a compute unit, with at most GA_MAXP pairs per thread.  The more rows share a
 // visit, the fewer bytes of K and V the block pulls per row.  Returns 0 when nothing fits.
 #define GA_SMEM_MAX (160 * 1024 - 512)  // dynamic LDS beside the kernel's static arrays
 static int ga_pick_T(int L, int G, int Dv, int K, int nchunk, int q_block, size_t* smem_out) {
@@ -627,7 +628,7 @@ static int ga_pick_T(int L, int G, int Dv, int K, int nchunk, int q_block, size_
   const size_t fixed = (size_t)nchunk * 4;
   if (fixed + per_q > GA_SMEM_MAX) return 0;
   long T = (long)((GA_SMEM_MAX - fixed) / per_q);
-  if (T * K > 8 * GA_THREADS) T = (8 * GA_THREADS) / K;
+  if (T * K > GA_MAXP * GA_THREADS) T = (GA_MAXP * GA_THREADS) / K;
   if (T > L) T = L;
   if (T >= 8 && q_block <= 8 && 8 % q_block == 0) T &= ~7L;
   else T -= T % q_block;
