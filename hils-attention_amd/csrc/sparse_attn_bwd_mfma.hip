@@ -345,6 +345,7 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
 // scaled by a power of two from the bound  scale * 2 * max_row(sum_k|w| * |dO|_1) * max|V| * max|K|.
 // ---------------------------------------------------------------------------
 #define BQ_THREADS 512
+#define BQ_MAXP 16  // (query, slot) pairs of a block per thread
 #define BQ_WAVES (BQ_THREADS / 64)
 
 struct BqDims {
@@ -362,7 +363,7 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
   constexpr int KS = D / 32, VS = DV / 32;
   constexpr int DT = D / 16;
   constexpr int QT = 16 / G;
-  constexpr int MAXP = 8;
+  constexpr int MAXP = BQ_MAXP;
   extern __shared__ int smem_i[];
   const int R = dm.T * G;
   int* q_acc = smem_i;                       // (R + 1) x D fixed point; row R takes padding rows
@@ -627,18 +628,18 @@ void hils_ga_pack_launch(const void* a, const void* b, void* ap, void* bp, float
 // T queries per workgroup of the dQ kernel such that the fixed-point tile, the chunk histogram
 // and the pair list fit in LDS; 0 when the shape does not fit.
 static int bq_pick_T(int L, int G, int D, int K, int nchunk, size_t* smem_out) {
-  int T = (128 * 1024) / (G * D * 4);
-  if (T * K > 8 * BQ_THREADS) T = (8 * BQ_THREADS) / K;
+  // the largest block that fits: the more rows share a visit, the fewer K/V bytes per row
+  const size_t limit = 156 * 1024;
+  const size_t per_q = (size_t)G * D * 4 + (size_t)K * 4;
+  const size_t fixed = (size_t)D * 4 + (size_t)nchunk * 4;  // spare row, histogram
+  if (fixed + per_q > limit) return 0;
+  long T = (long)((limit - fixed) / per_q);
+  if (T * K > BQ_MAXP * BQ_THREADS) T = (BQ_MAXP * BQ_THREADS) / K;
   if (T > L) T = L;
-  while (T >= 1) {
-    const size_t smem = (size_t)(T * G + 1) * D * 4 + (size_t)nchunk * 4 + (size_t)T * K * 4;
-    if (smem <= 156 * 1024) {
-      *smem_out = smem;
-      return T;
-    }
-    T /= 2;
-  }
-  return 0;
+  if (T >= 8) T &= ~7L;
+  if (T < 1) return 0;
+  *smem_out = fixed + (size_t)T * per_q;
+  return (int)T;
 }
 
 struct BwLayout {
