@@ -191,13 +191,21 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
   const int npair = p_hi - p_lo;
   const int nround = (npair + PPR - 1) / PPR;
 
-  auto pair_of = [&](int round, int row) -> uint32_t {  // pair of a round's row; ~0u for padding rows
+  // Loads below are unconditional from clamped addresses, the pair entries as relaxed atomic
+  // loads: a load inside a branch is waited for inside it, and a plain load may be moved next to
+  // its use; either way the gathers of a round would queue up behind one another's latency.
+  auto pair_ok = [&](int round, int row) -> bool {  // false for padding rows
+    return row < ROWS && round * PPR + row / G < npair;
+  };
+  auto pair_of = [&](int round, int row) -> uint32_t {  // pair of a round's row (pair 0 of the chunk for padding rows)
     const int pi = round * PPR + row / G;
-    return (row < ROWS && pi < npair) ? pairs[p_lo + pi] : 0xffffffffu;
+    return __hip_atomic_load(pairs + p_lo + (pair_ok(round, row) ? pi : 0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   uint32_t pk_q[NQ], pk_o[NO], pk_r;
   uint4 xq[NQ], xo[NO];
-  float r_l2 = INFINITY, r_w = 0.f, r_dl = 0.f;
+  float r_l2 = INFINITY, r_dl = 0.f;
+  bf16_t r_wb = 0;
+  bool r_ok = false;
   auto load_pairs = [&](int round) {
 #pragma unroll
     for (int u = 0; u < NQ; ++u) pk_q[u] = pair_of(round, q_row0 + u * QRS);
@@ -205,28 +213,25 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
     for (int u = 0; u < NO; ++u) pk_o[u] = pair_of(round, o_row0 + u * ORS);
     pk_r = pair_of(round, tid);
   };
-  auto fetch = [&]() {
+  auto fetch = [&](int round) {  // gathers of `round`, whose pairs load_pairs(round) fetched
 #pragma unroll
     for (int u = 0; u < NQ; ++u) {
-      xq[u] = make_uint4(0, 0, 0, 0);
-      if (pk_q[u] != 0xffffffffu)
-        xq[u] = *(const uint4*)(q + ((b * dm.L + (pk_q[u] >> 8)) * (long)dm.HQ + hk * G + (q_row0 + u * QRS) % G) * D + q_pc * 8);
+      // padding rows read the row of the chunk's first pair (finite values): their P is 0, so they add nothing
+      xq[u] = *(const uint4*)(q + ((b * dm.L + (pk_q[u] >> 8)) * (long)dm.HQ + hk * G + (q_row0 + u * QRS) % G) * D + q_pc * 8);
     }
 #pragma unroll
     for (int u = 0; u < NO; ++u) {
-      xo[u] = make_uint4(0, 0, 0, 0);
-      if (pk_o[u] != 0xffffffffu)
-        xo[u] = *(const uint4*)(d_o + ((b * dm.L + (pk_o[u] >> 8)) * (long)dm.HQ + hk * G + (o_row0 + u * ORS) % G) * DV + o_pc * 8);
+      xo[u] = *(const uint4*)(d_o + ((b * dm.L + (pk_o[u] >> 8)) * (long)dm.HQ + hk * G + (o_row0 + u * ORS) % G) * DV + o_pc * 8);
     }
-    r_l2 = INFINITY;  // padding rows: P = 0
-    r_w = 0.f;
-    r_dl = 0.f;
-    if (pk_r != 0xffffffffu) {
-      const long rowi = (b * dm.L + (pk_r >> 8)) * (long)dm.HQ + hk * G + tid % G;
-      r_l2 = lse[rowi * dm.K + (pk_r & 255)];
-      if (r_l2 == HILS_NEG_INF) r_l2 = INFINITY;
-      r_w = bf2f(weights[rowi * dm.NW + (pk_r & 255)]);
-      r_dl = delta[rowi * dm.NW + (pk_r & 255)];
+    {
+      // raw values; what a padding row gets instead is decided where they are staged, so that
+      // nothing here has to wait for a load
+      r_ok = pair_ok(round, tid);
+      const uint32_t pk = pk_r;
+      const long rowi = (b * dm.L + (pk >> 8)) * (long)dm.HQ + hk * G + tid % G;
+      r_l2 = lse[rowi * dm.K + (pk & 255)];
+      r_wb = weights[rowi * dm.NW + (pk & 255)];
+      r_dl = delta[rowi * dm.NW + (pk & 255)];
     }
   };
   // row-major copy + transposed copy (dwords of two neighbouring rows) of one 16-byte piece
@@ -249,26 +254,26 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
     *(uint32_t*)(dst + 3 * CS) = (ev1 >> 16) | (od1 & 0xffff0000u);
   };
   load_pairs(0);
-  fetch();
+  fetch(0);
   load_pairs(1);
 
   for (int round = 0; round < nround; ++round) {
-    __syncthreads();  // the previous round's staging is no longer read
+    lds_barrier();  // the previous round's staging is no longer read
 #pragma unroll
     for (int u = 0; u < NQ; ++u) stage_piece(xq[u], q_row0 + u * QRS, q_pc, QPP, q_rm, QROW, q_tr, D);
 #pragma unroll
     for (int u = 0; u < NO; ++u) stage_piece(xo[u], o_row0 + u * ORS, o_pc, OPP, o_rm, OROW, o_tr, DV);
-    if (tid < ROWS) {
-      row_lse[tid] = r_l2;
-      row_w[tid] = r_w;
-      row_delta[tid] = r_dl;
+    if (tid < ROWS) {  // padding rows and empty slots: P = 0
+      row_lse[tid] = (r_ok && r_l2 != HILS_NEG_INF) ? r_l2 : INFINITY;
+      row_w[tid] = r_ok ? bf2f(r_wb) : 0.f;
+      row_delta[tid] = r_ok ? r_dl : 0.f;
     }
-    // next round's gathers fly during this round's arithmetic
+    // next round's gathers fly during this round's arithmetic (the barrier below orders LDS only)
     if (round + 1 < nround) {
-      fetch();
+      fetch(round + 1);
       load_pairs(round + 2);
     }
-    __syncthreads();
+    lds_barrier();
     const int rows_here = ((npair - round * PPR < PPR) ? npair - round * PPR : PPR) * G;
 #pragma unroll
     for (int sub = 0; sub < NSUB; ++sub) {
