@@ -509,12 +509,10 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
       const int t = tile * QT + tid / G;
       const int tc = t < L ? t : L - 1;
       const long rix = (b * L + tc) * (long)dm.HQ + hk * G + tid % G;
-      const float ls = lse[rix];
-      const bool live = t < L && ls > -1e30f;
-      r_lse = live ? ls * HILS_LOG2E : 0.f;
+      r_lse = lse[rix];  // raw: what a dead row gets is decided in stash(), nothing waits for a load here
       r_del = delta_in[rix];
       const int left = tc - dm.window + 1;
-      r_cs = live ? (dm.expand ? floordiv(left, dm.chunk) * dm.chunk : left) : 2147483647;
+      r_cs = t < L ? (dm.expand ? floordiv(left, dm.chunk) * dm.chunk : left) : 2147483647;
     }
   };
   auto stash = [&]() {
@@ -525,9 +523,10 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     for (int i = 0; i < OPASS; ++i)
       lzm_stash_pair<VPITCH>(do_s, dot_s, 2 * (tid / OSEG + OPPP * i), tid % OSEG, dor[i][0], dor[i][1]);
     if (tid < 64) {
-      lse_s[tid] = r_lse;
+      const bool live = r_lse > -1e30f;  // rows with an empty window have lse = -inf
+      lse_s[tid] = live ? r_lse * HILS_LOG2E : 0.f;
       del_s[tid] = r_del;
-      cs_s[tid] = r_cs;
+      cs_s[tid] = live ? r_cs : 2147483647;
     }
   };
   f32x4_t acck[2][DT], accv[2][DVT];
