@@ -213,7 +213,9 @@ def test_sparse_attn_decode_one_workgroup_per_row(pkg, orc, dev, B, HQ, H, D, K,
                                               # stages per round, D = 128 with Dv = 64 (the staged queries fill
                                               # the output tile exactly) and the other head-dim pairs
                                               (2, 128, 4, 2, 128, 64, 8), (1, 256, 8, 4, 128, 64, 16),
-                                              (3, 192, 8, 8, 128, 64, 4), (1, 128, 16, 4, 64, 128, 8)])
+                                              (3, 192, 8, 8, 128, 64, 4), (1, 128, 16, 4, 64, 128, 8),
+                                              # an odd number of weight elements: the tensor's last one has no aligned dword
+                                              (1, 129, 3, 3, 64, 64, 8), (1, 67, 1, 1, 64, 64, 4)])
 def test_sparse_attn_mfma_path_matches_generic_path(pkg, orc, dev, B, L, HQ, H, D, Dv, K):
     """The chunk-regrouped MFMA kernel (workspace given) against the shape-generic kernel
     (workspace NULL) and the oracle, output and per-chunk LSE, through the C ABI."""
