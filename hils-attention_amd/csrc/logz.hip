@@ -366,7 +366,8 @@ logz_bwd_dk_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
 
   const int seg = tid % SEGS, rp0 = tid / SEGS;
   uint4 qr[NPASS][2];
-  float zo = 0.f, zc = 0.f;
+  float zo = 0.f, zc = 0.f;  // raw log_z and d_log_z of this thread's (row, chunk); zin: inside the limits
+  bool zin = false;
   auto fetch = [&](int tile) {
 #pragma unroll
     for (int i = 0; i < NPASS; ++i)
@@ -383,10 +384,11 @@ logz_bwd_dk_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
       const bool in = t < dm.L && cc < dm.N && cc < lz_limit(dm, t < dm.L ? t : 0);
       const long zi = ((b * dm.L + (t < dm.L ? t : dm.L - 1)) * (long)dm.HQ + hk * G + row % G) * dm.N +
                       (cc < dm.N ? cc : dm.N - 1);
-      const float lz = log_z[zi], dl = d_log_z[zi];
-      const bool ok = in && lz > -1e30f;
-      zo = ok ? lz * HILS_LOG2E : 0.f;
-      zc = ok ? dl * dm.sm_scale : 0.f;
+      // raw values: what a row outside the limits gets is decided in stash(), so that nothing
+      // here waits for a load (which would also wait for the query rows issued before it)
+      zo = log_z[zi];
+      zc = d_log_z[zi];
+      zin = in;
     }
   };
   auto stash = [&]() {
@@ -394,8 +396,9 @@ logz_bwd_dk_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     for (int i = 0; i < NPASS; ++i)
       lzm_stash_pair<PITCH>(q_s, qt_s, 2 * (rp0 + PPP * i), seg, qr[i][0], qr[i][1]);
     if (tid < 128) {
-      off_s[tid >> 6][tid & 63] = zo;
-      coef_s[tid >> 6][tid & 63] = zc;
+      const bool ok = zin && zo > -1e30f;
+      off_s[tid >> 6][tid & 63] = ok ? zo * HILS_LOG2E : 0.f;
+      coef_s[tid >> 6][tid & 63] = ok ? zc * dm.sm_scale : 0.f;
     }
   };
   f32x4_t acc[2][DT];
