@@ -109,13 +109,16 @@ logz_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
   const int nc = lz_limit(dm, t_last);  // chunks the workgroup walks
   const float sc2 = dm.sm_scale * HILS_LOG2E;
 
-  uint4 kr[NP];
+  // (a native vector type: an array of HIP's uint4 struct that lives across the loop's back edge
+  // is kept in scratch memory by the compiler)
+  typedef unsigned lz_u32x4 __attribute__((ext_vector_type(4)));
+  lz_u32x4 kr[NP];
   auto fetch = [&](int c) {
 #pragma unroll
     for (int i = 0; i < NP; ++i) {
       const int p = tid + 256 * i;
       const int tok = p / (D / 8), seg = p % (D / 8);
-      kr[i] = *(const uint4*)(k + ((b * dm.L + c * 64 + tok) * (long)dm.H + hk) * D + seg * 8);
+      kr[i] = *(const lz_u32x4*)(k + ((b * dm.L + c * 64 + tok) * (long)dm.H + hk) * D + seg * 8);
     }
   };
   auto stash = [&](int buf) {
@@ -123,7 +126,7 @@ logz_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     for (int i = 0; i < NP; ++i) {
       const int p = tid + 256 * i;
       const int tok = p / (D / 8), seg = p % (D / 8);
-      *(uint4*)(&k_s[buf][tok * PITCH + seg * 16]) = kr[i];
+      *(lz_u32x4*)(&k_s[buf][tok * PITCH + seg * 16]) = kr[i];
     }
   };
   if (nc > 0) {
