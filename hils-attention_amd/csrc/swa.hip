@@ -70,29 +70,35 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
   }
   const float c2 = dm.sm_scale * HILS_LOG2E;
 
-  uint4 kr[KPASS], vr[VPASS][2];
+  // Prefetch registers: a native vector type (an array of HIP's uint4 struct that lives across
+  // the loop's back edge is kept in scratch memory) and loads without a branch around them (a
+  // load inside a branch is waited for at once).  Tokens past the end read the last row: their
+  // scores are masked and their probabilities are 0.
+  typedef unsigned swa_u32x4 __attribute__((ext_vector_type(4)));
+  swa_u32x4 kr[KPASS], vr[VPASS][2];
   auto fetch = [&](int tile) {
 #pragma unroll
     for (int i = 0; i < KPASS; ++i) {
       const int p = tid + 256 * i;
-      const int tok = tile * 64 + p / KSEG, seg = p % KSEG;
-      kr[i] = make_uint4(0, 0, 0, 0);
-      if (tok < dm.Lk) kr[i] = *(const uint4*)(k + ((b * dm.Lk + tok) * (long)dm.H + hk) * D + seg * 8);
+      int tok = tile * 64 + p / KSEG;
+      const int seg = p % KSEG;
+      tok = tok < dm.Lk ? tok : dm.Lk - 1;
+      kr[i] = *(const swa_u32x4*)(k + ((b * dm.Lk + tok) * (long)dm.H + hk) * D + seg * 8);
     }
 #pragma unroll
     for (int i = 0; i < VPASS; ++i)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const int tok = tile * 64 + 2 * (tid / VSEG + VPPP * i) + h;
-        vr[i][h] = make_uint4(0, 0, 0, 0);
-        if (tok < dm.Lk) vr[i][h] = *(const uint4*)(v + ((b * dm.Lk + tok) * (long)dm.H + hk) * DV + (tid % VSEG) * 8);
+        int tok = tile * 64 + 2 * (tid / VSEG + VPPP * i) + h;
+        tok = tok < dm.Lk ? tok : dm.Lk - 1;
+        vr[i][h] = *(const swa_u32x4*)(v + ((b * dm.Lk + tok) * (long)dm.H + hk) * DV + (tid % VSEG) * 8);
       }
   };
   auto stash = [&]() {
 #pragma unroll
     for (int i = 0; i < KPASS; ++i) {
       const int p = tid + 256 * i;
-      *(uint4*)(k_s + (p / KSEG) * PITCH + (p % KSEG) * 16) = kr[i];
+      *(swa_u32x4*)(k_s + (p / KSEG) * PITCH + (p % KSEG) * 16) = kr[i];
     }
 #pragma unroll
     for (int i = 0; i < VPASS; ++i) {
@@ -332,32 +338,36 @@ swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, cons
   }
   const float c2 = dm.sm_scale * HILS_LOG2E;
 
-  uint4 kr[KPASS][2], vr[VPASS];
+  // prefetch registers as in the forward kernel: native vectors, loads without branches, tokens
+  // past the end read the last row (their probabilities are masked to 0)
+  typedef unsigned swa_u32x4 __attribute__((ext_vector_type(4)));
+  swa_u32x4 kr[KPASS][2], vr[VPASS];
+  auto as_uint4 = [](const swa_u32x4& x) { return make_uint4(x.x, x.y, x.z, x.w); };
   auto fetch = [&](int tile) {
 #pragma unroll
     for (int i = 0; i < KPASS; ++i)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const int tok = tile * 64 + 2 * (tid / KSEG + KPPP * i) + h;
-        kr[i][h] = make_uint4(0, 0, 0, 0);
-        if (tok < L) kr[i][h] = *(const uint4*)(k + ((b * L + tok) * (long)dm.H + hk) * D + (tid % KSEG) * 8);
+        int tok = tile * 64 + 2 * (tid / KSEG + KPPP * i) + h;
+        tok = tok < L ? tok : L - 1;
+        kr[i][h] = *(const swa_u32x4*)(k + ((b * L + tok) * (long)dm.H + hk) * D + (tid % KSEG) * 8);
       }
 #pragma unroll
     for (int i = 0; i < VPASS; ++i) {
       const int p = tid + 256 * i;
-      const int tok = tile * 64 + p / VSEG;
-      vr[i] = make_uint4(0, 0, 0, 0);
-      if (tok < L) vr[i] = *(const uint4*)(v + ((b * L + tok) * (long)dm.H + hk) * DV + (p % VSEG) * 8);
+      int tok = tile * 64 + p / VSEG;
+      tok = tok < L ? tok : L - 1;
+      vr[i] = *(const swa_u32x4*)(v + ((b * L + tok) * (long)dm.H + hk) * DV + (p % VSEG) * 8);
     }
   };
   auto stash = [&]() {
 #pragma unroll
     for (int i = 0; i < KPASS; ++i)
-      lzm_stash_pair<PITCH>(k_s, kt_s, 2 * (tid / KSEG + KPPP * i), tid % KSEG, kr[i][0], kr[i][1]);
+      lzm_stash_pair<PITCH>(k_s, kt_s, 2 * (tid / KSEG + KPPP * i), tid % KSEG, as_uint4(kr[i][0]), as_uint4(kr[i][1]));
 #pragma unroll
     for (int i = 0; i < VPASS; ++i) {
       const int p = tid + 256 * i;
-      *(uint4*)(v_s + (p / VSEG) * VPITCH + (p % VSEG) * 16) = vr[i];
+      *(swa_u32x4*)(v_s + (p / VSEG) * VPITCH + (p % VSEG) * 16) = vr[i];
     }
   };
   f32x4_t acc[SWA_RT][DT];
