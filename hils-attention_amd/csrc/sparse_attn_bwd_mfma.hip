@@ -782,8 +782,8 @@ int hils_bw_run(const void* q, const void* k, const void* v, const void* weights
     int T = bq_pick_T(L, G, D, K, nchunk, &smem);
     if (T == 0) return -1;
     // small problems: rather every compute unit busy than the largest blocks
-    while (T >= 128 && (long)((L + T - 1) / T) * H * B < 256) {
-      T = (T / 2) & ~7;
+    while (T >= 72 && (long)((L + T - 1) / T) * H * B < 256) {
+      T -= 8;
       smem = (size_t)D * 4 + (size_t)nchunk * 4 + (size_t)T * ((size_t)G * D * 4 + (size_t)K * 4);
     }
     const int nblk = (L + T - 1) / T;
