@@ -1821,15 +1821,36 @@ topk_bwd_dlmk_kernel(const bf16_t* __restrict__ gs, const bf16_t* __restrict__ q
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   const long n_items = (long)(p_hi - p_lo) * g_n;
-  for (long it = grp; it < n_items; it += ngrp) {
-    const uint32_t pk = pairs[p_lo + it / g_n];
-    const int g = g_lo + (int)(it % g_n);
-    const long rg = (((b * L + (pk >> 8)) * h_kv + hk) * (long)G + g);
-    const float gv = bf2f(gs[rg * topk + (pk & 255)]) * sm_scale;
-    float f[8];
-    unpack8(*(const uint4*)(q + rg * D + pc * 8), f);
+  // four items per round: their pair entries, then their gradient and query loads, are in flight
+  // together (an item past the end re-reads the round's first item and counts for nothing)
+  constexpr int U = 4;
+  typedef unsigned tk_u32x4 __attribute__((ext_vector_type(4)));
+  for (long it = grp; it < n_items; it += (long)ngrp * U) {
+    uint32_t pk[U];
+    long itu[U];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = fmaf(gv, f[e], acc[e]);
+    for (int u = 0; u < U; ++u) {
+      const long i2 = it + (long)u * ngrp;
+      itu[u] = i2 < n_items ? i2 : it;
+      pk[u] = pairs[p_lo + itu[u] / g_n];
+    }
+    bf16_t gr[U];
+    tk_u32x4 qx[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int g = g_lo + (int)(itu[u] % g_n);
+      const long rg = (((b * L + (pk[u] >> 8)) * h_kv + hk) * (long)G + g);
+      gr[u] = gs[rg * topk + (pk[u] & 255)];
+      qx[u] = *(const tk_u32x4*)(q + rg * D + pc * 8);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float gv = (it + (long)u * ngrp < n_items) ? bf2f(gr[u]) * sm_scale : 0.f;
+      float f[8];
+      unpack8(make_uint4(qx[u].x, qx[u].y, qx[u].z, qx[u].w), f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = fmaf(gv, f[e], acc[e]);
+    }
   }
 #pragma unroll
   for (int e = 0; e < 8; ++e) red[(grp * pieces + pc) * 8 + e] = acc[e];
