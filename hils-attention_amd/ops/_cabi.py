@@ -98,9 +98,14 @@ def topk_fwd_workspace(device, B, L, N, h_kv, G):
     return torch.empty(n, dtype=torch.uint8, device=device)
 
 
+def sparse_attn_fwd_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n):
+    """Bytes of scratch hils_sparse_attn_fwd needs for this shape (0 = none)."""
+    return int(load().hils_sparse_attn_fwd_workspace(B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n))
+
+
 def sparse_attn_fwd_workspace(device, B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n):
     """Scratch tensor for hils_sparse_attn_fwd (None when the shape needs none)."""
-    n = load().hils_sparse_attn_fwd_workspace(B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n)
+    n = sparse_attn_fwd_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n)
     if n == 0:
         return None
     return torch.empty(n, dtype=torch.uint8, device=device)

@@ -6,6 +6,17 @@ import torch
 from . import _cabi
 
 
+def _check_kv_workspace(ws, need_bytes, device, what):
+    """The kernels index a caller-held workspace by the shape of the call it is passed to: one
+    packed for another (shorter) shape would be read and written past its end, so reject it."""
+    if (ws.device != device or ws.dtype != torch.uint8 or not ws.is_contiguous()
+            or ws.numel() < need_bytes):
+        raise ValueError(
+            f"kv_workspace must be a contiguous uint8 tensor on {device} of at least {need_bytes} "
+            f"bytes for this call ({what}); got {ws.dtype} x {ws.numel()} on {ws.device}.  Build it "
+            "with prepare_kv_workspace for this shape.")
+
+
 class _hils_block_M_attention_inverse(torch.autograd.Function):
     """Mirrors _hils_block_M_attention_inverse (ops/hils_fwd_bwd_head.py:771-913)."""
 
@@ -39,6 +50,10 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
             lse = torch.empty((B, L, HQ, K), dtype=torch.float32, device=q.device)
         ws_ready = 0
         if kv_workspace is not None:
+            need = _cabi.sparse_attn_fwd_workspace_bytes(B, L, L_kv, HQ, H, D, Dv, K, HQ, 1,
+                                                         int(block_size), 0.0)
+            _check_kv_workspace(kv_workspace, need, q.device,
+                                f"q_len {L}, kv_len {L_kv}, {HQ}/{H} heads, D {D}, Dv {Dv}, top-{K}")
             ws, ws_ready = kv_workspace, 1
         else:
             ws = _cabi.sparse_attn_fwd_workspace(q.device, B, L, L_kv, HQ, H, D, Dv, K, HQ, 1,

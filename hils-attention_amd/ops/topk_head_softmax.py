@@ -73,50 +73,49 @@ class SoftmaxTopKMaxPoolingFusedFn(torch.autograd.Function):
         return (dq, dlmk.to(k_in.dtype)) + (None,) * 12
 
 
+def _bias_per_group(bias, B, N, h_kv, G, device):
+    """Additive selection bias as a contiguous fp32 (B, N, h_kv, G) tensor, or None.
+    Accepts the flat per-query-head form (B, N, h_q) and the grouped form (B, N, h_kv, G)."""
+    if bias is None:
+        return None
+    want = {3: (B, N, h_kv * G), 4: (B, N, h_kv, G)}.get(bias.dim())
+    if want is None:
+        raise AssertionError(f"bias must be [B, S, h_q] or [B, S, h_kv, G], got {tuple(bias.shape)}")
+    assert tuple(bias.shape) == want, f"bias shape {tuple(bias.shape)} != {want}"
+    return bias.to(device=device, dtype=torch.float32).reshape(B, N, h_kv, G).contiguous()
+
+
+def _gumbel_rows(use_gumbel, noise, is_training, h_q, N, device):
+    """Gumbel noise per (query head, chunk) as fp32 (1, 1, h_q, N), or None when sampling is off.
+    Given noise is used as it is (no gradient); otherwise -log(-log(u)) is drawn here."""
+    if not use_gumbel and noise is None:
+        return None
+    assert is_training, "gumbel_noise is only supported in training mode"
+    want = (1, 1, h_q, N)
+    if noise is not None:
+        assert tuple(noise.shape) == want, f"gumbel_noise shape {tuple(noise.shape)} != {want}"
+        return noise.detach().to(device=device, dtype=torch.float32).contiguous()
+    u = torch.rand(want, device=device, dtype=torch.float32).clamp_(min=1e-20, max=1 - 1e-7)
+    return u.log_().neg_().log_().neg_()
+
+
 class SoftmaxTopKMaxPooling_Fused(torch.nn.Module):
-    """Mirrors SoftmaxTopKMaxPooling_Fused (ops/topk_head_softmax.py:1095-1207)."""
+    """Mirrors SoftmaxTopKMaxPooling_Fused (ops/topk_head_softmax.py:1095-1207): the selection
+    settings are fixed at construction, forward takes q (B,L,h_kv,G,D), chunk keys, lse_swa."""
 
     def __init__(self, topk, block_size, window_size, is_causal, is_training=True,
                  use_drop_mask=False, per_qhead_lmks=False):
         super().__init__()
-        self.topk = topk
-        self.block_size = block_size
-        self.window_size = window_size
-        self.is_causal = is_causal
-        self.is_training = is_training
-        self.use_drop_mask = use_drop_mask
-        self.per_qhead_lmks = per_qhead_lmks
+        self.topk, self.block_size, self.window_size = topk, block_size, window_size
+        self.is_causal, self.is_training = is_causal, is_training
+        self.use_drop_mask, self.per_qhead_lmks = use_drop_mask, per_qhead_lmks
 
     def forward(self, q, lmks, lse_swa, q_offset, drop_mask=None, sm_scale=None, bias=None,
                 use_gumbel=False, gumbel_noise=None, _debug=None):
         B, L, h_kv, G, D = q.shape
         N = lmks.shape[1]
-        bias_arg = None
-        if bias is not None:
-            bias_arg = bias.to(device=q.device, dtype=torch.float32)
-            if bias_arg.dim() == 3:
-                assert bias_arg.shape == (B, N, h_kv * G), (
-                    f"bias shape {tuple(bias_arg.shape)} != ({B}, {N}, {h_kv * G})")
-                bias_arg = bias_arg.reshape(B, N, h_kv, G).contiguous()
-            elif bias_arg.dim() == 4:
-                assert bias_arg.shape == (B, N, h_kv, G), (
-                    f"bias shape {tuple(bias_arg.shape)} != ({B}, {N}, {h_kv}, {G})")
-                bias_arg = bias_arg.contiguous()
-            else:
-                raise AssertionError(
-                    f"bias must be [B, S, h_q] or [B, S, h_kv, G], got {tuple(bias_arg.shape)}")
-        use_gumbel = bool(use_gumbel) or (gumbel_noise is not None)
-        gumbel_arg = None
-        if use_gumbel:
-            assert self.is_training, "gumbel_noise is only supported in training mode"
-            if gumbel_noise is None:
-                u = torch.rand(1, 1, h_kv * G, N, device=q.device, dtype=torch.float32)
-                u.clamp_(min=1e-20, max=1 - 1e-7)
-                gumbel_arg = -torch.log(-torch.log(u))
-            else:
-                assert gumbel_noise.shape == (1, 1, h_kv * G, N), (
-                    f"gumbel_noise shape {tuple(gumbel_noise.shape)} != ({1}, {1}, {h_kv * G}, {N})")
-                gumbel_arg = gumbel_noise.detach().to(device=q.device, dtype=torch.float32).contiguous()
+        bias_arg = _bias_per_group(bias, B, N, h_kv, G, q.device)
+        gumbel_arg = _gumbel_rows(use_gumbel, gumbel_noise, self.is_training, h_kv * G, N, q.device)
         # the reference's training-mode kernels take the query offset as 0 whatever is passed
         # (ops/topk_head_softmax.py:246,492)
         q_off = 0 if self.is_training else int(q_offset)
@@ -127,6 +126,37 @@ class SoftmaxTopKMaxPooling_Fused(torch.nn.Module):
 
 
 _SOFTMAX_MODULE_CACHE = {}
+
+
+def _group_heads(q, lmks, lse_swa, G):
+    """Bring the accepted input forms to one: q (B,L,h_kv,g,D), lmks (B,N,h_lmk,D), lse_swa
+    (B,L,h_kv,g), plus whether every query head has chunk keys of its own.
+
+    q may come flat (B,L,h_q,D) or grouped (B,L,h_kv,g,D).  Chunk keys whose last dimension is a
+    multiple of q's are split into that many heads.  ``G == 1``: the chunk keys are shared by the
+    heads of a group (h_lmk == h_kv; a flat q is grouped by h_q // h_lmk) or, for a grouped q
+    only, h_lmk == h_q selects per-head keys.  ``G > 1``: per-head keys, h_lmk == h_q, and q is
+    regrouped into h_q // G groups of G heads."""
+    B, L, D = q.shape[0], q.shape[1], q.shape[-1]
+    flat = q.dim() == 4
+    h_q = q.shape[2] if flat else q.shape[2] * q.shape[3]
+    if lmks.shape[3] != D:
+        assert lmks.shape[3] % D == 0, f"lmks D dim ({lmks.shape[3]}) must be divisible by q D dim ({D})"
+        lmks = lmks.reshape(lmks.shape[0], lmks.shape[1], -1, D)
+    h_lmk = lmks.shape[2]
+    if G > 1:
+        assert h_lmk == h_q, f"when G>1, lmks must have h_q ({h_q}) heads, got {h_lmk}"
+        assert h_q % G == 0, f"h_q ({h_q}) must be divisible by G ({G})"
+        h_kv, g, per_qhead = h_q // G, G, True
+    elif flat:
+        assert h_q % h_lmk == 0, f"h_q ({h_q}) must be divisible by lmks_h ({h_lmk})"
+        h_kv, g, per_qhead = h_lmk, h_q // h_lmk, False
+    else:
+        h_kv, g = q.shape[2], q.shape[3]
+        if h_lmk not in (h_kv, h_q):
+            raise AssertionError(f"lmks_h ({h_lmk}) must be h_kv ({h_kv}) or h_q ({h_q})")
+        per_qhead = h_lmk != h_kv
+    return q.reshape(B, L, h_kv, g, D), lmks, lse_swa.reshape(B, L, h_kv, g), per_qhead
 
 
 def online_softmax_topk_head(q, lmks, lse_swa, topk, block_size, window_size, is_causal=True,
@@ -142,60 +172,10 @@ def online_softmax_topk_head(q, lmks, lse_swa, topk, block_size, window_size, is
     ``_debug`` (a dict) additionally receives the fp32 ``sel_logits`` and ``lse_total`` the
     selection was made from.
     """
-    if q.dim() == 4:
-        B, L, h_q, D = q.shape
-        lmks_h = lmks.shape[2]
-        D_lmk = lmks.shape[3]
-        if D != D_lmk:
-            assert D_lmk % D == 0, f"lmks D dim ({D_lmk}) must be divisible by q D dim ({D})"
-            d_ratio = D_lmk // D
-            lmks = lmks.reshape(lmks.shape[0], lmks.shape[1], lmks_h * d_ratio, D)
-            lmks_h = lmks_h * d_ratio
-        if G == 1:
-            assert h_q % lmks_h == 0, f"h_q ({h_q}) must be divisible by lmks_h ({lmks_h})"
-            h_kv = lmks_h
-            G_eff = h_q // h_kv
-            per_qhead_lmks = False
-        else:
-            assert lmks_h == h_q, f"when G>1, lmks must have h_q ({h_q}) heads, got {lmks_h}"
-            assert h_q % G == 0, f"h_q ({h_q}) must be divisible by G ({G})"
-            h_kv = h_q // G
-            G_eff = G
-            per_qhead_lmks = True
-        q = q.view(B, L, h_kv, G_eff, D)
-    else:
-        B, L, h_kv, G_in, D = q.shape
-        h_q = h_kv * G_in
-        D_lmk = lmks.shape[3]
-        if D != D_lmk:
-            assert D_lmk % D == 0, f"lmks D dim ({D_lmk}) must be divisible by q D dim ({D})"
-            d_ratio = D_lmk // D
-            lmks = lmks.reshape(lmks.shape[0], lmks.shape[1], lmks.shape[2] * d_ratio, D)
-        lmks_h = lmks.shape[2]
-        if G == 1:
-            if lmks_h == h_kv:
-                per_qhead_lmks = False
-            elif lmks_h == h_q:
-                per_qhead_lmks = True
-            else:
-                raise AssertionError(f"lmks_h ({lmks_h}) must be h_kv ({h_kv}) or h_q ({h_q})")
-            G_eff = G_in
-        else:
-            assert lmks_h == h_q, f"when G>1, lmks must have h_q ({h_q}) heads, got {lmks_h}"
-            assert h_q % G == 0, f"h_q ({h_q}) must be divisible by G ({G})"
-            new_h_kv = h_q // G
-            if (new_h_kv != h_kv) or (G != G_in):
-                q = q.reshape(B, L, new_h_kv, G, D)
-                h_kv = new_h_kv
-            G_eff = G
-            per_qhead_lmks = True
-    lse_swa = lse_swa.reshape(B, L, h_kv, G_eff)
-    use_drop_mask = drop_mask is not None
-    cache_key = (topk, block_size, window_size, is_causal, is_training, use_drop_mask, per_qhead_lmks)
-    mod = _SOFTMAX_MODULE_CACHE.get(cache_key)
+    q, lmks, lse_swa, per_qhead = _group_heads(q, lmks, lse_swa, G)
+    key = (topk, block_size, window_size, is_causal, is_training, drop_mask is not None, per_qhead)
+    mod = _SOFTMAX_MODULE_CACHE.get(key)
     if mod is None:
-        mod = _SOFTMAX_MODULE_CACHE[cache_key] = SoftmaxTopKMaxPooling_Fused(
-            topk, block_size, window_size, is_causal, is_training, use_drop_mask,
-            per_qhead_lmks=per_qhead_lmks)
+        mod = _SOFTMAX_MODULE_CACHE[key] = SoftmaxTopKMaxPooling_Fused(*key)
     return mod(q, lmks, lse_swa, q_offset=q_offset, drop_mask=drop_mask, sm_scale=sm_scale,
                bias=bias, use_gumbel=use_gumbel, gumbel_noise=gumbel_noise, _debug=_debug)

@@ -11,9 +11,14 @@ import math
 
 import torch
 
-from ..ops.chunk_attn_pool_tilelang import chunk_mean_pool
-from ..ops.hils_fwd_bwd_head import HiLS_block_M_head
-from ..ops.hils_glue import topk_chunk_weights
+try:  # imported as part of the package ...
+    from ..ops.chunk_attn_pool_tilelang import chunk_mean_pool
+    from ..ops.hils_fwd_bwd_head import HiLS_block_M_head
+    from ..ops.hils_glue import topk_chunk_weights
+except ImportError:  # ... or with the package directory itself on sys.path (`from utils... import`)
+    from ops.chunk_attn_pool_tilelang import chunk_mean_pool
+    from ops.hils_fwd_bwd_head import HiLS_block_M_head
+    from ops.hils_glue import topk_chunk_weights
 
 
 class HiLSDynamicLayer:

@@ -38,7 +38,9 @@ lives in tests/test_oracle_*.py):
 
 * every function is pinned by closed forms, library routines
   (``F.scaled_dot_product_attention``, ``torch.distributions.Categorical``,
-  ``torch.topk``) and brute force on tiny inputs;
+  ``torch.topk``) and brute force on tiny inputs, including the option branches
+  (in-chunk slope of ``sparse_attn``, Gumbel noise of ``select_logits``, per-query-head
+  chunk keys of ``topk_logits``), each against a pure-Python enumeration;
 * the reference stores no golden vectors for this path, so none are used;
 * the tie-break of ``topk_select`` is pinned only by the reference's kernel text.
 """

@@ -103,3 +103,86 @@ def test_package_does_not_import_the_oracle():
             if f.endswith(".py"):
                 text = open(os.path.join(root, f)).read()
                 assert "oracle" not in text.replace("no oracle", ""), f"{f} mentions the oracle"
+
+
+def test_topk_head_grouping_forms(pkg):
+    """The accepted q / chunk-key / lse_swa forms all reduce to (B,L,h_kv,g,D) + (B,L,h_kv,g)."""
+    from hils_attention_amd.ops.topk_head_softmax import _group_heads, _bias_per_group, _gumbel_rows
+    B, L, N, D = 2, 8, 3, 16
+    lse3 = torch.zeros(B, L, 8)
+    # flat q, shared keys: groups follow the chunk keys' head count
+    q, lm, lse, per = _group_heads(torch.zeros(B, L, 8, D), torch.zeros(B, N, 2, D), lse3, 1)
+    assert q.shape == (B, L, 2, 4, D) and lse.shape == (B, L, 2, 4) and not per and lm.shape == (B, N, 2, D)
+    # flat q, per-head keys with G given
+    q, lm, lse, per = _group_heads(torch.zeros(B, L, 8, D), torch.zeros(B, N, 8, D), lse3, 4)
+    assert q.shape == (B, L, 2, 4, D) and per
+    # grouped q: the keys' head count decides; G > 1 regroups
+    q, _, _, per = _group_heads(torch.zeros(B, L, 2, 4, D), torch.zeros(B, N, 2, D), lse3, 1)
+    assert q.shape == (B, L, 2, 4, D) and not per
+    q, _, _, per = _group_heads(torch.zeros(B, L, 2, 4, D), torch.zeros(B, N, 8, D), lse3, 1)
+    assert q.shape == (B, L, 2, 4, D) and per
+    q, _, lse, per = _group_heads(torch.zeros(B, L, 2, 4, D), torch.zeros(B, N, 8, D), lse3.view(B, L, 2, 4), 2)
+    assert q.shape == (B, L, 4, 2, D) and lse.shape == (B, L, 4, 2) and per
+    # chunk keys with a multiple of q's head dim are split into heads
+    q, lm, _, per = _group_heads(torch.zeros(B, L, 8, D), torch.zeros(B, N, 1, 2 * D), lse3, 1)
+    assert lm.shape == (B, N, 2, D) and q.shape == (B, L, 2, 4, D)
+    with pytest.raises(AssertionError, match="must be h_kv"):
+        _group_heads(torch.zeros(B, L, 2, 4, D), torch.zeros(B, N, 3, D), lse3, 1)
+    with pytest.raises(AssertionError, match="divisible by q D"):
+        _group_heads(torch.zeros(B, L, 8, D), torch.zeros(B, N, 2, D + 8), lse3, 1)
+    # bias forms
+    b = _bias_per_group(torch.arange(B * N * 8.0).view(B, N, 8), B, N, 2, 4, "cpu")
+    assert b.shape == (B, N, 2, 4) and b.dtype == torch.float32 and b[1, 2, 1, 3] == B * N * 8 - 1
+    assert _bias_per_group(None, B, N, 2, 4, "cpu") is None
+    with pytest.raises(AssertionError, match="bias shape"):
+        _bias_per_group(torch.zeros(B, N, 7), B, N, 2, 4, "cpu")
+    with pytest.raises(AssertionError, match="bias must be"):
+        _bias_per_group(torch.zeros(B, N), B, N, 2, 4, "cpu")
+    # Gumbel noise: off, given, drawn; training only
+    assert _gumbel_rows(False, None, True, 8, N, "cpu") is None
+    g = torch.randn(1, 1, 8, N)
+    assert torch.equal(_gumbel_rows(False, g, True, 8, N, "cpu"), g)
+    d = _gumbel_rows(True, None, True, 8, N, "cpu")
+    assert d.shape == (1, 1, 8, N) and torch.isfinite(d).all()
+    with pytest.raises(AssertionError, match="training"):
+        _gumbel_rows(True, None, False, 8, N, "cpu")
+    with pytest.raises(AssertionError, match="gumbel_noise shape"):
+        _gumbel_rows(False, torch.zeros(1, 1, 4, N), True, 8, N, "cpu")
+
+
+def test_drop_in_route_imports_in_a_fresh_interpreter():
+    """With only the package directory on sys.path, every module the reference's layer imports
+    (`from ops.X import Y`, `from utils.hils_cache_utils import HiLSDynamicLayer`) resolves."""
+    import subprocess
+    import sys
+    code = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "from ops.hils_fwd_bwd_head import HiLS_block_M_head, prepare_kv_workspace\n"
+        "from ops.topk_head_softmax import online_softmax_topk_head, SoftmaxTopKMaxPooling_Fused\n"
+        "from ops.chunk_attn_pool_tilelang import chunk_attn_pool_tilelang, chunk_attn_pool_tilelang_shared_k, chunk_mean_pool\n"
+        "from ops.exact_chunk_log_z_tilelang import exact_chunk_log_z_tl\n"
+        "from ops.hsa_triton import HSA\n"
+        "from ops.flex_attn_tilelang import flex_attn_tl, flex_attn_tl_two_phase\n"
+        "from ops.rope_tilelang_fp32 import rope_rotary_pos_emb, single_tensor_rope_autograd\n"
+        "from ops.hils_glue import chunk_weights, topk_chunk_weights\n"
+        "from utils.hils_cache_utils import HiLSDynamicLayer\n"
+        "print('imports ok')\n" % entry.PKG_DIR)
+    res = subprocess.run([sys.executable, "-c", code], cwd="/tmp", capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0 and "imports ok" in res.stdout, res.stderr
+
+
+def test_short_or_foreign_kv_workspace_is_rejected(pkg):
+    """A packed-K/V workspace built for a shorter call must not reach the kernel."""
+    from hils_attention_amd.ops import _cabi
+    from hils_attention_amd.ops.hils_fwd_bwd_head import _check_kv_workspace
+    small = _cabi.sparse_attn_fwd_workspace_bytes(1, 1024, 1024, 8, 2, 128, 128, 8, 8, 1, 64, 0.0)
+    large = _cabi.sparse_attn_fwd_workspace_bytes(1, 4096, 4096, 8, 2, 128, 128, 8, 8, 1, 64, 0.0)
+    assert 0 < small < large
+    cpu = torch.device("cpu")
+    _check_kv_workspace(torch.empty(large, dtype=torch.uint8), large, cpu, "ok")
+    with pytest.raises(ValueError, match="at least"):
+        _check_kv_workspace(torch.empty(small, dtype=torch.uint8), large, cpu, "short")
+    with pytest.raises(ValueError, match="uint8"):
+        _check_kv_workspace(torch.empty(large, dtype=torch.int8), large, cpu, "dtype")
+    with pytest.raises(ValueError, match="kv_workspace"):
+        _check_kv_workspace(torch.empty(large, dtype=torch.uint8), large, torch.device("meta"), "device")

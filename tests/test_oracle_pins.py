@@ -173,6 +173,68 @@ def test_topk_select_is_exact_on_given_scores(orc):
     assert orc.topk_select(tie, torch.zeros(1, 1, 1, 1), None, 2).tolist() == [[[[0, 1]]]]
 
 
+def test_topk_gumbel_and_per_qhead_keys_brute_force(orc):
+    """Two option branches of the selection, each against a pure-Python enumeration.
+
+    Gumbel noise g[h_q, c] is added to the scaled logit of (query head, chunk) before both the
+    LSE and the selection (ops/topk_head_softmax.py:47-52 in the torch reference), the returned
+    scores stay raw.  Per-q-head chunk keys (B,N,h_kv*G,D): head h*G+g of the keys scores query
+    head (h, g); selection is still per KV head with the max over g."""
+    torch.manual_seed(21)
+    B, L, h_kv, G, D, N, S, topk, W = 1, 36, 2, 3, 8, 9, 4, 3, 1
+    scale = 1.0 / math.sqrt(D)
+    q = torch.randn(B, L, h_kv, G, D)
+    lse = torch.randn(B, L, h_kv * G)
+    shared = torch.randn(B, N, h_kv, D)
+    per_head = torch.randn(B, N, h_kv * G, D)
+    # the noise is large against the logits' spread, so it changes most selections
+    noise = torch.randn(1, 1, h_kv * G, N) * 3
+
+    def brute(lmks, per_qhead, gum):
+        out = torch.full((B, L, h_kv, topk), -1, dtype=torch.int32)
+        raw = torch.full((B, L, h_kv, G, N), float("nan"), dtype=torch.float64)
+        for t, h in itertools.product(range(L), range(h_kv)):
+            vis = list(range(max(0, (t - W + 1) // S)))
+            if not vis:
+                continue
+            pooled = {c: -math.inf for c in vis}
+            for g in range(G):
+                hq = h * G + g
+                lg = []
+                for c in vis:
+                    key = lmks[0, c, hq] if per_qhead else lmks[0, c, h]
+                    r = float(torch.dot(q[0, t, h, g].double(), key.double())) * scale
+                    raw[0, t, h, g, c] = r
+                    lg.append(r + (float(gum[0, 0, hq, c]) if gum is not None else 0.0))
+                lt = math.log(math.exp(float(lse[0, t, hq])) + sum(math.exp(x) for x in lg))
+                for c, x in zip(vis, lg):
+                    pooled[c] = max(pooled[c], x - lt)
+            sel = sorted(sorted(vis, key=lambda c: (-pooled[c], c))[:topk])
+            out[0, t, h, :len(sel)] = torch.tensor(sel, dtype=torch.int32)
+        return out, raw
+
+    plain, _ = orc.online_softmax_topk_head(q, shared, lse, topk, S, W)
+    for lmks, per_qhead, gum in [(shared, False, noise), (per_head, True, None), (per_head, True, noise)]:
+        idx, scores = orc.online_softmax_topk_head(q, lmks, lse, topk, S, W, gumbel_noise=gum)
+        want, raw = brute(lmks, per_qhead, gum)
+        assert torch.equal(idx, want), (per_qhead, gum is not None)
+        for t in (17, 35):
+            for h, g in itertools.product(range(h_kv), range(G)):
+                for j, c in enumerate(idx[0, t, h].tolist()):
+                    if c >= 0:  # raw scaled product: no noise in the returned score
+                        assert scores[0, t, h, g, j].item() == pytest.approx(raw[0, t, h, g, c].item(), abs=1e-5)
+    assert not torch.equal(orc.online_softmax_topk_head(q, shared, lse, topk, S, W, gumbel_noise=noise)[0], plain), \
+        "the noise must take part in the selection"
+    # a per-head key tensor that repeats the shared keys selects what the shared keys select
+    rep = shared.repeat_interleave(G, dim=2)
+    assert torch.equal(orc.online_softmax_topk_head(q, rep, lse, topk, S, W)[0], plain)
+    # swapping two heads' keys inside a group must matter (head h*G+g belongs to (h, g), not (g, h))
+    swapped = per_head.clone()
+    swapped[:, :, [0, 1]] = per_head[:, :, [1, 0]]
+    assert not torch.equal(orc.online_softmax_topk_head(q, swapped, lse, topk, S, W)[0],
+                           orc.online_softmax_topk_head(q, per_head, lse, topk, S, W)[0])
+
+
 # ------------------------------------------------------------------ sparse attention
 def test_sparse_attn_textbook_and_properties(orc):
     torch.manual_seed(5)
@@ -215,6 +277,51 @@ def test_sparse_attn_textbook_and_properties(orc):
         assert lse[0, t, hq, j].item() == pytest.approx(torch.logsumexp(s, 0).item(), abs=1e-5)
         acc += w1[0, t, hq, j] * (torch.softmax(s, 0) @ v[0, c * S:c * S + S - 1, hq // 2])
     assert torch.allclose(o1[0, t, hq], acc, atol=1e-5)
+
+
+def test_sparse_attn_slope_brute_force(orc):
+    """ALiBi-like slope inside a chunk: -slope[h_q] * max(0, (S - 2) - s) is added to the raw
+    q.k of token s BEFORE the scale (ops/hils_fwd_bwd_head.py:68-76), so the last unmasked token
+    (s = S - 2) gets no penalty and token 0 the largest.  Pure-Python loop per (query, head)."""
+    torch.manual_seed(22)
+    B, L, HQ, H, D, S, K = 1, 96, 4, 2, 8, 16, 2
+    G = HQ // H
+    q, k, v = torch.randn(B, L, HQ, D), torch.randn(B, L, H, D), torch.randn(B, L, H, D)
+    slope = torch.tensor([0.05, 0.2, 0.7, 1.5])
+    gen = torch.Generator().manual_seed(23)
+    idx = rand_indices(B, L, H, K, S, gen, fill_prob=0.8)
+    w = torch.rand(B, L, HQ, K)
+    scale = 0.3
+    for mask_last in (True, False):
+        o, lse = orc.sparse_attn(q, k, v, w, idx, chunk_size=S, sm_scale=scale, slope=slope,
+                                 mask_last_token=mask_last, return_lse=True)
+        for t in (20, 50, 95):
+            for hq in range(HQ):
+                acc = [0.0] * D
+                for j, c in enumerate(idx[0, t, hq // G].tolist()):
+                    if c < 0:
+                        continue
+                    ntok = S - 1 if mask_last else S
+                    logit = []
+                    for s_ in range(ntok):
+                        dot = sum(float(q[0, t, hq, d]) * float(k[0, c * S + s_, hq // G, d]) for d in range(D))
+                        logit.append((dot - float(slope[hq]) * max(0, S - 2 - s_)) * scale)
+                    m = max(logit)
+                    z = sum(math.exp(x - m) for x in logit)
+                    assert lse[0, t, hq, j].item() == pytest.approx(m + math.log(z), abs=1e-4)
+                    for s_ in range(ntok):
+                        p = math.exp(logit[s_] - m) / z
+                        for d in range(D):
+                            acc[d] += float(w[0, t, hq, j]) * p * float(v[0, c * S + s_, hq // G, d])
+                assert torch.allclose(o[0, t, hq], torch.tensor(acc), atol=1e-4)
+    # slope 0 is the plain operator; a large slope concentrates the mass on the last unmasked token
+    o0 = orc.sparse_attn(q, k, v, w, idx, chunk_size=S, sm_scale=scale, slope=torch.zeros(HQ))
+    assert torch.allclose(o0, orc.sparse_attn(q, k, v, w, idx, chunk_size=S, sm_scale=scale), atol=1e-6)
+    one = torch.full((B, L, H, 1), 1, dtype=torch.int32)
+    o_big = orc.sparse_attn(q, k, v, torch.ones(B, L, HQ, 1), one, chunk_size=S, sm_scale=scale,
+                            slope=torch.full((HQ,), 1e4))
+    want = v[0, S + S - 2].repeat_interleave(G, 0)  # token S-2 of chunk 1
+    assert torch.allclose(o_big[0, 40], want, atol=1e-4)
 
 
 def test_factorised_equals_dense_when_weights_are_true_masses(orc):

@@ -37,6 +37,9 @@ def errors(out, ref):
 
 def assert_close_bf16(out, ref, name="", max_abs=MAX_ABS, rel_l2=REL_L2):
     ma, scale, rel = errors(out, ref)
+    # the unscaled figure, beside the bar it is held to (max_abs * max(1, max|ref|))
+    note(f"    {name or 'tensor'}: max-abs {ma:.3e} (unscaled; max|ref| {scale:.3g}, bar {max_abs * scale:.3e}), "
+         f"rel-L2 {rel:.3e}")
     assert ma <= max_abs * scale, f"{name}: max-abs {ma:.4e} > {max_abs} * {scale:.3g}"
     assert rel <= rel_l2, f"{name}: rel-L2 {rel:.4e} > {rel_l2}"
     return ma, rel
