@@ -135,16 +135,23 @@ def bench_prefill(pkg, dev, steps, warmup):
     return sec, per, roof, cfg, data
 
 
+def config2_inputs(dev):
+    """Config 2 inputs: B4 L8192, 16 heads MHA, D64; q, k, v ~ N(0,1) (seed 1002), lse_swa = the
+    exact lse of the query's own chunk, in bf16 as the layer hands it over."""
+    B, L, HQ, H, D, S = 4, 8192, 16, 16, 64, 64
+    gen = torch.Generator(device=dev).manual_seed(1002)
+    q = gpu_randn((B, L, HQ, D), gen, dev)
+    k = gpu_randn((B, L, H, D), gen, dev)
+    v = gpu_randn((B, L, H, D), gen, dev)
+    return q, k, v, swa_lse_current_chunk(q, k, S).bfloat16()
+
+
 def bench_config2(pkg, dev, iters=5):
     """Config 2: B4 L8192, 16 heads MHA, D64, top-32: the same forward step as the headline
     (mean pool -> top-k -> inter-chunk softmax -> K/V packing -> sparse attention)."""
     from hils_attention_amd.ops import hils_fwd_bwd_head as attn_mod
     B, L, HQ, H, D, S, K, W = 4, 8192, 16, 16, 64, 64, 32, 1
-    gen = torch.Generator(device=dev).manual_seed(1002)
-    q = gpu_randn((B, L, HQ, D), gen, dev)
-    k = gpu_randn((B, L, H, D), gen, dev)
-    v = gpu_randn((B, L, H, D), gen, dev)
-    lse_swa = swa_lse_current_chunk(q, k, S).bfloat16()
+    q, k, v, lse_swa = config2_inputs(dev)
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
     t_all = t_attn = 0.0
     n_sel = 0
@@ -228,23 +235,38 @@ def bench_decode(pkg, dev, steps, warmup):
     return sec, per, roof
 
 
-def bench_train(pkg, dev, iters=3):
-    """Config 5: 345M-shaped training layer, forward + backward (B8 L8192, 16 heads MHA, D64, top-32):
-    mean pool -> top-k scores -> softmax over [scores, lse_swa] (torch autograd) -> sparse attention,
-    gradients to q, k, v through every op."""
-    B, L, HQ, H, D, S, K, W = 8, 8192, 16, 16, 64, 64, 32, 1
+def train_inputs(dev):
+    """Config 5 inputs: B8 L8192, 16 heads MHA, D64; q, k, v (leaves that require grad) and the
+    upstream gradient d_o ~ N(0,1) (seed 1005), lse_swa = the exact fp32 lse of the own chunk."""
+    B, L, HQ, H, D, S = 8, 8192, 16, 16, 64, 64
     gen = torch.Generator(device=dev).manual_seed(1005)
     q = gpu_randn((B, L, HQ, D), gen, dev).requires_grad_()
     k = gpu_randn((B, L, H, D), gen, dev).requires_grad_()
     v = gpu_randn((B, L, H, D), gen, dev).requires_grad_()
     d_o = gpu_randn((B, L, HQ, D), gen, dev)
-    lse_swa = swa_lse_current_chunk(q.detach(), k.detach(), S)
+    return q, k, v, d_o, swa_lse_current_chunk(q.detach(), k.detach(), S)
+
+
+def train_forward(pkg, q, k, v, lse_swa, keep=False):
+    """The training layer's remote branch: mean pool -> top-k scores -> softmax over
+    [scores, lse_swa] -> sparse attention.  Returns (o, idx), plus scores and weights with keep."""
+    S, K, W = 64, 32, 1
+    lmk = pkg.chunk_mean_pool(k, S)
+    idx, scores = pkg.online_softmax_topk_head(q, lmk, lse_swa, K, S, W, is_training=True)
+    w = pkg.chunk_weights(scores, lse_swa)
+    o = pkg.HiLS_block_M_head(q, k, v, w, idx, block_size=S, is_training=True)
+    return (o, idx, scores, w) if keep else (o, idx)
+
+
+def bench_train(pkg, dev, iters=3):
+    """Config 5: 345M-shaped training layer, forward + backward (B8 L8192, 16 heads MHA, D64, top-32):
+    mean pool -> top-k scores -> softmax over [scores, lse_swa] -> sparse attention, gradients to
+    q, k, v through every op."""
+    B, L, HQ, H, D, S, K, W = 8, 8192, 16, 16, 64, 64, 32, 1
+    q, k, v, d_o, lse_swa = train_inputs(dev)
 
     def fwd():
-        lmk = pkg.chunk_mean_pool(k, S)
-        idx, scores = pkg.online_softmax_topk_head(q, lmk, lse_swa, K, S, W, is_training=True)
-        w = torch.softmax(torch.cat([scores.float(), lse_swa.unsqueeze(-1)], -1), -1).to(q.dtype)
-        return pkg.HiLS_block_M_head(q, k, v, w, idx, block_size=S, is_training=True), idx
+        return train_forward(pkg, q, k, v, lse_swa)
 
     def fwd_bwd():
         for t in (q, k, v):

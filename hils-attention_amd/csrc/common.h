@@ -29,6 +29,19 @@ void hils_set_error(const char* fmt, ...);
     }                                                                      \
   } while (0)
 
+// Compute units of the current device (cached per device; no stream operation, so it is safe
+// under HIP graph capture).
+int hils_device_cus();
+
+// Raise a kernel's dynamic-LDS limit to `bytes` on the current device if it is not there yet.
+// One HilsLdsReserve per kernel instantiation (a function-local static); thread-safe, per device.
+#ifdef __cplusplus
+#include <atomic>
+#define HILS_LDS_RESERVE_DEVICES 64
+struct HilsLdsReserve { std::atomic<size_t> bytes[HILS_LDS_RESERVE_DEVICES]; };
+int hils_reserve_lds(HilsLdsReserve* state, const void* kernel, size_t bytes, const char* who);
+#endif
+
 typedef unsigned short bf16_t;  // raw bfloat16 bits
 
 #define HILS_NEG_INF (-INFINITY)

@@ -159,3 +159,96 @@ extern "C" int hils_chunk_weights(const void* scores, const void* lse_swa, int l
   HILS_CHECK_LAUNCH("hils_chunk_weights");
   return HILS_OK;
 }
+
+// Backward of the inter-chunk softmax.  One thread per (batch, query, query head) row: the logits
+// are rebuilt from the forward's inputs (so the probabilities are the unrounded fp32 ones the
+// reference's autograd uses), then d_logit_j = y_j * (d_w_j - sum_i y_i d_w_i).  Columns: K chunk
+// scores, the local-branch LSE, and with softmax1 a constant zero logit (no gradient).
+__global__ void __launch_bounds__(256)
+chunk_weights_bwd_kernel(const bf16_t* __restrict__ scores, const void* __restrict__ lse_ptr, int lse_bf16,
+                         const float* __restrict__ prior_b, const int32_t* __restrict__ indices,
+                         const bf16_t* __restrict__ d_weights, bf16_t* __restrict__ d_scores,
+                         float* __restrict__ d_lse, float* __restrict__ d_prior_b, long rows, int L, int HQ,
+                         int H, int N, int K, int softmax1) {
+  const long row = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= rows) return;
+  const int hq = (int)(row % HQ);
+  const long bt = row / HQ;
+  const long b = bt / L;
+  const int G = HQ / H;
+  const bf16_t* srow = scores + row * K;
+  const int NW = K + 1 + (softmax1 ? 1 : 0);
+  const bf16_t* grow = d_weights + row * NW;
+  const int32_t* irow = indices ? indices + (bt * H + hq / G) * (long)K : nullptr;
+  float x[GL_MAXK];
+  const float lse_v = lse_bf16 ? bf2f(((const bf16_t*)lse_ptr)[row]) : ((const float*)lse_ptr)[row];
+  float m = softmax1 ? fmaxf(lse_v, 0.f) : lse_v;
+#pragma unroll
+  for (int k = 0; k < GL_MAXK; ++k) {
+    if (k < K) {
+      float s = bf2f(srow[k]);
+      if (prior_b) {
+        int c = irow[k];
+        c = c < 0 ? 0 : c;
+        s = bf2f(f2bf(s + bf2f(f2bf(prior_b[(b * N + c) * (long)HQ + hq]))));
+      }
+      x[k] = s;
+      m = fmaxf(m, s);
+    }
+  }
+  bf16_t* drow = d_scores + row * K;
+  if (m == HILS_NEG_INF) {  // forward gave NaN weights for this row
+    for (int k = 0; k < K; ++k) drow[k] = 0x7fc0;
+    if (d_lse) d_lse[row] = __uint_as_float(0x7fc00000u);
+    return;
+  }
+  float sum = 0.f, dot = 0.f;
+#pragma unroll
+  for (int k = 0; k < GL_MAXK; ++k)
+    if (k < K) {
+      x[k] = __expf(x[k] - m);
+      sum += x[k];
+      dot += x[k] * bf2f(grow[k]);
+    }
+  const float el = __expf(lse_v - m);
+  const float gl = bf2f(grow[K]);
+  sum += el;
+  dot += el * gl;
+  if (softmax1) {
+    const float e0 = __expf(0.f - m);
+    sum += e0;
+    dot += e0 * bf2f(grow[K + 1]);
+  }
+  const float inv = 1.f / sum;
+  dot *= inv;  // sum_i y_i d_w_i
+#pragma unroll
+  for (int k = 0; k < GL_MAXK; ++k)
+    if (k < K) {
+      const float dl = x[k] * inv * (bf2f(grow[k]) - dot);
+      drow[k] = f2bf(dl);
+      if (d_prior_b && dl != 0.f) {  // empty slots gather chunk 0, as the forward does (their dl is 0 when the score is -inf)
+        const int c = irow[k] < 0 ? 0 : irow[k];
+        atomicAdd(d_prior_b + (b * N + c) * (long)HQ + hq, dl);
+      }
+    }
+  if (d_lse) d_lse[row] = el * inv * (gl - dot);
+}
+
+extern "C" int hils_chunk_weights_bwd(const void* scores, const void* lse_swa, int lse_bf16,
+                                      const float* prior_b, const int32_t* indices, const void* d_weights,
+                                      void* d_scores, float* d_lse, float* d_prior_b, int B, int L, int HQ,
+                                      int H, int N, int K, int softmax1, void* stream) {
+  HILS_REQUIRE(scores && lse_swa && d_weights && d_scores, "hils_chunk_weights_bwd: null pointer");
+  HILS_REQUIRE(!prior_b || indices, "hils_chunk_weights_bwd: prior_b needs indices");
+  HILS_REQUIRE(!d_prior_b || prior_b, "hils_chunk_weights_bwd: d_prior_b needs prior_b");
+  HILS_REQUIRE(B > 0 && L > 0 && HQ > 0 && H > 0 && HQ % H == 0, "hils_chunk_weights_bwd: bad head counts");
+  HILS_REQUIRE(K >= 1 && K <= GL_MAXK, "hils_chunk_weights_bwd: K (%d) must be in 1..%d", K, GL_MAXK);
+  const long rows = (long)B * L * HQ;
+  const long nblk = (rows + 255) / 256;
+  HILS_REQUIRE(nblk <= 2147483647L, "hils_chunk_weights_bwd: grid too large");
+  hipLaunchKernelGGL(chunk_weights_bwd_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16_t*)scores, lse_swa, lse_bf16, prior_b, indices, (const bf16_t*)d_weights,
+                     (bf16_t*)d_scores, d_lse, d_prior_b, rows, L, HQ, H, N, K, softmax1);
+  HILS_CHECK_LAUNCH("hils_chunk_weights_bwd");
+  return HILS_OK;
+}

@@ -14,9 +14,9 @@
 size_t hils_ga_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S,
                                int q_block, int WH, float sm_n);
 int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const void* weights,
-                              const int32_t* indices, const float* slope, void* o, float* lse,
-                              void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ,
-                              int H, int D, int Dv, int K, int NW, int S, float sm_scale,
+                              const int32_t* indices, const float* slope, const void* swa_o, int merge_col,
+                              void* o, float* lse, void* workspace, int workspace_ready, int B, int L,
+                              int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int S, float sm_scale,
                               int mask_last, int q_block, int WH, float sm_n, void* stream,
                               int* handled);
 
@@ -94,7 +94,7 @@ sparse_attn_fwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
     const int c = indices[irow * dm.K + kk];
     __syncthreads();
     if (c < 0 || c >= nchunk) {
-      if (lse && c < 0)
+      if (lse)  // empty or out-of-range slot
         for (int g = tid; g < G; g += SA_THREADS) lse[(bt * dm.HQ + hk * G + g) * (long)dm.K + kk] = HILS_NEG_INF;
       continue;
     }
@@ -285,25 +285,66 @@ extern "C" size_t hils_sparse_attn_fwd_workspace(int B, int L, int Lkv, int HQ, 
   return hils_ga_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n);
 }
 
+// o += swa_o * weights[..., col] for the paths that do not merge in their own epilogue:
+// one thread per 8 output elements.
+__global__ void __launch_bounds__(256)
+merge_local_kernel(bf16_t* __restrict__ o, const bf16_t* __restrict__ swa_o, const bf16_t* __restrict__ weights,
+                   long n8, int L, int HQ, int G, int Dv, int NW, int WH, int q_block, int col) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n8) return;
+  const int c8n = Dv / 8;
+  const long row = i / c8n;          // (b*L + t)*HQ + hq
+  const int hq = (int)(row % HQ);
+  const long bt = row / HQ;
+  const int t = (int)(bt % L);
+  const long b = bt / L;
+  const long wrow = (b * (L / q_block) + t / q_block) * WH + (WH == HQ ? hq : hq / G);
+  const float wl = bf2f(weights[wrow * NW + col]);
+  float a[8], c[8];
+  unpack8(*(const uint4*)(o + i * 8), a);
+  unpack8(*(const uint4*)(swa_o + i * 8), c);
+  uint4 x;
+  x.x = pack_bf2(fmaf(c[0], wl, a[0]), fmaf(c[1], wl, a[1]));
+  x.y = pack_bf2(fmaf(c[2], wl, a[2]), fmaf(c[3], wl, a[3]));
+  x.z = pack_bf2(fmaf(c[4], wl, a[4]), fmaf(c[5], wl, a[5]));
+  x.w = pack_bf2(fmaf(c[6], wl, a[6]), fmaf(c[7], wl, a[7]));
+  *(uint4*)(o + i * 8) = x;
+}
+
+static int sa_merge_local(void* o, const void* swa_o, const void* weights, int B, int L, int HQ, int H,
+                          int Dv, int NW, int WH, int q_block, int col, void* stream) {
+  const long n8 = (long)B * L * HQ * (Dv / 8);
+  HILS_REQUIRE((n8 + 255) / 256 <= 2147483647L, "hils_sparse_attn_fwd: grid too large");
+  hipLaunchKernelGGL(merge_local_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (bf16_t*)o, (const bf16_t*)swa_o, (const bf16_t*)weights, n8, L, HQ, HQ / H, Dv, NW, WH,
+                     q_block, col);
+  return HILS_OK;
+}
+
 extern "C" int hils_sparse_attn_fwd(const void* q, const void* k, const void* v,
                                     const void* weights, const int32_t* indices,
-                                    const float* slope, void* o, float* lse, void* workspace,
-                                    int workspace_ready, int B, int L, int Lkv, int HQ, int H,
-                                    int D, int Dv, int K, int NW, int WH, int q_block, int S,
-                                    float sm_scale, int mask_last, float sm_n, void* stream) {
+                                    const float* slope, const void* swa_o, void* o, float* lse,
+                                    void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ,
+                                    int H, int D, int Dv, int K, int NW, int WH, int q_block, int S,
+                                    float sm_scale, int mask_last, float sm_n, int merge_col,
+                                    void* stream) {
   HILS_REQUIRE(q && k && v && weights && indices && o, "hils_sparse_attn_fwd: null pointer");
   if (int rc = sa_check("hils_sparse_attn_fwd", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
+  HILS_REQUIRE(!swa_o || (merge_col >= 0 && merge_col < NW),
+               "hils_sparse_attn_fwd: merge_col (%d) must be a weight column (0..%d)", merge_col, NW - 1);
   if (hils_decode_covers(L, HQ, H, D, Dv, S, q_block, WH, sm_n, slope, lse) && Lkv >= S) {
     if (int rc = hils_sparse_attn_decode(q, k, v, weights, indices, o, workspace, B, L, Lkv, HQ, H, D,
                                          Dv, K, NW, sm_scale, mask_last, stream))
       return rc;
+    if (swa_o)
+      if (int rc = sa_merge_local(o, swa_o, weights, B, L, HQ, H, Dv, NW, WH, q_block, merge_col, stream)) return rc;
     HILS_CHECK_LAUNCH("hils_sparse_attn_fwd");
     return HILS_OK;
   }
   if (workspace && hils_ga_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n) > 0) {
     int handled = 0;
-    if (int rc = hils_sparse_attn_fwd_mfma(q, k, v, weights, indices, slope, o, lse, workspace,
-                                           workspace_ready, B, L, Lkv, HQ, H, D, Dv, K, NW, S,
+    if (int rc = hils_sparse_attn_fwd_mfma(q, k, v, weights, indices, slope, swa_o, merge_col, o, lse,
+                                           workspace, workspace_ready, B, L, Lkv, HQ, H, D, Dv, K, NW, S,
                                            sm_scale, mask_last, q_block, WH, sm_n, stream, &handled))
       return rc;
     if (handled) {
@@ -317,6 +358,8 @@ extern "C" int hils_sparse_attn_fwd(const void* q, const void* k, const void* v,
   hipLaunchKernelGGL(sparse_attn_fwd_simple, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS),
                      smem, (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k,
                      (const bf16_t*)v, (const bf16_t*)weights, indices, slope, (bf16_t*)o, lse, dm);
+  if (swa_o)
+    if (int rc = sa_merge_local(o, swa_o, weights, B, L, HQ, H, Dv, NW, WH, q_block, merge_col, stream)) return rc;
   HILS_CHECK_LAUNCH("hils_sparse_attn_fwd");
   return HILS_OK;
 }
@@ -335,16 +378,56 @@ extern "C" size_t hils_sparse_attn_bwd_workspace(int B, int L, int Lkv, int HQ, 
   return hils_bw_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n);
 }
 
+// Backward of the merge o = o_remote + swa_o * w[col]: d_swa_o = d_o * w[col], dw[col] = <d_o, swa_o>.
+// Dv/8 neighbouring lanes own one (query, head) row.
+__global__ void __launch_bounds__(256)
+merge_local_bwd_kernel(const bf16_t* __restrict__ d_o, const bf16_t* __restrict__ swa_o,
+                       const bf16_t* __restrict__ weights, bf16_t* __restrict__ d_swa_o, float* __restrict__ dw,
+                       long n8, int lpr, int NW, int col) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  const bool ok = i < n8;
+  const long row = (ok ? i : n8 - 1) / lpr;
+  const float wl = bf2f(weights[row * NW + col]);
+  float g[8], c[8];
+  float dot = 0.f;
+  if (ok) {
+    unpack8(*(const uint4*)(d_o + i * 8), g);
+    unpack8(*(const uint4*)(swa_o + i * 8), c);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dot = fmaf(g[e], c[e], dot);
+    uint4 x;
+    x.x = pack_bf2(g[0] * wl, g[1] * wl);
+    x.y = pack_bf2(g[2] * wl, g[3] * wl);
+    x.z = pack_bf2(g[4] * wl, g[5] * wl);
+    x.w = pack_bf2(g[6] * wl, g[7] * wl);
+    *(uint4*)(d_swa_o + i * 8) = x;
+  }
+  for (int o2 = 1; o2 < lpr; o2 <<= 1) dot += __shfl_xor(dot, o2, 64);
+  if (ok && (i % lpr) == 0) dw[row * NW + col] = dot;
+}
+
 extern "C" int hils_sparse_attn_bwd(const void* q, const void* k, const void* v,
                                     const void* weights, const int32_t* indices,
                                     const float* slope, const float* lse, const void* d_o,
                                     void* dq, float* dk, float* dv, float* dw, void* workspace, int B,
                                     int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int WH,
                                     int q_block, int S, float sm_scale, int mask_last, float sm_n,
-                                    void* stream) {
+                                    const void* swa_o, void* d_swa_o, int merge_col, void* stream) {
   HILS_REQUIRE(q && k && v && weights && indices && lse && d_o && dq && dk && dv && dw,
                "hils_sparse_attn_bwd: null pointer");
   if (int rc = sa_check("hils_sparse_attn_bwd", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
+  if (swa_o) {  // the forward merged the local branch: its gradient and that of its weight column
+    const int lpr = Dv / 8;
+    HILS_REQUIRE(d_swa_o && merge_col >= K && merge_col < NW && q_block == 1 && WH == HQ && lpr <= 64 &&
+                     (lpr & (lpr - 1)) == 0,
+                 "hils_sparse_attn_bwd: the merged local branch needs d_swa_o, a weight column in K..NW-1, "
+                 "per-query-head weights and Dv/8 a power of two");
+    const long n8 = (long)B * L * HQ * lpr;
+    HILS_REQUIRE((n8 + 255) / 256 <= 2147483647L, "hils_sparse_attn_bwd: grid too large");
+    hipLaunchKernelGGL(merge_local_bwd_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, (const bf16_t*)d_o, (const bf16_t*)swa_o, (const bf16_t*)weights,
+                       (bf16_t*)d_swa_o, dw, n8, lpr, NW, merge_col);
+  }
   if (workspace && hils_bw_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n) > 0 &&
       hils_bw_covers(L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n, slope)) {
     const int rc = hils_bw_run(q, k, v, weights, indices, lse, d_o, dq, dk, dv, dw, workspace, B, L, Lkv, HQ,

@@ -705,14 +705,8 @@ static int bq_launch(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, co
                      const float* kmax, const bf16_t* w, const int32_t* idx, const float* lse, bf16_t* dq,
                      float* dw, const BqDims& dm) {
   auto kern = bw_dq_kernel<D, DV, G>;
-  static size_t reserved = 0;  // per instantiation
-  if (smem > reserved) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
-      hils_set_error("hils_sparse_attn_bwd: cannot reserve %zu bytes of LDS", smem);
-      return HILS_ERR_LAUNCH;
-    }
-    reserved = smem;
-  }
+  static HilsLdsReserve reserved;  // per instantiation
+  if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_sparse_attn_bwd")) return rc;
   hipLaunchKernelGGL(kern, grid, dim3(BQ_THREADS), smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
   return HILS_OK;
 }

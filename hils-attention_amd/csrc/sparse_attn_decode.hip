@@ -163,14 +163,7 @@ __global__ void decode_reduce_kernel(const float* __restrict__ partial, bf16_t* 
 }
 
 static int de_pick_nsplit(int B, int L, int H, int K) {
-  static int cus = 0;  // looked up once (not a stream operation, but keep it out of graph capture)
-  if (cus == 0) {
-    int dev = 0, v = 0;
-    cus = 256;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      cus = v;
-  }
+  const int cus = hils_device_cus();
   const long rows = (long)B * L * H;
   // whole waves of one 16-wavefront workgroup per compute unit: no split, no partial sums
   if (K >= 16 && rows >= cus && (rows % cus == 0 || rows >= 8L * cus)) return 1;

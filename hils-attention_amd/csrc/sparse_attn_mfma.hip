@@ -103,31 +103,82 @@ struct GaDims {
   // have WH = HQ or H heads; sm_n * exp(-max) joins every chunk's softmax denominator
   int q_block, WH;
   float sm_n;
+  int merge_col;  // with a local-branch output given: the weight column that scales it
+};
+
+// Power-of-two fixed-point scale for sums bounded by `bound`: bound * scale < 2^GA_FX_LOG2_MAX.
+__device__ __forceinline__ float ga_fx_scale(float bound) {
+  if (!(bound > 0.f && bound < 3.0e38f)) return 1.f;
+  int e2 = GA_FX_LOG2_MAX - 1 - ilogbf(bound);
+  e2 = e2 > 90 ? 90 : (e2 < -90 ? -90 : e2);
+  return ldexpf(1.f, e2);
+}
+
+// ---- explicit operand loads --------------------------------------------------------------
+// The tile stream below keeps several global loads in flight across loop iterations (the next
+// tile's query rows, the next visit's K and V).  Which of them are outstanding at a use depends on
+// wavefront-uniform branches (does the chunk change?), and the compiler's wait-count insertion
+// merges such paths to "wait for nearly everything", which exposed one full memory latency per
+// tile.  So the loads of the stream are issued by inline assembly, which that pass does not track,
+// and the kernel waits itself: vector-memory loads return in issue order, so
+// `s_waitcnt vmcnt(N)` with N = the loads issued after the wanted one (a lower bound is always
+// safe; stores are never counted) guarantees it has landed.  A register that a load is still
+// writing must not be read or copied before its wait: the waits are followed by empty asm
+// statements that "modify" the registers, which orders every use behind the wait.
+typedef unsigned ga_u32x4 __attribute__((ext_vector_type(4)));
+
+template <int OFF>
+__device__ __forceinline__ void ga_load128(ga_u32x4& dst, unsigned voff, const void* sbase) {
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "+v"(dst) : "v"(voff), "s"(sbase), "n"(OFF));
+}
+__device__ __forceinline__ void ga_load16(unsigned& dst, unsigned voff, const void* sbase) {
+  asm volatile("global_load_ushort %0, %1, %2" : "+v"(dst) : "v"(voff), "s"(sbase));
+}
+template <int N>
+__device__ __forceinline__ void ga_vmwait() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N));
+}
+__device__ __forceinline__ void ga_pin(ga_u32x4& a) { asm volatile("" : "+v"(a)); }
+__device__ __forceinline__ void ga_pin(unsigned& a) { asm volatile("" : "+v"(a)); }
+__device__ __forceinline__ bf16x8_t ga_bf(const ga_u32x4& x) { return __builtin_bit_cast(bf16x8_t, x); }
+
+// One tile of the stream a wavefront works through: up to 16/G (query, slot) pairs of a visit.
+template <int KS>
+struct GaTile {
+  ga_u32x4 bq[KS];  // gathered query rows (B operand of S^T = K Q^T), this lane's pieces
+  unsigned wbits;   // this lane's row: its weight (bf16 bits)
+  float rs;         // ... and the fixed-point scale of its output row
+  int pk;           // ... and its pair (query of the block << 8 | slot)
+  int n;            // real pairs in the tile
+  int orow[4];      // output-tile element offsets of this lane's four accumulator rows
 };
 
 // Output tiles are accumulated in LDS as 32-bit fixed point: integer LDS atomics run at
 // full rate on this hardware (float LDS atomics do not), and integer addition is
 // associative, so the result does not depend on the order in which wavefronts add.
-// The scale is chosen per workgroup from bound = max_row(sum_k |w|) * max_visited|V|, which
-// bounds every output element because each P row is a convex combination.
+// The scale is chosen per output row from bound = sum_k |w_row,k| * max_visited|V|, which
+// bounds every element of the row because each P row is a convex combination: a row keeps
+// 20 bits below its own bound however small its weights are beside its neighbours'.
 template <int D, int DV, int G, bool SLOPE>
 __global__ void __launch_bounds__(GA_THREADS)
 sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* __restrict__ kp,
                        const bf16_t* __restrict__ vp, const float* __restrict__ vmax,
                        const bf16_t* __restrict__ weights, const int32_t* __restrict__ indices,
-                       const float* __restrict__ slope, bf16_t* __restrict__ o,
-                       float* __restrict__ lse, GaDims dm) {
+                       const float* __restrict__ slope, const bf16_t* __restrict__ swa_o,
+                       bf16_t* __restrict__ o, float* __restrict__ lse, GaDims dm) {
   constexpr int KS = D / 32;    // k-steps of S^T = K Q^T
   constexpr int DT = DV / 16;   // 16-wide output column tiles
   constexpr int QT = 16 / G;    // queries per 16-row tile
   constexpr int NT = GA_THREADS;
   constexpr int MAXP = GA_MAXP;  // pairs per thread: T*K <= MAXP * GA_THREADS
+  typedef GaTile<KS> Tile;
   extern __shared__ __align__(16) int smem_i[];
   const int R = dm.T * G;
   int* o_acc = smem_i;                       // R x DV fixed point
   int* cur = o_acc + (size_t)R * DV;         // nchunk: histogram -> running ends
   int* pairs = cur + dm.nchunk;              // T*K pairs (query << 8 | slot) grouped by chunk
   int* nadd = pairs + dm.T * dm.K;           // R: tiles added to each output row
+  float* rscale = (float*)(nadd + R);        // R: sum_k |w| of the row, then its fixed-point scale
   __shared__ float red[32];
   __shared__ int scan_s[NT / 64];
   __shared__ int next_s;
@@ -153,10 +204,11 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
 
   // ---- prologue.  All global loads of the block set-up are issued before anything waits:
   // the query rows to repack, the selected chunk indices, and the weight rows.
-  // (1) Packed copy of this block's query rows: within the G heads of a (query, KV head) the
+  // (0) Packed copy of this block's query rows: within the G heads of a (query, KV head) the
   // 16-byte pieces are interleaved head-minor, [piece][head][8], so that the B-operand loads
-  // of the G lanes that hold the heads of one query are contiguous.  Only this workgroup
-  // reads what it writes here (made visible by the barriers below).
+  // of the G lanes that hold the heads of one query are contiguous (whole cache lines; read in
+  // place, a row's four lanes would touch half a line each).  Only this workgroup reads what it
+  // writes here (made visible by the barriers below).
   constexpr int PPR = D / 8;
   constexpr int QPK = 10;  // pieces per thread in flight (a 72-query block of 4 heads, D = 128, has 9)
   const int npiece = dm.T * G * PPR;
@@ -175,7 +227,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     const unsigned long long hi = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     qtmp[e] = make_uint4((unsigned)lo, (unsigned)(lo >> 32), (unsigned)hi, (unsigned)(hi >> 32));
   }
-  // (2) selected chunk of every (query, slot) pair of the block
+  // (1) selected chunk of every (query, slot) pair of the block
   int creg[MAXP], preg[MAXP];
 #pragma unroll
   for (int e = 0; e < MAXP; ++e) {
@@ -189,12 +241,12 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     }
     creg[e] = c;
   }
-  // (3) weight rows, for the bound of the fixed-point scale: rows' sum of |w| over the K slots.
+  // (2) weight rows, for the bound of the fixed-point scale: a row's sum of |w| over the K slots.
   // A row is read as aligned dwords (rows start on any bf16), all loads in flight together.
   constexpr int WDW = 17;  // dwords per round: 32 slots + alignment slack
-  float wsum = 0.f;
   for (int row = tid; row < R; row += NT) {
     const int ql = row / G, g = row - ql * G;
+    float a = 0.f;
     if (t0 + ql < dm.L) {
       const long e0 = ((b * LB + (t0 + ql) / dm.q_block) * (long)dm.WH + (w_per_q ? hk * G + g : hk)) *
                       dm.NW;  // first element
@@ -205,7 +257,6 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       // counts for nothing.  The tensor's last element, when its index is even, has no such dword
       // and is read on its own by the one thread whose row ends there.
       const long last_dw = (tot_e - 2) & ~1L;
-      float a = 0.f;
       if (tot_e < 2) {
         a = fabsf(bf2f(weights[e0]));
       } else {
@@ -226,13 +277,15 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
         }
         if ((tot_e & 1) && e_end == tot_e) a += fabsf(bf2f(weights[tot_e - 1]));
       }
-      wsum = fmaxf(wsum, a);
     }
+    rscale[row] = a;  // only this thread touches the entry until the barrier behind the scan
   }
   // The packed copy goes through LDS (the output tile is not in use yet): pieces arrive in the
   // order of the source rows and leave in packed order, so that loads and stores are both
-  // contiguous 1 KiB per wavefront instruction.
-  uint4* stage = (uint4*)o_acc;  // npiece * 16 bytes <= R * DV * 4
+  // contiguous 1 KiB per wavefront instruction.  The staged pieces fit the output tile: a row has
+  // D / 8 pieces of 16 bytes against DV * 4 bytes of accumulators (D <= 2 * DV).
+  static_assert(D <= 2 * DV, "the staged query pieces must fit inside the output tile");
+  uint4* stage = (uint4*)o_acc;
 #pragma unroll
   for (int e = 0; e < QPK; ++e) {
     const int i = tid + e * NT;
@@ -278,8 +331,8 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     creg[e] = c;
     if (c >= 0) atomicAdd(&cur[c], 1);
   }
-  wsum = block_max_lds(wsum, red);  // barrier: histogram complete
-  // ... times max |V| over the visited chunks; exclusive scan of the histogram on the way
+  lds_barrier();  // histogram complete
+  // max |V| over the visited chunks; exclusive scan of the histogram on the way
   float vm = 0.f;
   const int per_thr = (dm.nchunk + NT - 1) / NT;
   const int c_lo = tid * per_thr;
@@ -304,55 +357,87 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     cur[c] = base;
     base += h;
   }
+  for (int row = tid; row < R; row += NT) rscale[row] = ga_fx_scale(rscale[row] * vm);
   lds_barrier();
 #pragma unroll
   for (int e = 0; e < MAXP; ++e)
     if (creg[e] >= 0) pairs[atomicAdd(&cur[creg[e]], 1)] = preg[e];
   __syncthreads();  // now chunk c owns pairs[cur[c-1] .. cur[c])
 
-  const float bound = wsum * vm;
-  float fx_scale = 1.f;
-  if (bound > 0.f && bound < 3.0e38f) {
-    int e2 = GA_FX_LOG2_MAX - 1 - ilogbf(bound);  // bound * 2^e2 < 2^GA_FX_LOG2_MAX
-    e2 = e2 > 90 ? 90 : (e2 < -90 ? -90 : e2);
-    fx_scale = ldexpf(1.f, e2);
-  }
-  const float fx_inv = 1.f / fx_scale;
   const float c2 = dm.sm_scale * HILS_LOG2E;
   const int qs = r / G, g = r - qs * G;  // this lane's row of a tile: query slot, head
   const int hq = hk * G + g;
   const float sl = SLOPE ? slope[hq] : 0.f;
-  // rows of a tile are addressed from the block's first query with 32-bit element offsets
-  const bf16_t* qb = qp + ((b * dm.L + t0) * (long)dm.HQ + hk * G) * D;
+  // rows of a tile are addressed from the block's first query with 32-bit byte offsets into the
+  // packed copy, in which the G heads of a query are interleaved per 16-byte piece: the lanes of
+  // one query read contiguous bytes
+  const char* qb = (const char*)(qp + ((b * dm.L + t0) * (long)dm.HQ + hk * G) * D);
   const bf16_t* wb = weights + ((b * LB + t0 / dm.q_block) * (long)dm.WH + (w_per_q ? hk * G : hk)) * dm.NW;
   float* lse_blk = lse ? lse + (b * dm.L + t0) * (long)dm.HQ * K : nullptr;  // the block's first row
-  const int q_lane = (j * G + g) * 8, w_lane = w_per_q ? g * dm.NW : 0;
-  const int q_step = dm.HQ * D;          // per query of the block
-  const int w_step = dm.WH * dm.NW;      // per group of q_block queries
+  const unsigned q_lane = (unsigned)((j * G + g) * 8) * 2u, w_lane = w_per_q ? (unsigned)(g * dm.NW) : 0u;
+  const unsigned q_step = (unsigned)dm.HQ * D * 2u;  // bytes per query of the block
+  const int w_step = dm.WH * dm.NW;                  // elements per group of q_block queries
 
   // ---- visits: a wavefront takes chunks from a shared counter; a visit is all pairs of the
   // block on one chunk, processed as tiles of up to QT pairs.  The tile stream of a wavefront
   // is software-pipelined so that no operand load is waited for right after it is issued:
-  //   iteration i:  issue Q(i+1);  O += P(i-1) V  [then V(chunk i) replaces V in place];
-  //                 S(i) = K Q(i)^T  [then K(chunk i+1) replaces K in place];  softmax -> P(i).
-  // K and V of a chunk are reloaded only when the next tile belongs to another chunk.
-  bf16x8_t ka[4][KS], vb[DT][2];
-  // operand loads: a wavefront-uniform 64-bit base plus this lane's 32-bit byte offset
+  //   step i:  issue Q(i+1);  O += P(i-1) V  [then V(chunk i) replaces V in place];
+  //            S(i) = K Q(i)^T  [then K(chunk i+1) replaces K in place];  softmax -> P(i).
+  // K and V of a chunk are reloaded only when the next tile belongs to another chunk.  Two tile
+  // records alternate between "current" and "next / previous", so nothing is copied per step.
+  ga_u32x4 ka[4][KS], vb[DT][2];
+  constexpr int NK = 4 * KS;   // loads of a K reload
+  constexpr int NV = 2 * DT;   // loads of a V reload
+  constexpr int NA = KS + 1;   // loads of a tile issue (query pieces + weight)
+  // operand loads: a wavefront-uniform 64-bit base plus this lane's 32-bit byte offset; the
+  // instruction's immediate offset reaches 4 KiB, so a chunk is addressed from 4 KiB-spaced bases
   const unsigned lane_b = lane * 16;
-  auto load_k = [&](int c, int mt) {
-    const char* kbase = (const char*)(kp + ((b * dm.H + hk) * (long)dm.nchunk + c) * (long)GA_S * D);
+  const char* kp_unit = (const char*)(kp + (b * dm.H + hk) * (long)dm.nchunk * GA_S * D);
+  const char* vp_unit = (const char*)(vp + (b * dm.H + hk) * (long)dm.nchunk * GA_S * DV);
+  auto load_k_all = [&](int c) {
+    const char* kbase = kp_unit + (long)c * (GA_S * D * 2);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const uint4 x = *(const uint4*)(kbase + (mt * KS + ks) * 1024 + lane_b);
-      ka[mt][ks] = *(const bf16x8_t*)&x;
-    }
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        constexpr int dummy = 0; (void)dummy;
+        const int piece = mt * KS + ks;  // 1 KiB pieces
+        const char* sb = kbase + (piece / 4) * 4096;
+        switch (piece % 4) {
+          case 0: ga_load128<0>(ka[mt][ks], lane_b, sb); break;
+          case 1: ga_load128<1024>(ka[mt][ks], lane_b, sb); break;
+          case 2: ga_load128<2048>(ka[mt][ks], lane_b, sb); break;
+          default: ga_load128<3072>(ka[mt][ks], lane_b, sb); break;
+        }
+      }
   };
-  auto load_v = [&](int c, int dt) {
-    const char* vbase = (const char*)(vp + ((b * dm.H + hk) * (long)dm.nchunk + c) * (long)GA_S * DV);
+  auto load_v_half = [&](int c, int d0, int nd) {  // column tiles d0 .. d0+nd-1
+    const char* vbase = vp_unit + (long)c * (GA_S * DV * 2);
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const uint4 x = *(const uint4*)(vbase + (dt * 2 + s) * 1024 + lane_b);
-      vb[dt][s] = *(const bf16x8_t*)&x;
+    for (int u = 0; u < nd; ++u)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const int piece = (d0 + u) * 2 + s2;
+        const char* sb = vbase + (piece / 4) * 4096;
+        switch (piece % 4) {
+          case 0: ga_load128<0>(vb[d0 + u][s2], lane_b, sb); break;
+          case 1: ga_load128<1024>(vb[d0 + u][s2], lane_b, sb); break;
+          case 2: ga_load128<2048>(vb[d0 + u][s2], lane_b, sb); break;
+          default: ga_load128<3072>(vb[d0 + u][s2], lane_b, sb); break;
+        }
+      }
+  };
+  auto pin_k = [&]() {
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ga_pin(ka[mt][ks]);
+  };
+  auto pin_v = [&]() {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      ga_pin(vb[dt][0]);
+      ga_pin(vb[dt][1]);
     }
   };
   const int npair_valid = cur[dm.nchunk - 1];  // pairs with a valid chunk
@@ -377,21 +462,44 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     p = vs2;
     ve = ve2;
   };
-  // A tile's gathered query rows (B operands), weight and output rows.  Padding rows of a
+  // A tile's gathered query rows (B operands), weight, row scale: NA loads.  Padding rows of a
   // visit's last tile repeat the tile's last pair with weight 0: their P is exactly 0 and is
-  // added to that pair's output rows.  Query rows come from the packed copy, in which the G
-  // heads of a query are interleaved per 16-byte piece: the lanes of one query read contiguous
-  // bytes.
-  uint4 bq_n[KS];
-  int w_n, pk_n, orow_n[4];
+  // added to that pair's output rows.
+  const char* wb_c = (const char*)wb;
+  auto issue_tile = [&](Tile& t, int p, int ve) {
+    t.n = (ve - p < QT) ? ve - p : QT;
+    const int last = t.n - 1;
+    t.pk = pairs[p + (qs < last ? qs : last)];
+    const unsigned ql = (unsigned)t.pk >> 8;
+    const unsigned qoff = __umul24(ql, q_step) + q_lane;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      switch (ks) {
+        case 0: ga_load128<0>(t.bq[ks], qoff, qb); break;
+        case 1: ga_load128<4 * G * 16>(t.bq[ks], qoff, qb); break;
+        case 2: ga_load128<2 * 4 * G * 16>(t.bq[ks], qoff, qb); break;
+        default: ga_load128<3 * 4 * G * 16>(t.bq[ks], qoff, qb); break;
+      }
+    }
+    const unsigned woff =
+        (__umul24(dm.q_block == 1 ? ql : ql / (unsigned)dm.q_block, (unsigned)w_step) + w_lane + (t.pk & 255)) * 2u;
+    ga_load16(t.wbits, woff, wb_c);
+    t.rs = rscale[ql * G + g];
+  };
+  auto pin_tile = [&](Tile& t) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ga_pin(t.bq[ks]);
+    ga_pin(t.wbits);
+  };
   // output rows 4j .. 4j+3 of a tile starting at pair p (element offsets of this lane's column)
-  auto tile_rows = [&](int p, int last, int* orow) {
+  auto tile_rows = [&](Tile& t, int p) {
+    const int last = t.n - 1;
     if constexpr (G >= 4) {  // the four rows are consecutive heads of one query
       const int qsl = (4 * j) / G;
       const int pk = pairs[p + (qsl < last ? qsl : last)];
       const int base = ((pk >> 8) * G + (4 * j) % G) * DV + r;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) orow[i] = base + i * DV;
+      for (int i = 0; i < 4; ++i) t.orow[i] = base + i * DV;
     } else {
       int pk_o[4];
 #pragma unroll
@@ -402,28 +510,13 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int rr = 4 * j + i;
-        orow[i] = ((pk_o[i] >> 8) * G + rr % G) * DV + r;
+        t.orow[i] = ((pk_o[i] >> 8) * G + rr % G) * DV + r;
       }
     }
   };
-  auto load_tile = [&](int p, int ve) {
-    const int last = ((ve - p < QT) ? ve - p : QT) - 1;
-    pk_n = pairs[p + (qs < last ? qs : last)];
-    tile_rows(p, last, orow_n);
-    const bf16_t* qrow = qb + ((pk_n >> 8) * q_step + q_lane);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) bq_n[ks] = *(const uint4*)(qrow + ks * (4 * G * 8));
-    w_n = 0;
-    if (j == 0 && qs <= last) {
-      const int ql = pk_n >> 8;
-      w_n = wb[(dm.q_block == 1 ? ql : ql / dm.q_block) * w_step + w_lane + (pk_n & 255)];
-    }
-  };
   bf16x8_t ap[2];   // P of the previous tile (A operand of O = P V)
-  int orow_p[4];    // its output rows
-  // S = K Q^T of the tile in (bq_c, w_c, pk_c), softmax, P -> ap; K(c_next) replaces K when asked
-  auto score_stage = [&](const uint4* bq_c, int w_c, int pk_c, int n, bool reload, int c_next) {
-    const float w_row = bf2f((bf16_t)rows_bcast0((unsigned)w_c));
+  // S = K Q^T of tile t (its operands have landed), softmax, P -> ap; K(c_next) replaces K when asked
+  auto score_stage = [&](Tile& t, bool reload, int c_next) {
     // four independent accumulation chains (token tiles), interleaved so that a chain's next
     // MFMA is issued only after three others
     f32x4_t st[4];
@@ -433,11 +526,8 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt)
-        st[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[mt][ks], *(const bf16x8_t*)&bq_c[ks], st[mt], 0, 0, 0);
-    if (reload) {
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt) load_k(c_next, mt);
-    }
+        st[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga_bf(ka[mt][ks]), ga_bf(t.bq[ks]), st[mt], 0, 0, 0);
+    if (reload) load_k_all(c_next);
     if (SLOPE) {
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt)
@@ -469,12 +559,13 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       }
     sum = rows_sum(sum);
     if (dm.sm_n != 0.f) sum += dm.sm_n * __builtin_amdgcn_exp2f(-mc);
-    if (lse && qs < n && j == 0) {
-      const int ql = pk_c >> 8, slot = pk_c & 255;
+    if (lse && qs < t.n && j == 0) {
+      const int ql = t.pk >> 8, slot = t.pk & 255;
       lse_blk[(ql * dm.HQ + hq) * K + slot] = mc + __builtin_amdgcn_logf(sum);
     }
-    if (j == 0) atomicAdd(&nadd[(pk_c >> 8) * G + g], 1);  // padding rows count on the row they are added to
-    const float f = w_row * fx_scale * __builtin_amdgcn_rcpf(sum);  // fixed-point scale (a power of two) folded into P
+    if (j == 0) atomicAdd(&nadd[(t.pk >> 8) * G + g], 1);  // padding rows count on the row they are added to
+    const float w_row = qs < t.n ? __uint_as_float(t.wbits << 16) : 0.f;
+    const float f = w_row * t.rs * __builtin_amdgcn_rcpf(sum);  // fixed-point scale (a power of two) folded into P
     // P as the A operand of O = P V: k-step s takes tokens of accumulator tiles 2s, 2s+1
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
@@ -486,9 +577,9 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       ap[s] = *(bf16x8_t*)&x;
     }
   };
-  // O += P V for the tile in (ap, orow_p); V(c_next) replaces V when asked
+  // O += P V for the tile whose rows are `orow` (V has landed); V(c_next) replaces V when asked
   const f32x4_t fx_bias = {GA_FX_BIAS, GA_FX_BIAS, GA_FX_BIAS, GA_FX_BIAS};
-  auto output_stage = [&](bool reload, int c_next) {
+  auto output_stage = [&](const int* orow, bool reload, int c_next) {
     // four column tiles at a time: their eight MFMAs interleaved (two-deep chains), then the
     // operand reload, then the fixed-point adds
 #pragma unroll
@@ -500,64 +591,90 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
         for (int u = 0; u < 4; ++u)
-          acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s2], vb[d0 + u][s2], acc[u], 0, 0, 0);
-      if (reload) {
-#pragma unroll
-        for (int u = 0; u < 4; ++u) load_v(c_next, d0 + u);
-      }
+          acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s2], ga_bf(vb[d0 + u][s2]), acc[u], 0, 0, 0);
+      if (reload) load_v_half(c_next, d0, 4);
 #pragma unroll
       for (int u = 0; u < 4; ++u)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          atomicAdd(&o_acc[orow_p[i] + (d0 + u) * 16], __float_as_int(acc[u][i]));
+          atomicAdd(&o_acc[orow[i] + (d0 + u) * 16], __float_as_int(acc[u][i]));
     }
   };
 
+  // ---- the stream.  Issue order of a step i (x_i = "tile i is on another chunk than tile i-1"):
+  //   A_i: query rows + weight of tile i+1 (NA loads, when there is a tile i+1)
+  //   B_i: V of tile i's chunk (NV loads, when x_i), behind the MFMAs of O += P(i-1) V
+  //   C_i: K of tile i+1's chunk (NK loads, when x_{i+1}), behind the MFMAs of S(i)
+  // O += P(i-1) V needs B_{i-1}: the loads behind it are C_{i-1} (NK when x_i) and A_i;
+  // S(i) needs C_{i-1} and A_{i-1}: the loads behind C_{i-1} are A_i and B_i (NV when x_i).
+  // Without a tile i+1 there is no A_i and the step simply waits for everything.
   int c_cur, p_cur = 0, ve_cur = 0;
   c_cur = grab(p_cur, ve_cur);
   if (c_cur >= 0) {
+    Tile ta, tb;
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) load_k(c_cur, mt);
-    load_tile(p_cur, ve_cur);
+    for (int ks = 0; ks < KS; ++ks) { ta.bq[ks] = (ga_u32x4){0, 0, 0, 0}; tb.bq[ks] = (ga_u32x4){0, 0, 0, 0}; }
+    ta.wbits = tb.wbits = 0;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) load_v(c_cur, dt);
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ka[mt][ks] = (ga_u32x4){0, 0, 0, 0};
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) vb[dt][0] = vb[dt][1] = (ga_u32x4){0, 0, 0, 0};
+    // step 0 (no previous tile): A_{-1} = tile 0, C_{-1} = K(c_0), then A_0, B_0 = V(c_0)
+    issue_tile(ta, p_cur, ve_cur);
+    tile_rows(ta, p_cur);
+    load_k_all(c_cur);
     int c_nxt = c_cur, p_nxt = p_cur, ve_nxt = ve_cur;
     advance(c_nxt, p_nxt, ve_nxt);
-    // first tile: scores only
-    {
-      uint4 bq_c[KS];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) bq_c[ks] = bq_n[ks];
-      const int w_c = w_n, pk_c = pk_n;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) orow_p[i] = orow_n[i];
-      const int n = (ve_cur - p_cur < QT) ? ve_cur - p_cur : QT;
-      if (c_nxt >= 0) load_tile(p_nxt, ve_nxt);
-      score_stage(bq_c, w_c, pk_c, n, c_nxt >= 0 && c_nxt != c_cur, c_nxt);
+    if (c_nxt >= 0) {
+      issue_tile(tb, p_nxt, ve_nxt);
+      tile_rows(tb, p_nxt);
     }
+    load_v_half(c_cur, 0, DT);
+    if (c_nxt >= 0) ga_vmwait<NA + NV>(); else ga_vmwait<NV>();
+    pin_k();
+    pin_tile(ta);
+    score_stage(ta, c_nxt >= 0 && c_nxt != c_cur, c_nxt);
     int c_prev = c_cur;
-    while (c_nxt >= 0) {
+    // one step: `cu` is the tile whose scores are due (its loads were issued a step ago), `nx`
+    // holds the previous tile's output rows until the output stage is through, then the tile
+    // after `cu`.
+    auto step = [&](Tile& cu, Tile& nx) {
       c_cur = c_nxt; p_cur = p_nxt; ve_cur = ve_nxt;
       advance(c_nxt, p_nxt, ve_nxt);
-      uint4 bq_c[KS];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) bq_c[ks] = bq_n[ks];
-      const int w_c = w_n, pk_c = pk_n;
-      int orow_c[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) orow_c[i] = orow_n[i];
-      const int n = (ve_cur - p_cur < QT) ? ve_cur - p_cur : QT;
-      if (c_nxt >= 0) load_tile(p_nxt, ve_nxt);
-      output_stage(c_cur != c_prev, c_cur);
-      score_stage(bq_c, w_c, pk_c, n, c_nxt >= 0 && c_nxt != c_cur, c_nxt);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) orow_p[i] = orow_c[i];
+      const bool more = c_nxt >= 0;
+      const bool x = c_cur != c_prev;
+      if (more) issue_tile(nx, p_nxt, ve_nxt);  // A_i; leaves nx.orow alone
+      if (!more) ga_vmwait<0>(); else if (x) ga_vmwait<NA + NK>(); else ga_vmwait<NA>();
+      pin_v();
+      output_stage(nx.orow, x, c_cur);          // B_i
+      if (more) tile_rows(nx, p_nxt);
+      if (!more) ga_vmwait<0>(); else if (x) ga_vmwait<NA + NV>(); else ga_vmwait<NA>();
+      pin_k();
+      pin_tile(cu);
+      score_stage(cu, more && c_nxt != c_cur, c_nxt);  // C_i
       c_prev = c_cur;
+    };
+    // the stream: tile 0 = ta (scored above), tile 1 = tb, tile 2 -> ta, ...
+    bool last_is_a = true;
+    while (c_nxt >= 0) {
+      step(tb, ta);
+      last_is_a = false;
+      if (c_nxt < 0) break;
+      step(ta, tb);
+      last_is_a = true;
     }
-    output_stage(false, 0);
+    int orow_last[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) orow_last[i] = last_is_a ? ta.orow[i] : tb.orow[i];
+    ga_vmwait<0>();
+    pin_v();
+    output_stage(orow_last, false, 0);
   }
   __syncthreads();
   constexpr int C8 = DV / 8;
+  const int wcol = dm.merge_col;
   for (int i = tid; i < R * C8; i += NT) {
     const int row = i / C8, c8 = i - row * C8;
     const int ql = row / G, g2 = row - ql * G;
@@ -565,15 +682,25 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     if (t < dm.L) {
       const int* src = o_acc + (size_t)row * DV + c8 * 8;
       const unsigned bias = (unsigned)nadd[row] * (unsigned)GA_FX_BIAS_BITS;  // wraps like the sums did
+      const float fx_inv = 1.f / rscale[row];  // a power of two: exact
       float f[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) f[e] = (float)(int)((unsigned)src[e] - bias) * fx_inv;
+      const long orow_g = ((b * dm.L + t) * (long)dm.HQ + hk * G + g2) * DV + c8 * 8;
+      if (swa_o) {  // o = remote branch + local branch * its inter-chunk weight, rounded once
+        const float wl = bf2f(weights[((b * LB + t / dm.q_block) * (long)dm.WH + (w_per_q ? hk * G + g2 : hk)) *
+                                          dm.NW + wcol]);
+        float sv[8];
+        unpack8(*(const uint4*)(swa_o + orow_g), sv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = fmaf(sv[e], wl, f[e]);
+      }
       uint4 x;
       x.x = pack_bf2(f[0], f[1]);
       x.y = pack_bf2(f[2], f[3]);
       x.z = pack_bf2(f[4], f[5]);
       x.w = pack_bf2(f[6], f[7]);
-      *(uint4*)(o + ((b * dm.L + t) * (long)dm.HQ + hk * G + g2) * DV + c8 * 8) = x;
+      *(uint4*)(o + orow_g) = x;
     }
   }
 }
@@ -581,40 +708,34 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
 template <int D, int DV, int G, bool SLOPE>
 static int ga_launch_s(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, bf16_t* qp, const bf16_t* k,
                        const bf16_t* vt, const float* vmax, const bf16_t* w, const int32_t* idx,
-                       const float* slope, bf16_t* o, float* lse, const GaDims& dm) {
+                       const float* slope, const bf16_t* swa_o, bf16_t* o, float* lse, const GaDims& dm) {
+  static_assert(D % 32 == 0 && DV % 16 == 0 && 16 % G == 0, "tile shapes of the MFMA forward");
   auto kern = sparse_attn_fwd_gather<D, DV, G, SLOPE>;
-  static size_t reserved = 0;  // per instantiation
-  if (smem > reserved) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)smem) != hipSuccess) {
-      hils_set_error("hils_sparse_attn_fwd: cannot reserve %zu bytes of LDS", smem);
-      return HILS_ERR_LAUNCH;
-    }
-    reserved = smem;
-  }
-  hipLaunchKernelGGL(kern, grid, dim3(GA_THREADS), smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
+  static HilsLdsReserve reserved;  // per instantiation
+  if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_sparse_attn_fwd")) return rc;
+  hipLaunchKernelGGL(kern, grid, dim3(GA_THREADS), smem, st, q, qp, k, vt, vmax, w, idx, slope, swa_o, o, lse, dm);
   return HILS_OK;
 }
 
 template <int D, int DV, int G>
 static int ga_launch(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, bf16_t* qp, const bf16_t* k,
                      const bf16_t* vt, const float* vmax, const bf16_t* w, const int32_t* idx,
-                     const float* slope, bf16_t* o, float* lse, const GaDims& dm) {
-  if (slope) return ga_launch_s<D, DV, G, true>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
-  return ga_launch_s<D, DV, G, false>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
+                     const float* slope, const bf16_t* swa_o, bf16_t* o, float* lse, const GaDims& dm) {
+  if (slope) return ga_launch_s<D, DV, G, true>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, swa_o, o, lse, dm);
+  return ga_launch_s<D, DV, G, false>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, swa_o, o, lse, dm);
 }
 
 template <int D, int DV>
 static int ga_dispatch_g(int G, dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, bf16_t* qp,
                          const bf16_t* k, const bf16_t* vt, const float* vmax, const bf16_t* w,
-                         const int32_t* idx, const float* slope, bf16_t* o, float* lse,
+                         const int32_t* idx, const float* slope, const bf16_t* swa_o, bf16_t* o, float* lse,
                          const GaDims& dm) {
   switch (G) {
-    case 1: return ga_launch<D, DV, 1>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
-    case 2: return ga_launch<D, DV, 2>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
-    case 4: return ga_launch<D, DV, 4>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
-    case 8: return ga_launch<D, DV, 8>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
-    case 16: return ga_launch<D, DV, 16>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, o, lse, dm);
+    case 1: return ga_launch<D, DV, 1>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, swa_o, o, lse, dm);
+    case 2: return ga_launch<D, DV, 2>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, swa_o, o, lse, dm);
+    case 4: return ga_launch<D, DV, 4>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, swa_o, o, lse, dm);
+    case 8: return ga_launch<D, DV, 8>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, swa_o, o, lse, dm);
+    case 16: return ga_launch<D, DV, 16>(grid, smem, st, q, qp, k, vt, vmax, w, idx, slope, swa_o, o, lse, dm);
   }
   return -1;
 }
@@ -634,7 +755,8 @@ static size_t ga_vmax_bytes(int B, int H, int nchunk) {
 // visit, the fewer bytes of K and V the block pulls per row.  Returns 0 when nothing fits.
 #define GA_SMEM_MAX (160 * 1024 - 512)  // dynamic LDS beside the kernel's static arrays
 static int ga_pick_T(int L, int G, int Dv, int K, int nchunk, int q_block, size_t* smem_out) {
-  const size_t per_q = (size_t)G * Dv * 4 + (size_t)K * 4 + (size_t)G * 4;
+  // per query: G output rows, K pairs, G add counts, G row scales
+  const size_t per_q = (size_t)G * Dv * 4 + (size_t)K * 4 + (size_t)G * 4 + (size_t)G * 4;
   const size_t fixed = (size_t)nchunk * 4;
   if (fixed + per_q > GA_SMEM_MAX) return 0;
   long T = (long)((GA_SMEM_MAX - fixed) / per_q);
@@ -663,14 +785,14 @@ size_t hils_ga_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int 
   if (T == 0 || T % q_block != 0) return 0;  // a query block holds whole index-sharing groups
   const int nchunk = Lkv / S;
   return ga_vt_bytes(B, H, nchunk, Dv) + ga_vt_bytes(B, H, nchunk, D) + ga_vmax_bytes(B, H, nchunk) +
-         (size_t)B * L * HQ * D * sizeof(bf16_t);  // packed K, packed V, per-chunk max|V|, packed Q
+         (size_t)B * L * HQ * D * sizeof(bf16_t);  // packed V, packed K, per-chunk max|V|, packed Q
 }
 
 // Returns HILS_OK and sets *handled = 1 when the MFMA path ran.
 int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const void* weights,
-                              const int32_t* indices, const float* slope, void* o, float* lse,
-                              void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ,
-                              int H, int D, int Dv, int K, int NW, int S, float sm_scale,
+                              const int32_t* indices, const float* slope, const void* swa_o, int merge_col,
+                              void* o, float* lse, void* workspace, int workspace_ready, int B, int L,
+                              int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int S, float sm_scale,
                               int mask_last, int q_block, int WH, float sm_n, void* stream,
                               int* handled) {
   *handled = 0;
@@ -693,13 +815,13 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
                        (size_t)GA_S * (dmax + 2) * sizeof(bf16_t), st, (const bf16_t*)k,
                        (const bf16_t*)v, kpk, vpk, vmax, Lkv, H, D, Dv, nchunk);
   }
-  GaDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale, q_block, WH, sm_n};
+  GaDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale, q_block, WH, sm_n, merge_col};
   const long per_xcd = (total + 7) / 8;
   dim3 grid((unsigned)(per_xcd * 8));
   int rc = -1;
 #define GA_CALL(D_, DV_)                                                                       \
   rc = ga_dispatch_g<D_, DV_>(G, grid, smem, st, (const bf16_t*)q, qpk, kpk, vpk, vmax,        \
-                              (const bf16_t*)weights, indices, slope, (bf16_t*)o, lse, dm)
+                              (const bf16_t*)weights, indices, slope, (const bf16_t*)swa_o, (bf16_t*)o, lse, dm)
   if (D == 64 && Dv == 64) GA_CALL(64, 64);
   else if (D == 128 && Dv == 128) GA_CALL(128, 128);
   else if (D == 64 && Dv == 128) GA_CALL(64, 128);

@@ -683,15 +683,8 @@ static int swa_bwd_launch(const bf16_t* q, const bf16_t* k, const bf16_t* v, con
   const size_t smem = (size_t)64 * (D * 2 + 16) + (size_t)D * LZM_PT + (size_t)64 * (DV * 2 + 16) +
                       (size_t)DV * LZM_PT + 3 * 64 * sizeof(float);
   auto kern = swa_bwd_dkdv_mfma<D, DV, G>;
-  static size_t reserved = 48 * 1024;  // per instantiation
-  if (smem > reserved) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) !=
-        hipSuccess) {
-      hils_set_error("hils_swa_bwd: cannot reserve %zu bytes of LDS", smem);
-      return HILS_ERR_LAUNCH;
-    }
-    reserved = smem;
-  }
+  static HilsLdsReserve reserved;  // per instantiation
+  if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_swa_bwd")) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)((dm.Lq + 127) / 128), (unsigned)dm.H, (unsigned)B), dim3(256),
                      smem, st, q, k, v, lse, d_o, delta, dk, dv, dm);
   return HILS_OK;

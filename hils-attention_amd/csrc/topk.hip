@@ -714,7 +714,9 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float yy = PLAIN ? acc[nt][i] * c2 : logit(acc[nt][i], c, i) * HILS_LOG2E;
+        // one rounding (acc * c2) whenever nothing is added to the logit, in both variants, so that
+        // the export variant and the plain one select from bit-identical lse_total
+        float yy = (PLAIN || (!bias && !gumbel)) ? acc[nt][i] * c2 : logit(acc[nt][i], c, i) * HILS_LOG2E;
         if (MASKED && !(c < lim[nt][i])) yy = HILS_NEG_INF;
         y[nt][i] = yy;
         d[nt][i] = yy - ref[nt][i];
@@ -1480,18 +1482,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   }
 }
 
-// compute units of the current device, looked up once (keeps the query out of HIP graph capture)
-static int topk_cus() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, v = 0;
-    cus = 256;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      cus = v;
-  }
-  return cus;
-}
+static int topk_cus() { return hils_device_cus(); }
 
 // rows = (query, KV head) pairs; the row kernel wants about one row per compute unit
 static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool plain) {
@@ -1513,15 +1504,8 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, i
 #define TOPK_ROW_CALL_W(D_, W_)                                                                   \
   do {                                                                                           \
     auto kern = topk_row_kernel<D_, 4, W_>;                                                      \
-    static size_t reserved = 48 * 1024;                                                          \
-    if (smem > reserved) {                                                                       \
-      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,     \
-                              (int)smem) != hipSuccess) {                                        \
-        hils_set_error("hils_topk_fwd: cannot reserve %zu bytes of LDS", smem);                  \
-        return HILS_ERR_LAUNCH;                                                                  \
-      }                                                                                          \
-      reserved = smem;                                                                           \
-    }                                                                                            \
+    static HilsLdsReserve reserved;                                                              \
+    if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_topk_fwd")) return rc; \
     hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(W_ * 64), smem, st,                      \
                        (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, indices, (bf16_t*)scores, \
                        lse_total, sel_logits, (bf16_t*)weights, L, N, NP, h_kv, G, topk,         \
@@ -1576,14 +1560,8 @@ static int topk_fwd_split(const void* q, const void* lmks, const float* lse_swa,
   } else if (N <= 256 * 16 && G <= 4) {
     TOPK_B_REG(4, 16);
   } else {
-    if (smem > 64 * 1024) {
-      static bool reserved = false;
-      if (!reserved) {
-        (void)hipFuncSetAttribute((const void*)topk_select_kernel,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024 + 4096);
-        reserved = true;
-      }
-    }
+    static HilsLdsReserve reserved;
+    if (int rc = hils_reserve_lds(&reserved, (const void*)topk_select_kernel, smem, "hils_topk_fwd")) return rc;
     hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)rows), dim3(TOPK_B_THREADS), smem, st, raw,
                        lse_swa, bias, gumbel, drop_mask, indices, (bf16_t*)scores, lse_total,
                        sel_logits, L, N, h_kv, G, topk, block_size, window_size, causal, q_offset);
@@ -1714,6 +1692,63 @@ extern "C" int hils_topk_fwd_weights(const void* q, const void* lmks, const floa
   if (fused) return HILS_OK;
   return hils_chunk_weights(scores, lse_swa, 0, nullptr, nullptr, weights, B, L, h_kv * G, h_kv, N, topk, 0,
                             stream);
+}
+
+// ---------------------------------------------------------------------------
+// hils_topk_fwd for callers that cannot allocate: the workspace is a file-scope device array.
+// Every GPU the library runs on holds its own copy of the array until the process ends; in host
+// code the array's name is only a stand-in, so its device address is looked up once per device
+// (with that device current) and that pointer is what the kernels get.
+// ---------------------------------------------------------------------------
+#define HILS_TOPK_SCRATCH_BYTES ((size_t)8 << 20)
+static __device__ __align__(256) unsigned char scratch[HILS_TOPK_SCRATCH_BYTES];
+static std::atomic<void*> g_scratch_ptr[HILS_LDS_RESERVE_DEVICES];
+
+static int topk_scratch_address(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= HILS_LDS_RESERVE_DEVICES) {
+    (void)hipGetLastError();
+    hils_set_error("hils_topk_fwd_noalloc: no current GPU (device ordinal %d)", dev);
+    return HILS_ERR_LAUNCH;
+  }
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      (void)hipGetLastError();
+      hils_set_error("hils_topk_fwd_noalloc: hipGetSymbolAddress failed on device %d: %s", dev,
+                     hipGetErrorString(e));
+      return HILS_ERR_LAUNCH;
+    }
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // the same address from whichever thread asks
+  }
+  *out = p;
+  return HILS_OK;
+}
+
+extern "C" size_t hils_topk_fwd_noalloc_max_workspace(void) { return HILS_TOPK_SCRATCH_BYTES; }
+
+extern "C" int hils_topk_fwd_noalloc(const void* q, const void* lmks, const float* lse_swa,
+                                     const float* bias, const float* gumbel, const int32_t* drop_mask,
+                                     int32_t* indices, void* scores, float* lse_total, float* sel_logits,
+                                     int B, int L, int N, int h_kv, int G, int D, int topk,
+                                     int block_size, int window_size, int causal, int q_offset,
+                                     int per_qhead, float sm_scale, void* stream) {
+  HILS_REQUIRE(B > 0 && L > 0 && N > 0 && h_kv > 0 && G > 0, "hils_topk_fwd_noalloc: sizes must be positive");
+  const size_t need = hils_topk_fwd_workspace(B, L, N, h_kv, G);
+  HILS_REQUIRE(need <= HILS_TOPK_SCRATCH_BYTES,
+               "hils_topk_fwd_noalloc: this shape needs %zu bytes of scratch, the built-in buffer holds %zu; "
+               "use hils_topk_fwd with a caller-allocated workspace",
+               need, (size_t)HILS_TOPK_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (need > 0)
+    if (int rc = topk_scratch_address(&ws)) return rc;
+  // every byte a kernel of this call reads from the buffer is written earlier in the same call
+  // (repacked chunk keys, or the logits parked between the two decode kernels): nothing to clear
+  int fused = 0;
+  return topk_fwd_impl(q, lmks, lse_swa, bias, gumbel, drop_mask, indices, scores, lse_total, sel_logits,
+                       ws, nullptr, &fused, B, L, N, h_kv, G, D, topk, block_size, window_size, causal,
+                       q_offset, per_qhead, sm_scale, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -23,12 +23,14 @@ SIGNATURES = {
     "hils_attn_pool_fwd": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
     "hils_attn_pool_bwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
     "hils_topk_fwd": [_P] * 11 + [_I] * 12 + [_F, _P],
+    "hils_topk_fwd_noalloc": [_P] * 10 + [_I] * 12 + [_F, _P],
     "hils_topk_fwd_weights": [_P] * 10 + [_I] * 12 + [_F, _P],
     "hils_topk_bwd": [_P] * 7 + [_I] * 8 + [_F, _P],
-    "hils_sparse_attn_fwd": [_P] * 9 + [_I] * 13 + [_F, _I, _F, _P],
+    "hils_sparse_attn_fwd": [_P] * 10 + [_I] * 13 + [_F, _I, _F, _I, _P],
     "hils_pack_kv_chunks": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
-    "hils_sparse_attn_bwd": [_P] * 13 + [_I] * 12 + [_F, _I, _F, _P],
+    "hils_sparse_attn_bwd": [_P] * 13 + [_I] * 12 + [_F, _I, _F, _P, _P, _I, _P],
     "hils_chunk_weights": [_P, _P, _I, _P, _P, _P] + [_I] * 7 + [_P],
+    "hils_chunk_weights_bwd": [_P, _P, _I] + [_P] * 6 + [_I] * 7 + [_P],
     "hils_chunk_logz_fwd": [_P, _P, _P] + [_I] * 7 + [_F, _I, _P],
     "hils_chunk_logz_bwd_dq": [_P] * 5 + [_I] * 7 + [_F, _P],
     "hils_chunk_logz_bwd_dk": [_P] * 5 + [_I] * 7 + [_F, _P],
@@ -56,6 +58,8 @@ def load():
     lib.hils_version.argtypes = []
     lib.hils_topk_fwd_workspace.restype = ctypes.c_size_t
     lib.hils_topk_fwd_workspace.argtypes = [_I] * 5
+    lib.hils_topk_fwd_noalloc_max_workspace.restype = ctypes.c_size_t
+    lib.hils_topk_fwd_noalloc_max_workspace.argtypes = []
     lib.hils_sparse_attn_fwd_workspace.restype = ctypes.c_size_t
     lib.hils_sparse_attn_fwd_workspace.argtypes = [_I] * 11 + [_F]
     lib.hils_topk_bwd_workspace.restype = ctypes.c_size_t

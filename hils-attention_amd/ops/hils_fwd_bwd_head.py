@@ -22,7 +22,7 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, weights, indices, block_size, sm_scale, mask_last_token,
-                is_training, slope=None, kv_workspace=None):
+                is_training, slope=None, kv_workspace=None, swa_o=None, swa_weight_index=None):
         assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
         assert weights.is_contiguous() and indices.is_contiguous()
         _cabi.require_gpu_bf16("HiLS_block_M_head", q, k, v)
@@ -44,6 +44,13 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
             slope_dev = slope.to(dtype=torch.float32, device=q.device).contiguous()
         w_in = weights.to(q.dtype).contiguous()
         idx_in = indices.to(torch.int32).contiguous()
+        swa_in, merge_col = None, 0
+        if swa_o is not None:
+            assert swa_o.shape == (B, L, HQ, Dv), f"swa_o shape {tuple(swa_o.shape)} != {(B, L, HQ, Dv)}"
+            merge_col = int(K if swa_weight_index is None else swa_weight_index) % num_weights
+            assert merge_col >= K, f"the local branch's weight column ({merge_col}) lies among the {K} chunk slots"
+            _cabi.require_gpu_bf16("HiLS_block_M_head", swa_o)
+            swa_in = swa_o.contiguous()
         o = torch.empty((B, L, HQ, Dv), dtype=q.dtype, device=q.device)
         lse = None
         if is_training:
@@ -59,14 +66,14 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
             ws = _cabi.sparse_attn_fwd_workspace(q.device, B, L, L_kv, HQ, H, D, Dv, K, HQ, 1,
                                                  int(block_size), 0.0)
         _cabi.call("hils_sparse_attn_fwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
-                   _cabi.ptr(idx_in), _cabi.ptr(slope_dev), _cabi.ptr(o), _cabi.ptr(lse),
+                   _cabi.ptr(idx_in), _cabi.ptr(slope_dev), _cabi.ptr(swa_in), _cabi.ptr(o), _cabi.ptr(lse),
                    _cabi.ptr(ws), ws_ready, B, L, L_kv, HQ, H, D, Dv, K, num_weights, HQ, 1, int(block_size),
-                   float(sm_scale), int(bool(mask_last_token)), 0.0)
+                   float(sm_scale), int(bool(mask_last_token)), 0.0, merge_col)
         ctx.is_training = bool(is_training)
         if is_training:
-            ctx.save_for_backward(q, k, v, w_in, idx_in, lse, slope_dev)
+            ctx.save_for_backward(q, k, v, w_in, idx_in, lse, slope_dev, swa_in)
             ctx.cfg = (B, L, L_kv, HQ, H, D, Dv, K, num_weights, int(block_size), float(sm_scale),
-                       int(bool(mask_last_token)))
+                       int(bool(mask_last_token)), merge_col)
             ctx.w_dtype = weights.dtype
         return o
 
@@ -76,8 +83,9 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
             raise RuntimeError(
                 "[_hils_block_M_attention_inverse] forward ran with is_training=False: the "
                 "per-chunk LSE needed by the backward was not saved.")
-        q, k, v, w_in, idx_in, lse, slope_dev = ctx.saved_tensors
-        B, L, L_kv, HQ, H, D, Dv, K, NW, S, sm_scale, mask_last = ctx.cfg
+        q, k, v, w_in, idx_in, lse, slope_dev, swa_in = ctx.saved_tensors
+        B, L, L_kv, HQ, H, D, Dv, K, NW, S, sm_scale, mask_last, merge_col = ctx.cfg
+        d_swa = torch.empty_like(swa_in) if swa_in is not None else None
         do = do.to(q.dtype).contiguous()
         dq = torch.empty_like(q)
         dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
@@ -89,15 +97,16 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
         _cabi.call("hils_sparse_attn_bwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
                    _cabi.ptr(idx_in), _cabi.ptr(slope_dev), _cabi.ptr(lse), _cabi.ptr(do),
                    _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), _cabi.ptr(ws),
-                   B, L, L_kv, HQ, H, D, Dv, K, NW, HQ, 1, S, sm_scale, mask_last, 0.0)
+                   B, L, L_kv, HQ, H, D, Dv, K, NW, HQ, 1, S, sm_scale, mask_last, 0.0,
+                   _cabi.ptr(swa_in), _cabi.ptr(d_swa), merge_col)
         return (dq, dk.to(k.dtype), dv.to(v.dtype), dw.to(ctx.w_dtype), None,
-                None, None, None, None, None, None)
+                None, None, None, None, None, None, d_swa, None)
 
 
 def HiLS_block_M_head(q, k, v, weights, indices, block_size=64, sm_scale=None, block_M=None,
                       mask_last_token=True, dtype="bfloat16", accum_dtype="float",
                       num_threads=None, num_threads_fwd=None, num_threads_bwd=None,
-                      is_training=True, slope=None, kv_workspace=None):
+                      is_training=True, slope=None, kv_workspace=None, swa_o=None, swa_weight_index=None):
     """o[t,h] = sum_k weights[t,h,k] * softmax_{j in chunk indices[t,k]}(sm_scale*q.K_j) V_j.
 
     q (B,L,HQ,D), k (B,Lkv,H,D), v (B,Lkv,H,Dv) bf16 contiguous; weights (B,L,HQ,>=K) (the
@@ -107,6 +116,11 @@ def HiLS_block_M_head(q, k, v, weights, indices, block_size=64, sm_scale=None, b
     ``dtype`` must be "bfloat16" and ``accum_dtype`` "float".  ``kv_workspace`` (not in the
     reference) is an optional tensor from ``prepare_kv_workspace`` for the same ``v``: the
     MFMA-operand-ordered copies of K and V the prefill kernel reads, reusable across calls.
+    ``swa_o`` (B,L,HQ,Dv), not in the reference either: the local branch's output; with it the
+    call returns the layer's merged output ``hils_o + swa_o * weights[..., swa_weight_index]``
+    (``torch.addcmul`` at models/FlashHiLS/hils_attention.py:617-623; ``swa_weight_index``
+    defaults to K, pass -2 with the softmax-1 sink column), with gradients to ``swa_o`` and to
+    that weight column.
     """
     B, L, HQ, D = q.shape
     _, L_kv, H, Dk = k.shape
@@ -116,7 +130,7 @@ def HiLS_block_M_head(q, k, v, weights, indices, block_size=64, sm_scale=None, b
         raise ValueError("HiLS_block_M_head: only dtype='bfloat16' with accum_dtype='float' is built")
     return _hils_block_M_attention_inverse.apply(
         q, k, v, weights, indices, block_size, sm_scale, mask_last_token, is_training, slope,
-        kv_workspace)
+        kv_workspace, swa_o, swa_weight_index)
 
 
 def prepare_kv_workspace(q_len, k, v, num_q_heads, topk, block_size=64):

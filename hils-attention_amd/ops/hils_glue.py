@@ -1,4 +1,4 @@
-"""Fused inter-chunk softmax of the HiLS layer (forward / inference).
+"""Fused inter-chunk softmax of the HiLS layer (forward and backward).
 
 The reference computes it with torch ops inside the layer
 (models/FlashHiLS/hils_attention.py:585-610): gather the prior bias at the selected chunks,
@@ -11,33 +11,62 @@ import torch
 from . import _cabi
 
 
+class _ChunkWeightsFn(torch.autograd.Function):
+    """softmax([scores (+ prior_b at the indices), lse_swa (, 0)]) with its backward, one kernel each."""
+
+    @staticmethod
+    def forward(ctx, scores, lse_swa, prior_b, indices, softmax1):
+        B, L, HQ, K = scores.shape
+        sc = scores.contiguous()
+        lse = lse_swa.reshape(B, L, HQ).contiguous()
+        if lse.dtype not in (torch.bfloat16, torch.float32):
+            lse = lse.float()
+        H, N = HQ, 1
+        pb = idx = None
+        if prior_b is not None:
+            assert indices is not None, "prior_b needs the selected indices"
+            H = indices.shape[2]
+            N = prior_b.shape[1]
+            assert prior_b.shape == (B, N, HQ), f"prior_b shape {tuple(prior_b.shape)} != {(B, N, HQ)}"
+            assert indices.shape == (B, L, H, K)
+            pb = prior_b.float().contiguous()
+            idx = indices.to(torch.int32).contiguous()
+        out = torch.empty((B, L, HQ, K + 1 + int(softmax1)), dtype=scores.dtype, device=scores.device)
+        _cabi.call("hils_chunk_weights", _cabi.ptr(sc), _cabi.ptr(lse), int(lse.dtype == torch.bfloat16),
+                   _cabi.ptr(pb), _cabi.ptr(idx), _cabi.ptr(out), B, L, HQ, H, N, K, int(softmax1))
+        ctx.save_for_backward(sc, lse, pb, idx)
+        ctx.cfg = (B, L, HQ, H, N, K, int(softmax1))
+        ctx.lse_meta = (lse_swa.shape, lse_swa.dtype)
+        ctx.prior_dtype = None if prior_b is None else prior_b.dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, d_w):
+        sc, lse, pb, idx = ctx.saved_tensors
+        B, L, HQ, H, N, K, softmax1 = ctx.cfg
+        d_w = d_w.to(sc.dtype).contiguous()
+        d_sc = torch.empty_like(sc)
+        d_lse = torch.empty((B, L, HQ), dtype=torch.float32, device=sc.device) if ctx.needs_input_grad[1] else None
+        d_pb = None
+        if pb is not None and ctx.needs_input_grad[2]:
+            d_pb = torch.zeros_like(pb)
+        _cabi.call("hils_chunk_weights_bwd", _cabi.ptr(sc), _cabi.ptr(lse), int(lse.dtype == torch.bfloat16),
+                   _cabi.ptr(pb), _cabi.ptr(idx), _cabi.ptr(d_w), _cabi.ptr(d_sc), _cabi.ptr(d_lse),
+                   _cabi.ptr(d_pb), B, L, HQ, H, N, K, softmax1)
+        if d_lse is not None:
+            shape, dtype = ctx.lse_meta
+            d_lse = d_lse.reshape(shape).to(dtype)
+        if d_pb is not None:
+            d_pb = d_pb.to(ctx.prior_dtype)
+        return d_sc, d_lse, d_pb, None, None
+
+
 def chunk_weights(scores, lse_swa, prior_b=None, indices=None, enable_softmax1=False):
     """scores (B,L,HQ,K) bf16, lse_swa (B,L,HQ) -> weights (B,L,HQ,K+1(+1)) bf16.
     ``prior_b`` (B,N,HQ) with ``indices`` (B,L,H,K) adds the gathered prior bias first.
-    Forward only: inputs that require grad are rejected."""
+    Differentiable in scores, lse_swa and prior_b."""
     _cabi.require_gpu_bf16("chunk_weights", scores)
-    if torch.is_grad_enabled() and (scores.requires_grad or lse_swa.requires_grad):
-        raise RuntimeError("chunk_weights is forward-only; use the torch ops of the layer for training")
-    B, L, HQ, K = scores.shape
-    lse = lse_swa.reshape(B, L, HQ).contiguous()
-    if lse.dtype not in (torch.bfloat16, torch.float32):
-        lse = lse.float()
-    H, N = HQ, 1
-    pb = idx = None
-    if prior_b is not None:
-        assert indices is not None, "prior_b needs the selected indices"
-        H = indices.shape[2]
-        N = prior_b.shape[1]
-        assert prior_b.shape == (B, N, HQ), f"prior_b shape {tuple(prior_b.shape)} != {(B, N, HQ)}"
-        assert indices.shape == (B, L, H, K)
-        pb = prior_b.float().contiguous()
-        idx = indices.to(torch.int32).contiguous()
-    out = torch.empty((B, L, HQ, K + 1 + (1 if enable_softmax1 else 0)), dtype=scores.dtype,
-                      device=scores.device)
-    _cabi.call("hils_chunk_weights", _cabi.ptr(scores.contiguous()), _cabi.ptr(lse),
-               int(lse.dtype == torch.bfloat16), _cabi.ptr(pb),
-               _cabi.ptr(idx), _cabi.ptr(out), B, L, HQ, H, N, K, int(bool(enable_softmax1)))
-    return out
+    return _ChunkWeightsFn.apply(scores, lse_swa, prior_b, indices, bool(enable_softmax1))
 
 
 def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causal=True, q_offset=0,

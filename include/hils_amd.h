@@ -76,6 +76,22 @@ int hils_topk_fwd(const void* q, const void* lmks, const float* lse_swa, const f
                   int h_kv, int G, int D, int topk, int block_size, int window_size, int causal,
                   int q_offset, int per_qhead, float sm_scale, void* stream);
 
+/* hils_topk_fwd for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments and results as hils_topk_fwd without the workspace: the scratch (repacked chunk keys
+ * for prefill-sized calls, parked logits for the two-kernel decode path) lives in a device array
+ * of hils_topk_fwd_noalloc_max_workspace() bytes (8 MiB) inside the library, one copy per GPU,
+ * held until the process ends.  Shapes whose hils_topk_fwd_workspace(...) exceeds that are
+ * rejected (status 1).  Calls no allocating routine; the first call on a device looks the array's
+ * address up once (do that call outside a graph capture).  Every call on a GPU shares that GPU's
+ * array: calls that overlap on one GPU (two streams, two host threads) race. */
+size_t hils_topk_fwd_noalloc_max_workspace(void);
+int hils_topk_fwd_noalloc(const void* q, const void* lmks, const float* lse_swa, const float* bias,
+                          const float* gumbel, const int32_t* drop_mask, int32_t* indices,
+                          void* scores, float* lse_total, float* sel_logits, int B, int L, int N,
+                          int h_kv, int G, int D, int topk, int block_size, int window_size,
+                          int causal, int q_offset, int per_qhead, float sm_scale, void* stream);
+
 /* hils_topk_fwd plus the layer's inter-chunk softmax in the same call (inference): also writes
  * weights (B,L,h_kv*G,topk+1) bf16 = softmax over [scores (as bf16), lse_swa], the K+1-way
  * softmax of models/FlashHiLS/hils_attention.py:604-610 without prior bias (what
@@ -102,14 +118,24 @@ int hils_topk_bwd(const void* g_scores, const void* q, const void* lmks, const i
 /* ---- inter-chunk softmax (layer glue) ------------------------------------------ */
 
 /* chunk_weights = softmax([scores_1..K (+ prior_b gathered at the indices), lse_swa (, 0)]).
- * Replaces the gather / cat / F.softmax glue of models/FlashHiLS/hils_attention.py:585-610
- * (forward only).  scores (B,L,HQ,K) bf16; lse_swa (B,L,HQ) fp32, or bf16 when lse_bf16 != 0;
- * prior_b (B,N,HQ) fp32 or
- * NULL; indices (B,L,H,K) int32 (needed with prior_b) -> weights (B,L,HQ,K+1(+1)) bf16, the
+ * Replaces the gather / cat / F.softmax glue of models/FlashHiLS/hils_attention.py:585-610.
+ * scores (B,L,HQ,K) bf16; lse_swa (B,L,HQ) fp32, or bf16 when lse_bf16 != 0; prior_b (B,N,HQ)
+ * fp32 or NULL; indices (B,L,H,K) int32 (needed with prior_b) -> weights (B,L,HQ,K+1(+1)) bf16, the
  * local-branch weight in column K, the softmax-1 sink (softmax1 != 0) in column K+1. */
 int hils_chunk_weights(const void* scores, const void* lse_swa, int lse_bf16, const float* prior_b,
                        const int32_t* indices, void* weights, int B, int L, int HQ, int H, int N,
                        int K, int softmax1, void* stream);
+
+/* Backward of hils_chunk_weights: the autograd of the same glue (F.softmax over the
+ * concatenated columns, the gather of prior_b, models/FlashHiLS/hils_attention.py:585-610).
+ * The forward's inputs again, d_weights (B,L,HQ,K+1(+1)) bf16 -> d_scores (B,L,HQ,K) bf16
+ * (written), d_lse (B,L,HQ) fp32 (written) or NULL, d_prior_b (B,N,HQ) fp32 (ACCUMULATED with
+ * atomics at the selected chunks: caller zero-fills) or NULL.  The probabilities are rebuilt in
+ * fp32 from the inputs, not read back from the bf16 weights. */
+int hils_chunk_weights_bwd(const void* scores, const void* lse_swa, int lse_bf16, const float* prior_b,
+                           const int32_t* indices, const void* d_weights, void* d_scores, float* d_lse,
+                           float* d_prior_b, int B, int L, int HQ, int H, int N, int K, int softmax1,
+                           void* stream);
 
 /* ---- sparse attention over the selected chunks ------------------------------ */
 
@@ -121,6 +147,11 @@ int hils_chunk_weights(const void* scores, const void* lse_swa, int lse_bf16, co
  * < 0 = empty slot; slope (HQ) fp32 or NULL.
  * Outputs: o (B,L,HQ,Dv) bf16; lse (B,L,HQ,K) fp32 per-chunk log2-domain LSE or NULL
  * (-inf for empty slots).
+ * swa_o (B,L,HQ,Dv) bf16 or NULL: the local (sliding-window) branch's output; when given, the
+ * layer's merge `torch.addcmul(hils_o, swa_o, chunk_weights[..., merge_col].unsqueeze(-1))`
+ * (models/FlashHiLS/hils_attention.py:617-623) happens in the same call:
+ * o = remote branch + swa_o * weights[..., merge_col], rounded once (merge_col = K for the plain
+ * K+1-way softmax, NW-2 with the softmax-1 sink column).
  * workspace: device scratch of hils_sparse_attn_fwd_workspace(...) bytes; the MFMA path
  * keeps MFMA-operand-ordered copies of K and V there.  workspace_ready != 0 says the copies from
  * an earlier call (or from hils_pack_kv_chunks) on the same k and v are still valid and is not
@@ -129,10 +160,10 @@ int hils_chunk_weights(const void* scores, const void* lse_swa, int lse_bf16, co
 size_t hils_sparse_attn_fwd_workspace(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K,
                                       int WH, int q_block, int S, float sm_n);
 int hils_sparse_attn_fwd(const void* q, const void* k, const void* v, const void* weights,
-                         const int32_t* indices, const float* slope, void* o, float* lse,
-                         void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ, int H,
-                         int D, int Dv, int K, int NW, int WH, int q_block, int S, float sm_scale,
-                         int mask_last, float sm_n, void* stream);
+                         const int32_t* indices, const float* slope, const void* swa_o, void* o,
+                         float* lse, void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ,
+                         int H, int D, int Dv, int K, int NW, int WH, int q_block, int S, float sm_scale,
+                         int mask_last, float sm_n, int merge_col, void* stream);
 /* Fills a workspace of hils_sparse_attn_fwd_workspace(...) bytes on its own: per 64-token
  * chunk of a (batch, KV head), K and V rewritten in the register order of the MFMA operands
  * the prefill kernel loads (every operand load becomes one contiguous 1 KiB burst), followed
@@ -151,7 +182,10 @@ int hils_pack_kv_chunks(const void* k, const void* v, void* workspace, int B, in
  * workspace: device scratch of hils_sparse_attn_bwd_workspace(...) bytes (0 = shape not covered)
  * for the MFMA kernels: an inverse index (pairs of (query, slot) grouped by chunk) is built there
  * and dK, dV are then computed chunk-major without atomics.  NULL selects the shape-generic
- * kernel for everything. */
+ * kernel for everything.
+ * swa_o / d_swa_o / merge_col: when the forward merged the local branch (swa_o given there), pass
+ * the same swa_o and merge_col: d_swa_o (B,L,HQ,Dv) bf16 = d_o * weights[..., merge_col] is written
+ * and dw[..., merge_col] = <d_o, swa_o> (q_block = 1, WH = HQ only).  NULL otherwise. */
 size_t hils_sparse_attn_bwd_workspace(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K,
                                       int WH, int q_block, int S, float sm_n);
 int hils_sparse_attn_bwd(const void* q, const void* k, const void* v, const void* weights,
@@ -159,7 +193,7 @@ int hils_sparse_attn_bwd(const void* q, const void* k, const void* v, const void
                          const void* d_o, void* dq, float* dk, float* dv, float* dw, void* workspace,
                          int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
                          int WH, int q_block, int S, float sm_scale, int mask_last, float sm_n,
-                         void* stream);
+                         const void* swa_o, void* d_swa_o, int merge_col, void* stream);
 
 /* ---- exact per-chunk log Z ---------------------------------------------------- */
 

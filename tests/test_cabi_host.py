@@ -39,6 +39,7 @@ def test_binding_matches_header(pkg):
     fns.pop("hils_sparse_attn_bwd_workspace")
     fns.pop("hils_topk_bwd_workspace")
     fns.pop("hils_topk_fwd_workspace")
+    fns.pop("hils_topk_fwd_noalloc_max_workspace")
     assert set(_cabi.SIGNATURES) == set(fns)
     for name, params in fns.items():
         argtypes = _cabi.SIGNATURES[name]
@@ -63,8 +64,8 @@ def test_argument_errors_are_reported_without_a_gpu(pkg):
     assert lib.hils_topk_fwd(buf, buf, buf, None, None, None, buf, buf, None, None, None,
                              1, 16, 4, 1, 1, 64, 1000, 64, 1, 1, 0, 0, 0.125, None) == 1
     assert b"topk" in lib.hils_last_error()
-    assert lib.hils_sparse_attn_fwd(buf, buf, buf, buf, buf, None, buf, None, None, 0,
-                                    1, 16, 64, 3, 2, 64, 64, 4, 4, 3, 1, 64, 0.125, 1, 0.0, None) == 1
+    assert lib.hils_sparse_attn_fwd(buf, buf, buf, buf, buf, None, None, buf, None, None, 0,
+                                    1, 16, 64, 3, 2, 64, 64, 4, 4, 3, 1, 64, 0.125, 1, 0.0, 0, None) == 1
     assert b"multiple of H" in lib.hils_last_error()
 
 

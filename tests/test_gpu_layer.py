@@ -62,8 +62,25 @@ def _chunk_weights_case(pkg, orc, dev, K):
         assert_close_bf16(w, ref, f"chunk_weights prior={prior} softmax1={s1}", max_abs=8e-3)
     w32 = pkg.chunk_weights(scores.to(dev), lse.float().to(dev))
     assert torch.equal(w32, pkg.chunk_weights(scores.to(dev), lse.to(dev)))
-    with pytest.raises(RuntimeError):
-        pkg.chunk_weights(scores.to(dev).requires_grad_(), lse.to(dev))
+    # backward: gradients of scores, lse_swa and prior_b against the oracle's autograd
+    for prior, s1 in ((False, False), (True, True)):
+        sc_d = scores.to(dev).requires_grad_()
+        lse_d = lse.float().to(dev).requires_grad_()
+        pb_d = pb.to(dev).requires_grad_() if prior else None
+        w = pkg.chunk_weights(sc_d, lse_d, pb_d, idx.to(dev) if prior else None, enable_softmax1=s1)
+        g = torch.randn(w.shape).bfloat16()
+        w.backward(g.to(dev))
+        sc_c = scores.float().requires_grad_()
+        lse_c = lse.float().requires_grad_()
+        pb_c = pb.bfloat16().float().requires_grad_() if prior else None
+        ref = orc.inter_chunk_softmax(sc_c, lse_c, pb_c, idx if prior else None, softmax1=s1)
+        ref.backward(g.float())
+        assert sc_d.grad.dtype == torch.bfloat16 and lse_d.grad.dtype == torch.float32
+        assert_close_bf16(sc_d.grad, sc_c.grad, f"d_scores prior={prior} softmax1={s1}", max_abs=8e-3)
+        assert_close_bf16(lse_d.grad, lse_c.grad, "d_lse_swa", max_abs=8e-3)
+        if prior:
+            # empty slots gather (and scatter to) chunk 0 on both sides, as torch.gather on the clamped indices does
+            assert_close_bf16(pb_d.grad, pb_c.grad, "d_prior_b", max_abs=2e-2)
 
 
 @pytest.mark.parametrize("B,L,N,HQ,H,D,K,off", [(32, 1, 2048, 32, 8, 128, 32, 2048 * 64 - 1),

@@ -175,8 +175,8 @@ def test_sparse_attn_per_chunk_lse(pkg, orc, dev):
     o = torch.empty(B, L, HQ, 64, dtype=torch.bfloat16, device=dev)
     lse = torch.empty(B, L, HQ, 4, dtype=torch.float32, device=dev)
     t = [x.to(dev) for x in (q, k, v, w, idx)]
-    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(o), _cabi.ptr(lse), None, 0,
-               B, L, L, HQ, 2, D, 64, 4, w.shape[-1], HQ, 1, 64, 1 / math.sqrt(D), 1, 0.0)
+    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, None, _cabi.ptr(o), _cabi.ptr(lse), None, 0,
+               B, L, L, HQ, 2, D, 64, 4, w.shape[-1], HQ, 1, 64, 1 / math.sqrt(D), 1, 0.0, 0)
     _, lse_ref = orc.sparse_attn(q, k, v, w, idx, chunk_size=64, return_lse=True)
     assert_close_f32(lse.cpu() / 1.4426950408889634, lse_ref, LSE_TOL, "per-chunk LSE")
 
@@ -229,9 +229,9 @@ def test_sparse_attn_mfma_path_matches_generic_path(pkg, orc, dev, B, L, HQ, H, 
     for use_ws in (False, True):
         o = torch.empty(B, L, HQ, Dv, dtype=torch.bfloat16, device=dev)
         lse = torch.empty(B, L, HQ, K, dtype=torch.float32, device=dev)
-        _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(o), _cabi.ptr(lse),
+        _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, None, _cabi.ptr(o), _cabi.ptr(lse),
                    _cabi.ptr(ws) if use_ws else None, 0,
-                   B, L, L, HQ, H, D, Dv, K, w.shape[-1], HQ, 1, 64, 1 / math.sqrt(D), 1, 0.0)
+                   B, L, L, HQ, H, D, Dv, K, w.shape[-1], HQ, 1, 64, 1 / math.sqrt(D), 1, 0.0, 0)
         torch.cuda.synchronize()
         outs.append((o.cpu(), lse.cpu()))
     ref, lse_ref = orc.sparse_attn(q, k, v, w, idx, chunk_size=64, return_lse=True)
@@ -257,8 +257,8 @@ def test_sparse_attn_bwd_mfma_path_matches_generic_path(pkg, dev, B, L, HQ, H, D
     o = torch.empty(B, L, HQ, Dv, dtype=torch.bfloat16, device=dev)
     lse = torch.empty(B, L, HQ, K, dtype=torch.float32, device=dev)
     scale = 1 / math.sqrt(D)
-    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(o), _cabi.ptr(lse), None, 0,
-               B, L, L, HQ, H, D, Dv, K, NW, HQ, 1, 64, scale, mask_last, 0.0)
+    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, None, _cabi.ptr(o), _cabi.ptr(lse), None, 0,
+               B, L, L, HQ, H, D, Dv, K, NW, HQ, 1, 64, scale, mask_last, 0.0, 0)
     ws = _cabi.sparse_attn_bwd_workspace(dev, B, L, L, HQ, H, D, Dv, K, HQ, 1, 64, 0.0)
     assert ws is not None, "this shape must be covered by the MFMA backward"
     res = []
@@ -269,9 +269,46 @@ def test_sparse_attn_bwd_mfma_path_matches_generic_path(pkg, dev, B, L, HQ, H, D
         dw = torch.zeros(B, L, HQ, NW, dtype=torch.float32, device=dev)
         _cabi.call("hils_sparse_attn_bwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(lse), _cabi.ptr(do.to(dev)),
                    _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), _cabi.ptr(ws) if use_ws else None,
-                   B, L, L, HQ, H, D, Dv, K, NW, HQ, 1, 64, scale, mask_last, 0.0)
+                   B, L, L, HQ, H, D, Dv, K, NW, HQ, 1, 64, scale, mask_last, 0.0, None, None, 0)
         torch.cuda.synchronize()
         res.append([x.float().cpu() for x in (dq, dk, dv, dw)])
     for name, a, b in zip(("dq", "dk", "dv", "dw"), res[1], res[0]):
         assert_close_bf16(a, b, f"{name} mfma vs generic")
     assert torch.count_nonzero(res[1][3][..., K:]).item() == 0  # weight columns beyond K get no gradient
+
+
+@pytest.mark.parametrize("B,L,HQ,H,D,Dv,K,extra_w,col", [(1, 512, 8, 2, 128, 128, 8, 1, None),   # MFMA path, column K
+                                                         (2, 320, 4, 4, 64, 64, 4, 2, -2),        # softmax-1 sink column behind
+                                                         (1, 200, 4, 2, 32, 32, 4, 1, None),      # shape-generic path
+                                                         (8, 1, 8, 2, 128, 128, 8, 1, None)])     # decode path
+def test_sparse_attn_merges_local_branch(pkg, orc, dev, B, L, HQ, H, D, Dv, K, extra_w, col):
+    """HiLS_block_M_head(..., swa_o=...) returns hils_o + swa_o * weights[..., col] (the layer's
+    addcmul merge) with gradients to swa_o and to that weight column, against the oracle."""
+    note(f"sparse_attn + merge B{B} L{L} HQ{HQ} H{H} D{D} K{K} col{col}")
+    S = 64 if D >= 64 else 16
+    Lkv = L if L > 1 else 2048
+    q, k, v, w, idx = make_case(B, L, HQ, H, D, Dv, K, S, seed=51, extra_w=extra_w, Lkv=Lkv)
+    gen = torch.Generator().manual_seed(52)
+    swa = torch.randn(B, L, HQ, Dv, generator=gen).bfloat16()
+    do = torch.randn(B, L, HQ, Dv, generator=gen).bfloat16()
+    train = L > 1
+    qd, kd, vd, wd, sd = (t.to(dev).requires_grad_(train) for t in (q, k, v, w, swa))
+    o = pkg.HiLS_block_M_head(qd, kd, vd, wd, idx.to(dev), block_size=S, is_training=train, swa_o=sd,
+                              swa_weight_index=col)
+    wcol = K if col is None else w.shape[-1] + col
+    qf, kf, vf, wf, sf = (t.float().requires_grad_(train) for t in (q, k, v, w, swa))
+    ref = orc.sparse_attn(qf, kf, vf, wf, idx, chunk_size=S) + sf * wf[..., wcol].unsqueeze(-1)
+    assert_close_bf16(o, ref, "merged o")
+    if not train:
+        return
+    o.backward(do.to(dev))
+    ref.backward(do.float())
+    assert_close_bf16(sd.grad, sf.grad, "d_swa_o")
+    assert_close_bf16(qd.grad, qf.grad, "dq")
+    assert_close_bf16(kd.grad, kf.grad, "dk")
+    assert_close_bf16(vd.grad, vf.grad, "dv")
+    valid = (idx >= 0).repeat_interleave(HQ // H, dim=2)
+    dw_ref = torch.zeros_like(wf.grad)
+    dw_ref[..., :K] = torch.where(valid, wf.grad[..., :K], torch.zeros(()))
+    dw_ref[..., wcol] = wf.grad[..., wcol]
+    assert_close_bf16(wd.grad, dw_ref, "dw (slots and the local branch's column)")
