@@ -1484,6 +1484,13 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
 
 static int topk_cus() { return hils_device_cus(); }
 
+// the one-pass prefill kernel (topk_group.hip)
+bool hils_topk_group_covers(int N, int G, int D, int topk, int per_qhead, bool plain);
+int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* lse_swa, int32_t* indices,
+                           void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
+                           int G, int D, int topk, int block_size, int window_size, int causal, int q_offset,
+                           float sm_scale, void* stream);
+
 // rows = (query, KV head) pairs; the row kernel wants about one row per compute unit
 static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool plain) {
   return plain && !per_qhead && G <= 4 && (D == 64 || D == 128) && N >= 256 && N <= TOPK_R_MAXN &&
@@ -1621,6 +1628,15 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
       hipLaunchKernelGGL(topk_pack_lmk_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
                          (const bf16_t*)lmks, (uint4*)workspace, N, h_kv, D, nblk16, total);
       packed = (const uint4*)workspace;
+      // up to 512 chunks and 32 winners, nothing added to the logits: the one-pass kernel
+      if (hils_topk_group_covers(N, G, D, topk, per_qhead, !bias && !gumbel && !drop_mask)) {
+        if (int rc2 = hils_topk_group_launch(q, packed, lse_swa, indices, scores, lse_total, sel_logits, B, L, N,
+                                             h_kv, G, D, topk, block_size, window_size, causal, q_offset,
+                                             sm_scale, stream))
+          return rc2;
+        HILS_CHECK_LAUNCH("hils_topk_fwd");
+        return HILS_OK;
+      }
     }
 #define HILS_TOPK_ROWS_P(G_, KS_, PL_, PK_)                                                         \
   hipLaunchKernelGGL((topk_fwd_rows_kernel<G_, KS_, PL_, PK_>), grid_r, dim3(64), smem, st,         \

@@ -300,3 +300,38 @@ def test_topk_split_and_fused_paths_agree(pkg, dev):
         outs.append((idx.cpu(), sc.float().cpu()))
     assert torch.equal(outs[0][0], outs[1][0])
     assert (outs[0][1] - outs[1][1]).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("L,N,h_kv,G,D,topk,dup", [
+    (8192, 128, 2, 1, 64, 32, False),    # MHA, config-2-like rows (16 queries per wavefront)
+    (4100, 64, 2, 2, 128, 16, False),    # G = 2, ragged length
+    (8192, 128, 1, 4, 128, 32, True),    # pairs of identical chunk keys: ties at the threshold
+    (4096, 64, 1, 3, 64, 5, True),       # G = 3 (one padding head row), odd k, ties
+    (2048, 32, 2, 4, 64, 1, False),      # a single winner
+    (32768, 512, 1, 4, 128, 32, False),  # the full 512 chunks of the headline shape, one KV head
+    (16384, 256, 1, 1, 128, 31, True),   # k not a power of two, ties, G = 1
+])
+def test_topk_one_pass_prefill_kernel(pkg, orc, dev, L, N, h_kv, G, D, topk, dup):
+    """The one-pass prefill kernel (chunk keys repacked into the workspace, up to 512 chunks and 32
+    winners): logits, lse_total, bit-exact selection, order, scores, across its head groupings."""
+    run_case(pkg, orc, dev, B=1, L=L, N=N, h_kv=h_kv, G=G, D=D, topk=topk, S=64, W=1, seed=61,
+             dup_keys=dup, training=False)
+
+
+def test_topk_one_pass_kernel_all_scores_equal(pkg, orc, dev):
+    """Every chunk key identical: all visible chunks tie, far more keys reach the lane bound than the
+    compaction holds (the search over all keys runs) and the winners are the lowest indices."""
+    note("one-pass top-k: all chunk keys equal")
+    B, L, N, h_kv, G, D, topk, S = 1, 16384, 256, 1, 4, 128, 16, 64
+    gen = torch.Generator().manual_seed(62)
+    q = torch.randn(B, L, h_kv * G, D, generator=gen).bfloat16()
+    lmks = torch.randn(1, 1, h_kv, D, generator=gen).bfloat16().expand(B, N, h_kv, D).contiguous()
+    lse = torch.zeros(B, L, h_kv * G)
+    dbg = {}
+    idx, scores = pkg.online_softmax_topk_head(q.to(dev), lmks.to(dev), lse.to(dev), topk, S, 1,
+                                               is_training=False, _debug=dbg)
+    lim = orc.causal_chunk_limit(L, 0, 1, S)
+    want = torch.arange(topk).view(1, 1, 1, topk).expand(B, L, h_kv, topk).clone()
+    want = torch.where(want < lim.view(1, L, 1, 1), want, torch.full_like(want, -1)).to(torch.int32)
+    assert torch.equal(idx.cpu(), want), "with all scores equal the lowest chunk indices must win"
+    assert torch.equal(idx.cpu(), orc.topk_select(dbg["sel_logits"].cpu(), dbg["lse_total"].cpu(), lim, topk))
