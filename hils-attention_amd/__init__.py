@@ -14,5 +14,5 @@ from .ops.exact_chunk_log_z_tilelang import exact_chunk_log_z_tl  # noqa: F401
 from .ops.hils_glue import chunk_weights, topk_chunk_weights  # noqa: F401
 from .ops.flex_attn_tilelang import flex_attn_tl, flex_attn_tl_two_phase  # noqa: F401
 from .ops.hils_fwd_bwd_head import prepare_kv_workspace  # noqa: F401
-from .utils.hils_cache_utils import HiLSDynamicLayer  # noqa: F401
+from .utils.hils_cache_utils import HiLSDynamicLayer, HiLSPagedLayer, paged_hils_attend  # noqa: F401
 from .ops.rope_tilelang_fp32 import rope_rotary_pos_emb, single_tensor_rope_autograd  # noqa: F401

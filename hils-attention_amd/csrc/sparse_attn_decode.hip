@@ -190,7 +190,8 @@ bool hils_decode_rows_covers(int D, int Dv, int G);
 void hils_sparse_attn_decode_rows(const void* q, const void* k, const void* v, const void* weights,
                                   const int32_t* indices, void* o, void* workspace, int nsplit,
                                   int B, int L, int Lkv, int HQ, int H, int D, int K, int NW,
-                                  float sm_scale, int mask_last, hipStream_t st);
+                                  float sm_scale, int mask_last, const int32_t* page_table, int max_pages,
+                                  int num_pages, hipStream_t st);
 
 int hils_sparse_attn_decode(const void* q, const void* k, const void* v, const void* weights,
                             const int32_t* indices, void* o, void* workspace, int B, int L, int Lkv,
@@ -206,7 +207,7 @@ int hils_sparse_attn_decode(const void* q, const void* k, const void* v, const v
   hipStream_t st = (hipStream_t)stream;
   if (hils_decode_rows_covers(D, Dv, HQ / H)) {
     hils_sparse_attn_decode_rows(q, k, v, weights, indices, o, workspace, nsplit, B, L, Lkv, HQ, H, D,
-                                 K, NW, sm_scale, mask_last, st);
+                                 K, NW, sm_scale, mask_last, nullptr, 0, 0, st);
   } else {
   const size_t smem = ((size_t)DE_WAVES * DE_S * 16 + (size_t)DE_WAVES * dm.G * Dv) * sizeof(float);
 #define DE_CALL(D_, DV_)                                                                           \
@@ -231,5 +232,37 @@ int hils_sparse_attn_decode(const void* q, const void* k, const void* v, const v
     hipLaunchKernelGGL(decode_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                        (const float*)workspace, (bf16_t*)o, rows, Dv, nsplit);
   }
+  return HILS_OK;
+}
+
+// Decode over a paged cache (page = chunk = 64 tokens): k_pages, v_pages (num_pages, H, 64, D) bf16;
+// page_table (B, max_pages) int32, chunk c of batch element b -> page id (negative = unmapped).
+extern "C" size_t hils_sparse_attn_decode_paged_workspace(int B, int L, int HQ, int H, int D, int K) {
+  return hils_decode_workspace_bytes(B, L, HQ, H, D, K);
+}
+
+extern "C" int hils_sparse_attn_decode_paged(const void* q, const void* k_pages, const void* v_pages,
+                                             const int32_t* page_table, const void* weights,
+                                             const int32_t* indices, void* o, void* workspace, int B, int L,
+                                             int HQ, int H, int D, int K, int NW, int max_pages, int num_pages,
+                                             float sm_scale, int mask_last, void* stream) {
+  HILS_REQUIRE(q && k_pages && v_pages && page_table && weights && indices && o,
+               "hils_sparse_attn_decode_paged: null pointer");
+  HILS_REQUIRE(B > 0 && L > 0 && HQ > 0 && H > 0 && HQ % H == 0 && K > 0 && NW >= K && max_pages > 0 && num_pages > 0,
+               "hils_sparse_attn_decode_paged: bad sizes");
+  HILS_REQUIRE(hils_decode_rows_covers(D, D, HQ / H),
+               "hils_sparse_attn_decode_paged: needs D = Dv in {64, 128} and at most 4 query heads per KV head");
+  HILS_REQUIRE((long)B * L <= 65535L * 32768L && H <= 65535, "hils_sparse_attn_decode_paged: grid too large");
+  const int nsplit = workspace ? de_pick_nsplit(B, L, H, K) : 1;
+  hipStream_t st = (hipStream_t)stream;
+  hils_sparse_attn_decode_rows(q, k_pages, v_pages, weights, indices, o, workspace, nsplit, B, L, 0, HQ, H, D, K,
+                               NW, sm_scale, mask_last, page_table, max_pages, num_pages, st);
+  if (nsplit > 1) {
+    const long rows = (long)B * L * HQ;
+    const long n = rows * D;
+    hipLaunchKernelGGL(decode_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                       (const float*)workspace, (bf16_t*)o, rows, D, nsplit);
+  }
+  HILS_CHECK_LAUNCH("hils_sparse_attn_decode_paged");
   return HILS_OK;
 }

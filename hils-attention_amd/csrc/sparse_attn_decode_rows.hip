@@ -18,6 +18,10 @@
 struct DrDims {
   int L, Lkv, HQ, H, G, K, NW, nchunk, nsplit, mask_last;
   float sm_scale;
+  // paged cache (page = chunk = 64 tokens): K and V are (num_pages, H, 64, D), the tokens of a
+  // (page, head) contiguous, and chunk c of batch element b lives in page page_table[b][c]
+  const int32_t* page_table;
+  int max_pages, num_pages;
 };
 
 template <int D, int GMAX, int NWAVE>
@@ -58,10 +62,18 @@ sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   for (int slot = s_begin + wave; slot < s_end; slot += NWAVE) {
     const int c = indices[(bt * dm.H + hk) * (long)K + slot];
     if (c < 0 || c >= dm.nchunk) continue;
-    const long row0 = (b * dm.Lkv + (long)c * DR_S + tsub) * dm.H + hk;
+    long row0, step;
+    if (dm.page_table) {
+      const int pg = dm.page_table[b * dm.max_pages + c];
+      if (pg < 0 || pg >= dm.num_pages) continue;  // an unmapped chunk contributes nothing
+      row0 = ((long)pg * dm.H + hk) * DR_S + tsub;
+      step = (long)TPI * D;
+    } else {
+      row0 = (b * dm.Lkv + (long)c * DR_S + tsub) * dm.H + hk;
+      step = (long)TPI * dm.H * D;
+    }
     const bf16_t* kp = k + row0 * D + piece * 8;
     const bf16_t* vp = v + row0 * D + piece * 8;
-    const long step = (long)TPI * dm.H * D;
     // flash-style pass over the chunk in NG groups of GI*TPI tokens; every token sub-group
     // (lanes with the same tsub) keeps its own running max / sum / accumulator
     float mrun[GMAX], lrun[GMAX], acc[GMAX][8];
@@ -163,9 +175,11 @@ bool hils_decode_rows_covers(int D, int Dv, int G) { return D == Dv && (D == 64 
 void hils_sparse_attn_decode_rows(const void* q, const void* k, const void* v, const void* weights,
                                   const int32_t* indices, void* o, void* workspace, int nsplit,
                                   int B, int L, int Lkv, int HQ, int H, int D, int K, int NW,
-                                  float sm_scale, int mask_last, hipStream_t st) {
+                                  float sm_scale, int mask_last, const int32_t* page_table, int max_pages,
+                                  int num_pages, hipStream_t st) {
   const int G = HQ / H;
-  DrDims dm{L, Lkv, HQ, H, G, K, NW, Lkv / DR_S, nsplit, mask_last, sm_scale};
+  DrDims dm{L, Lkv, HQ, H, G, K, NW, page_table ? max_pages : Lkv / DR_S, nsplit, mask_last, sm_scale,
+            page_table, max_pages, num_pages};
   dim3 grid(nsplit, H, (unsigned)((long)B * L));
   // nsplit == 1 with many slots: one workgroup of 16 wavefronts per (query, KV head), no partial sums
   const int nwave = (nsplit == 1 && K >= 16) ? 16 : DR_WAVES;

@@ -1278,7 +1278,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                 bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
                 float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
                 int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
-                float sm_scale) {
+                float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages) {
   constexpr int LR = D / 8, TPI = 64 / LR;
   constexpr int THREADS = NW * 64;       // NW = 8 or 16 wavefronts
   constexpr int EPT = TOPK_R_MAXN / THREADS;  // 64-chunk slots of a wavefront's share
@@ -1287,6 +1287,8 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   extern __shared__ float dyn[];
   float* logit_s = dyn;                       // [GMAX][NP] raw scaled logits
   float* pooled = dyn + (size_t)GMAX * NP;    // [NP]
+  // paged chunk keys, lmks = (num_pages, h_kv, D): the row's page ids are staged behind the pooled scores
+  int* page_s = (int*)(pooled + NP);          // [NP], only with a page table
   __shared__ TopkRowShared sh;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int piece = lane % LR, tsub = lane / LR;
@@ -1301,6 +1303,12 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
 #pragma unroll
   for (int g = 0; g < GMAX; ++g) swa[g] = (g < G) ? lse_swa[row * G + g] : 0.f;
   if (tid == 0) sh.next_group = 2 * NW;
+  if (page_table) {
+    for (int c = tid; c < lim; c += THREADS) {
+      int pg = c < max_pages ? page_table[b * max_pages + c] : -1;
+      page_s[c] = (pg >= 0 && pg < num_pages) ? pg : -1;
+    }
+  }
   __syncthreads();
 
   // ---- phase 1: logits of the visible chunks ----
@@ -1314,12 +1322,18 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     const int ngroups = (lim + KG - 1) / KG;
     const bf16_t* base = lmks + (b * N * (long)h_kv + hk) * D + piece * 8;
     const long cstride = (long)h_kv * D;
+    const bf16_t* pbase = lmks + (long)hk * D + piece * 8;  // paged: + page * h_kv * D
     auto fetch = [&](uint4 (&kr)[GI], int grp) {
 #pragma unroll
       for (int it = 0; it < GI; ++it) {
         int c = grp * KG + it * TPI + tsub;
         c = c < N ? c : N - 1;
-        kr[it] = *(const uint4*)(base + c * cstride);
+        if (page_table) {
+          const int pg = c < lim ? page_s[c] : -1;  // an unmapped chunk reads page 0 and is masked below
+          kr[it] = *(const uint4*)(pbase + (long)(pg < 0 ? 0 : pg) * cstride);
+        } else {
+          kr[it] = *(const uint4*)(base + c * cstride);
+        }
       }
     };
     auto consume = [&](const uint4 (&kr)[GI], int grp) {
@@ -1330,7 +1344,8 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
         for (int g = 0; g < GMAX; ++g)
           if (g < G) {
             const float sdot = row_sum<LR>(dot8_bf16(qp[g], kr[it], 0.f));
-            if (piece == 0 && c < N) logit_s[g * NP + c] = __fmul_rn(sdot, sm_scale);
+            if (piece == 0 && c < N)
+              logit_s[g * NP + c] = (page_table && c < lim && page_s[c] < 0) ? HILS_NEG_INF : __fmul_rn(sdot, sm_scale);
           }
       }
     };
@@ -1500,10 +1515,11 @@ static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool pla
 static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, int32_t* indices,
                         void* scores, float* lse_total, float* sel_logits, void* weights, int B, int L, int N, int h_kv, int G, int D,
                         int topk, int block_size, int window_size, int causal, int q_offset,
-                        float sm_scale, hipStream_t st) {
+                        float sm_scale, hipStream_t st, const int32_t* page_table = nullptr, int max_pages = 0,
+                        int num_pages = 0) {
   const long rows = (long)B * L * h_kv;
   const int NP = (N + 63) & ~63;
-  const size_t smem = (size_t)5 * NP * sizeof(float);
+  const size_t smem = (size_t)(page_table ? 6 : 5) * NP * sizeof(float);
   // one round of rows or less: 16 wavefronts per row (the whole compute unit streams one row);
   // more rows than compute units: 8, so that two workgroups share a unit and one row's selection
   // overlaps the other row's streaming
@@ -1516,7 +1532,8 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, i
     hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(W_ * 64), smem, st,                      \
                        (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, indices, (bf16_t*)scores, \
                        lse_total, sel_logits, (bf16_t*)weights, L, N, NP, h_kv, G, topk,         \
-                       block_size, window_size, causal, q_offset, sm_scale);                     \
+                       block_size, window_size, causal, q_offset, sm_scale, page_table, max_pages, \
+                       num_pages);                                                               \
   } while (0)
 #define TOPK_ROW_CALL(D_)                                                                        \
   do {                                                                                           \
@@ -1708,6 +1725,31 @@ extern "C" int hils_topk_fwd_weights(const void* q, const void* lmks, const floa
   if (fused) return HILS_OK;
   return hils_chunk_weights(scores, lse_swa, 0, nullptr, nullptr, weights, B, L, h_kv * G, h_kv, N, topk, 0,
                             stream);
+}
+
+// Decode over paged chunk keys (page = chunk = 64 tokens): lmk_pages (num_pages, h_kv, D) bf16 holds
+// the pooled key of every page, page_table (B, max_pages) maps chunk c of batch element b to its
+// page.  Selection + inter-chunk softmax as hils_topk_fwd_weights; one workgroup per (query, KV head).
+extern "C" int hils_topk_fwd_weights_paged(const void* q, const void* lmk_pages, const int32_t* page_table,
+                                           const float* lse_swa, int32_t* indices, void* scores, void* weights,
+                                           float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
+                                           int G, int D, int topk, int block_size, int window_size, int q_offset,
+                                           int max_pages, int num_pages, float sm_scale, void* stream) {
+  HILS_REQUIRE(q && lmk_pages && page_table && lse_swa && indices && scores && weights,
+               "hils_topk_fwd_weights_paged: null pointer");
+  HILS_REQUIRE(B > 0 && L > 0 && N > 0 && h_kv > 0 && max_pages >= N && num_pages > 0,
+               "hils_topk_fwd_weights_paged: sizes must be positive and the page table must cover N chunks");
+  HILS_REQUIRE(G >= 1 && G <= 4 && (D == 64 || D == 128) && N <= TOPK_R_MAXN && topk >= 1 && topk <= TOPK_MAXK &&
+                   block_size > 0,
+               "hils_topk_fwd_weights_paged: needs G <= 4, D in {64, 128}, N <= %d, topk <= %d", TOPK_R_MAXN,
+               TOPK_MAXK);
+  HILS_REQUIRE((long)B * L * h_kv <= 2147483647L, "hils_topk_fwd_weights_paged: grid too large");
+  if (int rc = topk_fwd_row(q, lmk_pages, lse_swa, indices, scores, lse_total, sel_logits, weights, B, L, N, h_kv,
+                            G, D, topk, block_size, window_size, 1, q_offset, sm_scale, (hipStream_t)stream,
+                            page_table, max_pages, num_pages))
+    return rc;
+  HILS_CHECK_LAUNCH("hils_topk_fwd_weights_paged");
+  return HILS_OK;
 }
 
 // ---------------------------------------------------------------------------

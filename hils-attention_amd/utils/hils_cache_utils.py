@@ -12,11 +12,13 @@ import math
 import torch
 
 try:  # imported as part of the package ...
-    from ..ops.chunk_attn_pool_tilelang import chunk_mean_pool
+    from ..ops import _cabi
+    from ..ops.chunk_attn_pool_tilelang import chunk_attn_pool_tilelang, chunk_mean_pool
     from ..ops.hils_fwd_bwd_head import HiLS_block_M_head
     from ..ops.hils_glue import topk_chunk_weights
 except ImportError:  # ... or with the package directory itself on sys.path (`from utils... import`)
-    from ops.chunk_attn_pool_tilelang import chunk_mean_pool
+    from ops import _cabi
+    from ops.chunk_attn_pool_tilelang import chunk_attn_pool_tilelang, chunk_mean_pool
     from ops.hils_fwd_bwd_head import HiLS_block_M_head
     from ops.hils_glue import topk_chunk_weights
 
@@ -104,3 +106,143 @@ class HiLSDynamicLayer:
         o = HiLS_block_M_head(q, self.keys, self.values, w, idx, block_size=S, sm_scale=sm_scale,
                               is_training=False)
         return o, w, idx
+
+
+class HiLSPagedLayer:
+    """KV cache of one HiLS layer in pages of one chunk (64 tokens), the layout a paged serving
+    backend keeps (the reference's SGLang backend requires page size = chunk size, README.md:262-264).
+
+    ``k_pages`` / ``v_pages``: (num_pages, H, 64, D), the 64 tokens of a (page, head) contiguous;
+    ``lmk_pages``: (num_pages, H, D), the pooled key of every full page: the mean of its 64 keys, or,
+    when ``update`` is given the chunks' prior queries ``mu_q``, the attention-pooled key with the
+    entropy bias ``prior_b`` (num_pages, h_q) beside it (what the reference keeps per layer in
+    ``_hils_prior_cache``, models/FlashHiLS/hils_attention.py:361-416); ``page_table``: (B, max_pages)
+    int32, chunk c of sequence b -> page, -1 = not mapped.  All sequences of the batch have the same
+    length (the kernels take one query offset, as the reference's do).  Pages come from a free list,
+    so the page order of a sequence is arbitrary."""
+
+    def __init__(self, num_pages, batch, max_pages_per_seq, num_kv_heads, head_dim, device,
+                 num_q_heads=None, chunk_pooling=True, page_order=None, dtype=torch.bfloat16):
+        self.S = 64
+        self.B, self.H, self.D = int(batch), int(num_kv_heads), int(head_dim)
+        self.num_pages, self.max_pages = int(num_pages), int(max_pages_per_seq)
+        self.k_pages = torch.zeros((num_pages, self.H, self.S, self.D), dtype=dtype, device=device)
+        self.v_pages = torch.zeros_like(self.k_pages)
+        self.lmk_pages = torch.zeros((num_pages, self.H, self.D), dtype=dtype, device=device)
+        self.prior_b = None
+        if num_q_heads is not None:
+            self.prior_b = torch.zeros((num_pages, int(num_q_heads)), dtype=torch.float32, device=device)
+        self.chunk_pooling = bool(chunk_pooling)
+        self.page_table = torch.full((self.B, self.max_pages), -1, dtype=torch.int32, device=device)
+        # pages are handed out from the end of this list
+        order = list(range(num_pages - 1, -1, -1)) if page_order is None else [int(p) for p in reversed(page_order)]
+        self.free_pages = order
+        self.seq_len = 0
+        self.pooled_chunks = 0
+
+    def get_seq_length(self):
+        return self.seq_len
+
+    def update(self, key_states, value_states, mu_q=None):
+        """Append (B, T, H, D) keys / values.  ``mu_q`` (B, new_full_chunks, h_q, D): the prior queries
+        of the chunks this call completes; with it their pooled keys are attention-pooled and the
+        entropy bias is kept (mean-pooled keys replace them when ``chunk_pooling``)."""
+        B, T, H, D = key_states.shape
+        assert (B, H, D) == (self.B, self.H, self.D)
+        S, dev = self.S, self.k_pages.device
+        a, b_end = self.seq_len, self.seq_len + T
+        need = (b_end + S - 1) // S
+        have = (a + S - 1) // S
+        assert need <= self.max_pages, "the page table is too short for this sequence length"
+        if need > have:
+            n_new = (need - have) * B
+            assert n_new <= len(self.free_pages), "out of pages"
+            new = torch.tensor([self.free_pages.pop() for _ in range(n_new)], dtype=torch.int32,
+                               device=dev).view(need - have, B).t()
+            self.page_table[:, have:need] = new
+        pos = torch.arange(a, b_end, device=dev)
+        pages = self.page_table[:, pos // S].long()                      # (B, T)
+        slots = (pos % S).view(1, T).expand(B, T)
+        hh = torch.arange(H, device=dev).view(1, 1, H)
+        self.k_pages[pages.unsqueeze(-1), hh, slots.unsqueeze(-1)] = key_states
+        self.v_pages[pages.unsqueeze(-1), hh, slots.unsqueeze(-1)] = value_states
+        self.seq_len = b_end
+        full = b_end // S
+        if full > self.pooled_chunks:
+            c0 = self.pooled_chunks
+            pg = self.page_table[:, c0:full].long().reshape(-1)          # (B * n) pages, batch-major
+            kk = self.k_pages[pg]                                        # (B*n, H, 64, D), a copy
+            pooled = None
+            if self.chunk_pooling or mu_q is None:
+                # every (page, head) is a 64-token sequence of its own for the pooling kernel
+                pooled = chunk_mean_pool(kk.view(-1, S, 1, D), S).view(-1, H, D)
+            if mu_q is not None:
+                hq = mu_q.shape[2]
+                G = hq // H
+                assert mu_q.shape == (B, full - c0, hq, D), f"mu_q shape {tuple(mu_q.shape)}"
+                kc = kk.permute(0, 2, 1, 3).repeat_interleave(G, dim=2).unsqueeze(1).contiguous()  # (B*n,1,64,hq,D)
+                lk, lb = chunk_attn_pool_tilelang(mu_q.reshape(-1, 1, hq, D).contiguous(), kc)
+                if self.prior_b is not None:
+                    self.prior_b[pg] = lb.reshape(-1, hq).float()
+                if pooled is None:
+                    assert G == 1, "attention-pooled chunk keys of a grouped layer are per query head"
+                    pooled = lk.reshape(-1, H, D)
+            self.lmk_pages[pg] = pooled.to(self.lmk_pages.dtype)
+            self.pooled_chunks = full
+
+    def gather_contiguous(self):
+        """(B, seq_len, H, D) keys and values in token order (for the local branch, or checks)."""
+        S = self.S
+        n = (self.seq_len + S - 1) // S
+        pg = self.page_table[:, :n].long()
+        k = self.k_pages[pg].permute(0, 1, 3, 2, 4).reshape(self.B, n * S, self.H, self.D)[:, : self.seq_len]
+        v = self.v_pages[pg].permute(0, 1, 3, 2, 4).reshape(self.B, n * S, self.H, self.D)[:, : self.seq_len]
+        return k.contiguous(), v.contiguous()
+
+    def hils_attend(self, q, lse_swa, topk, window_size, sm_scale=None, _debug=None):
+        """The remote branch for the last ``q.shape[1]`` positions: selection, inter-chunk softmax and
+        sparse attention straight on the pages.  Returns (o (B,Lq,h_q,D), weights (B,Lq,h_q,topk+1),
+        indices (B,Lq,H,topk) as chunk numbers of the sequence)."""
+        return paged_hils_attend(q, self.k_pages, self.v_pages, self.lmk_pages, self.page_table, lse_swa,
+                                 self.seq_len, topk, window_size, sm_scale=sm_scale, _debug=_debug)
+
+
+def paged_hils_attend(q, k_pages, v_pages, lmk_pages, page_table, lse_swa, seq_len, topk, window_size,
+                      sm_scale=None, _debug=None):
+    """Selection + inter-chunk softmax + sparse attention of the last ``q.shape[1]`` positions of a
+    ``seq_len``-token sequence kept in pages (layouts: see ``HiLSPagedLayer``)."""
+    _cabi.require_gpu_bf16("paged_hils_attend", q, k_pages, v_pages, lmk_pages)
+    B, Lq, HQ, D = q.shape
+    num_pages, H, S, Dk = k_pages.shape
+    assert S == 64 and Dk == D and v_pages.shape == k_pages.shape and lmk_pages.shape == (num_pages, H, D)
+    assert page_table.dtype == torch.int32 and page_table.shape[0] == B and page_table.is_contiguous()
+    assert HQ % H == 0
+    G = HQ // H
+    max_pages = page_table.shape[1]
+    N = seq_len // S  # chunks with a pooled key
+    assert 0 < N <= max_pages
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    dev = q.device
+    lse = lse_swa.reshape(B, Lq, HQ).float().contiguous()
+    indices = torch.empty((B, Lq, H, topk), dtype=torch.int32, device=dev)
+    scores = torch.empty((B, Lq, HQ, topk), dtype=q.dtype, device=dev)
+    weights = torch.empty((B, Lq, HQ, topk + 1), dtype=q.dtype, device=dev)
+    lse_total = sel_logits = None
+    if _debug is not None:
+        lse_total = torch.empty((B, Lq, H, G), dtype=torch.float32, device=dev)
+        sel_logits = torch.full((B, Lq, H, G, N), float("-inf"), dtype=torch.float32, device=dev)
+    qc = q.contiguous()
+    _cabi.call("hils_topk_fwd_weights_paged", _cabi.ptr(qc), _cabi.ptr(lmk_pages), _cabi.ptr(page_table),
+               _cabi.ptr(lse), _cabi.ptr(indices), _cabi.ptr(scores), _cabi.ptr(weights), _cabi.ptr(lse_total),
+               _cabi.ptr(sel_logits), B, Lq, N, H, G, D, int(topk), S, int(window_size), seq_len - Lq,
+               max_pages, num_pages, float(sm_scale))
+    if _debug is not None:
+        _debug.update(lse_total=lse_total, sel_logits=sel_logits, scores=scores)
+    o = torch.empty((B, Lq, HQ, D), dtype=q.dtype, device=dev)
+    n_ws = _cabi.load().hils_sparse_attn_decode_paged_workspace(B, Lq, HQ, H, D, int(topk))
+    ws = torch.empty(n_ws, dtype=torch.uint8, device=dev) if n_ws else None
+    _cabi.call("hils_sparse_attn_decode_paged", _cabi.ptr(qc), _cabi.ptr(k_pages), _cabi.ptr(v_pages),
+               _cabi.ptr(page_table), _cabi.ptr(weights), _cabi.ptr(indices), _cabi.ptr(o), _cabi.ptr(ws),
+               B, Lq, HQ, H, D, int(topk), topk + 1, max_pages, num_pages, float(sm_scale), 1)
+    return o, weights, indices

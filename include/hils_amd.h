@@ -195,6 +195,34 @@ int hils_sparse_attn_bwd(const void* q, const void* k, const void* v, const void
                          int WH, int q_block, int S, float sm_scale, int mask_last, float sm_n,
                          const void* swa_o, void* d_swa_o, int merge_col, void* stream);
 
+/* ---- decode over a paged cache (page = chunk = 64 tokens) ------------------------------ */
+
+/* The serving backend of the reference keeps the KV cache in pages of one chunk (README.md:262-264)
+ * and the layer's per-chunk keys beside it (models/FlashHiLS/hils_attention.py:361-416,
+ * utils/hils_cache_utils.py:8-76).  Layout here: k_pages, v_pages (num_pages, H, 64, D) bf16 (the 64
+ * tokens of a (page, head) contiguous: one 16 KiB read per selected chunk and tensor at D = 128);
+ * lmk_pages (num_pages, h_kv, D) bf16 = the pooled key of every page; page_table (B, max_pages)
+ * int32 maps chunk c of batch element b to its page (negative or >= num_pages = unmapped: the chunk
+ * is invisible to the selection and contributes nothing to the attention).
+ *
+ * hils_topk_fwd_weights_paged: selection + inter-chunk softmax as hils_topk_fwd_weights (shared
+ * chunk keys, no bias / noise / drop mask, causal), N = chunks of the sequence, L <= a few queries;
+ * lse_total / sel_logits optional as in hils_topk_fwd.
+ * hils_sparse_attn_decode_paged: hils_sparse_attn_fwd's decode path; indices are chunk numbers of the
+ * sequence (what the selection returns).  workspace: hils_sparse_attn_decode_paged_workspace bytes
+ * or NULL. */
+int hils_topk_fwd_weights_paged(const void* q, const void* lmk_pages, const int32_t* page_table,
+                                const float* lse_swa, int32_t* indices, void* scores, void* weights,
+                                float* lse_total, float* sel_logits, int B, int L, int N, int h_kv, int G,
+                                int D, int topk, int block_size, int window_size, int q_offset,
+                                int max_pages, int num_pages, float sm_scale, void* stream);
+size_t hils_sparse_attn_decode_paged_workspace(int B, int L, int HQ, int H, int D, int K);
+int hils_sparse_attn_decode_paged(const void* q, const void* k_pages, const void* v_pages,
+                                  const int32_t* page_table, const void* weights, const int32_t* indices,
+                                  void* o, void* workspace, int B, int L, int HQ, int H, int D, int K,
+                                  int NW, int max_pages, int num_pages, float sm_scale, int mask_last,
+                                  void* stream);
+
 /* ---- exact per-chunk log Z ---------------------------------------------------- */
 
 /* Forward.  Replaces exact_chunk_log_z_fwd (ops/exact_chunk_log_z_tilelang.py:25-137).

@@ -40,6 +40,7 @@ def test_binding_matches_header(pkg):
     fns.pop("hils_topk_bwd_workspace")
     fns.pop("hils_topk_fwd_workspace")
     fns.pop("hils_topk_fwd_noalloc_max_workspace")
+    fns.pop("hils_sparse_attn_decode_paged_workspace")
     assert set(_cabi.SIGNATURES) == set(fns)
     for name, params in fns.items():
         argtypes = _cabi.SIGNATURES[name]
