@@ -186,7 +186,7 @@ size_t hils_decode_workspace_bytes(int B, int L, int HQ, int H, int Dv, int K) {
   return nsplit == 1 ? 0 : (size_t)B * L * HQ * nsplit * Dv * sizeof(float);
 }
 
-bool hils_decode_rows_covers(int D, int Dv, int G);
+bool hils_decode_rows_covers(int D, int Dv, int G, int K);
 void hils_sparse_attn_decode_rows(const void* q, const void* k, const void* v, const void* weights,
                                   const int32_t* indices, void* o, void* workspace, int nsplit,
                                   int B, int L, int Lkv, int HQ, int H, int D, int K, int NW,
@@ -205,7 +205,7 @@ int hils_sparse_attn_decode(const void* q, const void* k, const void* v, const v
   DeDims dm{L, Lkv, HQ, H, HQ / H, K, NW, Lkv / DE_S, nsplit, mask_last, sm_scale};
   dim3 grid(nsplit, H, (unsigned)((long)B * L));
   hipStream_t st = (hipStream_t)stream;
-  if (hils_decode_rows_covers(D, Dv, HQ / H)) {
+  if (hils_decode_rows_covers(D, Dv, HQ / H, K)) {
     hils_sparse_attn_decode_rows(q, k, v, weights, indices, o, workspace, nsplit, B, L, Lkv, HQ, H, D,
                                  K, NW, sm_scale, mask_last, nullptr, 0, 0, st);
   } else {
@@ -250,8 +250,8 @@ extern "C" int hils_sparse_attn_decode_paged(const void* q, const void* k_pages,
                "hils_sparse_attn_decode_paged: null pointer");
   HILS_REQUIRE(B > 0 && L > 0 && HQ > 0 && H > 0 && HQ % H == 0 && K > 0 && NW >= K && max_pages > 0 && num_pages > 0,
                "hils_sparse_attn_decode_paged: bad sizes");
-  HILS_REQUIRE(hils_decode_rows_covers(D, D, HQ / H),
-               "hils_sparse_attn_decode_paged: needs D = Dv in {64, 128} and at most 4 query heads per KV head");
+  HILS_REQUIRE(hils_decode_rows_covers(D, D, HQ / H, K),
+               "hils_sparse_attn_decode_paged: needs D = Dv in {64, 128}, at most 4 query heads per KV head, K <= 1024");
   HILS_REQUIRE((long)B * L <= 65535L * 32768L && H <= 65535, "hils_sparse_attn_decode_paged: grid too large");
   const int nsplit = workspace ? de_pick_nsplit(B, L, H, K) : 1;
   hipStream_t st = (hipStream_t)stream;
