@@ -25,10 +25,22 @@ import __graft_entry__ as entry  # noqa: E402
 
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the readings of
-# a 512 MiB copy: x2.0 and x1.0), see profiles/hbm_traffic_fetch_write_size.md
-TRAFFIC_PREFILL_ATTN_BYTES = 4.53e9
-TRAFFIC_DECODE_STEP_BYTES = 4.05e8
+
+
+def measured_traffic(key):
+    """HBM bytes per launch of a kernel as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE.
+    The figures live in the committed counter summary, on lines `bench.traffic <key> <bytes>`;
+    None when the summary (or the key) is absent."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_fetch_write_size.md")
+    try:
+        with open(path) as fh:
+            for line in fh:
+                parts = line.split()
+                if len(parts) == 3 and parts[0] == "bench.traffic" and parts[1] == key:
+                    return float(parts[2])
+    except OSError:
+        pass
+    return None
 
 
 def gpu_randn(shape, gen, dev, scale=None, chunk=1 << 26):
@@ -127,7 +139,7 @@ def bench_prefill(pkg, dev, steps, warmup):
     attn_ms = per["attn"]
     roof = {"kernel": "sparse_attn_fwd_gather", "bound": "mfma",
             "achieved": flops / (attn_ms * 1e-3) / 1e12, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": flops / (attn_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, "traffic": TRAFFIC_PREFILL_ATTN_BYTES,
+            "frac": flops / (attn_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, "traffic": measured_traffic("prefill_attention_bytes_per_launch"),
             "flops_per_launch": flops, "ms_per_launch": attn_ms}
     cfg = {"workload": "prefill_fwd B1 L32768 hq32/hkv8 D128 chunk64 top32 causal (7B-shaped, config 3)",
            "global_batch": B, "seq_len": L, "n_sel": n_sel}
@@ -227,7 +239,7 @@ def bench_decode(pkg, dev, steps, warmup):
     total = lmk_bytes + kv_bytes + small
     roof = {"kernel": "topk_fwd + sparse_attn_fwd (decode step)", "bound": "hbm",
             "achieved": total / sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": total / sec / 1e9 / HBM_PEAK_GBS, "traffic": TRAFFIC_DECODE_STEP_BYTES, "bytes_per_step": total,
+            "frac": total / sec / 1e9 / HBM_PEAK_GBS, "traffic": measured_traffic("decode_step_bytes"), "bytes_per_step": total,
             "topk_gbs": lmk_bytes / (per["topk"] * 1e-3) / 1e9,
             "attn_gbs": kv_bytes / (per["attn"] * 1e-3) / 1e9}
     del kc, vc

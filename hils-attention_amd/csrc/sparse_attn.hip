@@ -369,9 +369,9 @@ bool hils_bw_covers(int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S, 
 size_t hils_bw_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S,
                                int q_block, int WH, float sm_n);
 int hils_bw_run(const void* q, const void* k, const void* v, const void* weights, const int32_t* indices,
-                const float* lse, const void* d_o, void* dq, float* dk, float* dv, float* dw,
+                const float* lse, const void* d_o, void* dq, void* dk, void* dv, float* dw,
                 void* workspace, int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
-                float sm_scale, int mask_last, void* stream);
+                float sm_scale, int mask_last, int kv16, void* stream);
 
 extern "C" size_t hils_sparse_attn_bwd_workspace(int B, int L, int Lkv, int HQ, int H, int D, int Dv,
                                                  int K, int WH, int q_block, int S, float sm_n) {
@@ -409,10 +409,11 @@ merge_local_bwd_kernel(const bf16_t* __restrict__ d_o, const bf16_t* __restrict_
 extern "C" int hils_sparse_attn_bwd(const void* q, const void* k, const void* v,
                                     const void* weights, const int32_t* indices,
                                     const float* slope, const float* lse, const void* d_o,
-                                    void* dq, float* dk, float* dv, float* dw, void* workspace, int B,
+                                    void* dq, void* dk, void* dv, float* dw, void* workspace, int B,
                                     int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int WH,
                                     int q_block, int S, float sm_scale, int mask_last, float sm_n,
-                                    const void* swa_o, void* d_swa_o, int merge_col, void* stream) {
+                                    const void* swa_o, void* d_swa_o, int merge_col, int kv_grad_bf16,
+                                    void* stream) {
   HILS_REQUIRE(q && k && v && weights && indices && lse && d_o && dq && dk && dv && dw,
                "hils_sparse_attn_bwd: null pointer");
   if (int rc = sa_check("hils_sparse_attn_bwd", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
@@ -431,20 +432,22 @@ extern "C" int hils_sparse_attn_bwd(const void* q, const void* k, const void* v,
   if (workspace && hils_bw_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n) > 0 &&
       hils_bw_covers(L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n, slope)) {
     const int rc = hils_bw_run(q, k, v, weights, indices, lse, d_o, dq, dk, dv, dw, workspace, B, L, Lkv, HQ,
-                               H, D, Dv, K, NW, sm_scale, mask_last, stream);
+                               H, D, Dv, K, NW, sm_scale, mask_last, kv_grad_bf16 ? 1 : 0, stream);
     if (rc > 0) return rc;
     if (rc == HILS_OK) {
       HILS_CHECK_LAUNCH("hils_sparse_attn_bwd");
       return HILS_OK;
     }
   }
+  HILS_REQUIRE(!kv_grad_bf16, "hils_sparse_attn_bwd: bf16 dk / dv need the workspace kernels (a workspace of "
+                              "hils_sparse_attn_bwd_workspace bytes > 0 and no slope)");
   SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n, 0};
   size_t smem = ((size_t)dm.G * (D + Dv) + 2 * (size_t)dm.G * S + 3 * dm.G) * sizeof(float);
   HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_bwd: G*(D+Dv+2S) too large for LDS");
   hipLaunchKernelGGL(sparse_attn_bwd_simple, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS),
                      smem, (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k,
                      (const bf16_t*)v, (const bf16_t*)weights, indices, slope, lse,
-                     (const bf16_t*)d_o, (bf16_t*)dq, dk, dv, dw, dm);
+                     (const bf16_t*)d_o, (bf16_t*)dq, (float*)dk, (float*)dv, dw, dm);
   HILS_CHECK_LAUNCH("hils_sparse_attn_bwd");
   return HILS_OK;
 }

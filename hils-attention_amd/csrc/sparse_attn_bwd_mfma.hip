@@ -126,6 +126,7 @@ bw_scatter_kernel(const int32_t* __restrict__ indices, int* __restrict__ cursor,
 struct BwDims {
   int L, Lkv, HQ, H, K, NW, nchunk, mask_last;
   float sm_scale;
+  int out16;  // dk, dv are bf16 tensors that this kernel overwrites (else fp32, added to)
 };
 
 template <int D, int DV, int G>
@@ -134,7 +135,7 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
                const bf16_t* __restrict__ weights, const float* __restrict__ lse,
                const float* __restrict__ delta, const bf16_t* __restrict__ d_o,
                const int* __restrict__ offsets, const uint32_t* __restrict__ pairs,
-               float* __restrict__ dk, float* __restrict__ dv, BwDims dm) {
+               void* __restrict__ dk_out, void* __restrict__ dv_out, BwDims dm) {
   // delta (B,L,HQ,NW) fp32: sum_tokens P dP of every (row, slot), written by the dQ kernel
   constexpr int KS = D / 32, VS = DV / 32;    // k-steps of the two 16x16x32 products
   constexpr int DT = D / 16, VT = DV / 16;    // 16-wide column tiles of dK, dV
@@ -160,7 +161,17 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
   const long b = blockIdx.z;
   const long cell = (b * dm.H + hk) * (long)dm.nchunk + c;
   const int p_lo = offsets[cell], p_hi = offsets[cell + 1];
-  if (p_lo == p_hi) return;
+  if (p_lo == p_hi) {
+    if (dm.out16) {  // nobody selected the chunk: its gradients are zero
+      bf16_t* dk16 = (bf16_t*)dk_out + ((b * dm.Lkv + (long)c * BW_S) * dm.H + hk) * D;
+      bf16_t* dv16 = (bf16_t*)dv_out + ((b * dm.Lkv + (long)c * BW_S) * dm.H + hk) * DV;
+      for (int i = tid; i < BW_S * (D / 8); i += 256)
+        *(uint4*)(dk16 + (long)(i / (D / 8)) * dm.H * D + (i % (D / 8)) * 8) = make_uint4(0, 0, 0, 0);
+      for (int i = tid; i < BW_S * (DV / 8); i += 256)
+        *(uint4*)(dv16 + (long)(i / (DV / 8)) * dm.H * DV + (i % (DV / 8)) * 8) = make_uint4(0, 0, 0, 0);
+    }
+    return;
+  }
 
   // this wavefront's 16 tokens of the chunk as B operands (k = feature, n = token)
   const long tok = (long)c * BW_S + wave * 16 + col;
@@ -275,51 +286,59 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
     }
     lds_barrier();
     const int rows_here = ((npair - round * PPR < PPR) ? npair - round * PPR : PPR) * G;
+    // two 16-row tiles at a time: their P and dS, side by side, are the A operands (m = token,
+    // k = 32 rows) of one 16x16x32 product per column tile; k index 8j + e stands for row
+    // 4j + e of the first tile (e < 4) or row 4j + e - 4 of the second
 #pragma unroll
-    for (int sub = 0; sub < NSUB; ++sub) {
+    for (int sub = 0; sub < NSUB; sub += 2) {
       if (sub * 16 < rows_here) {
-        // ---- S and dP of 16 rows x this wavefront's 16 tokens
-        f32x4_t s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+        uint2 xp[2], xds[2];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const uint4 a = *(const uint4*)(q_rm + (sub * 16 + col) * QROW + (ks * 32 + j * 8) * 2);
-          s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&kb[ks], s, 0, 0, 0);
-        }
+        for (int h2 = 0; h2 < 2; ++h2) {
+          const int sb = sub + h2;
+          // ---- S and dP of 16 rows x this wavefront's 16 tokens
+          f32x4_t s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < VS; ++ks) {
-          const uint4 a = *(const uint4*)(o_rm + (sub * 16 + col) * OROW + (ks * 32 + j * 8) * 2);
-          dp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&vb[ks], dp, 0, 0, 0);
-        }
-        // accumulator layout: column = token `col`, registers = rows 4j..4j+3
-        bw_s4 a_p, a_ds;
-        {
+          for (int ks = 0; ks < KS; ++ks) {
+            const uint4 a = *(const uint4*)(q_rm + (sb * 16 + col) * QROW + (ks * 32 + j * 8) * 2);
+            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&kb[ks], s, 0, 0, 0);
+          }
+#pragma unroll
+          for (int ks = 0; ks < VS; ++ks) {
+            const uint4 a = *(const uint4*)(o_rm + (sb * 16 + col) * OROW + (ks * 32 + j * 8) * 2);
+            dp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&vb[ks], dp, 0, 0, 0);
+          }
+          // accumulator layout: column = token `col`, registers = rows 4j..4j+3
           float pw[4], ds[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int r = sub * 16 + 4 * j + i;
+            const int r = sb * 16 + 4 * j + i;
             float pv = __builtin_amdgcn_exp2f(s[i] * c2 - row_lse[r]);
             if (masked_col) pv = 0.f;
             pw[i] = row_w[r] * pv;
             ds[i] = pw[i] * (dp[i] - row_delta[r]);
           }
-          uint2 x;
-          x.x = pack_bf2(pw[0], pw[1]);
-          x.y = pack_bf2(pw[2], pw[3]);
-          a_p = *(bw_s4*)&x;
-          x.x = pack_bf2(ds[0], ds[1]);
-          x.y = pack_bf2(ds[2], ds[3]);
-          a_ds = *(bw_s4*)&x;
+          xp[h2].x = pack_bf2(pw[0], pw[1]);
+          xp[h2].y = pack_bf2(pw[2], pw[3]);
+          xds[h2].x = pack_bf2(ds[0], ds[1]);
+          xds[h2].y = pack_bf2(ds[2], ds[3]);
         }
-        // ---- dK += dS^T Q, dV += (wP)^T dO: contraction over the 16 rows
+        const uint4 a_p = make_uint4(xp[0].x, xp[0].y, xp[1].x, xp[1].y);
+        const uint4 a_ds = make_uint4(xds[0].x, xds[0].y, xds[1].x, xds[1].y);
+        // ---- dK += dS^T Q, dV += (wP)^T dO: contraction over the 32 rows
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
-          const uint2 bq = *(const uint2*)(q_tr + (sub * D + t * 16 + col) * CS + j * 8);
-          acc_k[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_ds, *(const bw_s4*)&bq, acc_k[t], 0, 0, 0);
+          const uint2 b0 = *(const uint2*)(q_tr + (sub * D + t * 16 + col) * CS + j * 8);
+          const uint2 b1 = *(const uint2*)(q_tr + ((sub + 1) * D + t * 16 + col) * CS + j * 8);
+          const uint4 bq = make_uint4(b0.x, b0.y, b1.x, b1.y);
+          acc_k[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a_ds, *(const bf16x8_t*)&bq, acc_k[t], 0, 0, 0);
         }
 #pragma unroll
         for (int t = 0; t < VT; ++t) {
-          const uint2 bo = *(const uint2*)(o_tr + (sub * DV + t * 16 + col) * CS + j * 8);
-          acc_v[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_p, *(const bw_s4*)&bo, acc_v[t], 0, 0, 0);
+          const uint2 b0 = *(const uint2*)(o_tr + (sub * DV + t * 16 + col) * CS + j * 8);
+          const uint2 b1 = *(const uint2*)(o_tr + ((sub + 1) * DV + t * 16 + col) * CS + j * 8);
+          const uint4 bo = make_uint4(b0.x, b0.y, b1.x, b1.y);
+          acc_v[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a_p, *(const bf16x8_t*)&bo, acc_v[t], 0, 0, 0);
         }
       }
     }
@@ -328,12 +347,22 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const long tk = (long)c * BW_S + wave * 16 + 4 * j + i;
-    float* dkr = dk + ((b * dm.Lkv + tk) * dm.H + hk) * D;
-    float* dvr = dv + ((b * dm.Lkv + tk) * dm.H + hk) * DV;
+    const long rk = ((b * dm.Lkv + tk) * dm.H + hk) * D, rv = ((b * dm.Lkv + tk) * dm.H + hk) * DV;
+    if (dm.out16) {
+      bf16_t* dkr = (bf16_t*)dk_out + rk;
+      bf16_t* dvr = (bf16_t*)dv_out + rv;
 #pragma unroll
-    for (int t = 0; t < DT; ++t) dkr[t * 16 + col] += acc_k[t][i] * dm.sm_scale;
+      for (int t = 0; t < DT; ++t) dkr[t * 16 + col] = f2bf(acc_k[t][i] * dm.sm_scale);
 #pragma unroll
-    for (int t = 0; t < VT; ++t) dvr[t * 16 + col] += acc_v[t][i];
+      for (int t = 0; t < VT; ++t) dvr[t * 16 + col] = f2bf(acc_v[t][i]);
+    } else {
+      float* dkr = (float*)dk_out + rk;
+      float* dvr = (float*)dv_out + rv;
+#pragma unroll
+      for (int t = 0; t < DT; ++t) dkr[t * 16 + col] += acc_k[t][i] * dm.sm_scale;
+#pragma unroll
+      for (int t = 0; t < VT; ++t) dvr[t * 16 + col] += acc_v[t][i];
+    }
   }
 }
 
@@ -678,7 +707,7 @@ size_t hils_bw_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int 
 template <int D, int DV>
 static int bw_launch_dkdv(int G, dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* k,
                           const bf16_t* v, const bf16_t* w, const float* lse, const float* delta,
-                          const bf16_t* d_o, const int* offsets, const uint32_t* pairs, float* dk, float* dv,
+                          const bf16_t* d_o, const int* offsets, const uint32_t* pairs, void* dk, void* dv,
                           const BwDims& dm) {
 #define BW_CALL(G_)                                                                                 \
   hipLaunchKernelGGL((bw_dkdv_kernel<D, DV, G_>), grid, dim3(256), smem, st, q, k, v, w, lse, delta, d_o, \
@@ -746,11 +775,11 @@ void hils_build_chunk_index(const int32_t* indices, int* counts, int* offsets, i
 }
 
 // Whole backward on the MFMA kernels: dq (bf16, written), dw (fp32, written at the valid slots),
-// dk / dv (fp32, accumulated into the caller's buffers).
+// dk / dv (fp32, accumulated into the caller's buffers; or, with kv16, bf16 tensors that are overwritten).
 int hils_bw_run(const void* q, const void* k, const void* v, const void* weights, const int32_t* indices,
-                const float* lse, const void* d_o, void* dq, float* dk, float* dv, float* dw,
+                const float* lse, const void* d_o, void* dq, void* dk, void* dv, float* dw,
                 void* workspace, int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
-                float sm_scale, int mask_last, void* stream) {
+                float sm_scale, int mask_last, int kv16, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   const int nchunk = Lkv / BW_S;
   const size_t cells = (size_t)B * H * nchunk;
@@ -798,7 +827,16 @@ int hils_bw_run(const void* q, const void* k, const void* v, const void* weights
   }
   // ---- inverse index, then dK, dV
   hils_build_chunk_index(indices, counts, offsets, cursor, pairs, B, L, H, K, nchunk, stream);
-  BwDims dm{L, Lkv, HQ, H, K, NW, nchunk, mask_last, sm_scale};
+  BwDims dm{L, Lkv, HQ, H, K, NW, nchunk, mask_last, sm_scale, kv16};
+  if (kv16 && Lkv > nchunk * BW_S) {  // tokens behind the last whole chunk are never attended
+    for (int b2 = 0; b2 < B; ++b2) {
+      const long nk = (long)(Lkv - nchunk * BW_S) * H * D / 2, nv = (long)(Lkv - nchunk * BW_S) * H * Dv / 2;
+      int* pk = (int*)((bf16_t*)dk + ((long)b2 * Lkv + (long)nchunk * BW_S) * H * D);
+      int* pv = (int*)((bf16_t*)dv + ((long)b2 * Lkv + (long)nchunk * BW_S) * H * Dv);
+      hipLaunchKernelGGL(bw_fill_int_kernel, dim3((unsigned)((nk + 255) / 256)), dim3(256), 0, st, pk, 0, nk);
+      hipLaunchKernelGGL(bw_fill_int_kernel, dim3((unsigned)((nv + 255) / 256)), dim3(256), 0, st, pv, 0, nv);
+    }
+  }
   dim3 grid(nchunk, H, B);
   int rc = -1;
 #define BW_D(D_, DV_)                                                                              \

@@ -88,17 +88,22 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
         d_swa = torch.empty_like(swa_in) if swa_in is not None else None
         do = do.to(q.dtype).contiguous()
         dq = torch.empty_like(q)
-        dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
-        dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)
         dw = torch.zeros((B, L, HQ, NW), dtype=torch.float32, device=q.device)
         ws = None
         if slope_dev is None:
             ws = _cabi.sparse_attn_bwd_workspace(q.device, B, L, L_kv, HQ, H, D, Dv, K, HQ, 1, S, 0.0)
+        # the workspace kernels write dk / dv once, as bf16; the shape-generic one adds into fp32
+        kv16 = ws is not None and k.dtype == torch.bfloat16 and v.dtype == torch.bfloat16
+        if kv16:
+            dk, dv = torch.empty_like(k), torch.empty_like(v)
+        else:
+            dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
+            dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)
         _cabi.call("hils_sparse_attn_bwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
                    _cabi.ptr(idx_in), _cabi.ptr(slope_dev), _cabi.ptr(lse), _cabi.ptr(do),
                    _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), _cabi.ptr(ws),
                    B, L, L_kv, HQ, H, D, Dv, K, NW, HQ, 1, S, sm_scale, mask_last, 0.0,
-                   _cabi.ptr(swa_in), _cabi.ptr(d_swa), merge_col)
+                   _cabi.ptr(swa_in), _cabi.ptr(d_swa), merge_col, int(kv16))
         return (dq, dk.to(k.dtype), dv.to(v.dtype), dw.to(ctx.w_dtype), None,
                 None, None, None, None, None, None, d_swa, None)
 

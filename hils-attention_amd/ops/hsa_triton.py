@@ -58,8 +58,6 @@ class _attention(torch.autograd.Function):
         N, L, L_kv, HQ, H, D, Dv, K, q_x, S, sm_scale, sm_n = ctx.cfg
         do = do.to(q.dtype).contiguous()
         dq = torch.empty_like(q)
-        dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
-        dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)
         # The MFMA backward works on per-query indices and per-query-head weights: hand it the
         # block-shared rows expanded (small tensors) and fold the weight gradient back afterwards.
         ws = _cabi.sparse_attn_bwd_workspace(q.device, N, L, L_kv, HQ, H, D, Dv, K, HQ, 1, S, sm_n)
@@ -68,18 +66,21 @@ class _attention(torch.autograd.Function):
             idx_full = idx_in.repeat_interleave(q_x, dim=1).contiguous()
             w_full = w_in.repeat_interleave(q_x, dim=1).repeat_interleave(G, dim=2).contiguous()
             dw_full = torch.zeros((N, L, HQ, K), dtype=torch.float32, device=q.device)
+            dk, dv = torch.empty_like(k), torch.empty_like(v)  # written once, as bf16
             _cabi.call("hils_sparse_attn_bwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_full),
                        _cabi.ptr(idx_full), None, _cabi.ptr(lse), _cabi.ptr(do),
                        _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw_full), _cabi.ptr(ws),
-                       N, L, L_kv, HQ, H, D, Dv, K, K, HQ, 1, S, sm_scale, 0, sm_n, None, None, 0)
+                       N, L, L_kv, HQ, H, D, Dv, K, K, HQ, 1, S, sm_scale, 0, sm_n, None, None, 0, 1)
             dw = dw_full.view(N, L // q_x, q_x, H, G, K).sum(dim=(2, 4))
             return (dq, dk.to(k.dtype), dv.to(v.dtype), dw.to(ctx.w_dtype),
                     None, None, None, None, None, None)
         dw = torch.zeros(w_in.shape, dtype=torch.float32, device=q.device)
+        dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
+        dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)
         _cabi.call("hils_sparse_attn_bwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
                    _cabi.ptr(idx_in), None, _cabi.ptr(lse), _cabi.ptr(do),
                    _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), None,
-                   N, L, L_kv, HQ, H, D, Dv, K, K, H, q_x, S, sm_scale, 0, sm_n, None, None, 0)
+                   N, L, L_kv, HQ, H, D, Dv, K, K, H, q_x, S, sm_scale, 0, sm_n, None, None, 0, 0)
         return (dq, dk.to(k.dtype), dv.to(v.dtype), dw.to(ctx.w_dtype),
                 None, None, None, None, None, None)
 

@@ -177,7 +177,9 @@ int hils_pack_kv_chunks(const void* k, const void* v, void* workspace, int B, in
  * _fill_chunk_mask of ops/hsa_triton.py:201-597.
  * d_o (B,L,HQ,Dv) bf16, lse from the forward.
  * dq (B,L,HQ,D) bf16 (written); dk (B,Lkv,H,D) fp32, dv (B,Lkv,H,Dv) fp32 (ACCUMULATED
- * with atomics: caller zero-fills); dw fp32 (B,L/q_block,WH,NW) (accumulated with
+ * with atomics: caller zero-fills) - or, with kv_grad_bf16 != 0, bf16 tensors of those shapes that
+ * the call OVERWRITES (every element; only with the workspace kernels, an error otherwise: they
+ * sum a chunk's gradient in registers and write it once); dw fp32 (B,L/q_block,WH,NW) (accumulated with
  * atomics when q_block > 1 or WH != HQ, written otherwise: caller zero-fills).
  * workspace: device scratch of hils_sparse_attn_bwd_workspace(...) bytes (0 = shape not covered)
  * for the MFMA kernels: an inverse index (pairs of (query, slot) grouped by chunk) is built there
@@ -190,10 +192,10 @@ size_t hils_sparse_attn_bwd_workspace(int B, int L, int Lkv, int HQ, int H, int 
                                       int WH, int q_block, int S, float sm_n);
 int hils_sparse_attn_bwd(const void* q, const void* k, const void* v, const void* weights,
                          const int32_t* indices, const float* slope, const float* lse,
-                         const void* d_o, void* dq, float* dk, float* dv, float* dw, void* workspace,
+                         const void* d_o, void* dq, void* dk, void* dv, float* dw, void* workspace,
                          int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
                          int WH, int q_block, int S, float sm_scale, int mask_last, float sm_n,
-                         const void* swa_o, void* d_swa_o, int merge_col, void* stream);
+                         const void* swa_o, void* d_swa_o, int merge_col, int kv_grad_bf16, void* stream);
 
 /* ---- decode over a paged cache (page = chunk = 64 tokens) ------------------------------ */
 

@@ -262,18 +262,24 @@ def test_sparse_attn_bwd_mfma_path_matches_generic_path(pkg, dev, B, L, HQ, H, D
     ws = _cabi.sparse_attn_bwd_workspace(dev, B, L, L, HQ, H, D, Dv, K, HQ, 1, 64, 0.0)
     assert ws is not None, "this shape must be covered by the MFMA backward"
     res = []
-    for use_ws in (False, True):
+    for use_ws, kv16 in ((False, 0), (True, 0), (True, 1)):  # kv16: dk / dv written once as bf16
         dq = torch.empty_like(t[0])
-        dk = torch.zeros(t[1].shape, dtype=torch.float32, device=dev)
-        dv = torch.zeros(t[2].shape, dtype=torch.float32, device=dev)
+        if kv16:
+            dk, dv = torch.full_like(t[1], float("nan")), torch.full_like(t[2], float("nan"))
+        else:
+            dk = torch.zeros(t[1].shape, dtype=torch.float32, device=dev)
+            dv = torch.zeros(t[2].shape, dtype=torch.float32, device=dev)
         dw = torch.zeros(B, L, HQ, NW, dtype=torch.float32, device=dev)
         _cabi.call("hils_sparse_attn_bwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(lse), _cabi.ptr(do.to(dev)),
                    _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), _cabi.ptr(ws) if use_ws else None,
-                   B, L, L, HQ, H, D, Dv, K, NW, HQ, 1, 64, scale, mask_last, 0.0, None, None, 0)
+                   B, L, L, HQ, H, D, Dv, K, NW, HQ, 1, 64, scale, mask_last, 0.0, None, None, 0, kv16)
         torch.cuda.synchronize()
         res.append([x.float().cpu() for x in (dq, dk, dv, dw)])
     for name, a, b in zip(("dq", "dk", "dv", "dw"), res[1], res[0]):
         assert_close_bf16(a, b, f"{name} mfma vs generic")
+    for name, a, b in zip(("dk", "dv"), res[2][1:3], res[1][1:3]):
+        assert torch.isfinite(a).all(), f"{name}: the bf16 output mode must write every element"
+        assert_close_bf16(a, b.bfloat16().float(), f"{name} written as bf16 vs accumulated in fp32")
     assert torch.count_nonzero(res[1][3][..., K:]).item() == 0  # weight columns beyond K get no gradient
 
 
