@@ -13,16 +13,19 @@
 //   dV += (w P)^T dO      (16 tokens x Dv, 16x16x16 MFMA over the 16 rows)
 //   dK += scale dS^T Q    (16 tokens x D,  16x16x16 MFMA over the 16 rows)
 //
-// An accumulator-layout tile (lane: column = token, registers = rows 4j..4j+3) is exactly the A
-// operand of the 16x16x16 MFMA with the roles (row m = token, k = rows), so P and dS feed the
-// second pair of products without leaving registers.  Their B operands (k = rows, n = feature)
-// are read from a transposed copy of the gathered Q and dO rows that the workgroup stages in
-// LDS once per tile and all four wavefronts (16 tokens each) share.
+// An accumulator-layout tile (lane: column = token, registers = rows 4j..4j+3) is, two row tiles
+// side by side, exactly the A operand of the 16x16x32 MFMA with the roles (row m = token, k = 32
+// rows), so P and dS feed the second pair of products without leaving registers.  Their B operands
+// (k = rows, n = feature) are columns of the gathered Q and dO rows: the workgroup stages the rows
+// row-major in LDS once per round for all four wavefronts (16 tokens each), and the column reads
+// are the hardware's transposing LDS loads (a 16-lane group fetches a 4 x 16 block and every lane
+// receives one column of it).
 #include "decode_rows.h"
 #include "../../include/hils_amd.h"
 
 #define BW_S 64
 typedef short bw_s4 __attribute__((ext_vector_type(4)));
+typedef unsigned bw_u4 __attribute__((ext_vector_type(4)));  // a 16-byte piece as a register value
 
 __global__ void bw_fill_int_kernel(int* p, int value, long n) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -143,18 +146,10 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
   constexpr int NSUB = 256 / DMAX;            // 16-row tiles staged per round (4 or 2)
   constexpr int ROWS = 16 * NSUB;             // rows per round
   constexpr int PPR = ROWS / G;               // pairs per round
-  constexpr int QROW = D * 2 + 16;            // row-major staging: padded row (bytes)
+  constexpr int QROW = D * 2 + 16;            // staging: padded row (bytes)
   constexpr int OROW = DV * 2 + 16;
-  constexpr int CS = 40;                      // transposed staging: bytes per feature column (16 rows + pad)
-  extern __shared__ __attribute__((aligned(16))) char bw_smem[];
-  char* q_rm = bw_smem;                       // ROWS x QROW
-  char* o_rm = q_rm + ROWS * QROW;            // ROWS x OROW
-  char* q_tr = o_rm + ROWS * OROW;            // NSUB x D x CS
-  char* o_tr = q_tr + NSUB * D * CS;          // NSUB x DV x CS
-  float* row_lse = (float*)(o_tr + NSUB * DV * CS);
-  float* row_w = row_lse + ROWS;
-  float* row_delta = row_w + ROWS;
-
+  constexpr int BUF = ROWS * (QROW + OROW) + 3 * ROWS * 4;  // one staging buffer (bytes)
+  extern __shared__ __attribute__((aligned(16))) char bw_smem[];  // two staging buffers
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, j = lane >> 4;
   const int c = blockIdx.x, hk = blockIdx.y;
@@ -191,9 +186,7 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
   for (int t = 0; t < VT; ++t) acc_v[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   const float c2 = dm.sm_scale * HILS_LOG2E;
 
-  // Staging roles: thread -> (row, 16-byte piece), NQ (NO) items per thread and round.  The
-  // thread of the neighbouring row (row ^ 1, same piece) sits QPP (OPP) lanes away, so a pair of
-  // threads can assemble dwords of (row 2a, row 2a+1) for the transposed copy.
+  // Staging roles: thread -> (row, 16-byte piece), NQ (NO) items per thread and round.
   constexpr int QPP = D / 8, OPP = DV / 8;
   constexpr int NQ = ROWS * QPP / 256, NO = ROWS * OPP / 256;
   constexpr int QRS = 256 / QPP, ORS = 256 / OPP;  // row step between a thread's items
@@ -205,34 +198,34 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
   // Loads below are unconditional from clamped addresses, the pair entries as relaxed atomic
   // loads: a load inside a branch is waited for inside it, and a plain load may be moved next to
   // its use; either way the gathers of a round would queue up behind one another's latency.
-  auto pair_ok = [&](int round, int row) -> bool {  // false for padding rows
+  auto pair_ok = [&](int round, int row) __attribute__((always_inline)) -> bool {  // false for padding rows
     return row < ROWS && round * PPR + row / G < npair;
   };
-  auto pair_of = [&](int round, int row) -> uint32_t {  // pair of a round's row (pair 0 of the chunk for padding rows)
+  auto pair_of = [&](int round, int row) __attribute__((always_inline)) -> uint32_t {  // pair of a round's row (pair 0 of the chunk for padding rows)
     const int pi = round * PPR + row / G;
     return __hip_atomic_load(pairs + p_lo + (pair_ok(round, row) ? pi : 0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   uint32_t pk_q[NQ], pk_o[NO], pk_r;
-  uint4 xq[NQ], xo[NO];
+  bw_u4 xq[NQ], xo[NO];
   float r_l2 = INFINITY, r_dl = 0.f;
   bf16_t r_wb = 0;
   bool r_ok = false;
-  auto load_pairs = [&](int round) {
+  auto load_pairs = [&](int round) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < NQ; ++u) pk_q[u] = pair_of(round, q_row0 + u * QRS);
 #pragma unroll
     for (int u = 0; u < NO; ++u) pk_o[u] = pair_of(round, o_row0 + u * ORS);
     pk_r = pair_of(round, tid);
   };
-  auto fetch = [&](int round) {  // gathers of `round`, whose pairs load_pairs(round) fetched
+  auto fetch = [&](int round) __attribute__((always_inline)) {  // gathers of `round`, whose pairs load_pairs(round) fetched
 #pragma unroll
     for (int u = 0; u < NQ; ++u) {
       // padding rows read the row of the chunk's first pair (finite values): their P is 0, so they add nothing
-      xq[u] = *(const uint4*)(q + ((b * dm.L + (pk_q[u] >> 8)) * (long)dm.HQ + hk * G + (q_row0 + u * QRS) % G) * D + q_pc * 8);
+      xq[u] = *(const bw_u4*)(q + ((b * dm.L + (pk_q[u] >> 8)) * (long)dm.HQ + hk * G + (q_row0 + u * QRS) % G) * D + q_pc * 8);
     }
 #pragma unroll
     for (int u = 0; u < NO; ++u) {
-      xo[u] = *(const uint4*)(d_o + ((b * dm.L + (pk_o[u] >> 8)) * (long)dm.HQ + hk * G + (o_row0 + u * ORS) % G) * DV + o_pc * 8);
+      xo[u] = *(const bw_u4*)(d_o + ((b * dm.L + (pk_o[u] >> 8)) * (long)dm.HQ + hk * G + (o_row0 + u * ORS) % G) * DV + o_pc * 8);
     }
     {
       // raw values; what a padding row gets instead is decided where they are staged, so that
@@ -245,46 +238,48 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
       r_dl = delta[rowi * dm.NW + (pk & 255)];
     }
   };
-  // row-major copy + transposed copy (dwords of two neighbouring rows) of one 16-byte piece
-  auto stage_piece = [&](const uint4& x, int row, int pc, int lanes_apart, char* rm, int rowb, char* tr, int feat) {
-    *(uint4*)(rm + row * rowb + pc * 16) = x;
-    uint4 y;
-    y.x = __shfl_xor((int)x.x, lanes_apart, 64);
-    y.y = __shfl_xor((int)x.y, lanes_apart, 64);
-    y.z = __shfl_xor((int)x.z, lanes_apart, 64);
-    y.w = __shfl_xor((int)x.w, lanes_apart, 64);
-    const bool odd = row & 1;  // even rows write features 0..3 of the piece, odd rows 4..7
-    const uint32_t me0 = odd ? x.z : x.x, me1 = odd ? x.w : x.y;
-    const uint32_t ot0 = odd ? y.z : y.x, ot1 = odd ? y.w : y.y;
-    const uint32_t ev0 = odd ? ot0 : me0, od0 = odd ? me0 : ot0;
-    const uint32_t ev1 = odd ? ot1 : me1, od1 = odd ? me1 : ot1;
-    char* dst = tr + ((row >> 4) * feat + pc * 8 + (odd ? 4 : 0)) * CS + ((row & 15) & ~1) * 2;
-    *(uint32_t*)(dst + 0 * CS) = (ev0 & 0xffffu) | (od0 << 16);
-    *(uint32_t*)(dst + 1 * CS) = (ev0 >> 16) | (od0 & 0xffff0000u);
-    *(uint32_t*)(dst + 2 * CS) = (ev1 & 0xffffu) | (od1 << 16);
-    *(uint32_t*)(dst + 3 * CS) = (ev1 >> 16) | (od1 & 0xffff0000u);
-  };
-  load_pairs(0);
-  fetch(0);
-  load_pairs(1);
-
-  for (int round = 0; round < nround; ++round) {
-    lds_barrier();  // the previous round's staging is no longer read
+  // staging of the gathered rows of a round (in registers since fetch(round)) into buffer `buf`
+  auto stage = [&](int buf) __attribute__((always_inline)) {
+    char* q_rm = bw_smem + buf * BUF;       // ROWS x QROW
+    char* o_rm = q_rm + ROWS * QROW;        // ROWS x OROW
+    float* row_lse = (float*)(o_rm + ROWS * OROW);
+    float* row_w = row_lse + ROWS;
+    float* row_delta = row_w + ROWS;
 #pragma unroll
-    for (int u = 0; u < NQ; ++u) stage_piece(xq[u], q_row0 + u * QRS, q_pc, QPP, q_rm, QROW, q_tr, D);
+    for (int u = 0; u < NQ; ++u) *(bw_u4*)(q_rm + (q_row0 + u * QRS) * QROW + q_pc * 16) = xq[u];
 #pragma unroll
-    for (int u = 0; u < NO; ++u) stage_piece(xo[u], o_row0 + u * ORS, o_pc, OPP, o_rm, OROW, o_tr, DV);
+    for (int u = 0; u < NO; ++u) *(bw_u4*)(o_rm + (o_row0 + u * ORS) * OROW + o_pc * 16) = xo[u];
     if (tid < ROWS) {  // padding rows and empty slots: P = 0
       row_lse[tid] = (r_ok && r_l2 != HILS_NEG_INF) ? r_l2 : INFINITY;
       row_w[tid] = r_ok ? bf2f(r_wb) : 0.f;
       row_delta[tid] = r_ok ? r_dl : 0.f;
     }
-    // next round's gathers fly during this round's arithmetic (the barrier below orders LDS only)
-    if (round + 1 < nround) {
-      fetch(round + 1);
-      load_pairs(round + 2);
-    }
-    lds_barrier();
+  };
+  // one column-read of a staged tile: rows r0 + 4j .. r0 + 4j + 3 of columns c0 .. c0 + 15, this
+  // lane's column.  (Transposing load: lane l of a 16-lane group addresses row l/4, columns
+  // 4*(l%4) .. +3 of the 4 x 16 block and receives column l of it.)
+  typedef short bw_tr4 __attribute__((ext_vector_type(4)));
+  auto col_read = [&](const char* base, int rowb, int r0, int c0) __attribute__((always_inline)) -> uint2 {
+    const char* p = base + (r0 + 4 * j + (col >> 2)) * rowb + (c0 + 4 * (col & 3)) * 2;
+    const bw_tr4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) bw_tr4*)p);
+    return __builtin_bit_cast(uint2, v);
+  };
+  load_pairs(0);
+  fetch(0);
+  load_pairs(1);
+  stage(0);
+  if (nround > 1) {
+    fetch(1);
+    load_pairs(2);
+  }
+  lds_barrier();
+
+  for (int round = 0; round < nround; ++round) {
+    const char* q_rm = bw_smem + (round & 1) * BUF;
+    const char* o_rm = q_rm + ROWS * QROW;
+    const float* row_lse = (const float*)(o_rm + ROWS * OROW);
+    const float* row_w = row_lse + ROWS;
+    const float* row_delta = row_w + ROWS;
     const int rows_here = ((npair - round * PPR < PPR) ? npair - round * PPR : PPR) * G;
     // two 16-row tiles at a time: their P and dS, side by side, are the A operands (m = token,
     // k = 32 rows) of one 16x16x32 product per column tile; k index 8j + e stands for row
@@ -328,20 +323,30 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
         // ---- dK += dS^T Q, dV += (wP)^T dO: contraction over the 32 rows
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
-          const uint2 b0 = *(const uint2*)(q_tr + (sub * D + t * 16 + col) * CS + j * 8);
-          const uint2 b1 = *(const uint2*)(q_tr + ((sub + 1) * D + t * 16 + col) * CS + j * 8);
+          const uint2 b0 = col_read(q_rm, QROW, sub * 16, t * 16);
+          const uint2 b1 = col_read(q_rm, QROW, (sub + 1) * 16, t * 16);
           const uint4 bq = make_uint4(b0.x, b0.y, b1.x, b1.y);
           acc_k[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a_ds, *(const bf16x8_t*)&bq, acc_k[t], 0, 0, 0);
         }
 #pragma unroll
         for (int t = 0; t < VT; ++t) {
-          const uint2 b0 = *(const uint2*)(o_tr + (sub * DV + t * 16 + col) * CS + j * 8);
-          const uint2 b1 = *(const uint2*)(o_tr + ((sub + 1) * DV + t * 16 + col) * CS + j * 8);
+          const uint2 b0 = col_read(o_rm, OROW, sub * 16, t * 16);
+          const uint2 b1 = col_read(o_rm, OROW, (sub + 1) * 16, t * 16);
           const uint4 bo = make_uint4(b0.x, b0.y, b1.x, b1.y);
           acc_v[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a_p, *(const bf16x8_t*)&bo, acc_v[t], 0, 0, 0);
         }
       }
     }
+    // the next round's rows (gathered while this round computed) go to the other buffer, which
+    // was last read a round ago (before the previous barrier); its gathers follow
+    if (round + 1 < nround) {
+      stage((round + 1) & 1);
+      if (round + 2 < nround) {
+        fetch(round + 2);
+        load_pairs(round + 3);
+      }
+    }
+    lds_barrier();
   }
   // accumulators: column = feature t*16 + col, rows = tokens wave*16 + 4j + i
 #pragma unroll
@@ -714,8 +719,8 @@ static int bw_launch_dkdv(int G, dim3 grid, hipStream_t st, const bf16_t* q, con
                      offsets, pairs, dk, dv, dm)
   constexpr int DMAX = D > DV ? D : DV;
   constexpr int NSUB = 256 / DMAX;
-  const size_t smem = (size_t)16 * NSUB * (D * 2 + 16) + (size_t)16 * NSUB * (DV * 2 + 16) +
-                      (size_t)NSUB * (D + DV) * 40 + (size_t)3 * 16 * NSUB * sizeof(float);
+  const size_t smem = 2 * ((size_t)16 * NSUB * (D * 2 + 16) + (size_t)16 * NSUB * (DV * 2 + 16) +
+                           (size_t)3 * 16 * NSUB * sizeof(float));  // two staging buffers
   switch (G) {
     case 1: BW_CALL(1); break;
     case 2: BW_CALL(2); break;

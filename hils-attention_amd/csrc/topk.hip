@@ -1956,6 +1956,206 @@ topk_bwd_dlmk_kernel(const bf16_t* __restrict__ gs, const bf16_t* __restrict__ q
   }
 }
 
+// ---- backward as two small dense products per query block ----
+// The gradient of the gathered scores is a sparse (rows x chunks) matrix A with topk entries per
+// row: dq = sm_scale * A LMK and dlmk = sm_scale * A^T Q.  A workgroup owns TD_R consecutive rows
+// (queries x the heads that share the chunk keys) of one (batch, chunk-key head), scatters their
+// gradients into a dense bf16 tile of A in LDS (128 chunks at a time), and runs both products on
+// 16x16x32 MFMAs with the chunk keys and the query rows staged transposed beside it: no inverse
+// index, every input read once and coalesced.  dlmk tiles of the query blocks are added with
+// float atomics (the summation order over query blocks is not fixed).  The chunk indices of one
+// row must be distinct (they are when they come from the selection).
+#define TD_R 128        // rows per workgroup
+#define TD_NC 128       // chunks per tile (== TD_R: one thread-to-piece split serves rows and chunk keys)
+#define TD_THREADS 512
+#define TD_STRIDE 136   // elements per LDS row: 128 + 8, so that 16-byte operand reads of 16 rows hit 64 banks
+
+template <int D>
+__global__ void __launch_bounds__(TD_THREADS)
+topk_bwd_dense_kernel(const bf16_t* __restrict__ gs, const bf16_t* __restrict__ q,
+                      const bf16_t* __restrict__ lmks, const int32_t* __restrict__ indices,
+                      bf16_t* __restrict__ dq, float* __restrict__ dlmk, int L, int N, int h_kv, int G,
+                      int topk, int per_qhead, float sm_scale) {
+  constexpr int DT = D / 16, PPR = D / 8;
+  extern __shared__ __align__(16) bf16_t td_sm[];
+  bf16_t* A_s = td_sm;                        // [TD_R][TD_STRIDE]   A, row-major
+  bf16_t* At_s = A_s + TD_R * TD_STRIDE;      // [TD_NC][TD_STRIDE]  A transposed
+  bf16_t* Lt_s = At_s + TD_NC * TD_STRIDE;    // [D][TD_STRIDE]      chunk keys of the tile, feature-major
+  bf16_t* Qt_s = Lt_s + D * TD_STRIDE;        // [D][TD_STRIDE]      query rows, feature-major
+  __shared__ int cmax_s;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, j = lane >> 4;
+  // grid order (chunk-key head, batch) fastest, query block slowest: the workgroups in flight at
+  // one time add their dlmk tiles to different (batch, head) slices instead of all to the same one
+  const int lh = blockIdx.x;  // chunk-key head
+  const long b = blockIdx.y;
+  const int lmk_h = per_qhead ? h_kv * G : h_kv;
+  const int hk = per_qhead ? lh / G : lh;
+  const int g_lo = per_qhead ? lh % G : 0, g_n = per_qhead ? 1 : G;
+  const int TQ = TD_R / g_n;
+  const int t0 = blockIdx.z * TQ;
+  auto row_rg = [&](int row) -> long {  // row of gs / q / dq of a block row (valid rows only)
+    return ((b * L + t0 + row / g_n) * h_kv + hk) * (long)G + g_lo + row % g_n;
+  };
+  if (tid == 0) cmax_s = -1;
+  // Every global load of the first tile is issued before anything waits (clamped addresses, no
+  // branches around the loads): query pieces, chunk-key pieces, and the first NI (row, slot)
+  // entries of every thread with their gradients.
+  constexpr int NP = TD_R * PPR / TD_THREADS;  // 16-byte pieces per thread (rows and chunk keys alike)
+  constexpr int NI = 8;                        // (row, slot) entries per thread and batch
+  const int n_item = TD_R * topk;              // entries of the block, row-major like gs
+  uint4 qx[NP], lx[NP];
+#pragma unroll
+  for (int u = 0; u < NP; ++u) {
+    const int i = tid + u * TD_THREADS;
+    const int row = i / PPR, pc = i % PPR;     // the pieces of a row sit in neighbouring lanes
+    const int rc = (t0 + row / g_n < L) ? row : 0;  // row 0 of a block always exists
+    qx[u] = *(const uint4*)(q + row_rg(rc) * D + pc * 8);
+    const int cc = row < N ? row : N - 1;      // TD_NC == TD_R: the same split serves the chunk keys
+    lx[u] = *(const uint4*)(lmks + ((b * N + cc) * (long)lmk_h + lh) * D + pc * 8);
+  }
+  auto item_load = [&](int i, int& c, bf16_t& val) {  // entry i of the block (any i: clamped)
+    const int ic = i < n_item ? i : 0;
+    const int row = ic / topk, slot = ic - row * topk;
+    const bool ok = i < n_item && t0 + row / g_n < L;
+    const int rc = ok ? row : 0;
+    c = indices[((b * L + t0 + rc / g_n) * h_kv + hk) * (long)topk + slot];
+    val = gs[row_rg(rc) * topk + slot];
+    if (!ok || c >= N) c = -1;
+  };
+  int ci[NI];
+  bf16_t gv[NI];
+#pragma unroll
+  for (int u = 0; u < NI; ++u) item_load(tid + u * TD_THREADS, ci[u], gv[u]);
+#pragma unroll
+  for (int u = 0; u < NP; ++u) {
+    const int i = tid + u * TD_THREADS;
+    const int row = i / PPR, pc = i % PPR;
+    const bool ok = t0 + row / g_n < L;
+    const bf16_t* xs = (const bf16_t*)&qx[u];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) Qt_s[(pc * 8 + e) * TD_STRIDE + row] = ok ? xs[e] : (bf16_t)0;
+  }
+  f32x4_t acc_q[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t) acc_q[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  int cmax = 0;
+  for (int c0 = 0; c0 <= cmax; c0 += TD_NC) {
+    // clear both copies of A (the rows of At beyond the tile's chunks stay zero)
+    for (int i = tid; i < (TD_R + TD_NC) * TD_STRIDE / 8; i += TD_THREADS) ((uint4*)A_s)[i] = make_uint4(0, 0, 0, 0);
+    // chunk keys of the tile, feature-major
+#pragma unroll
+    for (int u = 0; u < NP; ++u) {
+      const int i = tid + u * TD_THREADS;
+      const int cl = i / PPR, pc = i % PPR;
+      if (c0 > 0) {
+        const int cc = c0 + cl < N ? c0 + cl : N - 1;
+        lx[u] = *(const uint4*)(lmks + ((b * N + cc) * (long)lmk_h + lh) * D + pc * 8);
+      }
+      const bool ok = c0 + cl < N;
+      const bf16_t* xs = (const bf16_t*)&lx[u];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) Lt_s[(pc * 8 + e) * TD_STRIDE + cl] = ok ? xs[e] : (bf16_t)0;
+    }
+    __syncthreads();
+    int my_max = -1;
+    for (int i0 = 0; i0 < n_item; i0 += NI * TD_THREADS) {
+      if (i0 > 0 || c0 > 0) {
+#pragma unroll
+        for (int u = 0; u < NI; ++u) item_load(i0 + tid + u * TD_THREADS, ci[u], gv[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < NI; ++u) {
+        const int c = ci[u];
+        my_max = c > my_max ? c : my_max;
+        if (c >= c0 && c < c0 + TD_NC) {
+          const int row = (i0 + tid + u * TD_THREADS) / topk;
+          A_s[row * TD_STRIDE + (c - c0)] = gv[u];
+          At_s[(c - c0) * TD_STRIDE + row] = gv[u];
+        }
+      }
+    }
+    if (c0 == 0) {  // largest chunk index of the block: how many tiles there are
+#pragma unroll
+      for (int o2 = 32; o2 >= 1; o2 >>= 1) {
+        const int y = __shfl_xor(my_max, o2, 64);
+        my_max = y > my_max ? y : my_max;
+      }
+      if (lane == 0 && my_max >= 0) atomicMax(&cmax_s, my_max);
+    }
+    __syncthreads();
+    cmax = cmax_s;
+    if (cmax >= c0) {  // (the first tile of a block with no valid entry has nothing to add)
+      // dq rows of this wavefront's row tile += A LMK
+#pragma unroll
+      for (int kc = 0; kc < TD_NC / 32; ++kc) {
+        const uint4 a = *(const uint4*)(A_s + (wave * 16 + col) * TD_STRIDE + kc * 32 + j * 8);
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+          const uint4 bb = *(const uint4*)(Lt_s + (t * 16 + col) * TD_STRIDE + kc * 32 + j * 8);
+          acc_q[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&bb, acc_q[t], 0, 0, 0);
+        }
+      }
+      // dlmk of this wavefront's chunk tile = A^T Q
+      const int c_tile = c0 + wave * 16;
+      if (c_tile <= cmax) {
+        f32x4_t acc_l[DT];
+#pragma unroll
+        for (int t = 0; t < DT; ++t) acc_l[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kr = 0; kr < TD_R / 32; ++kr) {
+          const uint4 a = *(const uint4*)(At_s + (wave * 16 + col) * TD_STRIDE + kr * 32 + j * 8);
+#pragma unroll
+          for (int t = 0; t < DT; ++t) {
+            const uint4 bb = *(const uint4*)(Qt_s + (t * 16 + col) * TD_STRIDE + kr * 32 + j * 8);
+            acc_l[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, *(const bf16x8_t*)&bb, acc_l[t], 0, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int c = c_tile + 4 * j + i;
+          if (c < N) {
+            float* dst = dlmk + ((b * N + c) * (long)lmk_h + lh) * D + col;
+#pragma unroll
+            for (int t = 0; t < DT; ++t) {
+              const float v = acc_l[t][i] * sm_scale;
+              if (v != 0.f) unsafeAtomicAdd(dst + t * 16, v);
+            }
+          }
+        }
+      }
+    }
+    __syncthreads();  // the tile is no longer read
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = wave * 16 + 4 * j + i;
+    if (t0 + row / g_n < L) {
+      bf16_t* dst = dq + row_rg(row) * D + col;
+#pragma unroll
+      for (int t = 0; t < DT; ++t) dst[t * 16] = f2bf(acc_q[t][i] * sm_scale);
+    }
+  }
+}
+
+static bool topk_bwd_dense_covers(int G, int D, int per_qhead) {
+  const int g_n = per_qhead ? 1 : G;
+  return (D == 64 || D == 128) && g_n >= 1 && g_n <= TD_R && TD_R % g_n == 0;
+}
+
+template <int D>
+static int topk_bwd_dense_launch(dim3 grid, hipStream_t st, const bf16_t* gs, const bf16_t* q, const bf16_t* lmks,
+                                 const int32_t* indices, bf16_t* dq, float* dlmk, int L, int N, int h_kv, int G,
+                                 int topk, int per_qhead, float sm_scale) {
+  const size_t smem = (size_t)(TD_R + TD_NC + 2 * D) * TD_STRIDE * sizeof(bf16_t);
+  auto kern = topk_bwd_dense_kernel<D>;
+  static HilsLdsReserve reserved;  // per instantiation
+  if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_topk_bwd")) return rc;
+  hipLaunchKernelGGL(kern, grid, dim3(TD_THREADS), smem, st, gs, q, lmks, indices, dq, dlmk, L, N, h_kv, G, topk,
+                     per_qhead, sm_scale);
+  return HILS_OK;
+}
+
 void hils_build_chunk_index(const int32_t* indices, int* counts, int* offsets, int* cursor, uint32_t* pairs,
                             int B, int L, int H, int K, int nchunk, void* stream);
 
@@ -1963,6 +2163,7 @@ static size_t topk_bwd_round(size_t n) { return (n + 255) & ~(size_t)255; }
 
 extern "C" size_t hils_topk_bwd_workspace(int B, int L, int N, int h_kv, int G, int D, int topk) {
   if (D % 8 != 0 || D > 2048 || topk > 256 || N > 12288 || L >= (1 << 24)) return 0;
+  if (topk_bwd_dense_covers(G, D, 0)) return 0;  // the dense kernel needs no scratch (and covers per-head keys too)
   const size_t cells = (size_t)B * h_kv * N;
   return 3 * topk_bwd_round((cells + 1) * 4) + topk_bwd_round((size_t)B * L * h_kv * topk * 4);
 }
@@ -1976,6 +2177,22 @@ extern "C" int hils_topk_bwd(const void* g_scores, const void* q, const void* lm
   const long rows = (long)B * L * h_kv;
   HILS_REQUIRE(rows <= 2147483647L, "hils_topk_bwd: grid too large");
   hipStream_t st = (hipStream_t)stream;
+  if (topk_bwd_dense_covers(G, D, per_qhead) && B <= 65535 &&
+      (L + TD_R / (per_qhead ? 1 : G) - 1) / (TD_R / (per_qhead ? 1 : G)) <= 65535) {
+    const int g_n = per_qhead ? 1 : G, TQ = TD_R / g_n;
+    const int lmk_h = per_qhead ? h_kv * G : h_kv;
+    dim3 grid(lmk_h, B, (unsigned)((L + TQ - 1) / TQ));
+    int rc;
+    if (D == 64)
+      rc = topk_bwd_dense_launch<64>(grid, st, (const bf16_t*)g_scores, (const bf16_t*)q, (const bf16_t*)lmks, indices,
+                                     (bf16_t*)dq, dlmk, L, N, h_kv, G, topk, per_qhead, sm_scale);
+    else
+      rc = topk_bwd_dense_launch<128>(grid, st, (const bf16_t*)g_scores, (const bf16_t*)q, (const bf16_t*)lmks, indices,
+                                      (bf16_t*)dq, dlmk, L, N, h_kv, G, topk, per_qhead, sm_scale);
+    if (rc) return rc;
+    HILS_CHECK_LAUNCH("hils_topk_bwd");
+    return HILS_OK;
+  }
   if (workspace && hils_topk_bwd_workspace(B, L, N, h_kv, G, D, topk) > 0 && h_kv * G <= 65535 && B <= 65535) {
     const size_t cells = (size_t)B * h_kv * N;
     char* ws = (char*)workspace;

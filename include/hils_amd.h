@@ -108,8 +108,14 @@ int hils_topk_fwd_weights(const void* q, const void* lmks, const float* lse_swa,
  * SoftmaxTopKMaxPoolingFusedFn.backward (ops/topk_head_softmax.py:1040-1092).
  * g_scores (B,L,h_kv,G,topk) bf16 -> dq (B,L,h_kv,G,D) bf16 (written),
  * dlmk fp32 (B,N,h_kv or h_kv*G,D) (ACCUMULATED: caller zero-fills).
- * workspace: device scratch of hils_topk_bwd_workspace(...) bytes; with it the chunk-key gradient
- * is summed chunk by chunk over an inverse index (no atomics); NULL selects the atomic kernel. */
+ * The chunk indices of one (query, KV head) row must be distinct (they are when they come from
+ * the selection).  With D in {64, 128} and G (shared chunk keys) a divisor of 128 the two gradients
+ * are two small dense MFMA products per block of 128 rows, over the rows' gradients scattered into
+ * a dense tile in LDS; the chunk-key tiles of the query blocks are added with float atomics, so the
+ * last bits of dlmk depend on the order the blocks finish in.  Other shapes:
+ * workspace: device scratch of hils_topk_bwd_workspace(...) bytes (0 when none is needed); with it
+ * the chunk-key gradient is summed chunk by chunk over an inverse index (no atomics); NULL selects
+ * the atomic kernel. */
 size_t hils_topk_bwd_workspace(int B, int L, int N, int h_kv, int G, int D, int topk);
 int hils_topk_bwd(const void* g_scores, const void* q, const void* lmks, const int32_t* indices,
                   void* dq, float* dlmk, void* workspace, int B, int L, int N, int h_kv, int G, int D,

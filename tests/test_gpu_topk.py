@@ -212,9 +212,12 @@ def test_topk_reduces_to_torch_topk(pkg, orc, dev):
             assert got == want
 
 
-def test_topk_backward(pkg, orc, dev):
-    B, L, N, h_kv, G, D, topk, S = 1, 512, 8, 2, 4, 64, 4, 64
-    note("topk backward")
+@pytest.mark.parametrize("B,L,N,h_kv,G,D,topk", [(1, 512, 8, 2, 4, 64, 4),        # dense-tile kernel, one tile
+                                                 (1, 8320, 130, 1, 2, 128, 16),   # two chunk tiles, ragged last row block
+                                                 (2, 200, 3, 2, 3, 64, 2)])       # group size not a divisor of 128: inverse-index kernels
+def test_topk_backward(pkg, orc, dev, B, L, N, h_kv, G, D, topk):
+    S = 64
+    note(f"topk backward B{B} L{L} N{N} h_kv{h_kv} G{G} D{D} top{topk}")
     torch.manual_seed(11)
     for per_qhead in (False, True):
         q = torch.randn(B, L, h_kv * G, D).bfloat16()
