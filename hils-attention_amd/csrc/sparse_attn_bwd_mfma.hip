@@ -130,10 +130,13 @@ struct BwDims {
   int L, Lkv, HQ, H, K, NW, nchunk, mask_last;
   float sm_scale;
   int out16;  // dk, dv are bf16 tensors that this kernel overwrites (else fp32, added to)
+  int B;
 };
 
 template <int D, int DV, int G>
-__global__ void __launch_bounds__(256)
+// (64-wide heads fit the register budget of four wavefronts per SIMD: four workgroups per compute
+// unit, whose two 19 KiB staging buffers each just fit the LDS)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((D <= 64 && DV <= 64) ? 4 : 2)))
 bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
                const bf16_t* __restrict__ weights, const float* __restrict__ lse,
                const float* __restrict__ delta, const bf16_t* __restrict__ d_o,
@@ -152,8 +155,15 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
   extern __shared__ __attribute__((aligned(16))) char bw_smem[];  // two staging buffers
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, j = lane >> 4;
-  const int c = blockIdx.x, hk = blockIdx.y;
-  const long b = blockIdx.z;
+  // XCD-aware order: hardware hands consecutive workgroup ids to the 8 XCDs in turn; an XCD works
+  // through the chunks of one (batch, KV head) at a time, so the query and dO rows that its
+  // workgroups gather (the same L rows for every chunk of the head) stay in its L2.
+  const int units = dm.H * dm.B;
+  const int slot = (int)(blockIdx.x / 8);
+  const int unit = (slot / dm.nchunk) * 8 + (int)(blockIdx.x % 8);
+  if (unit >= units) return;
+  const int c = slot % dm.nchunk, hk = unit % dm.H;
+  const long b = unit / dm.H;
   const long cell = (b * dm.H + hk) * (long)dm.nchunk + c;
   const int p_lo = offsets[cell], p_hi = offsets[cell + 1];
   if (p_lo == p_hi) {
@@ -529,15 +539,48 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
     const bf16_t* ka_c = ka + chunk * (long)BW_S * D + lane * 8;
     const bf16_t* va_c = va + chunk * (long)BW_S * DV + lane * 8;
     const bf16_t* kt_c = kt + chunk * (long)BW_S * D + lane * 8;
-    for (int p = vs; p < ve; p += QT) {
+    // Operands of the chunk: K and V as A operands of the two score products, K transposed as B
+    // operand of dQ = dS K.  With 64-wide heads all three stay in registers for every tile of the
+    // visit; wider heads reload them per tile (K transposed into the registers of the first set).
+    constexpr bool KEEP = D <= 64 && DV <= 64;
+    bw_u4 xa[4 * KS], ya[4 * VS], xt[KEEP ? 2 * DT : 1];
+    if (KEEP) {
+#pragma unroll
+      for (int u = 0; u < 4 * KS; ++u) xa[u] = *(const bw_u4*)(ka_c + u * 512);
+#pragma unroll
+      for (int u = 0; u < 4 * VS; ++u) ya[u] = *(const bw_u4*)(va_c + u * 512);
+#pragma unroll
+      for (int u = 0; u < 2 * DT; ++u) xt[u] = *(const bw_u4*)(kt_c + u * 512);
+    }
+    // rows of a tile starting at pair p: this lane's row (pair, gathered q and dO pieces, lse, weight)
+    bw_u4 bq[KS], bdo[VS], bq_n[KEEP ? KS : 1], bdo_n[KEEP ? VS : 1];
+    float l2 = 0.f, l2_n = 0.f;
+    bf16_t wb = 0, wb_n = 0;
+    int pk = 0, pk_n = 0;
+    auto load_rows = [&](int p, bw_u4* q_r, bw_u4* o_r, float& l_r, bf16_t& w_r, int& pk_r)
+                         __attribute__((always_inline)) {
       const int last = ((ve - p < QT) ? ve - p : QT) - 1;  // padding rows repeat the tile's last pair
-      // ---- operands of the two score products and the tile's rows
-      uint4 xa[4 * KS], ya[4 * VS];
+      pk_r = pairs[p + (qs < last ? qs : last)];
+      const long rowi = (b * dm.L + t0 + (pk_r >> 8)) * (long)dm.HQ + hq;
 #pragma unroll
-      for (int u = 0; u < 4 * KS; ++u) xa[u] = *(const uint4*)(ka_c + u * 512);
+      for (int ks = 0; ks < KS; ++ks) q_r[ks] = *(const bw_u4*)(q + rowi * D + ks * 32 + j * 8);
 #pragma unroll
-      for (int u = 0; u < 4 * VS; ++u) ya[u] = *(const uint4*)(va_c + u * 512);
-      const int pk = pairs[p + (qs < last ? qs : last)];
+      for (int ks = 0; ks < VS; ++ks) o_r[ks] = *(const bw_u4*)(d_o + rowi * DV + ks * 32 + j * 8);
+      l_r = lse[rowi * K + (pk_r & 255)];
+      w_r = weights[rowi * dm.NW + (pk_r & 255)];
+    };
+    if (KEEP) load_rows(vs, bq, bdo, l2, wb, pk);
+    for (int p = vs; p < ve; p += QT) {
+      const int last = ((ve - p < QT) ? ve - p : QT) - 1;
+      if (!KEEP) {
+        load_rows(p, bq, bdo, l2, wb, pk);
+#pragma unroll
+        for (int u = 0; u < 4 * KS; ++u) xa[u] = *(const bw_u4*)(ka_c + u * 512);
+#pragma unroll
+        for (int u = 0; u < 4 * VS; ++u) ya[u] = *(const bw_u4*)(va_c + u * 512);
+      }
+      const bool more = KEEP && p + QT < ve;
+      if (more) load_rows(p + QT, bq_n, bdo_n, l2_n, wb_n, pk_n);  // in flight behind this tile's arithmetic
       int pk_o[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -546,14 +589,8 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
       }
       const int ql = pk >> 8, slot = pk & 255;
       const long rowi = (b * dm.L + t0 + ql) * (long)dm.HQ + hq;
-      uint4 bq[KS], bdo[VS];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) bq[ks] = *(const uint4*)(q + rowi * D + ks * 32 + j * 8);
-#pragma unroll
-      for (int ks = 0; ks < VS; ++ks) bdo[ks] = *(const uint4*)(d_o + rowi * DV + ks * 32 + j * 8);
-      float l2 = lse[rowi * K + slot];
       if (l2 == HILS_NEG_INF) l2 = INFINITY;
-      const float w_row = bf2f(weights[rowi * dm.NW + slot]);
+      const float w_row = bf2f(wb);
       int orow[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -573,15 +610,18 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
       for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt)
-          st[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&xa[mt * KS + ks], *(const bf16x8_t*)&bq[ks], st[mt], 0, 0, 0);
+          st[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, xa[mt * KS + ks]),
+                                                           __builtin_bit_cast(bf16x8_t, bq[ks]), st[mt], 0, 0, 0);
 #pragma unroll
       for (int ks = 0; ks < VS; ++ks)
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt)
-          dpt[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&ya[mt * VS + ks], *(const bf16x8_t*)&bdo[ks], dpt[mt], 0, 0, 0);
-      // K of the chunk as B operand of dQ = dS K replaces the first operand set
+          dpt[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ya[mt * VS + ks]),
+                                                            __builtin_bit_cast(bf16x8_t, bdo[ks]), dpt[mt], 0, 0, 0);
+      if (!KEEP) {  // K of the chunk as B operand of dQ = dS K replaces the first operand set
 #pragma unroll
-      for (int u = 0; u < 2 * DT; ++u) xa[u] = *(const uint4*)(kt_c + u * 512);
+        for (int u = 0; u < 2 * DT; ++u) xa[u] = *(const bw_u4*)(kt_c + u * 512);
+      }
       // ---- P, delta, dS (this lane: row r of the tile, tokens mt*16 + 4j + i)
       float delta = 0.f;
 #pragma unroll
@@ -607,7 +647,7 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
         x.y = pack_bf2(f * st[2 * s2][2] * (dpt[2 * s2][2] - delta), f * st[2 * s2][3] * (dpt[2 * s2][3] - delta));
         x.z = pack_bf2(f * st[2 * s2 + 1][0] * (dpt[2 * s2 + 1][0] - delta), f * st[2 * s2 + 1][1] * (dpt[2 * s2 + 1][1] - delta));
         x.w = pack_bf2(f * st[2 * s2 + 1][2] * (dpt[2 * s2 + 1][2] - delta), f * st[2 * s2 + 1][3] * (dpt[2 * s2 + 1][3] - delta));
-        ap[s2] = *(bf16x8_t*)&x;
+        ap[s2] = __builtin_bit_cast(bf16x8_t, x);
       }
       // ---- dQ tile += dS K: four column tiles at a time
 #pragma unroll
@@ -618,12 +658,23 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-          for (int u = 0; u < 4; ++u)
-            acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s2], *(const bf16x8_t*)&xa[(d0 + u) * 2 + s2], acc[u], 0, 0, 0);
+          for (int u = 0; u < 4; ++u) {
+            const bw_u4 kb2 = KEEP ? xt[KEEP ? (d0 + u) * 2 + s2 : 0] : xa[(d0 + u) * 2 + s2];
+            acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s2], __builtin_bit_cast(bf16x8_t, kb2), acc[u], 0, 0, 0);
+          }
 #pragma unroll
         for (int u = 0; u < 4; ++u)
 #pragma unroll
           for (int i = 0; i < 4; ++i) atomicAdd(&q_acc[orow[i] + (d0 + u) * 16], __float2int_rn(acc[u][i]));
+      }
+      if (more) {  // the next tile's rows become the current ones
+#pragma unroll
+        for (int ks = 0; ks < (KEEP ? KS : 1); ++ks) bq[ks] = bq_n[ks];
+#pragma unroll
+        for (int ks = 0; ks < (KEEP ? VS : 1); ++ks) bdo[ks] = bdo_n[ks];
+        l2 = l2_n;
+        wb = wb_n;
+        pk = pk_n;
       }
     }
   }
@@ -832,7 +883,7 @@ int hils_bw_run(const void* q, const void* k, const void* v, const void* weights
   }
   // ---- inverse index, then dK, dV
   hils_build_chunk_index(indices, counts, offsets, cursor, pairs, B, L, H, K, nchunk, stream);
-  BwDims dm{L, Lkv, HQ, H, K, NW, nchunk, mask_last, sm_scale, kv16};
+  BwDims dm{L, Lkv, HQ, H, K, NW, nchunk, mask_last, sm_scale, kv16, B};
   if (kv16 && Lkv > nchunk * BW_S) {  // tokens behind the last whole chunk are never attended
     for (int b2 = 0; b2 < B; ++b2) {
       const long nk = (long)(Lkv - nchunk * BW_S) * H * D / 2, nv = (long)(Lkv - nchunk * BW_S) * H * Dv / 2;
@@ -842,7 +893,9 @@ int hils_bw_run(const void* q, const void* k, const void* v, const void* weights
       hipLaunchKernelGGL(bw_fill_int_kernel, dim3((unsigned)((nv + 255) / 256)), dim3(256), 0, st, pv, 0, nv);
     }
   }
-  dim3 grid(nchunk, H, B);
+  const long unit_rounds = ((long)H * B + 7) / 8;
+  if (unit_rounds * nchunk * 8 > 2147483647L) return -1;
+  dim3 grid((unsigned)(unit_rounds * nchunk * 8));
   int rc = -1;
 #define BW_D(D_, DV_)                                                                              \
   rc = bw_launch_dkdv<D_, DV_>(G, grid, st, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v,   \
