@@ -402,7 +402,11 @@ struct BqDims {
   float sm_scale;
 };
 
-template <int D, int DV, int G>
+// STAGE: the block's own query and dO rows are copied into LDS once (coalesced) and every tile
+// takes its row operands from there instead of gathering them from global memory once per (row,
+// slot) pair; chosen by the launcher when those rows fit beside the output tile without shrinking
+// the block much (narrow heads without grouping).
+template <int D, int DV, int G, bool STAGE>
 __global__ void __launch_bounds__(BQ_THREADS)
 bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const bf16_t* __restrict__ ka,
              const bf16_t* __restrict__ va, const bf16_t* __restrict__ kt, const float* __restrict__ vmax,
@@ -417,7 +421,10 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
   const int R = dm.T * G;
   int* q_acc = smem_i;                       // (R + 1) x D fixed point; row R takes padding rows
   int* cur = q_acc + (size_t)(R + 1) * D;    // nchunk: histogram -> running ends
-  int* pairs = cur + dm.nchunk;              // T*K pairs (query << 8 | slot) grouped by chunk
+  unsigned short* pairs = (unsigned short*)(cur + dm.nchunk);  // T*K pairs (query << 8 | slot) grouped by chunk (T, K <= 256)
+  constexpr int QROWB = D * 2 + 16, OROWB = DV * 2 + 16;       // staged rows, padded (bytes)
+  char* rows_q = (char*)pairs + (((size_t)dm.T * dm.K * 2 + 15) & ~(size_t)15);  // STAGE: R x QROWB
+  char* rows_o = rows_q + (size_t)R * QROWB;                                     //        R x OROWB
   __shared__ float red[32];
   __shared__ int scan_s[BQ_WAVES];
   __shared__ int next_s;
@@ -473,6 +480,20 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
   for (int i = tid; i < (R + 1) * D; i += BQ_THREADS) q_acc[i] = 0;
   for (int i = tid; i < dm.nchunk; i += BQ_THREADS) cur[i] = 0;
   if (tid == 0) next_s = 0;
+  if (STAGE) {  // rows beyond the sequence end are never addressed by a pair
+    for (int i = tid; i < R * (D / 8); i += BQ_THREADS) {
+      const int row = i / (D / 8), pc = i - row * (D / 8);
+      if (t0 + row / G < dm.L)
+        *(bw_u4*)(rows_q + row * QROWB + pc * 16) =
+            *(const bw_u4*)(q + ((b * dm.L + t0 + row / G) * (long)dm.HQ + hk * G + row % G) * D + pc * 8);
+    }
+    for (int i = tid; i < R * (DV / 8); i += BQ_THREADS) {
+      const int row = i / (DV / 8), pc = i - row * (DV / 8);
+      if (t0 + row / G < dm.L)
+        *(bw_u4*)(rows_o + row * OROWB + pc * 16) =
+            *(const bw_u4*)(d_o + ((b * dm.L + t0 + row / G) * (long)dm.HQ + hk * G + row % G) * DV + pc * 8);
+    }
+  }
   __syncthreads();
 #pragma unroll
   for (int e = 0; e < MAXP; ++e)
@@ -509,7 +530,7 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
   __syncthreads();
 #pragma unroll
   for (int e = 0; e < MAXP; ++e)
-    if (creg[e] >= 0) pairs[atomicAdd(&cur[creg[e]], 1)] = preg[e];
+    if (creg[e] >= 0) pairs[atomicAdd(&cur[creg[e]], 1)] = (unsigned short)preg[e];
   __syncthreads();  // now chunk c owns pairs[cur[c-1] .. cur[c])
 
   const float bound = 2.f * dm.sm_scale * rb * vm * km;
@@ -562,10 +583,18 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
       const int last = ((ve - p < QT) ? ve - p : QT) - 1;  // padding rows repeat the tile's last pair
       pk_r = pairs[p + (qs < last ? qs : last)];
       const long rowi = (b * dm.L + t0 + (pk_r >> 8)) * (long)dm.HQ + hq;
+      if (STAGE) {
+        const int row_l = (pk_r >> 8) * G + g;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) q_r[ks] = *(const bw_u4*)(q + rowi * D + ks * 32 + j * 8);
+        for (int ks = 0; ks < KS; ++ks) q_r[ks] = *(const bw_u4*)(rows_q + row_l * QROWB + (ks * 32 + j * 8) * 2);
 #pragma unroll
-      for (int ks = 0; ks < VS; ++ks) o_r[ks] = *(const bw_u4*)(d_o + rowi * DV + ks * 32 + j * 8);
+        for (int ks = 0; ks < VS; ++ks) o_r[ks] = *(const bw_u4*)(rows_o + row_l * OROWB + (ks * 32 + j * 8) * 2);
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) q_r[ks] = *(const bw_u4*)(q + rowi * D + ks * 32 + j * 8);
+#pragma unroll
+        for (int ks = 0; ks < VS; ++ks) o_r[ks] = *(const bw_u4*)(d_o + rowi * DV + ks * 32 + j * 8);
+      }
       l_r = lse[rowi * K + (pk_r & 255)];
       w_r = weights[rowi * dm.NW + (pk_r & 255)];
     };
@@ -716,19 +745,26 @@ void hils_ga_pack_launch(const void* a, const void* b, void* ap, void* bp, float
                          int H, int Da, int Db, void* stream);
 
 // T queries per workgroup of the dQ kernel such that the fixed-point tile, the chunk histogram
-// and the pair list fit in LDS; 0 when the shape does not fit.
-static int bq_pick_T(int L, int G, int D, int K, int nchunk, size_t* smem_out) {
+// and the pair list (and, with `stage`, the block's own query and dO rows) fit in LDS; 0 when the
+// shape does not fit.
+static size_t bq_smem_bytes(int T, int G, int D, int Dv, int K, int nchunk, bool stage) {
+  size_t n = (size_t)(T * G + 1) * D * 4 + (size_t)nchunk * 4 + (((size_t)T * K * 2 + 15) & ~(size_t)15);
+  if (stage) n += (size_t)T * G * ((size_t)D * 2 + 16 + (size_t)Dv * 2 + 16);
+  return n;
+}
+static int bq_pick_T(int L, int G, int D, int Dv, int K, int nchunk, bool stage, size_t* smem_out) {
   // the largest block that fits: the more rows share a visit, the fewer K/V bytes per row
   const size_t limit = 156 * 1024;
-  const size_t per_q = (size_t)G * D * 4 + (size_t)K * 4;
-  const size_t fixed = (size_t)D * 4 + (size_t)nchunk * 4;  // spare row, histogram
+  const size_t per_q = (size_t)G * D * 4 + (size_t)K * 2 + (stage ? (size_t)G * ((size_t)(D + Dv) * 2 + 32) : 0);
+  const size_t fixed = (size_t)D * 4 + (size_t)nchunk * 4 + 16;  // spare row, histogram, alignment
   if (fixed + per_q > limit) return 0;
   long T = (long)((limit - fixed) / per_q);
+  if (T > 256) T = 256;  // a pair is (query << 8 | slot) in 16 bits
   if (T * K > BQ_MAXP * BQ_THREADS) T = (BQ_MAXP * BQ_THREADS) / K;
   if (T > L) T = L;
   if (T >= 8) T &= ~7L;
   if (T < 1) return 0;
-  *smem_out = fixed + (size_t)T * per_q;
+  *smem_out = bq_smem_bytes((int)T, G, D, Dv, K, nchunk, stage);
   return (int)T;
 }
 
@@ -756,7 +792,7 @@ size_t hils_bw_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int 
                                int q_block, int WH, float sm_n) {
   if (!hils_bw_covers(L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n, nullptr)) return 0;
   size_t smem;
-  if (bq_pick_T(L, HQ / H, D, K, Lkv / S, &smem) == 0) return 0;
+  if (bq_pick_T(L, HQ / H, D, Dv, K, Lkv / S, false, &smem) == 0) return 0;
   return bw_layout(B, L, Lkv, H, D, Dv, K).total;
 }
 
@@ -784,12 +820,12 @@ static int bw_launch_dkdv(int G, dim3 grid, hipStream_t st, const bf16_t* q, con
   return HILS_OK;
 }
 
-template <int D, int DV, int G>
+template <int D, int DV, int G, bool STAGE>
 static int bq_launch(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, const bf16_t* d_o,
                      const bf16_t* ka, const bf16_t* va, const bf16_t* kt, const float* vmax,
                      const float* kmax, const bf16_t* w, const int32_t* idx, const float* lse, bf16_t* dq,
                      float* dw, const BqDims& dm) {
-  auto kern = bw_dq_kernel<D, DV, G>;
+  auto kern = bw_dq_kernel<D, DV, G, STAGE>;
   static HilsLdsReserve reserved;  // per instantiation
   if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_sparse_attn_bwd")) return rc;
   hipLaunchKernelGGL(kern, grid, dim3(BQ_THREADS), smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
@@ -797,18 +833,30 @@ static int bq_launch(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, co
 }
 
 template <int D, int DV>
-static int bq_dispatch_g(int G, dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, const bf16_t* d_o,
-                         const bf16_t* ka, const bf16_t* va, const bf16_t* kt, const float* vmax,
-                         const float* kmax, const bf16_t* w, const int32_t* idx, const float* lse,
-                         bf16_t* dq, float* dw, const BqDims& dm) {
+static int bq_dispatch_g(int G, bool stage, dim3 grid, size_t smem, hipStream_t st, const bf16_t* q,
+                         const bf16_t* d_o, const bf16_t* ka, const bf16_t* va, const bf16_t* kt,
+                         const float* vmax, const float* kmax, const bf16_t* w, const int32_t* idx,
+                         const float* lse, bf16_t* dq, float* dw, const BqDims& dm) {
+  if (stage)  // only built without head grouping (see bq_stage_pays)
+    return bq_launch<D, DV, 1, true>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
   switch (G) {
-    case 1: return bq_launch<D, DV, 1>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
-    case 2: return bq_launch<D, DV, 2>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
-    case 4: return bq_launch<D, DV, 4>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
-    case 8: return bq_launch<D, DV, 8>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
-    case 16: return bq_launch<D, DV, 16>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
+    case 1: return bq_launch<D, DV, 1, false>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
+    case 2: return bq_launch<D, DV, 2, false>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
+    case 4: return bq_launch<D, DV, 4, false>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
+    case 8: return bq_launch<D, DV, 8, false>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
+    case 16: return bq_launch<D, DV, 16, false>(grid, smem, st, q, d_o, ka, va, kt, vmax, kmax, w, idx, lse, dq, dw, dm);
   }
   return -1;
+}
+
+// Staging the block's rows in LDS pays when it costs little block size: the block shrinks by the
+// rows' bytes, and a smaller block pulls more K/V bytes per row.
+static bool bq_stage_pays(int L, int G, int D, int Dv, int K, int nchunk) {
+  if (G != 1) return false;
+  size_t a, b2;
+  const int t_plain = bq_pick_T(L, G, D, Dv, K, nchunk, false, &a);
+  const int t_stage = bq_pick_T(L, G, D, Dv, K, nchunk, true, &b2);
+  return t_stage > 0 && 4 * t_stage >= 3 * t_plain;
 }
 
 // Inverse index of an index tensor (B, L, H, K) with values in [0, nchunk) or < 0: counts,
@@ -858,12 +906,13 @@ int hils_bw_run(const void* q, const void* k, const void* v, const void* weights
   // ---- dQ, dW
   {
     size_t smem;
-    int T = bq_pick_T(L, G, D, K, nchunk, &smem);
+    const bool stage = bq_stage_pays(L, G, D, Dv, K, nchunk);
+    int T = bq_pick_T(L, G, D, Dv, K, nchunk, stage, &smem);
     if (T == 0) return -1;
     // small problems: rather every compute unit busy than the largest blocks
     while (T >= 72 && (long)((L + T - 1) / T) * H * B < 256) {
       T -= 8;
-      smem = (size_t)D * 4 + (size_t)nchunk * 4 + (size_t)T * ((size_t)G * D * 4 + (size_t)K * 4);
+      smem = bq_smem_bytes(T, G, D, Dv, K, nchunk, stage);
     }
     const int nblk = (L + T - 1) / T;
     const long total = (long)nblk * H * B;
@@ -872,7 +921,7 @@ int hils_bw_run(const void* q, const void* k, const void* v, const void* weights
     dim3 grid((unsigned)(((total + 7) / 8) * 8));
     int rc = -1;
 #define BQ_D(D_, DV_)                                                                                 \
-  rc = bq_dispatch_g<D_, DV_>(G, grid, smem, st, (const bf16_t*)q, (const bf16_t*)d_o, ka, va, kt, vmax, \
+  rc = bq_dispatch_g<D_, DV_>(G, stage, grid, smem, st, (const bf16_t*)q, (const bf16_t*)d_o, ka, va, kt, vmax, \
                               kmax, (const bf16_t*)weights, indices, lse, (bf16_t*)dq, dw, dm)
     if (D == 64 && Dv == 64) BQ_D(64, 64);
     else if (D == 128 && Dv == 128) BQ_D(128, 128);
