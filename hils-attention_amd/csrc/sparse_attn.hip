@@ -369,8 +369,8 @@ bool hils_bw_covers(int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S, 
 size_t hils_bw_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S,
                                int q_block, int WH, float sm_n);
 int hils_bw_run(const void* q, const void* k, const void* v, const void* weights, const int32_t* indices,
-                const float* lse, const void* d_o, void* dq, void* dk, void* dv, float* dw,
-                void* workspace, int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
+                const float* slope, const float* lse, const void* d_o, void* dq, void* dk, void* dv,
+                float* dw, void* workspace, int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
                 float sm_scale, int mask_last, int kv16, void* stream);
 
 extern "C" size_t hils_sparse_attn_bwd_workspace(int B, int L, int Lkv, int HQ, int H, int D, int Dv,
@@ -431,7 +431,7 @@ extern "C" int hils_sparse_attn_bwd(const void* q, const void* k, const void* v,
   }
   if (workspace && hils_bw_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n) > 0 &&
       hils_bw_covers(L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n, slope)) {
-    const int rc = hils_bw_run(q, k, v, weights, indices, lse, d_o, dq, dk, dv, dw, workspace, B, L, Lkv, HQ,
+    const int rc = hils_bw_run(q, k, v, weights, indices, slope, lse, d_o, dq, dk, dv, dw, workspace, B, L, Lkv, HQ,
                                H, D, Dv, K, NW, sm_scale, mask_last, kv_grad_bf16 ? 1 : 0, stream);
     if (rc > 0) return rc;
     if (rc == HILS_OK) {
@@ -440,7 +440,7 @@ extern "C" int hils_sparse_attn_bwd(const void* q, const void* k, const void* v,
     }
   }
   HILS_REQUIRE(!kv_grad_bf16, "hils_sparse_attn_bwd: bf16 dk / dv need the workspace kernels (a workspace of "
-                              "hils_sparse_attn_bwd_workspace bytes > 0 and no slope)");
+                              "hils_sparse_attn_bwd_workspace bytes > 0)");
   SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n, 0};
   size_t smem = ((size_t)dm.G * (D + Dv) + 2 * (size_t)dm.G * S + 3 * dm.G) * sizeof(float);
   HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_bwd: G*(D+Dv+2S) too large for LDS");

@@ -131,6 +131,7 @@ struct BwDims {
   float sm_scale;
   int out16;  // dk, dv are bf16 tensors that this kernel overwrites (else fp32, added to)
   int B;
+  const float* slope;  // per query head, or null: scores lose slope * max(0, 62 - token) before the softmax
 };
 
 template <int D, int DV, int G>
@@ -188,6 +189,14 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
   for (int ks = 0; ks < VS; ++ks)
     vb[ks] = *(const uint4*)(v + ((b * dm.Lkv + tok) * dm.H + hk) * DV + ks * 32 + j * 8);
   const bool masked_col = dm.mask_last && wave == 3 && col == 15;  // token 63 of the chunk
+  // distance penalty of this lane's token for its four accumulator rows (16 % G == 0: the head of
+  // row 4j + i is the same in every 16-row tile)
+  float pen[4] = {0.f, 0.f, 0.f, 0.f};
+  if (dm.slope) {
+    const int dist = BW_S - 2 - (wave * 16 + col);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pen[i] = dm.slope[hk * G + (4 * j + i) % G] * (float)(dist > 0 ? dist : 0);
+  }
 
   f32x4_t acc_k[DT], acc_v[VT];
 #pragma unroll
@@ -318,7 +327,7 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int r = sb * 16 + 4 * j + i;
-            float pv = __builtin_amdgcn_exp2f(s[i] * c2 - row_lse[r]);
+            float pv = __builtin_amdgcn_exp2f((s[i] - pen[i]) * c2 - row_lse[r]);
             if (masked_col) pv = 0.f;
             pw[i] = row_w[r] * pv;
             ds[i] = pw[i] * (dp[i] - row_delta[r]);
@@ -400,6 +409,7 @@ bw_dkdv_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const
 struct BqDims {
   int L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last;
   float sm_scale;
+  const float* slope;  // as in BwDims
 };
 
 // STAGE: the block's own query and dO rows are copied into LDS once (coalesced) and every tile
@@ -545,6 +555,7 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
   const float out_scale = dm.sm_scale * fx_scale;
   const int qs = r / G, g = r - qs * G;  // this lane's row of a tile: query slot, head
   const int hq = hk * G + g;
+  const float sl = dm.slope ? dm.slope[hq] : 0.f;
   const int npair_valid = cur[dm.nchunk - 1];
 
   for (;;) {
@@ -651,6 +662,15 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
 #pragma unroll
         for (int u = 0; u < 2 * DT; ++u) xa[u] = *(const bw_u4*)(kt_c + u * 512);
       }
+      if (dm.slope) {
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int dist = BW_S - 2 - (mt * 16 + j * 4 + i);
+            st[mt][i] -= sl * (float)(dist > 0 ? dist : 0);
+          }
+      }
       // ---- P, delta, dS (this lane: row r of the tile, tokens mt*16 + 4j + i)
       float delta = 0.f;
 #pragma unroll
@@ -738,7 +758,7 @@ bool hils_bw_covers(int L, int Lkv, int HQ, int H, int D, int Dv, int K, int S, 
   const int G = HQ / H;
   return S == BW_S && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) &&
          (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) && q_block == 1 && WH == HQ && sm_n >= 0.f &&
-         slope == nullptr && Lkv >= S && K <= 256 && L < (1 << 24) && Lkv / S <= 12288;
+         Lkv >= S && K <= 256 && L < (1 << 24) && Lkv / S <= 12288;
 }
 
 void hils_ga_pack_launch(const void* a, const void* b, void* ap, void* bp, float* bmax, int B, int Lkv,
@@ -881,8 +901,8 @@ void hils_build_chunk_index(const int32_t* indices, int* counts, int* offsets, i
 // Whole backward on the MFMA kernels: dq (bf16, written), dw (fp32, written at the valid slots),
 // dk / dv (fp32, accumulated into the caller's buffers; or, with kv16, bf16 tensors that are overwritten).
 int hils_bw_run(const void* q, const void* k, const void* v, const void* weights, const int32_t* indices,
-                const float* lse, const void* d_o, void* dq, void* dk, void* dv, float* dw,
-                void* workspace, int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
+                const float* slope, const float* lse, const void* d_o, void* dq, void* dk, void* dv,
+                float* dw, void* workspace, int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
                 float sm_scale, int mask_last, int kv16, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   const int nchunk = Lkv / BW_S;
@@ -917,7 +937,7 @@ int hils_bw_run(const void* q, const void* k, const void* v, const void* weights
     const int nblk = (L + T - 1) / T;
     const long total = (long)nblk * H * B;
     if (total > (1L << 30)) return -1;
-    BqDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale};
+    BqDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale, slope};
     dim3 grid((unsigned)(((total + 7) / 8) * 8));
     int rc = -1;
 #define BQ_D(D_, DV_)                                                                                 \
@@ -932,7 +952,7 @@ int hils_bw_run(const void* q, const void* k, const void* v, const void* weights
   }
   // ---- inverse index, then dK, dV
   hils_build_chunk_index(indices, counts, offsets, cursor, pairs, B, L, H, K, nchunk, stream);
-  BwDims dm{L, Lkv, HQ, H, K, NW, nchunk, mask_last, sm_scale, kv16, B};
+  BwDims dm{L, Lkv, HQ, H, K, NW, nchunk, mask_last, sm_scale, kv16, B, slope};
   if (kv16 && Lkv > nchunk * BW_S) {  // tokens behind the last whole chunk are never attended
     for (int b2 = 0; b2 < B; ++b2) {
       const long nk = (long)(Lkv - nchunk * BW_S) * H * D / 2, nv = (long)(Lkv - nchunk * BW_S) * H * Dv / 2;

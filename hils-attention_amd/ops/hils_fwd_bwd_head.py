@@ -89,9 +89,7 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
         do = do.to(q.dtype).contiguous()
         dq = torch.empty_like(q)
         dw = torch.zeros((B, L, HQ, NW), dtype=torch.float32, device=q.device)
-        ws = None
-        if slope_dev is None:
-            ws = _cabi.sparse_attn_bwd_workspace(q.device, B, L, L_kv, HQ, H, D, Dv, K, HQ, 1, S, 0.0)
+        ws = _cabi.sparse_attn_bwd_workspace(q.device, B, L, L_kv, HQ, H, D, Dv, K, HQ, 1, S, 0.0)
         # the workspace kernels write dk / dv once, as bf16; the shape-generic one adds into fp32
         kv16 = ws is not None and k.dtype == torch.bfloat16 and v.dtype == torch.bfloat16
         if kv16:

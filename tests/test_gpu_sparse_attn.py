@@ -165,6 +165,10 @@ def test_sparse_attn_bwd_options(pkg, orc, dev):
     note("sparse_attn_bwd options")
     run_bwd(pkg, orc, dev, 1, 256, 4, 2, 64, 64, 4, 64, seed=8, mask_last_token=False)
     run_bwd(pkg, orc, dev, 1, 256, 4, 2, 64, 64, 4, 64, seed=9, slope=torch.rand(4) * 0.1, sm_scale=0.2)
+    # slope on the MFMA backward with grouped 128-wide heads and with ungrouped 64-wide ones (rows staged in LDS)
+    run_bwd(pkg, orc, dev, 1, 384, 8, 2, 128, 128, 4, 64, seed=12, slope=torch.rand(8) * 0.2)
+    run_bwd(pkg, orc, dev, 2, 320, 4, 4, 64, 64, 4, 64, seed=13, slope=torch.rand(4) * 0.2)
+    run_bwd(pkg, orc, dev, 1, 200, 4, 2, 32, 32, 4, 16, seed=14, slope=torch.rand(4) * 0.2)  # shape-generic kernel
 
 
 def test_sparse_attn_per_chunk_lse(pkg, orc, dev):
