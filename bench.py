@@ -345,6 +345,18 @@ def bench_ops(pkg, dev, iters=3):
     out["attn_pool_fwd_bwd"] = {"workload": "B1 N512 S64 H32 D128 (includes the torch glue of the loss)",
                                 "us": timed(pool_fb) * 1e3}
     del kc, kc_g, mu, mu_g
+    # key preparation in one pass (RMS norm + rotary embedding + chunk mean) on the 32K prefill's K
+    Lp, Hk = 32768, 8
+    kx = gpu_randn((1, Lp, Hk, D), gen, dev)
+    nw = (torch.rand(D, device=dev, generator=gen) + 0.5).bfloat16()
+    ang = torch.rand(Lp, D // 2, device=dev, generator=gen) * 6.0
+    cos_t = torch.cat([ang.cos(), ang.cos()], -1).bfloat16()
+    sin_t = torch.cat([ang.sin(), ang.sin()], -1).bfloat16()
+    with torch.no_grad():
+        t = timed(lambda: pkg.norm_rope_pool(kx, nw, cos_t, sin_t, 64), 10)
+    out["norm_rope_pool_fwd"] = {"workload": "K of the 32K prefill: B1 L32768 H8 D128 chunk64", "us": t * 1e3,
+                                 "hbm_gbs": (2 * kx.numel() + 2 * cos_t.numel()) * 2 / (t * 1e-3) / 1e9}
+    del kx, nw, ang, cos_t, sin_t
     # exact chunk log-Z: B1 L8192 hq32/hkv8 D128, window 64
     L, HQ, HK = 8192, 32, 8
     q = gpu_randn((1, L, HQ, D), gen, dev)

@@ -16,3 +16,4 @@ from .ops.flex_attn_tilelang import flex_attn_tl, flex_attn_tl_two_phase  # noqa
 from .ops.hils_fwd_bwd_head import prepare_kv_workspace  # noqa: F401
 from .utils.hils_cache_utils import HiLSDynamicLayer, HiLSPagedLayer, paged_hils_attend  # noqa: F401
 from .ops.rope_tilelang_fp32 import rope_rotary_pos_emb, single_tensor_rope_autograd  # noqa: F401
+from .ops.norm_rope_pool import norm_rope_pool  # noqa: F401

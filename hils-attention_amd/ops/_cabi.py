@@ -37,6 +37,8 @@ SIGNATURES = {
     "hils_chunk_logz_bwd_dq": [_P] * 5 + [_I] * 7 + [_F, _P],
     "hils_chunk_logz_bwd_dk": [_P] * 5 + [_I] * 7 + [_F, _P],
     "hils_rope": [_P] * 4 + [_I] * 7 + [_F, _P],
+    "hils_norm_rope_pool_fwd": [_P] * 6 + [_I] * 6 + [_F, _P],
+    "hils_norm_rope_pool_bwd": [_P] * 8 + [_I] * 6 + [_F, _P],
     "hils_swa_fwd": [_P] * 5 + [_I] * 12 + [_F, _P],
     "hils_swa_bwd": [_P] * 11 + [_I] * 10 + [_F, _P],
 }

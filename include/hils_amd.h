@@ -284,6 +284,25 @@ int hils_swa_bwd(const void* q, const void* k, const void* v, const void* o, con
 int hils_rope(const void* x, const void* cos_t, const void* sin_t, void* out, int B, int L, int H,
               int D, int table_per_batch, int table_f32, int lo_only, float sin_sign, void* stream);
 
+/* Key (or query) preparation in one pass: per-head RMS norm, rotary embedding and the mean over
+ * every chunk.  Replaces the layer's sequence k_norm (models/FlashHiLS/hils_attention.py:314-321 with
+ * rms_norm of models/FlashHiLS/modeling_qwen_hils.py:80-86), apply_rotary_pos_emb
+ * (hils_attention.py:144-171, called at :479-483) and k_chunked.mean(dim=2) (:398,:460), which
+ * otherwise read and write the tensor once per step.
+ * x, out (B,L,H,D) bf16, D in {64,128,256}; norm_weight (D) bf16 or NULL (no norm); cos_t, sin_t
+ * (L,D) bf16 - (B,L,D) when table_per_batch != 0 - or both NULL (no rotation):
+ *   y = bf16(x * rsqrt(mean_d x^2 + eps)); z = bf16(norm_weight * y);
+ *   out = bf16(bf16(z*cos) + bf16(rotate_half(z)*sin)), rotate_half(z) = (-z_hi, z_lo);
+ *   lmk[b,n,h,:] = bf16(mean_s out[b,nS+s,h,:]) for the L/S whole chunks; lmk (B,L/S,H,D) bf16 or NULL.
+ * Backward: d_out (B,L,H,D) bf16 and/or d_lmk (B,L/S,H,D) bf16 -> dx bf16 (written), d_weight (D) fp32
+ * (ADDED to with float atomics: caller zero-fills; required when norm_weight is given). */
+int hils_norm_rope_pool_fwd(const void* x, const void* norm_weight, const void* cos_t, const void* sin_t,
+                            void* out, void* lmk, int B, int L, int H, int D, int S, int table_per_batch,
+                            float eps, void* stream);
+int hils_norm_rope_pool_bwd(const void* x, const void* norm_weight, const void* cos_t, const void* sin_t,
+                            const void* d_out, const void* d_lmk, void* dx, float* d_weight, int B, int L,
+                            int H, int D, int S, int table_per_batch, float eps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

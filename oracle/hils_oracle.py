@@ -26,6 +26,11 @@ reference repository root):
                              mask of ops/exact_chunk_log_z_tilelang.py:89-107
 * ``rope``                 - ops/rope_tilelang_fp32.py:48-62,125-134 (kernel arithmetic) and
                              :185-189 (the rotate-half torch formula its tests compare with)
+* ``rms_norm`` / ``rope_hf`` / ``norm_rope_pool``
+                           - models/FlashHiLS/modeling_qwen_hils.py:80-86 (rms_norm),
+                             models/FlashHiLS/hils_attention.py:137-171 (rotate_half,
+                             apply_rotary_pos_emb on tensors of the model dtype) and :314-321,
+                             :479-483, :398 (the order norm -> rotation -> chunk mean)
 * ``swa``                  - ops/flex_attn_tilelang.py:1355-1386 (mask definition) and
                              :108-121,155-171 (absolute positions with a cache offset)
 * ``hils_layer_forward``   - models/FlashHiLS/hils_attention.py:536-623 (op order,
@@ -336,6 +341,38 @@ def rope(x, cos, sin, *, lo_only: bool = False):
     c1, s1 = cos[..., :half], sin[..., :half]
     c2, s2 = (c1, s1) if lo_only else (cos[..., half:], sin[..., half:])
     return torch.cat([x1 * c1 - x2 * s1, x2 * c2 + x1 * s2], dim=-1)
+
+
+def rms_norm(x, weight, eps: float = 1e-6):
+    """models/FlashHiLS/modeling_qwen_hils.py:80-86: statistics in fp32, the normalised value cast
+    back to the input dtype, then multiplied by the weight (in that dtype)."""
+    x32 = x.to(torch.float32)
+    var = x32.pow(2).mean(-1, keepdim=True)
+    return weight * (x32 * torch.rsqrt(var + eps)).to(x.dtype)
+
+
+def rope_hf(x, cos, sin):
+    """models/FlashHiLS/hils_attention.py:137-171 for one tensor in (B,L,H,D) layout: x*cos +
+    rotate_half(x)*sin, rotate_half(x) = (-x_hi, x_lo), every operation in x's dtype."""
+    if cos.dim() == 2:
+        cos, sin = cos.unsqueeze(0), sin.unsqueeze(0)
+    cos, sin = cos.unsqueeze(2).to(x.dtype), sin.unsqueeze(2).to(x.dtype)
+    half = x.shape[-1] // 2
+    rot = torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+    return (x * cos) + (rot * sin)
+
+
+def norm_rope_pool(x, weight, cos, sin, chunk_size: int, eps: float = 1e-6):
+    """The layer's key preparation (hils_attention.py:314-321, :479-483, :398): optional per-head RMS
+    norm, optional rotation, mean over every whole chunk.  Runs in x's dtype (pass bf16 for the
+    layer's roundings, fp32 or fp64 for the exact function).  Returns (out, lmk)."""
+    out = x if weight is None else rms_norm(x, weight.to(x.dtype), eps)
+    if cos is not None:
+        out = rope_hf(out, cos, sin)
+    B, L, H, D = out.shape
+    N = L // chunk_size
+    lmk = out[:, :N * chunk_size].reshape(B, N, chunk_size, H, D).mean(dim=2)
+    return out, lmk
 
 
 # ----------------------------------------------------------------------------

@@ -67,3 +67,59 @@ def test_rope_argument_errors(pkg, dev):
         y = torch.randn(1, 8, 2, 40, device=dev).bfloat16()
         t = torch.randn(8, 40, device=dev).bfloat16()
         pkg.single_tensor_rope_autograd(y, t, t)
+
+
+@pytest.mark.parametrize("B,L,H,D,S,norm,rot,per_batch", [(1, 512, 4, 128, 64, True, True, False),
+                                                          (2, 200, 3, 64, 64, True, True, True),    # ragged tail chunk
+                                                          (1, 256, 2, 256, 32, True, False, False),  # norm only, 32-token chunks
+                                                          (2, 192, 8, 128, 64, False, True, False),  # rotation only
+                                                          (1, 128, 2, 64, 64, False, False, False)])  # plain chunk mean
+def test_norm_rope_pool(pkg, orc, dev, B, L, H, D, S, norm, rot, per_batch):
+    """One pass for the layer's key preparation: against the oracle run in bf16 (the layer's own
+    roundings: nearly every element identical, none further than two bf16 steps) and in fp64 (the
+    exact function), forward and backward."""
+    note(f"norm_rope_pool B{B} L{L} H{H} D{D} S{S} norm={norm} rot={rot}")
+    torch.manual_seed(41)
+    x = (torch.randn(B, L, H, D) * 1.5).bfloat16()
+    w = (torch.rand(D) + 0.5).bfloat16() if norm else None
+    cos = sin = None
+    if rot:
+        ang = torch.rand(B if per_batch else 1, L, D // 2) * 6.0
+        cos = torch.cat([ang.cos(), ang.cos()], -1).bfloat16()
+        sin = torch.cat([ang.sin(), ang.sin()], -1).bfloat16()
+        if not per_batch:
+            cos, sin = cos[0], sin[0]
+    xd = x.to(dev).requires_grad_()
+    wd = w.to(dev).requires_grad_() if norm else None
+    out, lmk = pkg.norm_rope_pool(xd, wd, None if cos is None else cos.to(dev), None if sin is None else sin.to(dev), S)
+    ref_o, ref_l = orc.norm_rope_pool(x, w, cos, sin, S)  # bf16 arithmetic, op by op
+    got_o, got_l = out.detach().cpu(), lmk.detach().cpu()
+    same = (got_o == ref_o).float().mean().item()
+    step = (got_o.float() - ref_o.float()).abs() / ref_o.float().abs().clamp_min(1e-3)
+    note(f"    out: {same * 100:.3f} % of the elements bit-identical, worst relative difference {step.max().item():.2e}")
+    # (a last-bit difference of the fp32 reciprocal square root can move the first rounding by one
+    # bf16 step, and a later rounding by one more)
+    assert same >= 0.995 and step.max().item() <= 2 ** -6
+    assert_close_bf16(got_l, ref_l.float(), "pooled keys vs bf16 oracle")
+    x64 = x.double().requires_grad_()
+    w64 = w.double().requires_grad_() if norm else None
+    o64, l64 = orc.norm_rope_pool(x64, w64, None if cos is None else cos.double(), None if sin is None else sin.double(), S)
+    assert_close_bf16(got_o, o64.detach().float(), "out vs fp64 oracle")
+    assert_close_bf16(got_l, l64.detach().float(), "pooled keys vs fp64 oracle")
+    g_o = torch.randn(B, L, H, D).bfloat16()
+    g_l = torch.randn(B, L // S, H, D).bfloat16()
+    (out.float() * g_o.to(dev).float()).sum().backward(retain_graph=True)
+    dx_o = xd.grad.clone(); xd.grad = None
+    (o64 * g_o.double()).sum().backward(retain_graph=True)
+    assert_close_bf16(dx_o.cpu(), x64.grad.float(), "dx from d_out alone"); x64.grad = None
+    if norm:
+        wd.grad = None; w64.grad = None
+    ((out.float() * g_o.to(dev).float()).sum() + (lmk.float() * g_l.to(dev).float()).sum()).backward()
+    ((o64 * g_o.double()).sum() + (l64 * g_l.double()).sum()).backward()
+    assert_close_bf16(xd.grad.cpu(), x64.grad.float(), "dx")
+    if norm:
+        assert_close_bf16(wd.grad.cpu(), w64.grad.float(), "d_weight")
+    # the query side: no pooled output
+    o_q, none = pkg.norm_rope_pool(x.to(dev), w.to(dev) if norm else None, None if cos is None else cos.to(dev),
+                                   None if sin is None else sin.to(dev), S, pool=False)
+    assert none is None and torch.equal(o_q.cpu(), got_o)

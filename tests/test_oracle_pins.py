@@ -488,3 +488,32 @@ def test_rope_is_a_rotation(orc):
     t, h, d = 3, 1, 2
     assert o2[1, t, h, d].item() == pytest.approx((x[1, t, h, d] * c[t, d] - x[1, t, h, d + 4] * s_[t, d]).item(), abs=1e-6)
     assert o2[1, t, h, d + 4].item() == pytest.approx((x[1, t, h, d + 4] * c[t, d + 4] + x[1, t, h, d] * s_[t, d + 4]).item(), abs=1e-6)
+
+
+def test_norm_rope_pool_pieces(orc):
+    """rms_norm against torch's own F.rms_norm and the unit-RMS property; rope_hf against complex
+    multiplication by e^{i angle} (the two halves are real and imaginary parts) and against the fp32
+    kernel formula of ``rope``; the pooled keys against a python loop."""
+    torch.manual_seed(31)
+    B, L, H, D, S = 2, 70, 3, 16, 8
+    x = torch.randn(B, L, H, D, dtype=torch.float64)
+    w = torch.rand(D, dtype=torch.float64) + 0.5
+    y = orc.rms_norm(x, w, 1e-6)
+    assert torch.allclose(y, torch.nn.functional.rms_norm(x, (D,), w, 1e-6), atol=1e-12)
+    assert torch.allclose((y / w).pow(2).mean(-1), torch.ones(B, L, H, dtype=torch.float64), atol=1e-5)
+    ang = torch.rand(L, D // 2, dtype=torch.float64) * 6.0
+    cos, sin = torch.cat([ang.cos(), ang.cos()], -1), torch.cat([ang.sin(), ang.sin()], -1)
+    r = orc.rope_hf(x, cos, sin)
+    z = torch.complex(x[..., :D // 2], x[..., D // 2:]) * torch.polar(torch.ones_like(ang), ang).view(1, L, 1, D // 2)
+    assert torch.allclose(r, torch.cat([z.real, z.imag], -1), atol=1e-12)
+    assert torch.allclose(r.float(), orc.rope(x.float(), cos.float(), sin.float()), atol=1e-5)
+    out, lmk = orc.norm_rope_pool(x, w, cos, sin, S, 1e-6)
+    assert torch.allclose(out, orc.rope_hf(orc.rms_norm(x, w, 1e-6), cos, sin), atol=0)
+    assert lmk.shape == (B, L // S, H, D)
+    for b in range(B):
+        for n in range(L // S):
+            want = sum(out[b, n * S + s_] for s_ in range(S)) / S
+            assert torch.allclose(lmk[b, n], want, atol=1e-12)
+    # without norm and rotation it is the plain chunk mean
+    out2, lmk2 = orc.norm_rope_pool(x, None, None, None, S)
+    assert out2 is x and torch.allclose(lmk2, orc.mean_pool(x, S).to(torch.float64), atol=1e-6)
