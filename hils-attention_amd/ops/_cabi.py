@@ -87,6 +87,17 @@ def ptr(t):
     return c_void_p(t.data_ptr())
 
 
+def gpu_readable(t, device):
+    """A contiguous tensor the kernels can read: ``t`` itself when it is contiguous in device memory
+    or in pinned host memory; otherwise a contiguous copy in device memory (a copy of a pinned
+    tensor made on the host would land in pageable memory, which the GPU cannot address)."""
+    if t.is_contiguous() and (t.is_cuda or t.is_pinned()):
+        return t
+    if t.is_cuda:
+        return t.contiguous()
+    return t.to(device, non_blocking=True).contiguous()
+
+
 def stream():
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -137,11 +148,13 @@ def sparse_attn_bwd_workspace(device, B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S
     return torch.empty(n, dtype=torch.uint8, device=device)
 
 
-def require_gpu_bf16(name, *tensors):
+def require_gpu_bf16(name, *tensors, pinned_ok=False):
+    """Every tensor is bf16 and readable by the GPU: in device memory or, with ``pinned_ok`` (an
+    offloaded KV cache), in pinned host memory, which the kernels read in place over the host link."""
     for t in tensors:
         if t is None:
             continue
-        if not t.is_cuda:
+        if not (t.is_cuda or (pinned_ok and t.is_pinned())):
             raise RuntimeError(f"{name}: tensors must live on the GPU (got {t.device}); "
                                "this package has no CPU path")
         if t.dtype != torch.bfloat16:

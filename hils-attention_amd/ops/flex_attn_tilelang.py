@@ -15,7 +15,8 @@ class _FlexAttnTL(torch.autograd.Function):
     def forward(ctx, q, k, v, window_size, chunk_size, mask_lmk, expand_to_chunk, use_cache, sm_scale,
                 kv_start):
         assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4
-        _cabi.require_gpu_bf16("flex_attn_tl", q, k, v)
+        _cabi.require_gpu_bf16("flex_attn_tl", q)
+        _cabi.require_gpu_bf16("flex_attn_tl", k, v, pinned_ok=bool(use_cache))  # an offloaded cache is read in place
         B, Lq, HQ, D = q.shape
         Lk, H = k.shape[1], k.shape[2]
         Dv = v.shape[-1]
@@ -27,7 +28,7 @@ class _FlexAttnTL(torch.autograd.Function):
         assert Lq <= Lk, f"Lq ({Lq}) must not exceed Lk ({Lk})"
         if sm_scale is None:
             sm_scale = 1.0 / math.sqrt(D)
-        q_c, k_c, v_c = q.contiguous(), k.contiguous(), v.contiguous()
+        q_c, k_c, v_c = q.contiguous(), _cabi.gpu_readable(k, q.device), _cabi.gpu_readable(v, q.device)
         o = torch.empty((B, Lq, HQ, Dv), dtype=q.dtype, device=q.device)
         lse = torch.empty((B, Lq, HQ), dtype=torch.float32, device=q.device)
         _cabi.call("hils_swa_fwd", _cabi.ptr(q_c), _cabi.ptr(k_c), _cabi.ptr(v_c), _cabi.ptr(o),

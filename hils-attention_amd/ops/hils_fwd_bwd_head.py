@@ -25,7 +25,9 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
                 is_training, slope=None, kv_workspace=None, swa_o=None, swa_weight_index=None):
         assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
         assert weights.is_contiguous() and indices.is_contiguous()
-        _cabi.require_gpu_bf16("HiLS_block_M_head", q, k, v)
+        _cabi.require_gpu_bf16("HiLS_block_M_head", q)
+        # inference may read K and V of an offloaded cache in place (pinned host memory)
+        _cabi.require_gpu_bf16("HiLS_block_M_head", k, v, pinned_ok=not is_training)
         B, L, HQ, D = q.shape
         L_kv, H, Dk = k.shape[1], k.shape[2], k.shape[-1]
         Dv = v.shape[-1]

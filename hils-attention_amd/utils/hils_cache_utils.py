@@ -6,7 +6,14 @@ re-concatenates K and V on every step, and the pooled chunk keys in ``_hils_prio
 tensors are allocated once at a capacity and written in place: the selection only looks at chunks
 the causal limit makes visible (``q_offset``), so the kernels can be handed the whole buffers and
 no tensor is copied or re-laid-out per step.  Mean-pooled chunk keys only (the layer's
-``enable_chunk_pooling`` mode)."""
+``enable_chunk_pooling`` mode).
+
+Offload.  Past the reference's thresholds (hidden size >= 4096 and more than 128K tokens,
+utils/hils_cache_utils.py:4-5,19-23) the reference moves K and V to pinned host memory and copies the
+whole cache back to the GPU on every update (:44-60).  Here K and V then LIVE in pinned host memory
+and are read in place: a decode step touches only the pooled chunk keys (which stay on the GPU), the
+top-k selected chunks and the local window, so the kernels fetch exactly those rows over the host
+link instead of the whole cache.  ``update`` then returns pinned host views."""
 import math
 
 import torch
@@ -23,18 +30,46 @@ except ImportError:  # ... or with the package directory itself on sys.path (`fr
     from ops.hils_glue import topk_chunk_weights
 
 
+_OFFLOAD_SEQ_THRESHOLD = 128 * 1024
+_OFFLOAD_HIDDEN_DIM_THRESHOLD = 4096
+
+
 class HiLSDynamicLayer:
-    """update() / get_seq_length() as in the reference's class; the buffers grow by doubling."""
+    """update() / get_seq_length() as in the reference's class; the buffers grow by doubling.
+    ``offload``: None = by the reference's thresholds, True / False = forced."""
 
     is_sliding = False
 
-    def __init__(self, chunk_size=64, capacity=0):
+    def __init__(self, chunk_size=64, capacity=0, offload=None):
         self.chunk_size = int(chunk_size)
         self.capacity = int(capacity)
         self.seq_len = 0
         self.pooled_chunks = 0  # chunks whose mean-pooled key is in lmk_k
         self.keys = self.values = self.lmk_k = None
         self.is_initialized = False
+        self._offload_choice = offload
+        self._offloading = False
+        self._hidden_dim = 0
+
+    def _should_offload(self, new_seq_len):
+        if self._offload_choice is not None:
+            return bool(self._offload_choice)
+        return self._hidden_dim >= _OFFLOAD_HIDDEN_DIM_THRESHOLD and new_seq_len > _OFFLOAD_SEQ_THRESHOLD
+
+    def _kv_buffer(self, shape):
+        """K / V storage: device memory, or pinned host memory once the layer offloads."""
+        if self._offloading:
+            return torch.zeros(shape, dtype=self.dtype, device="cpu", pin_memory=True)
+        return torch.zeros(shape, dtype=self.dtype, device=self.device)
+
+    def _move_to_host(self):
+        self._offloading = True
+        for name in ("keys", "values"):
+            old = getattr(self, name)
+            new = self._kv_buffer(tuple(old.shape))
+            new[:, : self.seq_len].copy_(old[:, : self.seq_len], non_blocking=True)
+            setattr(self, name, new)
+        torch.cuda.current_stream().synchronize()
 
     def lazy_initialization(self, key_states, value_states):
         B, T, H, D = key_states.shape
@@ -43,8 +78,10 @@ class HiLSDynamicLayer:
         cap = (cap + S - 1) // S * S
         self.capacity = cap
         self.dtype, self.device = key_states.dtype, key_states.device
-        self.keys = torch.empty((B, cap, H, D), dtype=self.dtype, device=self.device)
-        self.values = torch.empty((B, cap, H, value_states.shape[-1]), dtype=self.dtype, device=self.device)
+        self._hidden_dim = H * D
+        self._offloading = self._should_offload(T)
+        self.keys = self._kv_buffer((B, cap, H, D))
+        self.values = self._kv_buffer((B, cap, H, value_states.shape[-1]))
         self.lmk_k = torch.zeros((B, cap // S, H, D), dtype=self.dtype, device=self.device)
         self.is_initialized = True
 
@@ -56,8 +93,10 @@ class HiLSDynamicLayer:
         cap = (cap + S - 1) // S * S
         for name in ("keys", "values", "lmk_k"):
             old = getattr(self, name)
-            rows = cap // S if name == "lmk_k" else cap
-            new = torch.zeros((old.shape[0], rows) + tuple(old.shape[2:]), dtype=old.dtype, device=old.device)
+            if name == "lmk_k":
+                new = torch.zeros((old.shape[0], cap // S) + tuple(old.shape[2:]), dtype=old.dtype, device=old.device)
+            else:
+                new = self._kv_buffer((old.shape[0], cap) + tuple(old.shape[2:]))
             new[:, : old.shape[1]] = old
             setattr(self, name, new)
         self.capacity = cap
@@ -68,17 +107,24 @@ class HiLSDynamicLayer:
         if not self.is_initialized:
             self.lazy_initialization(key_states, value_states)
         T = key_states.shape[1]
+        if not self._offloading and self._should_offload(self.seq_len + T):
+            self._move_to_host()
         if self.seq_len + T > self.capacity:
             self._grow(self.seq_len + T)
         a, b = self.seq_len, self.seq_len + T
-        self.keys[:, a:b] = key_states
-        self.values[:, a:b] = value_states
+        self.keys[:, a:b].copy_(key_states, non_blocking=True)
+        self.values[:, a:b].copy_(value_states, non_blocking=True)
+        if self._offloading:  # the host copies are complete before anything reads the buffers
+            torch.cuda.current_stream().synchronize()
         self.seq_len = b
         S = self.chunk_size
         full = b // S
         if full > self.pooled_chunks:
             c0 = self.pooled_chunks
-            self.lmk_k[:, c0:full] = chunk_mean_pool(self.keys[:, c0 * S: full * S].contiguous(), S)
+            src = self.keys[:, c0 * S: full * S]
+            if self._offloading:  # the tokens of the chunks just completed: a small copy back
+                src = src.to(self.device, non_blocking=True)
+            self.lmk_k[:, c0:full] = chunk_mean_pool(src.contiguous(), S)
             self.pooled_chunks = full
         return self.keys[:, :b], self.values[:, :b]
 
