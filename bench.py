@@ -31,7 +31,7 @@ def measured_traffic(key):
     """HBM bytes per launch of a kernel as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE.
     The figures live in the committed counter summary, on lines `bench.traffic <key> <bytes>`;
     None when the summary (or the key) is absent."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic_fetch_write_size.md")
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_per_launch.txt")
     try:
         with open(path) as fh:
             for line in fh:
@@ -476,6 +476,8 @@ def main():
     ap.add_argument("--no-train", action="store_true", help="skip the config-5 forward+backward timing")
     ap.add_argument("--no-ops", action="store_true", help="skip the timings of the secondary operators")
     ap.add_argument("--no-prefill", action="store_true", help="profiling aid: decode step only")
+    ap.add_argument("--train-only", action="store_true",
+                    help="profiling aid: only the config-5 training layer forward+backward")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: run only a 512 MiB device copy (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters)")
@@ -496,6 +498,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes": int(src.numel())}))
+        return
+    if args.train_only:
+        print(json.dumps({"train_fwd_bwd": bench_train(pkg, dev)}))
         return
     if args.no_prefill:
         dsec, dper, droof = bench_decode(pkg, dev, max(args.steps, 20), args.warmup)
