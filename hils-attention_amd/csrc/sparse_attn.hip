@@ -34,19 +34,31 @@ struct SaDims {
   int skip_dkdv;  // backward: dK and dV come from the chunk-major kernel
 };
 
+// element access of the shape-generic kernels: bf16 tensors, or fp32 tensors (the fp32 mode)
+__device__ __forceinline__ float sa_ld(const bf16_t* p) { return bf2f(*p); }
+__device__ __forceinline__ float sa_ld(const float* p) { return *p; }
+__device__ __forceinline__ void sa_ld8(const bf16_t* p, float* f) { unpack8(*(const uint4*)p, f); }
+__device__ __forceinline__ void sa_ld8(const float* p, float* f) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+__device__ __forceinline__ void sa_st(bf16_t* p, float x) { *p = f2bf(x); }
+__device__ __forceinline__ void sa_st(float* p, float x) { *p = x; }
+
 // scores of slot chunk c for all (g, s): sc[g*S+s] = (q_g . K_s - slope_g*dist_s) * sm_scale,
 // -inf for the masked last token.  q_s holds the G query rows in fp32.
-__device__ __forceinline__ void sa_scores(const SaDims& dm, const float* q_s, const bf16_t* kbase,
+template <class T>
+__device__ __forceinline__ void sa_scores(const SaDims& dm, const float* q_s, const T* kbase,
                                           const float* slope_s, float* sc) {
   const int GS = dm.G * dm.S;
   for (int p = threadIdx.x; p < GS; p += SA_THREADS) {
     const int g = p / dm.S, s = p - g * dm.S;
-    const bf16_t* kr = kbase + (long)s * dm.H * dm.D;
+    const T* kr = kbase + (long)s * dm.H * dm.D;
     const float* qr = q_s + g * dm.D;
     float a = 0.f;
     for (int d8 = 0; d8 < dm.D / 8; ++d8) {
       float f[8];
-      unpack8(*(const uint4*)(kr + d8 * 8), f);
+      sa_ld8(kr + d8 * 8, f);
 #pragma unroll
       for (int j = 0; j < 8; ++j) a = fmaf(qr[d8 * 8 + j], f[j], a);
     }
@@ -60,11 +72,12 @@ __device__ __forceinline__ void sa_scores(const SaDims& dm, const float* q_s, co
   }
 }
 
+template <class T>
 __global__ void __launch_bounds__(SA_THREADS)
-sparse_attn_fwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
-                       const bf16_t* __restrict__ v, const bf16_t* __restrict__ weights,
+sparse_attn_fwd_simple(const T* __restrict__ q, const T* __restrict__ k,
+                       const T* __restrict__ v, const T* __restrict__ weights,
                        const int32_t* __restrict__ indices, const float* __restrict__ slope,
-                       bf16_t* __restrict__ o, float* __restrict__ lse, SaDims dm) {
+                       T* __restrict__ o, float* __restrict__ lse, SaDims dm) {
   extern __shared__ float smem[];
   float* q_s = smem;                       // G*D
   float* sc = q_s + dm.G * dm.D;           // G*S
@@ -82,7 +95,7 @@ sparse_attn_fwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
   const int nchunk = dm.Lkv / S;
 
   for (int i = tid; i < G * D; i += SA_THREADS)
-    q_s[i] = bf2f(q[(bt * dm.HQ + hk * G) * (long)D + i]);
+    q_s[i] = sa_ld(q + (bt * dm.HQ + hk * G) * (long)D + i);
   if (tid < G) slope_s[tid] = slope ? slope[hk * G + tid] : 0.f;
 
   float acc[SA_MAX_OUT];
@@ -100,10 +113,10 @@ sparse_attn_fwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
     }
     if (tid < G) {
       const long wrow = (b * LB + t / dm.q_block) * dm.WH + (dm.WH == dm.HQ ? hk * G + tid : hk);
-      w_s[tid] = bf2f(weights[wrow * dm.NW + kk]);
+      w_s[tid] = sa_ld(weights + wrow * dm.NW + kk);
     }
-    const bf16_t* kbase = k + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * D;
-    const bf16_t* vbase = v + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * Dv;
+    const T* kbase = k + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * D;
+    const T* vbase = v + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * Dv;
     sa_scores(dm, q_s, kbase, slope ? slope_s : nullptr, sc);
     __syncthreads();
     for (int g = wave; g < G; g += SA_THREADS / 64) {
@@ -132,7 +145,7 @@ sparse_attn_fwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
       if (oi < nout) {
         const int g = oi / Dv, dv = oi - g * Dv;
         float a = acc[j];
-        for (int s = 0; s < S; ++s) a = fmaf(sc[g * S + s], bf2f(vbase[(long)s * dm.H * Dv + dv]), a);
+        for (int s = 0; s < S; ++s) a = fmaf(sc[g * S + s], sa_ld(vbase + (long)s * dm.H * Dv + dv), a);
         acc[j] = a;
       }
     }
@@ -140,16 +153,17 @@ sparse_attn_fwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
 #pragma unroll
   for (int j = 0; j < SA_MAX_OUT; ++j) {
     const int oi = tid + j * SA_THREADS;
-    if (oi < nout) o[(bt * dm.HQ + hk * G) * (long)Dv + oi] = f2bf(acc[j]);
+    if (oi < nout) sa_st(o + (bt * dm.HQ + hk * G) * (long)Dv + oi, acc[j]);
   }
 }
 
+template <class T>
 __global__ void __launch_bounds__(SA_THREADS)
-sparse_attn_bwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
-                       const bf16_t* __restrict__ v, const bf16_t* __restrict__ weights,
+sparse_attn_bwd_simple(const T* __restrict__ q, const T* __restrict__ k,
+                       const T* __restrict__ v, const T* __restrict__ weights,
                        const int32_t* __restrict__ indices, const float* __restrict__ slope,
-                       const float* __restrict__ lse, const bf16_t* __restrict__ d_o,
-                       bf16_t* __restrict__ dq, float* __restrict__ dk, float* __restrict__ dv,
+                       const float* __restrict__ lse, const T* __restrict__ d_o,
+                       T* __restrict__ dq, float* __restrict__ dk, float* __restrict__ dv,
                        float* __restrict__ dw, SaDims dm) {
   extern __shared__ float smem[];
   const int G = dm.G, S = dm.S, D = dm.D, Dv = dm.Dv;
@@ -171,8 +185,8 @@ sparse_attn_bwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
   const int nchunk = dm.Lkv / S;
   const bool dw_atomic = dm.q_block > 1 || dm.WH != dm.HQ;
 
-  for (int i = tid; i < G * D; i += SA_THREADS) q_s[i] = bf2f(q[(bt * dm.HQ + hk * G) * (long)D + i]);
-  for (int i = tid; i < G * Dv; i += SA_THREADS) do_s[i] = bf2f(d_o[(bt * dm.HQ + hk * G) * (long)Dv + i]);
+  for (int i = tid; i < G * D; i += SA_THREADS) q_s[i] = sa_ld(q + (bt * dm.HQ + hk * G) * (long)D + i);
+  for (int i = tid; i < G * Dv; i += SA_THREADS) do_s[i] = sa_ld(d_o + (bt * dm.HQ + hk * G) * (long)Dv + i);
   if (tid < G) slope_s[tid] = slope ? slope[hk * G + tid] : 0.f;
 
   float dq_acc[SA_MAX_OUT];
@@ -186,19 +200,19 @@ sparse_attn_bwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
     if (c < 0 || c >= nchunk) continue;
     if (tid < G) {
       const long wrow = (b * LB + t / dm.q_block) * dm.WH + (dm.WH == dm.HQ ? hk * G + tid : hk);
-      w_s[tid] = bf2f(weights[wrow * dm.NW + kk]);
+      w_s[tid] = sa_ld(weights + wrow * dm.NW + kk);
     }
-    const bf16_t* kbase = k + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * D;
-    const bf16_t* vbase = v + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * Dv;
+    const T* kbase = k + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * D;
+    const T* vbase = v + ((b * dm.Lkv + (long)c * S) * dm.H + hk) * Dv;
     sa_scores(dm, q_s, kbase, slope ? slope_s : nullptr, p_s);
     // dPV[g][s] = dO_g . V_s
     for (int p = tid; p < G * S; p += SA_THREADS) {
       const int g = p / S, s = p - g * S;
-      const bf16_t* vr = vbase + (long)s * dm.H * Dv;
+      const T* vr = vbase + (long)s * dm.H * Dv;
       float a = 0.f;
       for (int d8 = 0; d8 < Dv / 8; ++d8) {
         float f[8];
-        unpack8(*(const uint4*)(vr + d8 * 8), f);
+        sa_ld8(vr + d8 * 8, f);
 #pragma unroll
         for (int j = 0; j < 8; ++j) a = fmaf(do_s[g * Dv + d8 * 8 + j], f[j], a);
       }
@@ -249,7 +263,7 @@ sparse_attn_bwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
       if (oi < nq) {
         const int g = oi / D, d = oi - g * D;
         float a = dq_acc[j];
-        for (int s = 0; s < S; ++s) a = fmaf(ds_s[g * S + s], bf2f(kbase[(long)s * dm.H * D + d]), a);
+        for (int s = 0; s < S; ++s) a = fmaf(ds_s[g * S + s], sa_ld(kbase + (long)s * dm.H * D + d), a);
         dq_acc[j] = a;
       }
     }
@@ -257,7 +271,7 @@ sparse_attn_bwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ 
 #pragma unroll
   for (int j = 0; j < SA_MAX_OUT; ++j) {
     const int oi = tid + j * SA_THREADS;
-    if (oi < nq) dq[(bt * dm.HQ + hk * G) * (long)D + oi] = f2bf(dq_acc[j]);
+    if (oi < nq) sa_st(dq + (bt * dm.HQ + hk * G) * (long)D + oi, dq_acc[j]);
   }
 }
 
@@ -355,7 +369,7 @@ extern "C" int hils_sparse_attn_fwd(const void* q, const void* k, const void* v,
   SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n, 0};
   size_t smem = ((size_t)dm.G * D + (size_t)dm.G * S + 2 * dm.G) * sizeof(float);
   HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_fwd: G*(D+S) too large for LDS");
-  hipLaunchKernelGGL(sparse_attn_fwd_simple, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS),
+  hipLaunchKernelGGL(sparse_attn_fwd_simple<bf16_t>, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS),
                      smem, (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k,
                      (const bf16_t*)v, (const bf16_t*)weights, indices, slope, (bf16_t*)o, lse, dm);
   if (swa_o)
@@ -444,10 +458,48 @@ extern "C" int hils_sparse_attn_bwd(const void* q, const void* k, const void* v,
   SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n, 0};
   size_t smem = ((size_t)dm.G * (D + Dv) + 2 * (size_t)dm.G * S + 3 * dm.G) * sizeof(float);
   HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_bwd: G*(D+Dv+2S) too large for LDS");
-  hipLaunchKernelGGL(sparse_attn_bwd_simple, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS),
+  hipLaunchKernelGGL(sparse_attn_bwd_simple<bf16_t>, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS),
                      smem, (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k,
                      (const bf16_t*)v, (const bf16_t*)weights, indices, slope, lse,
                      (const bf16_t*)d_o, (bf16_t*)dq, (float*)dk, (float*)dv, dw, dm);
   HILS_CHECK_LAUNCH("hils_sparse_attn_bwd");
+  return HILS_OK;
+}
+
+
+// ---- fp32 tensors (the reference's dtype="float32" mode): the shape-generic kernels on fp32 q, k,
+// v, weights, d_o; fp32 o and dq; everything computed in fp32 (no bf16 rounding of P) ----
+extern "C" int hils_sparse_attn_fwd_f32(const float* q, const float* k, const float* v, const float* weights,
+                                        const int32_t* indices, const float* slope, float* o, float* lse,
+                                        int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
+                                        int WH, int q_block, int S, float sm_scale, int mask_last, float sm_n,
+                                        void* stream) {
+  HILS_REQUIRE(q && k && v && weights && indices && o, "hils_sparse_attn_fwd_f32: null pointer");
+  if (int rc = sa_check("hils_sparse_attn_fwd_f32", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
+  HILS_REQUIRE(Lkv >= S, "hils_sparse_attn_fwd_f32: Lkv (%d) is shorter than one chunk (%d)", Lkv, S);
+  SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n, 0};
+  const size_t smem = ((size_t)dm.G * D + (size_t)dm.G * S + 2 * dm.G) * sizeof(float);
+  HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_fwd_f32: G*(D+S) too large for LDS");
+  hipLaunchKernelGGL(sparse_attn_fwd_simple<float>, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS), smem,
+                     (hipStream_t)stream, q, k, v, weights, indices, slope, o, lse, dm);
+  HILS_CHECK_LAUNCH("hils_sparse_attn_fwd_f32");
+  return HILS_OK;
+}
+
+extern "C" int hils_sparse_attn_bwd_f32(const float* q, const float* k, const float* v, const float* weights,
+                                        const int32_t* indices, const float* slope, const float* lse,
+                                        const float* d_o, float* dq, float* dk, float* dv, float* dw, int B,
+                                        int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int WH,
+                                        int q_block, int S, float sm_scale, int mask_last, float sm_n,
+                                        void* stream) {
+  HILS_REQUIRE(q && k && v && weights && indices && lse && d_o && dq && dk && dv && dw,
+               "hils_sparse_attn_bwd_f32: null pointer");
+  if (int rc = sa_check("hils_sparse_attn_bwd_f32", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
+  SaDims dm{L, Lkv, HQ, H, HQ / H, D, Dv, K, NW, WH, q_block, S, mask_last, sm_scale, sm_n, 0};
+  const size_t smem = ((size_t)dm.G * (D + Dv) + 2 * (size_t)dm.G * S + 3 * dm.G) * sizeof(float);
+  HILS_REQUIRE(smem <= 64 * 1024, "hils_sparse_attn_bwd_f32: G*(D+Dv+2S) too large for LDS");
+  hipLaunchKernelGGL(sparse_attn_bwd_simple<float>, dim3((unsigned)((long)B * L * H)), dim3(SA_THREADS), smem,
+                     (hipStream_t)stream, q, k, v, weights, indices, slope, lse, d_o, dq, dk, dv, dw, dm);
+  HILS_CHECK_LAUNCH("hils_sparse_attn_bwd_f32");
   return HILS_OK;
 }

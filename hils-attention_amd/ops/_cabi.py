@@ -31,6 +31,8 @@ SIGNATURES = {
     "hils_sparse_attn_fwd": [_P] * 10 + [_I] * 13 + [_F, _I, _F, _I, _P],
     "hils_pack_kv_chunks": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
     "hils_sparse_attn_bwd": [_P] * 13 + [_I] * 12 + [_F, _I, _F, _P, _P, _I, _I, _P],
+    "hils_sparse_attn_fwd_f32": [_P] * 8 + [_I] * 12 + [_F, _I, _F, _P],
+    "hils_sparse_attn_bwd_f32": [_P] * 12 + [_I] * 12 + [_F, _I, _F, _P],
     "hils_chunk_weights": [_P, _P, _I, _P, _P, _P] + [_I] * 7 + [_P],
     "hils_chunk_weights_bwd": [_P, _P, _I] + [_P] * 6 + [_I] * 7 + [_P],
     "hils_chunk_logz_fwd": [_P, _P, _P] + [_I] * 7 + [_F, _I, _P],

@@ -108,6 +108,64 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
                 None, None, None, None, None, None, d_swa, None)
 
 
+class _hils_block_M_attention_f32(torch.autograd.Function):
+    """The dtype="float32" mode (ops/hils_fwd_bwd_head.py:928-964 with dtype="float32"): fp32 q, k, v,
+    weights; every product and the softmax in fp32 on the shape-generic kernels."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, weights, indices, block_size, sm_scale, mask_last_token, is_training, slope):
+        for name, t in (("q", q), ("k", k), ("v", v)):
+            if not t.is_cuda:
+                raise RuntimeError(f"HiLS_block_M_head: {name} must live on the GPU (got {t.device}); "
+                                   "this package has no CPU path")
+            if t.dtype != torch.float32:
+                raise TypeError(f"HiLS_block_M_head(dtype='float32'): {name} must be float32, got {t.dtype}")
+        assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+        B, L, HQ, D = q.shape
+        L_kv, H, Dv = k.shape[1], k.shape[2], v.shape[-1]
+        K, NW = indices.shape[-1], weights.shape[-1]
+        assert indices.shape == (B, L, H, K), f"indices shape {tuple(indices.shape)} != {(B, L, H, K)}"
+        assert weights.shape[:3] == (B, L, HQ) and NW >= K, (
+            f"weights shape {tuple(weights.shape)} must be ({B}, {L}, {HQ}, >= {K})")
+        if sm_scale is None:
+            sm_scale = 1.0 / math.sqrt(D)
+        slope_dev = None
+        if slope is not None:
+            assert slope.shape == (HQ,), f"slope must be 1-D with shape ({HQ},), got {tuple(slope.shape)}"
+            slope_dev = slope.to(dtype=torch.float32, device=q.device).contiguous()
+        w_in = weights.to(torch.float32).contiguous()
+        idx_in = indices.to(torch.int32).contiguous()
+        o = torch.empty((B, L, HQ, Dv), dtype=torch.float32, device=q.device)
+        lse = torch.empty((B, L, HQ, K), dtype=torch.float32, device=q.device) if is_training else None
+        _cabi.call("hils_sparse_attn_fwd_f32", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
+                   _cabi.ptr(idx_in), _cabi.ptr(slope_dev), _cabi.ptr(o), _cabi.ptr(lse), B, L, L_kv, HQ, H, D, Dv,
+                   K, NW, HQ, 1, int(block_size), float(sm_scale), int(bool(mask_last_token)), 0.0)
+        ctx.is_training = bool(is_training)
+        if is_training:
+            ctx.save_for_backward(q, k, v, w_in, idx_in, lse, slope_dev)
+            ctx.cfg = (B, L, L_kv, HQ, H, D, Dv, K, NW, int(block_size), float(sm_scale), int(bool(mask_last_token)))
+            ctx.w_dtype = weights.dtype
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        if not getattr(ctx, "is_training", True):
+            raise RuntimeError(
+                "[_hils_block_M_attention_inverse] forward ran with is_training=False: the "
+                "per-chunk LSE needed by the backward was not saved.")
+        q, k, v, w_in, idx_in, lse, slope_dev = ctx.saved_tensors
+        B, L, L_kv, HQ, H, D, Dv, K, NW, S, sm_scale, mask_last = ctx.cfg
+        do = do.to(torch.float32).contiguous()
+        dq = torch.empty_like(q)
+        dk, dv = torch.zeros_like(k), torch.zeros_like(v)
+        dw = torch.zeros((B, L, HQ, NW), dtype=torch.float32, device=q.device)
+        _cabi.call("hils_sparse_attn_bwd_f32", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
+                   _cabi.ptr(idx_in), _cabi.ptr(slope_dev), _cabi.ptr(lse), _cabi.ptr(do), _cabi.ptr(dq),
+                   _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), B, L, L_kv, HQ, H, D, Dv, K, NW, HQ, 1, S,
+                   sm_scale, mask_last, 0.0)
+        return dq, dk, dv, dw.to(ctx.w_dtype), None, None, None, None, None, None
+
+
 def HiLS_block_M_head(q, k, v, weights, indices, block_size=64, sm_scale=None, block_M=None,
                       mask_last_token=True, dtype="bfloat16", accum_dtype="float",
                       num_threads=None, num_threads_fwd=None, num_threads_bwd=None,
@@ -118,7 +176,9 @@ def HiLS_block_M_head(q, k, v, weights, indices, block_size=64, sm_scale=None, b
     first K columns are read); indices (B,L,H,K) int32, negative = empty slot.  Call
     signature of ops/hils_fwd_bwd_head.py:928-934; ``block_M`` and the ``num_threads*``
     tuning knobs are accepted and ignored (tile shapes are chosen by the HIP launcher),
-    ``dtype`` must be "bfloat16" and ``accum_dtype`` "float".  ``kv_workspace`` (not in the
+    ``dtype`` "bfloat16" (the MFMA kernels) or "float32" (fp32 tensors, everything computed in fp32 on
+    the shape-generic kernels: the mode the reference's fp32 correctness test runs in) and
+    ``accum_dtype`` "float".  ``kv_workspace`` (not in the
     reference) is an optional tensor from ``prepare_kv_workspace`` for the same ``v``: the
     MFMA-operand-ordered copies of K and V the prefill kernel reads, reusable across calls.
     ``swa_o`` (B,L,HQ,Dv), not in the reference either: the local branch's output; with it the
@@ -131,8 +191,15 @@ def HiLS_block_M_head(q, k, v, weights, indices, block_size=64, sm_scale=None, b
     _, L_kv, H, Dk = k.shape
     assert D == Dk, f"Q head_dim ({D}) must equal K head_dim ({Dk})"
     assert HQ % H == 0, f"HQ={HQ} must be divisible by H={H}"
-    if dtype not in ("bfloat16", torch.bfloat16) or accum_dtype not in ("float", "float32", torch.float32):
-        raise ValueError("HiLS_block_M_head: only dtype='bfloat16' with accum_dtype='float' is built")
+    if accum_dtype not in ("float", "float32", torch.float32):
+        raise ValueError("HiLS_block_M_head: only accum_dtype='float' is built")
+    if dtype in ("float32", "float", torch.float32):
+        if kv_workspace is not None or swa_o is not None:
+            raise ValueError("HiLS_block_M_head(dtype='float32'): kv_workspace and swa_o belong to the bf16 kernels")
+        return _hils_block_M_attention_f32.apply(q, k, v, weights, indices, block_size, sm_scale,
+                                                 mask_last_token, is_training, slope)
+    if dtype not in ("bfloat16", torch.bfloat16):
+        raise ValueError("HiLS_block_M_head: dtype must be 'bfloat16' or 'float32'")
     return _hils_block_M_attention_inverse.apply(
         q, k, v, weights, indices, block_size, sm_scale, mask_last_token, is_training, slope,
         kv_workspace, swa_o, swa_weight_index)

@@ -203,6 +203,22 @@ int hils_sparse_attn_bwd(const void* q, const void* k, const void* v, const void
                          int WH, int q_block, int S, float sm_scale, int mask_last, float sm_n,
                          const void* swa_o, void* d_swa_o, int merge_col, int kv_grad_bf16, void* stream);
 
+/* fp32 tensors: the reference's dtype="float32" / accum_dtype="float" mode of HiLS_block_M_head
+ * (ops/hils_fwd_bwd_head.py:928-964; its test_correctness_fp32, :1045-1126, runs in it).  Same
+ * arguments as above with q, k, v, weights, d_o, o, dq as fp32 tensors; everything is computed in
+ * fp32 (P is not rounded to bf16) on the shape-generic kernels (any D, Dv multiple of 8, any chunk
+ * size, slope, HSA arguments); no workspace, no merged local branch.  dk, dv, dw as in
+ * hils_sparse_attn_bwd without a workspace (fp32, ACCUMULATED: caller zero-fills). */
+int hils_sparse_attn_fwd_f32(const float* q, const float* k, const float* v, const float* weights,
+                             const int32_t* indices, const float* slope, float* o, float* lse, int B,
+                             int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int WH,
+                             int q_block, int S, float sm_scale, int mask_last, float sm_n, void* stream);
+int hils_sparse_attn_bwd_f32(const float* q, const float* k, const float* v, const float* weights,
+                             const int32_t* indices, const float* slope, const float* lse,
+                             const float* d_o, float* dq, float* dk, float* dv, float* dw, int B, int L,
+                             int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int WH, int q_block,
+                             int S, float sm_scale, int mask_last, float sm_n, void* stream);
+
 /* ---- decode over a paged cache (page = chunk = 64 tokens) ------------------------------ */
 
 /* The serving backend of the reference keeps the KV cache in pages of one chunk (README.md:262-264)

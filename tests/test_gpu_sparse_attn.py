@@ -322,3 +322,49 @@ def test_sparse_attn_merges_local_branch(pkg, orc, dev, B, L, HQ, H, D, Dv, K, e
     dw_ref[..., :K] = torch.where(valid, wf.grad[..., :K], torch.zeros(()))
     dw_ref[..., wcol] = wf.grad[..., wcol]
     assert_close_bf16(wd.grad, dw_ref, "dw (slots and the local branch's column)")
+
+
+@pytest.mark.parametrize("B,L,HQ,H,D,K,S,slope", [(1, 1024, 8, 1, 64, 4, 32, False),   # the reference's own fp32 test shape
+                                                  (2, 384, 8, 2, 128, 6, 64, True)])
+def test_sparse_attn_fp32_mode(pkg, orc, dev, B, L, HQ, H, D, K, S, slope):
+    """dtype="float32": fp32 tensors in and out, everything computed in fp32.  The reference runs its
+    fp32 correctness test in this mode (ops/hils_fwd_bwd_head.py:1045-1126: B1 L1024 H1 HQ8 D64, 4 slots,
+    chunk 32; bars 5e-3 on o and 5e-3 RMS ratio on every gradient); here the bars are 1e-4 (fp32 sums in
+    another order)."""
+    note(f"sparse_attn fp32 mode B{B} L{L} HQ{HQ} H{H} D{D} K{K} S{S} slope={slope}")
+    gen = torch.Generator().manual_seed(42)
+    q = torch.randn(B, L, HQ, D, generator=gen)
+    k = torch.randn(B, L, H, D, generator=gen)
+    v = torch.randn(B, L, H, D, generator=gen)
+    idx = rand_indices(B, L, H, K, S, gen, causal=True, n_chunks=L // S)
+    logits = torch.randn(B, L, HQ, K, generator=gen)
+    logits.masked_fill_(idx.repeat_interleave(HQ // H, dim=2) < 0, float("-inf"))
+    w = torch.nan_to_num(torch.softmax(logits, dim=-1), 0.0)
+    do = torch.randn(B, L, HQ, D, generator=gen)
+    sl = torch.rand(HQ, generator=gen) * 0.2 if slope else None
+    kw = {"slope": sl} if slope else {}
+    qd, kd, vd, wd = (t.to(dev).requires_grad_() for t in (q, k, v, w))
+    o = pkg.HiLS_block_M_head(qd, kd, vd, wd, idx.to(dev), block_size=S, mask_last_token=True, dtype="float",
+                              accum_dtype="float", block_M=2, num_threads=64, is_training=True, **kw)
+    assert o.dtype == torch.float32
+    o.backward(do.to(dev))
+    torch.cuda.synchronize()
+    qf, kf, vf, wf = (t.clone().requires_grad_() for t in (q, k, v, w))
+    ref = orc.sparse_attn(qf, kf, vf, wf, idx, chunk_size=S, **kw)
+    ref.backward(do)
+
+    def ratio(a, b):
+        return ((a.cpu() - b).square().mean().sqrt() / b.square().mean().sqrt().clamp_min(1e-30)).item()
+
+    worst = (o.detach().cpu() - ref.detach()).abs().max().item()
+    note(f"    o max-abs {worst:.3e}")
+    assert worst <= 1e-4
+    for name, got, want in (("dq", qd.grad, qf.grad), ("dk", kd.grad, kf.grad), ("dv", vd.grad, vf.grad),
+                            ("dw", wd.grad, wf.grad)):
+        assert got.dtype == torch.float32
+        r = ratio(got, want)
+        note(f"    {name} RMS error ratio {r:.3e}")
+        assert r <= 1e-4, name
+    with pytest.raises(TypeError):
+        pkg.HiLS_block_M_head(qd.detach().bfloat16(), kd.detach(), vd.detach(), wd.detach(), idx.to(dev), block_size=S,
+                              dtype="float32")
