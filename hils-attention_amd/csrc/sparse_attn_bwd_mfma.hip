@@ -890,8 +890,11 @@ void hils_build_chunk_index(const int32_t* indices, int* counts, int* offsets, i
     const long n = cells + 1;
     hipLaunchKernelGGL(bw_fill_int_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, counts, 0, n);
   }
+  // segments of queries per workgroup: short enough for a few thousand workgroups (the LDS atomics of
+  // a workgroup on one chunk's counter serialise), long enough that a workgroup's one global atomic per
+  // chunk stays cheap
   int seg_len = L;
-  while ((long)B * H * ((L + seg_len - 1) / seg_len) < 512 && seg_len > 256) seg_len = (seg_len + 1) / 2;
+  while ((long)B * H * ((L + seg_len - 1) / seg_len) < 4096 && seg_len > 128) seg_len = (seg_len + 1) / 2;
   dim3 gs((L + seg_len - 1) / seg_len, H, B);
   hipLaunchKernelGGL(bw_count_kernel, gs, dim3(1024), (size_t)nchunk * 4, st, indices, counts, L, H, K, nchunk, seg_len);
   hipLaunchKernelGGL(bw_scan_kernel, dim3(1), dim3(1024), 0, st, counts, offsets, cursor, cells);
