@@ -187,7 +187,7 @@ size_t hils_decode_workspace_bytes(int B, int L, int HQ, int H, int Dv, int K) {
 }
 
 bool hils_decode_rows_covers(int D, int Dv, int G, int K);
-void hils_sparse_attn_decode_rows(const void* q, const void* k, const void* v, const void* weights,
+int hils_sparse_attn_decode_rows(const void* q, const void* k, const void* v, const void* weights,
                                   const int32_t* indices, void* o, void* workspace, int nsplit,
                                   int B, int L, int Lkv, int HQ, int H, int D, int K, int NW,
                                   float sm_scale, int mask_last, const int32_t* page_table, int max_pages,
@@ -206,8 +206,9 @@ int hils_sparse_attn_decode(const void* q, const void* k, const void* v, const v
   dim3 grid(nsplit, H, (unsigned)((long)B * L));
   hipStream_t st = (hipStream_t)stream;
   if (hils_decode_rows_covers(D, Dv, HQ / H, K)) {
-    hils_sparse_attn_decode_rows(q, k, v, weights, indices, o, workspace, nsplit, B, L, Lkv, HQ, H, D,
-                                 K, NW, sm_scale, mask_last, nullptr, 0, 0, st);
+    if (int rc = hils_sparse_attn_decode_rows(q, k, v, weights, indices, o, workspace, nsplit, B, L, Lkv, HQ, H, D,
+                                              K, NW, sm_scale, mask_last, nullptr, 0, 0, st))
+      return rc;
   } else {
   const size_t smem = ((size_t)DE_WAVES * DE_S * 16 + (size_t)DE_WAVES * dm.G * Dv) * sizeof(float);
 #define DE_CALL(D_, DV_)                                                                           \
@@ -251,12 +252,13 @@ extern "C" int hils_sparse_attn_decode_paged(const void* q, const void* k_pages,
   HILS_REQUIRE(B > 0 && L > 0 && HQ > 0 && H > 0 && HQ % H == 0 && K > 0 && NW >= K && max_pages > 0 && num_pages > 0,
                "hils_sparse_attn_decode_paged: bad sizes");
   HILS_REQUIRE(hils_decode_rows_covers(D, D, HQ / H, K),
-               "hils_sparse_attn_decode_paged: needs D = Dv in {64, 128}, at most 4 query heads per KV head, K <= 1024");
+               "hils_sparse_attn_decode_paged: needs D = Dv in {64, 128}, at most 16 query heads per KV head, K <= 128");
   HILS_REQUIRE((long)B * L <= 65535L * 32768L && H <= 65535, "hils_sparse_attn_decode_paged: grid too large");
   const int nsplit = workspace ? de_pick_nsplit(B, L, H, K) : 1;
   hipStream_t st = (hipStream_t)stream;
-  hils_sparse_attn_decode_rows(q, k_pages, v_pages, weights, indices, o, workspace, nsplit, B, L, 0, HQ, H, D, K,
-                               NW, sm_scale, mask_last, page_table, max_pages, num_pages, st);
+  if (int rc = hils_sparse_attn_decode_rows(q, k_pages, v_pages, weights, indices, o, workspace, nsplit, B, L, 0, HQ,
+                                            H, D, K, NW, sm_scale, mask_last, page_table, max_pages, num_pages, st))
+    return rc;
   if (nsplit > 1) {
     const long rows = (long)B * L * HQ;
     const long n = rows * D;

@@ -1,20 +1,34 @@
-// Decode sparse attention, row-streaming variant (D == Dv, G <= 4).
+// Decode sparse attention, row-streaming MFMA variant (D == Dv in {64, 128}, up to 16 query heads
+// per KV head).
 //
-// Every K and V load is a fully coalesced 16-byte lane load: LR = D/8 neighbouring lanes
-// read one 2*D-byte token row, 64/LR token rows per instruction.  q.K uses packed bf16
-// dot2 instructions plus a DPP reduction over the LR lanes of a row; because K and V rows
-// are mapped to lanes the same way, the softmax probabilities of a token already sit in
-// the lanes that hold that token's V row, so P V needs no data movement at all.
-#include "decode_rows.h"
+// The step is bound by reading K and V of the selected chunks once, so everything else is kept
+// out of the memory pipeline's way:
+//   * every K and V load is a fully coalesced 16-byte lane load (D/8 neighbouring lanes read one
+//     2*D-byte token row).  A chunk is a stream of eight groups of 16 tokens (K0..K3, V0..V3) and
+//     a wavefront keeps a ring of NR register groups: the group just consumed is re-issued for the
+//     one NR places further down the stream, across chunk boundaries alike, so NR-1 groups
+//     (4 KiB each at D = 128) per wavefront are always in flight;
+//   * a consumed group is written row-major into the wavefront's own LDS staging area (rows padded
+//     by 16 bytes, so that the row-wise writes and the column-wise operand reads are both free of
+//     bank conflicts) and read back as MFMA operands: S^T = K q^T with the query heads in the 16
+//     MFMA columns, O^T += V^T P with V^T read by the transposing LDS load;
+//   * the per-chunk softmax runs on the 16 accumulator values a lane holds (token 4j+i of each
+//     16-token tile, head = lane & 15), its two cross-row reductions on the row-swap instructions;
+//     the chunk weight is folded into P, so the output accumulators are never rescaled.
+// The arithmetic is a few hundred instructions per 32 KiB chunk; the wavefronts of a workgroup own
+// slots (selected chunks) round-robin and their outputs are summed through LDS at the end.
+#include <type_traits>
+#include "common.h"
 #include "../../include/hils_amd.h"
 
-#define DR_THREADS 256
-#ifndef DR_MINW
-#define DR_MINW 4
-#endif
-#define DR_WAVES (DR_THREADS / 64)
 #define DR_S 64
-#define DR_MAXSLOT 64  // slots a wavefront can own: K <= 256 over at least 4 wavefronts
+#define DR_QT 16       // tokens per register group
+#define DR_NR 8        // register groups in the ring
+#define DR_MAXSLOT 32  // slots a wavefront can own
+#define DR_NH 16       // MFMA columns = query heads per KV head the kernel can take
+
+typedef unsigned dr_u4 __attribute__((ext_vector_type(4)));  // a 16-byte piece as a register value
+typedef short dr_s4 __attribute__((ext_vector_type(4)));
 
 struct DrDims {
   int L, Lkv, HQ, H, G, K, NW, nchunk, nsplit, mask_last;
@@ -25,171 +39,220 @@ struct DrDims {
   int max_pages, num_pages;
 };
 
-template <int D, int GMAX, int NWAVE>
-__global__ void __launch_bounds__(NWAVE * 64, (NWAVE == 4 ? DR_MINW : 1))
+static size_t dr_smem_bytes(int D, int G, int nwave) {
+  return (size_t)nwave * 32 * (2 * D + 16)             // staging areas: 32 padded token rows
+         + (size_t)nwave * G * D * sizeof(float)       // partial outputs
+         + (size_t)nwave * DR_MAXSLOT * (sizeof(long) + sizeof(int))  // slot lists
+         + (size_t)nwave * DR_MAXSLOT * DR_NH * sizeof(bf16_t);       // slot weights
+}
+
+template <int D, int NWAVE>
+__global__ void __launch_bounds__(NWAVE * 64)
 sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                const bf16_t* __restrict__ v, const bf16_t* __restrict__ weights,
                                const int32_t* __restrict__ indices, bf16_t* __restrict__ o,
                                float* __restrict__ partial, DrDims dm) {
-  constexpr int LR = D / 8;        // lanes per token row
-  constexpr int TPI = 64 / LR;     // token rows per load instruction
-  constexpr int NI = DR_S / TPI;   // load instructions per chunk
-  // load instructions per pipelined group: two groups (K and V) are in flight per wavefront, and
-  // with four the 128 registers a 16-wavefront workgroup leaves each lane no longer hold them
-  constexpr int GI = 2;
-  constexpr int NG = NI / GI;      // groups per chunk
-  extern __shared__ float o_s[];   // [wave][G][D] partial outputs
+  constexpr int LR = D / 8;          // lanes per token row
+  constexpr int TPI = 64 / LR;       // token rows per load instruction
+  constexpr int GL = DR_QT / TPI;    // load instructions per group
+  constexpr int KS = D / 32;         // k-steps of S^T = K q^T
+  constexpr int MT = D / 16;         // 16-feature tiles of O^T
+  constexpr int NR = DR_NR;
+  constexpr int ROWB = 2 * D + 16;   // bytes of a staged token row
+  constexpr int STAGE_B = 32 * ROWB;
+  extern __shared__ __align__(16) char dr_smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, j = lane >> 4;
   const int piece = lane % LR, tsub = lane / LR;
   const int split = blockIdx.x, hk = blockIdx.y;
   const long bt = blockIdx.z;
   const long b = bt / dm.L;
   const int G = dm.G, K = dm.K;
 
-  uint4 qp[GMAX];  // this lane's 8 features of each query head, packed bf16
+  char* stage_w = dr_smem + (size_t)wave * STAGE_B;
+  float* o_s = (float*)(dr_smem + (size_t)NWAVE * STAGE_B);  // [wave][G][D]
+  long* sl_off_all = (long*)(o_s + (size_t)NWAVE * G * D);
+  int* sl_id_all = (int*)(sl_off_all + NWAVE * DR_MAXSLOT);
+  bf16_t* sl_w_all = (bf16_t*)(sl_id_all + NWAVE * DR_MAXSLOT);
+  long* sl_off = sl_off_all + wave * DR_MAXSLOT;
+  int* sl_id = sl_id_all + wave * DR_MAXSLOT;
+  bf16_t* sl_w = sl_w_all + (size_t)wave * DR_MAXSLOT * DR_NH;
+
+  // query heads as the B operand of S^T = K q^T: lane (head = col, j) holds features ks*32 + j*8 ..
+  bf16x8_t qb[KS];
 #pragma unroll
-  for (int g = 0; g < GMAX; ++g) {
-    qp[g] = make_uint4(0, 0, 0, 0);
-    if (g < G) qp[g] = *(const uint4*)(q + (bt * dm.HQ + hk * G + g) * (long)D + piece * 8);
+  for (int ks = 0; ks < KS; ++ks) {
+    dr_u4 t = {0u, 0u, 0u, 0u};
+    if (col < G) t = *(const dr_u4*)(q + (bt * dm.HQ + hk * G + col) * (long)D + ks * 32 + j * 8);
+    qb[ks] = __builtin_bit_cast(bf16x8_t, t);
   }
   const float c2 = dm.sm_scale * HILS_LOG2E;
-  // running output of this wavefront, kept in its private slice of LDS (lanes < LR own it)
-  for (int i = lane; i < G * D; i += 64) o_s[(size_t)wave * G * D + i] = 0.f;
 
+  // ---- this wavefront's slots (s_begin + wave, + NWAVE, ...) that hold a mapped chunk: lane i
+  // looks at the i-th of them, the valid ones are compacted in order; byte offset of the
+  // chunk's first row, slot number and the heads' weights go to LDS ----
   const int per_split = (K + dm.nsplit - 1) / dm.nsplit;
   const int s_begin = split * per_split;
   const int s_end = (s_begin + per_split < K) ? s_begin + per_split : K;
-  // this wavefront's slots (s_begin + wave, + NWAVE, ...) that hold a mapped chunk: first-row element
-  // offset and slot number, kept in LDS so that the load of the next group never waits for an index
-  long* sl_off = (long*)(o_s + (size_t)NWAVE * G * D) + (size_t)wave * DR_MAXSLOT;
-  int* sl_id = (int*)((long*)(o_s + (size_t)NWAVE * G * D) + (size_t)NWAVE * DR_MAXSLOT) + wave * DR_MAXSLOT;
-  int nsl = 0;
-  long step = (long)TPI * (dm.page_table ? D : dm.H * D);
-  for (int slot = s_begin + wave; slot < s_end; slot += NWAVE) {
-    const int c = indices[(bt * dm.H + hk) * (long)K + slot];
-    if (c < 0 || c >= dm.nchunk) continue;
+  int nsl;
+  {
+    const int slot = s_begin + wave + lane * NWAVE;
+    bool ok = lane < DR_MAXSLOT && slot < s_end;
+    int c = -1;
+    if (ok) c = indices[(bt * dm.H + hk) * (long)K + slot];
+    ok = ok && c >= 0 && c < dm.nchunk;
     long row0;
     if (dm.page_table) {
-      const int pg = dm.page_table[b * dm.max_pages + c];
-      if (pg < 0 || pg >= dm.num_pages) continue;  // an unmapped chunk contributes nothing
-      row0 = ((long)pg * dm.H + hk) * DR_S + tsub;
+      int pg = -1;
+      if (ok) pg = dm.page_table[b * dm.max_pages + c];
+      ok = ok && pg >= 0 && pg < dm.num_pages;  // an unmapped chunk contributes nothing
+      row0 = ((long)pg * dm.H + hk) * DR_S;
     } else {
-      row0 = (b * dm.Lkv + (long)c * DR_S + tsub) * dm.H + hk;
+      row0 = (b * dm.Lkv + (long)c * DR_S) * dm.H + hk;
     }
-    // every lane stores its own first row (tsub differs): the list is per lane group in registers
-    // of the loop below, so only lane 0's view goes to LDS and tsub is added back on use
-    if (lane == 0 && nsl < DR_MAXSLOT) {
-      sl_off[nsl] = (row0 - tsub) * D;
-      sl_id[nsl] = slot;
+    const unsigned long long m = __ballot(ok);
+    const int pos = __popcll(m & ((1ull << lane) - 1ull));
+    nsl = __popcll(m);
+    if (ok) {
+      sl_off[pos] = row0 * D * 2;  // bytes
+      sl_id[pos] = slot;
     }
-    ++nsl;
   }
   __builtin_amdgcn_wave_barrier();
-  const long lane_off = (long)tsub * (dm.page_table ? D : dm.H * D) + piece * 8;
+  for (int s0 = 0; s0 < nsl; s0 += 4) {
+    const int si = s0 + j;
+    if (si < nsl && col < G) sl_w[si * DR_NH + col] = weights[(bt * dm.HQ + hk * G + col) * (long)dm.NW + sl_id[si]];
+  }
+  __builtin_amdgcn_wave_barrier();
 
-  // The (slot, group) units of this wavefront form one stream; the K and V rows of unit u+1 are
-  // loaded while unit u is computed (two register buffers), so a load is never waited for right
-  // after its issue, across group and slot boundaries alike.
-  const int nu = nsl * NG;
-  uint4 kr[2][GI], vr[2][GI];
-  auto load_unit = [&](int u, uint4 (&kd)[GI], uint4 (&vd)[GI]) {
-    const int si = u / NG, grp = u - si * NG;
-    const long off = sl_off[si] + lane_off + (long)grp * GI * step;
+  // Addresses are a wavefront-uniform 64-bit base (tensor + chunk + group + load number, scalar
+  // registers) plus one 32-bit byte offset per lane: no per-load vector address arithmetic.
+  const unsigned step_b = (dm.page_table ? (unsigned)D : (unsigned)dm.H * D) * 2u;  // bytes between token rows
+  const unsigned lane_b = (unsigned)tsub * step_b + (unsigned)piece * 16u;
+  const char* kb = (const char*)k;
+  const char* vb = (const char*)v;
+  auto chunk_off = [&](int si) __attribute__((always_inline)) -> long {  // byte offset of the chunk's first row
+    const long x = sl_off[si];
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)x);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(x >> 32));
+    return (long)(((unsigned long)hi << 32) | lo);
+  };
+  // stream group s of a chunk: s < 4 tokens 16s.. of K, else tokens 16(s-4).. of V
+  auto issue = [&](dr_u4 (&dst)[GL], long coff, int s) __attribute__((always_inline)) {
+    const char* base = (s < 4 ? kb : vb) + coff + (size_t)((s & 3) * DR_QT) * step_b;
 #pragma unroll
-    for (int i = 0; i < GI; ++i) {
-      kd[i] = *(const uint4*)(k + off + i * step);
-      vd[i] = *(const uint4*)(v + off + i * step);
+    for (int i = 0; i < GL; ++i) dst[i] = *(const dr_u4*)(base + (size_t)(i * TPI) * step_b + lane_b);
+  };
+  // per-lane LDS addresses: everything else is an immediate offset
+  char* const w_addr = stage_w + tsub * ROWB + piece * 16;                          // row-wise write of a load
+  const char* const k_addr = stage_w + col * ROWB + j * 16;                         // K tile as A operand
+  const char* const t_addr = stage_w + (4 * j + (col >> 2)) * ROWB + (col & 3) * 8; // transposing read of V
+  auto stage = [&](const dr_u4 (&src)[GL], int row0) __attribute__((always_inline)) {
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < GL; ++i) *(dr_u4*)(w_addr + (row0 + i * TPI) * ROWB) = src[i];
+    __builtin_amdgcn_wave_barrier();
+  };
+
+  f32x4_t S[4], O[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) O[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  bf16x8_t pb[2];  // P of the chunk as B operands: tokens 0..31 and 32..63
+
+  // K group t (tokens 16t ..): one 16-token tile of S^T
+  auto consume_k = [&](const dr_u4 (&src)[GL], int t) __attribute__((always_inline)) {
+    stage(src, 0);
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const dr_u4 a = *(const dr_u4*)(k_addr + ks * 64);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), qb[ks], acc, 0, 0, 0);
+    }
+    S[t] = acc;
+  };
+  // V group t: staged beside its neighbour; after the second of a pair,
+  // O^T[feature][head] += V^T[feature][token] P[token][head] over the pair's 32 tokens.  A lane's
+  // eight k-slots are tokens 4j..4j+3 of the first and of the second 16-token tile, the order in
+  // which the S^T accumulators hold them; the transposing LDS load delivers V^T in that order
+  // (a 16-lane group addresses a 4 x 16 block, lane l row l/4 and columns 4(l%4).., and receives
+  // column l of it).
+  auto consume_v = [&](const dr_u4 (&src)[GL], int t) __attribute__((always_inline)) {
+    stage(src, (t & 1) * 16);
+    if (!(t & 1)) return;
+    typedef short dr_s8 __attribute__((ext_vector_type(8)));
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const dr_s4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) dr_s4*)(t_addr + mt * 32));
+      const dr_s4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) dr_s4*)(t_addr + mt * 32 + 16 * ROWB));
+      const dr_s8 a = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+      O[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), pb[t >> 1], O[mt], 0, 0, 0);
     }
   };
-  float mrun[GMAX], lrun[GMAX], acc[GMAX][8];
-  auto compute_unit = [&](int u, const uint4 (&kc)[GI], const uint4 (&vc)[GI]) {
-    const int si = u / NG, grp = u - si * NG;
-    if (grp == 0) {
+  // softmax over the chunk's 64 tokens per head, the chunk weight folded in
+  auto softmax = [&](int si) __attribute__((always_inline)) {
+    if (dm.mask_last && j == 3) S[3][3] = HILS_NEG_INF;
+    float mx = HILS_NEG_INF;
 #pragma unroll
-      for (int g = 0; g < GMAX; ++g) {
-        mrun[g] = HILS_NEG_INF;
-        lrun[g] = 0.f;
+    for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, S[t][i]);
+    mx = rows_max(mx);
+    const float mc = (mx > HILS_NEG_INF) ? mx * c2 : 0.f;
+    float l = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        S[t][i] = __builtin_amdgcn_exp2f(fmaf(S[t][i], c2, -mc));
+        l += S[t][i];
       }
+    l = rows_sum(l);
+    const float wr = (col < G) ? bf2f(sl_w[si * DR_NH + col]) : 0.f;
+    const float f = (l > 0.f) ? wr / l : 0.f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      dr_u4 pk;
+      pk.x = pack_bf2(S[2 * h][0] * f, S[2 * h][1] * f);
+      pk.y = pack_bf2(S[2 * h][2] * f, S[2 * h][3] * f);
+      pk.z = pack_bf2(S[2 * h + 1][0] * f, S[2 * h + 1][1] * f);
+      pk.w = pack_bf2(S[2 * h + 1][2] * f, S[2 * h + 1][3] * f);
+      pb[h] = __builtin_bit_cast(bf16x8_t, pk);
     }
-    // flash-style pass over the chunk in NG groups of GI*TPI tokens; every token sub-group
-    // (lanes with the same tsub) keeps its own running max / sum / accumulator
-    float sc[GMAX][GI];
-#pragma unroll
-    for (int i = 0; i < GI; ++i)
-#pragma unroll
-      for (int g = 0; g < GMAX; ++g)
-        if (g < G) {
-          float s = row_sum<LR>(dot8_bf16(qp[g], kc[i], 0.f));
-          if (dm.mask_last && grp == NG - 1 && i == GI - 1 && tsub == TPI - 1) s = HILS_NEG_INF;
-          sc[g][i] = s;
-        }
-#pragma unroll
-    for (int g = 0; g < GMAX; ++g)
-      if (g < G) {
-        float mn = mrun[g];
-#pragma unroll
-        for (int i = 0; i < GI; ++i) mn = fmaxf(mn, sc[g][i]);
-        if (mn > HILS_NEG_INF) {
-          const float corr = __builtin_amdgcn_exp2f((mrun[g] - mn) * c2);
-          lrun[g] *= corr;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) acc[g][e] *= corr;
-#pragma unroll
-          for (int i = 0; i < GI; ++i) {
-            sc[g][i] = __builtin_amdgcn_exp2f((sc[g][i] - mn) * c2);
-            lrun[g] += sc[g][i];
-          }
-          mrun[g] = mn;
-        } else {
-#pragma unroll
-          for (int i = 0; i < GI; ++i) sc[g][i] = 0.f;
-        }
-      }
-#pragma unroll
-    for (int i = 0; i < GI; ++i) {
-      float vf[8];
-      unpack8(vc[i], vf);
-#pragma unroll
-      for (int g = 0; g < GMAX; ++g)
-        if (g < G) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(sc[g][i], vf[e], acc[g][e]);
-        }
-    }
-    if (grp != NG - 1) return;
-    // merge the token sub-groups, normalise, weight and add to the running output
-    const int slot = sl_id[si];
-#pragma unroll
-    for (int g = 0; g < GMAX; ++g)
-      if (g < G) {
-        float m = mrun[g];
-#pragma unroll
-        for (int off = LR; off < 64; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
-        const float sc2 = (mrun[g] > HILS_NEG_INF) ? __builtin_amdgcn_exp2f((mrun[g] - m) * c2) : 0.f;
-        float l = lrun[g] * sc2;
-#pragma unroll
-        for (int off = LR; off < 64; off <<= 1) l += __shfl_xor(l, off, 64);
-        const float wr = bf2f(weights[(bt * dm.HQ + hk * G + g) * (long)dm.NW + slot]);
-        const float f = (l > 0.f) ? sc2 * wr / l : 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float x = acc[g][e] * f;
-#pragma unroll
-          for (int off = LR; off < 64; off <<= 1) x += __shfl_xor(x, off, 64);
-          if (lane < LR) o_s[((size_t)wave * G + g) * D + lane * 8 + e] += x;
-        }
-      }
   };
-  if (nu > 0) load_unit(0, kr[0], vr[0]);
-  for (int u = 0; u < nu; u += 2) {
-    if (u + 1 < nu) load_unit(u + 1, kr[1], vr[1]);
-    compute_unit(u, kr[0], vr[0]);
-    if (u + 1 < nu) {
-      if (u + 2 < nu) load_unit(u + 2, kr[0], vr[0]);
-      compute_unit(u + 1, kr[1], vr[1]);
+
+  // One chunk: its eight groups in stream order; ring place s % NR holds group s and is re-issued
+  // for the group NR places on (of this chunk or of the next one, at byte offset noff).  The last
+  // chunk of the wavefront is a second copy of the code without the next chunk's loads, so that
+  // no load is conditional.
+  dr_u4 R[NR][GL];
+  auto chunk = [&](int si, long coff, long noff, auto more) __attribute__((always_inline)) {
+    constexpr bool MORE = decltype(more)::value;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      if (s < 4) consume_k(R[s % NR], s);
+      else consume_v(R[s % NR], s - 4);
+      if (s == 3) softmax(si);
+      if (s + NR < 8) issue(R[s % NR], coff, s + NR);
+      else if (MORE) issue(R[s % NR], noff, s + NR - 8);
     }
+  };
+  if (nsl > 0) {
+    long coff = chunk_off(0);
+#pragma unroll
+    for (int s = 0; s < NR; ++s) issue(R[s], coff, s);
+    for (int si = 0; si + 1 < nsl; ++si) {
+      const long noff = chunk_off(si + 1);
+      chunk(si, coff, noff, std::true_type{});
+      coff = noff;
+    }
+    chunk(nsl - 1, coff, 0, std::false_type{});
+  }
+
+  // accumulator register i of tile mt in lane (head = col, j) is feature mt*16 + 4j + i
+  if (col < G) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      *(f32x4_t*)&o_s[((size_t)wave * G + col) * D + mt * 16 + 4 * j] = O[mt];
   }
   __syncthreads();
   for (int i = tid; i < G * D; i += NWAVE * 64) {
@@ -202,37 +265,39 @@ sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   }
 }
 
-// (a wavefront keeps a list of at most DR_MAXSLOT slots: K <= 1024 covers every split the launcher picks)
+// A workgroup of 8 (no split) or 4 wavefronts, DR_MAXSLOT slots per wavefront: K <= 128 covers
+// every split the launcher picks.
 bool hils_decode_rows_covers(int D, int Dv, int G, int K) {
-  return D == Dv && (D == 64 || D == 128) && G <= 4 && K <= 16 * DR_MAXSLOT;
+  return D == Dv && (D == 64 || D == 128) && G >= 1 && G <= DR_NH && K <= 4 * DR_MAXSLOT;
 }
 
-void hils_sparse_attn_decode_rows(const void* q, const void* k, const void* v, const void* weights,
-                                  const int32_t* indices, void* o, void* workspace, int nsplit,
-                                  int B, int L, int Lkv, int HQ, int H, int D, int K, int NW,
-                                  float sm_scale, int mask_last, const int32_t* page_table, int max_pages,
-                                  int num_pages, hipStream_t st) {
+template <int D, int NWAVE>
+static int dr_launch(dim3 grid, hipStream_t st, const void* q, const void* k, const void* v, const void* weights,
+                     const int32_t* indices, void* o, void* workspace, const DrDims& dm) {
+  const size_t smem = dr_smem_bytes(D, dm.G, NWAVE);
+  auto kern = sparse_attn_decode_rows_kernel<D, NWAVE>;
+  static HilsLdsReserve reserved;  // per instantiation
+  if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_sparse_attn_fwd (decode)")) return rc;
+  hipLaunchKernelGGL(kern, grid, dim3(NWAVE * 64), smem, st, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v,
+                     (const bf16_t*)weights, indices, (bf16_t*)o, (float*)workspace, dm);
+  return HILS_OK;
+}
+
+int hils_sparse_attn_decode_rows(const void* q, const void* k, const void* v, const void* weights,
+                                 const int32_t* indices, void* o, void* workspace, int nsplit,
+                                 int B, int L, int Lkv, int HQ, int H, int D, int K, int NW,
+                                 float sm_scale, int mask_last, const int32_t* page_table, int max_pages,
+                                 int num_pages, hipStream_t st) {
   const int G = HQ / H;
   DrDims dm{L, Lkv, HQ, H, G, K, NW, page_table ? max_pages : Lkv / DR_S, nsplit, mask_last, sm_scale,
             page_table, max_pages, num_pages};
   dim3 grid(nsplit, H, (unsigned)((long)B * L));
-  // nsplit == 1 with many slots: one workgroup of 16 wavefronts per (query, KV head), no partial sums
-  const int nwave = (nsplit == 1 && K >= 16) ? 16 : DR_WAVES;
-  // partial outputs [wave][G][D] + the wavefronts' slot lists (row offsets, slot numbers)
-  const size_t smem = (size_t)nwave * G * D * sizeof(float) + (size_t)nwave * DR_MAXSLOT * (sizeof(long) + sizeof(int));
-#define DR_CALL_W(D_, G_, W_)                                                                    \
-  hipLaunchKernelGGL((sparse_attn_decode_rows_kernel<D_, G_, W_>), grid, dim3(W_ * 64), smem, st, \
-                     (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)weights, \
-                     indices, (bf16_t*)o, (float*)workspace, dm)
-#define DR_CALL(D_, G_)                                                                          \
-  do {                                                                                           \
-    if (nwave == 16) DR_CALL_W(D_, G_, 16); else DR_CALL_W(D_, G_, DR_WAVES);                    \
-  } while (0)
+  // no split and many slots: one workgroup of 8 wavefronts per (query, KV head)
+  const bool wide = nsplit == 1 && K >= 16;
   if (D == 64) {
-    if (G == 1) DR_CALL(64, 1); else if (G == 2) DR_CALL(64, 2); else DR_CALL(64, 4);
-  } else {
-    if (G == 1) DR_CALL(128, 1); else if (G == 2) DR_CALL(128, 2); else DR_CALL(128, 4);
+    return wide ? dr_launch<64, 8>(grid, st, q, k, v, weights, indices, o, workspace, dm)
+                : dr_launch<64, 4>(grid, st, q, k, v, weights, indices, o, workspace, dm);
   }
-#undef DR_CALL_W
-#undef DR_CALL
+  return wide ? dr_launch<128, 8>(grid, st, q, k, v, weights, indices, o, workspace, dm)
+              : dr_launch<128, 4>(grid, st, q, k, v, weights, indices, o, workspace, dm);
 }

@@ -1271,7 +1271,7 @@ struct TopkRowShared {
   int next_group;
 };
 
-template <int D, int GMAX, int NW>
+template <int D, int GMAX, int NW, bool PAGED>
 __global__ void __launch_bounds__(NW * 64)
 topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                 const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
@@ -1284,11 +1284,12 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   constexpr int EPT = TOPK_R_MAXN / THREADS;  // 64-chunk slots of a wavefront's share
   constexpr int GI = 8;          // load instructions per register buffer
   constexpr int KG = GI * TPI;   // chunk keys per buffer
-  extern __shared__ float dyn[];
+  extern __shared__ __align__(16) float dyn[];
   float* logit_s = dyn;                       // [GMAX][NP] raw scaled logits
   float* pooled = dyn + (size_t)GMAX * NP;    // [NP]
   // paged chunk keys, lmks = (num_pages, h_kv, D): the row's page ids are staged behind the pooled scores
-  int* page_s = (int*)(pooled + NP);          // [NP], only with a page table
+  int* page_s = (int*)(pooled + NP);          // [NP], only with a page table (else 0 entries)
+  const int NPG = PAGED ? NP : 0;             // the wavefronts' staging areas follow
   __shared__ TopkRowShared sh;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int piece = lane % LR, tsub = lane / LR;
@@ -1303,55 +1304,91 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
 #pragma unroll
   for (int g = 0; g < GMAX; ++g) swa[g] = (g < G) ? lse_swa[row * G + g] : 0.f;
   if (tid == 0) sh.next_group = 2 * NW;
-  if (page_table) {
-    for (int c = tid; c < lim; c += THREADS) {
-      int pg = c < max_pages ? page_table[b * max_pages + c] : -1;
+  // the query heads as B operand of the logit products, lane (head = lane & 15, j = lane >> 4) holds
+  // features ks*32 + 8j ..; loaded here so that the barrier below has waited for them
+  typedef unsigned tr_u4 __attribute__((ext_vector_type(4)));
+  bf16x8_t qb[D / 32];
+#pragma unroll
+  for (int ks = 0; ks < D / 32; ++ks) {
+    tr_u4 t = {0u, 0u, 0u, 0u};
+    if ((lane & 15) < G) t = *(const tr_u4*)(q + (row * (long)G + (lane & 15)) * D + ks * 32 + (lane >> 4) * 8);
+    qb[ks] = __builtin_bit_cast(bf16x8_t, t);
+  }
+  // have them arrive here: a load still pending at the streaming loop's first use would make the
+  // compiler wait for every load in flight there, in every iteration
+#pragma unroll
+  for (int ks = 0; ks < D / 32; ++ks) asm volatile("" : "+v"(qb[ks]));
+  if (PAGED) {  // every entry a load or a mask may look at gets a value
+    for (int c = tid; c < NP; c += THREADS) {
+      int pg = (c < lim && c < max_pages) ? page_table[b * max_pages + c] : -1;
       page_s[c] = (pg >= 0 && pg < num_pages) ? pg : -1;
     }
   }
   __syncthreads();
 
-  // ---- phase 1: logits of the visible chunks ----
+  // ---- phase 1: logits of the visible chunks.  The chunk-key rows arrive by coalesced 16-byte lane
+  // loads (LR lanes per row), are written row-major (rows padded by 16 bytes: no bank conflicts
+  // either way) into the wavefront's staging area 16 keys at a time and read back as the A operand
+  // of S^T = LMK q^T, the query heads in the MFMA columns: a few instructions per key row, so the
+  // phase runs at the speed of the memory stream ----
   {
-    uint4 qp[GMAX];
-#pragma unroll
-    for (int g = 0; g < GMAX; ++g) {
-      qp[g] = make_uint4(0, 0, 0, 0);
-      if (g < G) qp[g] = *(const uint4*)(q + (row * (long)G + g) * D + piece * 8);
-    }
+    constexpr int KS = D / 32;
+    constexpr int ROWB = 2 * D + 16;
+    constexpr int LPT = 16 / TPI;  // load instructions per 16-key tile
+    char* stage_w = (char*)(page_s + NPG) + (size_t)wave * 16 * ROWB;
+    const int col = lane & 15, j = lane >> 4;
+    char* const w_addr = stage_w + tsub * ROWB + piece * 16;
+    const char* const k_addr = stage_w + col * ROWB + j * 16;
     const int ngroups = (lim + KG - 1) / KG;
     const bf16_t* base = lmks + (b * N * (long)h_kv + hk) * D + piece * 8;
     const long cstride = (long)h_kv * D;
     const bf16_t* pbase = lmks + (long)hk * D + piece * 8;  // paged: + page * h_kv * D
-    auto fetch = [&](uint4 (&kr)[GI], int grp) {
+    auto fetch = [&](tr_u4 (&kr)[GI], int grp) __attribute__((always_inline)) {
 #pragma unroll
       for (int it = 0; it < GI; ++it) {
         int c = grp * KG + it * TPI + tsub;
         c = c < N ? c : N - 1;
-        if (page_table) {
-          const int pg = c < lim ? page_s[c] : -1;  // an unmapped chunk reads page 0 and is masked below
-          kr[it] = *(const uint4*)(pbase + (long)(pg < 0 ? 0 : pg) * cstride);
+        if (PAGED) {
+          const int pg = page_s[c];  // an unmapped or invisible chunk reads page 0 and is masked below
+          kr[it] = *(const tr_u4*)(pbase + (long)(pg < 0 ? 0 : pg) * cstride);
         } else {
-          kr[it] = *(const uint4*)(base + c * cstride);
+          kr[it] = *(const tr_u4*)(base + c * cstride);
         }
       }
     };
-    auto consume = [&](const uint4 (&kr)[GI], int grp) {
+    auto consume = [&](const tr_u4 (&kr)[GI], int grp) __attribute__((always_inline)) {
 #pragma unroll
-      for (int it = 0; it < GI; ++it) {
-        const int c = grp * KG + it * TPI + tsub;
+      for (int tt = 0; tt < GI / LPT; ++tt) {
+        __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int g = 0; g < GMAX; ++g)
-          if (g < G) {
-            const float sdot = row_sum<LR>(dot8_bf16(qp[g], kr[it], 0.f));
-            if (piece == 0 && c < N)
-              logit_s[g * NP + c] = (page_table && c < lim && page_s[c] < 0) ? HILS_NEG_INF : __fmul_rn(sdot, sm_scale);
+        for (int ii = 0; ii < LPT; ++ii) *(tr_u4*)(w_addr + ii * TPI * ROWB) = kr[tt * LPT + ii];
+        __builtin_amdgcn_wave_barrier();
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const tr_u4 a = *(const tr_u4*)(k_addr + ks * 64);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), qb[ks], acc, 0, 0, 0);
+        }
+        // accumulator register i of lane (head = col, j) is key c0 + 4j + i
+        const int c0 = grp * KG + tt * 16 + 4 * j;
+        if (col < G) {
+          f32x4_t out;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) out[i] = __fmul_rn(acc[i], sm_scale);
+          if (PAGED) {  // c0 + 3 < NP: groups end at a multiple of 64 at most
+            typedef int tr_i4 __attribute__((ext_vector_type(4)));
+            const tr_i4 pg4 = *(const tr_i4*)&page_s[c0];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (pg4[i] < 0) out[i] = HILS_NEG_INF;
           }
+          *(f32x4_t*)&logit_s[col * NP + c0] = out;
+        }
       }
     };
     // Groups of KG keys are handed out through a counter in LDS: the wavefronts of a workgroup
     // are served unevenly by the memory system, a fixed share would wait for the slowest.
-    // The first two groups of every wavefront are fixed (wave, wave + 16), the rest drawn.
+    // The first two groups of every wavefront are fixed (wave, wave + NW), the rest drawn.
     auto draw = [&]() -> int {
       int v = 0;
       if (lane == 0) v = atomicAdd(&sh.next_group, 1);
@@ -1359,7 +1396,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     };
     // drawn group numbers only grow, so the first one past the end ends the wavefront's walk
     const int last = ngroups - 1;
-    uint4 ka[GI], kb[GI];
+    tr_u4 ka[GI], kb[GI];
     int ga = wave, gb = wave + NW;
     if (ngroups > 0) {
       fetch(ka, ga < last ? ga : last);
@@ -1519,14 +1556,17 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, i
                         int num_pages = 0) {
   const long rows = (long)B * L * h_kv;
   const int NP = (N + 63) & ~63;
-  const size_t smem = (size_t)(page_table ? 6 : 5) * NP * sizeof(float);
-  // one round of rows or less: 16 wavefronts per row (the whole compute unit streams one row);
-  // more rows than compute units: 8, so that two workgroups share a unit and one row's selection
-  // overlaps the other row's streaming
-  const bool wide = rows <= topk_cus();
-#define TOPK_ROW_CALL_W(D_, W_)                                                                   \
+  // raw logits [4][NP], pooled scores, page ids; then 16 padded key rows of staging per wavefront
+  const size_t smem_base = (size_t)(page_table ? 6 : 5) * NP * sizeof(float);
+  const size_t stage_b = (size_t)16 * (2 * D + 16);
+  // one round of rows or less: 16 wavefronts per row (the whole compute unit streams one row) if
+  // their staging areas fit the LDS beside the logits; more rows than compute units: 8, so that
+  // two workgroups share a unit and one row's selection overlaps the other row's streaming
+  const bool wide = rows <= topk_cus() && smem_base + 16 * stage_b + sizeof(TopkRowShared) <= 158 * 1024;
+  const size_t smem = smem_base + (wide ? 16 : 8) * stage_b;
+#define TOPK_ROW_CALL_W(D_, W_, P_)                                                               \
   do {                                                                                           \
-    auto kern = topk_row_kernel<D_, 4, W_>;                                                      \
+    auto kern = topk_row_kernel<D_, 4, W_, P_>;                                                  \
     static HilsLdsReserve reserved;                                                              \
     if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_topk_fwd")) return rc; \
     hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(W_ * 64), smem, st,                      \
@@ -1535,11 +1575,15 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, i
                        block_size, window_size, causal, q_offset, sm_scale, page_table, max_pages, \
                        num_pages);                                                               \
   } while (0)
-#define TOPK_ROW_CALL(D_)                                                                        \
+#define TOPK_ROW_CALL(D_, P_)                                                                    \
   do {                                                                                           \
-    if (wide) TOPK_ROW_CALL_W(D_, 16); else TOPK_ROW_CALL_W(D_, 8);                              \
+    if (wide) TOPK_ROW_CALL_W(D_, 16, P_); else TOPK_ROW_CALL_W(D_, 8, P_);                      \
   } while (0)
-  if (D == 64) TOPK_ROW_CALL(64); else TOPK_ROW_CALL(128);
+  if (page_table) {
+    if (D == 64) TOPK_ROW_CALL(64, true); else TOPK_ROW_CALL(128, true);
+  } else {
+    if (D == 64) TOPK_ROW_CALL(64, false); else TOPK_ROW_CALL(128, false);
+  }
 #undef TOPK_ROW_CALL
 #undef TOPK_ROW_CALL_W
   return HILS_OK;
