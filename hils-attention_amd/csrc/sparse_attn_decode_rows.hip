@@ -88,14 +88,26 @@ sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   }
   const float c2 = dm.sm_scale * HILS_LOG2E;
 
-  // ---- this wavefront's slots (s_begin + wave, + NWAVE, ...) that hold a mapped chunk: lane i
-  // looks at the i-th of them, the valid ones are compacted in order; byte offset of the
-  // chunk's first row, slot number and the heads' weights go to LDS ----
+  // ---- this wavefront's slots (s_begin + wave, + NWAVE, ...): lane i looks at the i-th of them, the
+  // ones that hold a mapped chunk are compacted in order (byte offset of the chunk's first row and
+  // i go to LDS).  The heads' weights of all of them are loaded alongside the indices, so the
+  // stream below starts one memory latency after the kernel ----
   const int per_split = (K + dm.nsplit - 1) / dm.nsplit;
   const int s_begin = split * per_split;
   const int s_end = (s_begin + per_split < K) ? s_begin + per_split : K;
+  const int nmine = (s_end - s_begin - wave + NWAVE - 1) / NWAVE;  // slots of this wavefront (may be <= 0)
   int nsl;
   {
+    bf16_t wv[DR_MAXSLOT / 4];
+#pragma unroll
+    for (int p4 = 0; p4 < DR_MAXSLOT / 4; ++p4) {
+      wv[p4] = 0;
+      if (p4 * 4 < nmine) {  // uniform
+        const int i = p4 * 4 + j;
+        if (i < nmine && col < G)
+          wv[p4] = weights[(bt * dm.HQ + hk * G + col) * (long)dm.NW + s_begin + wave + i * NWAVE];
+      }
+    }
     const int slot = s_begin + wave + lane * NWAVE;
     bool ok = lane < DR_MAXSLOT && slot < s_end;
     int c = -1;
@@ -115,13 +127,11 @@ sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
     nsl = __popcll(m);
     if (ok) {
       sl_off[pos] = row0 * D * 2;  // bytes
-      sl_id[pos] = slot;
+      sl_id[pos] = lane;
     }
-  }
-  __builtin_amdgcn_wave_barrier();
-  for (int s0 = 0; s0 < nsl; s0 += 4) {
-    const int si = s0 + j;
-    if (si < nsl && col < G) sl_w[si * DR_NH + col] = weights[(bt * dm.HQ + hk * G + col) * (long)dm.NW + sl_id[si]];
+#pragma unroll
+    for (int p4 = 0; p4 < DR_MAXSLOT / 4; ++p4)
+      if (p4 * 4 < nmine) sl_w[(p4 * 4 + j) * DR_NH + col] = wv[p4];
   }
   __builtin_amdgcn_wave_barrier();
 
@@ -207,7 +217,7 @@ sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
         l += S[t][i];
       }
     l = rows_sum(l);
-    const float wr = (col < G) ? bf2f(sl_w[si * DR_NH + col]) : 0.f;
+    const float wr = (col < G) ? bf2f(sl_w[sl_id[si] * DR_NH + col]) : 0.f;
     const float f = (l > 0.f) ? wr / l : 0.f;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {

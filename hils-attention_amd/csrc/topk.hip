@@ -1268,8 +1268,13 @@ struct TopkRowShared {
   int ncand[TOPK_R_WAVES];
   float4 red_m[TOPK_R_WAVES];  // per wavefront, one component per head
   float4 red_l[TOPK_R_WAVES];
+  uint32_t gmax[64];           // largest selection key of every 16-lane group of the workgroup
+  int wcnt[TOPK_R_WAVES];      // keys of a wavefront that reach the candidate bound
+  float tot[4];                // lse_total per head
+  uint32_t thr;                // the candidate bound
   int next_group;
 };
+#define TOPK_R_CAND 256  // candidates the single-wavefront final selection takes
 
 template <int D, int GMAX, int NW, bool PAGED>
 __global__ void __launch_bounds__(NW * 64)
@@ -1339,6 +1344,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     const int col = lane & 15, j = lane >> 4;
     char* const w_addr = stage_w + tsub * ROWB + piece * 16;
     const char* const k_addr = stage_w + col * ROWB + j * 16;
+    float m_run = HILS_NEG_INF, l_run = 0.f;
     const int ngroups = (lim + KG - 1) / KG;
     const bf16_t* base = lmks + (b * N * (long)h_kv + hk) * D + piece * 8;
     const long cstride = (long)h_kv * D;
@@ -1374,7 +1380,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
         if (col < G) {
           f32x4_t out;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) out[i] = __fmul_rn(acc[i], sm_scale);
+          for (int i = 0; i < 4; ++i) out[i] = (c0 + i < lim) ? __fmul_rn(acc[i], sm_scale) : HILS_NEG_INF;
           if (PAGED) {  // c0 + 3 < NP: groups end at a multiple of 64 at most
             typedef int tr_i4 __attribute__((ext_vector_type(4)));
             const tr_i4 pg4 = *(const tr_i4*)&page_s[c0];
@@ -1383,6 +1389,14 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
               if (pg4[i] < 0) out[i] = HILS_NEG_INF;
           }
           *(f32x4_t*)&logit_s[col * NP + c0] = out;
+          // running log-sum-exp of this lane's head over the keys it has seen
+          const float mn = fmaxf(fmaxf(m_run, fmaxf(out[0], out[1])), fmaxf(out[2], out[3]));
+          const float ms = (mn == HILS_NEG_INF) ? 0.f : mn * HILS_LOG2E;
+          float add = 0.f;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) add += __builtin_amdgcn_exp2f(fmaf(out[i], HILS_LOG2E, -ms));
+          l_run = fmaf(l_run, __builtin_amdgcn_exp2f(fmaf(m_run, HILS_LOG2E, -ms)), add);
+          m_run = mn;
         }
       }
     };
@@ -1411,97 +1425,163 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       gb = draw();
       fetch(kb, gb < last ? gb : last);
     }
+    // the wavefront's (max, sum) per head: the four lane rows of a column hold the same head
+    {
+      const float M = rows_max(m_run);
+      const float Ms = (M == HILS_NEG_INF) ? 0.f : M * HILS_LOG2E;
+      const float Lw = rows_sum(l_run * __builtin_amdgcn_exp2f(fmaf(m_run, HILS_LOG2E, -Ms)));
+      if (j == 0 && col < GMAX) {
+        ((float*)&sh.red_m[wave])[col] = (col < G) ? M : HILS_NEG_INF;
+        ((float*)&sh.red_l[wave])[col] = (col < G) ? Lw : 0.f;
+      }
+    }
   }
   __syncthreads();
 
-  // ---- phase 2: LSE per head.  Wavefront w owns the chunks [w*per, (w+1)*per): the same chunks it
-  // selects from later, so its pooled scores never leave the wavefront before the selection. ----
-  static_assert(GMAX == 4, "the cross-wavefront reductions carry four heads per float4");
-  const int per = ((N + NW - 1) / NW + 63) & ~63;  // <= 256 = 64 * EPT
-  const int cbase = wave * per;
-  float x[GMAX][EPT];
-  {
-    float m[GMAX], l[GMAX];
+  // ---- phase 2: LSE per head from the wavefronts' partial sums.  Work every wavefront would do
+  // alike costs its instruction count once per wavefront of a SIMD, so one wavefront per head does
+  // it and the result goes through LDS ----
+  static_assert(GMAX == 4 && NW >= GMAX, "the cross-wavefront reductions carry four heads per float4");
+  if (wave < GMAX) {
+    const int g = wave;
+    // every row of 16 lanes combines the NW (max, sum) pairs: the result is uniform without a broadcast
+    const bool has = (lane & 15) < NW;
+    const float mw = has ? ((const float*)&sh.red_m[lane & 15])[g] : HILS_NEG_INF;
+    const float lw = has ? ((const float*)&sh.red_l[lane & 15])[g] : 0.f;
+    const float mx = row_max16(mw);
+    const float part = (mw > HILS_NEG_INF) ? lw * __expf(mw - mx) : 0.f;
+    const float lsum = row_sum<16>(part);
+    const float lse_hils = (lsum > 0.f) ? mx + __logf(lsum) : HILS_NEG_INF;
+    float sw = swa[0];
 #pragma unroll
-    for (int g = 0; g < GMAX; ++g) {
-      m[g] = HILS_NEG_INF;
-#pragma unroll
-      for (int e = 0; e < EPT; ++e) {
-        const int c = cbase + e * 64 + lane;
-        x[g][e] = (g < G && e * 64 < per && c < lim) ? logit_s[g * NP + c] : HILS_NEG_INF;
-        m[g] = fmaxf(m[g], x[g][e]);
-      }
-      m[g] = wave_max_f(m[g]);
-      l[g] = 0.f;
-      if (m[g] > HILS_NEG_INF) {
-#pragma unroll
-        for (int e = 0; e < EPT; ++e) l[g] += __expf(x[g][e] - m[g]);
-      }
-      l[g] = wave_sum_f(l[g]);
-    }
+    for (int g2 = 1; g2 < GMAX; ++g2) sw = (g == g2) ? swa[g2] : sw;
+    // logaddexp on the hardware exp2/log2
+    const float hi = fmaxf(sw, lse_hils), lo = fminf(sw, lse_hils);
+    const float t = (lo == HILS_NEG_INF) ? hi : hi + __logf(1.f + __expf(lo - hi));
     if (lane == 0) {
-      sh.red_m[wave] = make_float4(m[0], m[1], m[2], m[3]);
-      sh.red_l[wave] = make_float4(l[0], l[1], l[2], l[3]);
+      sh.tot[g] = t;
+      if (lse_total_out && g < G) lse_total_out[row * G + g] = t;
     }
   }
   __syncthreads();
   float tot[GMAX];
-  {
-    // every row of 16 lanes combines the 16 (max, sum) pairs: the result is uniform without a broadcast
-    const bool has = (lane & 15) < NW;
-    const float4 m4 = has ? sh.red_m[lane & 15] : make_float4(HILS_NEG_INF, HILS_NEG_INF, HILS_NEG_INF, HILS_NEG_INF);
-    const float4 l4 = has ? sh.red_l[lane & 15] : make_float4(0.f, 0.f, 0.f, 0.f);
-    const float mw[GMAX] = {m4.x, m4.y, m4.z, m4.w}, lw[GMAX] = {l4.x, l4.y, l4.z, l4.w};
 #pragma unroll
-    for (int g = 0; g < GMAX; ++g) {
-      const float mx = row_max16(mw[g]);
-      const float part = (mw[g] > HILS_NEG_INF) ? lw[g] * __expf(mw[g] - mx) : 0.f;
-      const float lsum = row_sum<16>(part);
-      const float lse_hils = (lsum > 0.f) ? mx + __logf(lsum) : HILS_NEG_INF;
-      // logaddexp on the hardware exp2/log2
-      const float hi = fmaxf(swa[g], lse_hils), lo = fminf(swa[g], lse_hils);
-      tot[g] = (lo == HILS_NEG_INF) ? hi : hi + __logf(1.f + __expf(lo - hi));
-      if (lse_total_out && tid == 0 && g < G) lse_total_out[row * G + g] = tot[g];
-    }
-  }
-  // ---- phase 3: pooled scores of the own chunks, selection among them, winners (padded to topk
-  // entries with -inf) straight into this wavefront's slice of the merge list ----
+  for (int g = 0; g < GMAX; ++g) tot[g] = sh.tot[g];
+  // ---- phase 3: selection.  Wavefront w owns the chunks [w*per, (w+1)*per); the selection key of a
+  // chunk is max over the heads of (logit - lse_total) as an order-preserving integer ----
+  const int per = ((N + NW - 1) / NW + 63) & ~63;  // <= 64 * EPT
+  const int cbase = wave * per;
+  uint32_t key[EPT];
+  uint32_t lmax = 0u;
 #pragma unroll
   for (int e = 0; e < EPT; ++e) {
-    const int c = cbase + e * 64 + lane;
-    float best = HILS_NEG_INF;
+    key[e] = 0u;
+    if (e * 64 < per) {  // uniform: the slots past the wavefront's share cost nothing
+      const int c = cbase + e * 64 + lane;
+      const bool mine = c < lim;
+      float best = HILS_NEG_INF;
 #pragma unroll
-    for (int g = 0; g < GMAX; ++g)
-      if (g < G) {
-        const float nrm = (x[g][e] == HILS_NEG_INF) ? HILS_NEG_INF : __fsub_rn(x[g][e], tot[g]);
-        best = fmaxf(best, nrm);
-        if (sel_logits_out && e * 64 < per && c < N) sel_logits_out[(row * G + g) * (long)N + c] = x[g][e];
-      }
-    if (e * 64 < per && c < lim) pooled[c] = best;
+      for (int g = 0; g < GMAX; ++g)
+        if (g < G) {
+          const float xv = mine ? logit_s[g * NP + c] : HILS_NEG_INF;
+          const float nrm = (xv == HILS_NEG_INF) ? HILS_NEG_INF : __fsub_rn(xv, tot[g]);
+          best = fmaxf(best, nrm);
+          if (sel_logits_out && c < N) sel_logits_out[(row * G + g) * (long)N + c] = xv;
+        }
+      if (mine) pooled[c] = best;
+      key[e] = score_key(best);
+      lmax = key[e] > lmax ? key[e] : lmax;
+    }
   }
-  __builtin_amdgcn_wave_barrier();
+  // A lower bound of the topk-th largest key with few keys above it: the topk-th largest of the
+  // maxima of the workgroup's 16-lane groups (4 * NW of them), found by one wavefront.  The keys
+  // that reach it are compacted in chunk order into one list and a single wavefront selects
+  // among them.
   {
+    uint32_t gm = lmax, y;
+    y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gm, 0xB1, 0xF, 0xF, true);  gm = gm > y ? gm : y;
+    y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gm, 0x4E, 0xF, 0xF, true);  gm = gm > y ? gm : y;
+    y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gm, 0x141, 0xF, 0xF, true); gm = gm > y ? gm : y;
+    y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gm, 0x140, 0xF, 0xF, true); gm = gm > y ? gm : y;
+    if ((lane & 15) == 0) sh.gmax[wave * 4 + (lane >> 4)] = gm;
+    if (NW * 4 < 64 && tid >= NW * 4 && tid < 64) sh.gmax[tid] = 0u;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    uint32_t t = 1u;  // every valid key is >= 1
+    const uint32_t gv = sh.gmax[lane];
+    if (__popcll(__ballot(gv != 0u)) >= topk) {
+      const uint32_t hi = wave_max_u(gv);
+      const uint32_t lo = ~wave_max_u(gv ? ~gv : 0u);  // smallest non-zero group maximum
+      t = lane_kth_largest(gv, lo, hi, topk);
+    }
+    if (lane == 0) sh.thr = t;
+  }
+  __syncthreads();
+  const unsigned long long lt = (1ull << lane) - 1ull;
+  const uint32_t thr = sh.thr;
+  {
+    int cnt = 0;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e)
+      if (e * 64 < per) cnt += __popcll(__ballot(key[e] >= thr));
+    if (lane == 0) sh.wcnt[wave] = cnt;
+  }
+  __syncthreads();
+  int cand_base = 0, cand_total = 0;
+#pragma unroll
+  for (int w2 = 0; w2 < NW; ++w2) {
+    const int v = sh.wcnt[w2];
+    cand_total += v;
+    cand_base += (w2 < wave) ? v : 0;
+  }
+  if (cand_total <= TOPK_R_CAND) {
+    uint32_t* ck = (uint32_t*)sh.merge_s;  // NW * TOPK_MAXK >= 512 entries
+    int pos = cand_base;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      if (e * 64 < per) {
+        const bool pred = key[e] >= thr;
+        const unsigned long long m = __ballot(pred);
+        if (pred) {
+          const int o = pos + __popcll(m & lt);
+          ck[o] = key[e];
+          sh.merge_i[o] = cbase + e * 64 + lane;
+        }
+        pos += __popcll(m);
+      }
+    }
+    __syncthreads();
+    if (wave == 0) {
+      const int nc = wave_select<true, TOPK_R_CAND / 64>((const float*)ck, cand_total, 0, sh.cand_s[0], sh.cand_i[0], 0,
+                                                          topk, sh.merge_i);
+      if (lane == 0) sh.ncand[0] = nc;
+    }
+  } else {
+    // many keys at the bound (equal scores, or fewer than topk groups with a visible chunk while
+    // more than TOPK_R_CAND chunks are visible): every wavefront selects among its own chunks,
+    // winners (padded to topk entries with -inf) into its slice of the merge list, one wavefront merges
     int nc = 0;
     if (cbase < lim) {
       const int ns = (lim - cbase < per) ? lim - cbase : per;
       nc = wave_select<false, EPT>(pooled + cbase, ns, cbase, sh.merge_s + wave * topk,
-                                          sh.merge_i + wave * topk, 0, topk, nullptr, sh.cand_s[wave],
-                                          sh.cand_i[wave]);
+                                   sh.merge_i + wave * topk, 0, topk, nullptr, sh.cand_s[wave],
+                                   sh.cand_i[wave]);
     }
     if (lane >= nc && lane < topk) {
       sh.merge_s[wave * topk + lane] = HILS_NEG_INF;
       sh.merge_i[wave * topk + lane] = 0;
     }
-  }
-  __syncthreads();
-  if (wave == 0) {
-    const int total = NW * topk;
-    int nc = 0;
-    for (int p0 = 0; p0 < total; p0 += TOPK_NSEG) {
-      const int ns = (total - p0 < TOPK_NSEG) ? total - p0 : TOPK_NSEG;
-      nc = wave_select(sh.merge_s + p0, ns, 0, sh.cand_s[0], sh.cand_i[0], nc, topk, sh.merge_i + p0);
+    __syncthreads();
+    if (wave == 0) {
+      const int total = NW * topk;
+      int nc2 = 0;
+      for (int p0 = 0; p0 < total; p0 += TOPK_NSEG) {
+        const int ns = (total - p0 < TOPK_NSEG) ? total - p0 : TOPK_NSEG;
+        nc2 = wave_select(sh.merge_s + p0, ns, 0, sh.cand_s[0], sh.cand_i[0], nc2, topk, sh.merge_i + p0);
+      }
+      if (lane == 0) sh.ncand[0] = nc2;
     }
-    if (lane == 0) sh.ncand[0] = nc;
   }
   __syncthreads();
   // ---- phase 4: indices (ascending) and the raw scaled scores of the winners ----
