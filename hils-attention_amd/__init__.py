@@ -11,7 +11,7 @@ from .ops.topk_head_softmax import online_softmax_topk_head  # noqa: F401
 from .ops.hils_fwd_bwd_head import HiLS_block_M_head  # noqa: F401
 from .ops.hsa_triton import HSA  # noqa: F401
 from .ops.exact_chunk_log_z_tilelang import exact_chunk_log_z_tl  # noqa: F401
-from .ops.hils_glue import chunk_weights, topk_chunk_weights  # noqa: F401
+from .ops.hils_glue import chunk_weights, decode_step, topk_chunk_weights  # noqa: F401
 from .ops.flex_attn_tilelang import flex_attn_tl, flex_attn_tl_two_phase  # noqa: F401
 from .ops.hils_fwd_bwd_head import prepare_kv_workspace  # noqa: F401
 from .utils.hils_cache_utils import HiLSDynamicLayer, HiLSPagedLayer, paged_hils_attend  # noqa: F401

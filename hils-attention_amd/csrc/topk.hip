@@ -9,6 +9,7 @@
 // bitwise threshold search on order-preserving integer keys.  Ties: lower index wins.
 #include <type_traits>
 #include "decode_rows.h"
+#include "decode_rows_body.h"
 #include "../../include/hils_amd.h"
 
 #define TOPK_THREADS 256
@@ -1266,8 +1267,10 @@ struct TopkRowShared {
   float merge_s[TOPK_R_WAVES * TOPK_MAXK];
   int merge_i[TOPK_R_WAVES * TOPK_MAXK];
   int ncand[TOPK_R_WAVES];
-  float4 red_m[TOPK_R_WAVES];  // per wavefront, one component per head
-  float4 red_l[TOPK_R_WAVES];
+  // (max, sum of exponentials) of every streamed key group, one component per head: combined in a
+  // fixed order, so the log-sum-exp does not depend on which wavefront drew which group
+  float grp_m[TOPK_R_MAXN / 32][4];
+  float grp_l[TOPK_R_MAXN / 32][4];
   uint32_t gmax[64];           // largest selection key of every 16-lane group of the workgroup
   int wcnt[TOPK_R_WAVES];      // keys of a wavefront that reach the candidate bound
   float tot[4];                // lse_total per head
@@ -1276,20 +1279,22 @@ struct TopkRowShared {
 };
 #define TOPK_R_CAND 256  // candidates the single-wavefront final selection takes
 
+// One (query, KV head) row (row = (b*L + t)*h_kv + hk) by a workgroup of NW wavefronts; dyn = the
+// workgroup's dynamic LDS (topk_row_smem bytes).
 template <int D, int GMAX, int NW, bool PAGED>
-__global__ void __launch_bounds__(NW * 64)
-topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
-                const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
-                bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
-                float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
-                int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
-                float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages) {
+__device__ __forceinline__ void
+topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
+              const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
+              bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
+              float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
+              int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
+              float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages,
+              float* dyn, const long row) {
   constexpr int LR = D / 8, TPI = 64 / LR;
   constexpr int THREADS = NW * 64;       // NW = 8 or 16 wavefronts
   constexpr int EPT = TOPK_R_MAXN / THREADS;  // 64-chunk slots of a wavefront's share
   constexpr int GI = 8;          // load instructions per register buffer
   constexpr int KG = GI * TPI;   // chunk keys per buffer
-  extern __shared__ __align__(16) float dyn[];
   float* logit_s = dyn;                       // [GMAX][NP] raw scaled logits
   float* pooled = dyn + (size_t)GMAX * NP;    // [NP]
   // paged chunk keys, lmks = (num_pages, h_kv, D): the row's page ids are staged behind the pooled scores
@@ -1298,7 +1303,6 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   __shared__ TopkRowShared sh;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int piece = lane % LR, tsub = lane / LR;
-  const long row = blockIdx.x;  // (b*L + t)*h_kv + hk
   const int hk = (int)(row % h_kv);
   const long bt = row / h_kv;
   const int t = (int)(bt % L);
@@ -1344,7 +1348,6 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     const int col = lane & 15, j = lane >> 4;
     char* const w_addr = stage_w + tsub * ROWB + piece * 16;
     const char* const k_addr = stage_w + col * ROWB + j * 16;
-    float m_run = HILS_NEG_INF, l_run = 0.f;
     const int ngroups = (lim + KG - 1) / KG;
     const bf16_t* base = lmks + (b * N * (long)h_kv + hk) * D + piece * 8;
     const long cstride = (long)h_kv * D;
@@ -1363,6 +1366,7 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       }
     };
     auto consume = [&](const tr_u4 (&kr)[GI], int grp) __attribute__((always_inline)) {
+      float m_run = HILS_NEG_INF, l_run = 0.f;  // this lane's head over the group's keys it sees
 #pragma unroll
       for (int tt = 0; tt < GI / LPT; ++tt) {
         __builtin_amdgcn_wave_barrier();
@@ -1399,6 +1403,14 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
           m_run = mn;
         }
       }
+      // the group's (max, sum) per head: the four lane rows of a column hold the same head
+      const float M = rows_max(m_run);
+      const float Ms = (M == HILS_NEG_INF) ? 0.f : M * HILS_LOG2E;
+      const float Lg = rows_sum(l_run * __builtin_amdgcn_exp2f(fmaf(m_run, HILS_LOG2E, -Ms)));
+      if (j == 0 && col < GMAX) {  // lanes of heads past G never left (-inf, 0)
+        sh.grp_m[grp][col] = M;
+        sh.grp_l[grp][col] = Lg;
+      }
     };
     // Groups of KG keys are handed out through a counter in LDS: the wavefronts of a workgroup
     // are served unevenly by the memory system, a fixed share would wait for the slowest.
@@ -1425,32 +1437,25 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       gb = draw();
       fetch(kb, gb < last ? gb : last);
     }
-    // the wavefront's (max, sum) per head: the four lane rows of a column hold the same head
-    {
-      const float M = rows_max(m_run);
-      const float Ms = (M == HILS_NEG_INF) ? 0.f : M * HILS_LOG2E;
-      const float Lw = rows_sum(l_run * __builtin_amdgcn_exp2f(fmaf(m_run, HILS_LOG2E, -Ms)));
-      if (j == 0 && col < GMAX) {
-        ((float*)&sh.red_m[wave])[col] = (col < G) ? M : HILS_NEG_INF;
-        ((float*)&sh.red_l[wave])[col] = (col < G) ? Lw : 0.f;
-      }
-    }
   }
   __syncthreads();
 
-  // ---- phase 2: LSE per head from the wavefronts' partial sums.  Work every wavefront would do
+  // ---- phase 2: LSE per head from the key groups' partial sums.  Work every wavefront would do
   // alike costs its instruction count once per wavefront of a SIMD, so one wavefront per head does
   // it and the result goes through LDS ----
-  static_assert(GMAX == 4 && NW >= GMAX, "the cross-wavefront reductions carry four heads per float4");
+  static_assert(GMAX == 4 && NW >= GMAX, "one wavefront per head, four heads per group entry");
   if (wave < GMAX) {
     const int g = wave;
-    // every row of 16 lanes combines the NW (max, sum) pairs: the result is uniform without a broadcast
-    const bool has = (lane & 15) < NW;
-    const float mw = has ? ((const float*)&sh.red_m[lane & 15])[g] : HILS_NEG_INF;
-    const float lw = has ? ((const float*)&sh.red_l[lane & 15])[g] : 0.f;
-    const float mx = row_max16(mw);
-    const float part = (mw > HILS_NEG_INF) ? lw * __expf(mw - mx) : 0.f;
-    const float lsum = row_sum<16>(part);
+    const int ngroups = (lim + KG - 1) / KG;
+    float mw = HILS_NEG_INF;
+    for (int i = lane; i < ngroups; i += 64) mw = fmaxf(mw, sh.grp_m[i][g]);
+    const float mx = wave_max_f(mw);
+    float part = 0.f;
+    for (int i = lane; i < ngroups; i += 64) {
+      const float mi = sh.grp_m[i][g];
+      part += (mi > HILS_NEG_INF) ? sh.grp_l[i][g] * __expf(mi - mx) : 0.f;
+    }
+    const float lsum = wave_sum_f(part);
     const float lse_hils = (lsum > 0.f) ? mx + __logf(lsum) : HILS_NEG_INF;
     float sw = swa[0];
 #pragma unroll
@@ -1614,6 +1619,52 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   }
 }
 
+template <int D, int GMAX, int NW, bool PAGED>
+__global__ void __launch_bounds__(NW * 64)
+topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
+                const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
+                bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
+                float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
+                int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
+                float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages) {
+  extern __shared__ __align__(16) float topk_row_dyn[];
+  topk_row_body<D, GMAX, NW, PAGED>(q, lmks, lse_swa, indices, scores, lse_total_out, sel_logits_out, weights_out, L,
+                                    N, NP, h_kv, G, topk, block_size, window_size, causal, q_offset, sm_scale,
+                                    page_table, max_pages, num_pages, topk_row_dyn, (long)blockIdx.x);
+}
+
+// The remote branch of a decode step in one launch: the workgroup of a (query, KV head) row selects
+// the row's chunks and writes indices, scores and the inter-chunk softmax weights (topk_row_body),
+// then attends over the selected chunks (decode_rows_body) reading back what it has just written
+// (the barrier between the two makes a workgroup's own global writes visible to it).  The rows
+// drift apart, so while some compute units run the selection's tail the others keep the memory
+// system busy, and the step pays one launch.
+#define DS_WAVES 8
+struct DsArgs {
+  const bf16_t *q, *lmks, *k, *v;
+  const float* lse_swa;
+  int32_t* indices;
+  bf16_t *scores, *weights, *o;
+  float *lse_total, *sel_logits;
+  int L, N, NP, h_kv, G, topk, block_size, window_size, q_offset;
+  float sm_scale_sel;
+  const int32_t* page_table;
+  int max_pages, num_pages;
+  DrDims dr;
+};
+template <int D, bool PAGED>
+__global__ void __launch_bounds__(DS_WAVES * 64) decode_step_kernel(DsArgs a) {
+  extern __shared__ __align__(16) float ds_dyn[];
+  const long row = blockIdx.x;
+  topk_row_body<D, 4, DS_WAVES, PAGED>(a.q, a.lmks, a.lse_swa, a.indices, a.scores, a.lse_total, a.sel_logits,
+                                       a.weights, a.L, a.N, a.NP, a.h_kv, a.G, a.topk, a.block_size,
+                                       a.window_size, 1, a.q_offset, a.sm_scale_sel, a.page_table, a.max_pages,
+                                       a.num_pages, ds_dyn, row);
+  __syncthreads();
+  decode_rows_body<D, DS_WAVES>(a.q, a.k, a.v, a.weights, a.indices, a.o, nullptr, a.dr, (char*)ds_dyn, 0,
+                                (int)(row % a.h_kv), row / a.h_kv);
+}
+
 static int topk_cus() { return hils_device_cus(); }
 
 // the one-pass prefill kernel (topk_group.hip)
@@ -1666,6 +1717,95 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, i
   }
 #undef TOPK_ROW_CALL
 #undef TOPK_ROW_CALL_W
+  return HILS_OK;
+}
+
+// ---- the remote branch of a decode step in one launch (decode_step_kernel) ----
+bool hils_decode_rows_covers(int D, int Dv, int G, int K);
+
+extern "C" int hils_decode_step_covers(int B, int L, int N, int HQ, int H, int D, int topk, int block_size) {
+  if (B <= 0 || L <= 0 || H <= 0 || HQ <= 0 || HQ % H != 0 || topk < 1 || topk > TOPK_MAXK || block_size != DR_S)
+    return 0;
+  const int G = HQ / H;
+  return topk_use_row((long)B * L * H, N, G, D, 0, true) && hils_decode_rows_covers(D, D, G, topk) ? 1 : 0;
+}
+
+static int decode_step_launch(const void* q, const void* lmks, const void* k, const void* v, const float* lse_swa,
+                              int32_t* indices, void* scores, void* weights, void* o, float* lse_total,
+                              float* sel_logits, int B, int L, int Lkv, int N, int HQ, int H, int D, int topk,
+                              int block_size, int window_size, int q_offset, float sm_scale_sel,
+                              float sm_scale_attn, int mask_last, const int32_t* page_table, int max_pages,
+                              int num_pages, hipStream_t st) {
+  const int G = HQ / H;
+  const long rows = (long)B * L * H;
+  const int NP = (N + 63) & ~63;
+  const size_t sel_b = (size_t)(page_table ? 6 : 5) * NP * sizeof(float) + (size_t)DS_WAVES * 16 * (2 * D + 16);
+  const size_t att_b = dr_smem_bytes(D, G, DS_WAVES);
+  const size_t smem = sel_b > att_b ? sel_b : att_b;
+  DsArgs a;
+  a.q = (const bf16_t*)q; a.lmks = (const bf16_t*)lmks; a.k = (const bf16_t*)k; a.v = (const bf16_t*)v;
+  a.lse_swa = lse_swa; a.indices = indices;
+  a.scores = (bf16_t*)scores; a.weights = (bf16_t*)weights; a.o = (bf16_t*)o;
+  a.lse_total = lse_total; a.sel_logits = sel_logits;
+  a.L = L; a.N = N; a.NP = NP; a.h_kv = H; a.G = G; a.topk = topk; a.block_size = block_size;
+  a.window_size = window_size; a.q_offset = q_offset; a.sm_scale_sel = sm_scale_sel;
+  a.page_table = page_table; a.max_pages = max_pages; a.num_pages = num_pages;
+  a.dr = DrDims{L, Lkv, HQ, H, G, topk, topk + 1, page_table ? max_pages : Lkv / DR_S, 1, mask_last,
+                sm_scale_attn, page_table, max_pages, num_pages};
+#define DS_CALL(D_, P_)                                                                            \
+  do {                                                                                             \
+    auto kern = decode_step_kernel<D_, P_>;                                                        \
+    static HilsLdsReserve reserved;                                                                \
+    if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_decode_step")) return rc; \
+    hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(DS_WAVES * 64), smem, st, a);              \
+  } while (0)
+  if (page_table) {
+    if (D == 64) DS_CALL(64, true); else DS_CALL(128, true);
+  } else {
+    if (D == 64) DS_CALL(64, false); else DS_CALL(128, false);
+  }
+#undef DS_CALL
+  return HILS_OK;
+}
+
+extern "C" int hils_decode_step(const void* q, const void* lmks, const void* k, const void* v,
+                                const float* lse_swa, int32_t* indices, void* scores, void* weights, void* o,
+                                float* lse_total, float* sel_logits, int B, int L, int Lkv, int N, int HQ, int H,
+                                int D, int topk, int block_size, int window_size, int q_offset,
+                                float sm_scale_sel, float sm_scale_attn, int mask_last, void* stream) {
+  HILS_REQUIRE(q && lmks && k && v && lse_swa && indices && scores && weights && o, "hils_decode_step: null pointer");
+  HILS_REQUIRE(B > 0 && L > 0 && N > 0 && H > 0 && HQ > 0 && HQ % H == 0, "hils_decode_step: bad sizes");
+  HILS_REQUIRE(Lkv >= (long)N * block_size, "hils_decode_step: the cache (%d tokens) is shorter than %d chunks", Lkv, N);
+  HILS_REQUIRE(hils_decode_step_covers(B, L, N, HQ, H, D, topk, block_size),
+               "hils_decode_step: shape not covered (hils_decode_step_covers): use hils_topk_fwd_weights + hils_sparse_attn_fwd");
+  HILS_REQUIRE((long)B * L * H <= 2147483647L, "hils_decode_step: grid too large");
+  if (int rc = decode_step_launch(q, lmks, k, v, lse_swa, indices, scores, weights, o, lse_total, sel_logits, B, L,
+                                  Lkv, N, HQ, H, D, topk, block_size, window_size, q_offset, sm_scale_sel,
+                                  sm_scale_attn, mask_last, nullptr, 0, 0, (hipStream_t)stream))
+    return rc;
+  HILS_CHECK_LAUNCH("hils_decode_step");
+  return HILS_OK;
+}
+
+extern "C" int hils_decode_step_paged(const void* q, const void* lmk_pages, const void* k_pages,
+                                      const void* v_pages, const int32_t* page_table, const float* lse_swa,
+                                      int32_t* indices, void* scores, void* weights, void* o, float* lse_total,
+                                      float* sel_logits, int B, int L, int N, int HQ, int H, int D, int topk,
+                                      int block_size, int window_size, int q_offset, int max_pages, int num_pages,
+                                      float sm_scale_sel, float sm_scale_attn, int mask_last, void* stream) {
+  HILS_REQUIRE(q && lmk_pages && k_pages && v_pages && page_table && lse_swa && indices && scores && weights && o,
+               "hils_decode_step_paged: null pointer");
+  HILS_REQUIRE(B > 0 && L > 0 && N > 0 && H > 0 && HQ > 0 && HQ % H == 0 && max_pages >= N && num_pages > 0,
+               "hils_decode_step_paged: sizes must be positive and the page table must cover N chunks");
+  HILS_REQUIRE(hils_decode_step_covers(B, L, N, HQ, H, D, topk, block_size),
+               "hils_decode_step_paged: shape not covered (hils_decode_step_covers): use hils_topk_fwd_weights_paged + hils_sparse_attn_decode_paged");
+  HILS_REQUIRE((long)B * L * H <= 2147483647L, "hils_decode_step_paged: grid too large");
+  if (int rc = decode_step_launch(q, lmk_pages, k_pages, v_pages, lse_swa, indices, scores, weights, o, lse_total,
+                                  sel_logits, B, L, 0, N, HQ, H, D, topk, block_size, window_size, q_offset,
+                                  sm_scale_sel, sm_scale_attn, mask_last, page_table, max_pages, num_pages,
+                                  (hipStream_t)stream))
+    return rc;
+  HILS_CHECK_LAUNCH("hils_decode_step_paged");
   return HILS_OK;
 }
 

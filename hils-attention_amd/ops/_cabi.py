@@ -27,6 +27,8 @@ SIGNATURES = {
     "hils_topk_fwd_weights": [_P] * 10 + [_I] * 12 + [_F, _P],
     "hils_topk_fwd_weights_paged": [_P] * 9 + [_I] * 12 + [_F, _P],
     "hils_sparse_attn_decode_paged": [_P] * 8 + [_I] * 9 + [_F, _I, _P],
+    "hils_decode_step": [_P] * 11 + [_I] * 11 + [_F, _F, _I, _P],
+    "hils_decode_step_paged": [_P] * 12 + [_I] * 12 + [_F, _F, _I, _P],
     "hils_topk_bwd": [_P] * 7 + [_I] * 8 + [_F, _P],
     "hils_sparse_attn_fwd": [_P] * 10 + [_I] * 13 + [_F, _I, _F, _I, _P],
     "hils_pack_kv_chunks": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
@@ -68,6 +70,8 @@ def load():
     lib.hils_topk_fwd_noalloc_max_workspace.argtypes = []
     lib.hils_sparse_attn_decode_paged_workspace.restype = ctypes.c_size_t
     lib.hils_sparse_attn_decode_paged_workspace.argtypes = [_I] * 6
+    lib.hils_decode_step_covers.restype = c_int
+    lib.hils_decode_step_covers.argtypes = [_I] * 8
     lib.hils_sparse_attn_fwd_workspace.restype = ctypes.c_size_t
     lib.hils_sparse_attn_fwd_workspace.argtypes = [_I] * 11 + [_F]
     lib.hils_topk_bwd_workspace.restype = ctypes.c_size_t

@@ -97,3 +97,52 @@ def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causa
                _cabi.ptr(weights), _cabi.ptr(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),
                int(window_size), int(bool(is_causal)), int(q_offset), 0, scale)
     return indices, scores, weights
+
+
+def decode_step(q, lmks, k, v, lse_swa, topk, block_size, window_size, q_offset=0, sm_scale=None,
+                mask_last_token=True, _debug=None):
+    """Inference: the remote branch of a decode step, ``topk_chunk_weights`` followed by
+    ``HiLS_block_M_head(..., is_training=False)`` on the selected chunks, in one kernel launch (one
+    workgroup per (query, KV head) selects and then attends).  q (B,L,h_q,D), lmks (B,N,h_kv,D), k, v
+    (B,Lkv,h_kv,D) bf16 (k, v may live in pinned host memory), lse_swa (B,L,h_q) -> o (B,L,h_q,D),
+    weights (B,L,h_q,topk+1), indices (B,L,h_kv,topk), scores (B,L,h_q,topk).  Shapes the fused kernel
+    does not take (few rows, short caches, more than four query heads per KV head, ...) run as the
+    two calls."""
+    import math
+    from .hils_fwd_bwd_head import HiLS_block_M_head
+    _cabi.require_gpu_bf16("decode_step", q, lmks)
+    _cabi.require_gpu_bf16("decode_step", k, v, pinned_ok=True)
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, lmks, k, v, lse_swa)):
+        raise RuntimeError("decode_step is forward-only")
+    B, L, h_q, D = q.shape
+    N, h_kv = lmks.shape[1], lmks.shape[2]
+    Lkv = k.shape[1]
+    assert lmks.shape[0] == B and lmks.shape[3] == D and k.shape == v.shape and k.shape[0] == B
+    assert k.shape[2] == h_kv and k.shape[3] == D and h_q % h_kv == 0
+    scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(D)
+    lib = _cabi.load()
+    if not (lib.hils_decode_step_covers(B, L, N, h_q, h_kv, D, int(topk), int(block_size)) and Lkv >= N * block_size):
+        idx, sc, w = topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, q_offset=q_offset,
+                                        sm_scale=scale)
+        o = HiLS_block_M_head(q, k, v, w, idx, block_size=block_size, sm_scale=scale,
+                              mask_last_token=mask_last_token, is_training=False)
+        return o, w, idx, sc
+    dev = q.device
+    G = h_q // h_kv
+    lse = lse_swa.reshape(B, L, h_q).float().contiguous()
+    indices = torch.empty((B, L, h_kv, topk), dtype=torch.int32, device=dev)
+    scores = torch.empty((B, L, h_q, topk), dtype=q.dtype, device=dev)
+    weights = torch.empty((B, L, h_q, topk + 1), dtype=q.dtype, device=dev)
+    o = torch.empty((B, L, h_q, D), dtype=q.dtype, device=dev)
+    lse_total = sel_logits = None
+    if _debug is not None:
+        lse_total = torch.empty((B, L, h_kv, G), dtype=torch.float32, device=dev)
+        sel_logits = torch.full((B, L, h_kv, G, N), float("-inf"), dtype=torch.float32, device=dev)
+    kk, vv = _cabi.gpu_readable(k, dev), _cabi.gpu_readable(v, dev)
+    _cabi.call("hils_decode_step", _cabi.ptr(q.contiguous()), _cabi.ptr(lmks.contiguous()), _cabi.ptr(kk),
+               _cabi.ptr(vv), _cabi.ptr(lse), _cabi.ptr(indices), _cabi.ptr(scores), _cabi.ptr(weights),
+               _cabi.ptr(o), _cabi.ptr(lse_total), _cabi.ptr(sel_logits), B, L, Lkv, N, h_q, h_kv, D, int(topk),
+               int(block_size), int(window_size), int(q_offset), scale, scale, int(bool(mask_last_token)))
+    if _debug is not None:
+        _debug.update(lse_total=lse_total, sel_logits=sel_logits)
+    return o, weights, indices, scores

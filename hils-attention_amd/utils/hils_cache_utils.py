@@ -22,12 +22,12 @@ try:  # imported as part of the package ...
     from ..ops import _cabi
     from ..ops.chunk_attn_pool_tilelang import chunk_attn_pool_tilelang, chunk_mean_pool
     from ..ops.hils_fwd_bwd_head import HiLS_block_M_head
-    from ..ops.hils_glue import topk_chunk_weights
+    from ..ops.hils_glue import decode_step, topk_chunk_weights
 except ImportError:  # ... or with the package directory itself on sys.path (`from utils... import`)
     from ops import _cabi
     from ops.chunk_attn_pool_tilelang import chunk_attn_pool_tilelang, chunk_mean_pool
     from ops.hils_fwd_bwd_head import HiLS_block_M_head
-    from ops.hils_glue import topk_chunk_weights
+    from ops.hils_glue import decode_step, topk_chunk_weights
 
 
 _OFFLOAD_SEQ_THRESHOLD = 128 * 1024
@@ -147,10 +147,9 @@ class HiLSDynamicLayer:
         S = self.chunk_size
         if sm_scale is None:
             sm_scale = 1.0 / math.sqrt(q.shape[-1])
-        idx, _, w = topk_chunk_weights(q, self.lmk_k, lse_swa, topk, S, window_size,
-                                       q_offset=self.seq_len - q.shape[1], sm_scale=sm_scale)
-        o = HiLS_block_M_head(q, self.keys, self.values, w, idx, block_size=S, sm_scale=sm_scale,
-                              is_training=False)
+        # one launch when the shape allows it (decode_step falls back to the two calls otherwise)
+        o, w, idx, _ = decode_step(q, self.lmk_k, self.keys, self.values, lse_swa, topk, S, window_size,
+                                   q_offset=self.seq_len - q.shape[1], sm_scale=sm_scale)
         return o, w, idx
 
 
@@ -279,6 +278,17 @@ def paged_hils_attend(q, k_pages, v_pages, lmk_pages, page_table, lse_swa, seq_l
         lse_total = torch.empty((B, Lq, H, G), dtype=torch.float32, device=dev)
         sel_logits = torch.full((B, Lq, H, G, N), float("-inf"), dtype=torch.float32, device=dev)
     qc = q.contiguous()
+    if _cabi.load().hils_decode_step_covers(B, Lq, N, HQ, H, D, int(topk), S):
+        # selection and attention of a row by one workgroup, one launch
+        o = torch.empty((B, Lq, HQ, D), dtype=q.dtype, device=dev)
+        _cabi.call("hils_decode_step_paged", _cabi.ptr(qc), _cabi.ptr(lmk_pages), _cabi.ptr(k_pages),
+                   _cabi.ptr(v_pages), _cabi.ptr(page_table), _cabi.ptr(lse), _cabi.ptr(indices), _cabi.ptr(scores),
+                   _cabi.ptr(weights), _cabi.ptr(o), _cabi.ptr(lse_total), _cabi.ptr(sel_logits), B, Lq, N, HQ, H, D,
+                   int(topk), S, int(window_size), seq_len - Lq, max_pages, num_pages, float(sm_scale),
+                   float(sm_scale), 1)
+        if _debug is not None:
+            _debug.update(lse_total=lse_total, sel_logits=sel_logits, scores=scores)
+        return o, weights, indices
     _cabi.call("hils_topk_fwd_weights_paged", _cabi.ptr(qc), _cabi.ptr(lmk_pages), _cabi.ptr(page_table),
                _cabi.ptr(lse), _cabi.ptr(indices), _cabi.ptr(scores), _cabi.ptr(weights), _cabi.ptr(lse_total),
                _cabi.ptr(sel_logits), B, Lq, N, H, G, D, int(topk), S, int(window_size), seq_len - Lq,

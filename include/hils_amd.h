@@ -247,6 +247,33 @@ int hils_sparse_attn_decode_paged(const void* q, const void* k_pages, const void
                                   int NW, int max_pages, int num_pages, float sm_scale, int mask_last,
                                   void* stream);
 
+/* ---- the remote branch of a decode step in one launch ---------------------------------- */
+
+/* hils_topk_fwd_weights followed by the decode path of hils_sparse_attn_fwd (contiguous cache) or
+ * hils_topk_fwd_weights_paged followed by hils_sparse_attn_decode_paged (paged cache), fused: what
+ * the layer runs per generated token between the local branch and the merge
+ * (models/FlashHiLS/hils_attention.py:568-623 on the cached keys of utils/hils_cache_utils.py:34-62).
+ * One workgroup per (query, KV head) row selects the row's chunks, writes indices / scores / weights
+ * and then attends over the chunks it has selected: one launch instead of two, and the rows'
+ * selection tails overlap other rows' memory streams.  Outputs as the two calls give them; o
+ * (B,L,HQ,D) bf16 is the remote branch's output (the caller adds swa_o * weights[..., topk]).
+ * lse_total / sel_logits optional as in hils_topk_fwd.  q (B,L,HQ,D); lmks (B,N,H,D) or lmk_pages;
+ * k, v (B,Lkv,H,D) with Lkv >= N * 64 or k_pages, v_pages (num_pages,H,64,D).
+ * Covered shapes (hils_decode_step_covers returns 1): shared chunk keys, causal, block_size 64,
+ * D = Dv in {64, 128}, HQ/H <= 4, 256 <= N <= 4096, topk <= 64, at least 96 rows B*L*H. */
+int hils_decode_step_covers(int B, int L, int N, int HQ, int H, int D, int topk, int block_size);
+int hils_decode_step(const void* q, const void* lmks, const void* k, const void* v, const float* lse_swa,
+                     int32_t* indices, void* scores, void* weights, void* o, float* lse_total,
+                     float* sel_logits, int B, int L, int Lkv, int N, int HQ, int H, int D, int topk,
+                     int block_size, int window_size, int q_offset, float sm_scale_sel,
+                     float sm_scale_attn, int mask_last, void* stream);
+int hils_decode_step_paged(const void* q, const void* lmk_pages, const void* k_pages, const void* v_pages,
+                           const int32_t* page_table, const float* lse_swa, int32_t* indices, void* scores,
+                           void* weights, void* o, float* lse_total, float* sel_logits, int B, int L, int N,
+                           int HQ, int H, int D, int topk, int block_size, int window_size, int q_offset,
+                           int max_pages, int num_pages, float sm_scale_sel, float sm_scale_attn,
+                           int mask_last, void* stream);
+
 /* ---- exact per-chunk log Z ---------------------------------------------------- */
 
 /* Forward.  Replaces exact_chunk_log_z_fwd (ops/exact_chunk_log_z_tilelang.py:25-137).

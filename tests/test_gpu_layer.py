@@ -149,3 +149,36 @@ def test_decode_step_replays_as_hip_graph(pkg, orc, dev):
     # and the eager result itself against the oracle
     ref = orc.sparse_attn(q.cpu(), kc.cpu(), vc.cpu(), e_w.cpu(), e_idx.cpu(), chunk_size=S)
     assert_close_bf16(e_o, ref, "decode step output")
+
+
+@pytest.mark.parametrize("B,Lq,Lkv,HQ,H,D,K", [(32, 1, 32768, 32, 8, 128, 32), (16, 1, 16512, 8, 8, 64, 16),
+                                               (50, 2, 20480, 4, 1, 128, 8), (24, 1, 65536, 12, 4, 64, 64),
+                                               # not taken by the one-launch kernel (few rows): the two calls
+                                               (2, 1, 4096, 8, 2, 128, 16)])
+def test_decode_step_one_launch(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
+    """decode_step (selection + inter-chunk softmax + attention of a row by one workgroup) against the
+    two separate calls and against the oracle."""
+    note(f"decode_step B{B} Lq{Lq} Lkv{Lkv} HQ{HQ} H{H} D{D} K{K}")
+    gen = torch.Generator().manual_seed(81)
+    q = torch.randn(B, Lq, HQ, D, generator=gen).bfloat16()
+    k = torch.randn(B, Lkv, H, D, generator=gen).bfloat16()
+    v = torch.randn(B, Lkv, H, D, generator=gen).bfloat16()
+    lse = torch.randn(B, Lq, HQ, generator=gen) * 3 + 5
+    qd, kd, vd, lsed = q.to(dev), k.to(dev), v.to(dev), lse.to(dev)
+    N = Lkv // 64
+    lmk = pkg.chunk_mean_pool(kd[:, : N * 64].contiguous(), 64)
+    dbg = {}
+    o1, w1, idx1, sc1 = pkg.decode_step(qd, lmk, kd, vd, lsed, K, 64, 1, q_offset=Lkv - Lq, _debug=dbg)
+    idx0, sc0, w0 = pkg.topk_chunk_weights(qd, lmk, lsed, K, 64, 1, q_offset=Lkv - Lq)
+    o0 = pkg.HiLS_block_M_head(qd, kd, vd, w0, idx0, block_size=64, is_training=False)
+    assert torch.equal(idx1, idx0) and torch.equal(sc1, sc0) and torch.equal(w1, w0)
+    assert_close_bf16(o1, o0.float(), "one launch vs two calls")
+    if dbg:  # the one-launch kernel ran: selection rule on its own logits
+        lim = orc.causal_chunk_limit(Lq, Lkv - Lq, 1, 64)
+        want = orc.topk_select(dbg["sel_logits"].cpu(), dbg["lse_total"].cpu(), lim, K)
+        assert torch.equal(idx1.cpu(), want)
+    ref = orc.sparse_attn(q, k, v, w1.cpu(), idx1.cpu(), chunk_size=64)
+    assert_close_bf16(o1, ref, "decode_step output")
+    # twice the same call: bit-identical (the selection's log-sum-exp is summed in a fixed order)
+    o2, w2, idx2, sc2 = pkg.decode_step(qd, lmk, kd, vd, lsed, K, 64, 1, q_offset=Lkv - Lq)
+    assert torch.equal(o2, o1) and torch.equal(idx2, idx1) and torch.equal(w2, w1)

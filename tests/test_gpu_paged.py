@@ -40,13 +40,13 @@ def test_paged_decode_matches_contiguous(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K)
     lse = torch.randn(B, Lq, HQ, generator=gen) * 3 + 5
     qd, kd, vd, lsed = q.to(dev), k.to(dev), v.to(dev), lse.to(dev)
     lmk = pkg.chunk_mean_pool(kd, 64)
-    idx0, sc0, w0 = pkg.topk_chunk_weights(qd, lmk, lsed, K, 64, 1, q_offset=Lkv - Lq)
-    o0 = pkg.HiLS_block_M_head(qd, kd, vd, w0, idx0, block_size=64, is_training=False)
+    # the token-major cache through the same route (one launch where the shape allows it, else two calls)
+    o0, w0, idx0, sc0 = pkg.decode_step(qd, lmk, kd, vd, lsed, K, 64, 1, q_offset=Lkv - Lq)
     k_pages, v_pages, lmk_pages, table = _paged_copy(k, v, lmk.cpu(), dev, seed=72)
     dbg = {}
     o1, w1, idx1 = pkg.paged_hils_attend(qd, k_pages, v_pages, lmk_pages, table, lsed, Lkv, K, 1, _debug=dbg)
     assert torch.equal(idx1, idx0), "indices differ between the paged and the token-major cache"
-    same_kernels = Lkv // 64 >= 256 and B * Lq * H >= 96  # both calls on the one-workgroup-per-row kernel
+    same_kernels = Lkv // 64 >= 256 and B * Lq * H >= 96  # both on the one-launch kernel
     if same_kernels:
         assert torch.equal(dbg["scores"], sc0) and torch.equal(w1, w0)
         assert torch.equal(o1, o0), "attention output differs between the paged and the token-major cache"
