@@ -2,12 +2,12 @@
 // the start of the chunk that holds (query - window + 1) up to itself (or from query - window + 1
 // exactly), optionally without the landmark key of every chunk; outputs o and the natural-log LSE.
 //
-// A workgroup of four wavefronts owns 128/G consecutive queries of one KV head (32 score rows per
-// wavefront: query x head of the group, held as matrix B operands).  The keys and values of the
-// window stream through LDS in 64-token tiles: K row-major (A operand of the transposed scores
-// K Q^T), V transposed (B operand of O += P V, whose contraction runs over the tokens).  With the
-// rows as matrix columns a row's 64 scores lie in 16 registers of 4 lanes (in-lane softmax plus
-// one row-swap reduction) and the probabilities are already the A operand of the second product.
+// A wavefront owns 32 score rows (query x head of the group), held as matrix B operands; the keys
+// and values of the window pass through LDS in 64-token tiles: K row-major (A operand of the
+// transposed scores K Q^T), V as the B operand of O += P V, whose contraction runs over the tokens.
+// With the rows as matrix columns a row's 64 scores lie in 16 registers of 4 lanes (in-lane softmax
+// plus one row-swap reduction) and the probabilities are already the A operand of the second product.
+#include <type_traits>
 #include "stream_tiles.h"
 #include "../../include/hils_amd.h"
 
@@ -18,26 +18,59 @@ struct SwaDims {
   float sm_scale;
 };
 
-template <int D, int DV, int G, int RT>
-__global__ void __launch_bounds__(256, (RT == 1 ? 3 : 2))
-swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
-             bf16_t* __restrict__ o, float* __restrict__ lse, SwaDims dm, int n_qt) {
+// Forward.  A workgroup of eight wavefronts owns 256/G consecutive queries of one KV head: 32 score
+// rows (query x head of the group) per wavefront, held as matrix B operands.  The keys and values the
+// block can see (its queries' windows: two or three 64-token tiles at window 64) are loaded once, all
+// loads in flight together, and stay in LDS row-major (rows padded by 16 bytes); a longer window is
+// worked through in phases of SWA_RES tiles.  S^T = K Q^T takes K rows as A operands, O += P V takes V
+// through the transposing LDS load, in the token order in which the S^T accumulators hold P.  A
+// wavefront skips the tiles none of its rows can see and masks only the tiles that straddle a row's
+// window start, its diagonal, the end of the keys or a landmark; running max / sum per row as in
+// flash attention.
+#define SWA_RES 4      // tiles resident in LDS
+#define SWA_FWD_RT 2   // 16-row tiles per wavefront
+#define SWA_FWD_WAVES 8
+
+template <int D, int DV>
+static size_t swa_fwd_smem() {
+  const size_t tiles = (size_t)SWA_RES * 64 * ((2 * D + 16) + (2 * DV + 16));
+  const size_t outs = (size_t)SWA_FWD_WAVES * 16 * SWA_FWD_RT * (2 * DV + 16);
+  return (tiles > outs ? tiles : outs) + (size_t)SWA_FWD_WAVES * SWA_FWD_RT * 16 * sizeof(float);
+}
+
+template <int D, int DV, int G>
+__global__ void __launch_bounds__(SWA_FWD_WAVES * 64)
+swa_fwd_blk(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+            bf16_t* __restrict__ o, float* __restrict__ lse, SwaDims dm, int n_qt) {
+  constexpr int RT = SWA_FWD_RT, NWV = SWA_FWD_WAVES, NT = NWV * 64;
   constexpr int KS = D / 32, DT = DV / 16;
-  constexpr int QW = 16 * RT / G, QB = 4 * QW;
-  constexpr int PITCH = D * 2 + 16;
-  constexpr int KSEG = D / 8, KPASS = 64 * KSEG / 256;        // K tile: 16-byte pieces per thread
-  constexpr int VSEG = DV / 8, VPPP = 256 / VSEG, VPASS = 32 / VPPP;  // V tile: row pairs per pass
+  constexpr int QW = 16 * RT / G > 0 ? 16 * RT / G : 1;  // queries per wavefront (G <= 16: >= 2)
+  constexpr int QB = NWV * 16 * RT / G;                  // queries per workgroup
+  constexpr int KP = D * 2 + 16, VP = DV * 2 + 16;       // bytes per staged row
+  constexpr int KSEG = D / 8, VSEG = DV / 8;
+  constexpr int KPT = 64 * KSEG / NT, VPT = 64 * VSEG / NT;  // 16-byte pieces per thread and tile
+  static_assert(KPT >= 1 && VPT >= 1 && KPT * NT == 64 * KSEG && VPT * NT == 64 * VSEG,
+                "every thread stages whole pieces of a tile");
+  constexpr int TILE_B = 64 * KP + 64 * VP;
   constexpr int OP = DV * 2 + 16;  // bytes per staged output row
-  constexpr int KBYTES = 64 * PITCH > 64 * RT * OP ? 64 * PITCH : 64 * RT * OP;
-  __shared__ __align__(16) unsigned char k_s[KBYTES];  // K tile; the output tile at the end
-  __shared__ __align__(16) unsigned char vt_s[DV * LZM_PT];
-  __shared__ __align__(16) float bc_s[4][RT][16];  // per wavefront: per-row factors, transposed read
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  typedef unsigned swa_u32x4 __attribute__((ext_vector_type(4)));
+  typedef short swa_s4 __attribute__((ext_vector_type(4)));
+  typedef short swa_s8 __attribute__((ext_vector_type(8)));
+  extern __shared__ __align__(16) unsigned char swa_dyn[];
+  constexpr size_t TILES_B = (size_t)SWA_RES * TILE_B;
+  constexpr size_t OUTS_B = (size_t)NWV * 16 * RT * OP;
+  float* bc_all = (float*)(swa_dyn + (TILES_B > OUTS_B ? TILES_B : OUTS_B));  // [wave][rt][16] row factors
+  const int tid = threadIdx.x, lane = tid & 63;
+  // in a scalar register: what is derived from it (the wavefront's key range, "does this tile need
+  // masks") then steers scalar branches instead of lane masks
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, j = lane >> 4;
+  float* bc_s = bc_all + wave * RT * 16;
   const int qt = n_qt - 1 - (int)blockIdx.x;
   const int hk = blockIdx.y;
   const long b = blockIdx.z;
-  const int t0 = qt * QB + wave * QW;
+  const int tq0 = qt * QB;
+  const int t0 = tq0 + wave * QW;
   const int q_off = dm.kv_start + dm.Lk - dm.Lq;  // absolute position of query 0
 
   bf16x8_t qa[RT][KS];
@@ -54,64 +87,47 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qa[rt][ks] = *(const bf16x8_t*)(qp + ks * 32);
   }
-  // key range of the workgroup (raw indices into k / v)
+  // visible key positions of this lane's rows as [vlo, vlo + vspan]; a row that sees nothing gets a
+  // start no position reaches
+  int vlo[RT];
+  unsigned vspan[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int last = dm.kv_start + dm.Lk - 1;
+    const int hi = qabs[rt] < last ? qabs[rt] : last;
+    const bool some = hi >= cstart[rt];
+    vlo[rt] = some ? cstart[rt] : 0x7fffffff;
+    vspan[rt] = some ? (unsigned)(hi - cstart[rt]) : 0u;
+  }
+  auto win_lo = [&](int t) -> int {  // first raw key index query t can see (may be negative)
+    const int left = q_off + t - dm.window + 1;
+    return (dm.expand ? floordiv(left, dm.chunk) * dm.chunk : left) - dm.kv_start;
+  };
+  // key range of the workgroup and of this wavefront (raw indices into k / v)
   int tile_lo, tile_hi;
   {
-    const int tq0 = qt * QB;
     int tq1 = tq0 + QB - 1;
     if (tq1 > dm.Lq - 1) tq1 = dm.Lq - 1;
-    const int left_abs = q_off + tq0 - dm.window + 1;
-    int lo = (dm.expand ? floordiv(left_abs, dm.chunk) * dm.chunk : left_abs) - dm.kv_start;
-    int hi = q_off + tq1 - dm.kv_start + 1;
+    int lo = win_lo(tq0), hi = q_off + tq1 - dm.kv_start + 1;
     lo = lo < 0 ? 0 : lo;
     hi = hi > dm.Lk ? dm.Lk : hi;
     tile_lo = lo / 64;
     tile_hi = (hi + 63) / 64;  // may be <= tile_lo: nothing visible
   }
+  int w_lo, w_hi, w_in_lo, w_in_hi;  // the wavefront's visible range and the part of it no row masks
+  {
+    const int ta = t0 < dm.Lq ? t0 : dm.Lq - 1;
+    int tb = t0 + (16 * RT - 1) / G;
+    tb = tb < dm.Lq ? tb : dm.Lq - 1;
+    w_lo = win_lo(ta);
+    w_hi = q_off + tb - dm.kv_start + 1;
+    w_in_lo = win_lo(tb);                     // every row sees keys from here ...
+    w_in_hi = q_off + ta - dm.kv_start + 1;   // ... up to (excluding) here
+    if (w_in_hi > dm.Lk) w_in_hi = dm.Lk;
+    if (t0 >= dm.Lq) w_hi = w_lo;             // a wavefront of dead rows
+  }
   const float c2 = dm.sm_scale * HILS_LOG2E;
 
-  // Prefetch registers: a native vector type (an array of HIP's uint4 struct that lives across
-  // the loop's back edge is kept in scratch memory) and loads without a branch around them (a
-  // load inside a branch is waited for at once).  Tokens past the end read the last row: their
-  // scores are masked and their probabilities are 0.
-  typedef unsigned swa_u32x4 __attribute__((ext_vector_type(4)));
-  swa_u32x4 kr[KPASS], vr[VPASS][2];
-  auto fetch = [&](int tile) {
-#pragma unroll
-    for (int i = 0; i < KPASS; ++i) {
-      const int p = tid + 256 * i;
-      int tok = tile * 64 + p / KSEG;
-      const int seg = p % KSEG;
-      tok = tok < dm.Lk ? tok : dm.Lk - 1;
-      kr[i] = *(const swa_u32x4*)(k + ((b * dm.Lk + tok) * (long)dm.H + hk) * D + seg * 8);
-    }
-#pragma unroll
-    for (int i = 0; i < VPASS; ++i)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        int tok = tile * 64 + 2 * (tid / VSEG + VPPP * i) + h;
-        tok = tok < dm.Lk ? tok : dm.Lk - 1;
-        vr[i][h] = *(const swa_u32x4*)(v + ((b * dm.Lk + tok) * (long)dm.H + hk) * DV + (tid % VSEG) * 8);
-      }
-  };
-  auto stash = [&]() {
-#pragma unroll
-    for (int i = 0; i < KPASS; ++i) {
-      const int p = tid + 256 * i;
-      *(swa_u32x4*)(k_s + (p / KSEG) * PITCH + (p % KSEG) * 16) = kr[i];
-    }
-#pragma unroll
-    for (int i = 0; i < VPASS; ++i) {
-      const int row0 = 2 * (tid / VSEG + VPPP * i), seg = tid % VSEG;
-      const uint32_t aw[4] = {vr[i][0].x, vr[i][0].y, vr[i][0].z, vr[i][0].w};
-      const uint32_t bw[4] = {vr[i][1].x, vr[i][1].y, vr[i][1].z, vr[i][1].w};
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        *(uint32_t*)(vt_s + (seg * 8 + 2 * w) * LZM_PT + row0 * 2) = __builtin_amdgcn_perm(bw[w], aw[w], 0x05040100u);
-        *(uint32_t*)(vt_s + (seg * 8 + 2 * w + 1) * LZM_PT + row0 * 2) = __builtin_amdgcn_perm(bw[w], aw[w], 0x07060302u);
-      }
-    }
-  };
   f32x4_t acc[RT][DT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
@@ -123,58 +139,64 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
     m_run[rt] = HILS_NEG_INF;
     l_run[rt] = 0.f;
   }
-  if (tile_lo < tile_hi) {
-    fetch(tile_lo);
-    stash();
-  }
-  __syncthreads();
-  for (int tile = tile_lo; tile < tile_hi; ++tile) {
-    fetch(tile + 1 < tile_hi ? tile + 1 : tile);
-    float p[RT][4][4];
+
+  // one resident tile: scores, masks where a row needs them, running softmax, O += P V
+  auto tile_step = [&](int tile, const unsigned char* k_s, const unsigned char* v_s) __attribute__((always_inline)) {
+    f32x4_t p[RT][4];  // scores, then probabilities: accumulator tiles (token tt*16 + 4j + i, row lane & 15)
     {
-      f32x4_t st[RT][4];
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) st[rt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int tt = 0; tt < 4; ++tt) p[rt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8_t a = *(const bf16x8_t*)(k_s + (tt * 16 + col) * PITCH + ks * 64 + j * 16);
+          const bf16x8_t a = *(const bf16x8_t*)(k_s + (tt * 16 + col) * KP + ks * 64 + j * 16);
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt)
-            st[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qa[rt][ks], st[rt][tt], 0, 0, 0);
+            p[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qa[rt][ks], p[rt][tt], 0, 0, 0);
+          // (keeps the operand reads of later steps from being hoisted here: registers)
+          if (ks == KS - 1 && (tt & 1)) __builtin_amdgcn_sched_barrier(0);
         }
-      // visibility of this lane's 16 tokens: bit tt*4+i; the landmark test does not depend on the row
-      unsigned lmk_ok = 0xffffu;
-      if (dm.mask_lmk) {
-        lmk_ok = 0u;
+      const bool inner = !dm.mask_lmk && tile * 64 >= w_in_lo && tile * 64 + 64 <= w_in_hi;  // uniform
+      if (!inner) {
+        // visibility of this lane's 16 tokens: bit tt*4+i; the landmark test does not depend on the row
+        unsigned lmk_ok = 0xffffu;
+        if (dm.mask_lmk) {
+          lmk_ok = 0u;
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt)
+          for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int ta = dm.kv_start + tile * 64 + tt * 16 + 4 * j + i + 1;
-            const bool lm = dm.chunk_pow2 ? ((ta & (dm.chunk - 1)) == 0) : (ta % dm.chunk == 0);
-            lmk_ok |= lm ? 0u : (1u << (tt * 4 + i));
-          }
+            for (int i = 0; i < 4; ++i) {
+              const int ta = dm.kv_start + tile * 64 + tt * 16 + 4 * j + i + 1;
+              const bool lm = dm.chunk_pow2 ? ((ta & (dm.chunk - 1)) == 0) : (ta % dm.chunk == 0);
+              lmk_ok |= lm ? 0u : (1u << (tt * 4 + i));
+            }
+        }
+        // a token at absolute position ta is visible to a row iff vlo <= ta <= vhi (window start, the
+        // query itself or the last key): one unsigned compare of ta - vlo against vhi - vlo, no branches
+        const int tok_abs0 = dm.kv_start + tile * 64 + 4 * j;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          const unsigned base = (unsigned)(tok_abs0 - vlo[rt]);
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              bool vis = base + (unsigned)(tt * 16 + i) <= vspan[rt];
+              if (dm.mask_lmk) vis = vis & (((lmk_ok >> (tt * 4 + i)) & 1u) != 0u);
+              p[rt][tt][i] = vis ? p[rt][tt][i] : HILS_NEG_INF;
+            }
+        }
       }
-      const int tok_abs0 = dm.kv_start + tile * 64 + 4 * j;
-      const int raw_left = dm.Lk - tile * 64 - 4 * j;  // tokens tt*16+i < raw_left exist
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
         float mx = HILS_NEG_INF;
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int ta = tok_abs0 + tt * 16 + i;
-            const bool vis = ta >= cstart[rt] && ta <= qabs[rt] && (tt * 16 + i) < raw_left &&
-                             ((lmk_ok >> (tt * 4 + i)) & 1u);
-            const float sv = vis ? st[rt][tt][i] : HILS_NEG_INF;
-            p[rt][tt][i] = sv;
-            mx = fmaxf(mx, sv);
-          }
+          for (int i = 0; i < 4; ++i) mx = fmaxf(mx, p[rt][tt][i]);
         mx = rows_max(mx);
         const float m_new = fmaxf(m_run[rt], mx);
         const bool any = m_new > HILS_NEG_INF;
@@ -185,48 +207,135 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float e = __builtin_amdgcn_exp2f(p[rt][tt][i] * c2 - mc);  // masked: exp2(-inf) = 0
+            const float e = __builtin_amdgcn_exp2f(fmaf(p[rt][tt][i], c2, -mc));  // masked: exp2(-inf) = 0
             p[rt][tt][i] = e;
             sum += e;
           }
         sum = rows_sum(sum);
         l_run[rt] = l_run[rt] * corr + sum;
         m_run[rt] = m_new;
-        if (j == 0) bc_s[wave][rt][col] = corr;
+        if (j == 0) bc_s[rt * 16 + col] = corr;
       }
     }
+    __builtin_amdgcn_wave_barrier();
     // rescale the output accumulators: their rows are 4j+i, the factors live per lane & 15
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      const float4 c4 = *(const float4*)&bc_s[wave][rt][4 * j];
+      const float4 c4 = *(const float4*)&bc_s[rt * 16 + 4 * j];
       const float cf[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[rt][dt][i] *= cf[i];
     }
-    lzm_grad_product<DV, RT>(vt_s, p, acc, col, j);
+    __builtin_amdgcn_wave_barrier();
+    // O += P V: a lane's eight k-slots are tokens 4j..4j+3 of two neighbouring 16-token tiles; the
+    // transposing load (a 16-lane group addresses a 4 x 16 block, lane l row l/4 and columns 4(l%4)..,
+    // and receives column l of it) delivers V in that order
+    const unsigned char* t_addr = v_s + (4 * j + (col >> 2)) * VP + (col & 3) * 8;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      bf16x8_t a[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        swa_u32x4 u;
+        u.x = pack_bf2(p[rt][2 * h][0], p[rt][2 * h][1]);
+        u.y = pack_bf2(p[rt][2 * h][2], p[rt][2 * h][3]);
+        u.z = pack_bf2(p[rt][2 * h + 1][0], p[rt][2 * h + 1][1]);
+        u.w = pack_bf2(p[rt][2 * h + 1][2], p[rt][2 * h + 1][3]);
+        a[rt] = __builtin_bit_cast(bf16x8_t, u);
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const unsigned char* p0 = t_addr + (2 * h * 16) * VP + dt * 32;
+        const swa_s4 b0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) swa_s4*)p0);
+        const swa_s4 b1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) swa_s4*)(p0 + 16 * VP));
+        const swa_s8 bb = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          acc[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt], __builtin_bit_cast(bf16x8_t, bb), acc[rt][dt], 0, 0, 0);
+        if ((dt & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+
+  // loads of a phase of N resident tiles, two tiles in flight (tokens past the end read the last row:
+  // their scores are masked); one copy of the code per N, so no load is conditional
+  auto phase = [&](int tile0, auto n_const) __attribute__((always_inline)) {
+    constexpr int N = decltype(n_const)::value;
+    swa_u32x4 kr[2][KPT], vr[2][VPT];  // two tiles' loads in flight
+    auto issue = [&](int ti, swa_u32x4 (&kd)[KPT], swa_u32x4 (&vd)[VPT]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < KPT; ++i) {
+        const int pc = tid + NT * i;
+        int tok = (tile0 + ti) * 64 + pc / KSEG;
+        tok = tok < dm.Lk ? tok : dm.Lk - 1;
+        kd[i] = *(const swa_u32x4*)(k + ((b * dm.Lk + tok) * (long)dm.H + hk) * D + (pc % KSEG) * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        const int pc = tid + NT * i;
+        int tok = (tile0 + ti) * 64 + pc / VSEG;
+        tok = tok < dm.Lk ? tok : dm.Lk - 1;
+        vd[i] = *(const swa_u32x4*)(v + ((b * dm.Lk + tok) * (long)dm.H + hk) * DV + (pc % VSEG) * 8);
+      }
+    };
+    auto stash = [&](int ti, const swa_u32x4 (&kd)[KPT], const swa_u32x4 (&vd)[VPT]) __attribute__((always_inline)) {
+      unsigned char* k_s = swa_dyn + (size_t)ti * TILE_B;
+      unsigned char* v_s = k_s + 64 * KP;
+#pragma unroll
+      for (int i = 0; i < KPT; ++i) {
+        const int pc = tid + NT * i;
+        *(swa_u32x4*)(k_s + (pc / KSEG) * KP + (pc % KSEG) * 16) = kd[i];
+      }
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        const int pc = tid + NT * i;
+        *(swa_u32x4*)(v_s + (pc / VSEG) * VP + (pc % VSEG) * 16) = vd[i];
+      }
+    };
+    issue(0, kr[0], vr[0]);
+    if (N > 1) issue(1, kr[1], vr[1]);
+#pragma unroll
+    for (int ti = 0; ti < N; ++ti) {
+      stash(ti, kr[ti & 1], vr[ti & 1]);
+      if (ti + 2 < N) issue(ti + 2, kr[ti & 1], vr[ti & 1]);
+    }
+  };
+  for (int tile0 = tile_lo; tile0 < tile_hi; tile0 += SWA_RES) {
+    if (tile0 != tile_lo) __syncthreads();  // the previous phase's tiles are no longer read
+    const int n = tile_hi - tile0 < SWA_RES ? tile_hi - tile0 : SWA_RES;
+    if (SWA_RES >= 4 && n == 4) phase(tile0, std::integral_constant<int, SWA_RES >= 4 ? 4 : 1>{});
+    else if (SWA_RES >= 3 && n == 3) phase(tile0, std::integral_constant<int, SWA_RES >= 3 ? 3 : 1>{});
+    else if (n == 2) phase(tile0, std::integral_constant<int, 2>{});
+    else phase(tile0, std::integral_constant<int, 1>{});
     __syncthreads();
-    stash();
-    __syncthreads();
+    for (int ti = 0; ti < n; ++ti) {  // one copy of the tile code
+      const int tile = tile0 + ti;
+      if (tile * 64 < w_hi && tile * 64 + 64 > w_lo) {  // uniform: some row of the wavefront sees the tile
+        const unsigned char* k_s = swa_dyn + (size_t)ti * TILE_B;
+        tile_step(tile, k_s, k_s + 64 * KP);
+      }
+    }
   }
   // ---- finalize: o = acc / l, lse = ln(l) + max * scale ----
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const float inv = l_run[rt] > 0.f ? 1.f / l_run[rt] : 0.f;
-    if (j == 0) bc_s[wave][rt][col] = inv;
+    if (j == 0) bc_s[rt * 16 + col] = inv;
     const int row = rt * 16 + col;
     const int t = t0 + row / G, g = row % G;
     if (j == 0 && t < dm.Lq)
       lse[(b * dm.Lq + t) * (long)dm.HQ + hk * G + g] =
           l_run[rt] > 0.f ? (m_run[rt] * c2 + __builtin_amdgcn_logf(l_run[rt])) * HILS_LN2 : HILS_NEG_INF;
   }
-  // the loop's last barrier has passed: the K buffer is free.  Each wavefront parks its normalised
-  // rows there as bf16 and writes them out as 16-byte pieces (a query's heads are contiguous).
-  unsigned char* ob = k_s + wave * (16 * RT) * OP;
+  __syncthreads();  // every wavefront is through with the tiles: their LDS becomes the output stage
+  // Each wavefront parks its normalised rows as bf16 and writes them out as 16-byte pieces (a query's
+  // heads are contiguous).
+  unsigned char* ob = swa_dyn + (size_t)wave * (16 * RT) * OP;
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const float4 c4 = *(const float4*)&bc_s[wave][rt][4 * j];
+    const float4 c4 = *(const float4*)&bc_s[rt * 16 + 4 * j];
     const float cf[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -237,8 +346,8 @@ swa_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const b
   __builtin_amdgcn_wave_barrier();
   constexpr int OSEG = DV / 8;
 #pragma unroll
-  for (int p = 0; p < 16 * RT * OSEG / 64; ++p) {
-    const int pc = p * 64 + lane;
+  for (int pp = 0; pp < 16 * RT * OSEG / 64; ++pp) {
+    const int pc = pp * 64 + lane;
     const int row = pc / OSEG, seg = pc % OSEG;
     const int t = t0 + row / G, g = row % G;
     if (t < dm.Lq)
@@ -416,7 +525,7 @@ swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, cons
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int ta = tok0 + tt * 16 + i;
-            const bool vis = ta >= cstart[rt] && ta <= qabs[rt] && ((lmk_ok >> (tt * 4 + i)) & 1u);
+            const bool vis = (ta >= cstart[rt]) & (ta <= qabs[rt]) & (((lmk_ok >> (tt * 4 + i)) & 1u) != 0u);  // no short circuit: no branches
             const float pv = vis ? __builtin_amdgcn_exp2f(st[rt][tt][i] * c2 - lse2[rt]) : 0.f;
             ds[rt][tt][i] = pv * (dp[rt][tt][i] - delta[rt]) * dm.sm_scale;
           }
@@ -593,7 +702,7 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
 #pragma unroll
           for (int tt = 0; tt < 2; ++tt) {
             const int tok = tok_w + tt * 16 + col;
-            const bool vis = tok >= cs[i] && tok <= t && ((lmk_ok >> tt) & 1u);
+            const bool vis = (tok >= cs[i]) & (tok <= t) & (((lmk_ok >> tt) & 1u) != 0u);  // no short circuit: no branches
             const float pv = vis ? __builtin_amdgcn_exp2f(st[tt][rr][i] * c2 - ls[i]) : 0.f;
             p[tt][rr][i] = pv;
             ds[tt][rr][i] = pv * (dp[tt][rr][i] - dl[i]) * dm.sm_scale;
@@ -622,22 +731,27 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     }
 }
 
-// rows per wavefront of the forward kernel: 16 * SWA_FWD_RT(D, DV)
-#define SWA_FWD_RT(D_, DV_) (((D_) + (DV_) > 128) ? 1 : 2)
+template <int D, int DV, int G>
+static int swa_fwd_launch(dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* k, const bf16_t* v,
+                          bf16_t* o, float* lse, const SwaDims& dm, int n_qt) {
+  const size_t smem = swa_fwd_smem<D, DV>();
+  auto kern = swa_fwd_blk<D, DV, G>;
+  static HilsLdsReserve reserved;  // per instantiation
+  if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_swa_fwd")) return rc;
+  hipLaunchKernelGGL(kern, grid, dim3(SWA_FWD_WAVES * 64), smem, st, q, k, v, o, lse, dm, n_qt);
+  return HILS_OK;
+}
+
 template <int D, int DV>
-static void swa_launch_g(int G, dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* k,
-                         const bf16_t* v, bf16_t* o, float* lse, const SwaDims& dm, int n_qt) {
-#define SWA_CALL(G_)                                                                             \
-  hipLaunchKernelGGL((swa_fwd_mfma<D, DV, G_, SWA_FWD_RT(D, DV)>), grid, dim3(256), 0, st, q, k, v, \
-                     o, lse, dm, n_qt)
+static int swa_launch_g(int G, dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* k,
+                        const bf16_t* v, bf16_t* o, float* lse, const SwaDims& dm, int n_qt) {
   switch (G) {
-    case 1: SWA_CALL(1); break;
-    case 2: SWA_CALL(2); break;
-    case 4: SWA_CALL(4); break;
-    case 8: SWA_CALL(8); break;
-    default: SWA_CALL(16); break;
+    case 1: return swa_fwd_launch<D, DV, 1>(grid, st, q, k, v, o, lse, dm, n_qt);
+    case 2: return swa_fwd_launch<D, DV, 2>(grid, st, q, k, v, o, lse, dm, n_qt);
+    case 4: return swa_fwd_launch<D, DV, 4>(grid, st, q, k, v, o, lse, dm, n_qt);
+    case 8: return swa_fwd_launch<D, DV, 8>(grid, st, q, k, v, o, lse, dm, n_qt);
+    default: return swa_fwd_launch<D, DV, 16>(grid, st, q, k, v, o, lse, dm, n_qt);
   }
-#undef SWA_CALL
 }
 
 extern "C" int hils_swa_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int B,
@@ -659,15 +773,17 @@ extern "C" int hils_swa_fwd(const void* q, const void* k, const void* v, void* o
   HILS_REQUIRE((long)kv_start + Lk < 2147483647L / 2, "hils_swa_fwd: positions overflow 32 bits");
   SwaDims dm{Lq, Lk, HQ, H, window, chunk, mask_lmk, expand_to_chunk, kv_start,
              (chunk & (chunk - 1)) == 0, sm_scale};
-  const int QB = 4 * 16 * SWA_FWD_RT(D, Dv) / G;  // rows of a workgroup / group size (>= 1: G <= 16)
+  const int QB = SWA_FWD_WAVES * 16 * SWA_FWD_RT / G;  // queries of a workgroup (>= 16: G <= 16)
   const int n_qt = (Lq + QB - 1) / QB;
   const dim3 grid((unsigned)n_qt, (unsigned)H, (unsigned)B);
   hipStream_t st = (hipStream_t)stream;
   const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k, *vv = (const bf16_t*)v;
-  if (D == 64 && Dv == 64) swa_launch_g<64, 64>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
-  else if (D == 128 && Dv == 128) swa_launch_g<128, 128>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
-  else if (D == 64) swa_launch_g<64, 128>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
-  else swa_launch_g<128, 64>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
+  int rc;
+  if (D == 64 && Dv == 64) rc = swa_launch_g<64, 64>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
+  else if (D == 128 && Dv == 128) rc = swa_launch_g<128, 128>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
+  else if (D == 64) rc = swa_launch_g<64, 128>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
+  else rc = swa_launch_g<128, 64>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
+  if (rc) return rc;
   HILS_CHECK_LAUNCH("hils_swa_fwd");
   return HILS_OK;
 }
