@@ -1281,7 +1281,7 @@ struct TopkRowShared {
 
 // One (query, KV head) row (row = (b*L + t)*h_kv + hk) by a workgroup of NW wavefronts; dyn = the
 // workgroup's dynamic LDS (topk_row_smem bytes).
-template <int D, int GMAX, int NW, bool PAGED>
+template <int D, int GMAX, int NW, bool PAGED, int GI = 8>  // GI: load instructions per register buffer
 __device__ __forceinline__ void
 topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
               const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
@@ -1293,7 +1293,7 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   constexpr int LR = D / 8, TPI = 64 / LR;
   constexpr int THREADS = NW * 64;       // NW = 8 or 16 wavefronts
   constexpr int EPT = TOPK_R_MAXN / THREADS;  // 64-chunk slots of a wavefront's share
-  constexpr int GI = 8;          // load instructions per register buffer
+  static_assert(GI == 8 || GI == 16, "a key group is 8 or 16 load instructions");
   constexpr int KG = GI * TPI;   // chunk keys per buffer
   float* logit_s = dyn;                       // [GMAX][NP] raw scaled logits
   float* pooled = dyn + (size_t)GMAX * NP;    // [NP]

@@ -210,6 +210,20 @@ def test_sparse_attn_decode_one_workgroup_per_row(pkg, orc, dev, B, HQ, H, D, K,
     fwd_check(pkg, orc, dev, q, k, v, w, idx, 64)
 
 
+@pytest.mark.parametrize("B,Lq,HQ,H,D,K,Lkv,mask_last", [
+    (3, 1, 16, 2, 64, 5, 2048, True),       # 8 query heads per KV head, fewer slots than wavefronts
+    (2, 2, 32, 2, 128, 40, 4096, True),     # 16 heads per KV head, two queries
+    (1, 3, 8, 8, 64, 128, 16384, False),    # the most slots the row kernel takes, last token not masked
+    (5, 1, 12, 4, 128, 1, 1024, True),      # 3 heads per KV head, a single slot
+    (300, 1, 6, 2, 64, 16, 1024, True)])    # more rows than compute units
+def test_sparse_attn_decode_group_sizes_and_slot_counts(pkg, orc, dev, B, Lq, HQ, H, D, K, Lkv, mask_last):
+    """The decode kernel at its other group sizes (up to 16 query heads in the matrix columns), slot
+    counts (1 ... 128) and workgroup layouts (slots split over workgroups / one workgroup per row)."""
+    note(f"sparse_attn decode B{B} Lq{Lq} HQ{HQ} H{H} D{D} K{K} Lkv{Lkv}")
+    q, k, v, w, idx = make_case(B, Lq, HQ, H, D, D, K, 64, seed=14, Lkv=Lkv, fill_prob=0.85)
+    fwd_check(pkg, orc, dev, q, k, v, w, idx, 64, mask_last_token=mask_last)
+
+
 @pytest.mark.parametrize("B,L,HQ,H,D,Dv,K", [(1, 1024, 8, 2, 128, 128, 8), (2, 512, 4, 4, 64, 64, 16),
                                               (1, 700, 16, 1, 64, 128, 4), (1, 512, 8, 4, 128, 64, 32),
                                               (1, 300, 16, 2, 64, 64, 8),
