@@ -182,3 +182,32 @@ def test_decode_step_one_launch(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
     # twice the same call: bit-identical (the selection's log-sum-exp is summed in a fixed order)
     o2, w2, idx2, sc2 = pkg.decode_step(qd, lmk, kd, vd, lsed, K, 64, 1, q_offset=Lkv - Lq)
     assert torch.equal(o2, o1) and torch.equal(idx2, idx1) and torch.equal(w2, w1)
+
+
+@pytest.mark.parametrize("q_pos", [10, 700, 1000, 5000])
+def test_decode_step_on_a_mostly_empty_cache(pkg, orc, dev, q_pos):
+    """A cache buffer far longer than the sequence (the in-place cache hands the kernels its whole
+    buffers): only the chunks before the query are visible, fewer than topk of them or none at all."""
+    note(f"decode_step with the query at position {q_pos} of a 32768-token buffer")
+    B, Lq, Lkv, HQ, H, D, K = 12, 1, 32768, 16, 8, 128, 16
+    gen = torch.Generator().manual_seed(83)
+    q = torch.randn(B, Lq, HQ, D, generator=gen).bfloat16()
+    k = torch.randn(B, Lkv, H, D, generator=gen).bfloat16()
+    v = torch.randn(B, Lkv, H, D, generator=gen).bfloat16()
+    lse = torch.randn(B, Lq, HQ, generator=gen) * 3 + 5
+    qd, kd, vd, lsed = q.to(dev), k.to(dev), v.to(dev), lse.to(dev)
+    lmk = pkg.chunk_mean_pool(kd, 64)
+    dbg = {}
+    o1, w1, idx1, sc1 = pkg.decode_step(qd, lmk, kd, vd, lsed, K, 64, 1, q_offset=q_pos, _debug=dbg)
+    assert dbg, "this shape is meant to run on the one-launch kernel"
+    lim = orc.causal_chunk_limit(Lq, q_pos, 1, 64)
+    want = orc.topk_select(dbg["sel_logits"].cpu(), dbg["lse_total"].cpu(), lim, K)
+    assert torch.equal(idx1.cpu(), want)
+    nvis = int(lim[0])
+    assert (idx1 >= 0).sum().item() == B * H * min(K, nvis) and int(idx1.max().item()) < max(nvis, 1)
+    idx0, sc0, w0 = pkg.topk_chunk_weights(qd, lmk, lsed, K, 64, 1, q_offset=q_pos)
+    assert torch.equal(idx1, idx0) and torch.equal(sc1, sc0) and torch.equal(w1, w0)
+    ref = orc.sparse_attn(q, k, v, w1.cpu(), idx1.cpu(), chunk_size=64)
+    assert_close_bf16(o1, ref, "decode_step output")
+    if nvis == 0:  # nothing remote to attend to: all the weight on the local branch
+        assert torch.count_nonzero(o1).item() == 0 and torch.all(w1[..., K].float() == 1.0)
