@@ -165,7 +165,7 @@ __global__ void decode_reduce_kernel(const float* __restrict__ partial, bf16_t* 
 static int de_pick_nsplit(int B, int L, int H, int K) {
   const int cus = hils_device_cus();
   const long rows = (long)B * L * H;
-  // whole waves of one 16-wavefront workgroup per compute unit: no split, no partial sums
+  // one workgroup per row and whole rounds of rows over the compute units: no split, no partial sums
   if (K >= 16 && rows >= cus && (rows % cus == 0 || rows >= 8L * cus)) return 1;
   int nsplit = 1;
   // aim for >= 4 workgroups per CU, at least one slot per wavefront

@@ -203,7 +203,7 @@ def test_sparse_attn_decode_shape(pkg, orc, dev):
 @pytest.mark.parametrize("B,HQ,H,D,K,Lkv", [(32, 32, 8, 128, 32, 4096), (64, 8, 4, 64, 16, 2048),
                                             (256, 4, 1, 128, 24, 2048)])
 def test_sparse_attn_decode_one_workgroup_per_row(pkg, orc, dev, B, HQ, H, D, K, Lkv):
-    """Decode with a multiple of 256 (query, KV head) rows: one 16-wavefront workgroup per row,
+    """Decode with a multiple of 256 (query, KV head) rows: one workgroup per row,
     slots spread over its wavefronts and summed in LDS (no split over workgroups)."""
     note(f"sparse_attn decode rows B{B} HQ{HQ} H{H} D{D} K{K} Lkv{Lkv}")
     q, k, v, w, idx = make_case(B, 1, HQ, H, D, D, K, 64, seed=13, Lkv=Lkv, fill_prob=0.9)
