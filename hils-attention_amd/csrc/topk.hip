@@ -1558,8 +1558,12 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     }
     __syncthreads();
     if (wave == 0) {
-      const int nc = wave_select<true, TOPK_R_CAND / 64>((const float*)ck, cand_total, 0, sh.cand_s[0], sh.cand_i[0], 0,
-                                                          topk, sh.merge_i);
+      // (the usual case, about 1.4 topk candidates, is one key per lane)
+      const int nc = cand_total <= 64
+                         ? wave_select<true, 1>((const float*)ck, cand_total, 0, sh.cand_s[0], sh.cand_i[0], 0, topk,
+                                                sh.merge_i)
+                         : wave_select<true, TOPK_R_CAND / 64>((const float*)ck, cand_total, 0, sh.cand_s[0],
+                                                               sh.cand_i[0], 0, topk, sh.merge_i);
       if (lane == 0) sh.ncand[0] = nc;
     }
   } else {
