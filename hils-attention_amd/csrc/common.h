@@ -160,3 +160,34 @@ __host__ __device__ __forceinline__ int visible_limit(int t_global, int window, 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+// Sum of |w| over the K bf16 elements e0 .. e0+K-1 of a tensor of tot_e elements (a weight row may
+// start on any element).  The row is read as aligned dwords, a batch of loads in flight together and
+// none of them inside a branch (a load inside a branch is waited for inside it): an index is clamped
+// to the last even one whose dword lies inside the tensor and a clamped dword counts for nothing; the
+// tensor's last element, when its index is even, has no such dword and is read on its own by the
+// one thread whose row ends there.
+__device__ __forceinline__ float hils_abs_row_sum_bf16(const bf16_t* __restrict__ w, long e0, int K, long tot_e) {
+  constexpr int WDW = 17;  // dwords per round: 32 elements + alignment slack
+  if (tot_e < 2) return fabsf(bf2f(w[e0]));
+  const long e_end = e0 + K;
+  const long last_dw = (tot_e - 2) & ~1L;
+  float a = 0.f;
+  for (long eb = e0 & ~1L; eb < e_end; eb += 2 * WDW) {
+    uint32_t wd[WDW];
+#pragma unroll
+    for (int u = 0; u < WDW; ++u) {
+      const long ee = eb + 2 * u;
+      wd[u] = *(const uint32_t*)(w + (ee < last_dw ? ee : last_dw));
+    }
+#pragma unroll
+    for (int u = 0; u < WDW; ++u) {
+      const long ee = eb + 2 * u;
+      const bool here = ee <= last_dw;
+      if (here && ee >= e0 && ee < e_end) a += fabsf(__uint_as_float(wd[u] << 16));
+      if (here && ee + 1 >= e0 && ee + 1 < e_end) a += fabsf(__uint_as_float(wd[u] & 0xffff0000u));
+    }
+  }
+  if ((tot_e & 1) && e_end == tot_e) a += fabsf(bf2f(w[tot_e - 1]));
+  return a;
+}

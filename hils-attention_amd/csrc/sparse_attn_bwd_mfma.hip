@@ -474,8 +474,7 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
     const int ql = row / G, g = row - ql * G;
     if (t0 + ql < dm.L) {
       const long rowi = (b * dm.L + t0 + ql) * (long)dm.HQ + hk * G + g;
-      float a = 0.f;
-      for (int s2 = 0; s2 < K; ++s2) a += fabsf(bf2f(weights[rowi * dm.NW + s2]));
+      const float a = hils_abs_row_sum_bf16(weights, rowi * dm.NW, K, (long)dm.B * dm.L * dm.HQ * dm.NW);
       float l1 = 0.f;
 #pragma unroll
       for (int p8 = 0; p8 < DV / 8; ++p8) {

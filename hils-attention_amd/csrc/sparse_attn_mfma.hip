@@ -241,42 +241,15 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     }
     creg[e] = c;
   }
-  // (2) weight rows, for the bound of the fixed-point scale: a row's sum of |w| over the K slots.
-  // A row is read as aligned dwords (rows start on any bf16), all loads in flight together.
-  constexpr int WDW = 17;  // dwords per round: 32 slots + alignment slack
+  // (2) weight rows, for the bound of the fixed-point scale: a row's sum of |w| over the K slots
+  // (aligned dword loads, all in flight together)
   for (int row = tid; row < R; row += NT) {
     const int ql = row / G, g = row - ql * G;
     float a = 0.f;
     if (t0 + ql < dm.L) {
       const long e0 = ((b * LB + (t0 + ql) / dm.q_block) * (long)dm.WH + (w_per_q ? hk * G + g : hk)) *
                       dm.NW;  // first element
-      const long e_end = e0 + K;
-      const long tot_e = (long)dm.B * LB * dm.WH * dm.NW;
-      // dwords are loaded without a branch (a load inside a branch is waited for inside it), from
-      // an index clamped to the last even one whose dword lies inside the tensor; a clamped dword
-      // counts for nothing.  The tensor's last element, when its index is even, has no such dword
-      // and is read on its own by the one thread whose row ends there.
-      const long last_dw = (tot_e - 2) & ~1L;
-      if (tot_e < 2) {
-        a = fabsf(bf2f(weights[e0]));
-      } else {
-        for (long eb = e0 & ~1L; eb < e_end; eb += 2 * WDW) {
-          uint32_t wd[WDW];
-#pragma unroll
-          for (int u = 0; u < WDW; ++u) {
-            const long ee = eb + 2 * u;
-            wd[u] = *(const uint32_t*)(weights + (ee < last_dw ? ee : last_dw));
-          }
-#pragma unroll
-          for (int u = 0; u < WDW; ++u) {
-            const long ee = eb + 2 * u;
-            const bool here = ee <= last_dw;
-            if (here && ee >= e0 && ee < e_end) a += fabsf(__uint_as_float(wd[u] << 16));
-            if (here && ee + 1 >= e0 && ee + 1 < e_end) a += fabsf(__uint_as_float(wd[u] & 0xffff0000u));
-          }
-        }
-        if ((tot_e & 1) && e_end == tot_e) a += fabsf(bf2f(weights[tot_e - 1]));
-      }
+      a = hils_abs_row_sum_bf16(weights, e0, K, (long)dm.B * LB * dm.WH * dm.NW);
     }
     rscale[row] = a;  // only this thread touches the entry until the barrier behind the scan
   }
