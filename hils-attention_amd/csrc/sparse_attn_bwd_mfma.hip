@@ -489,19 +489,34 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
   for (int i = tid; i < (R + 1) * D; i += BQ_THREADS) q_acc[i] = 0;
   for (int i = tid; i < dm.nchunk; i += BQ_THREADS) cur[i] = 0;
   if (tid == 0) next_s = 0;
-  if (STAGE) {  // rows beyond the sequence end are never addressed by a pair
-    for (int i = tid; i < R * (D / 8); i += BQ_THREADS) {
-      const int row = i / (D / 8), pc = i - row * (D / 8);
-      if (t0 + row / G < dm.L)
-        *(bw_u4*)(rows_q + row * QROWB + pc * 16) =
-            *(const bw_u4*)(q + ((b * dm.L + t0 + row / G) * (long)dm.HQ + hk * G + row % G) * D + pc * 8);
-    }
-    for (int i = tid; i < R * (DV / 8); i += BQ_THREADS) {
-      const int row = i / (DV / 8), pc = i - row * (DV / 8);
-      if (t0 + row / G < dm.L)
-        *(bw_u4*)(rows_o + row * OROWB + pc * 16) =
-            *(const bw_u4*)(d_o + ((b * dm.L + t0 + row / G) * (long)dm.HQ + hk * G + row % G) * DV + pc * 8);
-    }
+  if (STAGE) {
+    // rows beyond the sequence end are never addressed by a pair: they re-read the last row.  Four
+    // loads in flight per thread and none inside a branch (a load inside a branch is waited for there).
+    auto stage_rows = [&](const bf16_t* src, char* dst, int rowb, int npc) __attribute__((always_inline)) {
+      const int n = R * npc;
+      for (int i0 = 0; i0 < n; i0 += 4 * BQ_THREADS) {
+        bw_u4 t[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * BQ_THREADS + tid;
+          const int ic = i < n ? i : n - 1;
+          const int row = ic / npc, pc = ic - row * npc;
+          int tq = t0 + row / G;
+          tq = tq < dm.L ? tq : dm.L - 1;
+          t[u] = *(const bw_u4*)(src + ((b * dm.L + tq) * (long)dm.HQ + hk * G + row % G) * (npc * 8) + pc * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * BQ_THREADS + tid;
+          if (i < n) {
+            const int row = i / npc, pc = i - row * npc;
+            *(bw_u4*)(dst + row * rowb + pc * 16) = t[u];
+          }
+        }
+      }
+    };
+    stage_rows(q, rows_q, QROWB, D / 8);
+    stage_rows(d_o, rows_o, OROWB, DV / 8);
   }
   __syncthreads();
 #pragma unroll
