@@ -488,6 +488,30 @@ def cpu_baseline(data, n_queries=4096):
                       f"{dt:.2f} s", "seconds": dt}
 
 
+def bench_stream_probe(pkg, dev, gib=4, reps=20):
+    """TB/s of hils_stream_probe over a buffer far larger than the 256 MiB last-level cache."""
+    from importlib import import_module
+    cabi = import_module(pkg.__name__ + ".ops._cabi")
+    cabi.load()
+    buf = torch.empty(gib << 30, dtype=torch.uint8, device=dev).fill_(1)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    out = {"bytes": int(buf.numel())}
+    for name, pattern in (("contiguous", 0), ("rows_256B_stride_2KiB", 1)):
+        def run():
+            cabi.call("hils_stream_probe", buf.data_ptr(), buf.numel(), pattern, sink.data_ptr())
+        for _ in range(3):
+            run()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        out[name] = {"ms": round(ms, 4), "TB_per_s": round(buf.numel() / ms / 1e9, 3)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -503,6 +527,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: run only a 512 MiB device copy (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--stream-probe", action="store_true",
+                    help="measurement aid: the rate of a kernel that only loads, contiguous and as "
+                         "256-byte rows at a 2 KiB stride (what the streaming kernels can reach)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives are part of the hot "
@@ -520,6 +547,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes": int(src.numel())}))
+        return
+    if args.stream_probe:
+        print(json.dumps({"stream_probe": bench_stream_probe(pkg, dev)}))
         return
     if args.train_only:
         print(json.dumps({"train_fwd_bwd": bench_train(pkg, dev)}))

@@ -70,6 +70,8 @@ def load():
     lib.hils_topk_fwd_noalloc_max_workspace.argtypes = []
     lib.hils_sparse_attn_decode_paged_workspace.restype = ctypes.c_size_t
     lib.hils_sparse_attn_decode_paged_workspace.argtypes = [_I] * 6
+    lib.hils_stream_probe.restype = c_int
+    lib.hils_stream_probe.argtypes = [_P, ctypes.c_size_t, _I, _P, _P]
     lib.hils_decode_step_covers.restype = c_int
     lib.hils_decode_step_covers.argtypes = [_I] * 8
     lib.hils_sparse_attn_fwd_workspace.restype = ctypes.c_size_t

@@ -274,6 +274,15 @@ int hils_decode_step_paged(const void* q, const void* lmk_pages, const void* k_p
                            int max_pages, int num_pages, float sm_scale_sel, float sm_scale_attn,
                            int mask_last, void* stream);
 
+/* ---- measurement aid ---------------------------------------------------------------- */
+
+/* A kernel that only loads `bytes` bytes of buf (no counterpart in the reference): the rate any
+ * streaming kernel can reach on this GPU.  pattern 0: contiguous shares per workgroup; pattern 1:
+ * the buffer as a (tokens, 8 heads, 128) bf16 tensor read one head per workgroup (256-byte rows at
+ * a 2 KiB stride, what the token-major decode kernels read).  sink: 4 bytes of device memory.
+ * Both patterns skip a tail of the buffer that does not fill a whole round of loads. */
+int hils_stream_probe(const void* buf, size_t bytes, int pattern, void* sink, void* stream);
+
 /* ---- exact per-chunk log Z ---------------------------------------------------- */
 
 /* Forward.  Replaces exact_chunk_log_z_fwd (ops/exact_chunk_log_z_tilelang.py:25-137).

@@ -42,6 +42,7 @@ def test_binding_matches_header(pkg):
     fns.pop("hils_topk_fwd_noalloc_max_workspace")
     fns.pop("hils_sparse_attn_decode_paged_workspace")
     fns.pop("hils_decode_step_covers")
+    fns.pop("hils_stream_probe")
     assert set(_cabi.SIGNATURES) == set(fns)
     for name, params in fns.items():
         argtypes = _cabi.SIGNATURES[name]
@@ -69,6 +70,10 @@ def test_argument_errors_are_reported_without_a_gpu(pkg):
     assert lib.hils_sparse_attn_fwd(buf, buf, buf, buf, buf, None, None, buf, None, None, 0,
                                     1, 16, 64, 3, 2, 64, 64, 4, 4, 3, 1, 64, 0.125, 1, 0.0, 0, None) == 1
     assert b"multiple of H" in lib.hils_last_error()
+    assert lib.hils_stream_probe(buf, 64 << 20, 2, buf, None) == 1
+    assert b"pattern" in lib.hils_last_error()
+    assert lib.hils_stream_probe(buf, 1 << 20, 0, buf, None) == 1
+    assert b"64 MiB" in lib.hils_last_error()
 
 
 def test_no_cpu_fallback(pkg):
