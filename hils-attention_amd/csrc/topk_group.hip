@@ -26,11 +26,15 @@
 #define TG_NB 32     // chunk blocks of 16 a lane row can hold (N <= 512)
 #define TG_CAND 128  // compacted candidates per query (8 per lane)
 
-__device__ __forceinline__ uint32_t tg_score_key(float f) {  // larger float <-> larger key; 0 = not a candidate
-  if (!(f > HILS_NEG_INF)) return 0u;  // -inf and NaN
-  f = f + 0.0f;                        // -0 -> +0
+// Order-preserving unsigned image of a finite score (larger score <-> larger key, -0 as +0) and its
+// inverse.  Every finite score has a key above 0x00800000, so 0 stands for "no key".
+__device__ __forceinline__ uint32_t tg_score_key(float f) {
+  f = f + 0.0f;  // -0 -> +0
   const uint32_t u = __float_as_uint(f);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float tg_key_score(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
 // all-reduce over the 16 lanes of a lane row
@@ -58,6 +62,13 @@ __device__ __forceinline__ float tg_row_max_f(float x) {
   x = fmaxf(x, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x140, 0xF, 0xF, false)));
   return x;
 }
+__device__ __forceinline__ float tg_row_min_f(float x) {
+  x = fminf(x, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xF, 0xF, false)));
+  x = fminf(x, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xF, 0xF, false)));
+  x = fminf(x, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x141, 0xF, 0xF, false)));
+  x = fminf(x, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x140, 0xF, 0xF, false)));
+  return x;
+}
 // exclusive prefix sum over the 16 lanes of a lane row (lanes shifted in from outside read 0)
 __device__ __forceinline__ int tg_row_excl_scan(int x) {
   int s = x;
@@ -68,55 +79,71 @@ __device__ __forceinline__ int tg_row_excl_scan(int x) {
   return s - x;
 }
 
-// K-th largest of the keys a lane row holds, NE per lane (0 = no key), all non-zero keys in
-// [lo, hi] and at least K of them: returns T with count(key >= T) >= K > count(key > T).
+// Threshold of the K largest keys a lane row holds, NE per lane (0 = no key), all non-zero keys in
+// [lo, hi] and at least K of them: returns T in [lo, hi] with count(key >= T) >= K >= count(key > T)
+// and count(key > T) + count(key == T) >= K.  The bitwise search of a lane row stops as soon as a
+// probe at or above lo counts exactly K keys (the winners are then known, exact is set and no tie
+// needs breaking: with about 1.5 K keys in the range that takes a third of the steps of a search
+// down to the last bit, and unless the K-th and (K+1)-th largest keys are equal some probe does);
+// rows that are not live take no part, and the loop, which is wavefront-uniform, ends when no row
+// is live.
 template <int NE>
-__device__ __forceinline__ uint32_t tg_kth_largest(const uint32_t (&k)[NE], uint32_t lo, uint32_t hi, int K) {
+__device__ __forceinline__ uint32_t tg_kth_largest(const uint32_t (&k)[NE], uint32_t lo, uint32_t hi, int K,
+                                                   bool live, bool& exact) {
   const uint32_t diff = lo ^ hi;
-  // bits above the highest differing one are shared by every key; the search runs over the rest,
-  // as many steps as the lane row with the widest range needs (the loop is wavefront-uniform)
+  // bits above the highest differing one are shared by every key; the search runs over the rest
   const int top = diff ? 31 - __clz((int)diff) : -1;
   uint32_t T = (top >= 31 || top < 0) ? (top < 0 ? lo : 0u) : (lo & ~((2u << top) - 1u));
-  int top_w = top;
-  top_w = max(top_w, __builtin_amdgcn_readlane(top, 16));
-  top_w = max(top_w, __builtin_amdgcn_readlane(top, 32));
-  top_w = max(top_w, __builtin_amdgcn_readlane(top, 48));
-  top_w = max(top_w, __builtin_amdgcn_readlane(top, 0));
+  live = live & (top >= 0);
+  const int top_l = live ? top : -1;
+  int top_w = __builtin_amdgcn_readlane(top_l, 0);
+  top_w = max(top_w, __builtin_amdgcn_readlane(top_l, 16));
+  top_w = max(top_w, __builtin_amdgcn_readlane(top_l, 32));
+  top_w = max(top_w, __builtin_amdgcn_readlane(top_l, 48));
   for (int bit = top_w; bit >= 0; --bit) {
+    if (!__any(live)) break;
     const uint32_t c = T | (1u << bit);
     int cl = 0;
 #pragma unroll
     for (int e = 0; e < NE; ++e) cl += (k[e] >= c) ? 1 : 0;
     const int cnt = tg_row_sum_i(cl);
-    if (bit <= top && cnt >= K) T = c;
+    const bool act = live & (bit <= top);
+    if (act & (cnt >= K)) T = c;
+    if (act & (cnt == K) & (c >= lo)) {
+      live = false;
+      exact = true;
+    }
   }
   return T;
 }
 
-// NB: chunk blocks the launch covers (every query of the launch sees at most 16*NB chunks and at
-// least 16*(NB-9)+1, so only the last nine blocks can hold invisible chunks); t_base: first query.
-// Everything is unrolled over the NB blocks: register-resident data has no other way of being
-// indexed, and the host splits a call into launches by NB so that early queries do not pay for 32.
+// NB: chunk blocks the launch covers, 8, 16 or 32.  Every query of the launch sees at most 16*NB
+// chunks and more than 16*NB/2 (NB = 8: any number), so only the blocks from NMASK on can hold
+// invisible chunks; t_base: first query.  Everything is unrolled over the NB blocks: register-resident
+// data has no other way of being indexed, and the host splits a call into launches by NB so that
+// early queries do not pay for 32.  (A 24-block instantiation for the queries that see 257..384
+// chunks ran no faster than this kernel at 32; the time goes by the schedule the compiler finds at
+// the given register budget as much as by the work.)
 #define TG_WAVES 4  // wavefronts per workgroup, each with queries of its own (they never synchronise)
 template <int GMAX, int KS, int NB, bool EXPORT>
 __global__ void __launch_bounds__(64 * TG_WAVES)
-    __attribute__((amdgpu_waves_per_eu(NB <= 8 ? 5 : (NB <= 16 ? 4 : (NB <= 24 ? 3 : 2)))))
+    __attribute__((amdgpu_waves_per_eu(NB <= 8 ? 5 : (NB <= 16 ? 4 : 2))))
 topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lmk_packed,
                       const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
                       bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
                       float* __restrict__ sel_logits_out, int L, int N, int h_kv, int G, int topk,
                       int block_size, int window_size, int causal, int q_offset, float sm_scale,
-                      int t_base, int t_end) {
+                      int t_base, int t_end, int bs_shift) {
   constexpr int D = KS * 32;
   constexpr int QPL = 4 / GMAX;   // queries per lane (its four accumulator rows)
   constexpr int NQ = 16 / GMAX;   // queries per wavefront
-  constexpr int NMASK = EXPORT ? 0 : (NB > 9 ? NB - 9 : 0);  // blocks below it are visible to every row
+  constexpr int NMASK = EXPORT ? 0 : (NB > 8 ? NB / 2 : 0);  // blocks below it are visible to every row
   __shared__ uint32_t cand_w[TG_WAVES][4][TG_CAND];          // compacted candidate keys, per lane row
   __shared__ uint32_t words_w[TG_WAVES][4][16], wbase_w[TG_WAVES][4][16];  // winner map of a query and its word prefix counts
-  __shared__ int stage_i_w[TG_WAVES][NQ * 32];               // winners' chunk indices, [query][slot]
-  __shared__ __align__(16) bf16_t stage_s_w[TG_WAVES][NQ * GMAX * 32];  // their raw scores, [query][head][slot]
+  __shared__ __align__(16) int stage_i_w[TG_WAVES][NQ * 32];               // winners' chunk indices, [query][slot]
+  __shared__ __align__(16) bf16_t stage_s_w[TG_WAVES][NQ * GMAX * 32];  // their raw scores, [query][slot][head]
 
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   uint32_t (*cand)[TG_CAND] = cand_w[wave];
   uint32_t (*words)[16] = words_w[wave];
   uint32_t (*wbase)[16] = wbase_w[wave];
@@ -128,19 +155,25 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   const int hk = blockIdx.y;
   const long b = blockIdx.z;
 
+  // chunks a query sees (visible_limit of common.h; bs_shift >= 0: the chunk size is 1 << bs_shift and
+  // the division is an arithmetic shift, which rounds towards minus infinity as floordiv does)
   auto limit_of = [&](int tq) -> int {
-    int lm = causal ? visible_limit(tq + q_offset, window_size, block_size) : N;
+    const int a = window_size > 0 ? tq + q_offset - window_size + 1 : tq + q_offset;
+    int lm = causal ? (bs_shift >= 0 ? (a >> bs_shift) : floordiv(a, block_size)) : N;
     return lm < 0 ? 0 : (lm > N ? N : lm);
   };
-  // accumulator row 4j+i <-> (query t0 + (4j+i)/GMAX, head (4j+i)%GMAX)
+  // accumulator row 4j+i <-> (query t0 + (4j+i)/GMAX, head (4j+i)%GMAX): a lane has QPL queries
   int lim[4];
   bool rowok[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = 4 * j + i;
-    const int tq = t0 + r / GMAX;
-    rowok[i] = tq < t_end && (r % GMAX) < G;
-    lim[i] = rowok[i] ? limit_of(tq) : 0;
+  for (int u = 0; u < QPL; ++u) {
+    const int tq = t0 + j * QPL + u;
+    const int lq = tq < t_end ? limit_of(tq) : 0;
+#pragma unroll
+    for (int e = 0; e < GMAX; ++e) {
+      rowok[u * GMAX + e] = (tq < t_end) & (e < G);
+      lim[u * GMAX + e] = e < G ? lq : 0;
+    }
   }
   const int nb_real = (N + 15) / 16;  // blocks the packed chunk keys hold
 
@@ -172,7 +205,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   // the keys of two blocks travel together, one such group ahead of their use (the loads of a
   // block issued right before its MFMAs would each expose a full memory latency)
   typedef unsigned tg_u32x4 __attribute__((ext_vector_type(4)));
-  constexpr int PB = 2;  // blocks per load group
+  constexpr int PB = NB >= 32 ? 2 : 1;  // blocks per load group (two groups are live: 16 registers per block and group)
   static_assert(NB % PB == 0, "blocks come in load groups");
   auto load_group = [&](int g0, tg_u32x4 (&dst)[PB][KS]) {
 #pragma unroll
@@ -215,11 +248,17 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
     load_group(0, ba);
 #pragma unroll
     for (int g0 = 0; g0 < NB; g0 += 2 * PB) {
+      // scheduling barriers: left to itself the compiler, when registers are short, sinks the loads
+      // of the next group to their uses and every MFMA then waits a full memory latency
       if (g0 + PB < NB) load_group(g0 + PB, bb2);
+      __builtin_amdgcn_sched_barrier(0);
       use_group(g0, ba);
+      __builtin_amdgcn_sched_barrier(0);
       if (g0 + PB < NB) {
         if (g0 + 2 * PB < NB) load_group(g0 + 2 * PB, ba);
+        __builtin_amdgcn_sched_barrier(0);
         use_group(g0 + PB, bb2);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   }
@@ -250,103 +289,137 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   }
 
   // outputs start as "no winner"
-  for (int e = lane; e < NQ * 32; e += 64) stage_i[e] = -1;
-  for (int e = lane; e < NQ * GMAX * 32; e += 64) stage_s[e] = 0xff80;  // -inf
+  for (int e = lane; e < NQ * 8; e += 64) ((int4*)stage_i)[e] = make_int4(-1, -1, -1, -1);
+  ((uint4*)stage_s)[lane] = make_uint4(0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u);  // 512 x -inf
   __builtin_amdgcn_wave_barrier();
 
   // ---- selection, one query of every lane row at a time ----
 #pragma unroll
   for (int u = 0; u < QPL; ++u) {
     const int qi = j * QPL + u;  // query of the wavefront this lane row works on
-    // selection key of chunk nt*16+col: max over the heads of (logit - lse_total), one fp32
-    // subtraction each; -inf and NaN give key 0 (-inf - lse is -inf or NaN, and fmaxf skips NaN)
-    uint32_t key[NB];
+    // selection score of chunk nt*16+col: max over the heads of (logit - lse_total), one fp32
+    // subtraction each; -inf where the chunk is not visible (-inf - lse is -inf or NaN, and fmaxf
+    // skips NaN).  Scores are compared as floats (+0 == -0, as in the reference's sort); only the few
+    // candidates of the threshold search are turned into integer keys.
+    float key[NB];
 #pragma unroll
     for (int nt = 0; nt < NB; ++nt) {
       float best = HILS_NEG_INF;
 #pragma unroll
       for (int e = 0; e < GMAX; ++e) best = fmaxf(best, __fsub_rn(x[nt][u * GMAX + e], lse_tot[u * GMAX + e]));
-      key[nt] = tg_score_key(best);
+      key[nt] = best;
     }
-    // the two largest keys of the lane, the number of valid ones
-    uint32_t m1 = 0u, m2 = 0u;
+    // the two largest scores of the lane, the number of valid ones
+    float m1 = HILS_NEG_INF, m2 = HILS_NEG_INF;
     int nv = 0;
 #pragma unroll
     for (int nt = 0; nt < NB; ++nt) {
-      const uint32_t kk = key[nt];
-      const uint32_t lo2 = kk < m1 ? kk : m1;
-      m2 = lo2 > m2 ? lo2 : m2;
-      m1 = kk > m1 ? kk : m1;
-      nv += kk != 0u;
+      const float kk = key[nt];
+      m2 = fmaxf(m2, fminf(kk, m1));
+      m1 = fmaxf(m1, kk);
+      nv += (kk > HILS_NEG_INF) ? 1 : 0;
     }
     const int nvalid = tg_row_sum_i(nv);
-    uint32_t T = 1u;        // every valid key wins ...
-    int cutoff = 1 << 30;   // ... and among the keys equal to T those with a chunk index <= cutoff
+    float Tf = HILS_NEG_INF;  // every valid score wins ...
+    int cutoff = -1;          // ... and among the scores equal to Tf those with a chunk index <= cutoff
+    bool cut = false;         // cutoff excludes some of them
     if (__any(nvalid > topk)) {
-      const uint32_t hi = tg_row_max_u(m1);
-      const uint32_t bound = tg_row_min_u(m2);  // >= 2 keys per lane reach it: >= 32 >= topk in all
+      const bool want = nvalid > topk;
+      const float hi = tg_row_max_f(m1);
+      const float bound = tg_row_min_f(m2);  // >= 2 scores per lane reach it: >= 32 >= topk in all
+      // a query that keeps everything has no candidates; -inf (a lane with fewer than two scores)
+      // makes every register one, which sends the wavefront to the search over all scores below
+      const float cbound = want ? bound : __builtin_inff();
       int nc = 0;
 #pragma unroll
-      for (int nt = 0; nt < NB; ++nt) nc += (key[nt] >= bound && key[nt] != 0u) ? 1 : 0;
+      for (int nt = 0; nt < NB; ++nt) nc += (key[nt] >= cbound) ? 1 : 0;
       const int ntot = tg_row_sum_i(nc);
-      const bool want = nvalid > topk;
-      if (!__any(want && (ntot > TG_CAND || bound == 0u))) {
+      uint32_t T;
+      bool exact = false;
+      if (!__any(want & ((ntot > TG_CAND) | !(bound > HILS_NEG_INF)))) {
         // compact the candidates of the lane row (any order) and take at most 8 per lane
         int pos = tg_row_excl_scan(nc);
 #pragma unroll
         for (int nt = 0; nt < NB; ++nt) {
-          if (key[nt] >= bound && key[nt] != 0u) {
-            cand[j][pos] = key[nt];
+          if (key[nt] >= cbound) {
+            cand[j][pos] = __float_as_uint(key[nt]);
             ++pos;
           }
         }
         __builtin_amdgcn_wave_barrier();
         uint32_t ck[TG_CAND / 16];
 #pragma unroll
-        for (int e = 0; e < TG_CAND / 16; ++e) ck[e] = (e * 16 + col < ntot) ? cand[j][e * 16 + col] : 0u;
+        for (int e = 0; e < TG_CAND / 16; ++e)
+          ck[e] = (e * 16 + col < ntot) ? tg_score_key(__uint_as_float(cand[j][e * 16 + col])) : 0u;
         __builtin_amdgcn_wave_barrier();
-        const uint32_t Tc = tg_kth_largest(ck, bound, hi, topk);
-        if (want) T = Tc;
+        const uint32_t lo_k = tg_score_key(want ? bound : 0.f), hi_k = tg_score_key(want ? hi : 0.f);
+        T = tg_kth_largest(ck, lo_k, hi_k, topk, want & (ntot != topk), exact);
+        if (ntot == topk) {  // exactly the candidates win
+          T = lo_k;
+          exact = true;
+        }
       } else {
-        // rare: too many keys at the bound (many equal scores) or a lane with fewer than two
-        // keys while the query has more than topk: search over all keys of the lane row
+        // rare: too many scores at the bound (many equal ones) or a lane with fewer than two
+        // scores while the query has more than topk: search over all scores of the lane row
+        uint32_t uk[NB];
         uint32_t mn = 0xffffffffu;
 #pragma unroll
-        for (int nt = 0; nt < NB; ++nt)
-          if (key[nt] != 0u) mn = key[nt] < mn ? key[nt] : mn;
-        mn = tg_row_min_u(mn);
-        const uint32_t Tc = tg_kth_largest(key, mn == 0xffffffffu ? 1u : mn, hi ? hi : 1u, topk);
-        if (want) T = Tc;
-      }
-      // ties at the threshold: the lowest chunk indices win
-      int ngt = 0, neq = 0;
-#pragma unroll
-      for (int nt = 0; nt < NB; ++nt) {
-        ngt += (key[nt] > T) ? 1 : 0;
-        neq += (key[nt] == T) ? 1 : 0;
-      }
-      ngt = tg_row_sum_i(ngt);
-      neq = tg_row_sum_i(neq);
-      const int need = topk - ngt;  // keys equal to T still to take (>= 1 when want)
-      if (__any(want && neq > need)) {
-        // smallest index C with count(key == T and chunk <= C) >= need, bit by bit (chunks < 512)
-        int C = 0;
-        for (int bit = 8; bit >= 0; --bit) {
-          const int c2 = C | (1 << bit);  // count the ties below c2
-          int cl = 0;
-#pragma unroll
-          for (int nt = 0; nt < NB; ++nt) cl += (key[nt] == T && nt * 16 + col < c2) ? 1 : 0;
-          if (tg_row_sum_i(cl) < need) C = c2;
+        for (int nt = 0; nt < NB; ++nt) {
+          uk[nt] = (key[nt] > HILS_NEG_INF) ? tg_score_key(key[nt]) : 0u;
+          if (uk[nt] != 0u) mn = uk[nt] < mn ? uk[nt] : mn;
         }
-        if (want && neq > need) cutoff = C;
+        mn = tg_row_min_u(mn);
+        const uint32_t hi_k = (hi > HILS_NEG_INF) ? tg_score_key(hi) : 1u;
+        T = tg_kth_largest(uk, mn == 0xffffffffu ? 1u : mn, hi_k, topk, want, exact);
+      }
+      if (want) {
+        Tf = tg_key_score(T);
+        cutoff = 1 << 30;
+      }
+      // ties at the threshold (only where the search ran down to the last bit): the lowest chunk
+      // indices win
+      const bool loose = want & !exact;
+      if (__any(loose)) {
+        int ngt = 0, neq = 0;
+#pragma unroll
+        for (int nt = 0; nt < NB; ++nt) {
+          ngt += (key[nt] > Tf) ? 1 : 0;
+          neq += (key[nt] == Tf) ? 1 : 0;
+        }
+        ngt = tg_row_sum_i(ngt);
+        neq = tg_row_sum_i(neq);
+        const int need = topk - ngt;  // scores equal to Tf still to take
+        if (__any(loose & (neq > need))) {
+          // smallest index C with count(score == Tf and chunk <= C) >= need, bit by bit (chunks < 512)
+          int C = 0;
+          for (int bit = 8; bit >= 0; --bit) {
+            const int c2 = C | (1 << bit);  // count the ties below c2
+            int cl = 0;
+#pragma unroll
+            for (int nt = 0; nt < NB; ++nt) cl += ((key[nt] == Tf) & (nt * 16 + col < c2)) ? 1 : 0;
+            if (tg_row_sum_i(cl) < need) C = c2;
+          }
+          if (loose & (neq > need)) {
+            cutoff = C;
+            cut = true;
+          }
+        }
       }
     }
     // winners of this lane as a bit mask over its blocks
     uint32_t mask = 0u;
+    if (__any(cut)) {
 #pragma unroll
-    for (int nt = NB - 1; nt >= 0; --nt) {
-      const bool win = key[nt] != 0u && (key[nt] > T || (key[nt] == T && nt * 16 + col <= cutoff));
-      mask = (mask << 1) | (win ? 1u : 0u);
+      for (int nt = NB - 1; nt >= 0; --nt) {
+        const bool win = (key[nt] > Tf) | ((key[nt] == Tf) & (nt * 16 + col <= cutoff));
+        mask = (mask << 1) | (win ? 1u : 0u);
+      }
+    } else {
+      // no tie to break in this wavefront: everything from the threshold up wins (a query that keeps
+      // all its valid scores has Tf = -inf: the lowest finite float stands in for it)
+      const float Tlow = fmaxf(Tf, -3.402823466e38f);
+#pragma unroll
+      for (int nt = NB - 1; nt >= 0; --nt) mask = (mask << 1) | ((key[nt] >= Tlow) ? 1u : 0u);
     }
     // 512-bit map of the winning chunks (chunk c = bit c): word w holds blocks 2w and 2w+1
     words[j][col] = 0u;
@@ -370,9 +443,15 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
         const int slot = (int)wbase[j][w] + __popc(words[j][w] & ((1u << (c & 31)) - 1u));
         if (slot < topk) {
           stage_i[qi * 32 + slot] = c;
-#pragma unroll
-          for (int e = 0; e < GMAX; ++e)
-            if (e < G) stage_s[(qi * GMAX + e) * 32 + slot] = f2bf(x[nt][u * GMAX + e]);
+          // the heads of the winner in one store (heads past G are never read back)
+          bf16_t* dst = &stage_s[(qi * 32 + slot) * GMAX];
+          if constexpr (GMAX == 4) {
+            *(uint2*)dst = make_uint2(pack_bf2(x[nt][u * 4], x[nt][u * 4 + 1]), pack_bf2(x[nt][u * 4 + 2], x[nt][u * 4 + 3]));
+          } else if constexpr (GMAX == 2) {
+            *(uint32_t*)dst = pack_bf2(x[nt][u * 2], x[nt][u * 2 + 1]);
+          } else {
+            *dst = f2bf(x[nt][u]);
+          }
         }
       }
     }
@@ -380,15 +459,21 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   }
 
   // ---- write out: indices (B,L,h_kv,topk) int32, scores (B,L,h_kv,G,topk) bf16 ----
-  for (int e = lane; e < NQ * topk; e += 64) {
-    const int qi = e / topk, k = e - qi * topk;
-    if (t0 + qi < t_end) indices[((b * L + t0 + qi) * (long)h_kv + hk) * topk + k] = stage_i[qi * 32 + k];
+  // the stage is walked in its own padded order (32 slots per row): no division by topk, and a
+  // lane row stores consecutive slots of one output row
+  const long row0 = ((b * L + t0) * (long)h_kv + hk);  // (query t0, this KV head); the next query is h_kv further
+  int32_t* ind0 = indices + row0 * topk;
+  bf16_t* sc0 = scores + row0 * G * topk;
+#pragma unroll
+  for (int e0 = 0; e0 < NQ * 32; e0 += 64) {
+    const int e = e0 + lane, qi = e >> 5, k = e & 31;
+    if ((k < topk) & (t0 + qi < t_end)) ind0[qi * h_kv * topk + k] = stage_i[e];
   }
-  for (int e = lane; e < NQ * G * topk; e += 64) {
-    const int qi = e / (G * topk), rem = e - qi * (G * topk);
-    const int g = rem / topk, k = rem - g * topk;
-    if (t0 + qi < t_end)
-      scores[(((b * L + t0 + qi) * (long)h_kv + hk) * G + g) * topk + k] = stage_s[(qi * GMAX + g) * 32 + k];
+#pragma unroll
+  for (int e0 = 0; e0 < NQ * GMAX * 32; e0 += 64) {
+    const int e = e0 + lane, k = e & 31, g = (e >> 5) % GMAX, qi = e / (32 * GMAX);
+    if ((k < topk) & (g < G) & (t0 + qi < t_end))
+      sc0[(qi * h_kv * G + g) * topk + k] = stage_s[(qi * 32 + k) * GMAX + g];
   }
 }
 
@@ -405,19 +490,19 @@ static void tg_launch_range(int NB, bool exp, dim3 grid, hipStream_t st, const b
 #define TG_CALL(NB_, EX_)                                                                              \
   hipLaunchKernelGGL((topk_fwd_group_kernel<GMAX, KS, NB_, EX_>), grid, dim3(64 * TG_WAVES), 0, st, q, pk, lse_swa, \
                      indices, scores, lse_total, sel_logits, L, N, h_kv, G, topk, block_size, window_size, \
-                     causal, q_offset, sm_scale, t_base, t_end)
+                     causal, q_offset, sm_scale, t_base, t_end, bs_shift)
+  const int bs_shift = (block_size > 0 && (block_size & (block_size - 1)) == 0) ? __builtin_ctz(block_size) : -1;
   if (exp) { TG_CALL(32, true); return; }
   switch (NB) {
     case 8: TG_CALL(8, false); break;
     case 16: TG_CALL(16, false); break;
-    case 24: TG_CALL(24, false); break;
     default: TG_CALL(32, false); break;
   }
 #undef TG_CALL
 }
 
 // lmk_packed: the chunk keys in topk_pack_lmk_kernel's order.  The queries are split by how many
-// chunks they can see (8, 16, 24 or 32 blocks of 16) into one launch each.
+// chunks they can see (at most 8, 16 or 32 blocks of 16) into one launch each.
 int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* lse_swa, int32_t* indices,
                            void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
                            int G, int D, int topk, int block_size, int window_size, int causal, int q_offset,
@@ -436,7 +521,7 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
     int NB = 32, t_hi = L;
     if (!exp) {
       const int lm = limit_of(t);
-      NB = lm <= 128 ? 8 : (lm <= 256 ? 16 : (lm <= 384 ? 24 : 32));
+      NB = lm <= 128 ? 8 : (lm <= 256 ? 16 : 32);
       if (NB < 32) {
         int lo = t, hi = L;  // first query whose limit exceeds 16 * NB
         while (lo < hi) {
