@@ -410,6 +410,7 @@ struct BqDims {
   int L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last;
   float sm_scale;
   const float* slope;  // as in BwDims
+  uint32_t k_magic;    // hils_udiv_magic(K)
 };
 
 // STAGE: the block's own query and dO rows are copied into LDS once (coalesced) and every tile
@@ -461,7 +462,7 @@ bw_dq_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ d_o, const
     int c = -1;
     preg[e] = 0;
     if (i < npair) {
-      const int ql = i / K, slot = i - ql * K;
+      const int ql = (int)hils_udiv((uint32_t)i, (uint32_t)K, dm.k_magic), slot = i - ql * K;
       preg[e] = (ql << 8) | slot;
       if (t0 + ql < dm.L) c = indices[((b * dm.L + t0 + ql) * dm.H + hk) * (long)K + slot];
     }
@@ -954,7 +955,7 @@ int hils_bw_run(const void* q, const void* k, const void* v, const void* weights
     const int nblk = (L + T - 1) / T;
     const long total = (long)nblk * H * B;
     if (total > (1L << 30)) return -1;
-    BqDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale, slope};
+    BqDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale, slope, hils_udiv_magic((uint32_t)K)};
     dim3 grid((unsigned)(((total + 7) / 8) * 8));
     int rc = -1;
 #define BQ_D(D_, DV_)                                                                                 \

@@ -104,6 +104,7 @@ struct GaDims {
   int q_block, WH;
   float sm_n;
   int merge_col;  // with a local-branch output given: the weight column that scales it
+  uint32_t k_magic, qb_magic;  // hils_udiv_magic of K and q_block (pair index < 2^16, query index < 2^24)
 };
 
 // Power-of-two fixed-point scale for sums bounded by `bound`: bound * scale < 2^GA_FX_LOG2_MAX.
@@ -235,9 +236,9 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     int c = -1;
     preg[e] = 0;
     if (i < npair) {
-      const int ql = i / K, slot = i - ql * K;
+      const int ql = (int)hils_udiv((uint32_t)i, (uint32_t)K, dm.k_magic), slot = i - ql * K;
       preg[e] = (ql << 8) | slot;
-      if (t0 + ql < dm.L) c = indices[((b * LB + (t0 + ql) / dm.q_block) * dm.H + hk) * (long)K + slot];
+      if (t0 + ql < dm.L) c = indices[((b * LB + (long)hils_udiv((uint32_t)(t0 + ql), (uint32_t)dm.q_block, dm.qb_magic)) * dm.H + hk) * (long)K + slot];
     }
     creg[e] = c;
   }
@@ -247,7 +248,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     const int ql = row / G, g = row - ql * G;
     float a = 0.f;
     if (t0 + ql < dm.L) {
-      const long e0 = ((b * LB + (t0 + ql) / dm.q_block) * (long)dm.WH + (w_per_q ? hk * G + g : hk)) *
+      const long e0 = ((b * LB + (long)hils_udiv((uint32_t)(t0 + ql), (uint32_t)dm.q_block, dm.qb_magic)) * (long)dm.WH + (w_per_q ? hk * G + g : hk)) *
                       dm.NW;  // first element
       a = hils_abs_row_sum_bf16(weights, e0, K, (long)dm.B * LB * dm.WH * dm.NW);
     }
@@ -294,7 +295,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
     if (c < -1 || c >= dm.nchunk) c = -1;
     if (c < 0 && lse) {
       const int i = tid + e * NT;
-      const int ql = i / K, slot = i - ql * K;
+      const int ql = (int)hils_udiv((uint32_t)i, (uint32_t)K, dm.k_magic), slot = i - ql * K;
       if (i < npair && t0 + ql < dm.L) {
 #pragma unroll
         for (int g = 0; g < G; ++g)
@@ -661,7 +662,7 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
       for (int e = 0; e < 8; ++e) f[e] = (float)(int)((unsigned)src[e] - bias) * fx_inv;
       const long orow_g = ((b * dm.L + t) * (long)dm.HQ + hk * G + g2) * DV + c8 * 8;
       if (swa_o) {  // o = remote branch + local branch * its inter-chunk weight, rounded once
-        const float wl = bf2f(weights[((b * LB + t / dm.q_block) * (long)dm.WH + (w_per_q ? hk * G + g2 : hk)) *
+        const float wl = bf2f(weights[((b * LB + (long)hils_udiv((uint32_t)t, (uint32_t)dm.q_block, dm.qb_magic)) * (long)dm.WH + (w_per_q ? hk * G + g2 : hk)) *
                                           dm.NW + wcol]);
         float sv[8];
         unpack8(*(const uint4*)(swa_o + orow_g), sv);
@@ -788,7 +789,8 @@ int hils_sparse_attn_fwd_mfma(const void* q, const void* k, const void* v, const
                        (size_t)GA_S * (dmax + 2) * sizeof(bf16_t), st, (const bf16_t*)k,
                        (const bf16_t*)v, kpk, vpk, vmax, Lkv, H, D, Dv, nchunk);
   }
-  GaDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale, q_block, WH, sm_n, merge_col};
+  GaDims dm{L, Lkv, HQ, H, B, K, NW, T, nblk, nchunk, mask_last, sm_scale, q_block, WH, sm_n, merge_col,
+            hils_udiv_magic((uint32_t)K), hils_udiv_magic((uint32_t)q_block)};
   const long per_xcd = (total + 7) / 8;
   dim3 grid((unsigned)(per_xcd * 8));
   int rc = -1;
