@@ -281,7 +281,9 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
     const float mx = fmaxf(swa2, hils2), mn = fminf(swa2, hils2);
     float tot2 = mx;
     if (mn > HILS_NEG_INF) tot2 = mx + __builtin_amdgcn_logf(1.f + __builtin_amdgcn_exp2f(mn - mx));
-    lse_tot[i] = tot2 * HILS_LN2;
+    // a row that does not exist (a padding head of a group of three, a query past the end) must not
+    // reach the selection: its logits are not masked in the blocks every real row sees (they are 0 there)
+    lse_tot[i] = rowok[i] ? tot2 * HILS_LN2 : __builtin_inff();
     if (lse_total_out && col == 0 && rowok[i]) {
       const int r = 4 * j + i;
       lse_total_out[((b * L + t0 + r / GMAX) * (long)h_kv + hk) * G + r % GMAX] = lse_tot[i];

@@ -146,12 +146,15 @@ def test_topk_one_kernel_path_many_chunks(pkg, orc, dev):
              one_kernel=True)
 
 
-@pytest.mark.parametrize("G,D,L,N,topk,W", [(4, 128, 2050, 33, 32, 1), (2, 64, 777, 13, 8, 64),
-                                            (3, 128, 300, 5, 4, 1), (4, 64, 40, 600, 16, 1)])
-def test_topk_inference_variant_matches_export_variant(pkg, dev, G, D, L, N, topk, W):
+@pytest.mark.parametrize("G,D,L,N,topk,W,S", [(4, 128, 2050, 33, 32, 1, 64), (2, 64, 777, 13, 8, 64, 64),
+                                              (3, 128, 300, 5, 4, 1, 64), (4, 64, 40, 600, 16, 1, 64),
+                                              (3, 64, 9000, 150, 9, 1, 64),
+                                              # a chunk size that is no power of two (visibility by division)
+                                              (4, 128, 6000, 125, 16, 1, 48), (1, 64, 5000, 50, 7, 30, 100)])
+def test_topk_inference_variant_matches_export_variant(pkg, dev, G, D, L, N, topk, W, S):
     """The kernel variant without logit export / bias / noise / drop mask (the one inference
     runs) must give the same indices and scores as the exporting variant checked above."""
-    note(f"topk plain-vs-export G{G} D{D} L{L} N{N} k{topk} W{W}")
+    note(f"topk plain-vs-export G{G} D{D} L{L} N{N} k{topk} W{W} S{S}")
     gen = torch.Generator().manual_seed(123)
     h_kv = 2
     q = torch.randn(1, L, h_kv, G, D, generator=gen).bfloat16().to(dev)
@@ -159,7 +162,7 @@ def test_topk_inference_variant_matches_export_variant(pkg, dev, G, D, L, N, top
     lmks[:, 1::2] = lmks[:, 0::2][:, : lmks[:, 1::2].shape[1]]  # exact ties
     lmks = lmks.to(dev)
     lse = (torch.randn(1, L, h_kv * G, generator=gen) * 3 + 5).to(dev)
-    off = max(0, N * 64 - L)
+    off = max(0, N * S - L)
     outs = []
     for dbg in ({"no_workspace": True}, None):
         if dbg is None:
@@ -168,9 +171,9 @@ def test_topk_inference_variant_matches_export_variant(pkg, dev, G, D, L, N, top
             sc = torch.empty(1, L, h_kv, G, topk, dtype=torch.bfloat16, device=dev)
             _cabi.call("hils_topk_fwd", _cabi.ptr(q), _cabi.ptr(lmks), _cabi.ptr(lse.view(1, L, h_kv, G).contiguous()),
                        None, None, None, _cabi.ptr(idx), _cabi.ptr(sc), None, None, None, 1, L, N, h_kv, G, D,
-                       topk, 64, W, 1, off, 0, D ** -0.5)
+                       topk, S, W, 1, off, 0, D ** -0.5)
         else:
-            idx, sc = pkg.online_softmax_topk_head(q, lmks, lse, topk, 64, W, q_offset=off,
+            idx, sc = pkg.online_softmax_topk_head(q, lmks, lse, topk, S, W, q_offset=off,
                                                    is_training=False, _debug=dbg)
             sc = sc.view(1, L, h_kv, G, topk)
         torch.cuda.synchronize()
@@ -319,6 +322,34 @@ def test_topk_one_pass_prefill_kernel(pkg, orc, dev, L, N, h_kv, G, D, topk, dup
     winners): logits, lse_total, bit-exact selection, order, scores, across its head groupings."""
     run_case(pkg, orc, dev, B=1, L=L, N=N, h_kv=h_kv, G=G, D=D, topk=topk, S=64, W=1, seed=61,
              dup_keys=dup, training=False)
+
+
+@pytest.mark.parametrize("G,D,L,N,topk,W,S,h_kv", [
+    (4, 128, 12800, 200, 32, 1, 64, 2),   # queries of the 8- and 16-block launches
+    (4, 64, 32000, 500, 32, 1, 64, 1),    # all three launches
+    (1, 64, 9000, 250, 16, 1, 64, 2),     # 16 queries per wavefront
+    (3, 128, 7000, 140, 9, 64, 64, 1),    # a padding head row, odd k, a wide window
+    (4, 128, 6000, 125, 16, 1, 48, 1),    # chunk sizes that are no power of two (visibility by division)
+    (1, 64, 5000, 50, 7, 30, 100, 2)])
+def test_topk_one_pass_kernel_launches_match_export_variant(pkg, dev, G, D, L, N, topk, W, S, h_kv):
+    """The one-pass prefill kernel as inference launches it (one instantiation per range of visible
+    chunk counts, no logit export) against its exporting instantiation, which the cases above check
+    against the oracle; pairs of identical chunk keys put exact ties at the threshold."""
+    note(f"one-pass top-k launches G{G} D{D} L{L} N{N} k{topk} W{W} S{S}")
+    gen = torch.Generator().manual_seed(321)
+    q = torch.randn(1, L, h_kv * G, D, generator=gen).bfloat16().to(dev)
+    lmks = torch.randn(1, N, h_kv, D, generator=gen).bfloat16()
+    lmks[:, 1::2] = lmks[:, 0::2][:, : lmks[:, 1::2].shape[1]]
+    lmks = lmks.to(dev)
+    lse = (torch.randn(1, L, h_kv * G, generator=gen) * 3 + 5).to(dev)
+    off = max(0, N * S - L)
+    dbg = {}
+    idx0, sc0 = pkg.online_softmax_topk_head(q, lmks, lse, topk, S, W, q_offset=off, is_training=False, _debug=dbg)
+    idx1, sc1 = pkg.online_softmax_topk_head(q, lmks, lse, topk, S, W, q_offset=off, is_training=False)
+    assert torch.equal(idx0, idx1), "indices differ between the launches and the exporting variant"
+    assert torch.equal(sc0.view(torch.int16), sc1.view(torch.int16)), "scores differ"
+    lim = torch.div(torch.arange(L, device=dev) + off - W + 1, S, rounding_mode="floor").clamp(0, N)
+    assert torch.equal((idx1 >= 0).sum(-1), lim.clamp_max(topk).view(1, L, 1).expand(1, L, h_kv))
 
 
 def test_topk_one_pass_kernel_all_scores_equal(pkg, orc, dev):
