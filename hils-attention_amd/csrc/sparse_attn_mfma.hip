@@ -15,6 +15,9 @@
 #include "../../include/hils_amd.h"
 
 #define GA_THREADS 512
+#ifndef GA_THREADS_NARROW
+#define GA_THREADS_NARROW 768  // D = Dv = 64
+#endif
 #define GA_WAVES (GA_THREADS / 64)
 #define GA_S 64                 // chunk size this kernel is built for
 #define GA_MAXP 16              // (query, slot) pairs of a block per thread
@@ -160,8 +163,8 @@ struct GaTile {
 // The scale is chosen per output row from bound = sum_k |w_row,k| * max_visited|V|, which
 // bounds every element of the row because each P row is a convex combination: a row keeps
 // 20 bits below its own bound however small its weights are beside its neighbours'.
-template <int D, int DV, int G, bool SLOPE>
-__global__ void __launch_bounds__(GA_THREADS)
+template <int D, int DV, int G, bool SLOPE, int NT>
+__global__ void __launch_bounds__(NT)
 sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* __restrict__ kp,
                        const bf16_t* __restrict__ vp, const float* __restrict__ vmax,
                        const bf16_t* __restrict__ weights, const int32_t* __restrict__ indices,
@@ -170,7 +173,6 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
   constexpr int KS = D / 32;    // k-steps of S^T = K Q^T
   constexpr int DT = DV / 16;   // 16-wide output column tiles
   constexpr int QT = 16 / G;    // queries per 16-row tile
-  constexpr int NT = GA_THREADS;
   constexpr int MAXP = GA_MAXP;  // pairs per thread: T*K <= MAXP * GA_THREADS
   typedef GaTile<KS> Tile;
   extern __shared__ __align__(16) int smem_i[];
@@ -684,10 +686,13 @@ static int ga_launch_s(dim3 grid, size_t smem, hipStream_t st, const bf16_t* q, 
                        const bf16_t* vt, const float* vmax, const bf16_t* w, const int32_t* idx,
                        const float* slope, const bf16_t* swa_o, bf16_t* o, float* lse, const GaDims& dm) {
   static_assert(D % 32 == 0 && DV % 16 == 0 && 16 % G == 0, "tile shapes of the MFMA forward");
-  auto kern = sparse_attn_fwd_gather<D, DV, G, SLOPE>;
+  // Narrow heads leave the wavefronts under 168 registers: twelve of them per workgroup (one workgroup
+  // per compute unit, its size is what sets the occupancy) instead of eight.
+  constexpr int NT = (D <= 64 && DV <= 64) ? GA_THREADS_NARROW : GA_THREADS;
+  auto kern = sparse_attn_fwd_gather<D, DV, G, SLOPE, NT>;
   static HilsLdsReserve reserved;  // per instantiation
   if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_sparse_attn_fwd")) return rc;
-  hipLaunchKernelGGL(kern, grid, dim3(GA_THREADS), smem, st, q, qp, k, vt, vmax, w, idx, slope, swa_o, o, lse, dm);
+  hipLaunchKernelGGL(kern, grid, dim3(NT), smem, st, q, qp, k, vt, vmax, w, idx, slope, swa_o, o, lse, dm);
   return HILS_OK;
 }
 
