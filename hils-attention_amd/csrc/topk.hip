@@ -1676,7 +1676,7 @@ bool hils_topk_group_covers(int N, int G, int D, int topk, int per_qhead, bool p
 int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* lse_swa, int32_t* indices,
                            void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
                            int G, int D, int topk, int block_size, int window_size, int causal, int q_offset,
-                           float sm_scale, void* stream);
+                           float sm_scale, int lse_bf16, void* stream);
 
 // rows = (query, KV head) pairs; the row kernel wants about one row per compute unit
 static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool plain) {
@@ -1818,6 +1818,15 @@ static bool topk_use_split(int B, int L, int N, int h_kv) {
   return fused_wgs < 2L * topk_cus() && N >= 256 && N <= 16384;
 }
 
+// Shapes that hils_topk_fwd_weights hands to the one-pass prefill kernel, the only one that reads
+// lse_swa in bf16 (mirrors the dispatch of topk_fwd_impl; the workspace must be given).
+extern "C" int hils_topk_lse16_covers(int B, int L, int N, int h_kv, int G, int D, int topk) {
+  if (B <= 0 || L <= 0 || N <= 0 || h_kv <= 0 || G <= 0) return 0;
+  if (topk_use_split(B, L, N, h_kv)) return 0;
+  if (L <= 4 && topk_use_row((long)B * L * h_kv, N, G, D, 0, true)) return 0;
+  return hils_topk_group_covers(N, G, D, topk, 0, true) ? 1 : 0;
+}
+
 extern "C" size_t hils_topk_fwd_workspace(int B, int L, int N, int h_kv, int G) {
   // many queries: room for the chunk keys repacked into MFMA operand order (head dim up to 128)
   if (!topk_use_split(B, L, N, h_kv))
@@ -1868,7 +1877,8 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
                          int32_t* indices, void* scores, float* lse_total, float* sel_logits,
                          void* workspace, void* weights, int* weights_fused, int B, int L, int N,
                          int h_kv, int G, int D, int topk, int block_size, int window_size,
-                         int causal, int q_offset, int per_qhead, float sm_scale, void* stream) {
+                         int causal, int q_offset, int per_qhead, float sm_scale, void* stream,
+                         int lse_bf16 = 0) {
   HILS_REQUIRE(q && lmks && lse_swa && indices && scores, "hils_topk_fwd: null pointer");
   HILS_REQUIRE(B > 0 && L > 0 && N > 0 && h_kv > 0 && G > 0 && D > 0, "hils_topk_fwd: sizes must be positive");
   HILS_REQUIRE(topk >= 1 && topk <= TOPK_MAXK, "hils_topk_fwd: topk (%d) must be in 1..%d", topk, TOPK_MAXK);
@@ -1876,6 +1886,9 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
   HILS_REQUIRE(block_size > 0, "hils_topk_fwd: block_size must be positive");
   HILS_REQUIRE(h_kv <= 65535 && B <= 65535, "hils_topk_fwd: h_kv/B too large for the grid");
   hipStream_t st = (hipStream_t)stream;
+  HILS_REQUIRE(!lse_bf16 || hils_topk_lse16_covers(B, L, N, h_kv, G, D, topk),
+               "hils_topk_fwd_weights_lse16: shape not taken by the one-pass prefill kernel "
+               "(ask hils_topk_lse16_covers and pass lse_swa in fp32 otherwise)");
   // few queries per (batch, KV head) (decode, short continuations): one workgroup per row whenever
   // there are enough rows to occupy the machine, however many more there are
   if ((topk_use_split(B, L, N, h_kv) || L <= 4) &&
@@ -1917,7 +1930,7 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
       if (hils_topk_group_covers(N, G, D, topk, per_qhead, !bias && !gumbel && !drop_mask)) {
         if (int rc2 = hils_topk_group_launch(q, packed, lse_swa, indices, scores, lse_total, sel_logits, B, L, N,
                                              h_kv, G, D, topk, block_size, window_size, causal, q_offset,
-                                             sm_scale, stream))
+                                             sm_scale, lse_bf16, stream))
           return rc2;
         HILS_CHECK_LAUNCH("hils_topk_fwd");
         return HILS_OK;
@@ -1992,6 +2005,22 @@ extern "C" int hils_topk_fwd_weights(const void* q, const void* lmks, const floa
     return rc;
   if (fused) return HILS_OK;
   return hils_chunk_weights(scores, lse_swa, 0, nullptr, nullptr, weights, B, L, h_kv * G, h_kv, N, topk, 0,
+                            stream);
+}
+
+extern "C" int hils_topk_fwd_weights_lse16(const void* q, const void* lmks, const void* lse_swa_bf16,
+                                           int32_t* indices, void* scores, void* weights, void* workspace,
+                                           int B, int L, int N, int h_kv, int G, int D, int topk,
+                                           int block_size, int window_size, int causal, int q_offset,
+                                           float sm_scale, void* stream) {
+  HILS_REQUIRE(weights && workspace, "hils_topk_fwd_weights_lse16: null pointer");
+  int fused = 0;
+  if (int rc = topk_fwd_impl(q, lmks, (const float*)lse_swa_bf16, nullptr, nullptr, nullptr, indices, scores,
+                             nullptr, nullptr, workspace, weights, &fused, B, L, N, h_kv, G, D, topk,
+                             block_size, window_size, causal, q_offset, 0, sm_scale, stream, 1))
+    return rc;
+  if (fused) return HILS_OK;
+  return hils_chunk_weights(scores, lse_swa_bf16, 1, nullptr, nullptr, weights, B, L, h_kv * G, h_kv, N, topk, 0,
                             stream);
 }
 

@@ -133,7 +133,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
                       bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
                       float* __restrict__ sel_logits_out, int L, int N, int h_kv, int G, int topk,
                       int block_size, int window_size, int causal, int q_offset, float sm_scale,
-                      int t_base, int t_end, int bs_shift) {
+                      int t_base, int t_end, int bs_shift, int lse_bf16) {
   constexpr int D = KS * 32;
   constexpr int QPL = 4 / GMAX;   // queries per lane (its four accumulator rows)
   constexpr int NQ = 16 / GMAX;   // queries per wavefront
@@ -195,7 +195,9 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   for (int i = 0; i < 4; ++i) {
     const int r = 4 * j + i;
     const int tq = t0 + r / GMAX, g = r % GMAX;
-    const float x = lse_swa[((b * L + (rowok[i] ? tq : t0)) * (long)h_kv + hk) * G + (rowok[i] ? g : 0)];
+    const long li = ((b * L + (rowok[i] ? tq : t0)) * (long)h_kv + hk) * G + (rowok[i] ? g : 0);
+    float x;  // the layer hands lse_swa over in its hidden dtype (hils_attention.py:547)
+    if (lse_bf16) x = bf2f(((const bf16_t*)lse_swa)[li]); else x = lse_swa[li];
     swa[i] = rowok[i] ? x : HILS_NEG_INF;
   }
 
@@ -488,11 +490,12 @@ template <int GMAX, int KS>
 static void tg_launch_range(int NB, bool exp, dim3 grid, hipStream_t st, const bf16_t* q, const uint4* pk,
                             const float* lse_swa, int32_t* indices, bf16_t* scores, float* lse_total,
                             float* sel_logits, int L, int N, int h_kv, int G, int topk, int block_size,
-                            int window_size, int causal, int q_offset, float sm_scale, int t_base, int t_end) {
+                            int window_size, int causal, int q_offset, float sm_scale, int t_base, int t_end,
+                            int lse_bf16) {
 #define TG_CALL(NB_, EX_)                                                                              \
   hipLaunchKernelGGL((topk_fwd_group_kernel<GMAX, KS, NB_, EX_>), grid, dim3(64 * TG_WAVES), 0, st, q, pk, lse_swa, \
                      indices, scores, lse_total, sel_logits, L, N, h_kv, G, topk, block_size, window_size, \
-                     causal, q_offset, sm_scale, t_base, t_end, bs_shift)
+                     causal, q_offset, sm_scale, t_base, t_end, bs_shift, lse_bf16)
   const int bs_shift = (block_size > 0 && (block_size & (block_size - 1)) == 0) ? __builtin_ctz(block_size) : -1;
   if (exp) { TG_CALL(32, true); return; }
   switch (NB) {
@@ -508,7 +511,7 @@ static void tg_launch_range(int NB, bool exp, dim3 grid, hipStream_t st, const b
 int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* lse_swa, int32_t* indices,
                            void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
                            int G, int D, int topk, int block_size, int window_size, int causal, int q_offset,
-                           float sm_scale, void* stream) {
+                           float sm_scale, int lse_bf16, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   const int GM = (G == 1) ? 1 : 4;
   const int NQ = 16 / GM;
@@ -537,7 +540,7 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
 #define TG_RANGE(G_, KS_)                                                                             \
   tg_launch_range<G_, KS_>(NB, exp, grid, st, (const bf16_t*)q, (const uint4*)lmk_packed, lse_swa, indices, \
                            (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk, block_size,   \
-                           window_size, causal, q_offset, sm_scale, t, t_hi)
+                           window_size, causal, q_offset, sm_scale, t, t_hi, lse_bf16)
     if (GM == 1) { if (D == 64) TG_RANGE(1, 2); else TG_RANGE(1, 4); }
     else { if (D == 64) TG_RANGE(4, 2); else TG_RANGE(4, 4); }
 #undef TG_RANGE

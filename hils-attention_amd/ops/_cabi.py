@@ -25,6 +25,7 @@ SIGNATURES = {
     "hils_topk_fwd": [_P] * 11 + [_I] * 12 + [_F, _P],
     "hils_topk_fwd_noalloc": [_P] * 10 + [_I] * 12 + [_F, _P],
     "hils_topk_fwd_weights": [_P] * 10 + [_I] * 12 + [_F, _P],
+    "hils_topk_fwd_weights_lse16": [_P] * 7 + [_I] * 11 + [_F, _P],
     "hils_topk_fwd_weights_paged": [_P] * 9 + [_I] * 12 + [_F, _P],
     "hils_sparse_attn_decode_paged": [_P] * 8 + [_I] * 9 + [_F, _I, _P],
     "hils_decode_step": [_P] * 11 + [_I] * 11 + [_F, _F, _I, _P],
@@ -72,6 +73,8 @@ def load():
     lib.hils_sparse_attn_decode_paged_workspace.argtypes = [_I] * 6
     lib.hils_stream_probe.restype = c_int
     lib.hils_stream_probe.argtypes = [_P, ctypes.c_size_t, _I, _P, _P]
+    lib.hils_topk_lse16_covers.restype = c_int
+    lib.hils_topk_lse16_covers.argtypes = [_I] * 7
     lib.hils_decode_step_covers.restype = c_int
     lib.hils_decode_step_covers.argtypes = [_I] * 8
     lib.hils_sparse_attn_fwd_workspace.restype = ctypes.c_size_t

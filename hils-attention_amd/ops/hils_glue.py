@@ -87,11 +87,19 @@ def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causa
     G = h_q // h_kv
     scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(D)
     dev = q.device
-    lse = lse_swa.reshape(B, L, h_q).float().contiguous()
     indices = torch.empty((B, L, h_kv, topk), dtype=torch.int32, device=dev)
     scores = torch.empty((B, L, h_q, topk), dtype=q.dtype, device=dev)
     weights = torch.empty((B, L, h_q, topk + 1), dtype=q.dtype, device=dev)
     ws = _cabi.topk_fwd_workspace(dev, B, L, N, h_kv, G)
+    if (lse_swa.dtype == torch.bfloat16 and ws is not None
+            and _cabi.load().hils_topk_lse16_covers(B, L, N, h_kv, G, D, int(topk))):
+        # lse_swa as the layer hands it over (bf16): read in place, no conversion pass
+        _cabi.call("hils_topk_fwd_weights_lse16", _cabi.ptr(q.contiguous()), _cabi.ptr(lmks.contiguous()),
+                   _cabi.ptr(lse_swa.reshape(B, L, h_q).contiguous()), _cabi.ptr(indices), _cabi.ptr(scores),
+                   _cabi.ptr(weights), _cabi.ptr(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),
+                   int(window_size), int(bool(is_causal)), int(q_offset), scale)
+        return indices, scores, weights
+    lse = lse_swa.reshape(B, L, h_q).float().contiguous()
     _cabi.call("hils_topk_fwd_weights", _cabi.ptr(q.contiguous()), _cabi.ptr(lmks.contiguous()),
                _cabi.ptr(lse), None, None, None, _cabi.ptr(indices), _cabi.ptr(scores),
                _cabi.ptr(weights), _cabi.ptr(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),

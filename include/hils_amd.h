@@ -104,6 +104,18 @@ int hils_topk_fwd_weights(const void* q, const void* lmks, const float* lse_swa,
                           int G, int D, int topk, int block_size, int window_size, int causal,
                           int q_offset, int per_qhead, float sm_scale, void* stream);
 
+/* hils_topk_fwd_weights for lse_swa in bf16, the dtype the reference's layer hands it over in
+ * (lse_sum.to(hidden_states.dtype), models/FlashHiLS/hils_attention.py:547; its kernels read it in
+ * that dtype, ops/topk_head_softmax.py:1291-1367): saves the conversion pass.  Only the shapes
+ * hils_topk_lse16_covers accepts (many queries, shared chunk keys, G in {1,3,4}, N <= 512, topk <= 32,
+ * no bias / noise / drop mask: the one-pass prefill kernel), with the workspace of
+ * hils_topk_fwd_workspace; other shapes are rejected and take hils_topk_fwd_weights with fp32. */
+int hils_topk_lse16_covers(int B, int L, int N, int h_kv, int G, int D, int topk);
+int hils_topk_fwd_weights_lse16(const void* q, const void* lmks, const void* lse_swa_bf16, int32_t* indices,
+                                void* scores, void* weights, void* workspace, int B, int L, int N, int h_kv,
+                                int G, int D, int topk, int block_size, int window_size, int causal,
+                                int q_offset, float sm_scale, void* stream);
+
 /* Sparse backward of the score gather.  Replaces the dense scatter + two torch.bmm of
  * SoftmaxTopKMaxPoolingFusedFn.backward (ops/topk_head_softmax.py:1040-1092).
  * g_scores (B,L,h_kv,G,topk) bf16 -> dq (B,L,h_kv,G,D) bf16 (written),

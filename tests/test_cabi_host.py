@@ -42,6 +42,7 @@ def test_binding_matches_header(pkg):
     fns.pop("hils_topk_fwd_noalloc_max_workspace")
     fns.pop("hils_sparse_attn_decode_paged_workspace")
     fns.pop("hils_decode_step_covers")
+    fns.pop("hils_topk_lse16_covers")
     fns.pop("hils_stream_probe")
     assert set(_cabi.SIGNATURES) == set(fns)
     for name, params in fns.items():

@@ -114,6 +114,24 @@ def test_topk_with_fused_weights_matches_two_calls(pkg, dev, B, L, N, HQ, H, D, 
         assert torch.equal(w1.view(torch.int16), w0.view(torch.int16))
 
 
+@pytest.mark.parametrize("L,N,HQ,H,D,K", [(3000, 47, 8, 2, 128, 16), (9000, 300, 3, 1, 64, 32),
+                                          (2048, 32, 8, 4, 64, 8), (1500, 24, 16, 1, 128, 8)])
+def test_topk_weights_reads_bf16_lse_in_place(pkg, dev, L, N, HQ, H, D, K):
+    """lse_swa in bf16, as the layer hands it over: the one-pass prefill kernel reads it in place
+    (other shapes convert it first); either way the result is that of the fp32 copy of the same values."""
+    note(f"topk+weights bf16 lse L{L} N{N} HQ{HQ} H{H} D{D} K{K}")
+    gen = torch.Generator().manual_seed(78)
+    q = torch.randn(1, L, HQ, D, generator=gen).bfloat16().to(dev)
+    lmk = torch.randn(1, N, H, D, generator=gen).bfloat16().to(dev)
+    lse16 = (torch.randn(1, L, HQ, generator=gen) * 5 + 10).bfloat16().to(dev)
+    off = max(0, N * 64 - L)
+    idx0, sc0, w0 = pkg.topk_chunk_weights(q, lmk, lse16.float(), K, 64, 1, q_offset=off)
+    idx1, sc1, w1 = pkg.topk_chunk_weights(q, lmk, lse16, K, 64, 1, q_offset=off)
+    assert torch.equal(idx0, idx1)
+    assert torch.equal(sc0.view(torch.int16), sc1.view(torch.int16))
+    assert torch.equal(w0.view(torch.int16), w1.view(torch.int16))
+
+
 def test_decode_step_replays_as_hip_graph(pkg, orc, dev):
     """The decode step (selection + inter-chunk softmax, then sparse attention) captured as one HIP
     graph: every replay, with eager work and synchronisations in between and with new inputs
