@@ -569,11 +569,21 @@ sparse_attn_fwd_gather(const bf16_t* __restrict__ q, bf16_t* qp, const bf16_t* _
         for (int u = 0; u < 4; ++u)
           acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[s2], ga_bf(vb[d0 + u][s2]), acc[u], 0, 0, 0);
       if (reload) load_v_half(c_next, d0, 4);
+      if constexpr (G >= 4) {
+        // the lane's four rows are consecutive heads of one query: one address, the rest are offsets
+        // the instruction carries
+        int* o0 = o_acc + orow[0];
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < 4; ++u)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          atomicAdd(&o_acc[orow[i] + (d0 + u) * 16], __float_as_int(acc[u][i]));
+          for (int i = 0; i < 4; ++i) atomicAdd(o0 + i * DV + (d0 + u) * 16, __float_as_int(acc[u][i]));
+      } else {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            atomicAdd(&o_acc[orow[i] + (d0 + u) * 16], __float_as_int(acc[u][i]));
+      }
     }
   };
 
@@ -757,7 +767,7 @@ size_t hils_ga_workspace_bytes(int B, int L, int Lkv, int HQ, int H, int D, int 
   const bool ok = S == GA_S && (D == 64 || D == 128) && (Dv == 64 || Dv == 128) &&
                   (G == 1 || G == 2 || G == 4 || G == 8 || G == 16) && q_block >= 1 &&
                   L % q_block == 0 && (WH == HQ || WH == H) && sm_n >= 0.f && L >= 64 && Lkv >= S &&
-                  K >= 1 && K <= 256;
+                  K >= 1 && K <= 256 && (long)L * q_block < (1L << 31);  // hils_udiv by q_block stays exact
   if (!ok) return 0;
   size_t smem;
   const int T = ga_pick_T(L, G, Dv, K, Lkv / S, q_block, &smem);
