@@ -18,12 +18,23 @@ __global__ void mean_pool_fwd_kernel(const uint4* __restrict__ k, uint4* __restr
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (cg < cols8) {
     const uint4* base = k + (chunk * S) * (long)cols8 + cg;
-    for (int s = ts; s < S; s += TS) {
-      uint4 v = base[(long)s * cols8];
-      float f[8];
-      unpack8(v, f);
+    // four of the slice's rows in flight per lane (one load at a time left the kernel waiting a
+    // memory latency per row); rows past the chunk re-read its last row and add nothing
+    for (int s0 = ts; s0 < S; s0 += 4 * TS) {
+      uint4 v[4];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] += f[i];
+      for (int u = 0; u < 4; ++u) {
+        const int s = s0 + u * TS;
+        v[u] = base[(long)(s < S ? s : S - 1) * cols8];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        float f[8];
+        unpack8(v[u], f);
+        const float on = s0 + u * TS < S ? 1.f : 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(f[i], on, acc[i]);
+      }
     }
   }
   float* mine = smem + ((size_t)ts * blockDim.x + threadIdx.x) * 8;
