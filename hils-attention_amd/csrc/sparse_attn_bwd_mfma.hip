@@ -35,6 +35,35 @@ __global__ void bw_fill_int_kernel(int* p, int value, long n) {
 // ---------------------------------------------------------------------------
 // Inverse index: pairs (query << 8 | slot) grouped by (batch, KV head, chunk).
 // ---------------------------------------------------------------------------
+// The index entries (query t_lo + r, slot s) of one KV head for the queries of a segment, walked by a
+// workgroup of 1024: thread tid takes entries tid, tid + 1024, ... of the segment's rows x K entries
+// (consecutive threads read consecutive slots of a row).  (r, s) advance by (1024 / K, 1024 % K) per
+// step, so that nothing is divided inside the loop, and four loads are in flight per thread (a
+// clamped row is loaded for a step past the end and skipped).  f(t, slot, chunk).
+template <class F>
+__device__ __forceinline__ void bw_walk_indices(const int32_t* __restrict__ seg0, int t_lo, int rows, int H, int K,
+                                                F f) {
+  const int qK = 1024 / K, rK = 1024 % K;
+  int r = (int)threadIdx.x / K, sl = (int)threadIdx.x - r * K;
+  const long rstride = (long)H * K;
+  while (r < rows) {
+    int rr[4], ss[4], cc[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      rr[u] = r;
+      ss[u] = sl;
+      sl += rK;
+      r += qK;
+      if (sl >= K) { sl -= K; ++r; }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) cc[u] = seg0[(long)(rr[u] < rows ? rr[u] : rows - 1) * rstride + ss[u]];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (rr[u] < rows) f(t_lo + rr[u], ss[u], cc[u]);
+  }
+}
+
 // counts[(b*H + h) * nchunk + c] = number of valid entries equal to c; one workgroup per
 // (batch, KV head, segment of queries), LDS histogram first.
 __global__ void __launch_bounds__(1024)
@@ -47,12 +76,10 @@ bw_count_kernel(const int32_t* __restrict__ indices, int* __restrict__ counts, i
   const int t_hi = (t_lo + seg_len < L) ? t_lo + seg_len : L;
   for (int i = threadIdx.x; i < nchunk; i += 1024) hist[i] = 0;
   __syncthreads();
-  const long n = (long)(t_hi - t_lo) * K;
-  for (long i = threadIdx.x; i < n; i += 1024) {
-    const int t = t_lo + (int)(i / K), slot = (int)(i % K);
-    const int c = indices[((b * L + t) * H + h) * (long)K + slot];
+  const int32_t* seg0 = indices + ((b * L + t_lo) * H + h) * (long)K;
+  bw_walk_indices(seg0, t_lo, t_hi - t_lo, H, K, [&](int, int, int c) {
     if (c >= 0 && c < nchunk) atomicAdd(&hist[c], 1);
-  }
+  });
   __syncthreads();
   int* out = counts + (b * H + h) * (long)nchunk;
   for (int i = threadIdx.x; i < nchunk; i += 1024)
@@ -104,23 +131,19 @@ bw_scatter_kernel(const int32_t* __restrict__ indices, int* __restrict__ cursor,
   int* cur = cursor + (b * H + h) * (long)nchunk;
   for (int i = threadIdx.x; i < nchunk; i += 1024) pos[i] = 0;
   __syncthreads();
-  const long n = (long)(t_hi - t_lo) * K;
-  for (long i = threadIdx.x; i < n; i += 1024) {
-    const int t = t_lo + (int)(i / K), slot = (int)(i % K);
-    const int c = indices[((b * L + t) * H + h) * (long)K + slot];
+  const int32_t* seg0 = indices + ((b * L + t_lo) * H + h) * (long)K;
+  bw_walk_indices(seg0, t_lo, t_hi - t_lo, H, K, [&](int, int, int c) {
     if (c >= 0 && c < nchunk) atomicAdd(&pos[c], 1);
-  }
+  });
   __syncthreads();
   for (int i = threadIdx.x; i < nchunk; i += 1024) {
     const int cnt = pos[i];
     pos[i] = cnt ? atomicAdd(&cur[i], cnt) : 0;
   }
   __syncthreads();
-  for (long i = threadIdx.x; i < n; i += 1024) {
-    const int t = t_lo + (int)(i / K), slot = (int)(i % K);
-    const int c = indices[((b * L + t) * H + h) * (long)K + slot];
+  bw_walk_indices(seg0, t_lo, t_hi - t_lo, H, K, [&](int t, int slot, int c) {
     if (c >= 0 && c < nchunk) pairs[atomicAdd(&pos[c], 1)] = ((uint32_t)t << 8) | (uint32_t)slot;
-  }
+  });
 }
 
 // ---------------------------------------------------------------------------
