@@ -7,14 +7,15 @@
 // nt*16+col, so a query's logits for up to 512 chunks lie in the 16 lanes of one lane row, 32 per
 // lane.  From there, without touching memory again:
 //   * the log-sum-exp of every row (in-lane maxima and sums, one 16-lane reduction per row),
-//   * the selection key of every (query, chunk): max over the heads of logit - lse_total, as an
-//     order-preserving unsigned key (in-lane: the heads of a query are registers of one lane),
+//   * the selection score of every (query, chunk): max over the heads of logit - lse_total, a float
+//     (in-lane: the heads of a query are registers of one lane),
 //   * the top-K per query, the four lane rows working on four queries at once: the K-th largest
-//     key is bracketed from the two largest keys of every lane (their minimum over the lanes is a
-//     lower bound with at least 32 keys above it), the keys above the bound (about 1.5 K of 512)
-//     are compacted through LDS to at most 8 per lane and the exact threshold is found on those by
-//     a bitwise search whose counts are 16-lane DPP reductions (no ballots, no scalar round trip);
-//     ties at the threshold go to the lower chunk indices,
+//     score is bracketed from the two largest scores of every lane (their minimum over the lanes is
+//     a lower bound with at least 32 scores above it), the scores above the bound (about 1.5 K of
+//     512) are compacted through LDS to at most 8 per lane, turned into order-preserving unsigned
+//     keys, and the threshold is found on those by a bitwise search whose counts are 16-lane DPP
+//     reductions (no ballots, no scalar round trip) and which stops at the first probe that counts
+//     exactly K; ties at the threshold go to the lower chunk indices,
 //   * the ascending order of the winners from a 512-bit map of the winning chunks in LDS
 //     (rank = set bits below the chunk), and the winners' raw scores straight from the logits.
 // Covers shared chunk keys, G <= 4, D in {64, 128}, N <= 512, topk <= 32, no bias / Gumbel noise /
