@@ -125,7 +125,10 @@ __device__ __forceinline__ uint32_t tg_kth_largest(const uint32_t (&k)[NE], uint
 // early queries do not pay for 32.  (A 24-block instantiation for the queries that see 257..384
 // chunks ran no faster than this kernel at 32; the time goes by the schedule the compiler finds at
 // the given register budget as much as by the work.)
-#define TG_WAVES 4  // wavefronts per workgroup, each with queries of its own (they never synchronise)
+// Wavefronts per workgroup, each with queries of its own (they never synchronise).  A workgroup keeps
+// its registers and LDS until its slowest wavefront is through (the threshold searches differ in
+// length): 4 per workgroup ran 3.5 % slower than 2, and 8 ran 17 % slower; 1 was no faster than 2.
+#define TG_WAVES 2
 template <int GMAX, int KS, int NB, bool EXPORT>
 __global__ void __launch_bounds__(64 * TG_WAVES)
     __attribute__((amdgpu_waves_per_eu(NB <= 8 ? 5 : (NB <= 16 ? 4 : 2))))
