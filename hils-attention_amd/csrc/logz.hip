@@ -156,19 +156,21 @@ logz_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
       }
 #pragma unroll
     for (int rt = 0; rt < LZM_RT; ++rt) {
+      // the maximum is taken over the raw products (the scale is positive) and the scale is applied
+      // inside the exponent's fused multiply-add: no separate scaling pass
       float x[16];
 #pragma unroll
       for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) x[tt * 4 + i] = acc[rt][tt][i] * sc2;
+        for (int i = 0; i < 4; ++i) x[tt * 4 + i] = acc[rt][tt][i];
       if (dm.mask_lmk && j == 3) x[15] = HILS_NEG_INF;  // token 63 = tile 3, lane row 3, register 3
-      float m = x[0];
+      float m = fmaxf(x[0], x[1]);
 #pragma unroll
-      for (int i = 1; i < 16; ++i) m = fmaxf(m, x[i]);
-      m = rows_max(m);
+      for (int i = 2; i < 16; i += 2) m = fmaxf(fmaxf(m, x[i]), x[i + 1]);
+      m = rows_max(m) * sc2;  // in log2 units, as the sum below
       float s = 0.f;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s += __builtin_amdgcn_exp2f(x[i] - m);
+      for (int i = 0; i < 16; ++i) s += __builtin_amdgcn_exp2f(fmaf(x[i], sc2, -m));
       s = rows_sum(s);
       const float val = (c < lim[rt]) ? (m + __builtin_amdgcn_logf(s)) * HILS_LN2 : HILS_NEG_INF;
       if (j == (c & 3)) keep[rt] = val;
