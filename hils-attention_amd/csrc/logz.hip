@@ -71,8 +71,11 @@ logz_fwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
 // K Q^T so that the 64 tokens of one row lie in 16 registers of 4 lanes: the log-sum-exp is an
 // in-lane reduction plus one row-swap reduction.
 #define LZM_RT 2  // 16-row tiles per wavefront
+// (the occupancy hint also keeps the score accumulators in ordinary registers: without it the
+// compiler, free to use 512 registers at this workgroup size, parks them in accumulation registers
+// and copies every score back for the softmax)
 template <int D, int G>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3)))
 logz_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
               float* __restrict__ log_z, LzDims dm, int n_qt) {
   constexpr int KS = D / 32;
@@ -205,7 +208,7 @@ logz_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
 // the gradient product.
 // dQ: a wavefront owns 32 score rows (query x head), the chunks' keys stream.
 template <int D, int G>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 logz_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                  const float* __restrict__ log_z, const float* __restrict__ d_log_z,
                  bf16_t* __restrict__ dq, LzDims dm, int n_qt) {
@@ -334,7 +337,7 @@ logz_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
 // dK: a workgroup owns two chunks (wavefront: 32 tokens of one chunk), the score rows of the
 // queries behind them stream in tiles of 64 rows (64/G queries x G heads).
 template <int D, int G>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 logz_bwd_dk_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                  const float* __restrict__ log_z, const float* __restrict__ d_log_z,
                  bf16_t* __restrict__ dk, LzDims dm) {
