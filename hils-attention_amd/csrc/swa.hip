@@ -379,7 +379,9 @@ __device__ __forceinline__ unsigned swa_lmk_bits(const SwaDims& dm, int tok0) {
 
 // dQ (and delta): a wavefront owns 32 score rows; K (row-major and transposed) and V stream.
 template <int D, int DV, int G>
-__global__ void __launch_bounds__(256)
+// (narrow heads fit 256 registers: the hint then gives two wavefronts per SIMD and keeps the
+// accumulators out of accumulation registers; wide heads need more and run one wavefront per SIMD)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((D <= 64 && DV <= 64) ? 2 : 1)))
 swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
                 const bf16_t* __restrict__ o, const float* __restrict__ lse,
                 const bf16_t* __restrict__ d_o, const float* __restrict__ d_lse,
@@ -552,7 +554,9 @@ swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, cons
 // score rows (query x head) that can see them stream in tiles of 64 rows, Q and dO both row-major
 // and transposed, with the rows' lse, delta and window start beside them.
 template <int D, int DV, int G>
-__global__ void __launch_bounds__(256)
+// (narrow heads fit 256 registers: the hint then gives two wavefronts per SIMD and keeps the
+// accumulators out of accumulation registers; wide heads need more and run one wavefront per SIMD)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((D <= 64 && DV <= 64) ? 2 : 1)))
 swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                   const bf16_t* __restrict__ v, const float* __restrict__ lse,
                   const bf16_t* __restrict__ d_o, const float* __restrict__ delta_in,
