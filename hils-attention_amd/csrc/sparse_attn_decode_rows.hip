@@ -3,7 +3,7 @@
 #include "decode_rows_body.h"
 
 template <int D, int NWAVE>
-__global__ void __launch_bounds__(NWAVE * 64)
+__global__ void __launch_bounds__(NWAVE * 64) __attribute__((amdgpu_waves_per_eu(2)))
 sparse_attn_decode_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                const bf16_t* __restrict__ v, const bf16_t* __restrict__ weights,
                                const int32_t* __restrict__ indices, bf16_t* __restrict__ o,
