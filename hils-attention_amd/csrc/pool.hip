@@ -271,7 +271,7 @@ attn_pool_fwd_rows(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k
 // heads h = wave, wave + 4, ... with the dK sum in registers, the four sums meet in LDS (two
 // rounds), head 0 receives the total and heads 1..H-1 are zeroed.
 template <int D, bool SHARED>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 attn_pool_bwd_rows(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k,
                    const float* __restrict__ p_saved, const float* __restrict__ lmk_b,
                    const bf16_t* __restrict__ g_k, const float* __restrict__ g_b,
