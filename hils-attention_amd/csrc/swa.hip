@@ -18,31 +18,54 @@ struct SwaDims {
   float sm_scale;
 };
 
-// Forward.  A workgroup of eight wavefronts owns 256/G consecutive queries of one KV head: 32 score
+// Workgroup order.  Neighbouring blocks of a head read the same key / value (or query) tiles, and the
+// hardware hands consecutive workgroup ids to the 8 XCDs in turn: with the block index in the grid's
+// fastest dimension every tile was fetched from HBM by as many XCDs (L2s) as blocks share it.  The grids
+// here are one-dimensional, id -> (xcd, slot), and each XCD walks one contiguous share of the
+// (batch, head, block) list.  False for the padding ids of the last share.
+__device__ __forceinline__ bool swa_xcd_unit(int n_blk, int H, int B, int& blk, int& hk, long& b) {
+  const int total = n_blk * H * B;
+  const int per_xcd = (total + 7) / 8;
+  const int vid = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+  if (vid >= total) return false;
+  const int unit = vid / n_blk;
+  blk = vid - unit * n_blk;
+  hk = unit % H;
+  b = unit / H;
+  return true;
+}
+static dim3 swa_xcd_grid(int n_blk, int H, int B) { return dim3((unsigned)(((long)n_blk * H * B + 7) / 8 * 8)); }
+
+// Forward.  A workgroup of NWV wavefronts owns NWV*32/G consecutive queries of one KV head: 32 score
 // rows (query x head of the group) per wavefront, held as matrix B operands.  The keys and values the
 // block can see (its queries' windows: two or three 64-token tiles at window 64) are loaded once, all
 // loads in flight together, and stay in LDS row-major (rows padded by 16 bytes); a longer window is
-// worked through in phases of SWA_RES tiles.  S^T = K Q^T takes K rows as A operands, O += P V takes V
+// worked through in phases of RES resident tiles.  S^T = K Q^T takes K rows as A operands, O += P V takes V
 // through the transposing LDS load, in the token order in which the S^T accumulators hold P.  A
 // wavefront skips the tiles none of its rows can see and masks only the tiles that straddle a row's
 // window start, its diagonal, the end of the keys or a landmark; running max / sum per row as in
 // flash attention.
-#define SWA_RES 4      // tiles resident in LDS
+// Two shapes of workgroup.  Wide: eight wavefronts, four resident tiles (139 KiB of LDS at D = Dv =
+// 128, one workgroup per compute unit: its load, compute and store phases follow each other with
+// nothing to overlap them).  Narrow: four wavefronts, two resident tiles (70 KiB), two workgroups per
+// compute unit, one loading while the other computes; taken when no block of 128/G queries needs more
+// than two tiles (window <= 64 at chunk 64), at the price of every tile being staged by twice as many
+// workgroups (L2 hits).
 #define SWA_FWD_RT 2   // 16-row tiles per wavefront
-#define SWA_FWD_WAVES 8
+#define SWA_LAZY 6.f   // log2 of the growth of a row's maximum that moves its reference point
 
-template <int D, int DV>
+template <int D, int DV, int NWV, int RES>
 static size_t swa_fwd_smem() {
-  const size_t tiles = (size_t)SWA_RES * 64 * ((2 * D + 16) + (2 * DV + 16));
-  const size_t outs = (size_t)SWA_FWD_WAVES * 16 * SWA_FWD_RT * (2 * DV + 16);
-  return (tiles > outs ? tiles : outs) + (size_t)SWA_FWD_WAVES * SWA_FWD_RT * 16 * sizeof(float);
+  const size_t tiles = (size_t)RES * 64 * ((2 * D + 16) + (2 * DV + 16));
+  const size_t outs = (size_t)NWV * 16 * SWA_FWD_RT * (2 * DV + 16);
+  return (tiles > outs ? tiles : outs) + (size_t)NWV * SWA_FWD_RT * 16 * sizeof(float);
 }
 
-template <int D, int DV, int G>
-__global__ void __launch_bounds__(SWA_FWD_WAVES * 64)
+template <int D, int DV, int G, int NWV, int RES>
+__global__ void __launch_bounds__(NWV * 64) __attribute__((amdgpu_waves_per_eu(2)))
 swa_fwd_blk(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
-            bf16_t* __restrict__ o, float* __restrict__ lse, SwaDims dm, int n_qt) {
-  constexpr int RT = SWA_FWD_RT, NWV = SWA_FWD_WAVES, NT = NWV * 64;
+            bf16_t* __restrict__ o, float* __restrict__ lse, SwaDims dm, int n_qt, int n_b) {
+  constexpr int RT = SWA_FWD_RT, NT = NWV * 64;
   constexpr int KS = D / 32, DT = DV / 16;
   constexpr int QW = 16 * RT / G > 0 ? 16 * RT / G : 1;  // queries per wavefront (G <= 16: >= 2)
   constexpr int QB = NWV * 16 * RT / G;                  // queries per workgroup
@@ -57,7 +80,7 @@ swa_fwd_blk(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf
   typedef short swa_s4 __attribute__((ext_vector_type(4)));
   typedef short swa_s8 __attribute__((ext_vector_type(8)));
   extern __shared__ __align__(16) unsigned char swa_dyn[];
-  constexpr size_t TILES_B = (size_t)SWA_RES * TILE_B;
+  constexpr size_t TILES_B = (size_t)RES * TILE_B;
   constexpr size_t OUTS_B = (size_t)NWV * 16 * RT * OP;
   float* bc_all = (float*)(swa_dyn + (TILES_B > OUTS_B ? TILES_B : OUTS_B));  // [wave][rt][16] row factors
   const int tid = threadIdx.x, lane = tid & 63;
@@ -66,9 +89,10 @@ swa_fwd_blk(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, j = lane >> 4;
   float* bc_s = bc_all + wave * RT * 16;
-  const int qt = n_qt - 1 - (int)blockIdx.x;
-  const int hk = blockIdx.y;
-  const long b = blockIdx.z;
+  int qt, hk;
+  long b;
+  if (!swa_xcd_unit(n_qt, dm.H, n_b, qt, hk, b)) return;
+  qt = n_qt - 1 - qt;
   const int tq0 = qt * QB;
   const int t0 = tq0 + wave * QW;
   const int q_off = dm.kv_start + dm.Lk - dm.Lq;  // absolute position of query 0
@@ -143,6 +167,7 @@ swa_fwd_blk(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf
   // one resident tile: scores, masks where a row needs them, running softmax, O += P V
   auto tile_step = [&](int tile, const unsigned char* k_s, const unsigned char* v_s) __attribute__((always_inline)) {
     f32x4_t p[RT][4];  // scores, then probabilities: accumulator tiles (token tt*16 + 4j + i, row lane & 15)
+    bool rescale = false;
     {
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
@@ -198,10 +223,17 @@ swa_fwd_blk(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf
 #pragma unroll
           for (int i = 0; i < 4; ++i) mx = fmaxf(mx, p[rt][tt][i]);
         mx = rows_max(mx);
-        const float m_new = fmaxf(m_run[rt], mx);
+        // The reference point of the exponentials follows the running maximum only when that grows by
+        // more than 2^SWA_LAZY (or when the row has nothing accumulated yet): until then probabilities
+        // up to 2^SWA_LAZY enter sum and output alike, which the final division cancels, and the
+        // output accumulators need no rescaling (most tiles: the branch below is wavefront-uniform).
+        const bool fresh = l_run[rt] == 0.f;
+        const bool move = fresh | ((mx - m_run[rt]) * c2 > SWA_LAZY);
+        const float m_new = move ? fmaxf(m_run[rt], mx) : m_run[rt];
         const bool any = m_new > HILS_NEG_INF;
-        const float corr = any ? __builtin_amdgcn_exp2f((m_run[rt] - m_new) * c2) : 1.f;  // exp2(-inf) = 0
+        const float corr = (move & any & !fresh) ? __builtin_amdgcn_exp2f((m_run[rt] - m_new) * c2) : 1.f;
         const float mc = any ? m_new * c2 : 0.f;
+        rescale |= corr != 1.f;
         float sum = 0.f;
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
@@ -219,14 +251,16 @@ swa_fwd_blk(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf
     }
     __builtin_amdgcn_wave_barrier();
     // rescale the output accumulators: their rows are 4j+i, the factors live per lane & 15
+    if (__any(rescale)) {
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      const float4 c4 = *(const float4*)&bc_s[rt * 16 + 4 * j];
-      const float cf[4] = {c4.x, c4.y, c4.z, c4.w};
+      for (int rt = 0; rt < RT; ++rt) {
+        const float4 c4 = *(const float4*)&bc_s[rt * 16 + 4 * j];
+        const float cf[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[rt][dt][i] *= cf[i];
+          for (int i = 0; i < 4; ++i) acc[rt][dt][i] *= cf[i];
+      }
     }
     __builtin_amdgcn_wave_barrier();
     // O += P V: a lane's eight k-slots are tokens 4j..4j+3 of two neighbouring 16-token tiles; the
@@ -302,11 +336,11 @@ swa_fwd_blk(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf
       if (ti + 2 < N) issue(ti + 2, kr[ti & 1], vr[ti & 1]);
     }
   };
-  for (int tile0 = tile_lo; tile0 < tile_hi; tile0 += SWA_RES) {
+  for (int tile0 = tile_lo; tile0 < tile_hi; tile0 += RES) {
     if (tile0 != tile_lo) __syncthreads();  // the previous phase's tiles are no longer read
-    const int n = tile_hi - tile0 < SWA_RES ? tile_hi - tile0 : SWA_RES;
-    if (SWA_RES >= 4 && n == 4) phase(tile0, std::integral_constant<int, SWA_RES >= 4 ? 4 : 1>{});
-    else if (SWA_RES >= 3 && n == 3) phase(tile0, std::integral_constant<int, SWA_RES >= 3 ? 3 : 1>{});
+    const int n = tile_hi - tile0 < RES ? tile_hi - tile0 : RES;
+    if (RES >= 4 && n == 4) phase(tile0, std::integral_constant<int, RES >= 4 ? 4 : 1>{});
+    else if (RES >= 3 && n == 3) phase(tile0, std::integral_constant<int, RES >= 3 ? 3 : 1>{});
     else if (n == 2) phase(tile0, std::integral_constant<int, 2>{});
     else phase(tile0, std::integral_constant<int, 1>{});
     __syncthreads();
@@ -377,17 +411,25 @@ __device__ __forceinline__ unsigned swa_lmk_bits(const SwaDims& dm, int tok0) {
   return ok;
 }
 
+// 16-row tiles per wavefront of the backward kernels: two for narrow heads; one for wide heads, whose two
+// tiles need more than 256 registers (one wavefront per SIMD, nothing to overlap a wait with)
+#ifndef SWA_RT_NARROW
+#define SWA_RT_NARROW 2
+#endif
+constexpr int swa_dq_rt(int D, int DV) { return (D <= 64 && DV <= 64) ? SWA_RT_NARROW : 1; }
+
 // dQ (and delta): a wavefront owns 32 score rows; K (row-major and transposed) and V stream.
 template <int D, int DV, int G>
 // (narrow heads fit 256 registers: the hint then gives two wavefronts per SIMD and keeps the
 // accumulators out of accumulation registers; wide heads need more and run one wavefront per SIMD)
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((D <= 64 && DV <= 64) ? 2 : 1)))
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
                 const bf16_t* __restrict__ o, const float* __restrict__ lse,
                 const bf16_t* __restrict__ d_o, const float* __restrict__ d_lse,
-                bf16_t* __restrict__ dq, float* __restrict__ delta_out, SwaDims dm, int n_qt) {
+                bf16_t* __restrict__ dq, float* __restrict__ delta_out, SwaDims dm, int n_qt, int n_b) {
+  constexpr int RT = swa_dq_rt(D, DV);
   constexpr int KS = D / 32, VS = DV / 32, DT = D / 16;
-  constexpr int QW = 16 * SWA_RT / G, QB = 4 * QW;
+  constexpr int QW = 16 * RT / G > 0 ? 16 * RT / G : 1, QB = 4 * 16 * RT / G;
   constexpr int PITCH = D * 2 + 16, VPITCH = DV * 2 + 16;
   constexpr int KSEG = D / 8, KPPP = 256 / KSEG, KPASS = 32 / KPPP;
   constexpr int VSEG = DV / 8, VPASS = 64 * VSEG / 256;
@@ -396,17 +438,18 @@ swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, cons
   __shared__ __align__(16) unsigned char v_s[64 * VPITCH];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, j = lane >> 4;
-  const int qt = n_qt - 1 - (int)blockIdx.x;
-  const int hk = blockIdx.y;
-  const long b = blockIdx.z;
+  int qt, hk;
+  long b;
+  if (!swa_xcd_unit(n_qt, dm.H, n_b, qt, hk, b)) return;
+  qt = n_qt - 1 - qt;
   const int t0 = qt * QB + wave * QW;
   const int L = dm.Lq;
 
-  bf16x8_t qa[SWA_RT][KS], doa[SWA_RT][VS];
-  int qabs[SWA_RT], cstart[SWA_RT];
-  float lse2[SWA_RT], delta[SWA_RT];
+  bf16x8_t qa[RT][KS], doa[RT][VS];
+  int qabs[RT], cstart[RT];
+  float lse2[RT], delta[RT];
 #pragma unroll
-  for (int rt = 0; rt < SWA_RT; ++rt) {
+  for (int rt = 0; rt < RT; ++rt) {
     const int row = rt * 16 + col;
     const int t = t0 + row / G, g = row % G;
     const int tc = t < L ? t : L - 1;
@@ -481,9 +524,9 @@ swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, cons
       *(swa_u32x4*)(v_s + (p / VSEG) * VPITCH + (p % VSEG) * 16) = vr[i];
     }
   };
-  f32x4_t acc[SWA_RT][DT];
+  f32x4_t acc[RT][DT];
 #pragma unroll
-  for (int rt = 0; rt < SWA_RT; ++rt)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   fetch(tile_lo);
@@ -491,11 +534,11 @@ swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, cons
   __syncthreads();
   for (int tile = tile_lo; tile < tile_hi; ++tile) {
     fetch(tile + 1 < tile_hi ? tile + 1 : tile);
-    float ds[SWA_RT][4][4];
+    float ds[RT][4][4];
     {
-      f32x4_t st[SWA_RT][4], dp[SWA_RT][4];
+      f32x4_t st[RT][4], dp[RT][4];
 #pragma unroll
-      for (int rt = 0; rt < SWA_RT; ++rt)
+      for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
           st[rt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -507,21 +550,21 @@ swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, cons
         for (int ks = 0; ks < KS; ++ks) {
           const bf16x8_t a = *(const bf16x8_t*)(k_s + (tt * 16 + col) * PITCH + ks * 64 + j * 16);
 #pragma unroll
-          for (int rt = 0; rt < SWA_RT; ++rt)
+          for (int rt = 0; rt < RT; ++rt)
             st[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qa[rt][ks], st[rt][tt], 0, 0, 0);
         }
 #pragma unroll
         for (int vs = 0; vs < VS; ++vs) {
           const bf16x8_t a = *(const bf16x8_t*)(v_s + (tt * 16 + col) * VPITCH + vs * 64 + j * 16);
 #pragma unroll
-          for (int rt = 0; rt < SWA_RT; ++rt)
+          for (int rt = 0; rt < RT; ++rt)
             dp[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, doa[rt][vs], dp[rt][tt], 0, 0, 0);
         }
       }
       const int tok0 = tile * 64 + 4 * j;
       const unsigned lmk_ok = swa_lmk_bits(dm, tok0);
 #pragma unroll
-      for (int rt = 0; rt < SWA_RT; ++rt)
+      for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
@@ -532,13 +575,13 @@ swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, cons
             ds[rt][tt][i] = pv * (dp[rt][tt][i] - delta[rt]) * dm.sm_scale;
           }
     }
-    lzm_grad_product<D, SWA_RT>(kt_s, ds, acc, col, j);
+    lzm_grad_product<D, RT>(kt_s, ds, acc, col, j);
     __syncthreads();
     stash();
     __syncthreads();
   }
 #pragma unroll
-  for (int rt = 0; rt < SWA_RT; ++rt)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = rt * 16 + 4 * j + i;
@@ -550,17 +593,18 @@ swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, cons
     }
 }
 
-// dK, dV: a workgroup owns 128 tokens of one KV head (32 per wavefront, as matrix B operands); the
+// dK, dV: a workgroup owns 64 * TT tokens of one KV head (TT 16-token tiles per wavefront, as matrix B
+// operands: two for narrow heads, one for wide heads, whose two tiles need more than 256 registers); the
 // score rows (query x head) that can see them stream in tiles of 64 rows, Q and dO both row-major
 // and transposed, with the rows' lse, delta and window start beside them.
 template <int D, int DV, int G>
-// (narrow heads fit 256 registers: the hint then gives two wavefronts per SIMD and keeps the
-// accumulators out of accumulation registers; wide heads need more and run one wavefront per SIMD)
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((D <= 64 && DV <= 64) ? 2 : 1)))
+// (the hint gives two wavefronts per SIMD and keeps the accumulators out of accumulation registers)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                   const bf16_t* __restrict__ v, const float* __restrict__ lse,
                   const bf16_t* __restrict__ d_o, const float* __restrict__ delta_in,
-                  bf16_t* __restrict__ dk, bf16_t* __restrict__ dv, SwaDims dm) {
+                  bf16_t* __restrict__ dk, bf16_t* __restrict__ dv, SwaDims dm, int n_kb, int n_b) {
+  constexpr int TT = swa_dq_rt(D, DV);
   constexpr int KS = D / 32, VS = DV / 32, DT = D / 16, DVT = DV / 16;
   constexpr int QT = 64 / G;
   constexpr int PITCH = D * 2 + 16, VPITCH = DV * 2 + 16;
@@ -576,16 +620,17 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
   int* cs_s = (int*)(del_s + 64);                 // 64: window start of the row (INT_MAX: dead row)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, j = lane >> 4;
-  const int hk = blockIdx.y;
-  const long b = blockIdx.z;
+  int kb, hk;
+  long b;
+  if (!swa_xcd_unit(n_kb, dm.H, n_b, kb, hk, b)) return;
   const int L = dm.Lq;
-  const int j0 = (int)blockIdx.x * 128;
-  const int tok_w = j0 + wave * 32;  // first owned token of the wavefront
+  const int j0 = kb * (64 * TT);
+  const int tok_w = j0 + wave * (16 * TT);  // first owned token of the wavefront
 
-  bf16x8_t ka[2][KS], va[2][VS];
+  bf16x8_t ka[TT][KS], va[TT][VS];
   unsigned lmk_ok = 0u;  // bit tt: owned token tt*16 + col is not a landmark
 #pragma unroll
-  for (int tt = 0; tt < 2; ++tt) {
+  for (int tt = 0; tt < TT; ++tt) {
     const int tok = tok_w + tt * 16 + col;
     const int tc = tok < L ? tok : L - 1;  // tokens past the end are never visible
     const bf16_t* kp = k + ((b * L + tc) * (long)dm.H + hk) * D + j * 8;
@@ -598,7 +643,7 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     if (!lm && tok < L) lmk_ok |= 1u << tt;
   }
   // queries that can see a token of [j0, j1]: j0 <= t <= (last window that starts at or before j1)
-  int j1 = j0 + 127;
+  int j1 = j0 + 64 * TT - 1;
   if (j1 > L - 1) j1 = L - 1;
   long t_hi = dm.expand ? ((long)(j1 / dm.chunk) + 1) * dm.chunk + dm.window - 2 : (long)j1 + dm.window - 1;
   if (t_hi > L - 1) t_hi = L - 1;
@@ -652,9 +697,9 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
       cs_s[tid] = live ? r_cs : 2147483647;
     }
   };
-  f32x4_t acck[2][DT], accv[2][DVT];
+  f32x4_t acck[TT][DT], accv[TT][DVT];
 #pragma unroll
-  for (int tt = 0; tt < 2; ++tt) {
+  for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acck[tt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -665,11 +710,11 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
   __syncthreads();
   for (int tile = tile0; tile < n_tiles; ++tile) {
     fetch(tile + 1 < n_tiles ? tile + 1 : tile);
-    float p[2][4][4], ds[2][4][4];  // [owned token tile][streamed row tile][row 4j+i]
+    float p[TT][4][4], ds[TT][4][4];  // [owned token tile][streamed row tile][row 4j+i]
     {
-      f32x4_t st[2][4], dp[2][4];
+      f32x4_t st[TT][4], dp[TT][4];
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt)
+      for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
           st[tt][rr] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -681,14 +726,14 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
         for (int ks = 0; ks < KS; ++ks) {
           const bf16x8_t a = *(const bf16x8_t*)(q_s + (rr * 16 + col) * PITCH + ks * 64 + j * 16);
 #pragma unroll
-          for (int tt = 0; tt < 2; ++tt)
+          for (int tt = 0; tt < TT; ++tt)
             st[tt][rr] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ka[tt][ks], st[tt][rr], 0, 0, 0);
         }
 #pragma unroll
         for (int vs = 0; vs < VS; ++vs) {
           const bf16x8_t a = *(const bf16x8_t*)(do_s + (rr * 16 + col) * VPITCH + vs * 64 + j * 16);
 #pragma unroll
-          for (int tt = 0; tt < 2; ++tt)
+          for (int tt = 0; tt < TT; ++tt)
             dp[tt][rr] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, va[tt][vs], dp[tt][rr], 0, 0, 0);
         }
       }
@@ -704,7 +749,7 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
         for (int i = 0; i < 4; ++i) {
           const int t = tq0 + (rr * 16 + 4 * j + i) / G;
 #pragma unroll
-          for (int tt = 0; tt < 2; ++tt) {
+          for (int tt = 0; tt < TT; ++tt) {
             const int tok = tok_w + tt * 16 + col;
             const bool vis = (tok >= cs[i]) & (tok <= t) & (((lmk_ok >> tt) & 1u) != 0u);  // no short circuit: no branches
             const float pv = vis ? __builtin_amdgcn_exp2f(st[tt][rr][i] * c2 - ls[i]) : 0.f;
@@ -714,14 +759,14 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
         }
       }
     }
-    lzm_grad_product<DV, 2>(dot_s, p, accv, col, j);
-    lzm_grad_product<D, 2>(qt_s, ds, acck, col, j);
+    lzm_grad_product<DV, TT>(dot_s, p, accv, col, j);
+    lzm_grad_product<D, TT>(qt_s, ds, acck, col, j);
     __syncthreads();
     stash();
     __syncthreads();
   }
 #pragma unroll
-  for (int tt = 0; tt < 2; ++tt)
+  for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int tok = tok_w + tt * 16 + 4 * j + i;
@@ -735,26 +780,58 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     }
 }
 
-template <int D, int DV, int G>
-static int swa_fwd_launch(dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* k, const bf16_t* v,
-                          bf16_t* o, float* lse, const SwaDims& dm, int n_qt) {
-  const size_t smem = swa_fwd_smem<D, DV>();
-  auto kern = swa_fwd_blk<D, DV, G>;
+template <int D, int DV, int G, int NWV, int RES>
+static int swa_fwd_launch_shape(int B, hipStream_t st, const bf16_t* q, const bf16_t* k, const bf16_t* v,
+                                bf16_t* o, float* lse, const SwaDims& dm) {
+  const size_t smem = swa_fwd_smem<D, DV, NWV, RES>();
+  auto kern = swa_fwd_blk<D, DV, G, NWV, RES>;
   static HilsLdsReserve reserved;  // per instantiation
   if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_swa_fwd")) return rc;
-  hipLaunchKernelGGL(kern, grid, dim3(SWA_FWD_WAVES * 64), smem, st, q, k, v, o, lse, dm, n_qt);
+  const int QB = NWV * 16 * SWA_FWD_RT / G;  // queries of a workgroup (>= 8: G <= 16)
+  const int n_qt = (dm.Lq + QB - 1) / QB;
+  hipLaunchKernelGGL(kern, swa_xcd_grid(n_qt, dm.H, B), dim3(NWV * 64), smem, st, q, k, v, o, lse, dm, n_qt, B);
   return HILS_OK;
 }
 
+// The most 64-token tiles a block of QB queries reads (over the last blocks: the first ones are
+// clipped at key 0, and the pattern repeats with the alignment of blocks, chunks and tiles).
+static int swa_fwd_block_tiles(const SwaDims& dm, int QB) {
+  const int n_qt = (dm.Lq + QB - 1) / QB;
+  const long q_off = (long)dm.kv_start + dm.Lk - dm.Lq;
+  int most = 0;
+  for (int qt = n_qt - 1; qt >= 0 && qt >= n_qt - 256; --qt) {
+    const long tq0 = (long)qt * QB;
+    long tq1 = tq0 + QB - 1;
+    if (tq1 > dm.Lq - 1) tq1 = dm.Lq - 1;
+    const long left = q_off + tq0 - dm.window + 1;
+    long lo = dm.expand ? (left >= 0 ? left / dm.chunk : -((-left + dm.chunk - 1) / dm.chunk)) * dm.chunk : left;
+    lo -= dm.kv_start;
+    long hi = q_off + tq1 - dm.kv_start + 1;
+    if (lo < 0) lo = 0;
+    if (hi > dm.Lk) hi = dm.Lk;
+    const int n = (int)((hi + 63) / 64 - lo / 64);
+    if (n > most) most = n;
+  }
+  return most;
+}
+
+template <int D, int DV, int G>
+static int swa_fwd_launch(int B, hipStream_t st, const bf16_t* q, const bf16_t* k, const bf16_t* v,
+                          bf16_t* o, float* lse, const SwaDims& dm) {
+  if (swa_fwd_block_tiles(dm, 4 * 16 * SWA_FWD_RT / G) <= 2)
+    return swa_fwd_launch_shape<D, DV, G, 4, 2>(B, st, q, k, v, o, lse, dm);
+  return swa_fwd_launch_shape<D, DV, G, 8, 4>(B, st, q, k, v, o, lse, dm);
+}
+
 template <int D, int DV>
-static int swa_launch_g(int G, dim3 grid, hipStream_t st, const bf16_t* q, const bf16_t* k,
-                        const bf16_t* v, bf16_t* o, float* lse, const SwaDims& dm, int n_qt) {
+static int swa_launch_g(int G, int B, hipStream_t st, const bf16_t* q, const bf16_t* k,
+                        const bf16_t* v, bf16_t* o, float* lse, const SwaDims& dm) {
   switch (G) {
-    case 1: return swa_fwd_launch<D, DV, 1>(grid, st, q, k, v, o, lse, dm, n_qt);
-    case 2: return swa_fwd_launch<D, DV, 2>(grid, st, q, k, v, o, lse, dm, n_qt);
-    case 4: return swa_fwd_launch<D, DV, 4>(grid, st, q, k, v, o, lse, dm, n_qt);
-    case 8: return swa_fwd_launch<D, DV, 8>(grid, st, q, k, v, o, lse, dm, n_qt);
-    default: return swa_fwd_launch<D, DV, 16>(grid, st, q, k, v, o, lse, dm, n_qt);
+    case 1: return swa_fwd_launch<D, DV, 1>(B, st, q, k, v, o, lse, dm);
+    case 2: return swa_fwd_launch<D, DV, 2>(B, st, q, k, v, o, lse, dm);
+    case 4: return swa_fwd_launch<D, DV, 4>(B, st, q, k, v, o, lse, dm);
+    case 8: return swa_fwd_launch<D, DV, 8>(B, st, q, k, v, o, lse, dm);
+    default: return swa_fwd_launch<D, DV, 16>(B, st, q, k, v, o, lse, dm);
   }
 }
 
@@ -773,20 +850,17 @@ extern "C" int hils_swa_fwd(const void* q, const void* k, const void* v, void* o
                "hils_swa_fwd: head dims (%d, %d) must be 64 or 128", D, Dv);
   HILS_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8 || G == 16,
                "hils_swa_fwd: group size %d must be 1, 2, 4, 8 or 16", G);
-  HILS_REQUIRE(H <= 65535 && B <= 65535, "hils_swa_fwd: H/B too large for the grid");
+  HILS_REQUIRE(((long)Lq / 8 + 1) * H * B < (1L << 31) - 8, "hils_swa_fwd: B * H * Lq too large for the grid");
   HILS_REQUIRE((long)kv_start + Lk < 2147483647L / 2, "hils_swa_fwd: positions overflow 32 bits");
   SwaDims dm{Lq, Lk, HQ, H, window, chunk, mask_lmk, expand_to_chunk, kv_start,
              (chunk & (chunk - 1)) == 0, sm_scale};
-  const int QB = SWA_FWD_WAVES * 16 * SWA_FWD_RT / G;  // queries of a workgroup (>= 16: G <= 16)
-  const int n_qt = (Lq + QB - 1) / QB;
-  const dim3 grid((unsigned)n_qt, (unsigned)H, (unsigned)B);
   hipStream_t st = (hipStream_t)stream;
   const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k, *vv = (const bf16_t*)v;
   int rc;
-  if (D == 64 && Dv == 64) rc = swa_launch_g<64, 64>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
-  else if (D == 128 && Dv == 128) rc = swa_launch_g<128, 128>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
-  else if (D == 64) rc = swa_launch_g<64, 128>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
-  else rc = swa_launch_g<128, 64>(G, grid, st, qq, kk, vv, (bf16_t*)o, lse, dm, n_qt);
+  if (D == 64 && Dv == 64) rc = swa_launch_g<64, 64>(G, B, st, qq, kk, vv, (bf16_t*)o, lse, dm);
+  else if (D == 128 && Dv == 128) rc = swa_launch_g<128, 128>(G, B, st, qq, kk, vv, (bf16_t*)o, lse, dm);
+  else if (D == 64) rc = swa_launch_g<64, 128>(G, B, st, qq, kk, vv, (bf16_t*)o, lse, dm);
+  else rc = swa_launch_g<128, 64>(G, B, st, qq, kk, vv, (bf16_t*)o, lse, dm);
   if (rc) return rc;
   HILS_CHECK_LAUNCH("hils_swa_fwd");
   return HILS_OK;
@@ -796,17 +870,18 @@ template <int D, int DV, int G>
 static int swa_bwd_launch(const bf16_t* q, const bf16_t* k, const bf16_t* v, const bf16_t* o,
                           const float* lse, const bf16_t* d_o, const float* d_lse, bf16_t* dq, bf16_t* dk,
                           bf16_t* dv, float* delta, int B, const SwaDims& dm, hipStream_t st) {
-  const int QB = 4 * 16 * SWA_RT / G;
+  const int QB = 4 * 16 * swa_dq_rt(D, DV) / G;
   const int n_qt = (dm.Lq + QB - 1) / QB;
-  hipLaunchKernelGGL((swa_bwd_dq_mfma<D, DV, G>), dim3((unsigned)n_qt, (unsigned)dm.H, (unsigned)B),
-                     dim3(256), 0, st, q, k, v, o, lse, d_o, d_lse, dq, delta, dm, n_qt);
+  hipLaunchKernelGGL((swa_bwd_dq_mfma<D, DV, G>), swa_xcd_grid(n_qt, dm.H, B),
+                     dim3(256), 0, st, q, k, v, o, lse, d_o, d_lse, dq, delta, dm, n_qt, B);
   const size_t smem = (size_t)64 * (D * 2 + 16) + (size_t)D * LZM_PT + (size_t)64 * (DV * 2 + 16) +
                       (size_t)DV * LZM_PT + 3 * 64 * sizeof(float);
   auto kern = swa_bwd_dkdv_mfma<D, DV, G>;
   static HilsLdsReserve reserved;  // per instantiation
   if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_swa_bwd")) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)((dm.Lq + 127) / 128), (unsigned)dm.H, (unsigned)B), dim3(256),
-                     smem, st, q, k, v, lse, d_o, delta, dk, dv, dm);
+  const int n_kb = (dm.Lq + 64 * swa_dq_rt(D, DV) - 1) / (64 * swa_dq_rt(D, DV));
+  hipLaunchKernelGGL(kern, swa_xcd_grid(n_kb, dm.H, B), dim3(256), smem, st, q, k, v, lse, d_o, delta, dk, dv, dm,
+                     n_kb, B);
   return HILS_OK;
 }
 
@@ -836,7 +911,7 @@ extern "C" int hils_swa_bwd(const void* q, const void* k, const void* v, const v
                "hils_swa_bwd: head dims (%d, %d) must be 64 or 128", D, Dv);
   HILS_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8 || G == 16,
                "hils_swa_bwd: group size %d must be 1, 2, 4, 8 or 16", G);
-  HILS_REQUIRE(H <= 65535 && B <= 65535, "hils_swa_bwd: H/B too large for the grid");
+  HILS_REQUIRE(((long)L / 8 + 1) * H * B < (1L << 31) - 8, "hils_swa_bwd: B * H * L too large for the grid");
   HILS_REQUIRE((long)L + window < 2147483647L / 2, "hils_swa_bwd: positions overflow 32 bits");
   SwaDims dm{L, L, HQ, H, window, chunk, mask_lmk, expand_to_chunk, 0, (chunk & (chunk - 1)) == 0, sm_scale};
   hipStream_t st = (hipStream_t)stream;
