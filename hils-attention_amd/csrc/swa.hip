@@ -818,8 +818,12 @@ static int swa_fwd_block_tiles(const SwaDims& dm, int QB) {
 template <int D, int DV, int G>
 static int swa_fwd_launch(int B, hipStream_t st, const bf16_t* q, const bf16_t* k, const bf16_t* v,
                           bf16_t* o, float* lse, const SwaDims& dm) {
-  if (swa_fwd_block_tiles(dm, 4 * 16 * SWA_FWD_RT / G) <= 2)
-    return swa_fwd_launch_shape<D, DV, G, 4, 2>(B, st, q, k, v, o, lse, dm);
+  const int tiles = swa_fwd_block_tiles(dm, 4 * 16 * SWA_FWD_RT / G);
+  if (tiles <= 2) return swa_fwd_launch_shape<D, DV, G, 4, 2>(B, st, q, k, v, o, lse, dm);
+  // narrow heads: four resident tiles are 72 KiB, and two 4-wavefront workgroups fit a compute unit
+  // where one 8-wavefront workgroup does (150 registers: three wavefronts per SIMD)
+  if constexpr (D <= 64 && DV <= 64)
+    if (tiles <= 4) return swa_fwd_launch_shape<D, DV, G, 4, 4>(B, st, q, k, v, o, lse, dm);
   return swa_fwd_launch_shape<D, DV, G, 8, 4>(B, st, q, k, v, o, lse, dm);
 }
 
