@@ -42,6 +42,11 @@ def test_swa_mask_variants(pkg, orc, dev):
     # chunk size that is not a power of two; explicit scale; different value head dim
     run(pkg, orc, dev, 1, 333, 333, 4, 1, 128, 64, 100, 48, sm_scale=0.05)
     run(pkg, orc, dev, 1, 200, 200, 2, 2, 64, 128, 30, 20, expand=False)
+    # sharp softmax over several key tiles: a row's running maximum both jumps far (the accumulated
+    # output is rescaled) and creeps (it is not), for 8- and 4-wavefront workgroups
+    run(pkg, orc, dev, 1, 500, 500, 4, 2, 64, 64, 200, 64, sm_scale=0.7)
+    run(pkg, orc, dev, 1, 500, 500, 8, 2, 128, 128, 64, 64, sm_scale=0.5)
+    run(pkg, orc, dev, 1, 500, 500, 4, 4, 64, 64, 100, 64, sm_scale=0.6, expand=False)
 
 
 def test_swa_inference_cache_and_truncated_cache(pkg, orc, dev):
