@@ -186,19 +186,6 @@ swa_fwd_blk(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf
         }
       const bool inner = !dm.mask_lmk && tile * 64 >= w_in_lo && tile * 64 + 64 <= w_in_hi;  // uniform
       if (!inner) {
-        // visibility of this lane's 16 tokens: bit tt*4+i; the landmark test does not depend on the row
-        unsigned lmk_ok = 0xffffu;
-        if (dm.mask_lmk) {
-          lmk_ok = 0u;
-#pragma unroll
-          for (int tt = 0; tt < 4; ++tt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int ta = dm.kv_start + tile * 64 + tt * 16 + 4 * j + i + 1;
-              const bool lm = dm.chunk_pow2 ? ((ta & (dm.chunk - 1)) == 0) : (ta % dm.chunk == 0);
-              lmk_ok |= lm ? 0u : (1u << (tt * 4 + i));
-            }
-        }
         // a token at absolute position ta is visible to a row iff vlo <= ta <= vhi (window start, the
         // query itself or the last key): one unsigned compare of ta - vlo against vhi - vlo, no branches
         const int tok_abs0 = dm.kv_start + tile * 64 + 4 * j;
@@ -208,10 +195,20 @@ swa_fwd_blk(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf
 #pragma unroll
           for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
+            for (int i = 0; i < 4; ++i)
+              p[rt][tt][i] = (base + (unsigned)(tt * 16 + i) <= vspan[rt]) ? p[rt][tt][i] : HILS_NEG_INF;
+        }
+        // landmarks (the last position of every chunk) in a pass of their own behind a uniform branch:
+        // the test does not depend on the row, and the common call masks none
+        if (dm.mask_lmk) {
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
             for (int i = 0; i < 4; ++i) {
-              bool vis = base + (unsigned)(tt * 16 + i) <= vspan[rt];
-              if (dm.mask_lmk) vis = vis & (((lmk_ok >> (tt * 4 + i)) & 1u) != 0u);
-              p[rt][tt][i] = vis ? p[rt][tt][i] : HILS_NEG_INF;
+              const int ta = tok_abs0 + tt * 16 + i + 1;
+              const bool lm = dm.chunk_pow2 ? ((ta & (dm.chunk - 1)) == 0) : (ta % dm.chunk == 0);
+#pragma unroll
+              for (int rt = 0; rt < RT; ++rt) p[rt][tt][i] = lm ? HILS_NEG_INF : p[rt][tt][i];
             }
         }
       }
@@ -479,6 +476,14 @@ swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, cons
     delta[rt] = part - (d_lse ? d_lse[rix] : 0.f);
     if (j == 0 && t < L) delta_out[rix] = delta[rt];
   }
+  int vlo[RT];
+  unsigned vspan[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const bool some = qabs[rt] >= cstart[rt];
+    vlo[rt] = some ? cstart[rt] : 0x7fffffff;
+    vspan[rt] = some ? (unsigned)(qabs[rt] - cstart[rt]) : 0u;
+  }
   int tile_lo, tile_hi;
   {
     const int tq0 = qt * QB;
@@ -561,19 +566,32 @@ swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, cons
             dp[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, doa[rt][vs], dp[rt][tt], 0, 0, 0);
         }
       }
+      // token ta is visible to a row iff window start <= ta <= query: one unsigned compare of
+      // ta - start against query - start (a dead row has a start no token reaches)
       const int tok0 = tile * 64 + 4 * j;
-      const unsigned lmk_ok = swa_lmk_bits(dm, tok0);
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
+      for (int rt = 0; rt < RT; ++rt) {
+        const unsigned base = (unsigned)(tok0 - vlo[rt]);
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int ta = tok0 + tt * 16 + i;
-            const bool vis = (ta >= cstart[rt]) & (ta <= qabs[rt]) & (((lmk_ok >> (tt * 4 + i)) & 1u) != 0u);  // no short circuit: no branches
+            const bool vis = base + (unsigned)(tt * 16 + i) <= vspan[rt];
             const float pv = vis ? __builtin_amdgcn_exp2f(st[rt][tt][i] * c2 - lse2[rt]) : 0.f;
             ds[rt][tt][i] = pv * (dp[rt][tt][i] - delta[rt]) * dm.sm_scale;
           }
+      }
+      if (dm.mask_lmk) {  // landmarks in a pass of their own behind a uniform branch (row-independent)
+        const unsigned lmk_ok = swa_lmk_bits(dm, tok0);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const bool ok = ((lmk_ok >> (tt * 4 + i)) & 1u) != 0u;
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) ds[rt][tt][i] = ok ? ds[rt][tt][i] : 0.f;
+          }
+      }
     }
     lzm_grad_product<D, RT>(kt_s, ds, acc, col, j);
     __syncthreads();
@@ -642,6 +660,11 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     const bool lm = dm.mask_lmk && (dm.chunk_pow2 ? (((tok + 1) & (dm.chunk - 1)) == 0) : ((tok + 1) % dm.chunk == 0));
     if (!lm && tok < L) lmk_ok |= 1u << tt;
   }
+  // owned token of this lane per tile, or a position far below every window for a landmark / a
+  // token past the end
+  int tokv[TT];
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt) tokv[tt] = ((lmk_ok >> tt) & 1u) ? tok_w + tt * 16 + col : -(1 << 30);
   // queries that can see a token of [j0, j1]: j0 <= t <= (last window that starts at or before j1)
   int j1 = j0 + 64 * TT - 1;
   if (j1 > L - 1) j1 = L - 1;
@@ -747,11 +770,13 @@ swa_bwd_dkdv_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
         const int cs[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+          // window start <= token <= query as one unsigned compare of query - token against
+          // query - start + 1 (0 for a dead row, whose start no query reaches)
           const int t = tq0 + (rr * 16 + 4 * j + i) / G;
+          const unsigned span1 = t >= cs[i] ? (unsigned)(t - cs[i]) + 1u : 0u;
 #pragma unroll
           for (int tt = 0; tt < TT; ++tt) {
-            const int tok = tok_w + tt * 16 + col;
-            const bool vis = (tok >= cs[i]) & (tok <= t) & (((lmk_ok >> tt) & 1u) != 0u);  // no short circuit: no branches
+            const bool vis = (unsigned)(t - tokv[tt]) < span1;
             const float pv = vis ? __builtin_amdgcn_exp2f(st[tt][rr][i] * c2 - ls[i]) : 0.f;
             p[tt][rr][i] = pv;
             ds[tt][rr][i] = pv * (dp[tt][rr][i] - dl[i]) * dm.sm_scale;
