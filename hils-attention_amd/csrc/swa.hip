@@ -11,8 +11,6 @@
 #include "stream_tiles.h"
 #include "../../include/hils_amd.h"
 
-#define SWA_RT 2  // 16-row tiles per wavefront
-
 struct SwaDims {
   int Lq, Lk, HQ, H, window, chunk, mask_lmk, expand, kv_start, chunk_pow2;
   float sm_scale;
@@ -410,15 +408,11 @@ __device__ __forceinline__ unsigned swa_lmk_bits(const SwaDims& dm, int tok0) {
 
 // 16-row tiles per wavefront of the backward kernels: two for narrow heads; one for wide heads, whose two
 // tiles need more than 256 registers (one wavefront per SIMD, nothing to overlap a wait with)
-#ifndef SWA_RT_NARROW
-#define SWA_RT_NARROW 2
-#endif
-constexpr int swa_dq_rt(int D, int DV) { return (D <= 64 && DV <= 64) ? SWA_RT_NARROW : 1; }
+constexpr int swa_dq_rt(int D, int DV) { return (D <= 64 && DV <= 64) ? 2 : 1; }
 
-// dQ (and delta): a wavefront owns 32 score rows; K (row-major and transposed) and V stream.
+// dQ (and delta): a wavefront owns 16 * RT score rows; K (row-major and transposed) and V stream.
 template <int D, int DV, int G>
-// (narrow heads fit 256 registers: the hint then gives two wavefronts per SIMD and keeps the
-// accumulators out of accumulation registers; wide heads need more and run one wavefront per SIMD)
+// (the hint gives two wavefronts per SIMD and keeps the accumulators out of accumulation registers)
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
                 const bf16_t* __restrict__ o, const float* __restrict__ lse,
