@@ -71,13 +71,26 @@ logz_fwd_simple(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
 // K Q^T so that the 64 tokens of one row lie in 16 registers of 4 lanes: the log-sum-exp is an
 // in-lane reduction plus one row-swap reduction.
 #define LZM_RT 2  // 16-row tiles per wavefront
+
+// Workgroup order of the matrix-core kernels: one-dimensional grids in which all blocks of a
+// (batch, KV head) unit run on one XCD (the hardware hands consecutive workgroup ids to the 8 XCDs in
+// turn: id -> (xcd, slot); unit = 8 * (slot / n_blk) + xcd), so that the keys (or query rows) the
+// unit's workgroups stream are fetched into one L2 once instead of into all eight.  False for the
+// padding ids of a unit count that is not a multiple of 8.
+__device__ __forceinline__ bool lz_xcd_unit(int n_blk, int n_unit, int& unit, int& blk) {
+  const int xcd = (int)(blockIdx.x % 8), slot = (int)(blockIdx.x / 8);
+  unit = (slot / n_blk) * 8 + xcd;
+  blk = slot % n_blk;
+  return unit < n_unit;
+}
+static dim3 lz_xcd_grid(int n_blk, int n_unit) { return dim3((unsigned)(8 * ((n_unit + 7) / 8) * n_blk)); }
 // (the occupancy hint also keeps the score accumulators in ordinary registers: without it the
 // compiler, free to use 512 registers at this workgroup size, parks them in accumulation registers
 // and copies every score back for the softmax)
 template <int D, int G>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3)))
 logz_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
-              float* __restrict__ log_z, LzDims dm, int n_qt) {
+              float* __restrict__ log_z, LzDims dm, int n_qt, int n_unit) {
   constexpr int KS = D / 32;
   constexpr int QW = 16 * LZM_RT / G;  // queries per wavefront
   constexpr int QB = 4 * QW;           // queries per workgroup
@@ -86,9 +99,11 @@ logz_fwd_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
   __shared__ __align__(16) unsigned char k_s[2][64 * PITCH];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, j = lane >> 4;
-  const int qt = n_qt - 1 - (int)blockIdx.x;  // longest rows first
-  const int hk = blockIdx.y;
-  const long b = blockIdx.z;
+  int unit, qt;
+  if (!lz_xcd_unit(n_qt, n_unit, unit, qt)) return;
+  qt = n_qt - 1 - qt;  // longest rows first
+  const int hk = unit % dm.H;
+  const long b = unit / dm.H;
   const int t0 = qt * QB + wave * QW;
 
   bf16x8_t qa[LZM_RT][KS];
@@ -211,7 +226,7 @@ template <int D, int G>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 logz_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                  const float* __restrict__ log_z, const float* __restrict__ d_log_z,
-                 bf16_t* __restrict__ dq, LzDims dm, int n_qt) {
+                 bf16_t* __restrict__ dq, LzDims dm, int n_qt, int n_unit) {
   constexpr int KS = D / 32, DT = D / 16;
   constexpr int QW = 16 * LZM_RT / G, QB = 4 * QW;
   constexpr int PITCH = D * 2 + 16;
@@ -222,9 +237,11 @@ logz_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
   __shared__ __align__(16) unsigned char kt_s[D * LZM_PT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, j = lane >> 4;
-  const int qt = n_qt - 1 - (int)blockIdx.x;
-  const int hk = blockIdx.y;
-  const long b = blockIdx.z;
+  int unit, qt;
+  if (!lz_xcd_unit(n_qt, n_unit, unit, qt)) return;
+  qt = n_qt - 1 - qt;
+  const int hk = unit % dm.H;
+  const long b = unit / dm.H;
   const int t0 = qt * QB + wave * QW;
 
   bf16x8_t qa[LZM_RT][KS];
@@ -340,7 +357,7 @@ template <int D, int G>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 logz_bwd_dk_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                  const float* __restrict__ log_z, const float* __restrict__ d_log_z,
-                 bf16_t* __restrict__ dk, LzDims dm) {
+                 bf16_t* __restrict__ dk, LzDims dm, int n_pair, int n_unit) {
   constexpr int KS = D / 32, DT = D / 16;
   constexpr int QT = 64 / G;  // queries per streamed tile
   constexpr int PITCH = D * 2 + 16;
@@ -351,9 +368,18 @@ logz_bwd_dk_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
   __shared__ __align__(16) float coef_s[2][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, j = lane >> 4;
-  const int c0 = 2 * (int)blockIdx.x, ch = wave >> 1;
-  const int hk = blockIdx.y;
-  const long b = blockIdx.z;
+  // Workgroup order.  The workgroups of one (batch, KV head) stream the same query rows, each from the
+  // first query behind its chunks to the last one: they walk the tiles from the END, so that all of
+  // them are on the same tile at the same time, and the one-dimensional grid puts them on one XCD
+  // (the hardware hands consecutive workgroup ids to the 8 XCDs in turn: id -> (xcd, slot)), whose L2
+  // then serves all but the first reader of a tile.  Walking forward from different starting points
+  // in the hardware's order, every read of a tile missed (L2 hit rate 2 %, the kernel waiting on
+  // HBM latency at one wavefront per SIMD).  The chunk pairs of a unit come longest walk first.
+  int unit, pair;
+  if (!lz_xcd_unit(n_pair, n_unit, unit, pair)) return;
+  const int c0 = 2 * pair, ch = wave >> 1;
+  const int hk = unit % dm.H;
+  const long b = unit / dm.H;
   const int tok0 = (c0 + ch) * 64 + (wave & 1) * 32;  // first owned token
 
   bf16x8_t ka[2][KS];
@@ -415,12 +441,12 @@ logz_bwd_dk_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[tt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   if (tile0 < n_tiles) {
-    fetch(tile0);
+    fetch(n_tiles - 1);
     stash();
   }
   __syncthreads();
-  for (int tile = tile0; tile < n_tiles; ++tile) {
-    fetch(tile + 1 < n_tiles ? tile + 1 : tile);
+  for (int tile = n_tiles - 1; tile >= tile0; --tile) {
+    fetch(tile > tile0 ? tile - 1 : tile);
     float p[2][4][4];  // [owned token tile][streamed row tile][row 4j+i]
     {
       f32x4_t st[2][4];
@@ -626,10 +652,11 @@ extern "C" int hils_chunk_logz_fwd(const void* q, const void* k, float* log_z, i
   if (lz_mfma_covers(G, D, S, H, B)) {
     const int QB = 4 * 16 * LZM_RT / G;
     const int n_qt = (L + QB - 1) / QB;
-    const dim3 grid((unsigned)n_qt, (unsigned)H, (unsigned)B);
+    HILS_REQUIRE(((long)B * H + 7) / 8 * 8 * n_qt < (1L << 31), "hils_chunk_logz_fwd: B * H * L too large for the grid");
+    const dim3 grid = lz_xcd_grid(n_qt, B * H);
 #define LZ_LAUNCH(DD, GG)                                                                      \
   hipLaunchKernelGGL((logz_fwd_mfma<DD, GG>), grid, dim3(256), 0, (hipStream_t)stream,         \
-                     (const bf16_t*)q, (const bf16_t*)k, log_z, dm, n_qt)
+                     (const bf16_t*)q, (const bf16_t*)k, log_z, dm, n_qt, B * H)
     LZ_DISPATCH(D, G);
 #undef LZ_LAUNCH
     HILS_CHECK_LAUNCH("hils_chunk_logz_fwd");
@@ -653,10 +680,11 @@ extern "C" int hils_chunk_logz_bwd_dq(const void* q, const void* k, const float*
     const int G = HQ / H;
     const int QB = 4 * 16 * LZM_RT / G;
     const int n_qt = (L + QB - 1) / QB;
-    const dim3 grid((unsigned)n_qt, (unsigned)H, (unsigned)B);
+    HILS_REQUIRE(((long)B * H + 7) / 8 * 8 * n_qt < (1L << 31), "hils_chunk_logz_bwd_dq: B * H * L too large for the grid");
+    const dim3 grid = lz_xcd_grid(n_qt, B * H);
 #define LZ_LAUNCH(DD, GG)                                                                      \
   hipLaunchKernelGGL((logz_bwd_dq_mfma<DD, GG>), grid, dim3(256), 0, (hipStream_t)stream,      \
-                     (const bf16_t*)q, (const bf16_t*)k, log_z, d_log_z, (bf16_t*)dq, dm, n_qt)
+                     (const bf16_t*)q, (const bf16_t*)k, log_z, d_log_z, (bf16_t*)dq, dm, n_qt, B * H)
     LZ_DISPATCH(D, G);
 #undef LZ_LAUNCH
     HILS_CHECK_LAUNCH("hils_chunk_logz_bwd_dq");
@@ -678,10 +706,13 @@ extern "C" int hils_chunk_logz_bwd_dk(const void* q, const void* k, const float*
   HILS_REQUIRE(S * D <= LZ_MAX_ACC * LZ_THREADS, "hils_chunk_logz_bwd_dk: S*D (%d) too large", S * D);
   LzDims dm{L, HQ, H, G, D, S, window, (L + S - 1) / S, 0, sm_scale};
   if (lz_mfma_covers(G, D, S, H, B)) {
-    const dim3 grid((unsigned)((dm.N + 1) / 2), (unsigned)H, (unsigned)B);
+    const int n_pair = (dm.N + 1) / 2;
+    HILS_REQUIRE(((long)B * H + 7) / 8 * 8 * n_pair < (1L << 31), "hils_chunk_logz_bwd_dk: B * H * N too large for the grid");
+    const int n_unit = B * H;
+    const dim3 grid = lz_xcd_grid(n_pair, n_unit);
 #define LZ_LAUNCH(DD, GG)                                                                      \
   hipLaunchKernelGGL((logz_bwd_dk_mfma<DD, GG>), grid, dim3(256), 0, (hipStream_t)stream,      \
-                     (const bf16_t*)q, (const bf16_t*)k, log_z, d_log_z, (bf16_t*)dk, dm)
+                     (const bf16_t*)q, (const bf16_t*)k, log_z, d_log_z, (bf16_t*)dk, dm, n_pair, n_unit)
     LZ_DISPATCH(D, G);
 #undef LZ_LAUNCH
     HILS_CHECK_LAUNCH("hils_chunk_logz_bwd_dk");
