@@ -527,6 +527,8 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="profiling aid: decode step only")
     ap.add_argument("--train-only", action="store_true",
                     help="profiling aid: only the config-5 training layer forward+backward")
+    ap.add_argument("--ops-only", action="store_true",
+                    help="profiling aid: only the secondary operators (pooling, log-Z, sliding window, RoPE, HSA)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: run only a 512 MiB device copy (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters)")
@@ -556,6 +558,9 @@ def main():
         return
     if args.train_only:
         print(json.dumps({"train_fwd_bwd": bench_train(pkg, dev)}))
+        return
+    if args.ops_only:
+        print(json.dumps({"ops": bench_ops(pkg, dev)}))
         return
     if args.no_prefill:
         dsec, dper, droof = bench_decode(pkg, dev, max(args.steps, 20), args.warmup)
