@@ -118,20 +118,21 @@ __device__ __forceinline__ uint32_t tg_kth_largest(const uint32_t (&k)[NE], uint
   return T;
 }
 
-// NB: chunk blocks the launch covers, 8, 16 or 32.  Every query of the launch sees at most 16*NB
+// NB: chunk blocks the launch covers, 8, 16, 24 or 32.  Every query of the launch sees at most 16*NB
 // chunks and more than 16*NB/2 (NB = 8: any number), so only the blocks from NMASK on can hold
 // invisible chunks; t_base: first query.  Everything is unrolled over the NB blocks: register-resident
 // data has no other way of being indexed, and the host splits a call into launches by NB so that
-// early queries do not pay for 32.  (A 24-block instantiation for the queries that see 257..384
-// chunks ran no faster than this kernel at 32; the time goes by the schedule the compiler finds at
-// the given register budget as much as by the work.)
+// early queries do not pay for 32.  (The 24-block instantiation pays through its occupancy: held to
+// 168 registers it runs three wavefronts per SIMD with ten spilled dwords, 114 us for the queries that
+// see 257..384 chunks against 133 us of the 32-block kernel; at two wavefronts per SIMD it was no
+// faster than 32 blocks.)
 // Wavefronts per workgroup, each with queries of its own (they never synchronise).  A workgroup keeps
 // its registers and LDS until its slowest wavefront is through (the threshold searches differ in
 // length): 4 per workgroup ran 3.5 % slower than 2, and 8 ran 17 % slower; 1 was no faster than 2.
 #define TG_WAVES 2
 template <int GMAX, int KS, int NB, bool EXPORT>
 __global__ void __launch_bounds__(64 * TG_WAVES)
-    __attribute__((amdgpu_waves_per_eu(NB <= 8 ? 5 : (NB <= 16 ? 4 : 2))))
+    __attribute__((amdgpu_waves_per_eu(NB <= 8 ? 5 : (NB <= 16 ? 4 : (NB <= 24 ? 3 : 2)))))
 topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lmk_packed,
                       const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
                       bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
@@ -505,13 +506,14 @@ static void tg_launch_range(int NB, bool exp, dim3 grid, hipStream_t st, const b
   switch (NB) {
     case 8: TG_CALL(8, false); break;
     case 16: TG_CALL(16, false); break;
+    case 24: TG_CALL(24, false); break;
     default: TG_CALL(32, false); break;
   }
 #undef TG_CALL
 }
 
 // lmk_packed: the chunk keys in topk_pack_lmk_kernel's order.  The queries are split by how many
-// chunks they can see (at most 8, 16 or 32 blocks of 16) into one launch each.
+// chunks they can see (at most 8, 16, 24 or 32 blocks of 16) into one launch each.
 int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* lse_swa, int32_t* indices,
                            void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
                            int G, int D, int topk, int block_size, int window_size, int causal, int q_offset,
@@ -530,7 +532,7 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
     int NB = 32, t_hi = L;
     if (!exp) {
       const int lm = limit_of(t);
-      NB = lm <= 128 ? 8 : (lm <= 256 ? 16 : 32);
+      NB = lm <= 128 ? 8 : (lm <= 256 ? 16 : (lm <= 384 ? 24 : 32));
       if (NB < 32) {
         int lo = t, hi = L;  // first query whose limit exceeds 16 * NB
         while (lo < hi) {
