@@ -326,7 +326,9 @@ def test_topk_one_pass_prefill_kernel(pkg, orc, dev, L, N, h_kv, G, D, topk, dup
 
 @pytest.mark.parametrize("G,D,L,N,topk,W,S,h_kv", [
     (4, 128, 12800, 200, 32, 1, 64, 2),   # queries of the 8- and 16-block launches
-    (4, 64, 32000, 500, 32, 1, 64, 1),    # all three launches
+    (4, 64, 32000, 500, 32, 1, 64, 1),    # all four launches
+    (1, 128, 22000, 343, 32, 1, 64, 1),   # the 24-block launch without head grouping
+    (3, 64, 24000, 375, 16, 1, 64, 1),    # ... and with a padding head row
     (1, 64, 9000, 250, 16, 1, 64, 2),     # 16 queries per wavefront
     (3, 128, 7000, 140, 9, 64, 64, 1),    # a padding head row, odd k, a wide window
     (4, 128, 6000, 125, 16, 1, 48, 1),    # chunk sizes that are no power of two (visibility by division)
