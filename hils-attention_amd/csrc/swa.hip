@@ -412,8 +412,10 @@ constexpr int swa_dq_rt(int D, int DV) { return (D <= 64 && DV <= 64) ? 2 : 1; }
 
 // dQ (and delta): a wavefront owns 16 * RT score rows; K (row-major and transposed) and V stream.
 template <int D, int DV, int G>
-// (the hint gives two wavefronts per SIMD and keeps the accumulators out of accumulation registers)
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+// (the hint keeps the accumulators out of accumulation registers; wide heads with their one tile per
+// wavefront are held to 168 registers, five spilled dwords, for three wavefronts per SIMD: 52 KiB of LDS
+// let three workgroups share a compute unit)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((D > 64 && DV > 64) ? 3 : 2)))
 swa_bwd_dq_mfma(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
                 const bf16_t* __restrict__ o, const float* __restrict__ lse,
                 const bf16_t* __restrict__ d_o, const float* __restrict__ d_lse,
