@@ -23,6 +23,22 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
+
+def _load_inputs():
+    """The synthetic-input builders live with the parity tests (tests/util.py), which check the
+    kernels on exactly the tensors timed here."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("hils_test_util", os.path.join(ROOT, "tests", "util.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+_inputs = _load_inputs()
+gpu_randn, swa_lse_current_chunk = _inputs.gpu_randn, _inputs.swa_lse_current_chunk
+prefill_inputs, config2_inputs = _inputs.prefill_inputs, _inputs.config2_inputs
+train_inputs, train_forward = _inputs.train_inputs, _inputs.train_forward
+
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 
@@ -43,35 +59,6 @@ def measured_traffic(key):
     return None
 
 
-def gpu_randn(shape, gen, dev, scale=None, chunk=1 << 26):
-    """bf16 N(0,1) tensor generated on the GPU in slices (no fp32 copy of the whole tensor)."""
-    out = torch.empty(shape, dtype=torch.bfloat16, device=dev)
-    flat = out.view(-1)
-    for s in range(0, flat.numel(), chunk):
-        e = min(flat.numel(), s + chunk)
-        flat[s:e] = torch.randn(e - s, device=dev, generator=gen).bfloat16()
-    if scale is not None:
-        out.mul_(scale.to(torch.bfloat16))
-    return out
-
-
-def swa_lse_current_chunk(q, k, S):
-    """Exact lse of the local branch for window 1: keys of the query's own chunk up to the
-    query, landmark (last token of the chunk) masked.  (B,L,HQ) fp32, computed with torch."""
-    B, L, HQ, D = q.shape
-    H = k.shape[2]
-    G = HQ // H
-    N = L // S
-    qc = q.view(B, N, S, H, G, D).float()
-    kc = k.view(B, N, S, H, D).float()
-    s = torch.einsum("bnihgd,bnjhd->bnhgij", qc, kc) / math.sqrt(D)
-    i = torch.arange(S, device=q.device).view(S, 1)
-    j = torch.arange(S, device=q.device).view(1, S)
-    s = s.masked_fill((j > i) | (j == S - 1), float("-inf"))
-    lse = torch.logsumexp(s, dim=-1)  # (B,N,H,G,S)
-    return lse.permute(0, 1, 4, 2, 3).reshape(B, L, HQ).contiguous()
-
-
 def time_steps(fn, steps, warmup):
     for _ in range(warmup):
         fn()
@@ -87,12 +74,7 @@ def bench_prefill(pkg, dev, steps, warmup):
     from hils_attention_amd.ops import hils_fwd_bwd_head as attn_mod
     B, L, HQ, H, D, S, K, W = 1, 32768, 32, 8, 128, 64, 32, 1
     G = HQ // H
-    gen = torch.Generator(device=dev).manual_seed(1003)
-    hs = torch.rand(HQ, device=dev, generator=gen) * 1.5 + 0.5
-    q = gpu_randn((B, L, HQ, D), gen, dev, hs.view(1, 1, HQ, 1))
-    k = gpu_randn((B, L, H, D), gen, dev, hs[::G].view(1, 1, H, 1))
-    v = gpu_randn((B, L, H, D), gen, dev)
-    lse_swa = swa_lse_current_chunk(q, k, S).bfloat16()  # the layer hands it over in bf16
+    q, k, v, lse_swa = prefill_inputs(dev)  # lse_swa in bf16, as the layer hands it over
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
     state = {}
     acc = {"pool": 0.0, "topk": 0.0, "glue": 0.0, "vt": 0.0, "attn": 0.0, "n": 0}
@@ -145,17 +127,6 @@ def bench_prefill(pkg, dev, steps, warmup):
            "global_batch": B, "seq_len": L, "n_sel": n_sel}
     data = {"q": q, "k": k, "v": v, "lse_swa": lse_swa}
     return sec, per, roof, cfg, data
-
-
-def config2_inputs(dev):
-    """Config 2 inputs: B4 L8192, 16 heads MHA, D64; q, k, v ~ N(0,1) (seed 1002), lse_swa = the
-    exact lse of the query's own chunk, in bf16 as the layer hands it over."""
-    B, L, HQ, H, D, S = 4, 8192, 16, 16, 64, 64
-    gen = torch.Generator(device=dev).manual_seed(1002)
-    q = gpu_randn((B, L, HQ, D), gen, dev)
-    k = gpu_randn((B, L, H, D), gen, dev)
-    v = gpu_randn((B, L, H, D), gen, dev)
-    return q, k, v, swa_lse_current_chunk(q, k, S).bfloat16()
 
 
 def bench_config2(pkg, dev, iters=5):
@@ -270,29 +241,6 @@ def bench_decode(pkg, dev, steps, warmup):
     del kc, vc
     torch.cuda.empty_cache()
     return sec, per, roof
-
-
-def train_inputs(dev):
-    """Config 5 inputs: B8 L8192, 16 heads MHA, D64; q, k, v (leaves that require grad) and the
-    upstream gradient d_o ~ N(0,1) (seed 1005), lse_swa = the exact fp32 lse of the own chunk."""
-    B, L, HQ, H, D, S = 8, 8192, 16, 16, 64, 64
-    gen = torch.Generator(device=dev).manual_seed(1005)
-    q = gpu_randn((B, L, HQ, D), gen, dev).requires_grad_()
-    k = gpu_randn((B, L, H, D), gen, dev).requires_grad_()
-    v = gpu_randn((B, L, H, D), gen, dev).requires_grad_()
-    d_o = gpu_randn((B, L, HQ, D), gen, dev)
-    return q, k, v, d_o, swa_lse_current_chunk(q.detach(), k.detach(), S)
-
-
-def train_forward(pkg, q, k, v, lse_swa, keep=False):
-    """The training layer's remote branch: mean pool -> top-k scores -> softmax over
-    [scores, lse_swa] -> sparse attention.  Returns (o, idx), plus scores and weights with keep."""
-    S, K, W = 64, 32, 1
-    lmk = pkg.chunk_mean_pool(k, S)
-    idx, scores = pkg.online_softmax_topk_head(q, lmk, lse_swa, K, S, W, is_training=True)
-    w = pkg.chunk_weights(scores, lse_swa)
-    o = pkg.HiLS_block_M_head(q, k, v, w, idx, block_size=S, is_training=True)
-    return (o, idx, scores, w) if keep else (o, idx)
 
 
 def bench_train(pkg, dev, iters=3):
@@ -491,30 +439,6 @@ def cpu_baseline(data, n_queries=4096):
                       f"{dt:.2f} s", "seconds": dt}
 
 
-def bench_stream_probe(pkg, dev, gib=4, reps=20):
-    """TB/s of hils_stream_probe over a buffer far larger than the 256 MiB last-level cache."""
-    from importlib import import_module
-    cabi = import_module(pkg.__name__ + ".ops._cabi")
-    cabi.load()
-    buf = torch.empty(gib << 30, dtype=torch.uint8, device=dev).fill_(1)
-    sink = torch.zeros(1, dtype=torch.int32, device=dev)
-    out = {"bytes": int(buf.numel())}
-    for name, pattern in (("contiguous", 0), ("rows_256B_stride_2KiB", 1)):
-        def run():
-            cabi.call("hils_stream_probe", buf.data_ptr(), buf.numel(), pattern, sink.data_ptr())
-        for _ in range(3):
-            run()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            run()
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / reps
-        out[name] = {"ms": round(ms, 4), "TB_per_s": round(buf.numel() / ms / 1e9, 3)}
-    return out
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -532,9 +456,6 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: run only a 512 MiB device copy (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters)")
-    ap.add_argument("--stream-probe", action="store_true",
-                    help="measurement aid: the rate of a kernel that only loads, contiguous and as "
-                         "256-byte rows at a 2 KiB stride (what the streaming kernels can reach)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives are part of the hot "
@@ -552,9 +473,6 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes": int(src.numel())}))
-        return
-    if args.stream_probe:
-        print(json.dumps({"stream_probe": bench_stream_probe(pkg, dev)}))
         return
     if args.train_only:
         print(json.dumps({"train_fwd_bwd": bench_train(pkg, dev)}))

@@ -338,12 +338,19 @@ static int sa_merge_local(void* o, const void* swa_o, const void* weights, int B
 extern "C" int hils_sparse_attn_fwd(const void* q, const void* k, const void* v,
                                     const void* weights, const int32_t* indices,
                                     const float* slope, const void* swa_o, void* o, float* lse,
-                                    void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ,
-                                    int H, int D, int Dv, int K, int NW, int WH, int q_block, int S,
-                                    float sm_scale, int mask_last, float sm_n, int merge_col,
+                                    void* workspace, size_t workspace_bytes, int workspace_ready, int B, int L,
+                                    int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int WH, int q_block,
+                                    int S, float sm_scale, int mask_last, float sm_n, int merge_col,
                                     void* stream) {
   HILS_REQUIRE(q && k && v && weights && indices && o, "hils_sparse_attn_fwd: null pointer");
   if (int rc = sa_check("hils_sparse_attn_fwd", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
+  {
+    const size_t need = hils_sparse_attn_fwd_workspace(B, L, Lkv, HQ, H, D, Dv, K, WH, q_block, S, sm_n);
+    HILS_REQUIRE(!workspace || workspace_bytes >= need,
+                 "hils_sparse_attn_fwd: workspace of %zu bytes is shorter than the %zu bytes "
+                 "hils_sparse_attn_fwd_workspace returns for this shape (a workspace packed for another "
+                 "shape cannot be reused)", workspace_bytes, need);
+  }
   HILS_REQUIRE(!swa_o || (merge_col >= 0 && merge_col < NW),
                "hils_sparse_attn_fwd: merge_col (%d) must be a weight column (0..%d)", merge_col, NW - 1);
   if (hils_decode_covers(L, HQ, H, D, Dv, S, q_block, WH, sm_n, slope, lse) && Lkv >= S) {
@@ -423,7 +430,8 @@ merge_local_bwd_kernel(const bf16_t* __restrict__ d_o, const bf16_t* __restrict_
 extern "C" int hils_sparse_attn_bwd(const void* q, const void* k, const void* v,
                                     const void* weights, const int32_t* indices,
                                     const float* slope, const float* lse, const void* d_o,
-                                    void* dq, void* dk, void* dv, float* dw, void* workspace, int B,
+                                    void* dq, void* dk, void* dv, float* dw, void* workspace,
+                                    size_t workspace_bytes, int B,
                                     int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int WH,
                                     int q_block, int S, float sm_scale, int mask_last, float sm_n,
                                     const void* swa_o, void* d_swa_o, int merge_col, int kv_grad_bf16,
@@ -431,6 +439,12 @@ extern "C" int hils_sparse_attn_bwd(const void* q, const void* k, const void* v,
   HILS_REQUIRE(q && k && v && weights && indices && lse && d_o && dq && dk && dv && dw,
                "hils_sparse_attn_bwd: null pointer");
   if (int rc = sa_check("hils_sparse_attn_bwd", B, L, Lkv, HQ, H, D, Dv, K, NW, WH, q_block, S)) return rc;
+  {
+    const size_t need = hils_bw_workspace_bytes(B, L, Lkv, HQ, H, D, Dv, K, S, q_block, WH, sm_n);
+    HILS_REQUIRE(!workspace || workspace_bytes >= need,
+                 "hils_sparse_attn_bwd: workspace of %zu bytes is shorter than the %zu bytes "
+                 "hils_sparse_attn_bwd_workspace returns for this shape", workspace_bytes, need);
+  }
   if (swa_o) {  // the forward merged the local branch: its gradient and that of its weight column
     const int lpr = Dv / 8;
     HILS_REQUIRE(d_swa_o && merge_col >= K && merge_col < NW && q_block == 1 && WH == HQ && lpr <= 64 &&

@@ -244,11 +244,16 @@ extern "C" size_t hils_sparse_attn_decode_paged_workspace(int B, int L, int HQ, 
 
 extern "C" int hils_sparse_attn_decode_paged(const void* q, const void* k_pages, const void* v_pages,
                                              const int32_t* page_table, const void* weights,
-                                             const int32_t* indices, void* o, void* workspace, int B, int L,
+                                             const int32_t* indices, void* o, void* workspace,
+                                             size_t workspace_bytes, int B, int L,
                                              int HQ, int H, int D, int K, int NW, int max_pages, int num_pages,
                                              float sm_scale, int mask_last, void* stream) {
   HILS_REQUIRE(q && k_pages && v_pages && page_table && weights && indices && o,
                "hils_sparse_attn_decode_paged: null pointer");
+  HILS_REQUIRE(!workspace || workspace_bytes >= hils_decode_workspace_bytes(B, L, HQ, H, D, K),
+               "hils_sparse_attn_decode_paged: workspace of %zu bytes is shorter than the %zu bytes "
+               "hils_sparse_attn_decode_paged_workspace returns for this shape", workspace_bytes,
+               hils_decode_workspace_bytes(B, L, HQ, H, D, K));
   HILS_REQUIRE(B > 0 && L > 0 && HQ > 0 && H > 0 && HQ % H == 0 && K > 0 && NW >= K && max_pages > 0 && num_pages > 0,
                "hils_sparse_attn_decode_paged: bad sizes");
   HILS_REQUIRE(hils_decode_rows_covers(D, D, HQ / H, K),

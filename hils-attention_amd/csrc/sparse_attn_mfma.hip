@@ -833,13 +833,19 @@ void hils_ga_pack_launch(const void* a, const void* b, void* ap, void* bp, float
                      (const bf16_t*)b, (bf16_t*)ap, (bf16_t*)bp, bmax, Lkv, H, Da, Db, nchunk);
 }
 
-extern "C" int hils_pack_kv_chunks(const void* k, const void* v, void* workspace, int B, int Lkv,
-                                   int H, int D, int Dv, void* stream) {
+extern "C" int hils_pack_kv_chunks(const void* k, const void* v, void* workspace, size_t workspace_bytes,
+                                   int B, int Lkv, int H, int D, int Dv, void* stream) {
   HILS_REQUIRE(k && v && workspace, "hils_pack_kv_chunks: null pointer");
   HILS_REQUIRE(B > 0 && Lkv >= GA_S && H > 0 && (D == 64 || D == 128) && (Dv == 64 || Dv == 128),
                "hils_pack_kv_chunks: bad sizes (Lkv >= 64, D and Dv in {64, 128})");
   HILS_REQUIRE(H <= 65535 && B <= 65535, "hils_pack_kv_chunks: H/B too large for the grid");
   const int nchunk = Lkv / GA_S;
+  {
+    const size_t need = ga_vt_bytes(B, H, nchunk, Dv) + ga_vt_bytes(B, H, nchunk, D) + ga_vmax_bytes(B, H, nchunk);
+    HILS_REQUIRE(workspace_bytes >= need,
+                 "hils_pack_kv_chunks: workspace of %zu bytes is shorter than the %zu bytes the packed K, V and "
+                 "per-chunk maxima of this shape take", workspace_bytes, need);
+  }
   bf16_t* vpk = (bf16_t*)workspace;
   bf16_t* kpk = (bf16_t*)((char*)workspace + ga_vt_bytes(B, H, nchunk, Dv));
   float* vmax = (float*)((char*)kpk + ga_vt_bytes(B, H, nchunk, D));

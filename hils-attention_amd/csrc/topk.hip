@@ -1875,7 +1875,7 @@ static int topk_fwd_split(const void* q, const void* lmks, const float* lse_swa,
 static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
                          const float* bias, const float* gumbel, const int32_t* drop_mask,
                          int32_t* indices, void* scores, float* lse_total, float* sel_logits,
-                         void* workspace, void* weights, int* weights_fused, int B, int L, int N,
+                         void* workspace, size_t workspace_bytes, void* weights, int* weights_fused, int B, int L, int N,
                          int h_kv, int G, int D, int topk, int block_size, int window_size,
                          int causal, int q_offset, int per_qhead, float sm_scale, void* stream,
                          int lse_bf16 = 0) {
@@ -1885,6 +1885,9 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
   HILS_REQUIRE(G <= 16, "hils_topk_fwd: group size %d not supported (max 16)", G);
   HILS_REQUIRE(block_size > 0, "hils_topk_fwd: block_size must be positive");
   HILS_REQUIRE(h_kv <= 65535 && B <= 65535, "hils_topk_fwd: h_kv/B too large for the grid");
+  HILS_REQUIRE(!workspace || workspace_bytes >= hils_topk_fwd_workspace(B, L, N, h_kv, G),
+               "hils_topk_fwd: workspace of %zu bytes is shorter than the %zu bytes hils_topk_fwd_workspace "
+               "returns for this shape", workspace_bytes, hils_topk_fwd_workspace(B, L, N, h_kv, G));
   hipStream_t st = (hipStream_t)stream;
   HILS_REQUIRE(!lse_bf16 || hils_topk_lse16_covers(B, L, N, h_kv, G, D, topk),
                "hils_topk_fwd_weights_lse16: shape not taken by the one-pass prefill kernel "
@@ -1982,25 +1985,25 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
 extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_swa,
                              const float* bias, const float* gumbel, const int32_t* drop_mask,
                              int32_t* indices, void* scores, float* lse_total, float* sel_logits,
-                             void* workspace, int B, int L, int N, int h_kv, int G, int D, int topk,
-                             int block_size, int window_size, int causal, int q_offset,
+                             void* workspace, size_t workspace_bytes, int B, int L, int N, int h_kv, int G,
+                             int D, int topk, int block_size, int window_size, int causal, int q_offset,
                              int per_qhead, float sm_scale, void* stream) {
   int fused = 0;
   return topk_fwd_impl(q, lmks, lse_swa, bias, gumbel, drop_mask, indices, scores, lse_total, sel_logits,
-                       workspace, nullptr, &fused, B, L, N, h_kv, G, D, topk, block_size, window_size,
+                       workspace, workspace_bytes, nullptr, &fused, B, L, N, h_kv, G, D, topk, block_size, window_size,
                        causal, q_offset, per_qhead, sm_scale, stream);
 }
 
 extern "C" int hils_topk_fwd_weights(const void* q, const void* lmks, const float* lse_swa,
                                      const float* bias, const float* gumbel, const int32_t* drop_mask,
                                      int32_t* indices, void* scores, void* weights, void* workspace,
-                                     int B, int L, int N, int h_kv, int G, int D, int topk,
+                                     size_t workspace_bytes, int B, int L, int N, int h_kv, int G, int D, int topk,
                                      int block_size, int window_size, int causal, int q_offset,
                                      int per_qhead, float sm_scale, void* stream) {
   HILS_REQUIRE(weights, "hils_topk_fwd_weights: null pointer");
   int fused = 0;
   if (int rc = topk_fwd_impl(q, lmks, lse_swa, bias, gumbel, drop_mask, indices, scores, nullptr, nullptr,
-                             workspace, weights, &fused, B, L, N, h_kv, G, D, topk, block_size,
+                             workspace, workspace_bytes, weights, &fused, B, L, N, h_kv, G, D, topk, block_size,
                              window_size, causal, q_offset, per_qhead, sm_scale, stream))
     return rc;
   if (fused) return HILS_OK;
@@ -2010,14 +2013,14 @@ extern "C" int hils_topk_fwd_weights(const void* q, const void* lmks, const floa
 
 extern "C" int hils_topk_fwd_weights_lse16(const void* q, const void* lmks, const void* lse_swa_bf16,
                                            int32_t* indices, void* scores, void* weights, void* workspace,
-                                           int B, int L, int N, int h_kv, int G, int D, int topk,
-                                           int block_size, int window_size, int causal, int q_offset,
+                                           size_t workspace_bytes, int B, int L, int N, int h_kv, int G, int D,
+                                           int topk, int block_size, int window_size, int causal, int q_offset,
                                            float sm_scale, void* stream) {
   HILS_REQUIRE(weights && workspace, "hils_topk_fwd_weights_lse16: null pointer");
   int fused = 0;
   if (int rc = topk_fwd_impl(q, lmks, (const float*)lse_swa_bf16, nullptr, nullptr, nullptr, indices, scores,
-                             nullptr, nullptr, workspace, weights, &fused, B, L, N, h_kv, G, D, topk,
-                             block_size, window_size, causal, q_offset, 0, sm_scale, stream, 1))
+                             nullptr, nullptr, workspace, workspace_bytes, weights, &fused, B, L, N, h_kv, G, D,
+                             topk, block_size, window_size, causal, q_offset, 0, sm_scale, stream, 1))
     return rc;
   if (fused) return HILS_OK;
   return hils_chunk_weights(scores, lse_swa_bf16, 1, nullptr, nullptr, weights, B, L, h_kv * G, h_kv, N, topk, 0,
@@ -2102,7 +2105,7 @@ extern "C" int hils_topk_fwd_noalloc(const void* q, const void* lmks, const floa
   // (repacked chunk keys, or the logits parked between the two decode kernels): nothing to clear
   int fused = 0;
   return topk_fwd_impl(q, lmks, lse_swa, bias, gumbel, drop_mask, indices, scores, lse_total, sel_logits,
-                       ws, nullptr, &fused, B, L, N, h_kv, G, D, topk, block_size, window_size, causal,
+                       ws, HILS_TOPK_SCRATCH_BYTES, nullptr, &fused, B, L, N, h_kv, G, D, topk, block_size, window_size, causal,
                        q_offset, per_qhead, sm_scale, stream);
 }
 
@@ -2466,10 +2469,13 @@ extern "C" size_t hils_topk_bwd_workspace(int B, int L, int N, int h_kv, int G, 
 }
 
 extern "C" int hils_topk_bwd(const void* g_scores, const void* q, const void* lmks,
-                             const int32_t* indices, void* dq, float* dlmk, void* workspace, int B,
-                             int L, int N, int h_kv, int G, int D, int topk, int per_qhead,
-                             float sm_scale, void* stream) {
+                             const int32_t* indices, void* dq, float* dlmk, void* workspace,
+                             size_t workspace_bytes, int B, int L, int N, int h_kv, int G, int D, int topk,
+                             int per_qhead, float sm_scale, void* stream) {
   HILS_REQUIRE(g_scores && q && lmks && indices && dq && dlmk, "hils_topk_bwd: null pointer");
+  HILS_REQUIRE(!workspace || workspace_bytes >= hils_topk_bwd_workspace(B, L, N, h_kv, G, D, topk),
+               "hils_topk_bwd: workspace of %zu bytes is shorter than the %zu bytes hils_topk_bwd_workspace "
+               "returns for this shape", workspace_bytes, hils_topk_bwd_workspace(B, L, N, h_kv, G, D, topk));
   HILS_REQUIRE(B > 0 && L > 0 && N > 0 && h_kv > 0 && G > 0 && D > 0 && topk > 0, "hils_topk_bwd: sizes must be positive");
   const long rows = (long)B * L * h_kv;
   HILS_REQUIRE(rows <= 2147483647L, "hils_topk_bwd: grid too large");

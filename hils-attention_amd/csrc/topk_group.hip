@@ -290,11 +290,15 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
     if (mn > HILS_NEG_INF) tot2 = mx + __builtin_amdgcn_logf(1.f + __builtin_amdgcn_exp2f(mn - mx));
     // a row that does not exist (a padding head of a group of three, a query past the end) must not
     // reach the selection: its logits are not masked in the blocks every real row sees (they are 0 there)
-    lse_tot[i] = rowok[i] ? tot2 * HILS_LN2 : __builtin_inff();
+    const float lt = tot2 * HILS_LN2;
     if (lse_total_out && col == 0 && rowok[i]) {
       const int r = 4 * j + i;
-      lse_total_out[((b * L + t0 + r / GMAX) * (long)h_kv + hk) * G + r % GMAX] = lse_tot[i];
+      lse_total_out[((b * L + t0 + r / GMAX) * (long)h_kv + hk) * G + r % GMAX] = lt;
     }
+    // A row that sees no chunk and has lse_swa = -inf has lse_total = -inf; its logits are all -inf,
+    // and -inf - -inf would be a NaN, which this file is compiled not to expect: such a row subtracts
+    // 0 instead (its scores stay -inf, nothing is selected).
+    lse_tot[i] = rowok[i] ? (tot2 > HILS_NEG_INF ? lt : 0.f) : __builtin_inff();
   }
 
   // outputs start as "no winner"
@@ -307,8 +311,8 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   for (int u = 0; u < QPL; ++u) {
     const int qi = j * QPL + u;  // query of the wavefront this lane row works on
     // selection score of chunk nt*16+col: max over the heads of (logit - lse_total), one fp32
-    // subtraction each; -inf where the chunk is not visible (-inf - lse is -inf or NaN, and fmaxf
-    // skips NaN).  Scores are compared as floats (+0 == -0, as in the reference's sort); only the few
+    // subtraction each; -inf where the chunk is not visible (lse_tot is never -inf, so no NaN is
+    // formed).  Scores are compared as floats (+0 == -0, as in the reference's sort); only the few
     // candidates of the threshold search are turned into integer keys.
     float key[NB];
 #pragma unroll

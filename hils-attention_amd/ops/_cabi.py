@@ -14,7 +14,7 @@ import torch
 _PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG_DIR, "libhils_amd.so")
 
-_P, _I, _F = c_void_p, c_int, c_float
+_P, _I, _F, _Z = c_void_p, c_int, c_float, ctypes.c_size_t
 
 # name -> argument types, in the order of include/hils_amd.h
 SIGNATURES = {
@@ -22,18 +22,18 @@ SIGNATURES = {
     "hils_mean_pool_bwd": [_P, _P, _I, _I, _I, _I, _I, _P],
     "hils_attn_pool_fwd": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
     "hils_attn_pool_bwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
-    "hils_topk_fwd": [_P] * 11 + [_I] * 12 + [_F, _P],
+    "hils_topk_fwd": [_P] * 11 + [_Z] + [_I] * 12 + [_F, _P],
     "hils_topk_fwd_noalloc": [_P] * 10 + [_I] * 12 + [_F, _P],
-    "hils_topk_fwd_weights": [_P] * 10 + [_I] * 12 + [_F, _P],
-    "hils_topk_fwd_weights_lse16": [_P] * 7 + [_I] * 11 + [_F, _P],
+    "hils_topk_fwd_weights": [_P] * 10 + [_Z] + [_I] * 12 + [_F, _P],
+    "hils_topk_fwd_weights_lse16": [_P] * 7 + [_Z] + [_I] * 11 + [_F, _P],
     "hils_topk_fwd_weights_paged": [_P] * 9 + [_I] * 12 + [_F, _P],
-    "hils_sparse_attn_decode_paged": [_P] * 8 + [_I] * 9 + [_F, _I, _P],
+    "hils_sparse_attn_decode_paged": [_P] * 8 + [_Z] + [_I] * 9 + [_F, _I, _P],
     "hils_decode_step": [_P] * 11 + [_I] * 11 + [_F, _F, _I, _P],
     "hils_decode_step_paged": [_P] * 12 + [_I] * 12 + [_F, _F, _I, _P],
-    "hils_topk_bwd": [_P] * 7 + [_I] * 8 + [_F, _P],
-    "hils_sparse_attn_fwd": [_P] * 10 + [_I] * 13 + [_F, _I, _F, _I, _P],
-    "hils_pack_kv_chunks": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
-    "hils_sparse_attn_bwd": [_P] * 13 + [_I] * 12 + [_F, _I, _F, _P, _P, _I, _I, _P],
+    "hils_topk_bwd": [_P] * 7 + [_Z] + [_I] * 8 + [_F, _P],
+    "hils_sparse_attn_fwd": [_P] * 10 + [_Z] + [_I] * 13 + [_F, _I, _F, _I, _P],
+    "hils_pack_kv_chunks": [_P, _P, _P, _Z, _I, _I, _I, _I, _I, _P],
+    "hils_sparse_attn_bwd": [_P] * 13 + [_Z] + [_I] * 12 + [_F, _I, _F, _P, _P, _I, _I, _P],
     "hils_sparse_attn_fwd_f32": [_P] * 8 + [_I] * 12 + [_F, _I, _F, _P],
     "hils_sparse_attn_bwd_f32": [_P] * 12 + [_I] * 12 + [_F, _I, _F, _P],
     "hils_chunk_weights": [_P, _P, _I, _P, _P, _P] + [_I] * 7 + [_P],
@@ -71,8 +71,6 @@ def load():
     lib.hils_topk_fwd_noalloc_max_workspace.argtypes = []
     lib.hils_sparse_attn_decode_paged_workspace.restype = ctypes.c_size_t
     lib.hils_sparse_attn_decode_paged_workspace.argtypes = [_I] * 6
-    lib.hils_stream_probe.restype = c_int
-    lib.hils_stream_probe.argtypes = [_P, ctypes.c_size_t, _I, _P, _P]
     lib.hils_topk_lse16_covers.restype = c_int
     lib.hils_topk_lse16_covers.argtypes = [_I] * 7
     lib.hils_decode_step_covers.restype = c_int
@@ -96,6 +94,11 @@ def ptr(t):
     if t is None:
         return None
     return c_void_p(t.data_ptr())
+
+
+def nbytes(t):
+    """Size in bytes of the buffer behind a workspace tensor (None -> 0)."""
+    return 0 if t is None else t.numel() * t.element_size()
 
 
 def gpu_readable(t, device):

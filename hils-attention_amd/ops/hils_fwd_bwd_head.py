@@ -69,7 +69,7 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
                                                  int(block_size), 0.0)
         _cabi.call("hils_sparse_attn_fwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
                    _cabi.ptr(idx_in), _cabi.ptr(slope_dev), _cabi.ptr(swa_in), _cabi.ptr(o), _cabi.ptr(lse),
-                   _cabi.ptr(ws), ws_ready, B, L, L_kv, HQ, H, D, Dv, K, num_weights, HQ, 1, int(block_size),
+                   _cabi.ptr(ws), _cabi.nbytes(ws), ws_ready, B, L, L_kv, HQ, H, D, Dv, K, num_weights, HQ, 1, int(block_size),
                    float(sm_scale), int(bool(mask_last_token)), 0.0, merge_col)
         ctx.is_training = bool(is_training)
         if is_training:
@@ -101,7 +101,7 @@ class _hils_block_M_attention_inverse(torch.autograd.Function):
             dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)
         _cabi.call("hils_sparse_attn_bwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
                    _cabi.ptr(idx_in), _cabi.ptr(slope_dev), _cabi.ptr(lse), _cabi.ptr(do),
-                   _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), _cabi.ptr(ws),
+                   _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), _cabi.ptr(ws), _cabi.nbytes(ws),
                    B, L, L_kv, HQ, H, D, Dv, K, NW, HQ, 1, S, sm_scale, mask_last, 0.0,
                    _cabi.ptr(swa_in), _cabi.ptr(d_swa), merge_col, int(kv16))
         return (dq, dk.to(k.dtype), dv.to(v.dtype), dw.to(ctx.w_dtype), None,
@@ -215,5 +215,5 @@ def prepare_kv_workspace(q_len, k, v, num_q_heads, topk, block_size=64):
                                          topk, num_q_heads, 1, int(block_size), 0.0)
     if ws is not None and q_len >= 64:
         _cabi.call("hils_pack_kv_chunks", _cabi.ptr(k.contiguous()), _cabi.ptr(v.contiguous()),
-                   _cabi.ptr(ws), B, L_kv, H, D, Dv)
+                   _cabi.ptr(ws), _cabi.nbytes(ws), B, L_kv, H, D, Dv)
     return ws

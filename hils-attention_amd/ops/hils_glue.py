@@ -96,13 +96,13 @@ def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causa
         # lse_swa as the layer hands it over (bf16): read in place, no conversion pass
         _cabi.call("hils_topk_fwd_weights_lse16", _cabi.ptr(q.contiguous()), _cabi.ptr(lmks.contiguous()),
                    _cabi.ptr(lse_swa.reshape(B, L, h_q).contiguous()), _cabi.ptr(indices), _cabi.ptr(scores),
-                   _cabi.ptr(weights), _cabi.ptr(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),
+                   _cabi.ptr(weights), _cabi.ptr(ws), _cabi.nbytes(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),
                    int(window_size), int(bool(is_causal)), int(q_offset), scale)
         return indices, scores, weights
     lse = lse_swa.reshape(B, L, h_q).float().contiguous()
     _cabi.call("hils_topk_fwd_weights", _cabi.ptr(q.contiguous()), _cabi.ptr(lmks.contiguous()),
                _cabi.ptr(lse), None, None, None, _cabi.ptr(indices), _cabi.ptr(scores),
-               _cabi.ptr(weights), _cabi.ptr(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),
+               _cabi.ptr(weights), _cabi.ptr(ws), _cabi.nbytes(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),
                int(window_size), int(bool(is_causal)), int(q_offset), 0, scale)
     return indices, scores, weights
 

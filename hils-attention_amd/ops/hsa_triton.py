@@ -43,7 +43,7 @@ class _attention(torch.autograd.Function):
         ws = _cabi.sparse_attn_fwd_workspace(q.device, N, L, L_kv, HQ, H, D, v.shape[-1], K, H, q_x,
                                              int(chunk_size), float(sm_n))
         _cabi.call("hils_sparse_attn_fwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
-                   _cabi.ptr(idx_in), None, None, _cabi.ptr(o), _cabi.ptr(lse), _cabi.ptr(ws), 0,
+                   _cabi.ptr(idx_in), None, None, _cabi.ptr(o), _cabi.ptr(lse), _cabi.ptr(ws), _cabi.nbytes(ws), 0,
                    N, L, L_kv, HQ, H, D, v.shape[-1], K, K, H, q_x, int(chunk_size),
                    float(sm_scale), 0, float(sm_n), 0)
         ctx.save_for_backward(q, k, v, w_in, idx_in, lse)
@@ -69,7 +69,7 @@ class _attention(torch.autograd.Function):
             dk, dv = torch.empty_like(k), torch.empty_like(v)  # written once, as bf16
             _cabi.call("hils_sparse_attn_bwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_full),
                        _cabi.ptr(idx_full), None, _cabi.ptr(lse), _cabi.ptr(do),
-                       _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw_full), _cabi.ptr(ws),
+                       _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw_full), _cabi.ptr(ws), _cabi.nbytes(ws),
                        N, L, L_kv, HQ, H, D, Dv, K, K, HQ, 1, S, sm_scale, 0, sm_n, None, None, 0, 1)
             dw = dw_full.view(N, L // q_x, q_x, H, G, K).sum(dim=(2, 4))
             return (dq, dk.to(k.dtype), dv.to(v.dtype), dw.to(ctx.w_dtype),
@@ -79,7 +79,7 @@ class _attention(torch.autograd.Function):
         dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)
         _cabi.call("hils_sparse_attn_bwd", _cabi.ptr(q), _cabi.ptr(k), _cabi.ptr(v), _cabi.ptr(w_in),
                    _cabi.ptr(idx_in), None, _cabi.ptr(lse), _cabi.ptr(do),
-                   _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), None,
+                   _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), None, 0,
                    N, L, L_kv, HQ, H, D, Dv, K, K, H, q_x, S, sm_scale, 0, sm_n, None, None, 0, 0)
         return (dq, dk.to(k.dtype), dv.to(v.dtype), dw.to(ctx.w_dtype),
                 None, None, None, None, None, None)

@@ -48,7 +48,7 @@ class SoftmaxTopKMaxPoolingFusedFn(torch.autograd.Function):
         _cabi.call("hils_topk_fwd", _cabi.ptr(q_in), _cabi.ptr(k_in), _cabi.ptr(lse_in),
                    _cabi.ptr(bias), _cabi.ptr(gumbel_noise), _cabi.ptr(drop_mask),
                    _cabi.ptr(indices), _cabi.ptr(scores), _cabi.ptr(lse_total),
-                   _cabi.ptr(sel_logits), _cabi.ptr(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),
+                   _cabi.ptr(sel_logits), _cabi.ptr(ws), _cabi.nbytes(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),
                    int(window_size), int(bool(is_causal)), int(q_offset), int(bool(per_qhead_lmks)),
                    scale)
         if debug is not None:
@@ -68,7 +68,7 @@ class SoftmaxTopKMaxPoolingFusedFn(torch.autograd.Function):
         dlmk = torch.zeros(k_in.shape, dtype=torch.float32, device=k_in.device)
         ws = _cabi.topk_bwd_workspace(q_in.device, B, L, N, h_kv, G, D, topk)
         _cabi.call("hils_topk_bwd", _cabi.ptr(gs), _cabi.ptr(q_in), _cabi.ptr(k_in),
-                   _cabi.ptr(indices), _cabi.ptr(dq), _cabi.ptr(dlmk), _cabi.ptr(ws), B, L, N, h_kv, G, D, topk,
+                   _cabi.ptr(indices), _cabi.ptr(dq), _cabi.ptr(dlmk), _cabi.ptr(ws), _cabi.nbytes(ws), B, L, N, h_kv, G, D, topk,
                    int(per_qhead), scale)
         return (dq, dlmk.to(k_in.dtype)) + (None,) * 12
 

@@ -299,6 +299,6 @@ def paged_hils_attend(q, k_pages, v_pages, lmk_pages, page_table, lse_swa, seq_l
     n_ws = _cabi.load().hils_sparse_attn_decode_paged_workspace(B, Lq, HQ, H, D, int(topk))
     ws = torch.empty(n_ws, dtype=torch.uint8, device=dev) if n_ws else None
     _cabi.call("hils_sparse_attn_decode_paged", _cabi.ptr(qc), _cabi.ptr(k_pages), _cabi.ptr(v_pages),
-               _cabi.ptr(page_table), _cabi.ptr(weights), _cabi.ptr(indices), _cabi.ptr(o), _cabi.ptr(ws),
+               _cabi.ptr(page_table), _cabi.ptr(weights), _cabi.ptr(indices), _cabi.ptr(o), _cabi.ptr(ws), _cabi.nbytes(ws),
                B, Lq, HQ, H, D, int(topk), topk + 1, max_pages, num_pages, float(sm_scale), 1)
     return o, weights, indices

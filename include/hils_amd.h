@@ -68,12 +68,15 @@ int hils_attn_pool_bwd(const void* mu_q, const void* k, const float* p, const fl
  * (decode) and a workspace, the logits are spread over many workgroups and parked there
  * before a separate selection kernel (or one workgroup per (query, KV head) keeps them in LDS
  * and needs no scratch); with many queries the chunk keys are first repacked there into MFMA
- * operand order.  Without a workspace one fused kernel reads the chunk keys as they are. */
+ * operand order.  Without a workspace one fused kernel reads the chunk keys as they are.
+ * workspace_bytes: size of the buffer behind `workspace` (here and in every entry point that takes
+ * a workspace); a non-NULL workspace shorter than the matching *_workspace(...) query is rejected
+ * with status 1 before anything is launched. */
 size_t hils_topk_fwd_workspace(int B, int L, int N, int h_kv, int G);
 int hils_topk_fwd(const void* q, const void* lmks, const float* lse_swa, const float* bias,
                   const float* gumbel, const int32_t* drop_mask, int32_t* indices, void* scores,
-                  float* lse_total, float* sel_logits, void* workspace, int B, int L, int N,
-                  int h_kv, int G, int D, int topk, int block_size, int window_size, int causal,
+                  float* lse_total, float* sel_logits, void* workspace, size_t workspace_bytes, int B, int L,
+                  int N, int h_kv, int G, int D, int topk, int block_size, int window_size, int causal,
                   int q_offset, int per_qhead, float sm_scale, void* stream);
 
 /* hils_topk_fwd for callers that cannot allocate device memory (code under HIP graph capture,
@@ -100,8 +103,8 @@ int hils_topk_fwd_noalloc(const void* q, const void* lmks, const float* lse_swa,
  * same stream.  No lse_total / sel_logits outputs. */
 int hils_topk_fwd_weights(const void* q, const void* lmks, const float* lse_swa, const float* bias,
                           const float* gumbel, const int32_t* drop_mask, int32_t* indices,
-                          void* scores, void* weights, void* workspace, int B, int L, int N, int h_kv,
-                          int G, int D, int topk, int block_size, int window_size, int causal,
+                          void* scores, void* weights, void* workspace, size_t workspace_bytes, int B, int L,
+                          int N, int h_kv, int G, int D, int topk, int block_size, int window_size, int causal,
                           int q_offset, int per_qhead, float sm_scale, void* stream);
 
 /* hils_topk_fwd_weights for lse_swa in bf16, the dtype the reference's layer hands it over in
@@ -112,9 +115,9 @@ int hils_topk_fwd_weights(const void* q, const void* lmks, const float* lse_swa,
  * hils_topk_fwd_workspace; other shapes are rejected and take hils_topk_fwd_weights with fp32. */
 int hils_topk_lse16_covers(int B, int L, int N, int h_kv, int G, int D, int topk);
 int hils_topk_fwd_weights_lse16(const void* q, const void* lmks, const void* lse_swa_bf16, int32_t* indices,
-                                void* scores, void* weights, void* workspace, int B, int L, int N, int h_kv,
-                                int G, int D, int topk, int block_size, int window_size, int causal,
-                                int q_offset, float sm_scale, void* stream);
+                                void* scores, void* weights, void* workspace, size_t workspace_bytes, int B,
+                                int L, int N, int h_kv, int G, int D, int topk, int block_size, int window_size,
+                                int causal, int q_offset, float sm_scale, void* stream);
 
 /* Sparse backward of the score gather.  Replaces the dense scatter + two torch.bmm of
  * SoftmaxTopKMaxPoolingFusedFn.backward (ops/topk_head_softmax.py:1040-1092).
@@ -130,8 +133,8 @@ int hils_topk_fwd_weights_lse16(const void* q, const void* lmks, const void* lse
  * the atomic kernel. */
 size_t hils_topk_bwd_workspace(int B, int L, int N, int h_kv, int G, int D, int topk);
 int hils_topk_bwd(const void* g_scores, const void* q, const void* lmks, const int32_t* indices,
-                  void* dq, float* dlmk, void* workspace, int B, int L, int N, int h_kv, int G, int D,
-                  int topk, int per_qhead, float sm_scale, void* stream);
+                  void* dq, float* dlmk, void* workspace, size_t workspace_bytes, int B, int L, int N,
+                  int h_kv, int G, int D, int topk, int per_qhead, float sm_scale, void* stream);
 
 /* ---- inter-chunk softmax (layer glue) ------------------------------------------ */
 
@@ -179,16 +182,16 @@ size_t hils_sparse_attn_fwd_workspace(int B, int L, int Lkv, int HQ, int H, int 
                                       int WH, int q_block, int S, float sm_n);
 int hils_sparse_attn_fwd(const void* q, const void* k, const void* v, const void* weights,
                          const int32_t* indices, const float* slope, const void* swa_o, void* o,
-                         float* lse, void* workspace, int workspace_ready, int B, int L, int Lkv, int HQ,
-                         int H, int D, int Dv, int K, int NW, int WH, int q_block, int S, float sm_scale,
-                         int mask_last, float sm_n, int merge_col, void* stream);
+                         float* lse, void* workspace, size_t workspace_bytes, int workspace_ready, int B,
+                         int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW, int WH, int q_block,
+                         int S, float sm_scale, int mask_last, float sm_n, int merge_col, void* stream);
 /* Fills a workspace of hils_sparse_attn_fwd_workspace(...) bytes on its own: per 64-token
  * chunk of a (batch, KV head), K and V rewritten in the register order of the MFMA operands
  * the prefill kernel loads (every operand load becomes one contiguous 1 KiB burst), followed
  * by max|V| of every chunk (fp32).  No counterpart in the reference (TileLang stages K/V
  * through shared memory on every use). */
-int hils_pack_kv_chunks(const void* k, const void* v, void* workspace, int B, int Lkv, int H, int D,
-                        int Dv, void* stream);
+int hils_pack_kv_chunks(const void* k, const void* v, void* workspace, size_t workspace_bytes, int B,
+                        int Lkv, int H, int D, int Dv, void* stream);
 
 /* Backward.  Replaces hierarchical_sparse_attention_bwd_dqkv_block_M_inverse
  * (ops/hils_fwd_bwd_head.py:506-766) and kernel_attn_bwd_dq / _attn_bwd_dkdv /
@@ -211,7 +214,7 @@ size_t hils_sparse_attn_bwd_workspace(int B, int L, int Lkv, int HQ, int H, int 
 int hils_sparse_attn_bwd(const void* q, const void* k, const void* v, const void* weights,
                          const int32_t* indices, const float* slope, const float* lse,
                          const void* d_o, void* dq, void* dk, void* dv, float* dw, void* workspace,
-                         int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
+                         size_t workspace_bytes, int B, int L, int Lkv, int HQ, int H, int D, int Dv, int K, int NW,
                          int WH, int q_block, int S, float sm_scale, int mask_last, float sm_n,
                          const void* swa_o, void* d_swa_o, int merge_col, int kv_grad_bf16, void* stream);
 
@@ -255,9 +258,9 @@ int hils_topk_fwd_weights_paged(const void* q, const void* lmk_pages, const int3
 size_t hils_sparse_attn_decode_paged_workspace(int B, int L, int HQ, int H, int D, int K);
 int hils_sparse_attn_decode_paged(const void* q, const void* k_pages, const void* v_pages,
                                   const int32_t* page_table, const void* weights, const int32_t* indices,
-                                  void* o, void* workspace, int B, int L, int HQ, int H, int D, int K,
-                                  int NW, int max_pages, int num_pages, float sm_scale, int mask_last,
-                                  void* stream);
+                                  void* o, void* workspace, size_t workspace_bytes, int B, int L, int HQ, int H,
+                                  int D, int K, int NW, int max_pages, int num_pages, float sm_scale,
+                                  int mask_last, void* stream);
 
 /* ---- the remote branch of a decode step in one launch ---------------------------------- */
 
@@ -285,15 +288,6 @@ int hils_decode_step_paged(const void* q, const void* lmk_pages, const void* k_p
                            int HQ, int H, int D, int topk, int block_size, int window_size, int q_offset,
                            int max_pages, int num_pages, float sm_scale_sel, float sm_scale_attn,
                            int mask_last, void* stream);
-
-/* ---- measurement aid ---------------------------------------------------------------- */
-
-/* A kernel that only loads `bytes` bytes of buf (no counterpart in the reference): the rate any
- * streaming kernel can reach on this GPU.  pattern 0: contiguous shares per workgroup; pattern 1:
- * the buffer as a (tokens, 8 heads, 128) bf16 tensor read one head per workgroup (256-byte rows at
- * a 2 KiB stride, what the token-major decode kernels read).  sink: 4 bytes of device memory.
- * Both patterns skip a tail of the buffer that does not fill a whole round of loads. */
-int hils_stream_probe(const void* buf, size_t bytes, int pattern, void* sink, void* stream);
 
 /* ---- exact per-chunk log Z ---------------------------------------------------- */
 

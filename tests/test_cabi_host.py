@@ -43,7 +43,6 @@ def test_binding_matches_header(pkg):
     fns.pop("hils_sparse_attn_decode_paged_workspace")
     fns.pop("hils_decode_step_covers")
     fns.pop("hils_topk_lse16_covers")
-    fns.pop("hils_stream_probe")
     assert set(_cabi.SIGNATURES) == set(fns)
     for name, params in fns.items():
         argtypes = _cabi.SIGNATURES[name]
@@ -53,6 +52,8 @@ def test_binding_matches_header(pkg):
                 assert a is ctypes.c_void_p, (name, p)
             elif p.startswith("float"):
                 assert a is ctypes.c_float, (name, p)
+            elif p.startswith("size_t"):
+                assert a is ctypes.c_size_t, (name, p)
             else:
                 assert a is ctypes.c_int, (name, p)
 
@@ -66,15 +67,11 @@ def test_argument_errors_are_reported_without_a_gpu(pkg):
     assert lib.hils_mean_pool_fwd(buf, buf, 1, 100, 1, 64, 64, None) == 1
     assert b"multiple" in lib.hils_last_error()
     assert lib.hils_topk_fwd(buf, buf, buf, None, None, None, buf, buf, None, None, None,
-                             1, 16, 4, 1, 1, 64, 1000, 64, 1, 1, 0, 0, 0.125, None) == 1
+                             0, 1, 16, 4, 1, 1, 64, 1000, 64, 1, 1, 0, 0, 0.125, None) == 1
     assert b"topk" in lib.hils_last_error()
-    assert lib.hils_sparse_attn_fwd(buf, buf, buf, buf, buf, None, None, buf, None, None, 0,
+    assert lib.hils_sparse_attn_fwd(buf, buf, buf, buf, buf, None, None, buf, None, None, 0, 0,
                                     1, 16, 64, 3, 2, 64, 64, 4, 4, 3, 1, 64, 0.125, 1, 0.0, 0, None) == 1
     assert b"multiple of H" in lib.hils_last_error()
-    assert lib.hils_stream_probe(buf, 64 << 20, 2, buf, None) == 1
-    assert b"pattern" in lib.hils_last_error()
-    assert lib.hils_stream_probe(buf, 1 << 20, 0, buf, None) == 1
-    assert b"64 MiB" in lib.hils_last_error()
 
 
 def test_no_cpu_fallback(pkg):
@@ -195,3 +192,38 @@ def test_short_or_foreign_kv_workspace_is_rejected(pkg):
         _check_kv_workspace(torch.empty(large, dtype=torch.int8), large, cpu, "dtype")
     with pytest.raises(ValueError, match="kv_workspace"):
         _check_kv_workspace(torch.empty(large, dtype=torch.uint8), large, torch.device("meta"), "device")
+
+
+def test_short_workspace_is_rejected_by_the_c_abi(pkg):
+    """Every entry point that takes a workspace also takes its size in bytes and rejects a buffer
+    shorter than its *_workspace(...) query before anything is launched (no GPU needed: the check
+    comes first; the pointers are never dereferenced on the host)."""
+    from hils_attention_amd.ops import _cabi
+    lib = _cabi.load()
+    buf = ctypes.c_void_p(256)
+    B, L, HQ, H, D, K, S = 1, 4096, 8, 2, 128, 8, 64
+    need = lib.hils_sparse_attn_fwd_workspace(B, L, L, HQ, H, D, D, K, HQ, 1, S, 0.0)
+    assert need > 0
+    rc = lib.hils_sparse_attn_fwd(buf, buf, buf, buf, buf, None, None, buf, None, buf, need - 1, 1,
+                                  B, L, L, HQ, H, D, D, K, K + 1, HQ, 1, S, 0.088, 1, 0.0, 0, None)
+    assert rc == 1 and b"shorter" in lib.hils_last_error()
+    rc = lib.hils_pack_kv_chunks(buf, buf, buf, 1024, B, L, H, D, D, None)
+    assert rc == 1 and b"shorter" in lib.hils_last_error()
+    need_b = lib.hils_sparse_attn_bwd_workspace(B, L, L, HQ, H, D, D, K, HQ, 1, S, 0.0)
+    assert need_b > 0
+    rc = lib.hils_sparse_attn_bwd(buf, buf, buf, buf, buf, None, buf, buf, buf, buf, buf, buf, buf, need_b - 1,
+                                  B, L, L, HQ, H, D, D, K, K + 1, HQ, 1, S, 0.088, 1, 0.0, None, None, 0, 0, None)
+    assert rc == 1 and b"shorter" in lib.hils_last_error()
+    N, h_kv, G = L // S, H, HQ // H
+    need_t = lib.hils_topk_fwd_workspace(B, L, N, h_kv, G)
+    assert need_t > 0
+    rc = lib.hils_topk_fwd(buf, buf, buf, None, None, None, buf, buf, None, None, buf, need_t - 1,
+                           B, L, N, h_kv, G, D, K, S, 1, 1, 0, 0, 0.088, None)
+    assert rc == 1 and b"shorter" in lib.hils_last_error()
+    rc = lib.hils_topk_fwd_weights(buf, buf, buf, None, None, None, buf, buf, buf, buf, need_t - 1,
+                                   B, L, N, h_kv, G, D, K, S, 1, 1, 0, 0, 0.088, None)
+    assert rc == 1 and b"shorter" in lib.hils_last_error()
+    need_tb = lib.hils_topk_bwd_workspace(B, L, N, h_kv, 3, D, K)   # G = 3: the inverse-index kernels
+    assert need_tb > 0
+    rc = lib.hils_topk_bwd(buf, buf, buf, buf, buf, buf, buf, need_tb - 1, B, L, N, h_kv, 3, D, K, 0, 0.088, None)
+    assert rc == 1 and b"shorter" in lib.hils_last_error()

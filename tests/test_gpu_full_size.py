@@ -7,7 +7,7 @@ import math
 import pytest
 import torch
 
-import bench
+import util
 from util import assert_close_bf16, note
 
 pytestmark = pytest.mark.gpu
@@ -40,11 +40,7 @@ def test_prefill_32k_properties(pkg, orc, dev, recipe):
         v = torch.randn(B, L, H, D, device=dev, generator=gen).bfloat16()
         lse_swa = torch.randn(B, L, HQ, device=dev, generator=gen) * 2 + 6
     else:
-        hs = torch.rand(HQ, device=dev, generator=gen) * 1.5 + 0.5
-        q = bench.gpu_randn((B, L, HQ, D), gen, dev, hs.view(1, 1, HQ, 1))
-        k = bench.gpu_randn((B, L, H, D), gen, dev, hs[::G].view(1, 1, H, 1))
-        v = bench.gpu_randn((B, L, H, D), gen, dev)
-        lse_swa = bench.swa_lse_current_chunk(q, k, S).bfloat16()
+        q, k, v, lse_swa = util.prefill_inputs(dev)
     lmk = pkg.chunk_mean_pool(k, S)
     # mean pool: closed form on every chunk
     ref_lmk = k.view(B, N, S, H, D).float().mean(2)
@@ -166,7 +162,7 @@ def test_prefill_config2_properties(pkg, orc, dev):
     note("full size: prefill B4 L8192 h16/16 D64 top32 (config 2)")
     B, L, HQ, H, D, S, K, W = 4, 8192, 16, 16, 64, 64, 32, 1
     G, N = 1, L // S
-    q, k, v, lse_swa = bench.config2_inputs(dev)
+    q, k, v, lse_swa = util.config2_inputs(dev)
     lmk = pkg.chunk_mean_pool(k, S)
     assert (lmk.float() - k.view(B, N, S, H, D).float().mean(2)).abs().max().item() <= 8e-3
     dbg = {}
@@ -220,8 +216,8 @@ def test_train_config5_forward_backward(pkg, orc, dev):
     note("full size: train layer fwd+bwd B8 L8192 h16/16 D64 top32 (config 5)")
     B, L, HQ, H, D, S, K, W = 8, 8192, 16, 16, 64, 64, 32, 1
     N = L // S
-    q, k, v, d_o, lse_swa = bench.train_inputs(dev)
-    o, idx, scores, w = bench.train_forward(pkg, q, k, v, lse_swa, keep=True)
+    q, k, v, d_o, lse_swa = util.train_inputs(dev)
+    o, idx, scores, w = util.train_forward(pkg, q, k, v, lse_swa, keep=True)
     o.backward(d_o)
     torch.cuda.synchronize()
     lim = torch.div(torch.arange(L, device=dev) - W + 1, S, rounding_mode="floor")

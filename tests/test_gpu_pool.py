@@ -25,7 +25,7 @@ def test_attn_pool_fwd(pkg, orc, dev, B, N, H, D, S):
     rk, rb, _ = orc.chunk_attn_pool(mu, k)
     assert lk.dtype == torch.bfloat16 and lb.dtype == torch.float32
     assert_close_bf16(lk, rk, "lmk_k")
-    assert_close_f32(lb, rb, 1e-3, "lmk_b")
+    assert_close_f32(lb, rb, 1e-4, "lmk_b")
 
 
 def test_attn_pool_default_scale_and_explicit(pkg, orc, dev):
@@ -38,7 +38,7 @@ def test_attn_pool_default_scale_and_explicit(pkg, orc, dev):
     c = pkg.chunk_attn_pool_tilelang(mu.to(dev), k.to(dev), sm_scale=0.3)
     rk, rb, _ = orc.chunk_attn_pool(mu, k, 0.3)
     assert_close_bf16(c[0], rk, "lmk_k scale 0.3")
-    assert_close_f32(c[1], rb, 1e-3, "lmk_b scale 0.3")
+    assert_close_f32(c[1], rb, 1e-4, "lmk_b scale 0.3")
 
 
 def test_attn_pool_last_token_masked(pkg, dev):
@@ -59,7 +59,7 @@ def test_attn_pool_compact(pkg, orc, dev):
     k = torch.randn(1, 8, 64, 2, 64).bfloat16()
     lk, lb = pkg.chunk_attn_pool_tilelang(mu.to(dev), k.to(dev), compact_lmk_k=True)
     assert torch.count_nonzero(lk).item() == 0
-    assert_close_f32(lb, orc.chunk_attn_pool(mu, k)[1], 1e-3, "lmk_b compact")
+    assert_close_f32(lb, orc.chunk_attn_pool(mu, k)[1], 1e-4, "lmk_b compact")
 
 
 def _pool_grads(orc, mu, k, gk, gb, scale=None):
@@ -124,7 +124,7 @@ def test_attn_pool_shared_k(pkg, orc, dev):
     lk, lb = pkg.chunk_attn_pool_tilelang_shared_k(mu_d, k_d)
     rk_, rb_, _ = orc.chunk_attn_pool(mu, k)
     assert_close_bf16(lk, rk_, "shared lmk_k")
-    assert_close_f32(lb, rb_, 1e-3, "shared lmk_b")
+    assert_close_f32(lb, rb_, 1e-4, "shared lmk_b")
     torch.autograd.backward([lk, lb], [gk.to(dev), gb.to(dev)])
     rmu, rk = _pool_grads(orc, mu, k, gk, gb)
     assert_close_bf16(mu_d.grad, rmu, "shared d_mu")

@@ -179,7 +179,7 @@ def test_sparse_attn_per_chunk_lse(pkg, orc, dev):
     o = torch.empty(B, L, HQ, 64, dtype=torch.bfloat16, device=dev)
     lse = torch.empty(B, L, HQ, 4, dtype=torch.float32, device=dev)
     t = [x.to(dev) for x in (q, k, v, w, idx)]
-    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, None, _cabi.ptr(o), _cabi.ptr(lse), None, 0,
+    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, None, _cabi.ptr(o), _cabi.ptr(lse), None, 0, 0,
                B, L, L, HQ, 2, D, 64, 4, w.shape[-1], HQ, 1, 64, 1 / math.sqrt(D), 1, 0.0, 0)
     _, lse_ref = orc.sparse_attn(q, k, v, w, idx, chunk_size=64, return_lse=True)
     assert_close_f32(lse.cpu() / 1.4426950408889634, lse_ref, LSE_TOL, "per-chunk LSE")
@@ -248,7 +248,7 @@ def test_sparse_attn_mfma_path_matches_generic_path(pkg, orc, dev, B, L, HQ, H, 
         o = torch.empty(B, L, HQ, Dv, dtype=torch.bfloat16, device=dev)
         lse = torch.empty(B, L, HQ, K, dtype=torch.float32, device=dev)
         _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, None, _cabi.ptr(o), _cabi.ptr(lse),
-                   _cabi.ptr(ws) if use_ws else None, 0,
+                   _cabi.ptr(ws) if use_ws else None, _cabi.nbytes(ws), 0,
                    B, L, L, HQ, H, D, Dv, K, w.shape[-1], HQ, 1, 64, 1 / math.sqrt(D), 1, 0.0, 0)
         torch.cuda.synchronize()
         outs.append((o.cpu(), lse.cpu()))
@@ -275,7 +275,7 @@ def test_sparse_attn_bwd_mfma_path_matches_generic_path(pkg, dev, B, L, HQ, H, D
     o = torch.empty(B, L, HQ, Dv, dtype=torch.bfloat16, device=dev)
     lse = torch.empty(B, L, HQ, K, dtype=torch.float32, device=dev)
     scale = 1 / math.sqrt(D)
-    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, None, _cabi.ptr(o), _cabi.ptr(lse), None, 0,
+    _cabi.call("hils_sparse_attn_fwd", *[_cabi.ptr(x) for x in t], None, None, _cabi.ptr(o), _cabi.ptr(lse), None, 0, 0,
                B, L, L, HQ, H, D, Dv, K, NW, HQ, 1, 64, scale, mask_last, 0.0, 0)
     ws = _cabi.sparse_attn_bwd_workspace(dev, B, L, L, HQ, H, D, Dv, K, HQ, 1, 64, 0.0)
     assert ws is not None, "this shape must be covered by the MFMA backward"
@@ -289,7 +289,7 @@ def test_sparse_attn_bwd_mfma_path_matches_generic_path(pkg, dev, B, L, HQ, H, D
             dv = torch.zeros(t[2].shape, dtype=torch.float32, device=dev)
         dw = torch.zeros(B, L, HQ, NW, dtype=torch.float32, device=dev)
         _cabi.call("hils_sparse_attn_bwd", *[_cabi.ptr(x) for x in t], None, _cabi.ptr(lse), _cabi.ptr(do.to(dev)),
-                   _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), _cabi.ptr(ws) if use_ws else None,
+                   _cabi.ptr(dq), _cabi.ptr(dk), _cabi.ptr(dv), _cabi.ptr(dw), _cabi.ptr(ws) if use_ws else None, _cabi.nbytes(ws),
                    B, L, L, HQ, H, D, Dv, K, NW, HQ, 1, 64, scale, mask_last, 0.0, None, None, 0, kv16)
         torch.cuda.synchronize()
         res.append([x.float().cpu() for x in (dq, dk, dv, dw)])

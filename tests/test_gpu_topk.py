@@ -170,7 +170,7 @@ def test_topk_inference_variant_matches_export_variant(pkg, dev, G, D, L, N, top
             idx = torch.empty(1, L, h_kv, topk, dtype=torch.int32, device=dev)
             sc = torch.empty(1, L, h_kv, G, topk, dtype=torch.bfloat16, device=dev)
             _cabi.call("hils_topk_fwd", _cabi.ptr(q), _cabi.ptr(lmks), _cabi.ptr(lse.view(1, L, h_kv, G).contiguous()),
-                       None, None, None, _cabi.ptr(idx), _cabi.ptr(sc), None, None, None, 1, L, N, h_kv, G, D,
+                       None, None, None, _cabi.ptr(idx), _cabi.ptr(sc), None, None, None, 0, 1, L, N, h_kv, G, D,
                        topk, S, W, 1, off, 0, D ** -0.5)
         else:
             idx, sc = pkg.online_softmax_topk_head(q, lmks, lse, topk, S, W, q_offset=off,
@@ -300,7 +300,7 @@ def test_topk_split_and_fused_paths_agree(pkg, dev):
         idx = torch.empty(B, L, h_kv, topk, dtype=torch.int32, device=dev)
         sc = torch.empty(B, L, h_kv, G, topk, dtype=torch.bfloat16, device=dev)
         _cabi.call("hils_topk_fwd", _cabi.ptr(q), _cabi.ptr(lmks), _cabi.ptr(lse), None, None, None,
-                   _cabi.ptr(idx), _cabi.ptr(sc), None, None, _cabi.ptr(w), B, L, N, h_kv, G, D, topk, 64, 1, 1,
+                   _cabi.ptr(idx), _cabi.ptr(sc), None, None, _cabi.ptr(w), _cabi.nbytes(w), B, L, N, h_kv, G, D, topk, 64, 1, 1,
                    N * 64, 0, D ** -0.5)
         torch.cuda.synchronize()
         outs.append((idx.cpu(), sc.float().cpu()))
@@ -371,3 +371,35 @@ def test_topk_one_pass_kernel_all_scores_equal(pkg, orc, dev):
     want = torch.where(want < lim.view(1, L, 1, 1), want, torch.full_like(want, -1)).to(torch.int32)
     assert torch.equal(idx.cpu(), want), "with all scores equal the lowest chunk indices must win"
     assert torch.equal(idx.cpu(), orc.topk_select(dbg["sel_logits"].cpu(), dbg["lse_total"].cpu(), lim, topk))
+
+
+def test_topk_one_pass_kernel_rows_without_any_mass(pkg, orc, dev):
+    """Rows whose lse_swa is -inf (the local branch saw no key: a landmark row with window 1) through
+    the one-pass prefill kernel, both launch variants.  In the first chunk such a row sees no chunk
+    either: lse_total is -inf, nothing is selected (indices -1, scores -inf) and no NaN is formed;
+    later rows select from the chunk logits alone."""
+    note("one-pass top-k: rows with lse_swa = -inf")
+    B, L, N, h_kv, G, D, topk, S, W = 1, 4096, 64, 2, 4, 128, 8, 64, 1
+    gen = torch.Generator().manual_seed(63)
+    q = torch.randn(B, L, h_kv * G, D, generator=gen).bfloat16()
+    lmks = torch.randn(B, N, h_kv, D, generator=gen).bfloat16()
+    lse = torch.randn(B, L, h_kv * G, generator=gen) * 3 + 5
+    lse[:, S - 1::S] = float("-inf")   # every landmark row
+    lse[:, :S:7] = float("-inf")       # and some more rows of the first chunk
+    lim = orc.causal_chunk_limit(L, 0, W, S)
+    outs = []
+    for dbg in ({}, None):
+        idx, scores = pkg.online_softmax_topk_head(q.to(dev), lmks.to(dev), lse.to(dev), topk, S, W,
+                                                   is_training=False, _debug=dbg)
+        torch.cuda.synchronize()
+        outs.append((idx.cpu(), scores.float().cpu()))
+        assert torch.all(idx[:, :S] == -1), "rows that see no chunk must select nothing"
+        assert torch.all(scores[:, :S].float() == float("-inf"))
+        assert not torch.isnan(scores.float()).any()
+        if dbg is not None:
+            lt = dbg["lse_total"].cpu()
+            assert torch.all(lt.view(B, L, -1)[:, :S][lse[:, :S] == float("-inf")] == float("-inf"))
+            want = orc.topk_select(dbg["sel_logits"].cpu(), lt, lim, topk)
+            assert torch.equal(idx.cpu(), want), "indices not bit-exact"
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    assert torch.equal((outs[0][0] >= 0).sum(-1), lim.clamp(0, topk).view(1, L, 1).expand(B, L, h_kv))

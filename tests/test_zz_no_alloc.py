@@ -15,7 +15,7 @@ def _call(_cabi, name, q, lmk, lse, bias, idx, sc, ws, B, L, N, h_kv, G, D, K, o
     args = [_cabi.ptr(q), _cabi.ptr(lmk), _cabi.ptr(lse), _cabi.ptr(bias), None, None, _cabi.ptr(idx),
             _cabi.ptr(sc), None, None]
     if name == "hils_topk_fwd":
-        args.append(_cabi.ptr(ws))
+        args += [_cabi.ptr(ws), _cabi.nbytes(ws)]
     _cabi.call(name, *args, B, L, N, h_kv, G, D, K, 64, 1, 1, off, 0, 1.0 / math.sqrt(D))
 
 
