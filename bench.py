@@ -166,7 +166,10 @@ def bench_decode(pkg, dev, steps, warmup):
     q = gpu_randn((B, 1, HQ, D), gen, dev)
     kc = gpu_randn((B, Lkv, H, D), gen, dev)
     vc = gpu_randn((B, Lkv, H, D), gen, dev)
+    from hils_attention_amd.ops.hils_glue import head_major_chunk_keys
     lmk = pkg.chunk_mean_pool(kc, S)  # precomputed pooled keys (untimed)
+    # the cache layers keep the pooled keys head-major, (B, H, chunks, D): a row's keys are contiguous
+    lmk_hm = head_major_chunk_keys(lmk)
     # fp32, as the sliding-window attention kernel hands its log-sum-exp over
     lse_swa = torch.randn(B, 1, HQ, device=dev, generator=gen) * 5 + 10
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
@@ -174,6 +177,9 @@ def bench_decode(pkg, dev, steps, warmup):
 
     def step():
         # the remote branch of the step in one launch: a row's workgroup selects, then attends
+        pkg.decode_step(q, lmk_hm, kc, vc, lse_swa, K, S, W, q_offset=Lkv - 1, lmk_head_major=True)
+
+    def step_token_major():  # the chunk keys in the reference's layout (B, chunks, H, D)
         pkg.decode_step(q, lmk, kc, vc, lse_swa, K, S, W, q_offset=Lkv - 1)
 
     def step2(record=False):
@@ -196,11 +202,18 @@ def bench_decode(pkg, dev, steps, warmup):
     # of microseconds together, are spread over at least 200 steps so that the figure is the steady state
     steps = max(steps, 200)
     eager_sec = time_steps(step, steps, warmup)
+    token_major_sec = time_steps(step_token_major, steps, warmup)
+    # the layer's default mode: a prior bias per (chunk, query head) in the selection and the softmax
+    prior_hm = torch.randn(B, H, N, HQ // H, device=dev, generator=gen)
+    prior_sec = time_steps(lambda: pkg.decode_step(q, lmk_hm, kc, vc, lse_swa, K, S, W, q_offset=Lkv - 1,
+                                                   prior_b=prior_hm, lmk_head_major=True), steps, warmup)
     two_call_sec = time_steps(step2, steps, warmup)
     for _ in range(min(steps, 5)):
         step2(record=True)
     per = {kk: vv / acc["n"] for kk, vv in acc.items() if kk != "n"}  # the two calls, each timed alone
     per["two_call_step"] = two_call_sec * 1e3
+    per["token_major_keys_step"] = token_major_sec * 1e3
+    per["prior_bias_step"] = prior_sec * 1e3
     # the serving loop replays the step as one HIP graph (no host work between kernels)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -225,9 +238,12 @@ def bench_decode(pkg, dev, steps, warmup):
     lmk_pages = torch.empty((n_pages, H, D), dtype=lmk.dtype, device=dev)
     lmk_pages[perm] = lmk.reshape(n_pages, H, D)
     table = perm.view(B, N).to(torch.int32).contiguous()
-    paged_sec = time_steps(lambda: pkg.paged_hils_attend(q, k_pages, v_pages, lmk_pages, table, lse_swa, Lkv, K, W),
-                           steps, warmup)
-    per["paged_step"] = paged_sec * 1e3
+    paged_sec = time_steps(lambda: pkg.paged_hils_attend(q, k_pages, v_pages, None, table, lse_swa, Lkv, K, W,
+                                                         lmk_dense=lmk_hm), steps, warmup)
+    per["paged_step"] = paged_sec * 1e3  # K, V in pages; the pooled keys per sequence, head-major
+    paged_lmk_sec = time_steps(lambda: pkg.paged_hils_attend(q, k_pages, v_pages, lmk_pages, table, lse_swa, Lkv, K, W),
+                               steps, warmup)
+    per["paged_keys_per_page_step"] = paged_lmk_sec * 1e3
     del k_pages, v_pages
     lmk_bytes = B * N * H * D * 2
     kv_bytes = B * H * K * S * D * 2 * 2

@@ -47,14 +47,22 @@ static inline size_t dr_smem_bytes(int D, int G, int nwave) {
          + (size_t)nwave * DR_MAXSLOT * DR_NH * sizeof(bf16_t);       // slot weights
 }
 
+struct DrNoHook {
+  __device__ __forceinline__ void operator()() const {}
+};
+
 // One (query, KV head) row by a workgroup of NWAVE wavefronts: `split` of dm.nsplit shares of the
 // slots, KV head hk, query bt = b * L + t; dr_smem = dr_smem_bytes(D, G, NWAVE) bytes of LDS.
-template <int D, int NWAVE>
+// weights and indices may point into LDS (the one-launch decode step hands the row's selection over
+// there: generic loads reach either memory).  `hook` runs once in every wavefront after its first
+// chunk's loads have been issued and before it writes the staging areas of dr_smem (that kernel puts
+// the barrier there that ends the selection's use of the same LDS).
+template <int D, int NWAVE, class Hook = DrNoHook>
 __device__ __forceinline__ void decode_rows_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                  const bf16_t* __restrict__ v, const bf16_t* __restrict__ weights,
                                                  const int32_t* __restrict__ indices, bf16_t* __restrict__ o,
                                                  float* __restrict__ partial, const DrDims& dm, char* dr_smem,
-                                                 int split, int hk, long bt) {
+                                                 int split, int hk, long bt, Hook hook = Hook{}) {
   constexpr int LR = D / 8;          // lanes per token row
   constexpr int TPI = 64 / LR;       // token rows per load instruction
   constexpr int GL = DR_QT / TPI;    // load instructions per group
@@ -250,12 +258,15 @@ __device__ __forceinline__ void decode_rows_body(const bf16_t* __restrict__ q, c
     long coff = chunk_off(0);
 #pragma unroll
     for (int s = 0; s < NR; ++s) issue(R[s], coff, s);
+    hook();
     for (int si = 0; si + 1 < nsl; ++si) {
       const long noff = chunk_off(si + 1);
       chunk(si, coff, noff, std::true_type{});
       coff = noff;
     }
     chunk(nsl - 1, coff, 0, std::false_type{});
+  } else {
+    hook();
   }
 
   // accumulator register i of tile mt in lane (head = col, j) is feature mt*16 + 4j + i

@@ -1274,6 +1274,9 @@ struct TopkRowShared {
   uint32_t gmax[64];           // largest selection key of every 16-lane group of the workgroup
   int wcnt[TOPK_R_WAVES];      // keys of a wavefront that reach the candidate bound
   float tot[4];                // lse_total per head
+  int rank[64];                            // one-launch decode step: candidates ahead of each candidate
+  int win_i[TOPK_MAXK];                    // ... the winners' chunks, ascending, -1 padded
+  bf16_t win_w[4 * (TOPK_MAXK + 1) + 2];   // ... and the heads' inter-chunk weights, [head][topk + 1]
   uint32_t thr;                // the candidate bound
   int next_group;
 };
@@ -1281,15 +1284,19 @@ struct TopkRowShared {
 
 // One (query, KV head) row (row = (b*L + t)*h_kv + hk) by a workgroup of NW wavefronts; dyn = the
 // workgroup's dynamic LDS (topk_row_smem bytes).
-template <int D, int GMAX, int NW, bool PAGED, int GI = 8>  // GI: load instructions per register buffer
+// FUSED (the one-launch decode step): the row's attention follows in the same workgroup.  Every
+// wavefront then works out the winners itself and leaves the row's indices and inter-chunk weights in
+// LDS (sh.win_i, sh.win_w: the same values from every wavefront), where the attention reads them
+// without waiting for anybody; wavefront 0 writes the selection's global outputs on the way.
+template <int D, int GMAX, int NW, bool PAGED, bool FUSED = false, int GI = 8>  // GI: load instructions per register buffer
 __device__ __forceinline__ void
 topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
-              const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
+              const float* __restrict__ lse_swa, const float* __restrict__ bias, int32_t* __restrict__ indices,
               bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
               float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
               int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
               float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages,
-              float* dyn, const long row) {
+              int lmk_hm, int lmk_cap, float* dyn, const long row, TopkRowShared* sh_p = nullptr) {
   constexpr int LR = D / 8, TPI = 64 / LR;
   constexpr int THREADS = NW * 64;       // NW = 8 or 16 wavefronts
   constexpr int EPT = TOPK_R_MAXN / THREADS;  // 64-chunk slots of a wavefront's share
@@ -1299,8 +1306,14 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   float* pooled = dyn + (size_t)GMAX * NP;    // [NP]
   // paged chunk keys, lmks = (num_pages, h_kv, D): the row's page ids are staged behind the pooled scores
   int* page_s = (int*)(pooled + NP);          // [NP], only with a page table (else 0 entries)
-  const int NPG = PAGED ? NP : 0;             // the wavefronts' staging areas follow
-  __shared__ TopkRowShared sh;
+  const int NPG = PAGED ? NP : 0;
+  // the row's additive bias (the layer's prior bias: added to the logits for the log-sum-exp and the
+  // selection, and, rounded the layer's way, to the winners' scores before the inter-chunk softmax),
+  // staged head-major like the logits; 0 for the chunks past the causal limit
+  float* bias_s = (float*)(page_s + NPG);     // [GMAX][NP], only with a bias
+  const int NBS = bias ? GMAX * NP : 0;       // the wavefronts' staging areas follow
+  __shared__ TopkRowShared sh_own;
+  TopkRowShared& sh = FUSED ? *sh_p : sh_own;  // FUSED: the caller's, which the attention reads after the return
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int piece = lane % LR, tsub = lane / LR;
   const int hk = (int)(row % h_kv);
@@ -1313,6 +1326,30 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
 #pragma unroll
   for (int g = 0; g < GMAX; ++g) swa[g] = (g < G) ? lse_swa[row * G + g] : 0.f;
   if (tid == 0) sh.next_group = 2 * NW;
+  if (bias) {
+    // chunk c of this row: the G biases are contiguous in all three layouts
+    for (int c = tid; c < NP; c += THREADS) {
+      float bv[GMAX];
+#pragma unroll
+      for (int g = 0; g < GMAX; ++g) bv[g] = 0.f;
+      if (c < lim) {
+        long e0;
+        if (PAGED) {
+          const int pg = c < max_pages ? page_table[b * max_pages + c] : -1;
+          e0 = ((long)((pg >= 0 && pg < num_pages) ? pg : 0) * h_kv + hk) * G;
+        } else if (lmk_hm) {
+          e0 = ((b * h_kv + hk) * (long)lmk_cap + c) * G;
+        } else {
+          e0 = ((b * N + c) * (long)h_kv + hk) * G;
+        }
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g)
+          if (g < G) bv[g] = bias[e0 + g];
+      }
+#pragma unroll
+      for (int g = 0; g < GMAX; ++g) bias_s[g * NP + c] = bv[g];
+    }
+  }
   // the query heads as B operand of the logit products, lane (head = lane & 15, j = lane >> 4) holds
   // features ks*32 + 8j ..; loaded here so that the barrier below has waited for them
   typedef unsigned tr_u4 __attribute__((ext_vector_type(4)));
@@ -1344,13 +1381,14 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     constexpr int KS = D / 32;
     constexpr int ROWB = 2 * D + 16;
     constexpr int LPT = 16 / TPI;  // load instructions per 16-key tile
-    char* stage_w = (char*)(page_s + NPG) + (size_t)wave * 16 * ROWB;
+    char* stage_w = (char*)(bias_s + NBS) + (size_t)wave * 16 * ROWB;
     const int col = lane & 15, j = lane >> 4;
     char* const w_addr = stage_w + tsub * ROWB + piece * 16;
     const char* const k_addr = stage_w + col * ROWB + j * 16;
     const int ngroups = (lim + KG - 1) / KG;
-    const bf16_t* base = lmks + (b * N * (long)h_kv + hk) * D + piece * 8;
-    const long cstride = (long)h_kv * D;
+    // dense chunk keys: (B, N, h_kv, D), or head-major (B, h_kv, lmk_cap, D) (a row's keys contiguous)
+    const bf16_t* base = lmks + (lmk_hm ? (b * h_kv + hk) * (long)lmk_cap * D : (b * N * (long)h_kv + hk) * D) + piece * 8;
+    const long cstride = (PAGED || !lmk_hm) ? (long)h_kv * D : (long)D;
     const bf16_t* pbase = lmks + (long)hk * D + piece * 8;  // paged: + page * h_kv * D
     auto fetch = [&](tr_u4 (&kr)[GI], int grp) __attribute__((always_inline)) {
 #pragma unroll
@@ -1381,10 +1419,10 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
         }
         // accumulator register i of lane (head = col, j) is key c0 + 4j + i
         const int c0 = grp * KG + tt * 16 + 4 * j;
-        if (col < G) {
+        if (col < GMAX) {  // (the rows of the heads past G hold -inf)
           f32x4_t out;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) out[i] = (c0 + i < lim) ? __fmul_rn(acc[i], sm_scale) : HILS_NEG_INF;
+          for (int i = 0; i < 4; ++i) out[i] = (c0 + i < lim && col < G) ? __fmul_rn(acc[i], sm_scale) : HILS_NEG_INF;
           if (PAGED) {  // c0 + 3 < NP: groups end at a multiple of 64 at most
             typedef int tr_i4 __attribute__((ext_vector_type(4)));
             const tr_i4 pg4 = *(const tr_i4*)&page_s[c0];
@@ -1393,6 +1431,11 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
               if (pg4[i] < 0) out[i] = HILS_NEG_INF;
           }
           *(f32x4_t*)&logit_s[col * NP + c0] = out;
+          if (bias) {  // -inf stays -inf: the staged bias is finite (0 past the causal limit)
+            const f32x4_t bb = *(const f32x4_t*)&bias_s[col * NP + c0];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[i] = __fadd_rn(out[i], bb[i]);
+          }
           // running log-sum-exp of this lane's head over the keys it has seen
           const float mn = fmaxf(fmaxf(m_run, fmaxf(out[0], out[1])), fmaxf(out[2], out[3]));
           const float ms = (mn == HILS_NEG_INF) ? 0.f : mn * HILS_LOG2E;
@@ -1478,24 +1521,36 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   const int cbase = wave * per;
   uint32_t key[EPT];
   uint32_t lmax = 0u;
+  // (the options are decided outside the unrolled loops: a run-time flag tested per element is a branch
+  // per element; the logit rows of the heads past G hold -inf, so every head is read alike)
+  auto form_keys = [&](auto with_bias) __attribute__((always_inline)) {
 #pragma unroll
-  for (int e = 0; e < EPT; ++e) {
-    key[e] = 0u;
-    if (e * 64 < per) {  // uniform: the slots past the wavefront's share cost nothing
-      const int c = cbase + e * 64 + lane;
-      const bool mine = c < lim;
-      float best = HILS_NEG_INF;
+    for (int e = 0; e < EPT; ++e) {
+      key[e] = 0u;
+      if (e * 64 < per) {  // uniform: the slots past the wavefront's share cost nothing
+        const int c = cbase + e * 64 + lane;
+        const bool mine = c < lim;
+        float best = HILS_NEG_INF;
 #pragma unroll
-      for (int g = 0; g < GMAX; ++g)
-        if (g < G) {
-          const float xv = mine ? logit_s[g * NP + c] : HILS_NEG_INF;
+        for (int g = 0; g < GMAX; ++g) {
+          float xv = mine ? logit_s[g * NP + c] : HILS_NEG_INF;
+          if (decltype(with_bias)::value) xv = mine ? __fadd_rn(xv, bias_s[g * NP + c]) : xv;  // the sum the log-sum-exp saw
           const float nrm = (xv == HILS_NEG_INF) ? HILS_NEG_INF : __fsub_rn(xv, tot[g]);
           best = fmaxf(best, nrm);
-          if (sel_logits_out && c < N) sel_logits_out[(row * G + g) * (long)N + c] = xv;
         }
-      if (mine) pooled[c] = best;
-      key[e] = score_key(best);
-      lmax = key[e] > lmax ? key[e] : lmax;
+        if (mine) pooled[c] = best;
+        key[e] = score_key(best);
+        lmax = key[e] > lmax ? key[e] : lmax;
+      }
+    }
+  };
+  if (bias) form_keys(std::true_type{}); else form_keys(std::false_type{});
+  if (sel_logits_out) {  // the exported selection logits (a debugging output)
+    for (int i = tid; i < G * N; i += THREADS) {
+      const int g = i / N, c = i - g * N;
+      float xv = c < lim ? logit_s[g * NP + c] : HILS_NEG_INF;
+      if (bias && c < lim) xv = __fadd_rn(xv, bias_s[g * NP + c]);
+      sel_logits_out[(row * G + g) * (long)N + c] = xv;
     }
   }
   // A lower bound of the topk-th largest key with few keys above it: the topk-th largest of the
@@ -1507,9 +1562,16 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gm, 0xB1, 0xF, 0xF, true);  gm = gm > y ? gm : y;
     y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gm, 0x4E, 0xF, 0xF, true);  gm = gm > y ? gm : y;
     y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gm, 0x141, 0xF, 0xF, true); gm = gm > y ? gm : y;
-    y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gm, 0x140, 0xF, 0xF, true); gm = gm > y ? gm : y;
-    if ((lane & 15) == 0) sh.gmax[wave * 4 + (lane >> 4)] = gm;
-    if (NW * 4 < 64 && tid >= NW * 4 && tid < 64) sh.gmax[tid] = 0u;
+    // 64 groups in all: 16-lane groups with 16 wavefronts, 8-lane groups with 8 (the bound is the
+    // topk-th largest of the 64 group maxima: with fewer, coarser groups it lets too many keys through)
+    if constexpr (NW >= 16) {
+      y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)gm, 0x140, 0xF, 0xF, true); gm = gm > y ? gm : y;
+      if ((lane & 15) == 0) sh.gmax[wave * 4 + (lane >> 4)] = gm;
+      if (NW * 4 < 64 && tid >= NW * 4 && tid < 64) sh.gmax[tid] = 0u;
+    } else {
+      static_assert(NW == 8 || NW >= 16, "group maxima: 8 or 16 wavefronts");
+      if ((lane & 7) == 0) sh.gmax[wave * 8 + (lane >> 3)] = gm;
+    }
   }
   __syncthreads();
   if (wave == 0) {
@@ -1531,6 +1593,7 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     for (int e = 0; e < EPT; ++e)
       if (e * 64 < per) cnt += __popcll(__ballot(key[e] >= thr));
     if (lane == 0) sh.wcnt[wave] = cnt;
+    if (FUSED && wave == 0) sh.rank[lane] = 0;
   }
   __syncthreads();
   int cand_base = 0, cand_total = 0;
@@ -1540,6 +1603,53 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     cand_total += v;
     cand_base += (w2 < wave) ? v : 0;
   }
+  // ---- FUSED: what every wavefront does once lane kk (kk < nc) holds winner kk's chunk (ascending) ----
+  auto fused_tail = [&](int widx, int nc) __attribute__((always_inline)) {
+    const bool has = lane < nc;
+    float xs[GMAX], wgt[GMAX], wloc[GMAX];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+      xs[g] = (has && g < G) ? logit_s[g * NP + widx] : HILS_NEG_INF;  // raw scaled score
+      // the layer's inter-chunk softmax over [scores as bf16 (+ bias as bf16, summed in bf16), lse_swa]
+      float x = HILS_NEG_INF;
+      if (has && g < G) {
+        x = bf2f(f2bf(xs[g]));
+        if (bias) x = bf2f(f2bf(x + bf2f(f2bf(bias_s[g * NP + widx]))));
+      }
+      const float m = fmaxf(wave_max_f(x), swa[g]);
+      if (m == HILS_NEG_INF) {  // every logit -inf: NaN row, as a softmax gives
+        wgt[g] = wloc[g] = __uint_as_float(0x7fc00000u);
+      } else {
+        const float e = (x == HILS_NEG_INF) ? 0.f : __expf(x - m);
+        const float el = __expf(swa[g] - m);
+        const float inv = 1.f / (wave_sum_f(e) + el);
+        wgt[g] = e * inv;
+        wloc[g] = el * inv;
+      }
+    }
+    if (wave == 0) {  // the selection's outputs
+      if (lane < topk) indices[row * topk + lane] = has ? widx : -1;
+#pragma unroll
+      for (int g = 0; g < GMAX; ++g)
+        if (g < G) {
+          if (lane < topk) scores[(row * G + g) * (long)topk + lane] = f2bf(xs[g]);
+          if (weights_out) {
+            bf16_t* wrow = weights_out + (row * G + g) * (long)(topk + 1);
+            if (lane < topk) wrow[lane] = f2bf(wgt[g]);
+            if (lane == 0) wrow[topk] = f2bf(wloc[g]);
+          }
+        }
+    }
+    // the row's indices and weights for the attention, in the layout of the global tensors
+    if (lane < topk) sh.win_i[lane] = has ? widx : -1;
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g)
+      if (g < G) {
+        if (lane < topk) sh.win_w[g * (topk + 1) + lane] = f2bf(wgt[g]);
+        if (lane == 0) sh.win_w[g * (topk + 1) + topk] = f2bf(wloc[g]);
+      }
+    __builtin_amdgcn_wave_barrier();
+  };
   if (cand_total <= TOPK_R_CAND) {
     uint32_t* ck = (uint32_t*)sh.merge_s;  // NW * TOPK_MAXK >= 512 entries
     int pos = cand_base;
@@ -1557,6 +1667,37 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       }
     }
     __syncthreads();
+    if constexpr (FUSED) {
+      if (cand_total <= 64) {
+        // One candidate per lane, in chunk order: its rank among the candidates (keys descending, ties
+        // to the lower chunk) says whether it wins, the winners before it give its slot.  Every
+        // wavefront does this for itself: no hand-over, no barrier before the attention's first loads.
+        // The 64 x 64 comparisons are shared out: wavefront w compares every candidate with candidates
+        // w * 64 / NW ..., the partial ranks meet in LDS.
+        const uint32_t kc = lane < cand_total ? ck[lane] : 0u;  // (valid keys are >= 1)
+        const int ci = lane < cand_total ? sh.merge_i[lane] : -1;
+        {
+          constexpr int JW = 64 / NW;
+          int part = 0;
+#pragma unroll
+          for (int u = 0; u < JW; ++u) {
+            const int jj = wave * JW + u;
+            const uint32_t kj = (uint32_t)__builtin_amdgcn_readlane((int)kc, jj);
+            part += ((kj > kc) | ((kj == kc) & (jj < lane))) ? 1 : 0;
+          }
+          if (part) atomicAdd(&sh.rank[lane], part);
+        }
+        lds_barrier();
+        const int rank = sh.rank[lane];
+        const bool win = lane < cand_total && rank < topk;
+        const unsigned long long wm = __ballot(win);
+        if (win) sh.cand_i[wave][__popcll(wm & lt)] = ci;
+        __builtin_amdgcn_wave_barrier();
+        const int nc = __popcll(wm);
+        fused_tail(lane < nc ? sh.cand_i[wave][lane] : -1, nc);
+        return;
+      }
+    }
     if (wave == 0) {
       // (the usual case, about 1.4 topk candidates, is one key per lane)
       const int nc = cand_total <= 64
@@ -1593,6 +1734,11 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     }
   }
   __syncthreads();
+  if constexpr (FUSED) {  // the selections that did not fit one lane per candidate: winners from LDS
+    const int nc = sh.ncand[0];
+    fused_tail(lane < nc ? sh.cand_i[0][lane] : -1, nc);
+    return;
+  }
   // ---- phase 4: indices (ascending) and the raw scaled scores of the winners ----
   const int nc = sh.ncand[0];
   for (int kk = tid; kk < topk; kk += THREADS) indices[row * topk + kk] = (kk < nc) ? sh.cand_i[0][kk] : -1;
@@ -1608,7 +1754,11 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
 #pragma unroll
     for (int g2 = 1; g2 < GMAX; ++g2) lse_g = (g == g2) ? swa[g2] : lse_g;
     float x = HILS_NEG_INF;
-    if (lane < topk && lane < nc) x = bf2f(f2bf(logit_s[g * NP + sh.cand_i[0][lane]]));
+    if (lane < topk && lane < nc) {
+      x = bf2f(f2bf(logit_s[g * NP + sh.cand_i[0][lane]]));
+      // the layer adds the gathered bias, cast to the scores' dtype, to the bf16 scores
+      if (bias) x = bf2f(f2bf(x + bf2f(f2bf(bias_s[g * NP + sh.cand_i[0][lane]]))));
+    }
     const float m = fmaxf(wave_max_f(x), lse_g);
     bf16_t* wrow = weights_out + (row * G + g) * (long)(topk + 1);
     if (m == HILS_NEG_INF) {  // every logit -inf: NaN row, as a softmax gives
@@ -1626,15 +1776,17 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
 template <int D, int GMAX, int NW, bool PAGED>
 __global__ void __launch_bounds__(NW * 64)
 topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
-                const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
+                const float* __restrict__ lse_swa, const float* __restrict__ bias, int32_t* __restrict__ indices,
                 bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
                 float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
                 int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
-                float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages) {
+                float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages,
+                int lmk_hm, int lmk_cap) {
   extern __shared__ __align__(16) float topk_row_dyn[];
-  topk_row_body<D, GMAX, NW, PAGED>(q, lmks, lse_swa, indices, scores, lse_total_out, sel_logits_out, weights_out, L,
-                                    N, NP, h_kv, G, topk, block_size, window_size, causal, q_offset, sm_scale,
-                                    page_table, max_pages, num_pages, topk_row_dyn, (long)blockIdx.x);
+  topk_row_body<D, GMAX, NW, PAGED>(q, lmks, lse_swa, bias, indices, scores, lse_total_out, sel_logits_out,
+                                    weights_out, L, N, NP, h_kv, G, topk, block_size, window_size, causal,
+                                    q_offset, sm_scale, page_table, max_pages, num_pages, lmk_hm, lmk_cap,
+                                    topk_row_dyn, (long)blockIdx.x);
 }
 
 // The remote branch of a decode step in one launch: the workgroup of a (query, KV head) row selects
@@ -1646,53 +1798,75 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
 #define DS_WAVES 8
 struct DsArgs {
   const bf16_t *q, *lmks, *k, *v;
-  const float* lse_swa;
+  const float *lse_swa, *bias;
   int32_t* indices;
   bf16_t *scores, *weights, *o;
   float *lse_total, *sel_logits;
   int L, N, NP, h_kv, G, topk, block_size, window_size, q_offset;
   float sm_scale_sel;
   const int32_t* page_table;
-  int max_pages, num_pages;
+  int max_pages, num_pages, lmk_hm, lmk_cap;
   DrDims dr;
 };
+// PAGED: the chunk keys (and the bias) are addressed through the page table; the attention reads
+// K and V through it whenever a.dr.page_table is set.
 template <int D, bool PAGED>
 __global__ void __launch_bounds__(DS_WAVES * 64) decode_step_kernel(DsArgs a) {
   extern __shared__ __align__(16) float ds_dyn[];
   const long row = blockIdx.x;
-  topk_row_body<D, 4, DS_WAVES, PAGED>(a.q, a.lmks, a.lse_swa, a.indices, a.scores, a.lse_total, a.sel_logits,
-                                       a.weights, a.L, a.N, a.NP, a.h_kv, a.G, a.topk, a.block_size,
-                                       a.window_size, 1, a.q_offset, a.sm_scale_sel, a.page_table, a.max_pages,
-                                       a.num_pages, ds_dyn, row);
-  __syncthreads();
-  decode_rows_body<D, DS_WAVES>(a.q, a.k, a.v, a.weights, a.indices, a.o, nullptr, a.dr, (char*)ds_dyn, 0,
-                                (int)(row % a.h_kv), row / a.h_kv);
+  __shared__ TopkRowShared ds_sh;
+  topk_row_body<D, 4, DS_WAVES, PAGED, true>(a.q, a.lmks, a.lse_swa, a.bias, a.indices, a.scores, a.lse_total,
+                                             a.sel_logits, a.weights, a.L, a.N, a.NP, a.h_kv, a.G, a.topk,
+                                             a.block_size, a.window_size, 1, a.q_offset, a.sm_scale_sel,
+                                             a.page_table, a.max_pages, a.num_pages, a.lmk_hm, a.lmk_cap, ds_dyn,
+                                             row, &ds_sh);
+  // The attention reads the row's indices and weights where the selection left them in LDS: the
+  // pointers are offset so that the row's entries of the (B, L, heads, ...) tensors fall there.  Its
+  // staging areas lie over the selection's logits: the barrier that separates the two uses runs in
+  // every wavefront once its first chunk's loads are in flight.
+  const int hk = (int)(row % a.h_kv);
+  const long bt = row / a.h_kv;
+  const bf16_t* w_row = ds_sh.win_w - (bt * a.dr.HQ + hk * a.G) * (long)a.dr.NW;
+  const int32_t* i_row = ds_sh.win_i - (bt * a.dr.H + hk) * (long)a.dr.K;
+  decode_rows_body<D, DS_WAVES>(a.q, a.k, a.v, w_row, i_row, a.o, nullptr, a.dr, (char*)ds_dyn, 0, hk, bt,
+                                [] __device__() { lds_barrier(); });  // (no wait for the loads in flight)
 }
 
 static int topk_cus() { return hils_device_cus(); }
 
 // the one-pass prefill kernel (topk_group.hip)
 bool hils_topk_group_covers(int N, int G, int D, int topk, int per_qhead, bool plain);
-int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* lse_swa, int32_t* indices,
-                           void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
+int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* lse_swa, const float* bias,
+                           int32_t* indices, void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
                            int G, int D, int topk, int block_size, int window_size, int causal, int q_offset,
                            float sm_scale, int lse_bf16, void* stream);
 
 // rows = (query, KV head) pairs; the row kernel wants about one row per compute unit
-static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool plain) {
+// LDS of a row workgroup before the wavefronts' staging areas: raw logits [4][NP], pooled scores, page
+// ids (paged chunk keys), the staged bias [4][NP]
+static size_t topk_row_smem_base(int N, bool paged, bool with_bias) {
+  const int NP = (N + 63) & ~63;
+  return (size_t)(5 + (paged ? 1 : 0) + (with_bias ? 4 : 0)) * NP * sizeof(float);
+}
+
+// plain: no Gumbel noise and no drop mask; a bias is staged in LDS beside the logits and must fit there
+static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool plain, bool with_bias = false,
+                         bool paged = false) {
+  if (with_bias && topk_row_smem_base(N, paged, true) + (size_t)8 * 16 * (2 * D + 16) + sizeof(TopkRowShared) > 158 * 1024)
+    return false;
   return plain && !per_qhead && G <= 4 && (D == 64 || D == 128) && N >= 256 && N <= TOPK_R_MAXN &&
          rows >= 96 && rows <= 2147483647L;
 }
 
-static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, int32_t* indices,
+static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, const float* bias, int32_t* indices,
                         void* scores, float* lse_total, float* sel_logits, void* weights, int B, int L, int N, int h_kv, int G, int D,
                         int topk, int block_size, int window_size, int causal, int q_offset,
                         float sm_scale, hipStream_t st, const int32_t* page_table = nullptr, int max_pages = 0,
-                        int num_pages = 0) {
+                        int num_pages = 0, int lmk_hm = 0, int lmk_cap = 0) {
   const long rows = (long)B * L * h_kv;
   const int NP = (N + 63) & ~63;
-  // raw logits [4][NP], pooled scores, page ids; then 16 padded key rows of staging per wavefront
-  const size_t smem_base = (size_t)(page_table ? 6 : 5) * NP * sizeof(float);
+  // then 16 padded key rows of staging per wavefront
+  const size_t smem_base = topk_row_smem_base(N, page_table != nullptr, bias != nullptr);
   const size_t stage_b = (size_t)16 * (2 * D + 16);
   // one round of rows or less: 16 wavefronts per row (the whole compute unit streams one row) if
   // their staging areas fit the LDS beside the logits; more rows than compute units: 8, so that
@@ -1705,10 +1879,10 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, i
     static HilsLdsReserve reserved;                                                              \
     if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_topk_fwd")) return rc; \
     hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(W_ * 64), smem, st,                      \
-                       (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, indices, (bf16_t*)scores, \
+                       (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, indices, (bf16_t*)scores, \
                        lse_total, sel_logits, (bf16_t*)weights, L, N, NP, h_kv, G, topk,         \
                        block_size, window_size, causal, q_offset, sm_scale, page_table, max_pages, \
-                       num_pages);                                                               \
+                       num_pages, lmk_hm, lmk_cap);                                              \
   } while (0)
 #define TOPK_ROW_CALL(D_, P_)                                                                    \
   do {                                                                                           \
@@ -1727,15 +1901,17 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, i
 // ---- the remote branch of a decode step in one launch (decode_step_kernel) ----
 bool hils_decode_rows_covers(int D, int Dv, int G, int K);
 
-extern "C" int hils_decode_step_covers(int B, int L, int N, int HQ, int H, int D, int topk, int block_size) {
+extern "C" int hils_decode_step_covers(int B, int L, int N, int HQ, int H, int D, int topk, int block_size,
+                                       int with_bias) {
   if (B <= 0 || L <= 0 || H <= 0 || HQ <= 0 || HQ % H != 0 || topk < 1 || topk > TOPK_MAXK || block_size != DR_S)
     return 0;
   const int G = HQ / H;
-  return topk_use_row((long)B * L * H, N, G, D, 0, true) && hils_decode_rows_covers(D, D, G, topk) ? 1 : 0;
+  // (paged chunk keys stage their page ids too: the stricter of the two LDS budgets)
+  return topk_use_row((long)B * L * H, N, G, D, 0, true, with_bias != 0, true) && hils_decode_rows_covers(D, D, G, topk) ? 1 : 0;
 }
 
 static int decode_step_launch(const void* q, const void* lmks, const void* k, const void* v, const float* lse_swa,
-                              int32_t* indices, void* scores, void* weights, void* o, float* lse_total,
+                              const float* bias, int lmk_paged, int lmk_hm, int lmk_cap, int32_t* indices, void* scores, void* weights, void* o, float* lse_total,
                               float* sel_logits, int B, int L, int Lkv, int N, int HQ, int H, int D, int topk,
                               int block_size, int window_size, int q_offset, float sm_scale_sel,
                               float sm_scale_attn, int mask_last, const int32_t* page_table, int max_pages,
@@ -1743,12 +1919,15 @@ static int decode_step_launch(const void* q, const void* lmks, const void* k, co
   const int G = HQ / H;
   const long rows = (long)B * L * H;
   const int NP = (N + 63) & ~63;
-  const size_t sel_b = (size_t)(page_table ? 6 : 5) * NP * sizeof(float) + (size_t)DS_WAVES * 16 * (2 * D + 16);
+  const size_t sel_b = topk_row_smem_base(N, lmk_paged != 0, bias != nullptr) + (size_t)DS_WAVES * 16 * (2 * D + 16);
+  HILS_REQUIRE(sel_b + sizeof(TopkRowShared) <= 158 * 1024,
+               "hils_decode_step: too many chunks (%d) to stage the bias beside the logits", N);
   const size_t att_b = dr_smem_bytes(D, G, DS_WAVES);
   const size_t smem = sel_b > att_b ? sel_b : att_b;
   DsArgs a;
   a.q = (const bf16_t*)q; a.lmks = (const bf16_t*)lmks; a.k = (const bf16_t*)k; a.v = (const bf16_t*)v;
-  a.lse_swa = lse_swa; a.indices = indices;
+  a.lse_swa = lse_swa; a.bias = bias; a.indices = indices;
+  a.lmk_hm = lmk_hm; a.lmk_cap = lmk_cap;
   a.scores = (bf16_t*)scores; a.weights = (bf16_t*)weights; a.o = (bf16_t*)o;
   a.lse_total = lse_total; a.sel_logits = sel_logits;
   a.L = L; a.N = N; a.NP = NP; a.h_kv = H; a.G = G; a.topk = topk; a.block_size = block_size;
@@ -1763,7 +1942,7 @@ static int decode_step_launch(const void* q, const void* lmks, const void* k, co
     if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_decode_step")) return rc; \
     hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(DS_WAVES * 64), smem, st, a);              \
   } while (0)
-  if (page_table) {
+  if (lmk_paged) {
     if (D == 64) DS_CALL(64, true); else DS_CALL(128, true);
   } else {
     if (D == 64) DS_CALL(64, false); else DS_CALL(128, false);
@@ -1773,19 +1952,22 @@ static int decode_step_launch(const void* q, const void* lmks, const void* k, co
 }
 
 extern "C" int hils_decode_step(const void* q, const void* lmks, const void* k, const void* v,
-                                const float* lse_swa, int32_t* indices, void* scores, void* weights, void* o,
-                                float* lse_total, float* sel_logits, int B, int L, int Lkv, int N, int HQ, int H,
-                                int D, int topk, int block_size, int window_size, int q_offset,
-                                float sm_scale_sel, float sm_scale_attn, int mask_last, void* stream) {
+                                const float* lse_swa, const float* bias, int32_t* indices, void* scores,
+                                void* weights, void* o, float* lse_total, float* sel_logits, int B, int L, int Lkv,
+                                int N, int HQ, int H, int D, int topk, int block_size, int window_size,
+                                int q_offset, float sm_scale_sel, float sm_scale_attn, int mask_last,
+                                int lmk_head_major, int lmk_cap, void* stream) {
   HILS_REQUIRE(q && lmks && k && v && lse_swa && indices && scores && weights && o, "hils_decode_step: null pointer");
   HILS_REQUIRE(B > 0 && L > 0 && N > 0 && H > 0 && HQ > 0 && HQ % H == 0, "hils_decode_step: bad sizes");
+  HILS_REQUIRE(!lmk_head_major || lmk_cap >= N, "hils_decode_step: lmk_cap (%d) must be at least N (%d)", lmk_cap, N);
   HILS_REQUIRE(Lkv >= (long)N * block_size, "hils_decode_step: the cache (%d tokens) is shorter than %d chunks", Lkv, N);
-  HILS_REQUIRE(hils_decode_step_covers(B, L, N, HQ, H, D, topk, block_size),
+  HILS_REQUIRE(hils_decode_step_covers(B, L, N, HQ, H, D, topk, block_size, bias != nullptr),
                "hils_decode_step: shape not covered (hils_decode_step_covers): use hils_topk_fwd_weights + hils_sparse_attn_fwd");
   HILS_REQUIRE((long)B * L * H <= 2147483647L, "hils_decode_step: grid too large");
-  if (int rc = decode_step_launch(q, lmks, k, v, lse_swa, indices, scores, weights, o, lse_total, sel_logits, B, L,
-                                  Lkv, N, HQ, H, D, topk, block_size, window_size, q_offset, sm_scale_sel,
-                                  sm_scale_attn, mask_last, nullptr, 0, 0, (hipStream_t)stream))
+  if (int rc = decode_step_launch(q, lmks, k, v, lse_swa, bias, 0, lmk_head_major, lmk_cap, indices, scores, weights, o,
+                                  lse_total, sel_logits, B, L, Lkv, N, HQ, H, D, topk, block_size, window_size,
+                                  q_offset, sm_scale_sel, sm_scale_attn, mask_last, nullptr, 0, 0,
+                                  (hipStream_t)stream))
     return rc;
   HILS_CHECK_LAUNCH("hils_decode_step");
   return HILS_OK;
@@ -1793,18 +1975,22 @@ extern "C" int hils_decode_step(const void* q, const void* lmks, const void* k, 
 
 extern "C" int hils_decode_step_paged(const void* q, const void* lmk_pages, const void* k_pages,
                                       const void* v_pages, const int32_t* page_table, const float* lse_swa,
-                                      int32_t* indices, void* scores, void* weights, void* o, float* lse_total,
-                                      float* sel_logits, int B, int L, int N, int HQ, int H, int D, int topk,
-                                      int block_size, int window_size, int q_offset, int max_pages, int num_pages,
-                                      float sm_scale_sel, float sm_scale_attn, int mask_last, void* stream) {
+                                      const float* bias, int32_t* indices, void* scores, void* weights, void* o,
+                                      float* lse_total, float* sel_logits, int B, int L, int N, int HQ, int H,
+                                      int D, int topk, int block_size, int window_size, int q_offset,
+                                      int max_pages, int num_pages, float sm_scale_sel, float sm_scale_attn,
+                                      int mask_last, int lmk_dense, int lmk_head_major, int lmk_cap, void* stream) {
+  HILS_REQUIRE(!lmk_dense || !lmk_head_major || lmk_cap >= N,
+               "hils_decode_step_paged: lmk_cap (%d) must be at least N (%d)", lmk_cap, N);
   HILS_REQUIRE(q && lmk_pages && k_pages && v_pages && page_table && lse_swa && indices && scores && weights && o,
                "hils_decode_step_paged: null pointer");
   HILS_REQUIRE(B > 0 && L > 0 && N > 0 && H > 0 && HQ > 0 && HQ % H == 0 && max_pages >= N && num_pages > 0,
                "hils_decode_step_paged: sizes must be positive and the page table must cover N chunks");
-  HILS_REQUIRE(hils_decode_step_covers(B, L, N, HQ, H, D, topk, block_size),
+  HILS_REQUIRE(hils_decode_step_covers(B, L, N, HQ, H, D, topk, block_size, bias != nullptr),
                "hils_decode_step_paged: shape not covered (hils_decode_step_covers): use hils_topk_fwd_weights_paged + hils_sparse_attn_decode_paged");
   HILS_REQUIRE((long)B * L * H <= 2147483647L, "hils_decode_step_paged: grid too large");
-  if (int rc = decode_step_launch(q, lmk_pages, k_pages, v_pages, lse_swa, indices, scores, weights, o, lse_total,
+  if (int rc = decode_step_launch(q, lmk_pages, k_pages, v_pages, lse_swa, bias, lmk_dense ? 0 : 1,
+                                  lmk_dense ? lmk_head_major : 0, lmk_cap, indices, scores, weights, o, lse_total,
                                   sel_logits, B, L, 0, N, HQ, H, D, topk, block_size, window_size, q_offset,
                                   sm_scale_sel, sm_scale_attn, mask_last, page_table, max_pages, num_pages,
                                   (hipStream_t)stream))
@@ -1875,7 +2061,8 @@ static int topk_fwd_split(const void* q, const void* lmks, const float* lse_swa,
 static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
                          const float* bias, const float* gumbel, const int32_t* drop_mask,
                          int32_t* indices, void* scores, float* lse_total, float* sel_logits,
-                         void* workspace, size_t workspace_bytes, void* weights, int* weights_fused, int B, int L, int N,
+                         void* workspace, size_t workspace_bytes, void* weights, const float* prior_b,
+                         int* weights_fused, int B, int L, int N,
                          int h_kv, int G, int D, int topk, int block_size, int window_size,
                          int causal, int q_offset, int per_qhead, float sm_scale, void* stream,
                          int lse_bf16 = 0) {
@@ -1894,11 +2081,14 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
                "(ask hils_topk_lse16_covers and pass lse_swa in fp32 otherwise)");
   // few queries per (batch, KV head) (decode, short continuations): one workgroup per row whenever
   // there are enough rows to occupy the machine, however many more there are
+  // (with a bias the row kernel's inter-chunk softmax adds that same bias to the winners' scores:
+  // it writes the weights only when the caller's prior bias is this bias)
   if ((topk_use_split(B, L, N, h_kv) || L <= 4) &&
-      topk_use_row((long)B * L * h_kv, N, G, D, per_qhead, !bias && !gumbel && !drop_mask)) {
-    *weights_fused = weights != nullptr;
-    if (int rc2 = topk_fwd_row(q, lmks, lse_swa, indices, scores, lse_total, sel_logits, weights, B, L, N, h_kv, G, D, topk,
-                               block_size, window_size, causal, q_offset, sm_scale, st))
+      topk_use_row((long)B * L * h_kv, N, G, D, per_qhead, !gumbel && !drop_mask, bias != nullptr)) {
+    const bool w_here = weights != nullptr && prior_b == bias;
+    *weights_fused = w_here;
+    if (int rc2 = topk_fwd_row(q, lmks, lse_swa, bias, indices, scores, lse_total, sel_logits, w_here ? weights : nullptr,
+                               B, L, N, h_kv, G, D, topk, block_size, window_size, causal, q_offset, sm_scale, st))
       return rc2;
     HILS_CHECK_LAUNCH("hils_topk_fwd");
     return HILS_OK;
@@ -1930,8 +2120,8 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
                          (const bf16_t*)lmks, (uint4*)workspace, N, h_kv, D, nblk16, total);
       packed = (const uint4*)workspace;
       // up to 512 chunks and 32 winners, nothing added to the logits: the one-pass kernel
-      if (hils_topk_group_covers(N, G, D, topk, per_qhead, !bias && !gumbel && !drop_mask)) {
-        if (int rc2 = hils_topk_group_launch(q, packed, lse_swa, indices, scores, lse_total, sel_logits, B, L, N,
+      if (hils_topk_group_covers(N, G, D, topk, per_qhead, !gumbel && !drop_mask)) {
+        if (int rc2 = hils_topk_group_launch(q, packed, lse_swa, bias, indices, scores, lse_total, sel_logits, B, L, N,
                                              h_kv, G, D, topk, block_size, window_size, causal, q_offset,
                                              sm_scale, lse_bf16, stream))
           return rc2;
@@ -1990,12 +2180,13 @@ extern "C" int hils_topk_fwd(const void* q, const void* lmks, const float* lse_s
                              int per_qhead, float sm_scale, void* stream) {
   int fused = 0;
   return topk_fwd_impl(q, lmks, lse_swa, bias, gumbel, drop_mask, indices, scores, lse_total, sel_logits,
-                       workspace, workspace_bytes, nullptr, &fused, B, L, N, h_kv, G, D, topk, block_size, window_size,
+                       workspace, workspace_bytes, nullptr, nullptr, &fused, B, L, N, h_kv, G, D, topk, block_size, window_size,
                        causal, q_offset, per_qhead, sm_scale, stream);
 }
 
 extern "C" int hils_topk_fwd_weights(const void* q, const void* lmks, const float* lse_swa,
-                                     const float* bias, const float* gumbel, const int32_t* drop_mask,
+                                     const float* bias, const float* prior_b, const float* gumbel,
+                                     const int32_t* drop_mask,
                                      int32_t* indices, void* scores, void* weights, void* workspace,
                                      size_t workspace_bytes, int B, int L, int N, int h_kv, int G, int D, int topk,
                                      int block_size, int window_size, int causal, int q_offset,
@@ -2003,27 +2194,27 @@ extern "C" int hils_topk_fwd_weights(const void* q, const void* lmks, const floa
   HILS_REQUIRE(weights, "hils_topk_fwd_weights: null pointer");
   int fused = 0;
   if (int rc = topk_fwd_impl(q, lmks, lse_swa, bias, gumbel, drop_mask, indices, scores, nullptr, nullptr,
-                             workspace, workspace_bytes, weights, &fused, B, L, N, h_kv, G, D, topk, block_size,
+                             workspace, workspace_bytes, weights, prior_b, &fused, B, L, N, h_kv, G, D, topk, block_size,
                              window_size, causal, q_offset, per_qhead, sm_scale, stream))
     return rc;
   if (fused) return HILS_OK;
-  return hils_chunk_weights(scores, lse_swa, 0, nullptr, nullptr, weights, B, L, h_kv * G, h_kv, N, topk, 0,
+  return hils_chunk_weights(scores, lse_swa, 0, prior_b, indices, weights, B, L, h_kv * G, h_kv, N, topk, 0,
                             stream);
 }
 
 extern "C" int hils_topk_fwd_weights_lse16(const void* q, const void* lmks, const void* lse_swa_bf16,
-                                           int32_t* indices, void* scores, void* weights, void* workspace,
+                                           const float* bias, const float* prior_b, int32_t* indices, void* scores, void* weights, void* workspace,
                                            size_t workspace_bytes, int B, int L, int N, int h_kv, int G, int D,
                                            int topk, int block_size, int window_size, int causal, int q_offset,
                                            float sm_scale, void* stream) {
   HILS_REQUIRE(weights && workspace, "hils_topk_fwd_weights_lse16: null pointer");
   int fused = 0;
-  if (int rc = topk_fwd_impl(q, lmks, (const float*)lse_swa_bf16, nullptr, nullptr, nullptr, indices, scores,
-                             nullptr, nullptr, workspace, workspace_bytes, weights, &fused, B, L, N, h_kv, G, D,
+  if (int rc = topk_fwd_impl(q, lmks, (const float*)lse_swa_bf16, bias, nullptr, nullptr, indices, scores,
+                             nullptr, nullptr, workspace, workspace_bytes, weights, prior_b, &fused, B, L, N, h_kv, G, D,
                              topk, block_size, window_size, causal, q_offset, 0, sm_scale, stream, 1))
     return rc;
   if (fused) return HILS_OK;
-  return hils_chunk_weights(scores, lse_swa_bf16, 1, nullptr, nullptr, weights, B, L, h_kv * G, h_kv, N, topk, 0,
+  return hils_chunk_weights(scores, lse_swa_bf16, 1, prior_b, indices, weights, B, L, h_kv * G, h_kv, N, topk, 0,
                             stream);
 }
 
@@ -2031,7 +2222,7 @@ extern "C" int hils_topk_fwd_weights_lse16(const void* q, const void* lmks, cons
 // the pooled key of every page, page_table (B, max_pages) maps chunk c of batch element b to its
 // page.  Selection + inter-chunk softmax as hils_topk_fwd_weights; one workgroup per (query, KV head).
 extern "C" int hils_topk_fwd_weights_paged(const void* q, const void* lmk_pages, const int32_t* page_table,
-                                           const float* lse_swa, int32_t* indices, void* scores, void* weights,
+                                           const float* lse_swa, const float* bias_pages, int32_t* indices, void* scores, void* weights,
                                            float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
                                            int G, int D, int topk, int block_size, int window_size, int q_offset,
                                            int max_pages, int num_pages, float sm_scale, void* stream) {
@@ -2044,9 +2235,11 @@ extern "C" int hils_topk_fwd_weights_paged(const void* q, const void* lmk_pages,
                "hils_topk_fwd_weights_paged: needs G <= 4, D in {64, 128}, N <= %d, topk <= %d", TOPK_R_MAXN,
                TOPK_MAXK);
   HILS_REQUIRE((long)B * L * h_kv <= 2147483647L, "hils_topk_fwd_weights_paged: grid too large");
-  if (int rc = topk_fwd_row(q, lmk_pages, lse_swa, indices, scores, lse_total, sel_logits, weights, B, L, N, h_kv,
-                            G, D, topk, block_size, window_size, 1, q_offset, sm_scale, (hipStream_t)stream,
-                            page_table, max_pages, num_pages))
+  HILS_REQUIRE(!bias_pages || topk_row_smem_base(N, true, true) + (size_t)8 * 16 * (2 * D + 16) + sizeof(TopkRowShared) <= 158 * 1024,
+               "hils_topk_fwd_weights_paged: too many chunks (%d) to stage the bias beside the logits", N);
+  if (int rc = topk_fwd_row(q, lmk_pages, lse_swa, bias_pages, indices, scores, lse_total, sel_logits, weights, B, L,
+                            N, h_kv, G, D, topk, block_size, window_size, 1, q_offset, sm_scale,
+                            (hipStream_t)stream, page_table, max_pages, num_pages))
     return rc;
   HILS_CHECK_LAUNCH("hils_topk_fwd_weights_paged");
   return HILS_OK;
@@ -2105,7 +2298,7 @@ extern "C" int hils_topk_fwd_noalloc(const void* q, const void* lmks, const floa
   // (repacked chunk keys, or the logits parked between the two decode kernels): nothing to clear
   int fused = 0;
   return topk_fwd_impl(q, lmks, lse_swa, bias, gumbel, drop_mask, indices, scores, lse_total, sel_logits,
-                       ws, HILS_TOPK_SCRATCH_BYTES, nullptr, &fused, B, L, N, h_kv, G, D, topk, block_size, window_size, causal,
+                       ws, HILS_TOPK_SCRATCH_BYTES, nullptr, nullptr, &fused, B, L, N, h_kv, G, D, topk, block_size, window_size, causal,
                        q_offset, per_qhead, sm_scale, stream);
 }
 

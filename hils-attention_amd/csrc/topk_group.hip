@@ -18,8 +18,10 @@
 //     exactly K; ties at the threshold go to the lower chunk indices,
 //   * the ascending order of the winners from a 512-bit map of the winning chunks in LDS
 //     (rank = set bits below the chunk), and the winners' raw scores straight from the logits.
-// Covers shared chunk keys, G <= 4, D in {64, 128}, N <= 512, topk <= 32, no bias / Gumbel noise /
-// drop mask; everything else runs on the kernels of topk.hip.
+// Covers shared chunk keys, G <= 4, D in {64, 128}, N <= 512, topk <= 32, an optional additive bias per
+// (chunk, head) (the layer's prior bias), no Gumbel noise / drop mask; everything else runs on the
+// kernels of topk.hip.  With a bias the registers hold the biased logits (what the log-sum-exp and
+// the selection work on) and a winner's raw score is its logit minus the bias again.
 #include <type_traits>
 #include "decode_rows.h"
 #include "../../include/hils_amd.h"
@@ -130,11 +132,12 @@ __device__ __forceinline__ uint32_t tg_kth_largest(const uint32_t (&k)[NE], uint
 // its registers and LDS until its slowest wavefront is through (the threshold searches differ in
 // length): 4 per workgroup ran 3.5 % slower than 2, and 8 ran 17 % slower; 1 was no faster than 2.
 #define TG_WAVES 2
-template <int GMAX, int KS, int NB, bool EXPORT>
+template <int GMAX, int KS, int NB, bool EXPORT, bool BIAS>
 __global__ void __launch_bounds__(64 * TG_WAVES)
     __attribute__((amdgpu_waves_per_eu(NB <= 8 ? 5 : (NB <= 16 ? 4 : (NB <= 24 ? 3 : 2)))))
 topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lmk_packed,
-                      const float* __restrict__ lse_swa, int32_t* __restrict__ indices,
+                      const float* __restrict__ lse_swa, const float* __restrict__ bias,
+                      int32_t* __restrict__ indices,
                       bf16_t* __restrict__ scores, float* __restrict__ lse_total_out,
                       float* __restrict__ sel_logits_out, int L, int N, int h_kv, int G, int topk,
                       int block_size, int window_size, int causal, int q_offset, float sm_scale,
@@ -223,10 +226,29 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
       for (int ks = 0; ks < KS; ++ks) dst[p2][ks] = *(const tg_u32x4*)&pbase[((long)nn * KS + ks) * 64];
     }
   };
+  // bias (B, N, h_kv, G) fp32: the G values of a (chunk, KV head) are contiguous; accumulator row
+  // 4j+i is head (4j+i) % GMAX
+  const float* bias_u = BIAS ? bias + (b * N * (long)h_kv + hk) * G : nullptr;
+  auto bias_of = [&](int c, float (&bv)[4]) {
+    const float* bp = bias_u + (long)(c < N ? c : N - 1) * h_kv * G;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) bv[i] = 0.f;
+    if constexpr (GMAX == 1) {
+      const float v0 = bp[0];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bv[i] = v0;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i % GMAX < G) bv[i] = bp[i % GMAX];
+    }
+  };
   auto use_group = [&](int g0, const tg_u32x4 (&src)[PB][KS]) {
 #pragma unroll
     for (int p2 = 0; p2 < PB; ++p2) {
       const int nt = g0 + p2;
+      float bv[4];
+      if constexpr (BIAS) bias_of(nt * 16 + col, bv);
       f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
@@ -235,6 +257,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float v = __fmul_rn(acc[i], sm_scale);
+        if constexpr (BIAS) v = __fadd_rn(v, bv[i]);
         if (nt >= NMASK) v = (c < lim[i]) ? v : HILS_NEG_INF;
         x[nt][i] = v;
       }
@@ -458,12 +481,21 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
           stage_i[qi * 32 + slot] = c;
           // the heads of the winner in one store (heads past G are never read back)
           bf16_t* dst = &stage_s[(qi * 32 + slot) * GMAX];
+          float raw[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) raw[i] = x[nt][i];
+          if constexpr (BIAS) {  // the returned scores carry no bias
+            float bv[4];
+            bias_of(c, bv);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) raw[i] = __fsub_rn(raw[i], bv[i]);
+          }
           if constexpr (GMAX == 4) {
-            *(uint2*)dst = make_uint2(pack_bf2(x[nt][u * 4], x[nt][u * 4 + 1]), pack_bf2(x[nt][u * 4 + 2], x[nt][u * 4 + 3]));
+            *(uint2*)dst = make_uint2(pack_bf2(raw[0], raw[1]), pack_bf2(raw[2], raw[3]));
           } else if constexpr (GMAX == 2) {
-            *(uint32_t*)dst = pack_bf2(x[nt][u * 2], x[nt][u * 2 + 1]);
+            *(uint32_t*)dst = pack_bf2(raw[u * 2], raw[u * 2 + 1]);
           } else {
-            *dst = f2bf(x[nt][u]);
+            *dst = f2bf(raw[u]);
           }
         }
       }
@@ -490,20 +522,21 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   }
 }
 
+// plain: no Gumbel noise and no drop mask (a bias is fine)
 bool hils_topk_group_covers(int N, int G, int D, int topk, int per_qhead, bool plain) {
   return plain && !per_qhead && (G == 1 || G == 3 || G == 4) && (D == 64 || D == 128) && N <= 16 * TG_NB &&
          topk <= 32;
 }
 
-template <int GMAX, int KS>
+template <int GMAX, int KS, bool BIAS>
 static void tg_launch_range(int NB, bool exp, dim3 grid, hipStream_t st, const bf16_t* q, const uint4* pk,
-                            const float* lse_swa, int32_t* indices, bf16_t* scores, float* lse_total,
+                            const float* lse_swa, const float* bias, int32_t* indices, bf16_t* scores, float* lse_total,
                             float* sel_logits, int L, int N, int h_kv, int G, int topk, int block_size,
                             int window_size, int causal, int q_offset, float sm_scale, int t_base, int t_end,
                             int lse_bf16) {
 #define TG_CALL(NB_, EX_)                                                                              \
-  hipLaunchKernelGGL((topk_fwd_group_kernel<GMAX, KS, NB_, EX_>), grid, dim3(64 * TG_WAVES), 0, st, q, pk, lse_swa, \
-                     indices, scores, lse_total, sel_logits, L, N, h_kv, G, topk, block_size, window_size, \
+  hipLaunchKernelGGL((topk_fwd_group_kernel<GMAX, KS, NB_, EX_, BIAS>), grid, dim3(64 * TG_WAVES), 0, st, q, pk, lse_swa, \
+                     bias, indices, scores, lse_total, sel_logits, L, N, h_kv, G, topk, block_size, window_size, \
                      causal, q_offset, sm_scale, t_base, t_end, bs_shift, lse_bf16)
   const int bs_shift = (block_size > 0 && (block_size & (block_size - 1)) == 0) ? __builtin_ctz(block_size) : -1;
   if (exp) { TG_CALL(32, true); return; }
@@ -518,7 +551,8 @@ static void tg_launch_range(int NB, bool exp, dim3 grid, hipStream_t st, const b
 
 // lmk_packed: the chunk keys in topk_pack_lmk_kernel's order.  The queries are split by how many
 // chunks they can see (at most 8, 16, 24 or 32 blocks of 16) into one launch each.
-int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* lse_swa, int32_t* indices,
+int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* lse_swa, const float* bias,
+                           int32_t* indices,
                            void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
                            int G, int D, int topk, int block_size, int window_size, int causal, int q_offset,
                            float sm_scale, int lse_bf16, void* stream) {
@@ -547,13 +581,18 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
       }
     }
     dim3 grid((t_hi - t + NQ * TG_WAVES - 1) / (NQ * TG_WAVES), h_kv, B);
+#define TG_RANGE_B(G_, KS_, B_)                                                                       \
+  tg_launch_range<G_, KS_, B_>(NB, exp, grid, st, (const bf16_t*)q, (const uint4*)lmk_packed, lse_swa, bias, \
+                               indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,   \
+                               block_size, window_size, causal, q_offset, sm_scale, t, t_hi, lse_bf16)
 #define TG_RANGE(G_, KS_)                                                                             \
-  tg_launch_range<G_, KS_>(NB, exp, grid, st, (const bf16_t*)q, (const uint4*)lmk_packed, lse_swa, indices, \
-                           (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk, block_size,   \
-                           window_size, causal, q_offset, sm_scale, t, t_hi, lse_bf16)
+  do {                                                                                                \
+    if (bias) TG_RANGE_B(G_, KS_, true); else TG_RANGE_B(G_, KS_, false);                             \
+  } while (0)
     if (GM == 1) { if (D == 64) TG_RANGE(1, 2); else TG_RANGE(1, 4); }
     else { if (D == 64) TG_RANGE(4, 2); else TG_RANGE(4, 4); }
 #undef TG_RANGE
+#undef TG_RANGE_B
     t = t_hi;
   }
   return HILS_OK;

@@ -24,12 +24,12 @@ SIGNATURES = {
     "hils_attn_pool_bwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
     "hils_topk_fwd": [_P] * 11 + [_Z] + [_I] * 12 + [_F, _P],
     "hils_topk_fwd_noalloc": [_P] * 10 + [_I] * 12 + [_F, _P],
-    "hils_topk_fwd_weights": [_P] * 10 + [_Z] + [_I] * 12 + [_F, _P],
-    "hils_topk_fwd_weights_lse16": [_P] * 7 + [_Z] + [_I] * 11 + [_F, _P],
-    "hils_topk_fwd_weights_paged": [_P] * 9 + [_I] * 12 + [_F, _P],
+    "hils_topk_fwd_weights": [_P] * 11 + [_Z] + [_I] * 12 + [_F, _P],
+    "hils_topk_fwd_weights_lse16": [_P] * 9 + [_Z] + [_I] * 11 + [_F, _P],
+    "hils_topk_fwd_weights_paged": [_P] * 10 + [_I] * 12 + [_F, _P],
     "hils_sparse_attn_decode_paged": [_P] * 8 + [_Z] + [_I] * 9 + [_F, _I, _P],
-    "hils_decode_step": [_P] * 11 + [_I] * 11 + [_F, _F, _I, _P],
-    "hils_decode_step_paged": [_P] * 12 + [_I] * 12 + [_F, _F, _I, _P],
+    "hils_decode_step": [_P] * 12 + [_I] * 11 + [_F, _F, _I, _I, _I, _P],
+    "hils_decode_step_paged": [_P] * 13 + [_I] * 12 + [_F, _F, _I, _I, _I, _I, _P],
     "hils_topk_bwd": [_P] * 7 + [_Z] + [_I] * 8 + [_F, _P],
     "hils_sparse_attn_fwd": [_P] * 10 + [_Z] + [_I] * 13 + [_F, _I, _F, _I, _P],
     "hils_pack_kv_chunks": [_P, _P, _P, _Z, _I, _I, _I, _I, _I, _P],
@@ -74,7 +74,7 @@ def load():
     lib.hils_topk_lse16_covers.restype = c_int
     lib.hils_topk_lse16_covers.argtypes = [_I] * 7
     lib.hils_decode_step_covers.restype = c_int
-    lib.hils_decode_step_covers.argtypes = [_I] * 8
+    lib.hils_decode_step_covers.argtypes = [_I] * 9
     lib.hils_sparse_attn_fwd_workspace.restype = ctypes.c_size_t
     lib.hils_sparse_attn_fwd_workspace.argtypes = [_I] * 11 + [_F]
     lib.hils_topk_bwd_workspace.restype = ctypes.c_size_t

@@ -69,13 +69,24 @@ def chunk_weights(scores, lse_swa, prior_b=None, indices=None, enable_softmax1=F
     return _ChunkWeightsFn.apply(scores, lse_swa, prior_b, indices, bool(enable_softmax1))
 
 
+def _prior_bias(prior_b, B, N, h_q):
+    """The layer's prior bias as a contiguous fp32 (B, N, h_q) tensor (None stays None)."""
+    if prior_b is None:
+        return None
+    assert prior_b.numel() == B * N * h_q and prior_b.shape[0] == B and prior_b.shape[1] == N, (
+        f"prior_b shape {tuple(prior_b.shape)} must be ({B}, {N}, {h_q})")
+    return prior_b.reshape(B, N, h_q).float().contiguous()
+
+
 def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causal=True, q_offset=0,
-                       sm_scale=None):
-    """Inference: ``online_softmax_topk_head`` (shared chunk keys, no bias / Gumbel / drop mask)
-    followed by ``chunk_weights`` in one call, for the serving loop.  q (B,L,h_q,D) bf16, lmks
-    (B,N,h_kv,D) bf16, lse_swa (B,L,h_q) -> indices (B,L,h_kv,topk) int32, scores (B,L,h_q,topk)
-    bf16, weights (B,L,h_q,topk+1) bf16.  With about one (query, KV head) row per compute unit
-    the selection kernel writes the weights itself; otherwise two kernels run."""
+                       sm_scale=None, prior_b=None):
+    """Inference: ``online_softmax_topk_head`` (shared chunk keys, no Gumbel / drop mask) followed by
+    ``chunk_weights`` in one call, for the serving loop.  q (B,L,h_q,D) bf16, lmks (B,N,h_kv,D) bf16,
+    lse_swa (B,L,h_q) -> indices (B,L,h_kv,topk) int32, scores (B,L,h_q,topk) bf16, weights
+    (B,L,h_q,topk+1) bf16.  ``prior_b`` (B,N,h_q): the layer's prior bias (its ``enable_prior_query``
+    mode, models/FlashHiLS/hils_attention.py:568-602), used as the selection's ``bias`` and gathered
+    into the softmax.  With about one (query, KV head) row per compute unit the selection kernel
+    writes the weights itself; otherwise two kernels run."""
     import math
     _cabi.require_gpu_bf16("topk_chunk_weights", q, lmks)
     if torch.is_grad_enabled() and (q.requires_grad or lmks.requires_grad or lse_swa.requires_grad):
@@ -87,6 +98,7 @@ def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causa
     G = h_q // h_kv
     scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(D)
     dev = q.device
+    pb = _prior_bias(prior_b, B, N, h_q)
     indices = torch.empty((B, L, h_kv, topk), dtype=torch.int32, device=dev)
     scores = torch.empty((B, L, h_q, topk), dtype=q.dtype, device=dev)
     weights = torch.empty((B, L, h_q, topk + 1), dtype=q.dtype, device=dev)
@@ -95,27 +107,48 @@ def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causa
             and _cabi.load().hils_topk_lse16_covers(B, L, N, h_kv, G, D, int(topk))):
         # lse_swa as the layer hands it over (bf16): read in place, no conversion pass
         _cabi.call("hils_topk_fwd_weights_lse16", _cabi.ptr(q.contiguous()), _cabi.ptr(lmks.contiguous()),
-                   _cabi.ptr(lse_swa.reshape(B, L, h_q).contiguous()), _cabi.ptr(indices), _cabi.ptr(scores),
-                   _cabi.ptr(weights), _cabi.ptr(ws), _cabi.nbytes(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),
-                   int(window_size), int(bool(is_causal)), int(q_offset), scale)
+                   _cabi.ptr(lse_swa.reshape(B, L, h_q).contiguous()), _cabi.ptr(pb), _cabi.ptr(pb),
+                   _cabi.ptr(indices), _cabi.ptr(scores), _cabi.ptr(weights), _cabi.ptr(ws), _cabi.nbytes(ws),
+                   B, L, N, h_kv, G, D, int(topk), int(block_size), int(window_size), int(bool(is_causal)),
+                   int(q_offset), scale)
         return indices, scores, weights
     lse = lse_swa.reshape(B, L, h_q).float().contiguous()
     _cabi.call("hils_topk_fwd_weights", _cabi.ptr(q.contiguous()), _cabi.ptr(lmks.contiguous()),
-               _cabi.ptr(lse), None, None, None, _cabi.ptr(indices), _cabi.ptr(scores),
-               _cabi.ptr(weights), _cabi.ptr(ws), _cabi.nbytes(ws), B, L, N, h_kv, G, D, int(topk), int(block_size),
-               int(window_size), int(bool(is_causal)), int(q_offset), 0, scale)
+               _cabi.ptr(lse), _cabi.ptr(pb), _cabi.ptr(pb), None, None, _cabi.ptr(indices), _cabi.ptr(scores),
+               _cabi.ptr(weights), _cabi.ptr(ws), _cabi.nbytes(ws), B, L, N, h_kv, G, D, int(topk),
+               int(block_size), int(window_size), int(bool(is_causal)), int(q_offset), 0, scale)
     return indices, scores, weights
 
 
+def head_major_chunk_keys(lmks, prior_b=None, capacity=None):
+    """Chunk keys (B,N,h_kv,D) (and the prior bias (B,N,h_q)) re-laid head-major, (B,h_kv,cap,D) and
+    (B,h_kv,cap,G): the N keys a decode row streams become one contiguous block.  What this
+    package's cache layers keep; ``decode_step(..., lmk_head_major=True)`` takes them."""
+    B, N, h_kv, D = lmks.shape
+    cap = N if capacity is None else int(capacity)
+    assert cap >= N
+    out = torch.zeros((B, h_kv, cap, D), dtype=lmks.dtype, device=lmks.device)
+    out[:, :, :N] = lmks.permute(0, 2, 1, 3)
+    if prior_b is None:
+        return out
+    G = prior_b.shape[2] // h_kv
+    pb = torch.zeros((B, h_kv, cap, G), dtype=torch.float32, device=lmks.device)
+    pb[:, :, :N] = prior_b.reshape(B, N, h_kv, G).permute(0, 2, 1, 3).float()
+    return out, pb
+
+
 def decode_step(q, lmks, k, v, lse_swa, topk, block_size, window_size, q_offset=0, sm_scale=None,
-                mask_last_token=True, _debug=None):
+                mask_last_token=True, _debug=None, prior_b=None, lmk_head_major=False, num_chunks=None):
     """Inference: the remote branch of a decode step, ``topk_chunk_weights`` followed by
     ``HiLS_block_M_head(..., is_training=False)`` on the selected chunks, in one kernel launch (one
     workgroup per (query, KV head) selects and then attends).  q (B,L,h_q,D), lmks (B,N,h_kv,D), k, v
     (B,Lkv,h_kv,D) bf16 (k, v may live in pinned host memory), lse_swa (B,L,h_q) -> o (B,L,h_q,D),
-    weights (B,L,h_q,topk+1), indices (B,L,h_kv,topk), scores (B,L,h_q,topk).  Shapes the fused kernel
-    does not take (few rows, short caches, more than four query heads per KV head, ...) run as the
-    two calls."""
+    weights (B,L,h_q,topk+1), indices (B,L,h_kv,topk), scores (B,L,h_q,topk).  ``prior_b`` (B,N,h_q):
+    the layer's prior bias (selection bias and the bias of the inter-chunk softmax).
+    ``lmk_head_major``: lmks is (B,h_kv,cap,D) and prior_b (B,h_kv,cap,G) (``head_major_chunk_keys``),
+    of which the first ``num_chunks`` (default cap) chunks are looked at.  Shapes the fused kernel does
+    not take (few rows, short caches, more than four query heads per KV head, ...) run as the two
+    calls."""
     import math
     from .hils_fwd_bwd_head import HiLS_block_M_head
     _cabi.require_gpu_bf16("decode_step", q, lmks)
@@ -123,20 +156,39 @@ def decode_step(q, lmks, k, v, lse_swa, topk, block_size, window_size, q_offset=
     if torch.is_grad_enabled() and any(t.requires_grad for t in (q, lmks, k, v, lse_swa)):
         raise RuntimeError("decode_step is forward-only")
     B, L, h_q, D = q.shape
-    N, h_kv = lmks.shape[1], lmks.shape[2]
+    if lmk_head_major:
+        h_kv, cap = lmks.shape[1], lmks.shape[2]
+        N = cap if num_chunks is None else int(num_chunks)
+        assert 0 < N <= cap
+    else:
+        N, h_kv = lmks.shape[1], lmks.shape[2]
+        cap = N
+        assert num_chunks is None or int(num_chunks) == N
     Lkv = k.shape[1]
     assert lmks.shape[0] == B and lmks.shape[3] == D and k.shape == v.shape and k.shape[0] == B
     assert k.shape[2] == h_kv and k.shape[3] == D and h_q % h_kv == 0
+    G = h_q // h_kv
     scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(D)
     lib = _cabi.load()
-    if not (lib.hils_decode_step_covers(B, L, N, h_q, h_kv, D, int(topk), int(block_size)) and Lkv >= N * block_size):
+    pb = None
+    if prior_b is not None:
+        if lmk_head_major:
+            assert prior_b.shape == (B, h_kv, cap, G), f"prior_b shape {tuple(prior_b.shape)} != {(B, h_kv, cap, G)}"
+            pb = prior_b.float().contiguous()
+        else:
+            pb = _prior_bias(prior_b, B, N, h_q)
+    if not (lib.hils_decode_step_covers(B, L, N, h_q, h_kv, D, int(topk), int(block_size), int(pb is not None))
+            and Lkv >= N * block_size):
+        if lmk_head_major:  # the two-call kernels read the reference's layout
+            lmks = lmks[:, :, :N].permute(0, 2, 1, 3).contiguous()
+            if pb is not None:
+                pb = pb[:, :, :N].permute(0, 2, 1, 3).reshape(B, N, h_q).contiguous()
         idx, sc, w = topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, q_offset=q_offset,
-                                        sm_scale=scale)
+                                        sm_scale=scale, prior_b=pb)
         o = HiLS_block_M_head(q, k, v, w, idx, block_size=block_size, sm_scale=scale,
                               mask_last_token=mask_last_token, is_training=False)
         return o, w, idx, sc
     dev = q.device
-    G = h_q // h_kv
     lse = lse_swa.reshape(B, L, h_q).float().contiguous()
     indices = torch.empty((B, L, h_kv, topk), dtype=torch.int32, device=dev)
     scores = torch.empty((B, L, h_q, topk), dtype=q.dtype, device=dev)
@@ -148,9 +200,10 @@ def decode_step(q, lmks, k, v, lse_swa, topk, block_size, window_size, q_offset=
         sel_logits = torch.full((B, L, h_kv, G, N), float("-inf"), dtype=torch.float32, device=dev)
     kk, vv = _cabi.gpu_readable(k, dev), _cabi.gpu_readable(v, dev)
     _cabi.call("hils_decode_step", _cabi.ptr(q.contiguous()), _cabi.ptr(lmks.contiguous()), _cabi.ptr(kk),
-               _cabi.ptr(vv), _cabi.ptr(lse), _cabi.ptr(indices), _cabi.ptr(scores), _cabi.ptr(weights),
-               _cabi.ptr(o), _cabi.ptr(lse_total), _cabi.ptr(sel_logits), B, L, Lkv, N, h_q, h_kv, D, int(topk),
-               int(block_size), int(window_size), int(q_offset), scale, scale, int(bool(mask_last_token)))
+               _cabi.ptr(vv), _cabi.ptr(lse), _cabi.ptr(pb), _cabi.ptr(indices), _cabi.ptr(scores),
+               _cabi.ptr(weights), _cabi.ptr(o), _cabi.ptr(lse_total), _cabi.ptr(sel_logits), B, L, Lkv, N, h_q,
+               h_kv, D, int(topk), int(block_size), int(window_size), int(q_offset), scale, scale,
+               int(bool(mask_last_token)), int(bool(lmk_head_major)), cap)
     if _debug is not None:
         _debug.update(lse_total=lse_total, sel_logits=sel_logits)
     return o, weights, indices, scores

@@ -96,13 +96,15 @@ int hils_topk_fwd_noalloc(const void* q, const void* lmks, const float* lse_swa,
                           int causal, int q_offset, int per_qhead, float sm_scale, void* stream);
 
 /* hils_topk_fwd plus the layer's inter-chunk softmax in the same call (inference): also writes
- * weights (B,L,h_kv*G,topk+1) bf16 = softmax over [scores (as bf16), lse_swa], the K+1-way
- * softmax of models/FlashHiLS/hils_attention.py:604-610 without prior bias (what
- * hils_chunk_weights computes from these scores).  With about one (query, KV head) row per
- * compute unit the selection kernel writes them itself; otherwise hils_chunk_weights runs on the
- * same stream.  No lse_total / sel_logits outputs. */
+ * weights (B,L,h_kv*G,topk+1) bf16 = softmax over [scores (as bf16) (+ prior_b gathered at the
+ * indices, cast to bf16), lse_swa], the K+1-way softmax of models/FlashHiLS/hils_attention.py:585-610
+ * (what hils_chunk_weights computes from these scores).  prior_b (B,N,h_kv*G) fp32 or NULL; the
+ * layer's default mode (enable_prior_query) passes one tensor as `bias` and as `prior_b`
+ * (hils_attention.py:568-602).  With about one (query, KV head) row per compute unit the selection
+ * kernel writes the weights itself (when prior_b == bias or both are NULL); otherwise
+ * hils_chunk_weights runs on the same stream.  No lse_total / sel_logits outputs. */
 int hils_topk_fwd_weights(const void* q, const void* lmks, const float* lse_swa, const float* bias,
-                          const float* gumbel, const int32_t* drop_mask, int32_t* indices,
+                          const float* prior_b, const float* gumbel, const int32_t* drop_mask, int32_t* indices,
                           void* scores, void* weights, void* workspace, size_t workspace_bytes, int B, int L,
                           int N, int h_kv, int G, int D, int topk, int block_size, int window_size, int causal,
                           int q_offset, int per_qhead, float sm_scale, void* stream);
@@ -111,10 +113,12 @@ int hils_topk_fwd_weights(const void* q, const void* lmks, const float* lse_swa,
  * (lse_sum.to(hidden_states.dtype), models/FlashHiLS/hils_attention.py:547; its kernels read it in
  * that dtype, ops/topk_head_softmax.py:1291-1367): saves the conversion pass.  Only the shapes
  * hils_topk_lse16_covers accepts (many queries, shared chunk keys, G in {1,3,4}, N <= 512, topk <= 32,
- * no bias / noise / drop mask: the one-pass prefill kernel), with the workspace of
- * hils_topk_fwd_workspace; other shapes are rejected and take hils_topk_fwd_weights with fp32. */
+ * no noise / drop mask: the one-pass prefill kernel), with the workspace of
+ * hils_topk_fwd_workspace; other shapes are rejected and take hils_topk_fwd_weights with fp32.
+ * bias / prior_b as in hils_topk_fwd_weights (NULL for none). */
 int hils_topk_lse16_covers(int B, int L, int N, int h_kv, int G, int D, int topk);
-int hils_topk_fwd_weights_lse16(const void* q, const void* lmks, const void* lse_swa_bf16, int32_t* indices,
+int hils_topk_fwd_weights_lse16(const void* q, const void* lmks, const void* lse_swa_bf16, const float* bias,
+                                const float* prior_b, int32_t* indices,
                                 void* scores, void* weights, void* workspace, size_t workspace_bytes, int B,
                                 int L, int N, int h_kv, int G, int D, int topk, int block_size, int window_size,
                                 int causal, int q_offset, float sm_scale, void* stream);
@@ -245,13 +249,15 @@ int hils_sparse_attn_bwd_f32(const float* q, const float* k, const float* v, con
  * is invisible to the selection and contributes nothing to the attention).
  *
  * hils_topk_fwd_weights_paged: selection + inter-chunk softmax as hils_topk_fwd_weights (shared
- * chunk keys, no bias / noise / drop mask, causal), N = chunks of the sequence, L <= a few queries;
- * lse_total / sel_logits optional as in hils_topk_fwd.
+ * chunk keys, no noise / drop mask, causal), N = chunks of the sequence, L <= a few queries;
+ * bias_pages (num_pages, h_kv*G) fp32 or NULL: the prior bias of every page (selection bias and the
+ * bias of the inter-chunk softmax, as the layer uses it); lse_total / sel_logits optional as in
+ * hils_topk_fwd.
  * hils_sparse_attn_decode_paged: hils_sparse_attn_fwd's decode path; indices are chunk numbers of the
  * sequence (what the selection returns).  workspace: hils_sparse_attn_decode_paged_workspace bytes
  * or NULL. */
 int hils_topk_fwd_weights_paged(const void* q, const void* lmk_pages, const int32_t* page_table,
-                                const float* lse_swa, int32_t* indices, void* scores, void* weights,
+                                const float* lse_swa, const float* bias_pages, int32_t* indices, void* scores, void* weights,
                                 float* lse_total, float* sel_logits, int B, int L, int N, int h_kv, int G,
                                 int D, int topk, int block_size, int window_size, int q_offset,
                                 int max_pages, int num_pages, float sm_scale, void* stream);
@@ -272,22 +278,31 @@ int hils_sparse_attn_decode_paged(const void* q, const void* k_pages, const void
  * and then attends over the chunks it has selected: one launch instead of two, and the rows'
  * selection tails overlap other rows' memory streams.  Outputs as the two calls give them; o
  * (B,L,HQ,D) bf16 is the remote branch's output (the caller adds swa_o * weights[..., topk]).
- * lse_total / sel_logits optional as in hils_topk_fwd.  q (B,L,HQ,D); lmks (B,N,H,D) or lmk_pages;
- * k, v (B,Lkv,H,D) with Lkv >= N * 64 or k_pages, v_pages (num_pages,H,64,D).
+ * lse_total / sel_logits optional as in hils_topk_fwd.  q (B,L,HQ,D); k, v (B,Lkv,H,D) with
+ * Lkv >= N * 64 or k_pages, v_pages (num_pages,H,64,D).
+ * Chunk keys: lmks (B,N,H,D), the layout of the reference's _hils_prior_cache; or, lmk_head_major != 0,
+ * (B,H,lmk_cap,D) with lmk_cap >= N chunks allocated per (batch, head): the N keys a row streams are
+ * then one contiguous block instead of 2*D-byte rows at a stride of H*2*D bytes (what this build's cache
+ * layers keep).  The paged entry point takes lmk_pages (num_pages,H,D) addressed through the page
+ * table, or, lmk_dense != 0, dense chunk keys in one of the two layouts above beside paged K and V.
+ * bias: the layer's prior bias (models/FlashHiLS/hils_attention.py:568-602: the selection's `bias`
+ * and the bias gathered into the inter-chunk softmax), fp32, NULL for none; laid out like the chunk
+ * keys with the G heads of a KV head in place of D: (B,N,H*G), (B,H,lmk_cap,G) or (num_pages,H*G).
  * Covered shapes (hils_decode_step_covers returns 1): shared chunk keys, causal, block_size 64,
- * D = Dv in {64, 128}, HQ/H <= 4, 256 <= N <= 4096, topk <= 64, at least 96 rows B*L*H. */
-int hils_decode_step_covers(int B, int L, int N, int HQ, int H, int D, int topk, int block_size);
+ * D = Dv in {64, 128}, HQ/H <= 4, 256 <= N <= 4096 (<= 3072 with a bias, which is staged in LDS),
+ * topk <= 64, at least 96 rows B*L*H. */
+int hils_decode_step_covers(int B, int L, int N, int HQ, int H, int D, int topk, int block_size, int with_bias);
 int hils_decode_step(const void* q, const void* lmks, const void* k, const void* v, const float* lse_swa,
-                     int32_t* indices, void* scores, void* weights, void* o, float* lse_total,
-                     float* sel_logits, int B, int L, int Lkv, int N, int HQ, int H, int D, int topk,
-                     int block_size, int window_size, int q_offset, float sm_scale_sel,
-                     float sm_scale_attn, int mask_last, void* stream);
+                     const float* bias, int32_t* indices, void* scores, void* weights, void* o,
+                     float* lse_total, float* sel_logits, int B, int L, int Lkv, int N, int HQ, int H, int D,
+                     int topk, int block_size, int window_size, int q_offset, float sm_scale_sel,
+                     float sm_scale_attn, int mask_last, int lmk_head_major, int lmk_cap, void* stream);
 int hils_decode_step_paged(const void* q, const void* lmk_pages, const void* k_pages, const void* v_pages,
-                           const int32_t* page_table, const float* lse_swa, int32_t* indices, void* scores,
-                           void* weights, void* o, float* lse_total, float* sel_logits, int B, int L, int N,
-                           int HQ, int H, int D, int topk, int block_size, int window_size, int q_offset,
-                           int max_pages, int num_pages, float sm_scale_sel, float sm_scale_attn,
-                           int mask_last, void* stream);
+                           const int32_t* page_table, const float* lse_swa, const float* bias, int32_t* indices,
+                           void* scores, void* weights, void* o, float* lse_total, float* sel_logits, int B,
+                           int L, int N, int HQ, int H, int D, int topk, int block_size, int window_size,
+                           int q_offset, int max_pages, int num_pages, float sm_scale_sel, float sm_scale_attn,
+                           int mask_last, int lmk_dense, int lmk_head_major, int lmk_cap, void* stream);
 
 /* ---- exact per-chunk log Z ---------------------------------------------------- */
 

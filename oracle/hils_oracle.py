@@ -415,9 +415,11 @@ def swa(q, k, v, *, window_size: int, chunk_size: int, mask_lmk: bool = True,
 # ----------------------------------------------------------------------------
 # layer glue and the dense equivalent
 # ----------------------------------------------------------------------------
-def inter_chunk_softmax(scores, lse_swa, prior_b=None, indices=None, softmax1=False):
+def inter_chunk_softmax(scores, lse_swa, prior_b=None, indices=None, softmax1=False, bf16_sum=False):
     """chunk_weights = softmax([scores_1..K (+ gathered prior bias), lse_swa (, 0)]).
-    scores (B,L,hq,K); returns fp32 (B,L,hq,K+1(+1))."""
+    scores (B,L,hq,K); returns fp32 (B,L,hq,K+1(+1)).  ``bf16_sum``: round the biased scores to bf16,
+    as the layer's ``scores + gathered.to(scores.dtype)`` on bf16 tensors does
+    (models/FlashHiLS/hils_attention.py:600-602); the default keeps the sum in fp32."""
     B, L, HQ, K = scores.shape
     sc = scores.float()
     if prior_b is not None:
@@ -425,6 +427,8 @@ def inter_chunk_softmax(scores, lse_swa, prior_b=None, indices=None, softmax1=Fa
         idx = indices.repeat_interleave(HQ // Hkv, dim=2).clamp_min(0).long()
         src = prior_b.float().unsqueeze(-1).expand(-1, -1, -1, K)
         sc = sc + torch.gather(src, 1, idx)
+        if bf16_sum:
+            sc = sc.bfloat16().float()
     cols = [sc, lse_swa.float().unsqueeze(-1)]
     if softmax1:
         cols.append(torch.zeros(B, L, HQ, 1))

@@ -220,7 +220,7 @@ def test_short_workspace_is_rejected_by_the_c_abi(pkg):
     rc = lib.hils_topk_fwd(buf, buf, buf, None, None, None, buf, buf, None, None, buf, need_t - 1,
                            B, L, N, h_kv, G, D, K, S, 1, 1, 0, 0, 0.088, None)
     assert rc == 1 and b"shorter" in lib.hils_last_error()
-    rc = lib.hils_topk_fwd_weights(buf, buf, buf, None, None, None, buf, buf, buf, buf, need_t - 1,
+    rc = lib.hils_topk_fwd_weights(buf, buf, buf, None, None, None, None, buf, buf, buf, buf, need_t - 1,
                                    B, L, N, h_kv, G, D, K, S, 1, 1, 0, 0, 0.088, None)
     assert rc == 1 and b"shorter" in lib.hils_last_error()
     need_tb = lib.hils_topk_bwd_workspace(B, L, N, h_kv, 3, D, K)   # G = 3: the inverse-index kernels
