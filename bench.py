@@ -333,7 +333,24 @@ def bench_ops(pkg, dev, iters=3):
 
     out["attn_pool_fwd_bwd"] = {"workload": "B1 N512 S64 H32 D128 (includes the torch glue of the loss)",
                                 "us": timed(pool_fb) * 1e3}
-    del kc, kc_g, mu, mu_g
+    del kc, kc_g, mu_g
+    # the same prior queries over K at the model's own 8 KV heads (four query heads per K tile)
+    kc8 = gpu_randn((1, N, S, 8, D), gen, dev)
+    with torch.no_grad():
+        t = timed(lambda: pkg.chunk_attn_pool(mu, kc8), 10)
+    out["attn_pool_gqa_fwd"] = {"workload": "B1 N512 S64 hq32/hkv8 D128", "us": t * 1e3,
+                                "hbm_gbs": (kc8.numel() * 2 + 2 * mu.numel() * 2 + N * S * H * 4) / (t * 1e-3) / 1e9}
+    mu_g, kc_g = mu.clone().requires_grad_(), kc8.clone().requires_grad_()
+
+    def pool_gqa_fb():
+        mu_g.grad = None
+        kc_g.grad = None
+        a, b = pkg.chunk_attn_pool(mu_g, kc_g)
+        (a.float().sum() + b.sum()).backward()
+
+    out["attn_pool_gqa_fwd_bwd"] = {"workload": "same (includes the torch glue of the loss)",
+                                    "us": timed(pool_gqa_fb, 10) * 1e3}
+    del kc8, kc_g, mu, mu_g
     # key preparation in one pass (RMS norm + rotary embedding + chunk mean) on the 32K prefill's K
     Lp, Hk = 32768, 8
     kx = gpu_randn((1, Lp, Hk, D), gen, dev)
@@ -393,6 +410,54 @@ def bench_ops(pkg, dev, iters=3):
 
     out["swa_fwd_bwd"] = {"workload": "same", "us": timed(swa_fb) * 1e3}
     del q, k, v, qg, kg, vg, d_o
+    # the local branch at the window the reference times it at (scripts/bench/bench_flex_attn_bwd_clamp.py:66-72:
+    # window 512, chunk 64, L16384; 16/2 heads of 64 with the window expanded to its chunk start, 32/32 heads
+    # of 128 without)
+    for name, HQ, HK, D, expand in (("w512_hq16_hkv2_d64", 16, 2, 64, True), ("w512_hq32_hkv32_d128", 32, 32, 128, False)):
+        L, Wn = 16384, 512
+        q = gpu_randn((1, L, HQ, D), gen, dev)
+        k = gpu_randn((1, L, HK, D), gen, dev)
+        v = gpu_randn((1, L, HK, D), gen, dev)
+        with torch.no_grad():
+            t = timed(lambda: pkg.flex_attn_tl(q, k, v, Wn, 64, expand_to_chunk=expand))
+        tt = torch.arange(L, device=dev)
+        lo = (tt - Wn + 1).clamp_min(0)
+        if expand:
+            lo = torch.div(lo, 64, rounding_mode="floor") * 64
+        # keys lo .. t, landmarks (positions 63 mod 64) excluded
+        n_lmk = torch.div(tt + 1, 64, rounding_mode="floor") - torch.div(lo, 64, rounding_mode="floor")
+        n_vis = float((tt - lo + 1 - n_lmk).sum().item())
+        flops = 4.0 * D * HQ * n_vis
+        out["swa_fwd_" + name] = {"workload": f"B1 L{L} hq{HQ}/hkv{HK} D{D} window{Wn} chunk64 expand_to_chunk={expand}",
+                                  "us": t * 1e3, "visible_tflops": flops / (t * 1e-3) / 1e12,
+                                  "hbm_gbs": (2 * q.numel() + k.numel() + v.numel()) * 2 / (t * 1e-3) / 1e9}
+        qg, kg, vg = (x.clone().requires_grad_() for x in (q, k, v))
+        d_o = gpu_randn((1, L, HQ, D), gen, dev)
+
+        def swa_fb512():
+            for x in (qg, kg, vg):
+                x.grad = None
+            o, lse = pkg.flex_attn_tl(qg, kg, vg, Wn, 64, expand_to_chunk=expand)
+            torch.autograd.backward([o, lse], [d_o, torch.ones_like(lse)])
+
+        t = timed(swa_fb512)
+        # the forward's two products (S, P V) and the backward's five (S again, dV, dP, dQ, dK)
+        out["swa_fwd_bwd_" + name] = {"workload": "same", "us": t * 1e3,
+                                      "visible_tflops": 3.5 * flops / (t * 1e-3) / 1e12,
+                                      "hbm_gbs": (4 * q.numel() + 2 * (k.numel() + v.numel())) * 2 / (t * 1e-3) / 1e9}
+        del q, k, v, qg, kg, vg, d_o
+    # chunk selection + inter-chunk weights of the 32K prefill, without and with the layer's prior bias
+    # (models/FlashHiLS/hils_attention.py:568-602: the bias of the selection and of the softmax)
+    q, k, v, lse_p = prefill_inputs(dev)
+    del v
+    lmk = pkg.chunk_mean_pool(k, 64)
+    prior = (torch.randn(1, lmk.shape[1], q.shape[2], device=dev, generator=gen) * 0.5).bfloat16()
+    with torch.no_grad():
+        t0 = timed(lambda: pkg.topk_chunk_weights(q, lmk, lse_p, 32, 64, 1), 5)
+        t1 = timed(lambda: pkg.topk_chunk_weights(q, lmk, lse_p, 32, 64, 1, prior_b=prior), 5)
+    out["topk_prefill"] = {"workload": "B1 L32768 hq32/hkv8 D128 N512 top32 (selection + weights)", "us": t0 * 1e3}
+    out["topk_prefill_bias"] = {"workload": "same, with a prior bias (B,N,h_q)", "us": t1 * 1e3}
+    del q, k, lse_p, lmk, prior
     # rotary embedding of q and k: B1 L32768 hq32/hkv8 D128
     L, HQ, HK, D = 32768, 32, 8, 128
     q = gpu_randn((1, L, HQ, D), gen, dev)

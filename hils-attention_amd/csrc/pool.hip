@@ -124,7 +124,7 @@ extern "C" int hils_mean_pool_bwd(const void* g_lmk, void* dk, int B, int L, int
 __global__ void __launch_bounds__(POOL_THREADS)
 attn_pool_fwd_kernel(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k,
                      bf16_t* __restrict__ lmk_k, float* __restrict__ lmk_b, float* __restrict__ p_out,
-                     int S, int H, int D, float sm_scale, int compact, int shared_k) {
+                     int S, int H, int HK, int D, float sm_scale, int compact, int shared_k) {
   extern __shared__ float smem[];
   const int DP = D + 1;
   float* ks = smem;              // S * DP
@@ -133,13 +133,13 @@ attn_pool_fwd_kernel(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__
   float* red = pr + S;           // 32
   const long bn = blockIdx.x;
   const int h = blockIdx.y;
-  const int kh = shared_k ? 0 : h;
+  const int kh = shared_k ? 0 : h / (H / HK);  // K has HK heads: H / HK query heads read each
   const int tid = threadIdx.x;
 
   const int d8 = D / 8;
   for (int i = tid; i < S * d8; i += POOL_THREADS) {
     const int s = i / d8, c = i - s * d8;
-    uint4 v = *(const uint4*)(k + ((bn * S + s) * (long)H + kh) * D + c * 8);
+    uint4 v = *(const uint4*)(k + ((bn * S + s) * (long)HK + kh) * D + c * 8);
     float f[8];
     unpack8(v, f);
 #pragma unroll
@@ -388,14 +388,159 @@ attn_pool_bwd_rows(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k
   }
 }
 
-// Backward.  Block per (bn, h) (or per bn looping over heads when K is shared, so that
-// the per-head dK can be summed into head 0 without atomics).
+// Grouped query heads (K with HK = H / G heads, the model's own KV head count): one wavefront per
+// (chunk, KV head) keeps that head's K tile in registers and runs its G prior queries over it, so K
+// is read once instead of G times and nothing is repeated in memory beforehand.  Same lane layout
+// and arithmetic as the per-head kernels above.
+template <int D>
+__global__ void __launch_bounds__(256)
+attn_pool_fwd_rows_gqa(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k,
+                       bf16_t* __restrict__ lmk_k, float* __restrict__ lmk_b, float* __restrict__ p_out,
+                       int H, int HK, float sm_scale, int compact) {
+  constexpr int S = 64, LR = D / 8, TPI = 64 / LR, NI = S / TPI;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int piece = lane % LR, tsub = lane / LR;
+  const int hgroups = (HK + 3) / 4;
+  const long bn = blockIdx.x / hgroups;
+  const int kh = (int)(blockIdx.x % hgroups) * 4 + wave;
+  if (kh >= HK) return;
+  const int G = H / HK;
+  const bf16_t* kp = k + ((bn * S + tsub) * (long)HK + kh) * D + piece * 8;
+  const long step = (long)TPI * HK * D;
+  uint4 kr[NI];
+#pragma unroll
+  for (int it = 0; it < NI; ++it) kr[it] = *(const uint4*)(kp + it * step);
+  for (int g = 0; g < G; ++g) {
+    const int h = kh * G + g;
+    const uint4 mq = *(const uint4*)(mu_q + (bn * H + h) * (long)D + piece * 8);
+    float a[NI];
+    float m = HILS_NEG_INF;
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      a[it] = row_sum<LR>(dot8_bf16(mq, kr[it], 0.f)) * sm_scale;
+      if (it == NI - 1 && tsub == TPI - 1) a[it] = HILS_NEG_INF;  // the chunk's last token is never pooled
+      m = fmaxf(m, a[it]);
+    }
+    m = pool_groups_max<LR>(m);
+    float e_sum = 0.f;
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      a[it] = (a[it] == HILS_NEG_INF) ? 0.f : __expf(a[it] - m);
+      e_sum += a[it];
+    }
+    e_sum = pool_groups_sum<LR>(e_sum);
+    const float inv = e_sum > 0.f ? 1.f / e_sum : 0.f;
+    float ent = 0.f;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      const float pv = a[it] * inv;
+      if (piece == 0) p_out[(bn * S + it * TPI + tsub) * (long)H + h] = pv;
+      if (pv > 0.f) ent += pv * __logf(pv);
+      float f[8];
+      unpack8(kr[it], f);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = fmaf(pv, f[i], acc[i]);
+    }
+    ent = pool_groups_sum<LR>(ent);
+    if (lane == 0) lmk_b[bn * H + h] = -ent;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = compact ? 0.f : pool_groups_sum<LR>(acc[i]);
+    if (tsub == 0) {
+      uint4 w;
+      w.x = pack_bf2(acc[0], acc[1]);
+      w.y = pack_bf2(acc[2], acc[3]);
+      w.z = pack_bf2(acc[4], acc[5]);
+      w.w = pack_bf2(acc[6], acc[7]);
+      *(uint4*)(lmk_k + (bn * H + h) * (long)D + piece * 8) = w;
+    }
+  }
+}
+
+// Its backward: dK of a KV head is the sum over its G query heads, kept in registers (fp32) and
+// rounded once.
+template <int D>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+attn_pool_bwd_rows_gqa(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k,
+                       const float* __restrict__ p_saved, const float* __restrict__ lmk_b,
+                       const bf16_t* __restrict__ g_k, const float* __restrict__ g_b,
+                       bf16_t* __restrict__ d_mu, bf16_t* __restrict__ d_k, int H, int HK, float sm_scale,
+                       int compact) {
+  constexpr int S = 64, LR = D / 8, TPI = 64 / LR, NI = S / TPI;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int piece = lane % LR, tsub = lane / LR;
+  const int hgroups = (HK + 3) / 4;
+  const long bn = blockIdx.x / hgroups;
+  const int kh = (int)(blockIdx.x % hgroups) * 4 + wave;
+  if (kh >= HK) return;
+  const int G = H / HK;
+  const bf16_t* kp = k + ((bn * S + tsub) * (long)HK + kh) * D + piece * 8;
+  const long step = (long)TPI * HK * D;
+  uint4 kr[NI];
+#pragma unroll
+  for (int it = 0; it < NI; ++it) kr[it] = *(const uint4*)(kp + it * step);
+  float dk_acc[NI][8];
+#pragma unroll
+  for (int it = 0; it < NI; ++it)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dk_acc[it][i] = 0.f;
+  for (int g = 0; g < G; ++g) {
+    const int h = kh * G + g;
+    const uint4 mq = *(const uint4*)(mu_q + (bn * H + h) * (long)D + piece * 8);
+    uint4 gq = make_uint4(0, 0, 0, 0);
+    if (!compact) gq = *(const uint4*)(g_k + (bn * H + h) * (long)D + piece * 8);
+    const float ent = lmk_b[bn * H + h], gb = g_b[bn * H + h];
+    float pv[NI], dl[NI];
+    float part = 0.f;
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      pv[it] = p_saved[(bn * S + it * TPI + tsub) * (long)H + h];
+      dl[it] = row_sum<LR>(dot8_bf16(gq, kr[it], 0.f));
+      part += pv[it] * dl[it];
+    }
+    const float delta = pool_groups_sum<LR>(part);
+    float muf[8], gkf[8];
+    unpack8(mq, muf);
+    unpack8(gq, gkf);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      const float x = pv[it] > 0.f ? pv[it] * ((dl[it] - delta) - gb * (__logf(pv[it]) + ent)) : 0.f;
+      float f[8];
+      unpack8(kr[it], f);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        acc[i] = fmaf(x, f[i], acc[i]);
+        dk_acc[it][i] += sm_scale * x * muf[i] + pv[it] * gkf[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = pool_groups_sum<LR>(acc[i]) * sm_scale;
+    if (tsub == 0) {
+      uint4 w;
+      w.x = pack_bf2(acc[0], acc[1]); w.y = pack_bf2(acc[2], acc[3]);
+      w.z = pack_bf2(acc[4], acc[5]); w.w = pack_bf2(acc[6], acc[7]);
+      *(uint4*)(d_mu + (bn * H + h) * (long)D + piece * 8) = w;
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NI; ++it) {
+    uint4 w;
+    w.x = pack_bf2(dk_acc[it][0], dk_acc[it][1]); w.y = pack_bf2(dk_acc[it][2], dk_acc[it][3]);
+    w.z = pack_bf2(dk_acc[it][4], dk_acc[it][5]); w.w = pack_bf2(dk_acc[it][6], dk_acc[it][7]);
+    *(uint4*)(d_k + ((bn * S + it * TPI + tsub) * (long)HK + kh) * D + piece * 8) = w;
+  }
+}
+
+// Backward.  Block per (bn, h); per bn looping over all heads when K is shared, per (bn, KV head)
+// looping over its query heads when K has fewer heads than mu_q, so that the per-head dK can be
+// summed without atomics.
 __global__ void __launch_bounds__(POOL_THREADS)
 attn_pool_bwd_kernel(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k,
                      const float* __restrict__ p_saved, const float* __restrict__ lmk_b,
                      const bf16_t* __restrict__ g_k, const float* __restrict__ g_b,
                      bf16_t* __restrict__ d_mu, bf16_t* __restrict__ d_k,
-                     int S, int H, int D, float sm_scale, int compact, int shared_k) {
+                     int S, int H, int HK, int D, float sm_scale, int compact, int shared_k) {
   extern __shared__ float smem[];
   const int DP = D + 1;
   float* ks = smem;                 // S * DP
@@ -404,23 +549,25 @@ attn_pool_bwd_kernel(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__
   float* pr = gk + D;               // S
   float* dl = pr + S;               // S  (dP, then dlogits)
   float* red = dl + S;              // 32
-  float* dk_acc = red + 32;         // S * D, only when shared_k
+  float* dk_acc = red + 32;         // S * D, only when several heads share a K tile
   const long bn = blockIdx.x;
   const int tid = threadIdx.x;
   const int d8 = D / 8;
-  const int h_begin = shared_k ? 0 : blockIdx.y;
-  const int h_end = shared_k ? H : blockIdx.y + 1;
+  const int G = H / HK;             // query heads per K head (1 unless K has fewer heads)
+  const bool summed = shared_k || G > 1;
+  const int h_begin = shared_k ? 0 : blockIdx.y * G;
+  const int h_end = shared_k ? H : h_begin + G;
+  const int kh = shared_k ? 0 : blockIdx.y;
 
-  if (shared_k)
+  if (summed)
     for (int i = tid; i < S * D; i += POOL_THREADS) dk_acc[i] = 0.f;
 
   for (int h = h_begin; h < h_end; ++h) {
-    const int kh = shared_k ? 0 : h;
     __syncthreads();
-    if (!shared_k || h == 0) {
+    if (h == h_begin) {
       for (int i = tid; i < S * d8; i += POOL_THREADS) {
         const int s = i / d8, c = i - s * d8;
-        uint4 v = *(const uint4*)(k + ((bn * S + s) * (long)H + kh) * D + c * 8);
+        uint4 v = *(const uint4*)(k + ((bn * S + s) * (long)HK + kh) * D + c * 8);
         float f[8];
         unpack8(v, f);
 #pragma unroll
@@ -453,7 +600,7 @@ attn_pool_bwd_kernel(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__
       for (int s = 0; s < S; ++s) a += dl[s] * ks[s * DP + d];
       d_mu[(bn * H + h) * (long)D + d] = f2bf(a * sm_scale);
     }
-    if (shared_k) {
+    if (summed) {
       for (int i = tid; i < S * D; i += POOL_THREADS) {
         const int s = i / D, d = i - s * D;
         dk_acc[i] += sm_scale * dl[s] * mu[d] + pr[s] * gk[d];
@@ -465,12 +612,14 @@ attn_pool_bwd_kernel(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__
       }
     }
   }
-  if (shared_k) {
+  if (summed) {
     __syncthreads();
     for (int i = tid; i < S * D; i += POOL_THREADS) {
       const int s = i / D, d = i - s * D;
-      d_k[((bn * S + s) * (long)H + 0) * D + d] = f2bf(dk_acc[i]);
+      d_k[((bn * S + s) * (long)HK + kh) * D + d] = f2bf(dk_acc[i]);
     }
+  }
+  if (shared_k) {
     for (long i = tid; i < (long)S * (H - 1) * D; i += POOL_THREADS) {
       const int s = (int)(i / ((long)(H - 1) * D));
       const long r = i - (long)s * (H - 1) * D;
@@ -479,19 +628,34 @@ attn_pool_bwd_kernel(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__
   }
 }
 
-static int pool_check(const char* name, int BN, int S, int H, int D) {
+static int pool_check(const char* name, int BN, int S, int H, int HK, int D, int shared_k) {
   HILS_REQUIRE(BN > 0 && S > 1 && H > 0 && D > 0, "%s: sizes must be positive (S > 1)", name);
   HILS_REQUIRE(D % 8 == 0, "%s: D (%d) must be a multiple of 8", name, D);
   HILS_REQUIRE(H <= 65535, "%s: H (%d) too large", name, H);
+  HILS_REQUIRE(HK > 0 && H % HK == 0, "%s: the heads of mu_q (%d) must be a multiple of the heads of k (%d)", name, H, HK);
+  HILS_REQUIRE(!shared_k || HK == H, "%s: shared_k reads head 0 of a k with as many heads as mu_q (%d), got %d", name,
+               H, HK);
   return HILS_OK;
 }
 
 extern "C" int hils_attn_pool_fwd(const void* mu_q, const void* k, void* lmk_k, float* lmk_b,
-                                  float* p, int BN, int S, int H, int D, float sm_scale,
+                                  float* p, int BN, int S, int H, int h_kv, int D, float sm_scale,
                                   int compact, int shared_k, void* stream) {
   HILS_REQUIRE(mu_q && k && lmk_k && lmk_b && p, "hils_attn_pool_fwd: null pointer");
-  if (int rc = pool_check("hils_attn_pool_fwd", BN, S, H, D)) return rc;
-  if (S == 64 && (D == 64 || D == 128) && (long)BN * ((H + 3) / 4) <= 2147483647L) {
+  if (int rc = pool_check("hils_attn_pool_fwd", BN, S, H, h_kv, D, shared_k)) return rc;
+  const int HK = h_kv;
+  if (S == 64 && (D == 64 || D == 128) && HK < H && (long)BN * ((HK + 3) / 4) <= 2147483647L) {
+    const dim3 grid((unsigned)((long)BN * ((HK + 3) / 4)));
+    if (D == 64)
+      hipLaunchKernelGGL(attn_pool_fwd_rows_gqa<64>, grid, dim3(256), 0, (hipStream_t)stream,
+                         (const bf16_t*)mu_q, (const bf16_t*)k, (bf16_t*)lmk_k, lmk_b, p, H, HK, sm_scale, compact);
+    else
+      hipLaunchKernelGGL(attn_pool_fwd_rows_gqa<128>, grid, dim3(256), 0, (hipStream_t)stream,
+                         (const bf16_t*)mu_q, (const bf16_t*)k, (bf16_t*)lmk_k, lmk_b, p, H, HK, sm_scale, compact);
+    HILS_CHECK_LAUNCH("hils_attn_pool_fwd");
+    return HILS_OK;
+  }
+  if (S == 64 && (D == 64 || D == 128) && HK == H && (long)BN * ((H + 3) / 4) <= 2147483647L) {
     const dim3 grid((unsigned)((long)BN * ((H + 3) / 4)));
     if (D == 64)
       hipLaunchKernelGGL(attn_pool_fwd_rows<64>, grid, dim3(256), 0, (hipStream_t)stream,
@@ -511,18 +675,32 @@ extern "C" int hils_attn_pool_fwd(const void* mu_q, const void* k, void* lmk_k, 
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   hipLaunchKernelGGL(attn_pool_fwd_kernel, dim3(BN, H), dim3(POOL_THREADS), smem,
                      (hipStream_t)stream, (const bf16_t*)mu_q, (const bf16_t*)k, (bf16_t*)lmk_k,
-                     lmk_b, p, S, H, D, sm_scale, compact, shared_k);
+                     lmk_b, p, S, H, HK, D, sm_scale, compact, shared_k);
   HILS_CHECK_LAUNCH("hils_attn_pool_fwd");
   return HILS_OK;
 }
 
 extern "C" int hils_attn_pool_bwd(const void* mu_q, const void* k, const float* p,
                                   const float* lmk_b, const void* g_k, const float* g_b,
-                                  void* d_mu, void* d_k, int BN, int S, int H, int D,
+                                  void* d_mu, void* d_k, int BN, int S, int H, int h_kv, int D,
                                   float sm_scale, int compact, int shared_k, void* stream) {
   HILS_REQUIRE(mu_q && k && p && lmk_b && g_k && g_b && d_mu && d_k, "hils_attn_pool_bwd: null pointer");
-  if (int rc = pool_check("hils_attn_pool_bwd", BN, S, H, D)) return rc;
-  if (S == 64 && (D == 64 || D == 128) && (long)BN * ((H + 3) / 4) <= 2147483647L) {
+  if (int rc = pool_check("hils_attn_pool_bwd", BN, S, H, h_kv, D, shared_k)) return rc;
+  const int HK = h_kv;
+  if (S == 64 && (D == 64 || D == 128) && HK < H && (long)BN * ((HK + 3) / 4) <= 2147483647L) {
+    const dim3 grid((unsigned)((long)BN * ((HK + 3) / 4)));
+    if (D == 64)
+      hipLaunchKernelGGL(attn_pool_bwd_rows_gqa<64>, grid, dim3(256), 0, (hipStream_t)stream,
+                         (const bf16_t*)mu_q, (const bf16_t*)k, p, lmk_b, (const bf16_t*)g_k, g_b,
+                         (bf16_t*)d_mu, (bf16_t*)d_k, H, HK, sm_scale, compact);
+    else
+      hipLaunchKernelGGL(attn_pool_bwd_rows_gqa<128>, grid, dim3(256), 0, (hipStream_t)stream,
+                         (const bf16_t*)mu_q, (const bf16_t*)k, p, lmk_b, (const bf16_t*)g_k, g_b,
+                         (bf16_t*)d_mu, (bf16_t*)d_k, H, HK, sm_scale, compact);
+    HILS_CHECK_LAUNCH("hils_attn_pool_bwd");
+    return HILS_OK;
+  }
+  if (S == 64 && (D == 64 || D == 128) && HK == H && (long)BN * ((H + 3) / 4) <= 2147483647L) {
     const dim3 grid((unsigned)((long)BN * (shared_k ? 1 : (H + 3) / 4)));
     const size_t xch = shared_k ? (size_t)2 * S * D * sizeof(float) : 0;
 #define POOL_BWD_ROWS(D_, SH_)                                                                      \
@@ -538,15 +716,16 @@ extern "C" int hils_attn_pool_bwd(const void* mu_q, const void* k, const float* 
     HILS_CHECK_LAUNCH("hils_attn_pool_bwd");
     return HILS_OK;
   }
-  size_t smem = ((size_t)S * (D + 1) + 2 * D + 2 * S + 32 + (shared_k ? (size_t)S * D : 0)) * sizeof(float);
+  const bool summed = shared_k || HK < H;
+  size_t smem = ((size_t)S * (D + 1) + 2 * D + 2 * S + 32 + (summed ? (size_t)S * D : 0)) * sizeof(float);
   HILS_REQUIRE(smem <= 160 * 1024, "hils_attn_pool_bwd: S*D (%d x %d) tile does not fit in LDS", S, D);
   if (smem > 64 * 1024)
     (void)hipFuncSetAttribute((const void*)attn_pool_bwd_kernel,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  dim3 grid(BN, shared_k ? 1 : H);
+  dim3 grid(BN, shared_k ? 1 : HK);
   hipLaunchKernelGGL(attn_pool_bwd_kernel, grid, dim3(POOL_THREADS), smem, (hipStream_t)stream,
                      (const bf16_t*)mu_q, (const bf16_t*)k, p, lmk_b, (const bf16_t*)g_k, g_b,
-                     (bf16_t*)d_mu, (bf16_t*)d_k, S, H, D, sm_scale, compact, shared_k);
+                     (bf16_t*)d_mu, (bf16_t*)d_k, S, H, HK, D, sm_scale, compact, shared_k);
   HILS_CHECK_LAUNCH("hils_attn_pool_bwd");
   return HILS_OK;
 }

@@ -20,8 +20,8 @@ _P, _I, _F, _Z = c_void_p, c_int, c_float, ctypes.c_size_t
 SIGNATURES = {
     "hils_mean_pool_fwd": [_P, _P, _I, _I, _I, _I, _I, _P],
     "hils_mean_pool_bwd": [_P, _P, _I, _I, _I, _I, _I, _P],
-    "hils_attn_pool_fwd": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
-    "hils_attn_pool_bwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
+    "hils_attn_pool_fwd": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "hils_attn_pool_bwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "hils_topk_fwd": [_P] * 11 + [_Z] + [_I] * 12 + [_F, _P],
     "hils_topk_fwd_noalloc": [_P] * 10 + [_I] * 12 + [_F, _P],
     "hils_topk_fwd_weights": [_P] * 11 + [_Z] + [_I] * 12 + [_F, _P],

@@ -23,13 +23,13 @@ import torch
 
 try:  # imported as part of the package ...
     from ..ops import _cabi
-    from ..ops.chunk_attn_pool_tilelang import chunk_attn_pool_tilelang, chunk_mean_pool
+    from ..ops.chunk_attn_pool_tilelang import chunk_attn_pool, chunk_mean_pool
     from ..ops.hils_fwd_bwd_head import HiLS_block_M_head
     from ..ops.hils_glue import chunk_weights, decode_step, topk_chunk_weights
     from ..ops.topk_head_softmax import online_softmax_topk_head
 except ImportError:  # ... or with the package directory itself on sys.path (`from utils... import`)
     from ops import _cabi
-    from ops.chunk_attn_pool_tilelang import chunk_attn_pool_tilelang, chunk_mean_pool
+    from ops.chunk_attn_pool_tilelang import chunk_attn_pool, chunk_mean_pool
     from ops.hils_fwd_bwd_head import HiLS_block_M_head
     from ops.hils_glue import chunk_weights, decode_step, topk_chunk_weights
     from ops.topk_head_softmax import online_softmax_topk_head
@@ -41,12 +41,10 @@ _OFFLOAD_HIDDEN_DIM_THRESHOLD = 4096
 
 def _attention_pooled(mu_q, k_chunks, num_kv_heads):
     """Prior queries mu_q (B,n,h_q,D) over the chunks k_chunks (B,n,S,H,D): attention-pooled keys
-    (B,n,h_q,D) and entropy bias (B,n,h_q) fp32 (models/FlashHiLS/hils_attention.py:66-135: K is
-    repeated to the query heads)."""
-    h_q = mu_q.shape[2]
-    G = h_q // num_kv_heads
-    kc = k_chunks if G == 1 else k_chunks.repeat_interleave(G, dim=3)
-    lk, lb = chunk_attn_pool_tilelang(mu_q.contiguous(), kc.contiguous())
+    (B,n,h_q,D) and entropy bias (B,n,h_q) fp32 (models/FlashHiLS/hils_attention.py:66-135; K stays
+    at its own head count)."""
+    assert k_chunks.shape[3] == num_kv_heads
+    lk, lb = chunk_attn_pool(mu_q.contiguous(), k_chunks.contiguous())
     return lk, lb.float()
 
 

@@ -31,20 +31,23 @@ int hils_mean_pool_bwd(const void* g_lmk, void* dk, int B, int L, int H, int D, 
 
 /* Attention pool forward.  Replaces chunk_attn_pool_fwd_kernel_fallback /
  * chunk_attn_pool_fwd_kernel behind ChunkAttnPoolFunction.forward
- * (ops/chunk_attn_pool_tilelang.py:329-410, :31-150, :540-570).
- * mu_q (BN,H,D) bf16, k (BN,S,H,D) bf16 -> lmk_k (BN,H,D) bf16, lmk_b (BN,H) fp32,
- * p (BN,S,H) fp32 (saved for backward).  compact != 0: lmk_k is written as zeros.
- * shared_k != 0: K is read from head 0 for every head. */
+ * (ops/chunk_attn_pool_tilelang.py:329-410, :31-150, :540-570), and the K head repeat in front of it
+ * (models/FlashHiLS/hils_attention.py:20-50, :339, :391: `_repeat_k_heads_for_gqa`).
+ * mu_q (BN,H,D) bf16, k (BN,S,h_kv,D) bf16 -> lmk_k (BN,H,D) bf16, lmk_b (BN,H) fp32,
+ * p (BN,S,H) fp32 (saved for backward).  H % h_kv == 0: query head h reads K head h / (H / h_kv)
+ * (h_kv == H: a K tile per head, the reference kernels' layout).  compact != 0: lmk_k is written as
+ * zeros.  shared_k != 0 (needs h_kv == H): K is read from head 0 for every head. */
 int hils_attn_pool_fwd(const void* mu_q, const void* k, void* lmk_k, float* lmk_b, float* p,
-                       int BN, int S, int H, int D, float sm_scale, int compact, int shared_k,
+                       int BN, int S, int H, int h_kv, int D, float sm_scale, int compact, int shared_k,
                        void* stream);
 /* Attention pool backward.  Replaces chunk_attn_pool_bwd_kernel_fallback /
  * chunk_attn_pool_bwd_kernel (ops/chunk_attn_pool_tilelang.py:425-533, :165-314).
- * g_k (BN,H,D) bf16, g_b (BN,H) fp32 -> d_mu (BN,H,D) bf16, d_k (BN,S,H,D) bf16.
+ * g_k (BN,H,D) bf16, g_b (BN,H) fp32 -> d_mu (BN,H,D) bf16, d_k (BN,S,h_kv,D) bf16 (h_kv < H: the sum
+ * over the H / h_kv query heads of a K head, accumulated in fp32 and rounded once).
  * shared_k != 0: d_k is summed over heads into head 0 and heads 1.. are zero. */
 int hils_attn_pool_bwd(const void* mu_q, const void* k, const float* p, const float* lmk_b,
                        const void* g_k, const float* g_b, void* d_mu, void* d_k,
-                       int BN, int S, int H, int D, float sm_scale, int compact, int shared_k,
+                       int BN, int S, int H, int h_kv, int D, float sm_scale, int compact, int shared_k,
                        void* stream);
 
 /* ---- top-k chunk selection -------------------------------------------------- */

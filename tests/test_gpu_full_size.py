@@ -71,6 +71,12 @@ def test_prefill_32k_properties(pkg, orc, dev, recipe):
     # ---- inter-chunk softmax + sparse attention ----
     w = pkg.chunk_weights(scores, lse_swa)
     assert (w.float().sum(-1) - 1).abs().max().item() < 2e-2
+    # the call the benchmark times (selection + weights in one call; with the benchmark's inputs lse_swa
+    # is bf16 and the launches are the variants that read it as bf16): same indices, scores and weights
+    idx_f, scores_f, w_f = pkg.topk_chunk_weights(q, lmk, lse_swa, K, S, W)
+    assert torch.equal(idx_f, idx) and torch.equal(scores_f, scores)
+    assert torch.equal(w_f, w), "fused weights differ from chunk_weights on the same scores"
+    del idx_f, scores_f, w_f
     o = pkg.HiLS_block_M_head(q, k, v, w, idx, block_size=S, is_training=False)
     tq = torch.tensor([0, 63, 64, 65, 127, 128, 129, 1000, 4095, 4096, 20000, L - 1])
     tq = torch.cat([tq, torch.randint(0, L, (20,), generator=torch.Generator().manual_seed(2))])
@@ -147,6 +153,43 @@ def test_decode_128k_properties(pkg, orc, dev):
     w_p = torch.cat([w[..., :K][..., perm], w[..., K:]], -1).contiguous()
     o_p = pkg.HiLS_block_M_head(q, kc, vc, w_p, idx[..., perm].contiguous(), block_size=S, is_training=False)
     assert (o_p.float() - o.float()).abs().max().item() <= 1e-2
+    del o_a, o_b, o_p, w_p, w_zero, drop
+    # ---- the one-launch step (what the benchmark's decode figure times) on the same cache ----
+    dbg1 = {}
+    o1, w1, idx1, sc1 = pkg.decode_step(q, lmk, kc, vc, lse_swa, K, S, W, q_offset=Lkv - 1, _debug=dbg1)
+    assert dbg1, "the one-launch kernel did not take the headline shape"
+    want1 = orc.topk_select(dbg1["sel_logits"].cpu(), dbg1["lse_total"].cpu(), lim.cpu(), K)
+    assert torch.equal(idx1.cpu(), want1), "one-launch selection differs from the rule on its own logits"
+    assert torch.equal(idx1, idx) and torch.equal(sc1, scores) and torch.equal(w1, w)
+    assert_close_bf16(o1, o.float(), "one launch vs two calls")
+    for b in bs:
+        ref = orc.sparse_attn(q[b:b + 1].cpu(), kc[b:b + 1].cpu(), vc[b:b + 1].cpu(), w1[b:b + 1].cpu(),
+                              idx1[b:b + 1].cpu(), chunk_size=S)
+        assert_close_bf16(o1[b:b + 1], ref, f"one-launch decode, batch element {b}")
+    # chunk keys head-major (the layout this package's cache layers keep): other addresses, same arithmetic
+    lmk_hm = pkg.head_major_chunk_keys(lmk)
+    o2, w2, idx2, sc2 = pkg.decode_step(q, lmk_hm, kc, vc, lse_swa, K, S, W, q_offset=Lkv - 1, lmk_head_major=True)
+    assert torch.equal(idx2, idx1) and torch.equal(sc2, sc1) and torch.equal(w2, w1) and torch.equal(o2, o1)
+    del o2, w2, idx2, sc2, dbg1
+    # ---- the same cache in pages handed out in random order ----
+    num_pages = B * N + 7
+    perm = torch.randperm(num_pages, device=dev, generator=gen)[: B * N].view(B, N)
+    k_pages = torch.empty(num_pages, H, S, D, dtype=torch.bfloat16, device=dev).normal_(generator=gen)
+    v_pages = torch.empty(num_pages, H, S, D, dtype=torch.bfloat16, device=dev).normal_(generator=gen)
+    lmk_pages = torch.empty(num_pages, H, D, dtype=torch.bfloat16, device=dev).normal_(generator=gen)
+    k_pages[perm] = kc.view(B, N, S, H, D).permute(0, 1, 3, 2, 4)
+    v_pages[perm] = vc.view(B, N, S, H, D).permute(0, 1, 3, 2, 4)
+    lmk_pages[perm] = lmk
+    table = torch.full((B, N + 3), -1, dtype=torch.int32, device=dev)
+    table[:, :N] = perm.to(torch.int32)
+    dbgp = {}
+    o3, w3, idx3 = pkg.paged_hils_attend(q, k_pages, v_pages, lmk_pages, table, lse_swa, Lkv, K, W, _debug=dbgp)
+    wantp = orc.topk_select(dbgp["sel_logits"].cpu(), dbgp["lse_total"].cpu(), lim.cpu(), K)
+    assert torch.equal(idx3.cpu(), wantp), "paged selection differs from the rule on its own logits"
+    assert torch.equal(idx3, idx1) and torch.equal(dbgp["scores"], sc1) and torch.equal(w3, w1)
+    assert torch.equal(o3, o1), "paged output differs from the token-major cache's"
+    o4, w4, idx4 = pkg.paged_hils_attend(q, k_pages, v_pages, None, table, lse_swa, Lkv, K, W, lmk_dense=lmk_hm)
+    assert torch.equal(idx4, idx1) and torch.equal(w4, w1) and torch.equal(o4, o1)
 
 
 def _sampled_queries(L, n, seed):

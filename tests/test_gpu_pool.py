@@ -134,6 +134,50 @@ def test_attn_pool_shared_k(pkg, orc, dev):
         pkg.chunk_attn_pool_tilelang_shared_k(mu_d[:, :, :8], k_d[:, :, :, :8])
 
 
+@pytest.mark.parametrize("B,N,H,HK,D,S", [(1, 40, 32, 8, 128, 64), (2, 9, 8, 2, 64, 64), (1, 5, 6, 3, 128, 64),
+                                           (1, 7, 16, 1, 64, 64),
+                                           # other chunk sizes / head dims: the kernels that stage K in LDS
+                                           (1, 6, 8, 2, 128, 32), (2, 3, 4, 2, 32, 16)])
+def test_attn_pool_grouped_query_heads(pkg, orc, dev, B, N, H, HK, D, S):
+    """K at the model's own KV head count (models/FlashHiLS/hils_attention.py:66-135): forward and
+    backward equal the oracle on K repeated to the query heads, dK being the sum over a group."""
+    note(f"attn_pool grouped B{B} N{N} H{H}/{HK} D{D} S{S}")
+    torch.manual_seed(43)
+    G = H // HK
+    mu = torch.randn(B, N, H, D).bfloat16()
+    k = torch.randn(B, N, S, HK, D).bfloat16()
+    gk = torch.randn(B, N, H, D).bfloat16()
+    gb = torch.randn(B, N, H)
+    mu_d = mu.to(dev).requires_grad_()
+    k_d = k.to(dev).requires_grad_()
+    lk, lb = pkg.chunk_attn_pool(mu_d, k_d)
+    k_rep = k.repeat_interleave(G, dim=3)
+    rk_, rb_, _ = orc.chunk_attn_pool(mu, k_rep)
+    assert lk.shape == (B, N, H, D) and lb.shape == (B, N, H) and lb.dtype == torch.float32
+    assert_close_bf16(lk, rk_, "grouped lmk_k")
+    assert_close_f32(lb, rb_, 1e-4, "grouped lmk_b")
+    # the same numbers as the per-head kernels on the repeated K (same arithmetic, K read once)
+    lk2, lb2 = pkg.chunk_attn_pool_tilelang(mu.to(dev), k_rep.to(dev))
+    assert torch.equal(lk2, lk) and torch.equal(lb2, lb)
+    torch.autograd.backward([lk, lb], [gk.to(dev), gb.to(dev)])
+    rmu, rk = _pool_grads(orc, mu, k_rep, gk, gb)
+    assert_close_bf16(mu_d.grad, rmu, "grouped d_mu")
+    assert k_d.grad.shape == k.shape
+    assert_close_bf16(k_d.grad, rk.view(B, N, S, HK, G, D).sum(4), "grouped d_k")
+
+
+def test_attn_pool_argument_errors(pkg, dev):
+    """The wrapper's own argument checks (models/FlashHiLS/hils_attention.py:113-131)."""
+    mu = torch.randn(1, 4, 6, 64, device=dev).bfloat16()
+    k = torch.randn(1, 4, 64, 4, 64, device=dev).bfloat16()
+    with pytest.raises(ValueError, match="multiple"):
+        pkg.chunk_attn_pool(mu, k)
+    with pytest.raises(ValueError, match="expected mu_q"):
+        pkg.chunk_attn_pool(mu[0], k)
+    with pytest.raises(ValueError, match="mismatch"):
+        pkg.chunk_attn_pool(mu[:, :3], k[:, :, :, :3])
+
+
 @pytest.mark.parametrize("B,L,H,D,S", [(1, 2048, 4, 64, 64), (2, 1024, 8, 128, 64), (1, 256, 2, 64, 32),
                                         (1, 128, 1, 8, 16)])
 def test_mean_pool(pkg, orc, dev, B, L, H, D, S):

@@ -73,6 +73,19 @@ def test_swa_landmark_query_row_sees_no_key(pkg, dev):
     (1, 513, 4, 4, 128, 64, 1, 64, False, False)])
 def test_swa_backward(pkg, orc, dev, B, L, HQ, H, D, Dv, W, S, mask_lmk, expand):
     """dq, dk, dv with gradients arriving through both outputs (o and lse)."""
+    _forward_backward(pkg, orc, dev, B, L, HQ, H, D, Dv, W, S, mask_lmk, expand)
+
+
+@pytest.mark.parametrize("HQ,H,D", [(16, 2, 64), (8, 8, 128)])
+@pytest.mark.parametrize("W", [256, 512])
+def test_swa_long_windows_forward_backward(pkg, orc, dev, HQ, H, D, W):
+    """Windows of several key tiles on a sequence of many query blocks: the windows and head shapes the
+    reference times this operator at (scripts/bench/bench_flex_attn_bwd_clamp.py:66-72), forward and
+    backward against the oracle."""
+    _forward_backward(pkg, orc, dev, 1, 2048, HQ, H, D, D, W, 64, True, True)
+
+
+def _forward_backward(pkg, orc, dev, B, L, HQ, H, D, Dv, W, S, mask_lmk, expand):
     note(f"swa_bwd B{B} L{L} HQ{HQ} H{H} D{D} Dv{Dv} W{W} S{S} lmk{mask_lmk} exp{expand}")
     gen = torch.Generator().manual_seed(7)
     q = torch.randn(B, L, HQ, D, generator=gen).bfloat16()
@@ -88,6 +101,8 @@ def test_swa_backward(pkg, orc, dev, B, L, HQ, H, D, Dv, W, S, mask_lmk, expand)
     ro, rlse = orc.swa(qf, kf, vf, window_size=W, chunk_size=S, mask_lmk=mask_lmk, expand_to_chunk=expand)
     rfin = torch.isfinite(rlse)
     assert torch.equal(fin.cpu(), rfin)
+    assert_close_bf16(o, ro.detach(), "swa o")
+    assert_close_f32(lse.detach(), rlse.detach(), LSE_TOL, "swa lse")
     ((ro * do.float()).sum() + torch.where(rfin, rlse, torch.zeros_like(rlse)).mul(dl).sum()).backward()
     assert_close_bf16(qd.grad, qf.grad, "swa dq")
     assert_close_bf16(kd.grad, kf.grad, "swa dk")
