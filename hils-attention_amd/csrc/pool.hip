@@ -457,10 +457,156 @@ attn_pool_fwd_rows_gqa(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict
   }
 }
 
+// The same forward with the logits on the matrix cores, for G <= 16.  A wavefront takes a (chunk, KV
+// head) tile; its K (read once, coalesced, into registers for the weighted sum) is also laid in
+// the wavefront's LDS and read back as the A operand of S^T = K mu^T (tokens x heads, the G heads
+// padded to 16 columns); a lane then holds 16 tokens of one head's column, so the softmax of all
+// heads runs at once, and P goes back through LDS (over the K tile, no longer needed there) to the
+// lanes that hold the token rows.  The vector ALU is left with the weighted sum.
+// (Tried and slower at 512 chunks x 8 KV heads, D = 128, where this takes 22.5 us: K read straight into
+// A-operand order instead of through LDS, 24.6 us; wavefronts that walk two tiles and touch the next
+// tile's lines ahead of the arithmetic, 25.5 us.)
+template <int D>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+attn_pool_fwd_gqa_mfma(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k,
+                       bf16_t* __restrict__ lmk_k, float* __restrict__ lmk_b, float* __restrict__ p_out,
+                       long tiles, int H, int HK, float sm_scale, int compact) {
+  constexpr int S = 64, LR = D / 8, TPI = 64 / LR, NI = S / TPI, KS = D / 32;
+  constexpr int PITCH = D * 2 + 16;  // bytes of a token row in LDS: 16-byte reads of 16 rows spread over the banks
+  static_assert(S * PITCH >= 16 * S * 4, "P of 16 heads fits over the K tile");
+  extern __shared__ __align__(16) unsigned char pool_lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int piece = lane % LR, tsub = lane / LR;
+  const int col = lane & 15, j = lane >> 4;
+  const int G = H / HK;
+  unsigned char* kl = pool_lds + (size_t)wave * (S * PITCH);
+  float* ps = (float*)kl;  // P, [head][token % TPI][token / TPI], once S is formed
+  const long step = (long)TPI * HK * D;
+  // tile = chunk * HK + KV head: neighbouring wavefronts read neighbouring pieces of the same token rows
+  auto load = [&](uint4 (&kr)[NI], long tile) {
+    const bf16_t* kp = k + (tile / HK * S + tsub) * (long)HK * D + (tile % HK) * (long)D + piece * 8;
+#pragma unroll
+    for (int it = 0; it < NI; ++it) kr[it] = *(const uint4*)(kp + it * step);
+  };
+  auto process = [&](const uint4 (&kr)[NI], long tile) {
+    const long bn = tile / HK;
+    const int kh = (int)(tile - bn * HK);
+    // B operand: column `col` is head kh * G + col (zero past G), lane group j holds k = 8j .. 8j+7 of a step
+    bf16x8_t mub[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (col < G) v = *(const uint4*)(mu_q + (bn * H + kh * G + col) * (long)D + ks * 32 + j * 8);
+      mub[ks] = *(bf16x8_t*)&v;
+    }
+#pragma unroll
+    for (int it = 0; it < NI; ++it) *(uint4*)(kl + (it * TPI + tsub) * PITCH + piece * 16) = kr[it];
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_wave_barrier();
+    f32x4_t st[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      st[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const uint4 a = *(const uint4*)(kl + (mt * 16 + col) * PITCH + ks * 64 + j * 16);
+        st[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8_t*)&a, mub[ks], st[mt], 0, 0, 0);
+      }
+    }
+    // st[mt][i] = <K[token mt*16 + 4j + i], mu[head col]>: softmax over the tokens of a column
+    float m = HILS_NEG_INF;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float x = st[mt][i] * sm_scale;
+        if (mt == 3 && i == 3 && j == 3) x = HILS_NEG_INF;  // the chunk's last token is never pooled
+        st[mt][i] = x;
+        m = fmaxf(m, x);
+      }
+    m = rows_max(m);
+    float e_sum = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float e = (st[mt][i] == HILS_NEG_INF) ? 0.f : __expf(st[mt][i] - m);
+        st[mt][i] = e;
+        e_sum += e;
+      }
+    e_sum = rows_sum(e_sum);
+    const float inv = e_sum > 0.f ? 1.f / e_sum : 0.f;
+    const int h = kh * G + col;  // (a head only where col < G)
+    float ent = 0.f;
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_wave_barrier();  // every lane's reads of the K tile are issued: P may overwrite it
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = st[mt][i] * inv;
+        const int t = mt * 16 + 4 * j + i;
+        if (col < G) p_out[(bn * S + t) * (long)H + h] = pv;
+        if (pv > 0.f) ent += pv * __logf(pv);
+        ps[col * S + (t % TPI) * NI + t / TPI] = pv;  // columns past G hold the softmax of zeros: finite, unused
+      }
+    ent = rows_sum(ent);
+    if (col < G && j == 0) lmk_b[bn * H + h] = -ent;
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_wave_barrier();
+    // lmk_k = P K, four heads at a time over the token rows in registers
+    for (int g0 = 0; g0 < G; g0 += 4) {
+      float acc[4][8];
+#pragma unroll
+      for (int gg = 0; gg < 4; ++gg)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[gg][i] = 0.f;
+      if (!compact) {
+#pragma unroll
+        for (int i4 = 0; i4 < NI; i4 += 4) {
+          __builtin_amdgcn_sched_barrier(0);  // (keeps the unpacked rows of later steps out of the registers of this one)
+          float4 pq[4];
+#pragma unroll
+          for (int gg = 0; gg < 4; ++gg) pq[gg] = *(const float4*)(ps + (g0 + gg) * S + tsub * NI + i4);  // g0 + gg < 16
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float f[8];
+            unpack8(kr[i4 + e], f);
+#pragma unroll
+            for (int gg = 0; gg < 4; ++gg) {
+              const float pv = e == 0 ? pq[gg].x : (e == 1 ? pq[gg].y : (e == 2 ? pq[gg].z : pq[gg].w));
+#pragma unroll
+              for (int i = 0; i < 8; ++i) acc[gg][i] = fmaf(pv, f[i], acc[gg][i]);
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int gg = 0; gg < 4; ++gg) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[gg][i] = pool_groups_sum<LR>(acc[gg][i]);
+        if (tsub == 0 && g0 + gg < G) {
+          uint4 w;
+          w.x = pack_bf2(acc[gg][0], acc[gg][1]);
+          w.y = pack_bf2(acc[gg][2], acc[gg][3]);
+          w.z = pack_bf2(acc[gg][4], acc[gg][5]);
+          w.w = pack_bf2(acc[gg][6], acc[gg][7]);
+          *(uint4*)(lmk_k + (bn * H + kh * G + g0 + gg) * (long)D + piece * 8) = w;
+        }
+      }
+    }
+  };
+  const long tile = (long)blockIdx.x * 4 + wave;
+  if (tile >= tiles) return;  // (the wavefronts of a workgroup never synchronise)
+  uint4 kr[NI];
+  load(kr, tile);
+  process(kr, tile);
+}
+
 // Its backward: dK of a KV head is the sum over its G query heads, kept in registers (fp32) and
 // rounded once.
 template <int D>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D > 64 ? 1 : 2)))
 attn_pool_bwd_rows_gqa(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict__ k,
                        const float* __restrict__ p_saved, const float* __restrict__ lmk_b,
                        const bf16_t* __restrict__ g_k, const float* __restrict__ g_b,
@@ -644,7 +790,27 @@ extern "C" int hils_attn_pool_fwd(const void* mu_q, const void* k, void* lmk_k, 
   HILS_REQUIRE(mu_q && k && lmk_k && lmk_b && p, "hils_attn_pool_fwd: null pointer");
   if (int rc = pool_check("hils_attn_pool_fwd", BN, S, H, h_kv, D, shared_k)) return rc;
   const int HK = h_kv;
-  if (S == 64 && (D == 64 || D == 128) && HK < H && (long)BN * ((HK + 3) / 4) <= 2147483647L) {
+  if (S == 64 && (D == 64 || D == 128) && HK < H && H / HK <= 16) {
+    const long tiles = (long)BN * HK;
+    const long nblk = (tiles + 3) / 4;
+    HILS_REQUIRE(nblk <= 2147483647L, "hils_attn_pool_fwd: grid too large");
+    const dim3 grid((unsigned)nblk);
+    const size_t smem = (size_t)4 * S * (D * 2 + 16);  // a padded K tile per wavefront
+    if (D == 64) {
+      static HilsLdsReserve reserved;
+      if (int rc = hils_reserve_lds(&reserved, (const void*)attn_pool_fwd_gqa_mfma<64>, smem, "hils_attn_pool_fwd")) return rc;
+      hipLaunchKernelGGL(attn_pool_fwd_gqa_mfma<64>, grid, dim3(256), smem, (hipStream_t)stream,
+                         (const bf16_t*)mu_q, (const bf16_t*)k, (bf16_t*)lmk_k, lmk_b, p, tiles, H, HK, sm_scale, compact);
+    } else {
+      static HilsLdsReserve reserved;
+      if (int rc = hils_reserve_lds(&reserved, (const void*)attn_pool_fwd_gqa_mfma<128>, smem, "hils_attn_pool_fwd")) return rc;
+      hipLaunchKernelGGL(attn_pool_fwd_gqa_mfma<128>, grid, dim3(256), smem, (hipStream_t)stream,
+                         (const bf16_t*)mu_q, (const bf16_t*)k, (bf16_t*)lmk_k, lmk_b, p, tiles, H, HK, sm_scale, compact);
+    }
+    HILS_CHECK_LAUNCH("hils_attn_pool_fwd");
+    return HILS_OK;
+  }
+  if (S == 64 && (D == 64 || D == 128) && HK < H && (long)BN * ((HK + 3) / 4) <= 2147483647L) {  // more than 16 heads a group
     const dim3 grid((unsigned)((long)BN * ((HK + 3) / 4)));
     if (D == 64)
       hipLaunchKernelGGL(attn_pool_fwd_rows_gqa<64>, grid, dim3(256), 0, (hipStream_t)stream,

@@ -150,6 +150,10 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   __shared__ uint32_t words_w[TG_WAVES][4][16], wbase_w[TG_WAVES][4][16];  // winner map of a query and its word prefix counts
   __shared__ __align__(16) int stage_i_w[TG_WAVES][NQ * 32];               // winners' chunk indices, [query][slot]
   __shared__ __align__(16) bf16_t stage_s_w[TG_WAVES][NQ * GMAX * 32];  // their raw scores, [query][slot][head]
+  // the bias of this (batch, KV head): [chunk][head, padded to 4] fp32, a copy per wavefront (they never
+  // synchronise); read back 16 bytes per lane right where a block's logits are formed, instead of
+  // global loads whose latency the compiler covers with registers this kernel does not have
+  __shared__ __align__(16) float bias_w[BIAS ? TG_WAVES : 1][BIAS ? NB * 16 : 1][4];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   uint32_t (*cand)[TG_CAND] = cand_w[wave];
@@ -228,20 +232,27 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   };
   // bias (B, N, h_kv, G) fp32: the G values of a (chunk, KV head) are contiguous; accumulator row
   // 4j+i is head (4j+i) % GMAX
-  const float* bias_u = BIAS ? bias + (b * N * (long)h_kv + hk) * G : nullptr;
-  auto bias_of = [&](int c, float (&bv)[4]) {
-    const float* bp = bias_u + (long)(c < N ? c : N - 1) * h_kv * G;
+  float (*bias_s)[4] = bias_w[BIAS ? wave : 0];
+  if constexpr (BIAS) {
+    const float* bias_u = bias + (b * N * (long)h_kv + hk) * G;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) bv[i] = 0.f;
-    if constexpr (GMAX == 1) {
-      const float v0 = bp[0];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) bv[i] = v0;
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (i % GMAX < G) bv[i] = bp[i % GMAX];
+    for (int c = lane; c < NB * 16; c += 64) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);  // chunks past N (never visible) and heads past G: 0
+      if (c < N) {
+        const float* bp = bias_u + (long)c * h_kv * G;
+        v.x = bp[0];
+        if (GMAX > 1 && G > 1) v.y = bp[1];
+        if (GMAX > 2 && G > 2) v.z = bp[2];
+        if (GMAX > 2 && G > 3) v.w = bp[3];
+      }
+      *(float4*)bias_s[c] = v;
     }
+  }
+  auto bias_of = [&](int c, float (&bv)[4]) {  // c < 16 * NB
+    const float4 v = *(const float4*)bias_s[c];
+    const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) bv[i] = e[i % GMAX];
   };
   auto use_group = [&](int g0, const tg_u32x4 (&src)[PB][KS]) {
 #pragma unroll
@@ -260,6 +271,9 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
         if constexpr (BIAS) v = __fadd_rn(v, bv[i]);
         if (nt >= NMASK) v = (c < lim[i]) ? v : HILS_NEG_INF;
         x[nt][i] = v;
+        // (pinned here: left alone the compiler forms some of these sums only where they are used and
+        // keeps product and bias alive in their place, which this kernel has no registers for)
+        if constexpr (BIAS) asm volatile("" : "+v"(x[nt][i]));
       }
       if (EXPORT) {
         if (sel_logits_out && c < N) {

@@ -135,7 +135,7 @@ def test_attn_pool_shared_k(pkg, orc, dev):
 
 
 @pytest.mark.parametrize("B,N,H,HK,D,S", [(1, 40, 32, 8, 128, 64), (2, 9, 8, 2, 64, 64), (1, 5, 6, 3, 128, 64),
-                                           (1, 7, 16, 1, 64, 64),
+                                           (1, 7, 16, 1, 64, 64), (1, 3, 32, 1, 128, 64),
                                            # other chunk sizes / head dims: the kernels that stage K in LDS
                                            (1, 6, 8, 2, 128, 32), (2, 3, 4, 2, 32, 16)])
 def test_attn_pool_grouped_query_heads(pkg, orc, dev, B, N, H, HK, D, S):
@@ -156,9 +156,10 @@ def test_attn_pool_grouped_query_heads(pkg, orc, dev, B, N, H, HK, D, S):
     assert lk.shape == (B, N, H, D) and lb.shape == (B, N, H) and lb.dtype == torch.float32
     assert_close_bf16(lk, rk_, "grouped lmk_k")
     assert_close_f32(lb, rb_, 1e-4, "grouped lmk_b")
-    # the same numbers as the per-head kernels on the repeated K (same arithmetic, K read once)
+    # and the per-head kernels on the repeated K (the logits are summed in another order)
     lk2, lb2 = pkg.chunk_attn_pool_tilelang(mu.to(dev), k_rep.to(dev))
-    assert torch.equal(lk2, lk) and torch.equal(lb2, lb)
+    assert_close_bf16(lk, lk2.float(), "grouped vs per-head lmk_k")
+    assert_close_f32(lb, lb2, 2e-5, "grouped vs per-head lmk_b")
     torch.autograd.backward([lk, lb], [gk.to(dev), gb.to(dev)])
     rmu, rk = _pool_grads(orc, mu, k_rep, gk, gb)
     assert_close_bf16(mu_d.grad, rmu, "grouped d_mu")
