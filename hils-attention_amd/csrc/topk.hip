@@ -1839,7 +1839,7 @@ bool hils_topk_group_covers(int N, int G, int D, int topk, int per_qhead, bool p
 int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* lse_swa, const float* bias,
                            int32_t* indices, void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
                            int G, int D, int topk, int block_size, int window_size, int causal, int q_offset,
-                           float sm_scale, int lse_bf16, void* stream);
+                           float sm_scale, int lse_bf16, int per_qhead, void* stream);
 
 // rows = (query, KV head) pairs; the row kernel wants about one row per compute unit
 // LDS of a row workgroup before the wavefronts' staging areas: raw logits [4][NP], pooled scores, page
@@ -2014,9 +2014,10 @@ extern "C" int hils_topk_lse16_covers(int B, int L, int N, int h_kv, int G, int 
 }
 
 extern "C" size_t hils_topk_fwd_workspace(int B, int L, int N, int h_kv, int G) {
-  // many queries: room for the chunk keys repacked into MFMA operand order (head dim up to 128)
+  // many queries: room for the chunk keys repacked into MFMA operand order (head dim up to 128; a key
+  // per query head when the caller's keys are per query head)
   if (!topk_use_split(B, L, N, h_kv))
-    return G <= 4 ? (size_t)B * h_kv * ((N + 15) / 16) * 16 * 128 * sizeof(bf16_t) : 0;
+    return G <= 4 ? (size_t)B * h_kv * G * ((N + 15) / 16) * 16 * 128 * sizeof(bf16_t) : 0;
   return (size_t)B * L * h_kv * G * N * sizeof(float);
 }
 
@@ -2102,6 +2103,19 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
     HILS_CHECK_LAUNCH("hils_topk_fwd");
     return HILS_OK;
   }
+  // one chunk key per query head: the one-pass kernel's four-wavefront form (G = 3, 4)
+  if (per_qhead && workspace && hils_topk_group_covers(N, G, D, topk, 1, !gumbel && !drop_mask)) {
+    const int nblk16 = (N + 15) / 16;
+    const long total = (long)B * h_kv * G * nblk16 * (D / 32) * 64;
+    hipLaunchKernelGGL(topk_pack_lmk_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                       (const bf16_t*)lmks, (uint4*)workspace, N, h_kv * G, D, nblk16, total);
+    if (int rc2 = hils_topk_group_launch(q, workspace, lse_swa, bias, indices, scores, lse_total, sel_logits, B, L, N,
+                                         h_kv, G, D, topk, block_size, window_size, causal, q_offset, sm_scale,
+                                         lse_bf16, 1, stream))
+      return rc2;
+    HILS_CHECK_LAUNCH("hils_topk_fwd");
+    return HILS_OK;
+  }
   if (!per_qhead && G <= 4 && (D == 64 || D == 128)) {
     const int segw = topk_rows_segw(N);
     const int NQ = (G == 1) ? 16 : 8;                                 // queries per wavefront
@@ -2123,7 +2137,7 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
       if (hils_topk_group_covers(N, G, D, topk, per_qhead, !gumbel && !drop_mask)) {
         if (int rc2 = hils_topk_group_launch(q, packed, lse_swa, bias, indices, scores, lse_total, sel_logits, B, L, N,
                                              h_kv, G, D, topk, block_size, window_size, causal, q_offset,
-                                             sm_scale, lse_bf16, stream))
+                                             sm_scale, lse_bf16, 0, stream))
           return rc2;
         HILS_CHECK_LAUNCH("hils_topk_fwd");
         return HILS_OK;

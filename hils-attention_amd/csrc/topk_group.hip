@@ -132,8 +132,13 @@ __device__ __forceinline__ uint32_t tg_kth_largest(const uint32_t (&k)[NE], uint
 // its registers and LDS until its slowest wavefront is through (the threshold searches differ in
 // length): 4 per workgroup ran 3.5 % slower than 2, and 8 ran 17 % slower; 1 was no faster than 2.
 #define TG_WAVES 2
-template <int GMAX, int KS, int NB, bool EXPORT, bool BIAS>
-__global__ void __launch_bounds__(64 * TG_WAVES)
+// PERQ: one chunk key per QUERY head (lmk_packed holds h_kv * G heads).  A workgroup is then four
+// wavefronts on 16 queries: for the logits wavefront w takes head w of all 16 queries (full MFMA
+// rows, that head's keys streamed once for 16 queries), and block by block the four wavefronts
+// trade accumulators through LDS so that each ends up with the rows the shared-key layout gives it
+// (its 4 queries x 4 heads); everything behind the logits is the same code.
+template <int GMAX, int KS, int NB, bool EXPORT, bool BIAS, bool PERQ>
+__global__ void __launch_bounds__(64 * (PERQ ? 4 : TG_WAVES))
     __attribute__((amdgpu_waves_per_eu(NB <= 8 ? 5 : (NB <= 16 ? 4 : (NB <= 24 ? 3 : 2)))))
 topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lmk_packed,
                       const float* __restrict__ lse_swa, const float* __restrict__ bias,
@@ -146,14 +151,16 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   constexpr int QPL = 4 / GMAX;   // queries per lane (its four accumulator rows)
   constexpr int NQ = 16 / GMAX;   // queries per wavefront
   constexpr int NMASK = EXPORT ? 0 : (NB > 8 ? NB / 2 : 0);  // blocks below it are visible to every row
-  __shared__ uint32_t cand_w[TG_WAVES][4][TG_CAND];          // compacted candidate keys, per lane row
-  __shared__ uint32_t words_w[TG_WAVES][4][16], wbase_w[TG_WAVES][4][16];  // winner map of a query and its word prefix counts
-  __shared__ __align__(16) int stage_i_w[TG_WAVES][NQ * 32];               // winners' chunk indices, [query][slot]
-  __shared__ __align__(16) bf16_t stage_s_w[TG_WAVES][NQ * GMAX * 32];  // their raw scores, [query][slot][head]
+  constexpr int TGW = PERQ ? 4 : TG_WAVES;                   // wavefronts per workgroup
+  static_assert(!PERQ || GMAX == 4, "per-query-head keys: four heads, four wavefronts");
+  __shared__ uint32_t cand_w[TGW][4][TG_CAND];          // compacted candidate keys, per lane row
+  __shared__ uint32_t words_w[TGW][4][16], wbase_w[TGW][4][16];  // winner map of a query and its word prefix counts
+  __shared__ __align__(16) int stage_i_w[TGW][NQ * 32];               // winners' chunk indices, [query][slot]
+  __shared__ __align__(16) bf16_t stage_s_w[TGW][NQ * GMAX * 32];  // their raw scores, [query][slot][head]
   // the bias of this (batch, KV head): [chunk][head, padded to 4] fp32, a copy per wavefront (they never
   // synchronise); read back 16 bytes per lane right where a block's logits are formed, instead of
   // global loads whose latency the compiler covers with registers this kernel does not have
-  __shared__ __align__(16) float bias_w[BIAS ? TG_WAVES : 1][BIAS ? NB * 16 : 1][4];
+  __shared__ __align__(16) float bias_w[BIAS ? TGW : 1][BIAS ? NB * 16 : 1][4];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   uint32_t (*cand)[TG_CAND] = cand_w[wave];
@@ -162,8 +169,10 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   int* stage_i = stage_i_w[wave];
   bf16_t* stage_s = stage_s_w[wave];
   const int lane = threadIdx.x & 63, col = lane & 15, j = lane >> 4;
-  const int t0 = t_base + (blockIdx.x * TG_WAVES + wave) * NQ;
-  if (t0 >= t_end) return;
+  const int t0 = t_base + (blockIdx.x * TGW + wave) * NQ;
+  const int t_wg = t_base + blockIdx.x * TGW * NQ;  // PERQ: the workgroup's 16 queries
+  if ((PERQ ? t_wg : t0) >= t_end) return;          // (PERQ: the wavefronts meet at barriers until the logits are in)
+  const int t_safe = PERQ ? t_wg : t0;              // a query of this launch, for the addresses of rows that have none
   const int hk = blockIdx.y;
   const long b = blockIdx.z;
 
@@ -193,11 +202,11 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   bf16x8_t afrag[KS];
   {
     const int r = lane & 15;
-    const int g = r % GMAX, tq = t0 + r / GMAX;
+    const int g = PERQ ? wave : r % GMAX, tq = PERQ ? t_wg + r : t0 + r / GMAX;
     const bool ok = tq < t_end && g < G;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      uint4 v = *(const uint4*)(q + (((b * L + (ok ? tq : t0)) * h_kv + hk) * (long)G + (ok ? g : 0)) * D + ks * 32 + j * 8);
+      uint4 v = *(const uint4*)(q + (((b * L + (ok ? tq : t_safe)) * h_kv + hk) * (long)G + (ok ? g : 0)) * D + ks * 32 + j * 8);
       if (!ok) v = make_uint4(0, 0, 0, 0);
       afrag[ks] = *(bf16x8_t*)&v;
     }
@@ -207,14 +216,15 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   for (int i = 0; i < 4; ++i) {
     const int r = 4 * j + i;
     const int tq = t0 + r / GMAX, g = r % GMAX;
-    const long li = ((b * L + (rowok[i] ? tq : t0)) * (long)h_kv + hk) * G + (rowok[i] ? g : 0);
+    const long li = ((b * L + (rowok[i] ? tq : t_safe)) * (long)h_kv + hk) * G + (rowok[i] ? g : 0);
     float x;  // the layer hands lse_swa over in its hidden dtype (hils_attention.py:547)
     if (lse_bf16) x = bf2f(((const bf16_t*)lse_swa)[li]); else x = lse_swa[li];
     swa[i] = rowok[i] ? x : HILS_NEG_INF;
   }
 
   // ---- the logits: x[nt][i] = sm_scale * <q_row, lmk_chunk>, -inf where the chunk is not visible ----
-  const uint4* pbase = lmk_packed + ((b * h_kv + hk) * (long)nb_real * KS) * 64 + lane;
+  const uint4* pbase = PERQ ? lmk_packed + (((b * h_kv + hk) * (long)G + (wave < G ? wave : 0)) * nb_real * KS) * 64 + lane
+                            : lmk_packed + ((b * h_kv + hk) * (long)nb_real * KS) * 64 + lane;
   float x[NB][4];
   // the keys of two blocks travel together, one such group ahead of their use (the loads of a
   // block issued right before its MFMAs would each expose a full memory latency)
@@ -254,26 +264,59 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
 #pragma unroll
     for (int i = 0; i < 4; ++i) bv[i] = e[i % GMAX];
   };
+  // PERQ: accumulators of a load group on their way between the wavefronts, [block][from wavefront =
+  // head][register][lane]; two buffers take turns, so that one barrier a group is enough
+  __shared__ float xch[PERQ ? 2 : 1][PERQ ? PB : 1][4][4][PERQ ? 64 : 1];
   auto use_group = [&](int g0, const tg_u32x4 (&src)[PB][KS]) {
+    const int buf = (g0 / PB) & 1;
+    if constexpr (PERQ) {
+#pragma unroll
+      for (int p2 = 0; p2 < PB; ++p2) {
+        const int nt = g0 + p2;
+        float bv[4];
+        if constexpr (BIAS) bias_of(nt * 16 + col, bv);
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[ks], __builtin_bit_cast(bf16x8_t, src[p2][ks]), acc, 0, 0, 0);
+        // rows 4j+i are queries here; the bias of (chunk, head = this wavefront)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v = __fmul_rn(acc[i], sm_scale);
+          if constexpr (BIAS) v = __fadd_rn(v, bv[wave]);
+          xch[buf][p2][wave][i][lane] = v;
+        }
+      }
+      __syncthreads();
+    }
 #pragma unroll
     for (int p2 = 0; p2 < PB; ++p2) {
       const int nt = g0 + p2;
       float bv[4];
-      if constexpr (BIAS) bias_of(nt * 16 + col, bv);
+      if constexpr (BIAS && !PERQ) bias_of(nt * 16 + col, bv);
       f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (!PERQ) {
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[ks], __builtin_bit_cast(bf16x8_t, src[p2][ks]), acc, 0, 0, 0);
+        for (int ks = 0; ks < KS; ++ks)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[ks], __builtin_bit_cast(bf16x8_t, src[p2][ks]), acc, 0, 0, 0);
+      }
       const int c = nt * 16 + col;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float v = __fmul_rn(acc[i], sm_scale);
-        if constexpr (BIAS) v = __fadd_rn(v, bv[i]);
+        float v;
+        if constexpr (PERQ) {
+          // row (query j of this wavefront, head i): wavefront i's register j of the lane that holds
+          // this chunk column for the queries 4 * wave .. 4 * wave + 3
+          v = xch[buf][p2][i][j][col + 16 * wave];
+        } else {
+          v = __fmul_rn(acc[i], sm_scale);
+          if constexpr (BIAS) v = __fadd_rn(v, bv[i]);
+        }
         if (nt >= NMASK) v = (c < lim[i]) ? v : HILS_NEG_INF;
         x[nt][i] = v;
         // (pinned here: left alone the compiler forms some of these sums only where they are used and
         // keeps product and bias alive in their place, which this kernel has no registers for)
-        if constexpr (BIAS) asm volatile("" : "+v"(x[nt][i]));
+        if constexpr (BIAS && !PERQ) asm volatile("" : "+v"(x[nt][i]));
       }
       if (EXPORT) {
         if (sel_logits_out && c < N) {
@@ -307,6 +350,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
     }
   }
 
+  if (PERQ && t0 >= t_end) return;  // no barrier behind this point
   // ---- lse_total per row = logaddexp(lse_swa, logsumexp of the visible logits) ----
   float lse_tot[4];
 #pragma unroll
@@ -538,18 +582,18 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
 
 // plain: no Gumbel noise and no drop mask (a bias is fine)
 bool hils_topk_group_covers(int N, int G, int D, int topk, int per_qhead, bool plain) {
-  return plain && !per_qhead && (G == 1 || G == 3 || G == 4) && (D == 64 || D == 128) && N <= 16 * TG_NB &&
-         topk <= 32;
+  if (per_qhead && G != 3 && G != 4) return false;  // (one head a group: the keys are shared anyway)
+  return plain && (G == 1 || G == 3 || G == 4) && (D == 64 || D == 128) && N <= 16 * TG_NB && topk <= 32;
 }
 
-template <int GMAX, int KS, bool BIAS>
+template <int GMAX, int KS, bool BIAS, bool PERQ>
 static void tg_launch_range(int NB, bool exp, dim3 grid, hipStream_t st, const bf16_t* q, const uint4* pk,
                             const float* lse_swa, const float* bias, int32_t* indices, bf16_t* scores, float* lse_total,
                             float* sel_logits, int L, int N, int h_kv, int G, int topk, int block_size,
                             int window_size, int causal, int q_offset, float sm_scale, int t_base, int t_end,
                             int lse_bf16) {
 #define TG_CALL(NB_, EX_)                                                                              \
-  hipLaunchKernelGGL((topk_fwd_group_kernel<GMAX, KS, NB_, EX_, BIAS>), grid, dim3(64 * TG_WAVES), 0, st, q, pk, lse_swa, \
+  hipLaunchKernelGGL((topk_fwd_group_kernel<GMAX, KS, NB_, EX_, BIAS, PERQ>), grid, dim3(64 * (PERQ ? 4 : TG_WAVES)), 0, st, q, pk, lse_swa, \
                      bias, indices, scores, lse_total, sel_logits, L, N, h_kv, G, topk, block_size, window_size, \
                      causal, q_offset, sm_scale, t_base, t_end, bs_shift, lse_bf16)
   const int bs_shift = (block_size > 0 && (block_size & (block_size - 1)) == 0) ? __builtin_ctz(block_size) : -1;
@@ -569,9 +613,10 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
                            int32_t* indices,
                            void* scores, float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
                            int G, int D, int topk, int block_size, int window_size, int causal, int q_offset,
-                           float sm_scale, int lse_bf16, void* stream) {
+                           float sm_scale, int lse_bf16, int per_qhead, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   const int GM = (G == 1) ? 1 : 4;
+  const int TGW = per_qhead ? 4 : TG_WAVES;
   const int NQ = 16 / GM;
   const bool exp = sel_logits != nullptr;
   auto limit_of = [&](int tq) -> int {
@@ -594,17 +639,18 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
         t_hi = lo;
       }
     }
-    dim3 grid((t_hi - t + NQ * TG_WAVES - 1) / (NQ * TG_WAVES), h_kv, B);
-#define TG_RANGE_B(G_, KS_, B_)                                                                       \
-  tg_launch_range<G_, KS_, B_>(NB, exp, grid, st, (const bf16_t*)q, (const uint4*)lmk_packed, lse_swa, bias, \
+    dim3 grid((t_hi - t + NQ * TGW - 1) / (NQ * TGW), h_kv, B);
+#define TG_RANGE_B(G_, KS_, B_, P_)                                                                   \
+  tg_launch_range<G_, KS_, B_, P_>(NB, exp, grid, st, (const bf16_t*)q, (const uint4*)lmk_packed, lse_swa, bias, \
                                indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,   \
                                block_size, window_size, causal, q_offset, sm_scale, t, t_hi, lse_bf16)
-#define TG_RANGE(G_, KS_)                                                                             \
+#define TG_RANGE(G_, KS_, P_)                                                                         \
   do {                                                                                                \
-    if (bias) TG_RANGE_B(G_, KS_, true); else TG_RANGE_B(G_, KS_, false);                             \
+    if (bias) TG_RANGE_B(G_, KS_, true, P_); else TG_RANGE_B(G_, KS_, false, P_);                     \
   } while (0)
-    if (GM == 1) { if (D == 64) TG_RANGE(1, 2); else TG_RANGE(1, 4); }
-    else { if (D == 64) TG_RANGE(4, 2); else TG_RANGE(4, 4); }
+    if (GM == 1) { if (D == 64) TG_RANGE(1, 2, false); else TG_RANGE(1, 4, false); }
+    else if (per_qhead) { if (D == 64) TG_RANGE(4, 2, true); else TG_RANGE(4, 4, true); }
+    else { if (D == 64) TG_RANGE(4, 2, false); else TG_RANGE(4, 4, false); }
 #undef TG_RANGE
 #undef TG_RANGE_B
     t = t_hi;

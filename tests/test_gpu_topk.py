@@ -82,6 +82,15 @@ def run_case(pkg, orc, dev, B, L, N, h_kv, G, D, topk, S, W, seed=42, q_offset=0
     want = torch.gather(aux["logits"], -1, safe).masked_fill(~valid.unsqueeze(3).expand(-1, -1, -1, G, -1),
                                                               float("-inf"))
     assert_close_bf16(scores.view(B, L, h_kv, G, topk), want, "scores")
+    if per_qhead and not one_kernel:
+        # without the logit export other launches run (queries bucketed by visible chunks): same results
+        idx2, scores2 = pkg.online_softmax_topk_head(
+            q_in.to(dev), lmks.to(dev), lse_swa.to(dev), topk, S, W, is_causal=is_causal,
+            q_offset=q_offset, is_training=training,
+            drop_mask=None if drop is None else drop.to(dev),
+            bias=None if bias is None else bias.to(dev),
+            gumbel_noise=None if gumbel is None else gumbel.to(dev), G=G)
+        assert torch.equal(idx2, idx) and torch.equal(scores2, scores), "export and plain launches differ"
     return idx, scores
 
 
@@ -117,6 +126,15 @@ def test_topk_per_qhead_lmks(pkg, orc, dev):
     run_case(pkg, orc, dev, B=1, L=512, N=8, h_kv=2, G=4, D=64, topk=4, S=64, W=1, per_qhead=True)
     run_case(pkg, orc, dev, B=1, L=300, N=5, h_kv=1, G=2, D=128, topk=8, S=64, W=1, per_qhead=True,
              use_bias=True)
+    # the one-pass kernel's form for a key per query head (G = 3, 4; N <= 512, topk <= 32): ragged query
+    # counts, every bucket of visible chunks, with and without the bias, another head dim, batch > 1
+    run_case(pkg, orc, dev, B=1, L=777, N=13, h_kv=2, G=4, D=128, topk=8, S=64, W=1, per_qhead=True)
+    run_case(pkg, orc, dev, B=2, L=2100, N=500, h_kv=1, G=4, D=64, topk=32, S=4, W=1, per_qhead=True,
+             use_bias=True, training=False)
+    run_case(pkg, orc, dev, B=1, L=1030, N=260, h_kv=2, G=3, D=128, topk=16, S=4, W=3, per_qhead=True,
+             use_bias=True)
+    run_case(pkg, orc, dev, B=1, L=70, N=300, h_kv=3, G=4, D=64, topk=32, S=64, W=0, per_qhead=True,
+             is_causal=False)
 
 
 def test_topk_chunked_prefill_and_decode(pkg, orc, dev):
