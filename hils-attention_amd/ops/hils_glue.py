@@ -79,22 +79,26 @@ def _prior_bias(prior_b, B, N, h_q):
 
 
 def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causal=True, q_offset=0,
-                       sm_scale=None, prior_b=None):
-    """Inference: ``online_softmax_topk_head`` (shared chunk keys, no Gumbel / drop mask) followed by
-    ``chunk_weights`` in one call, for the serving loop.  q (B,L,h_q,D) bf16, lmks (B,N,h_kv,D) bf16,
-    lse_swa (B,L,h_q) -> indices (B,L,h_kv,topk) int32, scores (B,L,h_q,topk) bf16, weights
-    (B,L,h_q,topk+1) bf16.  ``prior_b`` (B,N,h_q): the layer's prior bias (its ``enable_prior_query``
-    mode, models/FlashHiLS/hils_attention.py:568-602), used as the selection's ``bias`` and gathered
-    into the softmax.  With about one (query, KV head) row per compute unit the selection kernel
-    writes the weights itself; otherwise two kernels run."""
+                       sm_scale=None, prior_b=None, num_kv_heads=None):
+    """Inference: ``online_softmax_topk_head`` (no Gumbel / drop mask) followed by ``chunk_weights``
+    in one call, for the serving loop.  q (B,L,h_q,D) bf16, lmks (B,N,h_kv,D) bf16 (one chunk key per
+    KV head) or, with ``num_kv_heads`` given, (B,N,h_q,D) (one per query head, the layer's
+    attention-pooled keys), lse_swa (B,L,h_q) -> indices (B,L,h_kv,topk) int32, scores (B,L,h_q,topk)
+    bf16, weights (B,L,h_q,topk+1) bf16.  ``prior_b`` (B,N,h_q): the layer's prior bias (its
+    ``enable_prior_query`` mode, models/FlashHiLS/hils_attention.py:568-602), used as the selection's
+    ``bias`` and gathered into the softmax.  With about one (query, KV head) row per compute unit the
+    selection kernel writes the weights itself; otherwise two kernels run."""
     import math
     _cabi.require_gpu_bf16("topk_chunk_weights", q, lmks)
     if torch.is_grad_enabled() and (q.requires_grad or lmks.requires_grad or lse_swa.requires_grad):
         raise RuntimeError("topk_chunk_weights is forward-only")
     B, L, h_q, D = q.shape
-    N, h_kv = lmks.shape[1], lmks.shape[2]
+    N, h_lmk = lmks.shape[1], lmks.shape[2]
+    h_kv = h_lmk if num_kv_heads is None else int(num_kv_heads)
     assert lmks.shape[0] == B and lmks.shape[3] == D
     assert h_q % h_kv == 0, f"h_q ({h_q}) must be divisible by h_kv ({h_kv})"
+    assert h_lmk in (h_kv, h_q), f"lmks carries {h_lmk} heads: neither the {h_kv} KV heads nor the {h_q} query heads"
+    per_qhead = int(h_lmk != h_kv)
     G = h_q // h_kv
     scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(D)
     dev = q.device
@@ -103,7 +107,7 @@ def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causa
     scores = torch.empty((B, L, h_q, topk), dtype=q.dtype, device=dev)
     weights = torch.empty((B, L, h_q, topk + 1), dtype=q.dtype, device=dev)
     ws = _cabi.topk_fwd_workspace(dev, B, L, N, h_kv, G)
-    if (lse_swa.dtype == torch.bfloat16 and ws is not None
+    if (lse_swa.dtype == torch.bfloat16 and ws is not None and not per_qhead
             and _cabi.load().hils_topk_lse16_covers(B, L, N, h_kv, G, D, int(topk))):
         # lse_swa as the layer hands it over (bf16): read in place, no conversion pass
         _cabi.call("hils_topk_fwd_weights_lse16", _cabi.ptr(q.contiguous()), _cabi.ptr(lmks.contiguous()),
@@ -116,7 +120,7 @@ def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causa
     _cabi.call("hils_topk_fwd_weights", _cabi.ptr(q.contiguous()), _cabi.ptr(lmks.contiguous()),
                _cabi.ptr(lse), _cabi.ptr(pb), _cabi.ptr(pb), None, None, _cabi.ptr(indices), _cabi.ptr(scores),
                _cabi.ptr(weights), _cabi.ptr(ws), _cabi.nbytes(ws), B, L, N, h_kv, G, D, int(topk),
-               int(block_size), int(window_size), int(bool(is_causal)), int(q_offset), 0, scale)
+               int(block_size), int(window_size), int(bool(is_causal)), int(q_offset), per_qhead, scale)
     return indices, scores, weights
 
 

@@ -64,6 +64,40 @@ def test_prefill_selection_with_prior_bias(pkg, orc, dev, L, N, HQ, H, D, K, off
     assert not torch.equal(idx_nb, idx1)
 
 
+@pytest.mark.parametrize("L,N,HQ,H,D,K", [(3000, 47, 8, 2, 128, 16), (5000, 400, 4, 1, 64, 32)])
+def test_prefill_selection_with_a_key_per_query_head(pkg, orc, dev, L, N, HQ, H, D, K):
+    """The layer's default pooling (attention-pooled chunk keys, one per query head, with their prior
+    bias; models/FlashHiLS/hils_attention.py:391-416, 568-602) through topk_chunk_weights: same
+    indices and scores as the operator, weights against chunk_weights and the oracle."""
+    note(f"prefill selection, key per query head, L{L} N{N} HQ{HQ} H{H} D{D} K{K}")
+    B, S, W = 1, 64, 1
+    G = HQ // H
+    off = N * S - L if N * S > L else 0
+    gen = torch.Generator().manual_seed(402)
+    q = torch.randn(B, L, HQ, D, generator=gen).bfloat16()
+    lmk = torch.randn(B, N, HQ, D, generator=gen).bfloat16()
+    lse = (torch.randn(B, L, HQ, generator=gen) * 3 + 5).bfloat16().float()
+    pb = torch.randn(B, N, HQ, generator=gen) * 2
+    qd, lmkd, lsed, pbd = q.to(dev), lmk.to(dev), lse.to(dev), pb.to(dev)
+    dbg = {}
+    idx0, sc0 = pkg.online_softmax_topk_head(qd, lmkd, lsed, K, S, W, q_offset=off, is_training=False,
+                                             bias=pbd, G=G, _debug=dbg)
+    lim = orc.causal_chunk_limit(L, off, W, S)
+    want = orc.topk_select(dbg["sel_logits"].cpu(), dbg["lse_total"].cpu(), lim, K)
+    assert torch.equal(idx0.cpu(), want), "indices not bit-exact from the kernel's biased logits"
+    ridx, rsc, aux = orc.online_softmax_topk_head(q.view(B, L, H, G, D), lmk, lse, K, S, W, q_offset=off,
+                                                  bias=pb, return_aux=True)
+    assert_close_f32(dbg["sel_logits"].cpu(), aux["sel_logits"], 2e-3, "biased selection logits")
+    assert (idx0.cpu() == ridx).float().mean().item() >= 0.99
+    w0 = pkg.chunk_weights(sc0, lsed, pbd, idx0)
+    for lse_in in (lsed, lsed.bfloat16()):
+        idx1, sc1, w1 = pkg.topk_chunk_weights(qd, lmkd, lse_in, K, S, W, q_offset=off, prior_b=pbd, num_kv_heads=H)
+        assert torch.equal(idx1, idx0) and torch.equal(sc1.view(torch.int16), sc0.view(torch.int16))
+        assert (w1.float() - w0.float()).abs().max().item() <= 4e-3
+    w_ref = orc.inter_chunk_softmax(sc0.float().cpu(), lse, pb.bfloat16().float(), idx0.cpu(), bf16_sum=True)
+    assert (w0.float().cpu() - w_ref).abs().max().item() <= 8e-3
+
+
 @pytest.mark.parametrize("B,Lq,Lkv,HQ,H,D,K", [(32, 1, 32768, 32, 8, 128, 32), (16, 1, 16512, 8, 8, 64, 16),
                                                (50, 2, 20480, 4, 1, 128, 8), (2, 1, 4096, 8, 2, 128, 16)])
 def test_decode_step_with_prior_bias(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
