@@ -546,7 +546,6 @@ attn_pool_fwd_gqa_mfma(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict
       for (int i = 0; i < 4; ++i) {
         const float pv = st[mt][i] * inv;
         const int t = mt * 16 + 4 * j + i;
-        if (col < G) p_out[(bn * S + t) * (long)H + h] = pv;
         if (pv > 0.f) ent += pv * __logf(pv);
         ps[col * S + (t % TPI) * NI + t / TPI] = pv;  // columns past G hold the softmax of zeros: finite, unused
       }
@@ -554,6 +553,18 @@ attn_pool_fwd_gqa_mfma(const bf16_t* __restrict__ mu_q, const bf16_t* __restrict
     if (col < G && j == 0) lmk_b[bn * H + h] = -ent;
     __atomic_signal_fence(__ATOMIC_SEQ_CST);
     __builtin_amdgcn_wave_barrier();
+    // the saved P, (chunk, token, head): lane t writes token t's G heads, contiguous in memory (from the
+    // accumulator layout it would be 16 stores of 4 bytes per lane)
+    {
+      float* dst = p_out + (bn * S + lane) * (long)H + kh * G;
+      const float* src = ps + (lane % TPI) * NI + lane / TPI;
+      if ((G & 3) == 0) {
+        for (int g = 0; g < G; g += 4)
+          *(float4*)(dst + g) = make_float4(src[g * S], src[(g + 1) * S], src[(g + 2) * S], src[(g + 3) * S]);
+      } else {
+        for (int g = 0; g < G; ++g) dst[g] = src[g * S];
+      }
+    }
     // lmk_k = P K, four heads at a time over the token rows in registers
     for (int g0 = 0; g0 < G; g0 += 4) {
       float acc[4][8];
