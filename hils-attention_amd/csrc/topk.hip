@@ -1296,7 +1296,9 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
               float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
               int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
               float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages,
-              int lmk_hm, int lmk_cap, float* dyn, const long row, TopkRowShared* sh_p = nullptr) {
+              int lmk_hm, int lmk_cap, int perq, float* dyn, const long row, TopkRowShared* sh_p = nullptr) {
+  // perq: one chunk key per QUERY head, lmks = (B,N,h_kv*G,D) / (B,h_kv*G,lmk_cap,D) / (num_pages,h_kv*G,D):
+  // the row streams G key tensors, a key group of head g gives the logits of MFMA column g only
   constexpr int LR = D / 8, TPI = 64 / LR;
   constexpr int THREADS = NW * 64;       // NW = 8 or 16 wavefronts
   constexpr int EPT = TOPK_R_MAXN / THREADS;  // 64-chunk slots of a wavefront's share
@@ -1385,25 +1387,37 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     const int col = lane & 15, j = lane >> 4;
     char* const w_addr = stage_w + tsub * ROWB + piece * 16;
     const char* const k_addr = stage_w + col * ROWB + j * 16;
-    const int ngroups = (lim + KG - 1) / KG;
-    // dense chunk keys: (B, N, h_kv, D), or head-major (B, h_kv, lmk_cap, D) (a row's keys contiguous)
-    const bf16_t* base = lmks + (lmk_hm ? (b * h_kv + hk) * (long)lmk_cap * D : (b * N * (long)h_kv + hk) * D) + piece * 8;
-    const long cstride = (PAGED || !lmk_hm) ? (long)h_kv * D : (long)D;
-    const bf16_t* pbase = lmks + (long)hk * D + piece * 8;  // paged: + page * h_kv * D
-    auto fetch = [&](tr_u4 (&kr)[GI], int grp) __attribute__((always_inline)) {
+    // key groups of the row: KG chunks each, times the G heads when every query head has its own keys
+    // (group number = chunk group * G + head: the heads of a chunk are neighbours in memory)
+    const int GK = perq ? G : 1;                  // key tensors of the row
+    const int h_lmk = h_kv * GK;                  // heads of the key tensor
+    const int ngroups = ((lim + KG - 1) / KG) * GK;
+    // dense chunk keys: (B, N, h_lmk, D), or head-major (B, h_lmk, lmk_cap, D) (a row's keys contiguous)
+    const bf16_t* base = lmks + (lmk_hm ? (b * h_lmk + hk * GK) * (long)lmk_cap * D : (b * N * (long)h_lmk + hk * GK) * D) + piece * 8;
+    const long cstride = (PAGED || !lmk_hm) ? (long)h_lmk * D : (long)D;
+    const long gstride = (!PAGED && lmk_hm) ? (long)lmk_cap * D : (long)D;  // from a head to the next of the group
+    const bf16_t* pbase = lmks + (long)hk * GK * D + piece * 8;  // paged: + page * h_lmk * D
+    auto fetch = [&](tr_u4 (&kr)[GI], int vg) __attribute__((always_inline)) {
+      const int grp = perq ? vg / G : vg;
+      const long goff = perq ? (vg - grp * G) * gstride : 0;
 #pragma unroll
       for (int it = 0; it < GI; ++it) {
         int c = grp * KG + it * TPI + tsub;
         c = c < N ? c : N - 1;
         if (PAGED) {
           const int pg = page_s[c];  // an unmapped or invisible chunk reads page 0 and is masked below
-          kr[it] = *(const tr_u4*)(pbase + (long)(pg < 0 ? 0 : pg) * cstride);
+          kr[it] = *(const tr_u4*)(pbase + goff + (long)(pg < 0 ? 0 : pg) * cstride);
         } else {
-          kr[it] = *(const tr_u4*)(base + c * cstride);
+          kr[it] = *(const tr_u4*)(base + goff + c * cstride);
         }
       }
     };
-    auto consume = [&](const tr_u4 (&kr)[GI], int grp) __attribute__((always_inline)) {
+    auto consume = [&](const tr_u4 (&kr)[GI], int vg) __attribute__((always_inline)) {
+      const int grp = perq ? vg / G : vg;
+      const int gh = perq ? vg - grp * G : -1;  // the head these keys belong to (-1: to all heads)
+      // the MFMA columns this group fills: its head's (with the last head's keys also the columns past G,
+      // whose logit rows and sums hold -inf / 0 as with shared keys)
+      const bool mine = gh < 0 ? col < GMAX : (col == gh || (gh == G - 1 && col >= G && col < GMAX));
       float m_run = HILS_NEG_INF, l_run = 0.f;  // this lane's head over the group's keys it sees
 #pragma unroll
       for (int tt = 0; tt < GI / LPT; ++tt) {
@@ -1419,7 +1433,7 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
         }
         // accumulator register i of lane (head = col, j) is key c0 + 4j + i
         const int c0 = grp * KG + tt * 16 + 4 * j;
-        if (col < GMAX) {  // (the rows of the heads past G hold -inf)
+        if (mine) {  // (the rows of the heads past G hold -inf)
           f32x4_t out;
 #pragma unroll
           for (int i = 0; i < 4; ++i) out[i] = (c0 + i < lim && col < G) ? __fmul_rn(acc[i], sm_scale) : HILS_NEG_INF;
@@ -1450,7 +1464,7 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       const float M = rows_max(m_run);
       const float Ms = (M == HILS_NEG_INF) ? 0.f : M * HILS_LOG2E;
       const float Lg = rows_sum(l_run * __builtin_amdgcn_exp2f(fmaf(m_run, HILS_LOG2E, -Ms)));
-      if (j == 0 && col < GMAX) {  // lanes of heads past G never left (-inf, 0)
+      if (j == 0 && mine) {  // lanes of heads past G never left (-inf, 0)
         sh.grp_m[grp][col] = M;
         sh.grp_l[grp][col] = Lg;
       }
@@ -1781,11 +1795,11 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                 float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
                 int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
                 float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages,
-                int lmk_hm, int lmk_cap) {
+                int lmk_hm, int lmk_cap, int perq) {
   extern __shared__ __align__(16) float topk_row_dyn[];
   topk_row_body<D, GMAX, NW, PAGED>(q, lmks, lse_swa, bias, indices, scores, lse_total_out, sel_logits_out,
                                     weights_out, L, N, NP, h_kv, G, topk, block_size, window_size, causal,
-                                    q_offset, sm_scale, page_table, max_pages, num_pages, lmk_hm, lmk_cap,
+                                    q_offset, sm_scale, page_table, max_pages, num_pages, lmk_hm, lmk_cap, perq,
                                     topk_row_dyn, (long)blockIdx.x);
 }
 
@@ -1805,7 +1819,7 @@ struct DsArgs {
   int L, N, NP, h_kv, G, topk, block_size, window_size, q_offset;
   float sm_scale_sel;
   const int32_t* page_table;
-  int max_pages, num_pages, lmk_hm, lmk_cap;
+  int max_pages, num_pages, lmk_hm, lmk_cap, perq;
   DrDims dr;
 };
 // PAGED: the chunk keys (and the bias) are addressed through the page table; the attention reads
@@ -1818,8 +1832,8 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_step_kernel(DsArgs a) {
   topk_row_body<D, 4, DS_WAVES, PAGED, true>(a.q, a.lmks, a.lse_swa, a.bias, a.indices, a.scores, a.lse_total,
                                              a.sel_logits, a.weights, a.L, a.N, a.NP, a.h_kv, a.G, a.topk,
                                              a.block_size, a.window_size, 1, a.q_offset, a.sm_scale_sel,
-                                             a.page_table, a.max_pages, a.num_pages, a.lmk_hm, a.lmk_cap, ds_dyn,
-                                             row, &ds_sh);
+                                             a.page_table, a.max_pages, a.num_pages, a.lmk_hm, a.lmk_cap, a.perq,
+                                             ds_dyn, row, &ds_sh);
   // The attention reads the row's indices and weights where the selection left them in LDS: the
   // pointers are offset so that the row's entries of the (B, L, heads, ...) tensors fall there.  Its
   // staging areas lie over the selection's logits: the barrier that separates the two uses runs in
@@ -1854,7 +1868,8 @@ static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool pla
                          bool paged = false) {
   if (with_bias && topk_row_smem_base(N, paged, true) + (size_t)8 * 16 * (2 * D + 16) + sizeof(TopkRowShared) > 158 * 1024)
     return false;
-  return plain && !per_qhead && G <= 4 && (D == 64 || D == 128) && N >= 256 && N <= TOPK_R_MAXN &&
+  (void)per_qhead;  // shared chunk keys or one per query head: the same kernel
+  return plain && G <= 4 && (D == 64 || D == 128) && N >= 256 && N <= TOPK_R_MAXN &&
          rows >= 96 && rows <= 2147483647L;
 }
 
@@ -1862,7 +1877,7 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, c
                         void* scores, float* lse_total, float* sel_logits, void* weights, int B, int L, int N, int h_kv, int G, int D,
                         int topk, int block_size, int window_size, int causal, int q_offset,
                         float sm_scale, hipStream_t st, const int32_t* page_table = nullptr, int max_pages = 0,
-                        int num_pages = 0, int lmk_hm = 0, int lmk_cap = 0) {
+                        int num_pages = 0, int lmk_hm = 0, int lmk_cap = 0, int perq = 0) {
   const long rows = (long)B * L * h_kv;
   const int NP = (N + 63) & ~63;
   // then 16 padded key rows of staging per wavefront
@@ -1882,7 +1897,7 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, c
                        (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, indices, (bf16_t*)scores, \
                        lse_total, sel_logits, (bf16_t*)weights, L, N, NP, h_kv, G, topk,         \
                        block_size, window_size, causal, q_offset, sm_scale, page_table, max_pages, \
-                       num_pages, lmk_hm, lmk_cap);                                              \
+                       num_pages, lmk_hm, lmk_cap, perq);                                        \
   } while (0)
 #define TOPK_ROW_CALL(D_, P_)                                                                    \
   do {                                                                                           \
@@ -1911,7 +1926,7 @@ extern "C" int hils_decode_step_covers(int B, int L, int N, int HQ, int H, int D
 }
 
 static int decode_step_launch(const void* q, const void* lmks, const void* k, const void* v, const float* lse_swa,
-                              const float* bias, int lmk_paged, int lmk_hm, int lmk_cap, int32_t* indices, void* scores, void* weights, void* o, float* lse_total,
+                              const float* bias, int lmk_paged, int lmk_hm, int lmk_cap, int perq, int32_t* indices, void* scores, void* weights, void* o, float* lse_total,
                               float* sel_logits, int B, int L, int Lkv, int N, int HQ, int H, int D, int topk,
                               int block_size, int window_size, int q_offset, float sm_scale_sel,
                               float sm_scale_attn, int mask_last, const int32_t* page_table, int max_pages,
@@ -1927,7 +1942,7 @@ static int decode_step_launch(const void* q, const void* lmks, const void* k, co
   DsArgs a;
   a.q = (const bf16_t*)q; a.lmks = (const bf16_t*)lmks; a.k = (const bf16_t*)k; a.v = (const bf16_t*)v;
   a.lse_swa = lse_swa; a.bias = bias; a.indices = indices;
-  a.lmk_hm = lmk_hm; a.lmk_cap = lmk_cap;
+  a.lmk_hm = lmk_hm; a.lmk_cap = lmk_cap; a.perq = perq;
   a.scores = (bf16_t*)scores; a.weights = (bf16_t*)weights; a.o = (bf16_t*)o;
   a.lse_total = lse_total; a.sel_logits = sel_logits;
   a.L = L; a.N = N; a.NP = NP; a.h_kv = H; a.G = G; a.topk = topk; a.block_size = block_size;
@@ -1956,7 +1971,7 @@ extern "C" int hils_decode_step(const void* q, const void* lmks, const void* k, 
                                 void* weights, void* o, float* lse_total, float* sel_logits, int B, int L, int Lkv,
                                 int N, int HQ, int H, int D, int topk, int block_size, int window_size,
                                 int q_offset, float sm_scale_sel, float sm_scale_attn, int mask_last,
-                                int lmk_head_major, int lmk_cap, void* stream) {
+                                int lmk_head_major, int lmk_cap, int lmk_per_qhead, void* stream) {
   HILS_REQUIRE(q && lmks && k && v && lse_swa && indices && scores && weights && o, "hils_decode_step: null pointer");
   HILS_REQUIRE(B > 0 && L > 0 && N > 0 && H > 0 && HQ > 0 && HQ % H == 0, "hils_decode_step: bad sizes");
   HILS_REQUIRE(!lmk_head_major || lmk_cap >= N, "hils_decode_step: lmk_cap (%d) must be at least N (%d)", lmk_cap, N);
@@ -1964,7 +1979,7 @@ extern "C" int hils_decode_step(const void* q, const void* lmks, const void* k, 
   HILS_REQUIRE(hils_decode_step_covers(B, L, N, HQ, H, D, topk, block_size, bias != nullptr),
                "hils_decode_step: shape not covered (hils_decode_step_covers): use hils_topk_fwd_weights + hils_sparse_attn_fwd");
   HILS_REQUIRE((long)B * L * H <= 2147483647L, "hils_decode_step: grid too large");
-  if (int rc = decode_step_launch(q, lmks, k, v, lse_swa, bias, 0, lmk_head_major, lmk_cap, indices, scores, weights, o,
+  if (int rc = decode_step_launch(q, lmks, k, v, lse_swa, bias, 0, lmk_head_major, lmk_cap, lmk_per_qhead, indices, scores, weights, o,
                                   lse_total, sel_logits, B, L, Lkv, N, HQ, H, D, topk, block_size, window_size,
                                   q_offset, sm_scale_sel, sm_scale_attn, mask_last, nullptr, 0, 0,
                                   (hipStream_t)stream))
@@ -1979,7 +1994,8 @@ extern "C" int hils_decode_step_paged(const void* q, const void* lmk_pages, cons
                                       float* lse_total, float* sel_logits, int B, int L, int N, int HQ, int H,
                                       int D, int topk, int block_size, int window_size, int q_offset,
                                       int max_pages, int num_pages, float sm_scale_sel, float sm_scale_attn,
-                                      int mask_last, int lmk_dense, int lmk_head_major, int lmk_cap, void* stream) {
+                                      int mask_last, int lmk_dense, int lmk_head_major, int lmk_cap,
+                                      int lmk_per_qhead, void* stream) {
   HILS_REQUIRE(!lmk_dense || !lmk_head_major || lmk_cap >= N,
                "hils_decode_step_paged: lmk_cap (%d) must be at least N (%d)", lmk_cap, N);
   HILS_REQUIRE(q && lmk_pages && k_pages && v_pages && page_table && lse_swa && indices && scores && weights && o,
@@ -1990,7 +2006,7 @@ extern "C" int hils_decode_step_paged(const void* q, const void* lmk_pages, cons
                "hils_decode_step_paged: shape not covered (hils_decode_step_covers): use hils_topk_fwd_weights_paged + hils_sparse_attn_decode_paged");
   HILS_REQUIRE((long)B * L * H <= 2147483647L, "hils_decode_step_paged: grid too large");
   if (int rc = decode_step_launch(q, lmk_pages, k_pages, v_pages, lse_swa, bias, lmk_dense ? 0 : 1,
-                                  lmk_dense ? lmk_head_major : 0, lmk_cap, indices, scores, weights, o, lse_total,
+                                  lmk_dense ? lmk_head_major : 0, lmk_cap, lmk_per_qhead, indices, scores, weights, o, lse_total,
                                   sel_logits, B, L, 0, N, HQ, H, D, topk, block_size, window_size, q_offset,
                                   sm_scale_sel, sm_scale_attn, mask_last, page_table, max_pages, num_pages,
                                   (hipStream_t)stream))
@@ -2089,7 +2105,8 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
     const bool w_here = weights != nullptr && prior_b == bias;
     *weights_fused = w_here;
     if (int rc2 = topk_fwd_row(q, lmks, lse_swa, bias, indices, scores, lse_total, sel_logits, w_here ? weights : nullptr,
-                               B, L, N, h_kv, G, D, topk, block_size, window_size, causal, q_offset, sm_scale, st))
+                               B, L, N, h_kv, G, D, topk, block_size, window_size, causal, q_offset, sm_scale, st,
+                               nullptr, 0, 0, 0, 0, per_qhead))
       return rc2;
     HILS_CHECK_LAUNCH("hils_topk_fwd");
     return HILS_OK;
@@ -2239,7 +2256,7 @@ extern "C" int hils_topk_fwd_weights_paged(const void* q, const void* lmk_pages,
                                            const float* lse_swa, const float* bias_pages, int32_t* indices, void* scores, void* weights,
                                            float* lse_total, float* sel_logits, int B, int L, int N, int h_kv,
                                            int G, int D, int topk, int block_size, int window_size, int q_offset,
-                                           int max_pages, int num_pages, float sm_scale, void* stream) {
+                                           int max_pages, int num_pages, float sm_scale, int per_qhead, void* stream) {
   HILS_REQUIRE(q && lmk_pages && page_table && lse_swa && indices && scores && weights,
                "hils_topk_fwd_weights_paged: null pointer");
   HILS_REQUIRE(B > 0 && L > 0 && N > 0 && h_kv > 0 && max_pages >= N && num_pages > 0,
@@ -2253,7 +2270,7 @@ extern "C" int hils_topk_fwd_weights_paged(const void* q, const void* lmk_pages,
                "hils_topk_fwd_weights_paged: too many chunks (%d) to stage the bias beside the logits", N);
   if (int rc = topk_fwd_row(q, lmk_pages, lse_swa, bias_pages, indices, scores, lse_total, sel_logits, weights, B, L,
                             N, h_kv, G, D, topk, block_size, window_size, 1, q_offset, sm_scale,
-                            (hipStream_t)stream, page_table, max_pages, num_pages))
+                            (hipStream_t)stream, page_table, max_pages, num_pages, 0, 0, per_qhead))
     return rc;
   HILS_CHECK_LAUNCH("hils_topk_fwd_weights_paged");
   return HILS_OK;

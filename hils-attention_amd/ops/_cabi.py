@@ -26,10 +26,10 @@ SIGNATURES = {
     "hils_topk_fwd_noalloc": [_P] * 10 + [_I] * 12 + [_F, _P],
     "hils_topk_fwd_weights": [_P] * 11 + [_Z] + [_I] * 12 + [_F, _P],
     "hils_topk_fwd_weights_lse16": [_P] * 9 + [_Z] + [_I] * 11 + [_F, _P],
-    "hils_topk_fwd_weights_paged": [_P] * 10 + [_I] * 12 + [_F, _P],
+    "hils_topk_fwd_weights_paged": [_P] * 10 + [_I] * 12 + [_F, _I, _P],
     "hils_sparse_attn_decode_paged": [_P] * 8 + [_Z] + [_I] * 9 + [_F, _I, _P],
-    "hils_decode_step": [_P] * 12 + [_I] * 11 + [_F, _F, _I, _I, _I, _P],
-    "hils_decode_step_paged": [_P] * 13 + [_I] * 12 + [_F, _F, _I, _I, _I, _I, _P],
+    "hils_decode_step": [_P] * 12 + [_I] * 11 + [_F, _F, _I, _I, _I, _I, _P],
+    "hils_decode_step_paged": [_P] * 13 + [_I] * 12 + [_F, _F, _I, _I, _I, _I, _I, _P],
     "hils_topk_bwd": [_P] * 7 + [_Z] + [_I] * 8 + [_F, _P],
     "hils_sparse_attn_fwd": [_P] * 10 + [_Z] + [_I] * 13 + [_F, _I, _F, _I, _P],
     "hils_pack_kv_chunks": [_P, _P, _P, _Z, _I, _I, _I, _I, _I, _P],

@@ -124,17 +124,19 @@ def topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, is_causa
     return indices, scores, weights
 
 
-def head_major_chunk_keys(lmks, prior_b=None, capacity=None):
-    """Chunk keys (B,N,h_kv,D) (and the prior bias (B,N,h_q)) re-laid head-major, (B,h_kv,cap,D) and
+def head_major_chunk_keys(lmks, prior_b=None, capacity=None, num_kv_heads=None):
+    """Chunk keys (B,N,h,D) (and the prior bias (B,N,h_q)) re-laid head-major, (B,h,cap,D) and
     (B,h_kv,cap,G): the N keys a decode row streams become one contiguous block.  What this
-    package's cache layers keep; ``decode_step(..., lmk_head_major=True)`` takes them."""
-    B, N, h_kv, D = lmks.shape
+    package's cache layers keep; ``decode_step(..., lmk_head_major=True)`` takes them.  ``num_kv_heads``:
+    needed for the bias when lmks carries one key per query head (h = h_q)."""
+    B, N, h, D = lmks.shape
     cap = N if capacity is None else int(capacity)
     assert cap >= N
-    out = torch.zeros((B, h_kv, cap, D), dtype=lmks.dtype, device=lmks.device)
+    out = torch.zeros((B, h, cap, D), dtype=lmks.dtype, device=lmks.device)
     out[:, :, :N] = lmks.permute(0, 2, 1, 3)
     if prior_b is None:
         return out
+    h_kv = h if num_kv_heads is None else int(num_kv_heads)
     G = prior_b.shape[2] // h_kv
     pb = torch.zeros((B, h_kv, cap, G), dtype=torch.float32, device=lmks.device)
     pb[:, :, :N] = prior_b.reshape(B, N, h_kv, G).permute(0, 2, 1, 3).float()
@@ -150,9 +152,10 @@ def decode_step(q, lmks, k, v, lse_swa, topk, block_size, window_size, q_offset=
     weights (B,L,h_q,topk+1), indices (B,L,h_kv,topk), scores (B,L,h_q,topk).  ``prior_b`` (B,N,h_q):
     the layer's prior bias (selection bias and the bias of the inter-chunk softmax).
     ``lmk_head_major``: lmks is (B,h_kv,cap,D) and prior_b (B,h_kv,cap,G) (``head_major_chunk_keys``),
-    of which the first ``num_chunks`` (default cap) chunks are looked at.  Shapes the fused kernel does
-    not take (few rows, short caches, more than four query heads per KV head, ...) run as the two
-    calls."""
+    of which the first ``num_chunks`` (default cap) chunks are looked at.  lmks may carry h_q heads
+    instead of h_kv (one chunk key per query head, the layer's attention-pooled keys): (B,N,h_q,D) or,
+    head-major, (B,h_q,cap,D).  Shapes the fused kernel does not take (few rows, short caches, more
+    than four query heads per KV head, ...) run as the two calls."""
     import math
     from .hils_fwd_bwd_head import HiLS_block_M_head
     _cabi.require_gpu_bf16("decode_step", q, lmks)
@@ -160,17 +163,20 @@ def decode_step(q, lmks, k, v, lse_swa, topk, block_size, window_size, q_offset=
     if torch.is_grad_enabled() and any(t.requires_grad for t in (q, lmks, k, v, lse_swa)):
         raise RuntimeError("decode_step is forward-only")
     B, L, h_q, D = q.shape
+    h_kv = k.shape[2]
     if lmk_head_major:
-        h_kv, cap = lmks.shape[1], lmks.shape[2]
+        h_lmk, cap = lmks.shape[1], lmks.shape[2]
         N = cap if num_chunks is None else int(num_chunks)
         assert 0 < N <= cap
     else:
-        N, h_kv = lmks.shape[1], lmks.shape[2]
+        N, h_lmk = lmks.shape[1], lmks.shape[2]
         cap = N
         assert num_chunks is None or int(num_chunks) == N
     Lkv = k.shape[1]
     assert lmks.shape[0] == B and lmks.shape[3] == D and k.shape == v.shape and k.shape[0] == B
-    assert k.shape[2] == h_kv and k.shape[3] == D and h_q % h_kv == 0
+    assert k.shape[3] == D and h_q % h_kv == 0
+    assert h_lmk in (h_kv, h_q), f"lmks carries {h_lmk} heads: neither the {h_kv} KV heads nor the {h_q} query heads"
+    per_qhead = int(h_lmk != h_kv)
     G = h_q // h_kv
     scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(D)
     lib = _cabi.load()
@@ -188,7 +194,7 @@ def decode_step(q, lmks, k, v, lse_swa, topk, block_size, window_size, q_offset=
             if pb is not None:
                 pb = pb[:, :, :N].permute(0, 2, 1, 3).reshape(B, N, h_q).contiguous()
         idx, sc, w = topk_chunk_weights(q, lmks, lse_swa, topk, block_size, window_size, q_offset=q_offset,
-                                        sm_scale=scale, prior_b=pb)
+                                        sm_scale=scale, prior_b=pb, num_kv_heads=h_kv)
         o = HiLS_block_M_head(q, k, v, w, idx, block_size=block_size, sm_scale=scale,
                               mask_last_token=mask_last_token, is_training=False)
         return o, w, idx, sc
@@ -207,7 +213,7 @@ def decode_step(q, lmks, k, v, lse_swa, topk, block_size, window_size, q_offset=
                _cabi.ptr(vv), _cabi.ptr(lse), _cabi.ptr(pb), _cabi.ptr(indices), _cabi.ptr(scores),
                _cabi.ptr(weights), _cabi.ptr(o), _cabi.ptr(lse_total), _cabi.ptr(sel_logits), B, L, Lkv, N, h_q,
                h_kv, D, int(topk), int(block_size), int(window_size), int(q_offset), scale, scale,
-               int(bool(mask_last_token)), int(bool(lmk_head_major)), cap)
+               int(bool(mask_last_token)), int(bool(lmk_head_major)), cap, per_qhead)
     if _debug is not None:
         _debug.update(lse_total=lse_total, sel_logits=sel_logits)
     return o, weights, indices, scores

@@ -207,19 +207,8 @@ class HiLSDynamicLayer:
             sm_scale = 1.0 / math.sqrt(q.shape[-1])
         H = self.keys.shape[2]
         q_offset = self.seq_len - q.shape[1]
-        if self._lmk_hm.shape[1] != H:
-            # one chunk key per query head: the general selection kernels on the reference's layout
-            n = self.pooled_chunks
-            lmk = self.lmk_k[:, :n].contiguous()
-            pb = None if self._prior_hm is None else self.prior_b[:, :n].contiguous()
-            idx, sc = online_softmax_topk_head(q, lmk, lse_swa, topk, S, window_size, q_offset=q_offset,
-                                               is_training=False, sm_scale=sm_scale, bias=pb,
-                                               G=lmk.shape[2] // H, _debug=_debug)
-            w = chunk_weights(sc, lse_swa, pb, idx)
-            o = HiLS_block_M_head(q, self.keys, self.values, w, idx, block_size=S, sm_scale=sm_scale,
-                                  is_training=False)
-            return o, w, idx
-        # one launch when the shape allows it (decode_step falls back to the two calls otherwise)
+        # one launch when the shape allows it (decode_step falls back to the two calls otherwise); the chunk
+        # keys are per KV head or, kept from the attention pool, per query head
         o, w, idx, _ = decode_step(q, self._lmk_hm, self.keys, self.values, lse_swa, topk, S, window_size,
                                    q_offset=q_offset, sm_scale=sm_scale, prior_b=self._prior_hm,
                                    lmk_head_major=True, num_chunks=max(self.pooled_chunks, 1), _debug=_debug)
@@ -231,6 +220,7 @@ class HiLSPagedLayer:
     backend keeps (the reference's SGLang backend requires page size = chunk size, README.md:262-264).
 
     ``k_pages`` / ``v_pages``: (num_pages, H, 64, D), the 64 tokens of a (page, head) contiguous;
+    (with ``chunk_pooling=False`` and ``num_q_heads`` the chunk keys below carry h_q heads, one per query head)
     ``page_table``: (B, max_pages) int32, chunk c of sequence b -> page, -1 = not mapped.  The pooled
     key of every full chunk is kept twice: per page in ``lmk_pages`` (num_pages, H, D) (with
     ``prior_pages`` (num_pages, h_q) beside it), and per sequence, dense and head-major, in ``lmk_hm``
@@ -249,15 +239,17 @@ class HiLSPagedLayer:
         self.num_pages, self.max_pages = int(num_pages), int(max_pages_per_seq)
         self.k_pages = torch.zeros((num_pages, self.H, self.S, self.D), dtype=dtype, device=device)
         self.v_pages = torch.zeros_like(self.k_pages)
-        self.lmk_pages = torch.zeros((num_pages, self.H, self.D), dtype=dtype, device=device)
-        self.lmk_hm = torch.zeros((self.B, self.H, self.max_pages, self.D), dtype=dtype, device=device)
+        self.chunk_pooling = bool(chunk_pooling)
+        # chunk keys per KV head (chunk means) or, kept from the attention pool, per query head
+        self.h_lmk = self.H if (self.chunk_pooling or num_q_heads is None) else int(num_q_heads)
+        self.lmk_pages = torch.zeros((num_pages, self.h_lmk, self.D), dtype=dtype, device=device)
+        self.lmk_hm = torch.zeros((self.B, self.h_lmk, self.max_pages, self.D), dtype=dtype, device=device)
         self.prior_pages = self.prior_hm = None
         self.has_prior = False  # set once update() has been given prior queries
         if num_q_heads is not None:
             G = int(num_q_heads) // self.H
             self.prior_pages = torch.zeros((num_pages, int(num_q_heads)), dtype=torch.float32, device=device)
             self.prior_hm = torch.zeros((self.B, self.H, self.max_pages, G), dtype=torch.float32, device=device)
-        self.chunk_pooling = bool(chunk_pooling)
         self.page_table = torch.full((self.B, self.max_pages), -1, dtype=torch.int32, device=device)
         # pages are handed out from the end of this list
         order = list(range(num_pages - 1, -1, -1)) if page_order is None else [int(p) for p in reversed(page_order)]
@@ -319,13 +311,15 @@ class HiLSPagedLayer:
                 self.prior_hm[:, :, c0:full] = lb.view(B, n, H, G).permute(0, 2, 1, 3)
                 self.has_prior = True
                 if pooled is None:
-                    assert G == 1, "attention-pooled chunk keys of a grouped layer are per query head"
-                    pooled = lk.reshape(-1, H, D)
+                    assert hq == self.h_lmk, "attention-pooled chunk keys are per query head"
+                    pooled = lk.reshape(-1, hq, D)
             else:
                 assert not self.has_prior, "this cache keeps a prior bias: update() needs mu_q for new chunks"
+            assert pooled.shape[1] == self.h_lmk, (
+                "a layer built without chunk pooling keeps the attention pool's keys: update() needs mu_q")
             pooled = pooled.to(self.lmk_pages.dtype)
             self.lmk_pages[pg] = pooled
-            self.lmk_hm[:, :, c0:full] = pooled.view(B, n, H, D).permute(0, 2, 1, 3)
+            self.lmk_hm[:, :, c0:full] = pooled.view(B, n, self.h_lmk, D).permute(0, 2, 1, 3)
             self.pooled_chunks = full
 
     def gather_contiguous(self):
@@ -357,9 +351,9 @@ def paged_hils_attend(q, k_pages, v_pages, lmk_pages, page_table, lse_swa, seq_l
     """Selection + inter-chunk softmax + sparse attention of the last ``q.shape[1]`` positions of a
     ``seq_len``-token sequence kept in pages (layouts: see ``HiLSPagedLayer``).  Chunk keys: per page
     (``lmk_pages`` (num_pages,H,D), prior bias ``prior_pages`` (num_pages,h_q)) or per sequence,
-    head-major (``lmk_dense`` (B,H,cap,D), prior bias ``prior_dense`` (B,H,cap,G)); the prior bias, when
-    given, is the selection bias and the bias of the inter-chunk softmax
-    (models/FlashHiLS/hils_attention.py:568-602)."""
+    head-major (``lmk_dense`` (B,H,cap,D), prior bias ``prior_dense`` (B,H,cap,G)); either may carry h_q
+    heads in place of H (one chunk key per query head); the prior bias, when given, is the selection
+    bias and the bias of the inter-chunk softmax (models/FlashHiLS/hils_attention.py:568-602)."""
     dense = lmk_dense is not None
     _cabi.require_gpu_bf16("paged_hils_attend", q, k_pages, v_pages, lmk_dense if dense else lmk_pages)
     B, Lq, HQ, D = q.shape
@@ -372,16 +366,19 @@ def paged_hils_attend(q, k_pages, v_pages, lmk_pages, page_table, lse_swa, seq_l
     N = seq_len // S  # chunks with a pooled key
     assert 0 < N <= max_pages
     cap = 0
+    h_lmk = lmk_dense.shape[1] if dense else lmk_pages.shape[1]
+    assert h_lmk in (H, HQ), f"the chunk keys carry {h_lmk} heads: neither the {H} KV heads nor the {HQ} query heads"
+    per_qhead = int(h_lmk != H)
     if dense:
         cap = lmk_dense.shape[2]
-        assert lmk_dense.shape == (B, H, cap, D) and lmk_dense.is_contiguous() and cap >= N
+        assert lmk_dense.shape == (B, h_lmk, cap, D) and lmk_dense.is_contiguous() and cap >= N
         bias = None
         if prior_dense is not None:
             assert prior_dense.shape == (B, H, cap, G) and prior_dense.dtype == torch.float32
             bias = prior_dense.contiguous()
         lmk_arg = lmk_dense
     else:
-        assert lmk_pages.shape == (num_pages, H, D) and lmk_pages.is_contiguous()
+        assert lmk_pages.shape == (num_pages, h_lmk, D) and lmk_pages.is_contiguous()
         bias = None
         if prior_pages is not None:
             assert prior_pages.shape == (num_pages, HQ) and prior_pages.dtype == torch.float32
@@ -406,7 +403,7 @@ def paged_hils_attend(q, k_pages, v_pages, lmk_pages, page_table, lse_swa, seq_l
                    _cabi.ptr(v_pages), _cabi.ptr(page_table), _cabi.ptr(lse), _cabi.ptr(bias), _cabi.ptr(indices),
                    _cabi.ptr(scores), _cabi.ptr(weights), _cabi.ptr(o), _cabi.ptr(lse_total), _cabi.ptr(sel_logits),
                    B, Lq, N, HQ, H, D, int(topk), S, int(window_size), seq_len - Lq, max_pages, num_pages,
-                   float(sm_scale), float(sm_scale), 1, int(dense), int(dense), cap)
+                   float(sm_scale), float(sm_scale), 1, int(dense), int(dense), cap, per_qhead)
         if _debug is not None:
             _debug.update(lse_total=lse_total, sel_logits=sel_logits, scores=scores)
         return o, weights, indices
@@ -416,14 +413,15 @@ def paged_hils_attend(q, k_pages, v_pages, lmk_pages, page_table, lse_swa, seq_l
         lmk_tm = lmk_dense[:, :, :N].permute(0, 2, 1, 3).contiguous()
         pb = None if bias is None else bias[:, :, :N].permute(0, 2, 1, 3).reshape(B, N, HQ).contiguous()
         indices, scores, weights = topk_chunk_weights(qc, lmk_tm, lse, topk, S, window_size,
-                                                      q_offset=seq_len - Lq, sm_scale=sm_scale, prior_b=pb)
+                                                      q_offset=seq_len - Lq, sm_scale=sm_scale, prior_b=pb,
+                                                      num_kv_heads=H)
         if _debug is not None:
             _debug.update(scores=scores)
     else:
         _cabi.call("hils_topk_fwd_weights_paged", _cabi.ptr(qc), _cabi.ptr(lmk_pages), _cabi.ptr(page_table),
                    _cabi.ptr(lse), _cabi.ptr(bias), _cabi.ptr(indices), _cabi.ptr(scores), _cabi.ptr(weights),
                    _cabi.ptr(lse_total), _cabi.ptr(sel_logits), B, Lq, N, H, G, D, int(topk), S, int(window_size),
-                   seq_len - Lq, max_pages, num_pages, float(sm_scale))
+                   seq_len - Lq, max_pages, num_pages, float(sm_scale), per_qhead)
         if _debug is not None:
             _debug.update(lse_total=lse_total, sel_logits=sel_logits, scores=scores)
     o = torch.empty((B, Lq, HQ, D), dtype=q.dtype, device=dev)

@@ -251,8 +251,9 @@ int hils_sparse_attn_bwd_f32(const float* q, const float* k, const float* v, con
  * int32 maps chunk c of batch element b to its page (negative or >= num_pages = unmapped: the chunk
  * is invisible to the selection and contributes nothing to the attention).
  *
- * hils_topk_fwd_weights_paged: selection + inter-chunk softmax as hils_topk_fwd_weights (shared
- * chunk keys, no noise / drop mask, causal), N = chunks of the sequence, L <= a few queries;
+ * hils_topk_fwd_weights_paged: selection + inter-chunk softmax as hils_topk_fwd_weights (no noise /
+ * drop mask, causal), N = chunks of the sequence, L <= a few queries; per_qhead != 0: one pooled key per
+ * query head, lmk_pages (num_pages, h_kv*G, D);
  * bias_pages (num_pages, h_kv*G) fp32 or NULL: the prior bias of every page (selection bias and the
  * bias of the inter-chunk softmax, as the layer uses it); lse_total / sel_logits optional as in
  * hils_topk_fwd.
@@ -263,7 +264,7 @@ int hils_topk_fwd_weights_paged(const void* q, const void* lmk_pages, const int3
                                 const float* lse_swa, const float* bias_pages, int32_t* indices, void* scores, void* weights,
                                 float* lse_total, float* sel_logits, int B, int L, int N, int h_kv, int G,
                                 int D, int topk, int block_size, int window_size, int q_offset,
-                                int max_pages, int num_pages, float sm_scale, void* stream);
+                                int max_pages, int num_pages, float sm_scale, int per_qhead, void* stream);
 size_t hils_sparse_attn_decode_paged_workspace(int B, int L, int HQ, int H, int D, int K);
 int hils_sparse_attn_decode_paged(const void* q, const void* k_pages, const void* v_pages,
                                   const int32_t* page_table, const void* weights, const int32_t* indices,
@@ -288,10 +289,13 @@ int hils_sparse_attn_decode_paged(const void* q, const void* k_pages, const void
  * then one contiguous block instead of 2*D-byte rows at a stride of H*2*D bytes (what this build's cache
  * layers keep).  The paged entry point takes lmk_pages (num_pages,H,D) addressed through the page
  * table, or, lmk_dense != 0, dense chunk keys in one of the two layouts above beside paged K and V.
+ * lmk_per_qhead != 0: one chunk key per QUERY head (the layer's attention-pooled keys,
+ * models/FlashHiLS/hils_attention.py:391-396): HQ heads in place of H in all three key layouts; a row
+ * then streams HQ/H times the key bytes.
  * bias: the layer's prior bias (models/FlashHiLS/hils_attention.py:568-602: the selection's `bias`
  * and the bias gathered into the inter-chunk softmax), fp32, NULL for none; laid out like the chunk
  * keys with the G heads of a KV head in place of D: (B,N,H*G), (B,H,lmk_cap,G) or (num_pages,H*G).
- * Covered shapes (hils_decode_step_covers returns 1): shared chunk keys, causal, block_size 64,
+ * Covered shapes (hils_decode_step_covers returns 1): causal, block_size 64,
  * D = Dv in {64, 128}, HQ/H <= 4, 256 <= N <= 4096 (fewer with a bias, which is staged in LDS beside
  * the logits: about 3300 chunks, 3000 on the paged entry point, at D = 128; the covers function knows),
  * topk <= 64, at least 96 rows B*L*H. */
@@ -300,13 +304,15 @@ int hils_decode_step(const void* q, const void* lmks, const void* k, const void*
                      const float* bias, int32_t* indices, void* scores, void* weights, void* o,
                      float* lse_total, float* sel_logits, int B, int L, int Lkv, int N, int HQ, int H, int D,
                      int topk, int block_size, int window_size, int q_offset, float sm_scale_sel,
-                     float sm_scale_attn, int mask_last, int lmk_head_major, int lmk_cap, void* stream);
+                     float sm_scale_attn, int mask_last, int lmk_head_major, int lmk_cap, int lmk_per_qhead,
+                     void* stream);
 int hils_decode_step_paged(const void* q, const void* lmk_pages, const void* k_pages, const void* v_pages,
                            const int32_t* page_table, const float* lse_swa, const float* bias, int32_t* indices,
                            void* scores, void* weights, void* o, float* lse_total, float* sel_logits, int B,
                            int L, int N, int HQ, int H, int D, int topk, int block_size, int window_size,
                            int q_offset, int max_pages, int num_pages, float sm_scale_sel, float sm_scale_attn,
-                           int mask_last, int lmk_dense, int lmk_head_major, int lmk_cap, void* stream);
+                           int mask_last, int lmk_dense, int lmk_head_major, int lmk_cap, int lmk_per_qhead,
+                           void* stream);
 
 /* ---- exact per-chunk log Z ---------------------------------------------------- */
 

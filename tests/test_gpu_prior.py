@@ -145,6 +145,73 @@ def test_decode_step_with_prior_bias(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
     assert not torch.equal(idx3, idx1), "the bias must change the selection"
 
 
+@pytest.mark.parametrize("B,Lq,Lkv,HQ,H,D,K", [(32, 1, 32768, 32, 8, 128, 32), (50, 2, 20480, 4, 1, 128, 8),
+                                               (24, 1, 65536, 12, 4, 64, 64), (48, 1, 16512, 6, 2, 64, 16)])
+def test_decode_step_with_a_key_per_query_head(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
+    """The layer's default pooling in decode: one attention-pooled chunk key per query head and its
+    prior bias.  One launch per step; token-major, head-major and paged keys give the same bits; the
+    selection rule holds on the kernel's own logits, which match the oracle's per-head products."""
+    note(f"decode_step, key per query head, B{B} Lq{Lq} Lkv{Lkv} HQ{HQ} H{H} D{D} K{K}")
+    S, W = 64, 1
+    G, N, off = HQ // H, Lkv // 64, Lkv - Lq
+    gen = torch.Generator().manual_seed(405)
+    q = torch.randn(B, Lq, HQ, D, generator=gen).bfloat16()
+    k = torch.randn(B, Lkv, H, D, generator=gen).bfloat16()
+    v = torch.randn(B, Lkv, H, D, generator=gen).bfloat16()
+    lmk = torch.randn(B, N, HQ, D, generator=gen).bfloat16()
+    lse = torch.randn(B, Lq, HQ, generator=gen) * 3 + 5
+    pb = torch.randn(B, N, HQ, generator=gen) * 2
+    qd, kd, vd, lmkd, lsed, pbd = q.to(dev), k.to(dev), v.to(dev), lmk.to(dev), lse.to(dev), pb.to(dev)
+    dbg = {}
+    o1, w1, idx1, sc1 = pkg.decode_step(qd, lmkd, kd, vd, lsed, K, S, W, q_offset=off, prior_b=pbd, _debug=dbg)
+    assert dbg, "the one-launch kernel did not take this shape"
+    lim = orc.causal_chunk_limit(Lq, off, W, S)
+    want = orc.topk_select(dbg["sel_logits"].cpu(), dbg["lse_total"].cpu(), lim, K)
+    assert torch.equal(idx1.cpu(), want)
+    ridx, _, aux = orc.online_softmax_topk_head(q.view(B, Lq, H, G, D), lmk, lse, K, S, W, q_offset=off, bias=pb,
+                                                return_aux=True)
+    assert_close_f32(dbg["sel_logits"].cpu(), aux["sel_logits"], 2e-3, "biased selection logits")
+    assert_close_f32(dbg["lse_total"].cpu(), aux["lse_total"], 1e-3, "lse_total")
+    assert (idx1.cpu() == ridx).float().mean().item() >= 0.99
+    safe = idx1.cpu().long().clamp_min(0).unsqueeze(3).expand(-1, -1, -1, G, -1)
+    raw = torch.gather(aux["logits"], -1, safe).masked_fill((idx1.cpu() < 0).unsqueeze(3).expand(-1, -1, -1, G, -1),
+                                                             float("-inf"))
+    assert_close_bf16(sc1.view(B, Lq, H, G, K), raw, "scores carry no bias")
+    w_ref = orc.inter_chunk_softmax(sc1.float().cpu(), lse, pb.bfloat16().float(), idx1.cpu(), bf16_sum=True)
+    assert_close_bf16(w1, w_ref, "weights with prior bias", max_abs=8e-3)
+    assert_close_bf16(o1, orc.sparse_attn(q, k, v, w1.cpu(), idx1.cpu(), chunk_size=S), "decode_step output")
+    # the operators one by one (the selection alone runs on the same row kernel)
+    idx0, sc0 = pkg.online_softmax_topk_head(qd, lmkd, lsed, K, S, W, q_offset=off, is_training=False, bias=pbd, G=G)
+    assert torch.equal(idx1, idx0) and torch.equal(sc1, sc0)
+    w0 = pkg.chunk_weights(sc0, lsed, pbd, idx0)
+    assert (w1.float() - w0.float()).abs().max().item() <= 4e-3
+    # head-major keys and bias with spare capacity: the same bits
+    lmk_hm, pb_hm = pkg.head_major_chunk_keys(lmkd, pbd, capacity=N + 5, num_kv_heads=H)
+    o2, w2, idx2, sc2 = pkg.decode_step(qd, lmk_hm, kd, vd, lsed, K, S, W, q_offset=off, prior_b=pb_hm,
+                                        lmk_head_major=True, num_chunks=N)
+    assert torch.equal(idx2, idx1) and torch.equal(sc2, sc1) and torch.equal(w2, w1) and torch.equal(o2, o1)
+    # pages: keys per page and per sequence
+    if Lkv % 64 == 0:
+        num_pages = B * N + 3
+        perm = torch.randperm(num_pages, generator=gen)[: B * N].view(B, N).to(dev)
+        k_pages = torch.randn(num_pages, H, 64, D, generator=gen).bfloat16().to(dev)
+        v_pages = torch.randn(num_pages, H, 64, D, generator=gen).bfloat16().to(dev)
+        lmk_pages = torch.randn(num_pages, HQ, D, generator=gen).bfloat16().to(dev)
+        pb_pages = torch.randn(num_pages, HQ, generator=gen).to(dev)
+        k_pages[perm] = kd.view(B, N, 64, H, D).permute(0, 1, 3, 2, 4)
+        v_pages[perm] = vd.view(B, N, 64, H, D).permute(0, 1, 3, 2, 4)
+        lmk_pages[perm] = lmkd
+        pb_pages[perm] = pbd
+        table = torch.full((B, N + 2), -1, dtype=torch.int32, device=dev)
+        table[:, :N] = perm.to(torch.int32)
+        o3, w3, idx3 = pkg.paged_hils_attend(qd, k_pages, v_pages, lmk_pages, table, lsed, Lkv, K, W, prior_pages=pb_pages)
+        assert torch.equal(idx3, idx1) and torch.equal(w3, w1) and torch.equal(o3, o1)
+        lmk_hm2, pb_hm2 = pkg.head_major_chunk_keys(lmkd, pbd, capacity=N + 2, num_kv_heads=H)
+        o4, w4, idx4 = pkg.paged_hils_attend(qd, k_pages, v_pages, None, table, lsed, Lkv, K, W, lmk_dense=lmk_hm2,
+                                             prior_dense=pb_hm2)
+        assert torch.equal(idx4, idx1) and torch.equal(w4, w1) and torch.equal(o4, o1)
+
+
 def test_paged_decode_with_prior_bias(pkg, orc, dev):
     """The paged cache: per-page chunk keys / bias and the per-sequence head-major ones give the bits
     of the token-major decode step."""
@@ -188,7 +255,7 @@ def test_paged_decode_with_prior_bias(pkg, orc, dev):
     assert_close_bf16(o3, o4.float(), "paged two-call path vs dense two-call path")
 
 
-@pytest.mark.parametrize("G,chunk_pooling", [(4, True), (1, False), (2, False)])
+@pytest.mark.parametrize("G,chunk_pooling", [(4, True), (1, False), (2, False), (4, False)])
 def test_cache_layers_keep_and_use_the_prior(pkg, orc, dev, G, chunk_pooling):
     """HiLSDynamicLayer / HiLSPagedLayer filled incrementally with the chunks' prior queries: the
     entropy bias (and, without chunk pooling, the attention-pooled keys) match the oracle's attention
@@ -205,7 +272,7 @@ def test_cache_layers_keep_and_use_the_prior(pkg, orc, dev, G, chunk_pooling):
     kd, vd, mud = k.to(dev), v.to(dev), mu.to(dev)
     dyn = pkg.HiLSDynamicLayer(chunk_size=S, capacity=256, chunk_pooling=chunk_pooling)
     paged = None
-    if chunk_pooling or G == 1:
+    if True:
         paged = pkg.HiLSPagedLayer(num_pages=40, batch=B, max_pages_per_seq=12, num_kv_heads=H, head_dim=D,
                                    device=dev, num_q_heads=HQ, chunk_pooling=chunk_pooling,
                                    page_order=torch.randperm(40, generator=gen).tolist())
