@@ -207,6 +207,12 @@ def bench_decode(pkg, dev, steps, warmup):
     prior_hm = torch.randn(B, H, N, HQ // H, device=dev, generator=gen)
     prior_sec = time_steps(lambda: pkg.decode_step(q, lmk_hm, kc, vc, lse_swa, K, S, W, q_offset=Lkv - 1,
                                                    prior_b=prior_hm, lmk_head_major=True), steps, warmup)
+    # and with one chunk key per query head beside that bias (attention-pooled keys, the layer's default
+    # pooling): four times the key bytes per step
+    lmk_q_hm = gpu_randn((B, HQ, N, D), gen, dev)
+    perq_sec = time_steps(lambda: pkg.decode_step(q, lmk_q_hm, kc, vc, lse_swa, K, S, W, q_offset=Lkv - 1,
+                                                  prior_b=prior_hm, lmk_head_major=True), steps, warmup)
+    del lmk_q_hm
     two_call_sec = time_steps(step2, steps, warmup)
     for _ in range(min(steps, 5)):
         step2(record=True)
@@ -214,6 +220,7 @@ def bench_decode(pkg, dev, steps, warmup):
     per["two_call_step"] = two_call_sec * 1e3
     per["token_major_keys_step"] = token_major_sec * 1e3
     per["prior_bias_step"] = prior_sec * 1e3
+    per["key_per_query_head_prior_bias_step"] = perq_sec * 1e3
     # the serving loop replays the step as one HIP graph (no host work between kernels)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
