@@ -1820,6 +1820,7 @@ struct DsArgs {
   float sm_scale_sel;
   const int32_t* page_table;
   int max_pages, num_pages, lmk_hm, lmk_cap, perq;
+  int stagger_ticks;  // 100 MHz ticks by which every other row of an XCD starts late (0: none)
   DrDims dr;
 };
 // PAGED: the chunk keys (and the bias) are addressed through the page table; the attention reads
@@ -1829,6 +1830,15 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_step_kernel(DsArgs a) {
   extern __shared__ __align__(16) float ds_dyn[];
   const long row = blockIdx.x;
   __shared__ TopkRowShared ds_sh;
+  // With at most one row per compute unit all rows run in step: every compute unit streams keys, then
+  // every one sits in the selection's tail with the memory system idle, then every one streams K and V.
+  // Half of the rows (every other one of an XCD's) start a little late, so that one half's tail falls
+  // into the other half's streaming (75.5 -> 72.2 us at 256 rows of 2048 keys with 8 us; 5 us: 75.0,
+  // 12 us: 74.2; thirds or a continuous spread of the start times did less).
+  if (a.stagger_ticks > 0 && ((blockIdx.x >> 3) & 1)) {
+    const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+    while (__builtin_amdgcn_s_memrealtime() - t0 < (unsigned long long)a.stagger_ticks) __builtin_amdgcn_s_sleep(8);
+  }
   topk_row_body<D, 4, DS_WAVES, PAGED, true>(a.q, a.lmks, a.lse_swa, a.bias, a.indices, a.scores, a.lse_total,
                                              a.sel_logits, a.weights, a.L, a.N, a.NP, a.h_kv, a.G, a.topk,
                                              a.block_size, a.window_size, 1, a.q_offset, a.sm_scale_sel,
@@ -1943,6 +1953,7 @@ static int decode_step_launch(const void* q, const void* lmks, const void* k, co
   a.q = (const bf16_t*)q; a.lmks = (const bf16_t*)lmks; a.k = (const bf16_t*)k; a.v = (const bf16_t*)v;
   a.lse_swa = lse_swa; a.bias = bias; a.indices = indices;
   a.lmk_hm = lmk_hm; a.lmk_cap = lmk_cap; a.perq = perq;
+  a.stagger_ticks = rows <= topk_cus() ? 800 : 0;  // one round of rows: they would run in step
   a.scores = (bf16_t*)scores; a.weights = (bf16_t*)weights; a.o = (bf16_t*)o;
   a.lse_total = lse_total; a.sel_logits = sel_logits;
   a.L = L; a.N = N; a.NP = NP; a.h_kv = H; a.G = G; a.topk = topk; a.block_size = block_size;
