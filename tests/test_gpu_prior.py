@@ -146,7 +146,8 @@ def test_decode_step_with_prior_bias(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
 
 
 @pytest.mark.parametrize("B,Lq,Lkv,HQ,H,D,K", [(32, 1, 32768, 32, 8, 128, 32), (50, 2, 20480, 4, 1, 128, 8),
-                                               (24, 1, 65536, 12, 4, 64, 64), (48, 1, 16512, 6, 2, 64, 16)])
+                                               (24, 1, 65536, 12, 4, 64, 64), (48, 1, 16512, 6, 2, 64, 16),
+                                               (48, 1, 16384, 4, 2, 64, 8)])
 def test_decode_step_with_a_key_per_query_head(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
     """The layer's default pooling in decode: one attention-pooled chunk key per query head and its
     prior bias.  One launch per step; token-major, head-major and paged keys give the same bits; the
