@@ -1261,7 +1261,9 @@ __device__ __forceinline__ float wave_sum_f(float x) {
          (__int_as_float(__builtin_amdgcn_readlane(xi, 32)) + __int_as_float(__builtin_amdgcn_readlane(xi, 48)));
 }
 
-struct TopkRowShared {
+// GM: the query heads of a row the kernel is built for (4 or 8)
+template <int GM>
+struct TopkRowSharedT {
   float cand_s[TOPK_R_WAVES][64];
   int cand_i[TOPK_R_WAVES][64];
   float merge_s[TOPK_R_WAVES * TOPK_MAXK];
@@ -1269,14 +1271,14 @@ struct TopkRowShared {
   int ncand[TOPK_R_WAVES];
   // (max, sum of exponentials) of every streamed key group, one component per head: combined in a
   // fixed order, so the log-sum-exp does not depend on which wavefront drew which group
-  float grp_m[TOPK_R_MAXN / 32][4];
-  float grp_l[TOPK_R_MAXN / 32][4];
+  float grp_m[TOPK_R_MAXN / 32][GM];
+  float grp_l[TOPK_R_MAXN / 32][GM];
   uint32_t gmax[64];           // largest selection key of every 16-lane group of the workgroup
   int wcnt[TOPK_R_WAVES];      // keys of a wavefront that reach the candidate bound
-  float tot[4];                // lse_total per head
+  float tot[GM];               // lse_total per head
   int rank[64];                            // one-launch decode step: candidates ahead of each candidate
   int win_i[TOPK_MAXK];                    // ... the winners' chunks, ascending, -1 padded
-  bf16_t win_w[4 * (TOPK_MAXK + 1) + 2];   // ... and the heads' inter-chunk weights, [head][topk + 1]
+  bf16_t win_w[GM * (TOPK_MAXK + 1) + 2];   // ... and the heads' inter-chunk weights, [head][topk + 1]
   uint32_t thr;                // the candidate bound
   int next_group;
 };
@@ -1296,7 +1298,7 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
               float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
               int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
               float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages,
-              int lmk_hm, int lmk_cap, int perq, float* dyn, const long row, TopkRowShared* sh_p = nullptr) {
+              int lmk_hm, int lmk_cap, int perq, float* dyn, const long row, TopkRowSharedT<GMAX>* sh_p = nullptr) {
   // perq: one chunk key per QUERY head, lmks = (B,N,h_kv*G,D) / (B,h_kv*G,lmk_cap,D) / (num_pages,h_kv*G,D):
   // the row streams G key tensors, a key group of head g gives the logits of MFMA column g only
   constexpr int LR = D / 8, TPI = 64 / LR;
@@ -1314,8 +1316,8 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   // staged head-major like the logits; 0 for the chunks past the causal limit
   float* bias_s = (float*)(page_s + NPG);     // [GMAX][NP], only with a bias
   const int NBS = bias ? GMAX * NP : 0;       // the wavefronts' staging areas follow
-  __shared__ TopkRowShared sh_own;
-  TopkRowShared& sh = FUSED ? *sh_p : sh_own;  // FUSED: the caller's, which the attention reads after the return
+  __shared__ TopkRowSharedT<GMAX> sh_own;
+  TopkRowSharedT<GMAX>& sh = FUSED ? *sh_p : sh_own;  // FUSED: the caller's, which the attention reads after the return
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int piece = lane % LR, tsub = lane / LR;
   const int hk = (int)(row % h_kv);
@@ -1500,7 +1502,7 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   // ---- phase 2: LSE per head from the key groups' partial sums.  Work every wavefront would do
   // alike costs its instruction count once per wavefront of a SIMD, so one wavefront per head does
   // it and the result goes through LDS ----
-  static_assert(GMAX == 4 && NW >= GMAX, "one wavefront per head, four heads per group entry");
+  static_assert((GMAX == 4 || GMAX == 8) && NW >= GMAX, "one wavefront per head, four or eight heads per group entry");
   if (wave < GMAX) {
     const int g = wave;
     const int ngroups = (lim + KG - 1) / KG;
@@ -1825,11 +1827,11 @@ struct DsArgs {
 };
 // PAGED: the chunk keys (and the bias) are addressed through the page table; the attention reads
 // K and V through it whenever a.dr.page_table is set.
-template <int D, bool PAGED>
+template <int D, bool PAGED, int GMAX>
 __global__ void __launch_bounds__(DS_WAVES * 64) decode_step_kernel(DsArgs a) {
   extern __shared__ __align__(16) float ds_dyn[];
   const long row = blockIdx.x;
-  __shared__ TopkRowShared ds_sh;
+  __shared__ TopkRowSharedT<GMAX> ds_sh;
   // With at most one row per compute unit all rows run in step: every compute unit streams keys, then
   // every one sits in the selection's tail with the memory system idle, then every one streams K and V.
   // Half of the rows (every other one of an XCD's) start a little late, so that one half's tail falls
@@ -1839,7 +1841,7 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_step_kernel(DsArgs a) {
     const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
     while (__builtin_amdgcn_s_memrealtime() - t0 < (unsigned long long)a.stagger_ticks) __builtin_amdgcn_s_sleep(8);
   }
-  topk_row_body<D, 4, DS_WAVES, PAGED, true>(a.q, a.lmks, a.lse_swa, a.bias, a.indices, a.scores, a.lse_total,
+  topk_row_body<D, GMAX, DS_WAVES, PAGED, true>(a.q, a.lmks, a.lse_swa, a.bias, a.indices, a.scores, a.lse_total,
                                              a.sel_logits, a.weights, a.L, a.N, a.NP, a.h_kv, a.G, a.topk,
                                              a.block_size, a.window_size, 1, a.q_offset, a.sm_scale_sel,
                                              a.page_table, a.max_pages, a.num_pages, a.lmk_hm, a.lmk_cap, a.perq,
@@ -1866,20 +1868,24 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
                            float sm_scale, int lse_bf16, int per_qhead, void* stream);
 
 // rows = (query, KV head) pairs; the row kernel wants about one row per compute unit
-// LDS of a row workgroup before the wavefronts' staging areas: raw logits [4][NP], pooled scores, page
-// ids (paged chunk keys), the staged bias [4][NP]
-static size_t topk_row_smem_base(int N, bool paged, bool with_bias) {
+// LDS of a row workgroup before the wavefronts' staging areas: raw logits [gm][NP] (gm = 4 head slots, 8
+// with more than four query heads per KV head), pooled scores, page ids (paged chunk keys), the staged
+// bias [gm][NP]
+static size_t topk_row_smem_base(int N, int G, bool paged, bool with_bias) {
   const int NP = (N + 63) & ~63;
-  return (size_t)(5 + (paged ? 1 : 0) + (with_bias ? 4 : 0)) * NP * sizeof(float);
+  const int gm = G <= 4 ? 4 : 8;
+  return (size_t)(gm + 1 + (paged ? 1 : 0) + (with_bias ? gm : 0)) * NP * sizeof(float);
 }
+static size_t topk_row_shared_bytes(int G) { return G <= 4 ? sizeof(TopkRowSharedT<4>) : sizeof(TopkRowSharedT<8>); }
 
 // plain: no Gumbel noise and no drop mask; a bias is staged in LDS beside the logits and must fit there
 static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool plain, bool with_bias = false,
                          bool paged = false) {
-  if (with_bias && topk_row_smem_base(N, paged, true) + (size_t)8 * 16 * (2 * D + 16) + sizeof(TopkRowShared) > 158 * 1024)
+  if ((with_bias || G > 4) &&
+      topk_row_smem_base(N, G, paged, with_bias) + (size_t)8 * 16 * (2 * D + 16) + topk_row_shared_bytes(G) > 158 * 1024)
     return false;
   (void)per_qhead;  // shared chunk keys or one per query head: the same kernel
-  return plain && G <= 4 && (D == 64 || D == 128) && N >= 256 && N <= TOPK_R_MAXN &&
+  return plain && G <= 8 && (D == 64 || D == 128) && N >= 256 && N <= TOPK_R_MAXN &&
          rows >= 96 && rows <= 2147483647L;
 }
 
@@ -1891,16 +1897,16 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, c
   const long rows = (long)B * L * h_kv;
   const int NP = (N + 63) & ~63;
   // then 16 padded key rows of staging per wavefront
-  const size_t smem_base = topk_row_smem_base(N, page_table != nullptr, bias != nullptr);
+  const size_t smem_base = topk_row_smem_base(N, G, page_table != nullptr, bias != nullptr);
   const size_t stage_b = (size_t)16 * (2 * D + 16);
   // one round of rows or less: 16 wavefronts per row (the whole compute unit streams one row) if
   // their staging areas fit the LDS beside the logits; more rows than compute units: 8, so that
   // two workgroups share a unit and one row's selection overlaps the other row's streaming
-  const bool wide = rows <= topk_cus() && smem_base + 16 * stage_b + sizeof(TopkRowShared) <= 158 * 1024;
+  const bool wide = rows <= topk_cus() && smem_base + 16 * stage_b + topk_row_shared_bytes(G) <= 158 * 1024;
   const size_t smem = smem_base + (wide ? 16 : 8) * stage_b;
-#define TOPK_ROW_CALL_W(D_, W_, P_)                                                               \
+#define TOPK_ROW_CALL_G(D_, G_, W_, P_)                                                           \
   do {                                                                                           \
-    auto kern = topk_row_kernel<D_, 4, W_, P_>;                                                  \
+    auto kern = topk_row_kernel<D_, G_, W_, P_>;                                                 \
     static HilsLdsReserve reserved;                                                              \
     if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_topk_fwd")) return rc; \
     hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(W_ * 64), smem, st,                      \
@@ -1908,6 +1914,10 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, c
                        lse_total, sel_logits, (bf16_t*)weights, L, N, NP, h_kv, G, topk,         \
                        block_size, window_size, causal, q_offset, sm_scale, page_table, max_pages, \
                        num_pages, lmk_hm, lmk_cap, perq);                                        \
+  } while (0)
+#define TOPK_ROW_CALL_W(D_, W_, P_)                                                               \
+  do {                                                                                           \
+    if (G <= 4) TOPK_ROW_CALL_G(D_, 4, W_, P_); else TOPK_ROW_CALL_G(D_, 8, W_, P_);             \
   } while (0)
 #define TOPK_ROW_CALL(D_, P_)                                                                    \
   do {                                                                                           \
@@ -1920,6 +1930,7 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, c
   }
 #undef TOPK_ROW_CALL
 #undef TOPK_ROW_CALL_W
+#undef TOPK_ROW_CALL_G
   return HILS_OK;
 }
 
@@ -1944,9 +1955,9 @@ static int decode_step_launch(const void* q, const void* lmks, const void* k, co
   const int G = HQ / H;
   const long rows = (long)B * L * H;
   const int NP = (N + 63) & ~63;
-  const size_t sel_b = topk_row_smem_base(N, lmk_paged != 0, bias != nullptr) + (size_t)DS_WAVES * 16 * (2 * D + 16);
-  HILS_REQUIRE(sel_b + sizeof(TopkRowShared) <= 158 * 1024,
-               "hils_decode_step: too many chunks (%d) to stage the bias beside the logits", N);
+  const size_t sel_b = topk_row_smem_base(N, G, lmk_paged != 0, bias != nullptr) + (size_t)DS_WAVES * 16 * (2 * D + 16);
+  HILS_REQUIRE(sel_b + topk_row_shared_bytes(G) <= 158 * 1024,
+               "hils_decode_step: too many chunks (%d) for the logits (and the bias) of the row's heads in LDS", N);
   const size_t att_b = dr_smem_bytes(D, G, DS_WAVES);
   const size_t smem = sel_b > att_b ? sel_b : att_b;
   DsArgs a;
@@ -1961,12 +1972,16 @@ static int decode_step_launch(const void* q, const void* lmks, const void* k, co
   a.page_table = page_table; a.max_pages = max_pages; a.num_pages = num_pages;
   a.dr = DrDims{L, Lkv, HQ, H, G, topk, topk + 1, page_table ? max_pages : Lkv / DR_S, 1, mask_last,
                 sm_scale_attn, page_table, max_pages, num_pages};
-#define DS_CALL(D_, P_)                                                                            \
+#define DS_CALL_G(D_, P_, G_)                                                                      \
   do {                                                                                             \
-    auto kern = decode_step_kernel<D_, P_>;                                                        \
+    auto kern = decode_step_kernel<D_, P_, G_>;                                                    \
     static HilsLdsReserve reserved;                                                                \
     if (int rc = hils_reserve_lds(&reserved, (const void*)kern, smem, "hils_decode_step")) return rc; \
     hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(DS_WAVES * 64), smem, st, a);              \
+  } while (0)
+#define DS_CALL(D_, P_)                                                                            \
+  do {                                                                                             \
+    if (G <= 4) DS_CALL_G(D_, P_, 4); else DS_CALL_G(D_, P_, 8);                                   \
   } while (0)
   if (lmk_paged) {
     if (D == 64) DS_CALL(64, true); else DS_CALL(128, true);
@@ -1974,6 +1989,7 @@ static int decode_step_launch(const void* q, const void* lmks, const void* k, co
     if (D == 64) DS_CALL(64, false); else DS_CALL(128, false);
   }
 #undef DS_CALL
+#undef DS_CALL_G
   return HILS_OK;
 }
 
@@ -2044,7 +2060,7 @@ extern "C" size_t hils_topk_fwd_workspace(int B, int L, int N, int h_kv, int G) 
   // many queries: room for the chunk keys repacked into MFMA operand order (head dim up to 128; a key
   // per query head when the caller's keys are per query head)
   if (!topk_use_split(B, L, N, h_kv))
-    return G <= 4 ? (size_t)B * h_kv * G * ((N + 15) / 16) * 16 * 128 * sizeof(bf16_t) : 0;
+    return G <= 8 ? (size_t)B * h_kv * G * ((N + 15) / 16) * 16 * 128 * sizeof(bf16_t) : 0;
   return (size_t)B * L * h_kv * G * N * sizeof(float);
 }
 
@@ -2131,15 +2147,17 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
     HILS_CHECK_LAUNCH("hils_topk_fwd");
     return HILS_OK;
   }
-  // one chunk key per query head: the one-pass kernel's four-wavefront form (G = 3, 4)
-  if (per_qhead && workspace && hils_topk_group_covers(N, G, D, topk, 1, !gumbel && !drop_mask)) {
+  // the one-pass kernel with one chunk key per query head (a wavefront per head for the logits, G = 3..8),
+  // or with more than four query heads on shared keys (two wavefronts per four queries)
+  if ((per_qhead || G > 4) && workspace && hils_topk_group_covers(N, G, D, topk, per_qhead, !gumbel && !drop_mask)) {
     const int nblk16 = (N + 15) / 16;
-    const long total = (long)B * h_kv * G * nblk16 * (D / 32) * 64;
+    const int h_lmk = per_qhead ? h_kv * G : h_kv;
+    const long total = (long)B * h_lmk * nblk16 * (D / 32) * 64;
     hipLaunchKernelGGL(topk_pack_lmk_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                       (const bf16_t*)lmks, (uint4*)workspace, N, h_kv * G, D, nblk16, total);
+                       (const bf16_t*)lmks, (uint4*)workspace, N, h_lmk, D, nblk16, total);
     if (int rc2 = hils_topk_group_launch(q, workspace, lse_swa, bias, indices, scores, lse_total, sel_logits, B, L, N,
                                          h_kv, G, D, topk, block_size, window_size, causal, q_offset, sm_scale,
-                                         lse_bf16, 1, stream))
+                                         lse_bf16, per_qhead ? 1 : 0, stream))
       return rc2;
     HILS_CHECK_LAUNCH("hils_topk_fwd");
     return HILS_OK;
@@ -2272,13 +2290,13 @@ extern "C" int hils_topk_fwd_weights_paged(const void* q, const void* lmk_pages,
                "hils_topk_fwd_weights_paged: null pointer");
   HILS_REQUIRE(B > 0 && L > 0 && N > 0 && h_kv > 0 && max_pages >= N && num_pages > 0,
                "hils_topk_fwd_weights_paged: sizes must be positive and the page table must cover N chunks");
-  HILS_REQUIRE(G >= 1 && G <= 4 && (D == 64 || D == 128) && N <= TOPK_R_MAXN && topk >= 1 && topk <= TOPK_MAXK &&
+  HILS_REQUIRE(G >= 1 && G <= 8 && (D == 64 || D == 128) && N <= TOPK_R_MAXN && topk >= 1 && topk <= TOPK_MAXK &&
                    block_size > 0,
-               "hils_topk_fwd_weights_paged: needs G <= 4, D in {64, 128}, N <= %d, topk <= %d", TOPK_R_MAXN,
+               "hils_topk_fwd_weights_paged: needs G <= 8, D in {64, 128}, N <= %d, topk <= %d", TOPK_R_MAXN,
                TOPK_MAXK);
   HILS_REQUIRE((long)B * L * h_kv <= 2147483647L, "hils_topk_fwd_weights_paged: grid too large");
-  HILS_REQUIRE(!bias_pages || topk_row_smem_base(N, true, true) + (size_t)8 * 16 * (2 * D + 16) + sizeof(TopkRowShared) <= 158 * 1024,
-               "hils_topk_fwd_weights_paged: too many chunks (%d) to stage the bias beside the logits", N);
+  HILS_REQUIRE((!bias_pages && G <= 4) || topk_row_smem_base(N, G, true, bias_pages != nullptr) + (size_t)8 * 16 * (2 * D + 16) + topk_row_shared_bytes(G) <= 158 * 1024,
+               "hils_topk_fwd_weights_paged: too many chunks (%d) for the logits (and the bias) of the row's heads in LDS", N);
   if (int rc = topk_fwd_row(q, lmk_pages, lse_swa, bias_pages, indices, scores, lse_total, sel_logits, weights, B, L,
                             N, h_kv, G, D, topk, block_size, window_size, 1, q_offset, sm_scale,
                             (hipStream_t)stream, page_table, max_pages, num_pages, 0, 0, per_qhead))

@@ -18,7 +18,10 @@
 //     exactly K; ties at the threshold go to the lower chunk indices,
 //   * the ascending order of the winners from a 512-bit map of the winning chunks in LDS
 //     (rank = set bits below the chunk), and the winners' raw scores straight from the logits.
-// Covers shared chunk keys, G <= 4, D in {64, 128}, N <= 512, topk <= 32, an optional additive bias per
+// Five to eight query heads per KV head (HALF below) take two wavefronts per four queries, one for the
+// heads 0..3 and one for the rest: each forms the partial selection scores of its heads, the two
+// trade them through LDS, and both then select on the same scores and write their own heads' outputs.
+// Covers G = 1 and 3..8, D in {64, 128}, N <= 512, topk <= 32, an optional additive bias per
 // (chunk, head) (the layer's prior bias), no Gumbel noise / drop mask; everything else runs on the
 // kernels of topk.hip.  With a bias the registers hold the biased logits (what the log-sum-exp and
 // the selection work on) and a winner's raw score is its logit minus the bias again.
@@ -137,9 +140,13 @@ __device__ __forceinline__ uint32_t tg_kth_largest(const uint32_t (&k)[NE], uint
 // rows, that head's keys streamed once for 16 queries), and block by block the four wavefronts
 // trade accumulators through LDS so that each ends up with the rows the shared-key layout gives it
 // (its 4 queries x 4 heads); everything behind the logits is the same code.
-template <int GMAX, int KS, int NB, bool EXPORT, bool BIAS, bool PERQ>
-__global__ void __launch_bounds__(64 * (PERQ ? 4 : TG_WAVES))
-    __attribute__((amdgpu_waves_per_eu(NB <= 8 ? 5 : (NB <= 16 ? 4 : (NB <= 24 ? 3 : 2)))))
+// HALF (G = 5..8): the wavefronts come in pairs on the same four queries, wavefront 2p takes the heads
+// 0..3 and 2p+1 the heads 4..G-1; with PERQ a workgroup is eight wavefronts (head w's keys in
+// wavefront w) on 16 queries, otherwise one pair.
+template <int GMAX, int KS, int NB, bool EXPORT, bool BIAS, bool PERQ, bool HALF>
+__global__ void __launch_bounds__(64 * (PERQ ? (HALF ? 8 : 4) : TG_WAVES))
+    // (eight-wavefront workgroups: three per SIMD leave room for one workgroup only, i.e. two per SIMD)
+    __attribute__((amdgpu_waves_per_eu(NB <= 8 ? 5 : (NB <= 16 ? 4 : (NB <= 24 && !(PERQ && HALF) ? 3 : 2)))))
 topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lmk_packed,
                       const float* __restrict__ lse_swa, const float* __restrict__ bias,
                       int32_t* __restrict__ indices,
@@ -151,26 +158,46 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   constexpr int QPL = 4 / GMAX;   // queries per lane (its four accumulator rows)
   constexpr int NQ = 16 / GMAX;   // queries per wavefront
   constexpr int NMASK = EXPORT ? 0 : (NB > 8 ? NB / 2 : 0);  // blocks below it are visible to every row
-  constexpr int TGW = PERQ ? 4 : TG_WAVES;                   // wavefronts per workgroup
+  constexpr int TGW = PERQ ? (HALF ? 8 : 4) : TG_WAVES;      // wavefronts per workgroup
+  constexpr int QGROUPS = HALF ? TGW / 2 : TGW;              // ... and how many have queries of their own
   static_assert(!PERQ || GMAX == 4, "per-query-head keys: four heads, four wavefronts");
-  __shared__ uint32_t cand_w[TGW][4][TG_CAND];          // compacted candidate keys, per lane row
+  static_assert(!HALF || (GMAX == 4 && TG_WAVES == 2), "halves: four heads each, a pair per workgroup");
+  constexpr int PB = NB >= 32 ? 2 : 1;  // blocks per load group (two groups are live: 16 registers per block and group)
+  // LDS that several wavefronts share.  PERQ: accumulators of a load group on their way between the
+  // wavefronts, [buffer][block][from wavefront = head][register][lane]; two buffers take turns, so that
+  // one barrier a group is enough.  HALF: the selection scores a pair trades, [pair][block][lane].  With
+  // both the two uses follow each other in the same memory, and so do the eight wavefronts' selection
+  // areas (candidates and output stage), which would not fit beside them.
+  constexpr bool OVER = PERQ && HALF;
+  constexpr int XCH_F = PERQ ? 2 * PB * TGW * 4 * 64 : 0, KX_F = HALF ? QGROUPS * NB * 64 : 0;
+  constexpr int SEL_B = 4 * TG_CAND * 4 + NQ * 32 * 4 + NQ * GMAX * 32 * 2;  // bytes of a wavefront's selection areas
+  constexpr int XB_F = OVER ? (XCH_F > KX_F ? (XCH_F > TGW * SEL_B / 4 ? XCH_F : TGW * SEL_B / 4)
+                                            : (KX_F > TGW * SEL_B / 4 ? KX_F : TGW * SEL_B / 4))
+                            : (XCH_F + KX_F > 0 ? XCH_F + KX_F : 1);
+  __shared__ __align__(16) float xbuf[XB_F];
+  __shared__ uint32_t cand_w[OVER ? 1 : TGW][4][TG_CAND];          // compacted candidate keys, per lane row
   __shared__ uint32_t words_w[TGW][4][16], wbase_w[TGW][4][16];  // winner map of a query and its word prefix counts
-  __shared__ __align__(16) int stage_i_w[TGW][NQ * 32];               // winners' chunk indices, [query][slot]
-  __shared__ __align__(16) bf16_t stage_s_w[TGW][NQ * GMAX * 32];  // their raw scores, [query][slot][head]
+  __shared__ __align__(16) int stage_i_w[OVER ? 1 : TGW][NQ * 32];               // winners' chunk indices, [query][slot]
+  __shared__ __align__(16) bf16_t stage_s_w[OVER ? 1 : TGW][NQ * GMAX * 32];  // their raw scores, [query][slot][head]
   // the bias of this (batch, KV head): [chunk][head, padded to 4] fp32, a copy per wavefront (they never
   // synchronise); read back 16 bytes per lane right where a block's logits are formed, instead of
-  // global loads whose latency the compiler covers with registers this kernel does not have
-  __shared__ __align__(16) float bias_w[BIAS ? TGW : 1][BIAS ? NB * 16 : 1][4];
+  // global loads whose latency the compiler covers with registers this kernel does not have.
+  // (PERQ with HALF: the wavefronts meet at barriers anyway, one copy per half of the heads.)
+  __shared__ __align__(16) float bias_w[BIAS ? (OVER ? 2 : TGW) : 1][BIAS ? NB * 16 : 1][4];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  uint32_t (*cand)[TG_CAND] = cand_w[wave];
+  const int half = HALF ? (wave & 1) : 0;   // this wavefront's heads are 4 * half ..
+  const int pw = HALF ? (wave >> 1) : wave; // which of the workgroup's queries it has
+  const int gofs = 4 * half;
+  char* const sel_area = (char*)xbuf + (OVER ? wave * SEL_B : 0);
+  uint32_t (*cand)[TG_CAND] = OVER ? (uint32_t (*)[TG_CAND])sel_area : cand_w[OVER ? 0 : wave];
   uint32_t (*words)[16] = words_w[wave];
   uint32_t (*wbase)[16] = wbase_w[wave];
-  int* stage_i = stage_i_w[wave];
-  bf16_t* stage_s = stage_s_w[wave];
+  int* stage_i = OVER ? (int*)(sel_area + 4 * TG_CAND * 4) : stage_i_w[OVER ? 0 : wave];
+  bf16_t* stage_s = OVER ? (bf16_t*)(sel_area + 4 * TG_CAND * 4 + NQ * 32 * 4) : stage_s_w[OVER ? 0 : wave];
   const int lane = threadIdx.x & 63, col = lane & 15, j = lane >> 4;
-  const int t0 = t_base + (blockIdx.x * TGW + wave) * NQ;
-  const int t_wg = t_base + blockIdx.x * TGW * NQ;  // PERQ: the workgroup's 16 queries
+  const int t0 = t_base + (blockIdx.x * QGROUPS + pw) * NQ;
+  const int t_wg = t_base + blockIdx.x * QGROUPS * NQ;  // PERQ: the workgroup's 16 queries
   if ((PERQ ? t_wg : t0) >= t_end) return;          // (PERQ: the wavefronts meet at barriers until the logits are in)
   const int t_safe = PERQ ? t_wg : t0;              // a query of this launch, for the addresses of rows that have none
   const int hk = blockIdx.y;
@@ -192,8 +219,8 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
     const int lq = tq < t_end ? limit_of(tq) : 0;
 #pragma unroll
     for (int e = 0; e < GMAX; ++e) {
-      rowok[u * GMAX + e] = (tq < t_end) & (e < G);
-      lim[u * GMAX + e] = e < G ? lq : 0;
+      rowok[u * GMAX + e] = (tq < t_end) & (gofs + e < G);
+      lim[u * GMAX + e] = gofs + e < G ? lq : 0;
     }
   }
   const int nb_real = (N + 15) / 16;  // blocks the packed chunk keys hold
@@ -202,7 +229,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   bf16x8_t afrag[KS];
   {
     const int r = lane & 15;
-    const int g = PERQ ? wave : r % GMAX, tq = PERQ ? t_wg + r : t0 + r / GMAX;
+    const int g = PERQ ? wave : gofs + r % GMAX, tq = PERQ ? t_wg + r : t0 + r / GMAX;
     const bool ok = tq < t_end && g < G;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -215,7 +242,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = 4 * j + i;
-    const int tq = t0 + r / GMAX, g = r % GMAX;
+    const int tq = t0 + r / GMAX, g = gofs + r % GMAX;
     const long li = ((b * L + (rowok[i] ? tq : t_safe)) * (long)h_kv + hk) * G + (rowok[i] ? g : 0);
     float x;  // the layer hands lse_swa over in its hidden dtype (hils_attention.py:547)
     if (lse_bf16) x = bf2f(((const bf16_t*)lse_swa)[li]); else x = lse_swa[li];
@@ -229,7 +256,6 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   // the keys of two blocks travel together, one such group ahead of their use (the loads of a
   // block issued right before its MFMAs would each expose a full memory latency)
   typedef unsigned tg_u32x4 __attribute__((ext_vector_type(4)));
-  constexpr int PB = NB >= 32 ? 2 : 1;  // blocks per load group (two groups are live: 16 registers per block and group)
   static_assert(NB % PB == 0, "blocks come in load groups");
   auto load_group = [&](int g0, tg_u32x4 (&dst)[PB][KS]) {
 #pragma unroll
@@ -242,9 +268,23 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   };
   // bias (B, N, h_kv, G) fp32: the G values of a (chunk, KV head) are contiguous; accumulator row
   // 4j+i is head (4j+i) % GMAX
-  float (*bias_s)[4] = bias_w[BIAS ? wave : 0];
+  float (*bias_s)[4] = bias_w[BIAS ? (OVER ? half : wave) : 0];
   if constexpr (BIAS) {
     const float* bias_u = bias + (b * N * (long)h_kv + hk) * G;
+    if constexpr (HALF) {
+      // this half's heads; PERQ: the four wavefronts of a half fill its copy together (the first
+      // barrier of the logits comes before anybody reads it)
+      for (int c = OVER ? pw * 64 + lane : lane; c < NB * 16; c += OVER ? 64 * QGROUPS : 64) {
+        float e4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (c < N) {
+          const float* bp = bias_u + (long)c * h_kv * G + gofs;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (gofs + e < G) e4[e] = bp[e];
+        }
+        *(float4*)bias_s[c] = make_float4(e4[0], e4[1], e4[2], e4[3]);
+      }
+    } else {
 #pragma unroll
     for (int c = lane; c < NB * 16; c += 64) {
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);  // chunks past N (never visible) and heads past G: 0
@@ -257,6 +297,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
       }
       *(float4*)bias_s[c] = v;
     }
+    }
   }
   auto bias_of = [&](int c, float (&bv)[4]) {  // c < 16 * NB
     const float4 v = *(const float4*)bias_s[c];
@@ -264,9 +305,9 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
 #pragma unroll
     for (int i = 0; i < 4; ++i) bv[i] = e[i % GMAX];
   };
-  // PERQ: accumulators of a load group on their way between the wavefronts, [block][from wavefront =
-  // head][register][lane]; two buffers take turns, so that one barrier a group is enough
-  __shared__ float xch[PERQ ? 2 : 1][PERQ ? PB : 1][4][4][PERQ ? 64 : 1];
+  auto xch = [&](int buf, int p2, int w, int i, int l) -> float& {
+    return xbuf[(((buf * PB + p2) * TGW + w) * 4 + i) * 64 + l];
+  };
   auto use_group = [&](int g0, const tg_u32x4 (&src)[PB][KS]) {
     const int buf = (g0 / PB) & 1;
     if constexpr (PERQ) {
@@ -274,7 +315,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
       for (int p2 = 0; p2 < PB; ++p2) {
         const int nt = g0 + p2;
         float bv[4];
-        if constexpr (BIAS) bias_of(nt * 16 + col, bv);
+        if constexpr (BIAS && !HALF) bias_of(nt * 16 + col, bv);
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
@@ -283,8 +324,8 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           float v = __fmul_rn(acc[i], sm_scale);
-          if constexpr (BIAS) v = __fadd_rn(v, bv[wave]);
-          xch[buf][p2][wave][i][lane] = v;
+          if constexpr (BIAS && !HALF) v = __fadd_rn(v, bv[wave]);  // (HALF: added by the reader, which has its heads' bias)
+          xch(buf, p2, wave, i, lane) = v;
         }
       }
       __syncthreads();
@@ -293,7 +334,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
     for (int p2 = 0; p2 < PB; ++p2) {
       const int nt = g0 + p2;
       float bv[4];
-      if constexpr (BIAS && !PERQ) bias_of(nt * 16 + col, bv);
+      if constexpr (BIAS && (!PERQ || HALF)) bias_of(nt * 16 + col, bv);
       f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
       if constexpr (!PERQ) {
 #pragma unroll
@@ -305,9 +346,10 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
       for (int i = 0; i < 4; ++i) {
         float v;
         if constexpr (PERQ) {
-          // row (query j of this wavefront, head i): wavefront i's register j of the lane that holds
-          // this chunk column for the queries 4 * wave .. 4 * wave + 3
-          v = xch[buf][p2][i][j][col + 16 * wave];
+          // row (query j of this wavefront, head i of its heads): that head's wavefront's register j of
+          // the lane that holds this chunk column for the queries 4 * pw .. 4 * pw + 3
+          v = xch(buf, p2, gofs + i, j, col + 16 * pw);
+          if constexpr (BIAS && HALF) v = __fadd_rn(v, bv[i]);
         } else {
           v = __fmul_rn(acc[i], sm_scale);
           if constexpr (BIAS) v = __fadd_rn(v, bv[i]);
@@ -316,7 +358,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
         x[nt][i] = v;
         // (pinned here: left alone the compiler forms some of these sums only where they are used and
         // keeps product and bias alive in their place, which this kernel has no registers for)
-        if constexpr (BIAS && !PERQ) asm volatile("" : "+v"(x[nt][i]));
+        if constexpr (BIAS && (!PERQ || HALF)) asm volatile("" : "+v"(x[nt][i]));
       }
       if (EXPORT) {
         if (sel_logits_out && c < N) {
@@ -324,7 +366,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
           for (int i = 0; i < 4; ++i)
             if (rowok[i]) {
               const int r = 4 * j + i;
-              sel_logits_out[(((b * L + t0 + r / GMAX) * (long)h_kv + hk) * G + r % GMAX) * N + c] = x[nt][i];
+              sel_logits_out[(((b * L + t0 + r / GMAX) * (long)h_kv + hk) * G + gofs + r % GMAX) * N + c] = x[nt][i];
             }
         }
       }
@@ -350,7 +392,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
     }
   }
 
-  if (PERQ && t0 >= t_end) return;  // no barrier behind this point
+  if (PERQ && !HALF && t0 >= t_end) return;  // no barrier behind this point
   // ---- lse_total per row = logaddexp(lse_swa, logsumexp of the visible logits) ----
   float lse_tot[4];
 #pragma unroll
@@ -374,7 +416,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
     const float lt = tot2 * HILS_LN2;
     if (lse_total_out && col == 0 && rowok[i]) {
       const int r = 4 * j + i;
-      lse_total_out[((b * L + t0 + r / GMAX) * (long)h_kv + hk) * G + r % GMAX] = lt;
+      lse_total_out[((b * L + t0 + r / GMAX) * (long)h_kv + hk) * G + gofs + r % GMAX] = lt;
     }
     // A row that sees no chunk and has lse_swa = -inf has lse_total = -inf; its logits are all -inf,
     // and -inf - -inf would be a NaN, which this file is compiled not to expect: such a row subtracts
@@ -383,9 +425,12 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   }
 
   // outputs start as "no winner"
-  for (int e = lane; e < NQ * 8; e += 64) ((int4*)stage_i)[e] = make_int4(-1, -1, -1, -1);
-  ((uint4*)stage_s)[lane] = make_uint4(0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u);  // 512 x -inf
-  __builtin_amdgcn_wave_barrier();
+  auto clear_stage = [&]() {
+    for (int e = lane; e < NQ * 8; e += 64) ((int4*)stage_i)[e] = make_int4(-1, -1, -1, -1);
+    ((uint4*)stage_s)[lane] = make_uint4(0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u);  // 512 x -inf
+    __builtin_amdgcn_wave_barrier();
+  };
+  if constexpr (!OVER) clear_stage();  // (OVER: once the memory is the stage's)
 
   // ---- selection, one query of every lane row at a time ----
 #pragma unroll
@@ -402,6 +447,35 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
 #pragma unroll
       for (int e = 0; e < GMAX; ++e) best = fmaxf(best, __fsub_rn(x[nt][u * GMAX + e], lse_tot[u * GMAX + e]));
       key[nt] = best;
+    }
+    if constexpr (HALF) {
+      // the pair's scores: the first half's go to LDS, the second half's wavefront forms the maxima and
+      // leaves them there for the first (both go on with the same numbers, whatever a maximum of +0
+      // and -0 is).  A pair without queries takes part in the barriers and leaves behind them.
+      float* kxp = xbuf + (OVER ? 0 : XCH_F) + pw * NB * 64 + lane;
+      if constexpr (OVER) __syncthreads();  // everybody is through with the accumulators in this memory
+      if (half == 0) {
+#pragma unroll
+        for (int nt = 0; nt < NB; ++nt) kxp[nt * 64] = key[nt];
+      }
+      __syncthreads();
+      if (half == 1) {
+#pragma unroll
+        for (int nt = 0; nt < NB; ++nt) {
+          key[nt] = fmaxf(key[nt], kxp[nt * 64]);
+          kxp[nt * 64] = key[nt];
+        }
+      }
+      __syncthreads();
+      if (half == 0) {
+#pragma unroll
+        for (int nt = 0; nt < NB; ++nt) key[nt] = kxp[nt * 64];
+      }
+      if constexpr (OVER) {
+        __syncthreads();  // the selection areas lie over the scores
+        if (t0 >= t_end) return;
+        clear_stage();
+      }
     }
     // the two largest scores of the lane, the number of valid ones
     float m1 = HILS_NEG_INF, m2 = HILS_NEG_INF;
@@ -570,30 +644,30 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
 #pragma unroll
   for (int e0 = 0; e0 < NQ * 32; e0 += 64) {
     const int e = e0 + lane, qi = e >> 5, k = e & 31;
-    if ((k < topk) & (t0 + qi < t_end)) ind0[qi * h_kv * topk + k] = stage_i[e];
+    if ((k < topk) & (t0 + qi < t_end) & (half == 0)) ind0[qi * h_kv * topk + k] = stage_i[e];
   }
 #pragma unroll
   for (int e0 = 0; e0 < NQ * GMAX * 32; e0 += 64) {
     const int e = e0 + lane, k = e & 31, g = (e >> 5) % GMAX, qi = e / (32 * GMAX);
-    if ((k < topk) & (g < G) & (t0 + qi < t_end))
-      sc0[(qi * h_kv * G + g) * topk + k] = stage_s[(qi * 32 + k) * GMAX + g];
+    if ((k < topk) & (gofs + g < G) & (t0 + qi < t_end))
+      sc0[(qi * h_kv * G + gofs + g) * topk + k] = stage_s[(qi * 32 + k) * GMAX + g];
   }
 }
 
 // plain: no Gumbel noise and no drop mask (a bias is fine)
 bool hils_topk_group_covers(int N, int G, int D, int topk, int per_qhead, bool plain) {
-  if (per_qhead && G != 3 && G != 4) return false;  // (one head a group: the keys are shared anyway)
-  return plain && (G == 1 || G == 3 || G == 4) && (D == 64 || D == 128) && N <= 16 * TG_NB && topk <= 32;
+  if (per_qhead && (G < 3 || G > 8)) return false;  // (one head a group: the keys are shared anyway)
+  return plain && (G == 1 || (G >= 3 && G <= 8)) && (D == 64 || D == 128) && N <= 16 * TG_NB && topk <= 32;
 }
 
-template <int GMAX, int KS, bool BIAS, bool PERQ>
+template <int GMAX, int KS, bool BIAS, bool PERQ, bool HALF>
 static void tg_launch_range(int NB, bool exp, dim3 grid, hipStream_t st, const bf16_t* q, const uint4* pk,
                             const float* lse_swa, const float* bias, int32_t* indices, bf16_t* scores, float* lse_total,
                             float* sel_logits, int L, int N, int h_kv, int G, int topk, int block_size,
                             int window_size, int causal, int q_offset, float sm_scale, int t_base, int t_end,
                             int lse_bf16) {
 #define TG_CALL(NB_, EX_)                                                                              \
-  hipLaunchKernelGGL((topk_fwd_group_kernel<GMAX, KS, NB_, EX_, BIAS, PERQ>), grid, dim3(64 * (PERQ ? 4 : TG_WAVES)), 0, st, q, pk, lse_swa, \
+  hipLaunchKernelGGL((topk_fwd_group_kernel<GMAX, KS, NB_, EX_, BIAS, PERQ, HALF>), grid, dim3(64 * (PERQ ? (HALF ? 8 : 4) : TG_WAVES)), 0, st, q, pk, lse_swa, \
                      bias, indices, scores, lse_total, sel_logits, L, N, h_kv, G, topk, block_size, window_size, \
                      causal, q_offset, sm_scale, t_base, t_end, bs_shift, lse_bf16)
   const int bs_shift = (block_size > 0 && (block_size & (block_size - 1)) == 0) ? __builtin_ctz(block_size) : -1;
@@ -616,7 +690,8 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
                            float sm_scale, int lse_bf16, int per_qhead, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   const int GM = (G == 1) ? 1 : 4;
-  const int TGW = per_qhead ? 4 : TG_WAVES;
+  const bool halves = G > 4;  // two wavefronts per four queries
+  const int QGROUPS = halves ? (per_qhead ? 4 : 1) : (per_qhead ? 4 : TG_WAVES);  // wavefronts (pairs) of a workgroup with queries of their own
   const int NQ = 16 / GM;
   const bool exp = sel_logits != nullptr;
   auto limit_of = [&](int tq) -> int {
@@ -639,18 +714,20 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
         t_hi = lo;
       }
     }
-    dim3 grid((t_hi - t + NQ * TGW - 1) / (NQ * TGW), h_kv, B);
-#define TG_RANGE_B(G_, KS_, B_, P_)                                                                   \
-  tg_launch_range<G_, KS_, B_, P_>(NB, exp, grid, st, (const bf16_t*)q, (const uint4*)lmk_packed, lse_swa, bias, \
+    dim3 grid((t_hi - t + NQ * QGROUPS - 1) / (NQ * QGROUPS), h_kv, B);
+#define TG_RANGE_B(G_, KS_, B_, P_, H_)                                                               \
+  tg_launch_range<G_, KS_, B_, P_, H_>(NB, exp, grid, st, (const bf16_t*)q, (const uint4*)lmk_packed, lse_swa, bias, \
                                indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,   \
                                block_size, window_size, causal, q_offset, sm_scale, t, t_hi, lse_bf16)
-#define TG_RANGE(G_, KS_, P_)                                                                         \
+#define TG_RANGE(G_, KS_, P_, H_)                                                                     \
   do {                                                                                                \
-    if (bias) TG_RANGE_B(G_, KS_, true, P_); else TG_RANGE_B(G_, KS_, false, P_);                     \
+    if (bias) TG_RANGE_B(G_, KS_, true, P_, H_); else TG_RANGE_B(G_, KS_, false, P_, H_);             \
   } while (0)
-    if (GM == 1) { if (D == 64) TG_RANGE(1, 2, false); else TG_RANGE(1, 4, false); }
-    else if (per_qhead) { if (D == 64) TG_RANGE(4, 2, true); else TG_RANGE(4, 4, true); }
-    else { if (D == 64) TG_RANGE(4, 2, false); else TG_RANGE(4, 4, false); }
+    if (GM == 1) { if (D == 64) TG_RANGE(1, 2, false, false); else TG_RANGE(1, 4, false, false); }
+    else if (halves && per_qhead) { if (D == 64) TG_RANGE(4, 2, true, true); else TG_RANGE(4, 4, true, true); }
+    else if (halves) { if (D == 64) TG_RANGE(4, 2, false, true); else TG_RANGE(4, 4, false, true); }
+    else if (per_qhead) { if (D == 64) TG_RANGE(4, 2, true, false); else TG_RANGE(4, 4, true, false); }
+    else { if (D == 64) TG_RANGE(4, 2, false, false); else TG_RANGE(4, 4, false, false); }
 #undef TG_RANGE
 #undef TG_RANGE_B
     t = t_hi;

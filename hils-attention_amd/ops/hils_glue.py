@@ -155,7 +155,7 @@ def decode_step(q, lmks, k, v, lse_swa, topk, block_size, window_size, q_offset=
     of which the first ``num_chunks`` (default cap) chunks are looked at.  lmks may carry h_q heads
     instead of h_kv (one chunk key per query head, the layer's attention-pooled keys): (B,N,h_q,D) or,
     head-major, (B,h_q,cap,D).  Shapes the fused kernel does not take (few rows, short caches, more
-    than four query heads per KV head, ...) run as the two calls."""
+    than eight query heads per KV head, ...) run as the two calls."""
     import math
     from .hils_fwd_bwd_head import HiLS_block_M_head
     _cabi.require_gpu_bf16("decode_step", q, lmks)

@@ -19,7 +19,8 @@ def _oracle_step(orc, q, lmk, lse, pb, k, v, K, S, W, off, idx, scores_bf16):
 
 
 @pytest.mark.parametrize("L,N,HQ,H,D,K,off", [(4096, 64, 8, 2, 128, 16, 0), (9000, 300, 3, 1, 64, 32, 300 * 64 - 9000),
-                                             (2048, 32, 4, 4, 64, 8, 0), (6000, 500, 4, 1, 128, 32, 500 * 64 - 6000)])
+                                             (2048, 32, 4, 4, 64, 8, 0), (6000, 500, 4, 1, 128, 32, 500 * 64 - 6000),
+                                             (5000, 400, 16, 2, 64, 32, 400 * 64 - 5000), (3000, 47, 5, 1, 128, 16, 8)])
 def test_prefill_selection_with_prior_bias(pkg, orc, dev, L, N, HQ, H, D, K, off):
     """topk_chunk_weights(prior_b=) at prefill sizes: the one-pass selection kernel adds the bias to
     its logits, the softmax kernel gathers it.  Checked against the exporting variant of the operator
@@ -64,7 +65,9 @@ def test_prefill_selection_with_prior_bias(pkg, orc, dev, L, N, HQ, H, D, K, off
     assert not torch.equal(idx_nb, idx1)
 
 
-@pytest.mark.parametrize("L,N,HQ,H,D,K", [(3000, 47, 8, 2, 128, 16), (5000, 400, 4, 1, 64, 32)])
+@pytest.mark.parametrize("L,N,HQ,H,D,K", [(3000, 47, 8, 2, 128, 16), (5000, 400, 4, 1, 64, 32),
+                                          (5000, 400, 16, 2, 64, 32), (3000, 47, 7, 1, 128, 16),
+                                          (9000, 300, 12, 2, 128, 32)])
 def test_prefill_selection_with_a_key_per_query_head(pkg, orc, dev, L, N, HQ, H, D, K):
     """The layer's default pooling (attention-pooled chunk keys, one per query head, with their prior
     bias; models/FlashHiLS/hils_attention.py:391-416, 568-602) through topk_chunk_weights: same
@@ -99,7 +102,8 @@ def test_prefill_selection_with_a_key_per_query_head(pkg, orc, dev, L, N, HQ, H,
 
 
 @pytest.mark.parametrize("B,Lq,Lkv,HQ,H,D,K", [(32, 1, 32768, 32, 8, 128, 32), (16, 1, 16512, 8, 8, 64, 16),
-                                               (50, 2, 20480, 4, 1, 128, 8), (2, 1, 4096, 8, 2, 128, 16)])
+                                               (50, 2, 20480, 4, 1, 128, 8), (2, 1, 4096, 8, 2, 128, 16),
+                                               (64, 1, 32768, 16, 2, 64, 32), (16, 1, 65536, 40, 8, 128, 16)])
 def test_decode_step_with_prior_bias(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
     """decode_step(prior_b=): one launch per step with the bias staged beside the logits; the chunk
     keys and the bias token-major (the reference's layout) and head-major (the cache layers')."""
@@ -147,7 +151,8 @@ def test_decode_step_with_prior_bias(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
 
 @pytest.mark.parametrize("B,Lq,Lkv,HQ,H,D,K", [(32, 1, 32768, 32, 8, 128, 32), (50, 2, 20480, 4, 1, 128, 8),
                                                (24, 1, 65536, 12, 4, 64, 64), (48, 1, 16512, 6, 2, 64, 16),
-                                               (48, 1, 16384, 4, 2, 64, 8)])
+                                               (48, 1, 16384, 4, 2, 64, 8), (64, 1, 32768, 16, 2, 64, 32),
+                                               (48, 1, 65536, 14, 2, 128, 16)])
 def test_decode_step_with_a_key_per_query_head(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
     """The layer's default pooling in decode: one attention-pooled chunk key per query head and its
     prior bias.  One launch per step; token-major, head-major and paged keys give the same bits; the

@@ -296,12 +296,23 @@ def test_topk_split_path_options(pkg, orc, dev):
     (24, 1, 777, 4, 3, 128, 32, 500 * 64 + 7),
     (40, 2, 1536, 8, 4, 128, 32, 1536 * 64 - 2),  # more rows than compute units: 8-wavefront workgroups
     (128, 1, 256, 1, 4, 64, 8, 10),           # no chunk visible yet: all -1
-    (64, 2, 300, 2, 2, 128, 8, 64 * 3 + 5)])  # fewer visible chunks than topk
+    (64, 2, 300, 2, 2, 128, 8, 64 * 3 + 5),   # fewer visible chunks than topk
+    # five to eight query heads per KV head: eight head slots per row
+    (64, 1, 2048, 2, 8, 64, 32, 2048 * 64), (20, 1, 2500, 8, 6, 128, 16, 2500 * 64 - 3),
+    (300, 1, 700, 1, 5, 128, 8, 700 * 64)])
 def test_topk_workgroup_per_row_path(pkg, orc, dev, B, L, N, h_kv, G, D, topk, off):
     """About one (query, KV head) row per compute unit: one 16-wavefront workgroup per row streams the
     chunk keys, keeps the logits in LDS and selects (ragged N, limits below N, exact ties)."""
     run_case(pkg, orc, dev, B=B, L=L, N=N, h_kv=h_kv, G=G, D=D, topk=topk, S=64, W=1, q_offset=off,
              training=False, dup_keys=(N == 1000))
+
+
+@pytest.mark.parametrize("B,L,N,h_kv,G,D,topk,bias", [(64, 1, 1500, 2, 8, 64, 32, True), (100, 1, 1024, 1, 7, 128, 16, False),
+                                                     (48, 2, 600, 2, 5, 128, 8, True)])
+def test_topk_workgroup_per_row_path_key_per_query_head(pkg, orc, dev, B, L, N, h_kv, G, D, topk, bias):
+    """The same kernel with one chunk key per query head and five to eight heads per KV head."""
+    run_case(pkg, orc, dev, B=B, L=L, N=N, h_kv=h_kv, G=G, D=D, topk=topk, S=64, W=1, q_offset=N * 64 - L,
+             training=False, per_qhead=True, use_bias=bias)
 
 
 def test_topk_split_and_fused_paths_agree(pkg, dev):
@@ -334,6 +345,9 @@ def test_topk_split_and_fused_paths_agree(pkg, dev):
     (2048, 32, 2, 4, 64, 1, False),      # a single winner
     (32768, 512, 1, 4, 128, 32, False),  # the full 512 chunks of the headline shape, one KV head
     (16384, 256, 1, 1, 128, 31, True),   # k not a power of two, ties, G = 1
+    # five to eight query heads per KV head: two wavefronts per four queries trade their heads' scores
+    (8192, 128, 2, 8, 64, 32, False), (5000, 79, 1, 5, 128, 16, True), (4096, 64, 2, 7, 64, 5, True),
+    (16384, 256, 1, 8, 128, 32, True),
 ])
 def test_topk_one_pass_prefill_kernel(pkg, orc, dev, L, N, h_kv, G, D, topk, dup):
     """The one-pass prefill kernel (chunk keys repacked into the workspace, up to 512 chunks and 32
@@ -350,7 +364,9 @@ def test_topk_one_pass_prefill_kernel(pkg, orc, dev, L, N, h_kv, G, D, topk, dup
     (1, 64, 9000, 250, 16, 1, 64, 2),     # 16 queries per wavefront
     (3, 128, 7000, 140, 9, 64, 64, 1),    # a padding head row, odd k, a wide window
     (4, 128, 6000, 125, 16, 1, 48, 1),    # chunk sizes that are no power of two (visibility by division)
-    (1, 64, 5000, 50, 7, 30, 100, 2)])
+    (1, 64, 5000, 50, 7, 30, 100, 2),
+    (8, 64, 32000, 500, 32, 1, 64, 1),    # eight heads per KV head, all four launches
+    (6, 128, 20000, 313, 16, 1, 64, 2), (5, 64, 7000, 140, 9, 64, 48, 1)])
 def test_topk_one_pass_kernel_launches_match_export_variant(pkg, dev, G, D, L, N, topk, W, S, h_kv):
     """The one-pass prefill kernel as inference launches it (one instantiation per range of visible
     chunk counts, no logit export) against its exporting instantiation, which the cases above check
