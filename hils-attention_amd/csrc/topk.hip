@@ -542,8 +542,28 @@ topk_pack_lmk_kernel(const bf16_t* __restrict__ lmks, uint4* __restrict__ packed
   packed[i] = v;
 }
 
-template <int GMAX, int KS, bool PLAIN, bool PACKED>
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4)))
+// (the variants with a bias / noise / drop mask / export hold a block's bias beside its keys: three
+// wavefronts per SIMD instead of four, which their LDS allows anyway, rather than 100 bytes of scratch)
+// The additive bias (B, N, heads) fp32 head-major in blocks of 16 chunks, (B, heads, nblk16, 16), zero
+// past N: the 16 lanes of a chunk block then read one head's bias as 64 contiguous bytes (from the
+// caller's tensor every lane touches a cache line of its own, once per head).  One thread per element.
+__global__ void __launch_bounds__(256)
+topk_pack_bias_kernel(const float* __restrict__ bias, float* __restrict__ packed, int N, int heads, int nblk16,
+                      long total) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int col = (int)(i & 15);
+  long r = i >> 4;
+  const int blk = (int)(r % nblk16);
+  r /= nblk16;
+  const int h = (int)(r % heads);
+  const long b = r / heads;
+  const int c = blk * 16 + col;
+  packed[i] = c < N ? bias[(b * N + c) * (long)heads + h] : 0.f;
+}
+
+template <int GMAX, int KS, bool PLAIN, bool PACKED, bool PERQ = false, bool BIASONLY = false>
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(PLAIN ? 4 : 3, 4)))
 topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                      const float* __restrict__ lse_swa, const float* __restrict__ bias,
                      const float* __restrict__ gumbel, const int32_t* __restrict__ drop_mask,
@@ -551,9 +571,22 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
                      float* __restrict__ lse_total_out, float* __restrict__ sel_logits_out,
                      int L, int N, int h_kv, int G, int topk, int block_size, int window_size,
                      int causal, int q_offset, float sm_scale, int segw, int pool_floats,
-                     const uint4* __restrict__ lmk_packed) {
+                     const uint4* __restrict__ lmk_packed, const float* __restrict__ bias_packed,
+                     int lmk_group_heads) {
+  // lmk_group_heads (PERQ only): chunk-key heads per KV head, G (a key per query head) or 1 (shared keys
+  // walked head by head all the same: how more than four query heads per KV head run here)
+  // bias_packed: the bias in topk_pack_bias_kernel's order (or null: read from bias)
   // PLAIN: no bias, Gumbel noise, drop mask or logit export (the inference path)
   // PACKED: the chunk keys of the two passes come from lmk_packed (topk_pack_lmk_kernel's order)
+  // BIASONLY (not PLAIN, bias_packed given): a bias and nothing else (the layer's prior bias at inference).
+  // The general variant tests its optional inputs per element, and behind every such branch the compiler
+  // waits for all loads in flight, the next block's keys included; this one has no branch in its loops.
+  static_assert(!BIASONLY || (!PLAIN && PACKED), "the bias-only variant reads the packed bias");
+  // PERQ: one chunk key per QUERY head, lmks (B,N,h_kv*G,D) and lmk_packed with h_kv*G heads.  The tile
+  // rows are then 16 queries of one head (GMAX = 1) and the wavefront walks the G heads of its KV head
+  // one after the other, in both passes: a head's log-sum-exp waits in LDS, and the pooled score of a
+  // (query, chunk) is the running maximum over the heads of what the same lane wrote there before.
+  static_assert(!PERQ || (GMAX == 1 && PACKED), "a key per query head: 16 queries of one head per tile, packed keys");
   constexpr int D = KS * 32;
   constexpr int QPT = 16 / GMAX;            // queries per 16-row tile
   constexpr int NT = (GMAX == 4) ? 2 : 1;   // tiles per wavefront
@@ -566,6 +599,11 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
   int* scr_i = (int*)(scr_s + 64);
   float* car_s = (float*)(scr_i + 64);      // NQ x topk winners carried across segments
   int* car_i = (int*)(car_s + NQ * topk);
+  float* lt_s = (float*)(car_i + NQ * topk);  // PERQ: lse_total, [head][query]
+  const int LPG = PERQ ? lmk_group_heads : 1;
+  const int h_lmk = h_kv * LPG;               // heads of the chunk-key tensor
+  const int GH = PERQ ? G : 1;                // heads the wavefront walks
+  int cur_gh = 0;                             // ... and the one it is at
 
   const int lane = threadIdx.x, col = lane & 15, j = lane >> 4;
   const int t0 = blockIdx.x * NQ;
@@ -584,17 +622,17 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
     for (int i = 0; i < 4; ++i) {
       const int r = 4 * j + i;
       const int tq = t0 + nt * QPT + r / GMAX;
-      lim[nt][i] = (tq < L && (r % GMAX) < G) ? limit_of(tq) : 0;
+      lim[nt][i] = (tq < L && (PERQ || (r % GMAX) < G)) ? limit_of(tq) : 0;
     }
   const int t_last = (t0 + NQ - 1 < L) ? t0 + NQ - 1 : L - 1;
   const int nblk = (limit_of(t_last) + 15) / 16;
   // blocks below nfull are visible to every row: no masking there
-  const int nfull = (G == GMAX && t0 + NQ <= L) ? limit_of(t0) / 16 : 0;
+  const int nfull = ((PERQ || G == GMAX) && t0 + NQ <= L) ? limit_of(t0) / 16 : 0;
 
   bf16x8_t afrag[NT][KS];
-  {
+  auto load_a = [&](int gh) {  // the query rows as A operands (PERQ: of head gh)
     const int r = lane & 15;
-    const int g = r % GMAX;
+    const int g = PERQ ? gh : r % GMAX;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       const int tq = t0 + nt * QPT + r / GMAX;
@@ -606,11 +644,21 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
         afrag[nt][ks] = *(bf16x8_t*)&v;
       }
     }
-  }
+  };
+  load_a(0);
   // chunk keys as B operands; rows beyond N are read from row N-1 and masked by the caller
-  const long bstride = (long)h_kv * D;  // elements between consecutive chunk keys
-  const bf16_t* bbase = lmks + (b * N * (long)h_kv + hk) * D + j * 8;
-  const uint4* pbase = PACKED ? lmk_packed + ((b * h_kv + hk) * (long)((N + 15) / 16) * KS) * 64 + lane : nullptr;
+  const long bstride = (long)h_lmk * D;  // elements between consecutive chunk keys
+  const bf16_t* bbase;
+  const uint4* pbase;
+  const char* ubase;  // blocks that lie wholly inside [0, N): uniform block address + a 32-bit lane offset
+  auto set_head = [&](int gh) {  // the key head the loads below read (PERQ: head gh of the KV head's group)
+    const int hl = hk * LPG + (LPG > 1 ? gh : 0);
+    cur_gh = gh;
+    bbase = lmks + (b * N * (long)h_lmk + hl) * D + j * 8;
+    pbase = PACKED ? lmk_packed + ((b * h_lmk + hl) * (long)((N + 15) / 16) * KS) * 64 + lane : nullptr;
+    ubase = (const char*)lmks + ((b * N * (long)h_lmk + hl) * D) * 2;
+  };
+  set_head(0);
   auto load_b = [&](int blk, uint4* dst) {
     if (PACKED) {
       const int bc = blk < (N + 15) / 16 ? blk : (N + 15) / 16 - 1;  // a prefetch may run past the end
@@ -633,20 +681,55 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
         acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[nt][ks], *(const bf16x8_t*)&bb[ks], acc[nt], 0, 0, 0);
     }
   };
+  // the additive bias of a block's chunk column for this lane's heads (accumulator row 4j+i is head
+  // (4j+i) % GMAX): loaded together with the block's keys, unconditionally from a clamped address, so
+  // that the loads of a block are all in flight at once (a load behind a branch is waited for inside
+  // it, one memory latency per element)
+  struct BiasRow { float v[GMAX]; };
+  const bool bias_vec4 = !PLAIN && bias && G == 4 && (((size_t)bias) & 15) == 0;
+  auto load_bias = [&](int blk, BiasRow& dst) {
+    if (PLAIN || (!BIASONLY && !bias)) return;
+    if (BIASONLY || bias_packed) {
+      const int nb16 = (N + 15) / 16;
+      const float* p = bias_packed + ((b * h_kv + hk) * (long)G * nb16 + (blk < nb16 ? blk : nb16 - 1)) * 16 + col;
+      if (PERQ) {
+        dst.v[0] = p[(long)cur_gh * nb16 * 16];
+        return;
+      }
+#pragma unroll
+      for (int g = 0; g < GMAX; ++g) dst.v[g] = p[(long)(g < G ? g : 0) * nb16 * 16];
+      return;
+    }
+    int c = blk * 16 + col;
+    c = c < N ? c : N - 1;
+    const float* p = bias + ((b * N + c) * (long)h_kv + hk) * G;
+    if (PERQ) {
+      dst.v[0] = p[cur_gh];
+      return;
+    }
+    if (GMAX == 4 && bias_vec4) {  // four heads, 16-byte aligned rows: one load
+      const float4 t = *(const float4*)p;
+      dst.v[0] = t.x; dst.v[1 % GMAX] = t.y; dst.v[2 % GMAX] = t.z; dst.v[3 % GMAX] = t.w;
+      return;
+    }
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) dst.v[g] = p[g < G ? g : 0];
+  };
   // exact fp32 logit of accumulator element i of chunk c (before masking)
-  auto logit = [&](float acc, int c, int i) -> float {
+  auto logit = [&](float acc, int c, int i, const BiasRow& bz) -> float {
     float x = __fmul_rn(acc, sm_scale);
     if (!PLAIN) {
-      const int g = (4 * j + i) % GMAX;
-      if (c < N && g < G) {
-        if (bias) x = __fadd_rn(x, bias[((b * N + c) * (long)h_kv + hk) * G + g]);
+      const int g = PERQ ? cur_gh : (4 * j + i) % GMAX;
+      if (BIASONLY) {
+        // (chunks past N and heads past G get a finite value added and are masked by their limits)
+        x = __fadd_rn(x, bz.v[PERQ ? 0 : g]);
+      } else if (c < N && g < G) {
+        if (bias) x = __fadd_rn(x, bz.v[PERQ ? 0 : g]);
         if (gumbel) x = __fadd_rn(x, gumbel[(long)(hk * G + g) * N + c]);
       }
     }
     return x;
   };
-  // blocks that lie wholly inside [0, N): uniform block address + a 32-bit lane offset
-  const char* ubase = (const char*)lmks + ((b * N * (long)h_kv + hk) * D) * 2;
   const uint32_t lane_off = (uint32_t)((col * bstride + j * 8) * 2);
   auto load_b_full = [&](int blk, uint4* dst) {
     if (PACKED) {
@@ -668,15 +751,21 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
       else load_b_full(blk < hi ? blk : hi - 1, dst);
     };
     uint4 b0[KS], b1[KS];
+    BiasRow z0, z1;
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) z0.v[g] = z1.v[g] = 0.f;
     ld(lo, b0);
+    load_bias(lo, z0);
     int blk = lo;
     for (; blk + 1 < hi; blk += 2) {
       ld(blk + 1, b1);
-      body(b0, blk, masked_t);
+      load_bias(blk + 1, z1);
+      body(b0, blk, masked_t, z0);
       ld(blk + 2, b0);
-      body(b1, blk + 1, masked_t);
+      load_bias(blk + 2, z0);
+      body(b1, blk + 1, masked_t, z1);
     }
-    if (blk < hi) body(b0, blk, masked_t);
+    if (blk < hi) body(b0, blk, masked_t, z0);
   };
   auto for_blocks = [&](int lo, int hi, auto body) {
     const int mid = nfull < hi ? (nfull > lo ? nfull : lo) : hi;  // masking starts here
@@ -686,13 +775,19 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
 
   // ---------------- pass 1: sum of exp2(y - ref) per lane and row ----------------
   const float c2 = sm_scale * HILS_LOG2E;
+  float lse_tot[NT][4];
+  for (int gh = 0; gh < GH; ++gh) {
+  if (PERQ && gh > 0) {
+    set_head(gh);
+    load_a(gh);
+  }
   float swa[NT][4];  // lse_swa of this lane's rows (-inf for padding rows)
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int r = 4 * j + i;
-      const int tq = t0 + nt * QPT + r / GMAX, g = r % GMAX;
+      const int tq = t0 + nt * QPT + r / GMAX, g = PERQ ? gh : r % GMAX;
       // unconditional loads from a clamped address: all eight are in flight together (a load
       // inside a branch is waited for inside it, one memory latency after the other)
       const bool ok = tq < L && g < G;
@@ -704,7 +799,7 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) { ref[nt][i] = -1e30f; l[nt][i] = 0.f; }
-  for_blocks(0, nblk, [&](const uint4* bb, int blk, auto masked_t) {
+  for_blocks(0, nblk, [&](const uint4* bb, int blk, auto masked_t, const BiasRow& bz) {
     constexpr bool MASKED = decltype(masked_t)::value;
     const int c = blk * 16 + col;
     f32x4_t acc[NT];
@@ -717,7 +812,7 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
       for (int i = 0; i < 4; ++i) {
         // one rounding (acc * c2) whenever nothing is added to the logit, in both variants, so that
         // the export variant and the plain one select from bit-identical lse_total
-        float yy = (PLAIN || (!bias && !gumbel)) ? acc[nt][i] * c2 : logit(acc[nt][i], c, i) * HILS_LOG2E;
+        float yy = (PLAIN || (!BIASONLY && !bias && !gumbel)) ? acc[nt][i] * c2 : logit(acc[nt][i], c, i, bz) * HILS_LOG2E;
         if (MASKED && !(c < lim[nt][i])) yy = HILS_NEG_INF;
         y[nt][i] = yy;
         d[nt][i] = yy - ref[nt][i];
@@ -741,7 +836,6 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
   });
   // combine the 16 lanes (chunk columns) of each row; lse_total per row, in the log2 domain
   // with the hardware exp2/log2 (absolute error ~1e-6, far inside the 1e-4 the LSE needs)
-  float lse_tot[NT][4];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -755,11 +849,14 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
       if (mn > HILS_NEG_INF) tot2 = mx + __builtin_amdgcn_logf(1.f + __builtin_amdgcn_exp2f(mn - mx));
       const float tot = tot2 * HILS_LN2;
       const int r = 4 * j + i;
-      const int tq = t0 + nt * QPT + r / GMAX, g = r % GMAX;
+      const int tq = t0 + nt * QPT + r / GMAX, g = PERQ ? gh : r % GMAX;
       if (lse_total_out && col == 0 && tq < L && g < G)
         lse_total_out[((b * L + tq) * (long)h_kv + hk) * G + g] = tot;
       lse_tot[nt][i] = tot;
+      if (PERQ && col == 0) lt_s[gh * NQ + nt * QPT + r] = tot;  // waits for pass 2
     }
+  }  // heads
+  if (PERQ) __builtin_amdgcn_wave_barrier();
 
   // ---------------- pass 2: pooled scores per segment + selection ----------------
   int ncand_v = 0;  // lane qi holds the number of winners of query qi so far
@@ -768,7 +865,16 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
   for (int seg = 0; seg < nseg; ++seg) {
     const int seg_base = seg * segw;
     const int blk_end = ((seg + 1) * bps < nblk) ? (seg + 1) * bps : nblk;
-    for_blocks(seg * bps, blk_end, [&](const uint4* bb, int blk, auto masked_t) {
+    for (int gh = 0; gh < GH; ++gh) {
+    if (PERQ) {
+      set_head(gh);
+      if (GH > 1) load_a(gh);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lse_tot[nt][i] = lt_s[gh * NQ + nt * QPT + 4 * j + i];
+    }
+    for_blocks(seg * bps, blk_end, [&](const uint4* bb, int blk, auto masked_t, const BiasRow& bz) {
       constexpr bool MASKED = decltype(masked_t)::value;
       const int c = blk * 16 + col;
       f32x4_t acc[NT];
@@ -778,12 +884,12 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
         float nrm[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          float x = logit(acc[nt][i], c, i);
+          float x = logit(acc[nt][i], c, i, bz);
           if (MASKED && !(c < lim[nt][i])) x = HILS_NEG_INF;
-          if (!PLAIN) {
+          if (!PLAIN && !BIASONLY) {
             if (sel_logits_out && c < N) {
               const int r = 4 * j + i;
-              const int tq = t0 + nt * QPT + r / GMAX, g = r % GMAX;
+              const int tq = t0 + nt * QPT + r / GMAX, g = PERQ ? gh : r % GMAX;
               if (tq < L && g < G) sel_logits_out[(((b * L + tq) * (long)h_kv + hk) * G + g) * N + c] = x;
             }
           }
@@ -796,15 +902,17 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
 #pragma unroll
           for (int e = 1; e < GMAX; ++e) best = fmaxf(best, nrm[u * GMAX + e]);  // fmaxf ignores a NaN operand
           const int ql = nt * QPT + (4 * j) / GMAX + u;
-          if (!PLAIN) {
+          if (!PLAIN && !BIASONLY) {
             if (drop_mask && best > HILS_NEG_INF && t0 + ql < L && c < N &&
                 drop_mask[(b * L + t0 + ql) * (long)N + c] != 0)
               best = HILS_NEG_INF;
           }
-          pooled[ql * stride + (c - seg_base)] = best;
+          float* pp = &pooled[ql * stride + (c - seg_base)];
+          *pp = (PERQ && gh > 0) ? fmaxf(*pp, best) : best;  // (the same lane wrote the heads before)
         }
       }
     });
+    }  // heads
     __builtin_amdgcn_wave_barrier();
     const int ns = blk_end * 16 - seg_base;
 #pragma unroll 1
@@ -846,6 +954,11 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
   // pooled rows) as [query][head][slot], the layout of the output, and stored in 16-byte pieces.
   bf16_t* stage = (bf16_t*)pooled;
   const int ntile = (topk + 15) / 16;
+  for (int gh = 0; gh < GH; ++gh) {
+  if (PERQ) {
+    set_head(gh);
+    if (GH > 1) load_a(gh);
+  }
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
@@ -875,7 +988,7 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const int r = 4 * j + i;
-              const int g = r % GMAX;
+              const int g = PERQ ? gh : r % GMAX;
               if (r / GMAX == qq + u && g < G)
                 stage[(qi * G + g) * topk + slot] = f2bf(slot < ncs[u] ? __fmul_rn(acc[i], sm_scale) : HILS_NEG_INF);
             }
@@ -884,6 +997,7 @@ topk_fwd_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lm
       }
     }
   }
+  }  // heads
   __builtin_amdgcn_wave_barrier();
   const int row_e = G * topk;  // bf16 elements per query
   if ((row_e & 7) == 0) {
@@ -2056,11 +2170,26 @@ extern "C" int hils_topk_lse16_covers(int B, int L, int N, int h_kv, int G, int 
   return hils_topk_group_covers(N, G, D, topk, 0, true) ? 1 : 0;
 }
 
+static size_t topk_ws_key_bytes(int B, int N, int h_kv, int G) {
+  return (size_t)B * h_kv * G * ((N + 15) / 16) * 16 * 128 * sizeof(bf16_t);
+}
+// the bias of a call repacked behind the chunk keys of the workspace (topk_pack_bias_kernel)
+static const float* topk_pack_bias(const float* bias, void* workspace, int B, int N, int h_kv, int G, hipStream_t st) {
+  if (!bias || !workspace || G > 8) return nullptr;
+  float* out = (float*)((char*)workspace + topk_ws_key_bytes(B, N, h_kv, G));
+  const int nblk16 = (N + 15) / 16;
+  const long total = (long)B * h_kv * G * nblk16 * 16;
+  hipLaunchKernelGGL(topk_pack_bias_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, bias, out, N,
+                     h_kv * G, nblk16, total);
+  return out;
+}
+
 extern "C" size_t hils_topk_fwd_workspace(int B, int L, int N, int h_kv, int G) {
   // many queries: room for the chunk keys repacked into MFMA operand order (head dim up to 128; a key
   // per query head when the caller's keys are per query head)
+  // and behind them for an additive bias in blocks of 16 chunks per head
   if (!topk_use_split(B, L, N, h_kv))
-    return G <= 8 ? (size_t)B * h_kv * G * ((N + 15) / 16) * 16 * 128 * sizeof(bf16_t) : 0;
+    return G <= 8 ? topk_ws_key_bytes(B, N, h_kv, G) + (size_t)B * h_kv * G * ((N + 15) / 16) * 16 * sizeof(float) : 0;
   return (size_t)B * L * h_kv * G * N * sizeof(float);
 }
 
@@ -2162,6 +2291,40 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
     HILS_CHECK_LAUNCH("hils_topk_fwd");
     return HILS_OK;
   }
+  // one chunk key per query head outside that kernel's envelope (more than 512 chunks, more than 32
+  // winners, noise, a drop mask), or five to eight query heads on shared keys: the two-pass MFMA kernel,
+  // 16 queries a wavefront, head by head
+  if ((per_qhead || G > 4) && workspace && G <= 8 && (D == 64 || D == 128)) {
+    const int nblk16 = (N + 15) / 16;
+    const int h_lmk = per_qhead ? h_kv * G : h_kv;
+    const long total = (long)B * h_lmk * nblk16 * (D / 32) * 64;
+    hipLaunchKernelGGL(topk_pack_lmk_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                       (const bf16_t*)lmks, (uint4*)workspace, N, h_lmk, D, nblk16, total);
+    const int segw = topk_rows_segw(N);
+    const int NQ = 16;
+    int pool_floats = NQ * (segw + 16);
+    if (pool_floats < NQ * G * topk / 2) pool_floats = NQ * G * topk / 2;  // bf16 score staging
+    pool_floats = (pool_floats + 3) & ~3;
+    const size_t smem = sizeof(float) * ((size_t)pool_floats + 128 + (size_t)2 * NQ * topk + (size_t)G * NQ);
+    dim3 grid_r((L + NQ - 1) / NQ, h_kv, B);
+    const float* bias_pk = topk_pack_bias(bias, workspace, B, N, h_kv, G, st);
+#define HILS_TOPK_ROWS_Q(KS_, PL_, BO_)                                                             \
+  hipLaunchKernelGGL((topk_fwd_rows_kernel<1, KS_, PL_, true, true, BO_>), grid_r, dim3(64), smem, st, \
+                     (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, gumbel, drop_mask,       \
+                     indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,          \
+                     block_size, window_size, causal, q_offset, sm_scale, segw, pool_floats,        \
+                     (const uint4*)workspace, bias_pk, per_qhead ? G : 1)
+    const bool plain = !bias && !gumbel && !drop_mask && !sel_logits;
+    const bool bias_only = bias_pk && !gumbel && !drop_mask && !sel_logits;
+    if (D == 64) {
+      if (plain) HILS_TOPK_ROWS_Q(2, true, false); else if (bias_only) HILS_TOPK_ROWS_Q(2, false, true); else HILS_TOPK_ROWS_Q(2, false, false);
+    } else {
+      if (plain) HILS_TOPK_ROWS_Q(4, true, false); else if (bias_only) HILS_TOPK_ROWS_Q(4, false, true); else HILS_TOPK_ROWS_Q(4, false, false);
+    }
+#undef HILS_TOPK_ROWS_Q
+    HILS_CHECK_LAUNCH("hils_topk_fwd");
+    return HILS_OK;
+  }
   if (!per_qhead && G <= 4 && (D == 64 || D == 128)) {
     const int segw = topk_rows_segw(N);
     const int NQ = (G == 1) ? 16 : 8;                                 // queries per wavefront
@@ -2189,20 +2352,24 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
         return HILS_OK;
       }
     }
-#define HILS_TOPK_ROWS_P(G_, KS_, PL_, PK_)                                                         \
-  hipLaunchKernelGGL((topk_fwd_rows_kernel<G_, KS_, PL_, PK_>), grid_r, dim3(64), smem, st,         \
+    const float* bias_pk = topk_pack_bias(bias, workspace, B, N, h_kv, G, st);
+#define HILS_TOPK_ROWS_P(G_, KS_, PL_, PK_, BO_)                                                    \
+  hipLaunchKernelGGL((topk_fwd_rows_kernel<G_, KS_, PL_, PK_, false, BO_>), grid_r, dim3(64), smem, st, \
                      (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, gumbel, drop_mask,       \
                      indices, (bf16_t*)scores, lse_total, sel_logits, L, N, h_kv, G, topk,          \
-                     block_size, window_size, causal, q_offset, sm_scale, segw, pool_floats, packed)
+                     block_size, window_size, causal, q_offset, sm_scale, segw, pool_floats, packed, bias_pk, 1)
 #define HILS_TOPK_ROWS(G_, KS_)                                                                     \
   do {                                                                                             \
     if (plain) {                                                                                   \
-      if (packed) HILS_TOPK_ROWS_P(G_, KS_, true, true); else HILS_TOPK_ROWS_P(G_, KS_, true, false);   \
+      if (packed) HILS_TOPK_ROWS_P(G_, KS_, true, true, false); else HILS_TOPK_ROWS_P(G_, KS_, true, false, false);   \
+    } else if (bias_only) {                                                                        \
+      HILS_TOPK_ROWS_P(G_, KS_, false, true, true);                                                \
     } else {                                                                                       \
-      if (packed) HILS_TOPK_ROWS_P(G_, KS_, false, true); else HILS_TOPK_ROWS_P(G_, KS_, false, false); \
+      if (packed) HILS_TOPK_ROWS_P(G_, KS_, false, true, false); else HILS_TOPK_ROWS_P(G_, KS_, false, false, false); \
     }                                                                                              \
   } while (0)
     const bool plain = !bias && !gumbel && !drop_mask && !sel_logits;
+    const bool bias_only = packed && bias_pk && !gumbel && !drop_mask && !sel_logits;
     if (G == 1) {
       if (D == 64) HILS_TOPK_ROWS(1, 2); else HILS_TOPK_ROWS(1, 4);
     } else if (G == 2) {

@@ -82,14 +82,15 @@ def run_case(pkg, orc, dev, B, L, N, h_kv, G, D, topk, S, W, seed=42, q_offset=0
     want = torch.gather(aux["logits"], -1, safe).masked_fill(~valid.unsqueeze(3).expand(-1, -1, -1, G, -1),
                                                               float("-inf"))
     assert_close_bf16(scores.view(B, L, h_kv, G, topk), want, "scores")
-    if per_qhead and not one_kernel:
-        # without the logit export other launches run (queries bucketed by visible chunks): same results
+    if (per_qhead or use_bias) and not one_kernel:
+        # without the logit export other launches run (queries bucketed by visible chunks, the variants
+        # without per-element options): same results
         idx2, scores2 = pkg.online_softmax_topk_head(
             q_in.to(dev), lmks.to(dev), lse_swa.to(dev), topk, S, W, is_causal=is_causal,
             q_offset=q_offset, is_training=training,
             drop_mask=None if drop is None else drop.to(dev),
             bias=None if bias is None else bias.to(dev),
-            gumbel_noise=None if gumbel is None else gumbel.to(dev), G=G)
+            gumbel_noise=None if gumbel is None else gumbel.to(dev), G=G if per_qhead else 1)
         assert torch.equal(idx2, idx) and torch.equal(scores2, scores), "export and plain launches differ"
     return idx, scores
 
@@ -151,6 +152,39 @@ def test_topk_many_chunks_multi_segment(pkg, orc, dev):
              q_offset=1500 * 64, training=False)
     run_case(pkg, orc, dev, B=1, L=1, N=2048, h_kv=1, G=4, D=128, topk=64, S=64, W=1,
              q_offset=2048 * 64, training=False, dup_keys=True)
+
+
+def test_topk_prefill_beyond_512_chunks_with_bias(pkg, orc, dev):
+    """Long prefill (more chunks than the one-pass kernel holds) with the additive bias: the general
+    kernel loads a block's bias together with its keys."""
+    run_case(pkg, orc, dev, B=1, L=4000, N=700, h_kv=1, G=4, D=128, topk=32, S=64, W=1, q_offset=700 * 64 - 4000,
+             training=False, use_bias=True)
+    run_case(pkg, orc, dev, B=2, L=2500, N=530, h_kv=2, G=3, D=64, topk=16, S=64, W=1, q_offset=530 * 64 - 2500,
+             training=False, use_bias=True, dup_keys=True)
+    run_case(pkg, orc, dev, B=1, L=3000, N=600, h_kv=2, G=2, D=128, topk=8, S=64, W=1, q_offset=600 * 64 - 3000,
+             training=False, use_bias=True)
+    run_case(pkg, orc, dev, B=1, L=2000, N=520, h_kv=1, G=1, D=64, topk=8, S=64, W=0, is_causal=False,
+             training=True, use_bias=True, use_gumbel=True)
+    # five to eight query heads on shared keys: walked head by head
+    run_case(pkg, orc, dev, B=1, L=3000, N=600, h_kv=2, G=8, D=64, topk=32, S=64, W=1, q_offset=600 * 64 - 3000,
+             training=False, use_bias=True)
+    run_case(pkg, orc, dev, B=1, L=2100, N=530, h_kv=1, G=6, D=128, topk=40, S=64, W=1, q_offset=530 * 64 - 2100,
+             training=False, dup_keys=True)
+
+
+def test_topk_prefill_beyond_512_chunks_key_per_query_head(pkg, orc, dev):
+    """Long prefill with one chunk key per query head (outside the one-pass kernel: more than 512 chunks,
+    more than 32 winners, noise, a drop mask): the two-pass kernel walks the heads of a KV head."""
+    run_case(pkg, orc, dev, B=1, L=4000, N=700, h_kv=1, G=4, D=128, topk=32, S=64, W=1, q_offset=700 * 64 - 4000,
+             training=False, per_qhead=True)
+    run_case(pkg, orc, dev, B=2, L=2500, N=530, h_kv=2, G=8, D=64, topk=16, S=64, W=1, q_offset=530 * 64 - 2500,
+             training=False, per_qhead=True, use_bias=True, dup_keys=True)
+    run_case(pkg, orc, dev, B=1, L=3001, N=1100, h_kv=2, G=2, D=128, topk=8, S=64, W=70, q_offset=1100 * 64 - 3001,
+             training=False, per_qhead=True, use_bias=True)
+    run_case(pkg, orc, dev, B=1, L=1000, N=40, h_kv=1, G=3, D=64, topk=48, S=16, W=1, training=True,
+             per_qhead=True, use_bias=True, use_gumbel=True, use_drop=True)
+    run_case(pkg, orc, dev, B=1, L=777, N=300, h_kv=2, G=5, D=64, topk=40, S=64, W=0, is_causal=False,
+             per_qhead=True)
 
 
 def test_topk_one_kernel_path_many_chunks(pkg, orc, dev):
