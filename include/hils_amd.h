@@ -71,7 +71,9 @@ int hils_attn_pool_bwd(const void* mu_q, const void* k, const float* p, const fl
  * (decode) and a workspace, the logits are spread over many workgroups and parked there
  * before a separate selection kernel (or one workgroup per (query, KV head) keeps them in LDS
  * and needs no scratch); with many queries the chunk keys are first repacked there into MFMA
- * operand order.  Without a workspace one fused kernel reads the chunk keys as they are.
+ * operand order, and behind them a bias head-major in blocks of 16 chunks.  Without a workspace one
+ * fused kernel reads the chunk keys as they are (and, with a key per query head or more than four
+ * query heads per KV head, a much slower general kernel runs).
  * workspace_bytes: size of the buffer behind `workspace` (here and in every entry point that takes
  * a workspace); a non-NULL workspace shorter than the matching *_workspace(...) query is rejected
  * with status 1 before anything is launched. */
