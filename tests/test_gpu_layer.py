@@ -90,6 +90,9 @@ def _chunk_weights_case(pkg, orc, dev, K):
                                                 # prefill shapes: two kernels behind the one call
                                                 (1, 1024, 16, 8, 2, 128, 8, 0),
                                                 (2, 1000, 16, 4, 4, 64, 16, 24),
+                                                # eight and five query heads per KV head, decode and prefill
+                                                (64, 1, 2048, 16, 2, 64, 32, 2048 * 64 - 1),
+                                                (1, 2048, 32, 16, 2, 64, 16, 0), (1, 1500, 600, 10, 2, 128, 8, 600 * 64 - 1500),
                                                 (1, 2048, 32, 4, 2, 128, 32, 0),
                                                 (1, 512, 8, 8, 2, 64, 12, 0),
                                                 (1, 777, 40, 6, 2, 128, 32, 1800),   # three heads per KV head
@@ -115,7 +118,8 @@ def test_topk_with_fused_weights_matches_two_calls(pkg, dev, B, L, N, HQ, H, D, 
 
 
 @pytest.mark.parametrize("L,N,HQ,H,D,K", [(3000, 47, 8, 2, 128, 16), (9000, 300, 3, 1, 64, 32),
-                                          (2048, 32, 8, 4, 64, 8), (1500, 24, 16, 1, 128, 8)])
+                                          (2048, 32, 8, 4, 64, 8), (1500, 24, 16, 1, 128, 8),
+                                          (4096, 64, 16, 2, 64, 32), (3000, 47, 10, 2, 128, 16)])
 def test_topk_weights_reads_bf16_lse_in_place(pkg, dev, L, N, HQ, H, D, K):
     """lse_swa in bf16, as the layer hands it over: the one-pass prefill kernel reads it in place
     (other shapes convert it first); either way the result is that of the fp32 copy of the same values."""
@@ -175,6 +179,7 @@ def test_decode_step_replays_as_hip_graph(pkg, orc, dev):
 
 @pytest.mark.parametrize("B,Lq,Lkv,HQ,H,D,K", [(32, 1, 32768, 32, 8, 128, 32), (16, 1, 16512, 8, 8, 64, 16),
                                                (50, 2, 20480, 4, 1, 128, 8), (24, 1, 65536, 12, 4, 64, 64),
+                                               (64, 1, 32768, 16, 2, 64, 32), (20, 1, 65536, 40, 8, 128, 32),
                                                # not taken by the one-launch kernel (few rows): the two calls
                                                (2, 1, 4096, 8, 2, 128, 16)])
 def test_decode_step_one_launch(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
