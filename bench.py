@@ -465,6 +465,23 @@ def bench_ops(pkg, dev, iters=3):
     out["topk_prefill"] = {"workload": "B1 L32768 hq32/hkv8 D128 N512 top32 (selection + weights)", "us": t0 * 1e3}
     out["topk_prefill_bias"] = {"workload": "same, with a prior bias (B,N,h_q)", "us": t1 * 1e3}
     del q, k, lse_p, lmk, prior
+    # the same operator at the head counts of the reference's own model configurations (eight query heads per
+    # KV head; configs/hils_attention: 16/2 heads of 64, 32/4 heads of 128) and on a 128K prefill (2048 chunks),
+    # with shared chunk keys and in the layer's default mode (a key per query head + the prior bias)
+    for name, L, HQ, HK, D in (("hq16_hkv2_d64", 32768, 16, 2, 64), ("hq32_hkv4_d128", 32768, 32, 4, 128),
+                               ("128k_hq32_hkv8_d128", 131072, 32, 8, 128), ("128k_hq16_hkv2_d64", 131072, 16, 2, 64)):
+        N = L // 64
+        q = gpu_randn((1, L, HQ, D), gen, dev)
+        lmk = gpu_randn((1, N, HK, D), gen, dev)
+        lmk_q = gpu_randn((1, N, HQ, D), gen, dev)
+        lse_p = torch.randn(1, L, HQ, device=dev, generator=gen) * 3 + 5
+        prior = torch.randn(1, N, HQ, device=dev, generator=gen) * 0.5
+        with torch.no_grad():
+            t0 = timed(lambda: pkg.topk_chunk_weights(q, lmk, lse_p, 32, 64, 1), 3)
+            t1 = timed(lambda: pkg.topk_chunk_weights(q, lmk_q, lse_p, 32, 64, 1, prior_b=prior, num_kv_heads=HK), 3)
+        out["topk_prefill_" + name] = {"workload": f"B1 L{L} hq{HQ}/hkv{HK} D{D} N{N} top32 (selection + weights)",
+                                       "us": t0 * 1e3, "key_per_query_head_prior_bias_us": t1 * 1e3}
+        del q, lmk, lmk_q, lse_p, prior
     # rotary embedding of q and k: B1 L32768 hq32/hkv8 D128
     L, HQ, HK, D = 32768, 32, 8, 128
     q = gpu_randn((1, L, HQ, D), gen, dev)
