@@ -1412,7 +1412,12 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
               float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
               int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
               float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages,
-              int lmk_hm, int lmk_cap, int perq, float* dyn, const long row, TopkRowSharedT<GMAX>* sh_p = nullptr) {
+              int lmk_hm, int lmk_cap, int perq, int bias_inplace, float* dyn, const long row,
+              TopkRowSharedT<GMAX>* sh_p = nullptr) {
+  // bias_inplace (with a bias only): the staged bias and the logits share one array, a slot holding the
+  // bias until the chunk's logit is added to it; a winner's bias is then read again from global memory
+  // and its raw score is the biased logit minus that bias (one rounding of the sum away from the raw
+  // product, far inside the bf16 the score is returned in).  For rows whose two arrays do not fit the LDS.
   // perq: one chunk key per QUERY head, lmks = (B,N,h_kv*G,D) / (B,h_kv*G,lmk_cap,D) / (num_pages,h_kv*G,D):
   // the row streams G key tensors, a key group of head g gives the logits of MFMA column g only
   constexpr int LR = D / 8, TPI = 64 / LR;
@@ -1428,8 +1433,9 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   // the row's additive bias (the layer's prior bias: added to the logits for the log-sum-exp and the
   // selection, and, rounded the layer's way, to the winners' scores before the inter-chunk softmax),
   // staged head-major like the logits; 0 for the chunks past the causal limit
-  float* bias_s = (float*)(page_s + NPG);     // [GMAX][NP], only with a bias
-  const int NBS = bias ? GMAX * NP : 0;       // the wavefronts' staging areas follow
+  const bool inplace = bias && bias_inplace;
+  float* bias_s = inplace ? logit_s : (float*)(page_s + NPG);  // [GMAX][NP], only with a bias
+  const int NBS = (bias && !inplace) ? GMAX * NP : 0;          // the wavefronts' staging areas follow
   __shared__ TopkRowSharedT<GMAX> sh_own;
   TopkRowSharedT<GMAX>& sh = FUSED ? *sh_p : sh_own;  // FUSED: the caller's, which the attention reads after the return
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1499,7 +1505,7 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     constexpr int KS = D / 32;
     constexpr int ROWB = 2 * D + 16;
     constexpr int LPT = 16 / TPI;  // load instructions per 16-key tile
-    char* stage_w = (char*)(bias_s + NBS) + (size_t)wave * 16 * ROWB;
+    char* stage_w = (char*)((float*)(page_s + NPG) + NBS) + (size_t)wave * 16 * ROWB;
     const int col = lane & 15, j = lane >> 4;
     char* const w_addr = stage_w + tsub * ROWB + piece * 16;
     const char* const k_addr = stage_w + col * ROWB + j * 16;
@@ -1560,11 +1566,12 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
             for (int i = 0; i < 4; ++i)
               if (pg4[i] < 0) out[i] = HILS_NEG_INF;
           }
-          *(f32x4_t*)&logit_s[col * NP + c0] = out;
+          if (!inplace) *(f32x4_t*)&logit_s[col * NP + c0] = out;
           if (bias) {  // -inf stays -inf: the staged bias is finite (0 past the causal limit)
             const f32x4_t bb = *(const f32x4_t*)&bias_s[col * NP + c0];
 #pragma unroll
             for (int i = 0; i < 4; ++i) out[i] = __fadd_rn(out[i], bb[i]);
+            if (inplace) *(f32x4_t*)&logit_s[col * NP + c0] = out;
           }
           // running log-sum-exp of this lane's head over the keys it has seen
           const float mn = fmaxf(fmaxf(m_run, fmaxf(out[0], out[1])), fmaxf(out[2], out[3]));
@@ -1674,12 +1681,12 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
       }
     }
   };
-  if (bias) form_keys(std::true_type{}); else form_keys(std::false_type{});
+  if (bias && !inplace) form_keys(std::true_type{}); else form_keys(std::false_type{});
   if (sel_logits_out) {  // the exported selection logits (a debugging output)
     for (int i = tid; i < G * N; i += THREADS) {
       const int g = i / N, c = i - g * N;
       float xv = c < lim ? logit_s[g * NP + c] : HILS_NEG_INF;
-      if (bias && c < lim) xv = __fadd_rn(xv, bias_s[g * NP + c]);
+      if (bias && !inplace && c < lim) xv = __fadd_rn(xv, bias_s[g * NP + c]);
       sel_logits_out[(row * G + g) * (long)N + c] = xv;
     }
   }
@@ -1733,18 +1740,38 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     cand_total += v;
     cand_base += (w2 < wave) ? v : 0;
   }
+  // the bias of (chunk c, head g) and the raw scaled score of that pair
+  auto bias_at = [&](int c, int g) -> float {
+    if (!inplace) return bias_s[g * NP + c];
+    long e0;
+    if (PAGED) {
+      const int pg = page_s[c];
+      e0 = ((long)(pg < 0 ? 0 : pg) * h_kv + hk) * G;
+    } else if (lmk_hm) {
+      e0 = ((b * h_kv + hk) * (long)lmk_cap + c) * G;
+    } else {
+      e0 = ((b * N + c) * (long)h_kv + hk) * G;
+    }
+    return bias[e0 + g];
+  };
   // ---- FUSED: what every wavefront does once lane kk (kk < nc) holds winner kk's chunk (ascending) ----
   auto fused_tail = [&](int widx, int nc) __attribute__((always_inline)) {
     const bool has = lane < nc;
-    float xs[GMAX], wgt[GMAX], wloc[GMAX];
+    float xs[GMAX], wgt[GMAX], wloc[GMAX], bws[GMAX];
+    // (the winner's biases first, all heads' loads in flight together: read from global memory when the
+    // bias shares the logits' array)
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) bws[g] = (bias && has && g < G) ? bias_at(widx, g) : 0.f;
 #pragma unroll
     for (int g = 0; g < GMAX; ++g) {
       xs[g] = (has && g < G) ? logit_s[g * NP + widx] : HILS_NEG_INF;  // raw scaled score
+      const float bw = bws[g];
+      if (inplace && has && g < G) xs[g] = __fsub_rn(xs[g], bw);
       // the layer's inter-chunk softmax over [scores as bf16 (+ bias as bf16, summed in bf16), lse_swa]
       float x = HILS_NEG_INF;
       if (has && g < G) {
         x = bf2f(f2bf(xs[g]));
-        if (bias) x = bf2f(f2bf(x + bf2f(f2bf(bias_s[g * NP + widx]))));
+        if (bias) x = bf2f(f2bf(x + bf2f(f2bf(bw))));
       }
       const float m = fmaxf(wave_max_f(x), swa[g]);
       if (m == HILS_NEG_INF) {  // every logit -inf: NaN row, as a softmax gives
@@ -1874,7 +1901,8 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
   for (int kk = tid; kk < topk; kk += THREADS) indices[row * topk + kk] = (kk < nc) ? sh.cand_i[0][kk] : -1;
   for (int p = tid; p < topk * G; p += THREADS) {
     const int g = p / topk, kk = p - g * topk;
-    const float val = (kk < nc) ? logit_s[g * NP + sh.cand_i[0][kk]] : HILS_NEG_INF;
+    float val = (kk < nc) ? logit_s[g * NP + sh.cand_i[0][kk]] : HILS_NEG_INF;
+    if (inplace && kk < nc) val = __fsub_rn(val, bias_at(sh.cand_i[0][kk], g));
     scores[(row * G + g) * (long)topk + kk] = f2bf(val);
   }
   // optional: the layer's inter-chunk softmax over [scores (as bf16), lse_swa], one wavefront per head
@@ -1885,9 +1913,11 @@ topk_row_body(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
     for (int g2 = 1; g2 < GMAX; ++g2) lse_g = (g == g2) ? swa[g2] : lse_g;
     float x = HILS_NEG_INF;
     if (lane < topk && lane < nc) {
-      x = bf2f(f2bf(logit_s[g * NP + sh.cand_i[0][lane]]));
+      const int cw = sh.cand_i[0][lane];
+      const float bw = bias ? bias_at(cw, g) : 0.f;
+      x = bf2f(f2bf(inplace ? __fsub_rn(logit_s[g * NP + cw], bw) : logit_s[g * NP + cw]));
       // the layer adds the gathered bias, cast to the scores' dtype, to the bf16 scores
-      if (bias) x = bf2f(f2bf(x + bf2f(f2bf(bias_s[g * NP + sh.cand_i[0][lane]]))));
+      if (bias) x = bf2f(f2bf(x + bf2f(f2bf(bw))));
     }
     const float m = fmaxf(wave_max_f(x), lse_g);
     bf16_t* wrow = weights_out + (row * G + g) * (long)(topk + 1);
@@ -1911,12 +1941,12 @@ topk_row_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ lmks,
                 float* __restrict__ sel_logits_out, bf16_t* __restrict__ weights_out, int L, int N,
                 int NP, int h_kv, int G, int topk, int block_size, int window_size, int causal, int q_offset,
                 float sm_scale, const int32_t* __restrict__ page_table, int max_pages, int num_pages,
-                int lmk_hm, int lmk_cap, int perq) {
+                int lmk_hm, int lmk_cap, int perq, int bias_inplace) {
   extern __shared__ __align__(16) float topk_row_dyn[];
   topk_row_body<D, GMAX, NW, PAGED>(q, lmks, lse_swa, bias, indices, scores, lse_total_out, sel_logits_out,
                                     weights_out, L, N, NP, h_kv, G, topk, block_size, window_size, causal,
                                     q_offset, sm_scale, page_table, max_pages, num_pages, lmk_hm, lmk_cap, perq,
-                                    topk_row_dyn, (long)blockIdx.x);
+                                    bias_inplace, topk_row_dyn, (long)blockIdx.x);
 }
 
 // The remote branch of a decode step in one launch: the workgroup of a (query, KV head) row selects
@@ -1935,7 +1965,7 @@ struct DsArgs {
   int L, N, NP, h_kv, G, topk, block_size, window_size, q_offset;
   float sm_scale_sel;
   const int32_t* page_table;
-  int max_pages, num_pages, lmk_hm, lmk_cap, perq;
+  int max_pages, num_pages, lmk_hm, lmk_cap, perq, bias_inplace;
   int stagger_ticks;  // 100 MHz ticks by which every other row of an XCD starts late (0: none)
   DrDims dr;
 };
@@ -1959,7 +1989,7 @@ __global__ void __launch_bounds__(DS_WAVES * 64) decode_step_kernel(DsArgs a) {
                                              a.sel_logits, a.weights, a.L, a.N, a.NP, a.h_kv, a.G, a.topk,
                                              a.block_size, a.window_size, 1, a.q_offset, a.sm_scale_sel,
                                              a.page_table, a.max_pages, a.num_pages, a.lmk_hm, a.lmk_cap, a.perq,
-                                             ds_dyn, row, &ds_sh);
+                                             a.bias_inplace, ds_dyn, row, &ds_sh);
   // The attention reads the row's indices and weights where the selection left them in LDS: the
   // pointers are offset so that the row's entries of the (B, L, heads, ...) tensors fall there.  Its
   // staging areas lie over the selection's logits: the barrier that separates the two uses runs in
@@ -1985,19 +2015,27 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
 // LDS of a row workgroup before the wavefronts' staging areas: raw logits [gm][NP] (gm = 4 head slots, 8
 // with more than four query heads per KV head), pooled scores, page ids (paged chunk keys), the staged
 // bias [gm][NP]
-static size_t topk_row_smem_base(int N, int G, bool paged, bool with_bias) {
+// (inplace: the bias shares the logits' array)
+static size_t topk_row_smem_base(int N, int G, bool paged, bool with_bias, bool inplace) {
   const int NP = (N + 63) & ~63;
   const int gm = G <= 4 ? 4 : 8;
-  return (size_t)(gm + 1 + (paged ? 1 : 0) + (with_bias ? gm : 0)) * NP * sizeof(float);
+  return (size_t)(gm + 1 + (paged ? 1 : 0) + (with_bias && !inplace ? gm : 0)) * NP * sizeof(float);
 }
 static size_t topk_row_shared_bytes(int G) { return G <= 4 ? sizeof(TopkRowSharedT<4>) : sizeof(TopkRowSharedT<8>); }
+// Does a row workgroup of `waves` wavefronts fit the LDS?  *inplace: the bias has to share the logits' array.
+static bool topk_row_fits(int N, int G, int D, bool paged, bool with_bias, int waves, int* inplace) {
+  const size_t rest = (size_t)waves * 16 * (2 * D + 16) + topk_row_shared_bytes(G);
+  *inplace = 0;
+  if (topk_row_smem_base(N, G, paged, with_bias, false) + rest <= 158 * 1024) return true;
+  *inplace = 1;
+  return with_bias && topk_row_smem_base(N, G, paged, true, true) + rest <= 158 * 1024;
+}
 
 // plain: no Gumbel noise and no drop mask; a bias is staged in LDS beside the logits and must fit there
 static bool topk_use_row(long rows, int N, int G, int D, int per_qhead, bool plain, bool with_bias = false,
                          bool paged = false) {
-  if ((with_bias || G > 4) &&
-      topk_row_smem_base(N, G, paged, with_bias) + (size_t)8 * 16 * (2 * D + 16) + topk_row_shared_bytes(G) > 158 * 1024)
-    return false;
+  int inplace;
+  if ((D == 64 || D == 128) && !topk_row_fits(N, G, D, paged, with_bias, 8, &inplace)) return false;
   (void)per_qhead;  // shared chunk keys or one per query head: the same kernel
   return plain && G <= 8 && (D == 64 || D == 128) && N >= 256 && N <= TOPK_R_MAXN &&
          rows >= 96 && rows <= 2147483647L;
@@ -2011,13 +2049,19 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, c
   const long rows = (long)B * L * h_kv;
   const int NP = (N + 63) & ~63;
   // then 16 padded key rows of staging per wavefront
-  const size_t smem_base = topk_row_smem_base(N, G, page_table != nullptr, bias != nullptr);
   const size_t stage_b = (size_t)16 * (2 * D + 16);
   // one round of rows or less: 16 wavefronts per row (the whole compute unit streams one row) if
   // their staging areas fit the LDS beside the logits; more rows than compute units: 8, so that
   // two workgroups share a unit and one row's selection overlaps the other row's streaming
-  const bool wide = rows <= topk_cus() && smem_base + 16 * stage_b + topk_row_shared_bytes(G) <= 158 * 1024;
-  const size_t smem = smem_base + (wide ? 16 : 8) * stage_b;
+  // (with a bias: 16 only if that does not push the bias into the logits' array where 8 would not)
+  int ip16 = 0, ip8 = 0;
+  const bool fit16 = rows <= topk_cus() && topk_row_fits(N, G, D, page_table != nullptr, bias != nullptr, 16, &ip16);
+  const bool fit8 = topk_row_fits(N, G, D, page_table != nullptr, bias != nullptr, 8, &ip8);
+  HILS_REQUIRE(fit16 || fit8, "hils_topk_fwd: too many chunks (%d) for the logits of the row's heads in LDS", N);
+  const bool wide = fit16 && (!ip16 || !fit8 || ip8);
+  const int bias_inplace = wide ? ip16 : ip8;
+  const size_t smem = topk_row_smem_base(N, G, page_table != nullptr, bias != nullptr, bias_inplace != 0) +
+                      (wide ? 16 : 8) * stage_b;
 #define TOPK_ROW_CALL_G(D_, G_, W_, P_)                                                           \
   do {                                                                                           \
     auto kern = topk_row_kernel<D_, G_, W_, P_>;                                                 \
@@ -2027,7 +2071,7 @@ static int topk_fwd_row(const void* q, const void* lmks, const float* lse_swa, c
                        (const bf16_t*)q, (const bf16_t*)lmks, lse_swa, bias, indices, (bf16_t*)scores, \
                        lse_total, sel_logits, (bf16_t*)weights, L, N, NP, h_kv, G, topk,         \
                        block_size, window_size, causal, q_offset, sm_scale, page_table, max_pages, \
-                       num_pages, lmk_hm, lmk_cap, perq);                                        \
+                       num_pages, lmk_hm, lmk_cap, perq, bias_inplace);                          \
   } while (0)
 #define TOPK_ROW_CALL_W(D_, W_, P_)                                                               \
   do {                                                                                           \
@@ -2069,15 +2113,18 @@ static int decode_step_launch(const void* q, const void* lmks, const void* k, co
   const int G = HQ / H;
   const long rows = (long)B * L * H;
   const int NP = (N + 63) & ~63;
-  const size_t sel_b = topk_row_smem_base(N, G, lmk_paged != 0, bias != nullptr) + (size_t)DS_WAVES * 16 * (2 * D + 16);
-  HILS_REQUIRE(sel_b + topk_row_shared_bytes(G) <= 158 * 1024,
+  int bias_inplace = 0;
+  const bool sel_fits = topk_row_fits(N, G, D, lmk_paged != 0, bias != nullptr, DS_WAVES, &bias_inplace);
+  const size_t sel_b = topk_row_smem_base(N, G, lmk_paged != 0, bias != nullptr, bias_inplace != 0) +
+                       (size_t)DS_WAVES * 16 * (2 * D + 16);
+  HILS_REQUIRE(sel_fits,
                "hils_decode_step: too many chunks (%d) for the logits (and the bias) of the row's heads in LDS", N);
   const size_t att_b = dr_smem_bytes(D, G, DS_WAVES);
   const size_t smem = sel_b > att_b ? sel_b : att_b;
   DsArgs a;
   a.q = (const bf16_t*)q; a.lmks = (const bf16_t*)lmks; a.k = (const bf16_t*)k; a.v = (const bf16_t*)v;
   a.lse_swa = lse_swa; a.bias = bias; a.indices = indices;
-  a.lmk_hm = lmk_hm; a.lmk_cap = lmk_cap; a.perq = perq;
+  a.lmk_hm = lmk_hm; a.lmk_cap = lmk_cap; a.perq = perq; a.bias_inplace = bias_inplace;
   a.stagger_ticks = rows <= topk_cus() ? 800 : 0;  // one round of rows: they would run in step
   a.scores = (bf16_t*)scores; a.weights = (bf16_t*)weights; a.o = (bf16_t*)o;
   a.lse_total = lse_total; a.sel_logits = sel_logits;
@@ -2462,7 +2509,8 @@ extern "C" int hils_topk_fwd_weights_paged(const void* q, const void* lmk_pages,
                "hils_topk_fwd_weights_paged: needs G <= 8, D in {64, 128}, N <= %d, topk <= %d", TOPK_R_MAXN,
                TOPK_MAXK);
   HILS_REQUIRE((long)B * L * h_kv <= 2147483647L, "hils_topk_fwd_weights_paged: grid too large");
-  HILS_REQUIRE((!bias_pages && G <= 4) || topk_row_smem_base(N, G, true, bias_pages != nullptr) + (size_t)8 * 16 * (2 * D + 16) + topk_row_shared_bytes(G) <= 158 * 1024,
+  int paged_inplace;
+  HILS_REQUIRE(topk_row_fits(N, G, D, true, bias_pages != nullptr, 8, &paged_inplace),
                "hils_topk_fwd_weights_paged: too many chunks (%d) for the logits (and the bias) of the row's heads in LDS", N);
   if (int rc = topk_fwd_row(q, lmk_pages, lse_swa, bias_pages, indices, scores, lse_total, sel_logits, weights, B, L,
                             N, h_kv, G, D, topk, block_size, window_size, 1, q_offset, sm_scale,

@@ -298,10 +298,12 @@ int hils_sparse_attn_decode_paged(const void* q, const void* k_pages, const void
  * and the bias gathered into the inter-chunk softmax), fp32, NULL for none; laid out like the chunk
  * keys with the G heads of a KV head in place of D: (B,N,H*G), (B,H,lmk_cap,G) or (num_pages,H*G).
  * Covered shapes (hils_decode_step_covers returns 1): causal, block_size 64,
- * D = Dv in {64, 128}, HQ/H <= 8, 256 <= N <= 4096 (fewer with a bias, which is staged in LDS beside
- * the logits: about 3300 chunks, 3000 on the paged entry point, at D = 128; and fewer with more than
- * four query heads per KV head, whose logits take eight rows of LDS: 2752 chunks at D = 128 and 3200 at
- * D = 64, with a bias 1472 and 1664; the covers function knows), topk <= 64, at least 96 rows B*L*H. */
+ * D = Dv in {64, 128}, HQ/H <= 8, 256 <= N <= 4096 (with more than four query heads per KV head, whose
+ * logits take eight rows of LDS: 2752 chunks at D = 128 and 3200 at D = 64, 2496 / 2880 with chunk keys
+ * per page; the covers function knows), topk <= 64, at least 96 rows B*L*H.  A bias is staged in LDS
+ * beside the logits; where the two do not fit side by side (from about 2900 chunks at D = 128, half of
+ * that with eight head rows) it shares the logits' array and a winner's raw score is its biased logit
+ * minus the bias (one fp32 rounding away from the product, far inside the bf16 it is returned in). */
 int hils_decode_step_covers(int B, int L, int N, int HQ, int H, int D, int topk, int block_size, int with_bias);
 int hils_decode_step(const void* q, const void* lmks, const void* k, const void* v, const float* lse_swa,
                      const float* bias, int32_t* indices, void* scores, void* weights, void* o,

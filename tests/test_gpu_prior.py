@@ -103,7 +103,9 @@ def test_prefill_selection_with_a_key_per_query_head(pkg, orc, dev, L, N, HQ, H,
 
 @pytest.mark.parametrize("B,Lq,Lkv,HQ,H,D,K", [(32, 1, 32768, 32, 8, 128, 32), (16, 1, 16512, 8, 8, 64, 16),
                                                (50, 2, 20480, 4, 1, 128, 8), (2, 1, 4096, 8, 2, 128, 16),
-                                               (64, 1, 32768, 16, 2, 64, 32), (16, 1, 65536, 40, 8, 128, 16)])
+                                               (64, 1, 32768, 16, 2, 64, 32), (16, 1, 65536, 40, 8, 128, 16),
+                                               # logits and bias of the row do not fit the LDS side by side: one array
+                                               (48, 1, 131072, 16, 2, 64, 32), (12, 1, 196608, 32, 8, 128, 32)])
 def test_decode_step_with_prior_bias(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
     """decode_step(prior_b=): one launch per step with the bias staged beside the logits; the chunk
     keys and the bias token-major (the reference's layout) and head-major (the cache layers')."""
@@ -152,7 +154,8 @@ def test_decode_step_with_prior_bias(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
 @pytest.mark.parametrize("B,Lq,Lkv,HQ,H,D,K", [(32, 1, 32768, 32, 8, 128, 32), (50, 2, 20480, 4, 1, 128, 8),
                                                (24, 1, 65536, 12, 4, 64, 64), (48, 1, 16512, 6, 2, 64, 16),
                                                (48, 1, 16384, 4, 2, 64, 8), (64, 1, 32768, 16, 2, 64, 32),
-                                               (48, 1, 65536, 14, 2, 128, 16)])
+                                               (48, 1, 65536, 14, 2, 128, 16),
+                                               (48, 1, 131072, 16, 2, 64, 32)])  # bias and logits in one array
 def test_decode_step_with_a_key_per_query_head(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
     """The layer's default pooling in decode: one attention-pooled chunk key per query head and its
     prior bias.  One launch per step; token-major, head-major and paged keys give the same bits; the

@@ -341,8 +341,20 @@ def test_topk_workgroup_per_row_path(pkg, orc, dev, B, L, N, h_kv, G, D, topk, o
              training=False, dup_keys=(N == 1000))
 
 
+def test_topk_workgroup_per_row_path_bias_shares_the_logit_array(pkg, orc, dev):
+    """More chunks than the LDS holds logits and bias side by side for: the bias is staged in the logits'
+    array and a winner's bias is read again from global memory."""
+    run_case(pkg, orc, dev, B=12, L=1, N=3500, h_kv=8, G=4, D=128, topk=32, S=64, W=1, q_offset=3500 * 64 - 1,
+             training=False, use_bias=True)
+    run_case(pkg, orc, dev, B=100, L=1, N=4096, h_kv=1, G=3, D=64, topk=64, S=64, W=1, q_offset=4096 * 64 - 1,
+             training=False, use_bias=True, dup_keys=True)
+    run_case(pkg, orc, dev, B=30, L=2, N=3000, h_kv=2, G=6, D=128, topk=16, S=64, W=1, q_offset=3000 * 64 - 2,
+             training=False, use_bias=True)  # (eight head slots: over the in-place limit too, the two-kernel path)
+
+
 @pytest.mark.parametrize("B,L,N,h_kv,G,D,topk,bias", [(64, 1, 1500, 2, 8, 64, 32, True), (100, 1, 1024, 1, 7, 128, 16, False),
-                                                     (48, 2, 600, 2, 5, 128, 8, True)])
+                                                     (48, 2, 600, 2, 5, 128, 8, True),
+                                                     (48, 1, 2048, 2, 8, 64, 32, True)])  # bias and logits in one array
 def test_topk_workgroup_per_row_path_key_per_query_head(pkg, orc, dev, B, L, N, h_kv, G, D, topk, bias):
     """The same kernel with one chunk key per query head and five to eight heads per KV head."""
     run_case(pkg, orc, dev, B=B, L=L, N=N, h_kv=h_kv, G=G, D=D, topk=topk, S=64, W=1, q_offset=N * 64 - L,
