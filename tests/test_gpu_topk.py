@@ -453,16 +453,17 @@ def test_topk_one_pass_kernel_all_scores_equal(pkg, orc, dev):
     assert torch.equal(idx.cpu(), orc.topk_select(dbg["sel_logits"].cpu(), dbg["lse_total"].cpu(), lim, topk))
 
 
-def test_topk_one_pass_kernel_rows_without_any_mass(pkg, orc, dev):
+@pytest.mark.parametrize("G,D,per_qhead", [(4, 128, False), (8, 64, False), (5, 128, False), (4, 64, True), (7, 64, True)])
+def test_topk_one_pass_kernel_rows_without_any_mass(pkg, orc, dev, G, D, per_qhead):
     """Rows whose lse_swa is -inf (the local branch saw no key: a landmark row with window 1) through
     the one-pass prefill kernel, both launch variants.  In the first chunk such a row sees no chunk
     either: lse_total is -inf, nothing is selected (indices -1, scores -inf) and no NaN is formed;
     later rows select from the chunk logits alone."""
     note("one-pass top-k: rows with lse_swa = -inf")
-    B, L, N, h_kv, G, D, topk, S, W = 1, 4096, 64, 2, 4, 128, 8, 64, 1
+    B, L, N, h_kv, topk, S, W = 1, 4096, 64, 2, 8, 64, 1
     gen = torch.Generator().manual_seed(63)
     q = torch.randn(B, L, h_kv * G, D, generator=gen).bfloat16()
-    lmks = torch.randn(B, N, h_kv, D, generator=gen).bfloat16()
+    lmks = torch.randn(B, N, h_kv * G if per_qhead else h_kv, D, generator=gen).bfloat16()
     lse = torch.randn(B, L, h_kv * G, generator=gen) * 3 + 5
     lse[:, S - 1::S] = float("-inf")   # every landmark row
     lse[:, :S:7] = float("-inf")       # and some more rows of the first chunk
@@ -470,7 +471,7 @@ def test_topk_one_pass_kernel_rows_without_any_mass(pkg, orc, dev):
     outs = []
     for dbg in ({}, None):
         idx, scores = pkg.online_softmax_topk_head(q.to(dev), lmks.to(dev), lse.to(dev), topk, S, W,
-                                                   is_training=False, _debug=dbg)
+                                                   is_training=False, G=G if per_qhead else 1, _debug=dbg)
         torch.cuda.synchronize()
         outs.append((idx.cpu(), scores.float().cpu()))
         assert torch.all(idx[:, :S] == -1), "rows that see no chunk must select nothing"
