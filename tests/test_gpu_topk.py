@@ -103,6 +103,8 @@ def test_topk_reference_shape(pkg, orc, dev):
 @pytest.mark.parametrize("G,D", [(1, 64), (2, 128), (4, 128), (8, 64), (16, 64), (3, 64)])
 def test_topk_group_sizes(pkg, orc, dev, G, D):
     run_case(pkg, orc, dev, B=1, L=640, N=10, h_kv=2, G=G, D=D, topk=4, S=64, W=1)
+    # and without a workspace: the kernel that reads the chunk keys as they are
+    run_case(pkg, orc, dev, B=1, L=640, N=10, h_kv=2, G=G, D=D, topk=4, S=64, W=1, one_kernel=True)
 
 
 @pytest.mark.parametrize("L", [999, 1023, 1100, 17])
