@@ -2325,7 +2325,7 @@ static int topk_fwd_impl(const void* q, const void* lmks, const float* lse_swa,
   }
   // the one-pass kernel with one chunk key per query head (a wavefront per head for the logits, G = 3..8),
   // or with more than four query heads on shared keys (two wavefronts per four queries)
-  if ((per_qhead || G > 4) && workspace && hils_topk_group_covers(N, G, D, topk, per_qhead, !gumbel && !drop_mask)) {
+  if ((per_qhead || G > 4) && workspace && hils_topk_group_covers(N, G, D, topk, per_qhead, !gumbel && !drop_mask)) {  // (G = 2..8 / 5..8)
     const int nblk16 = (N + 15) / 16;
     const int h_lmk = per_qhead ? h_kv * G : h_kv;
     const long total = (long)B * h_lmk * nblk16 * (D / 32) * 64;

@@ -21,7 +21,7 @@
 // Five to eight query heads per KV head (HALF below) take two wavefronts per four queries, one for the
 // heads 0..3 and one for the rest: each forms the partial selection scores of its heads, the two
 // trade them through LDS, and both then select on the same scores and write their own heads' outputs.
-// Covers G = 1 and 3..8, D in {64, 128}, N <= 512, topk <= 32, an optional additive bias per
+// Covers G = 1..8, D in {64, 128}, N <= 512, topk <= 32, an optional additive bias per
 // (chunk, head) (the layer's prior bias), no Gumbel noise / drop mask; everything else runs on the
 // kernels of topk.hip.  With a bias the registers hold the biased logits (what the log-sum-exp and
 // the selection work on) and a winner's raw score is its logit minus the bias again.
@@ -656,8 +656,8 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
 
 // plain: no Gumbel noise and no drop mask (a bias is fine)
 bool hils_topk_group_covers(int N, int G, int D, int topk, int per_qhead, bool plain) {
-  if (per_qhead && (G < 3 || G > 8)) return false;  // (one head a group: the keys are shared anyway)
-  return plain && (G == 1 || (G >= 3 && G <= 8)) && (D == 64 || D == 128) && N <= 16 * TG_NB && topk <= 32;
+  if (per_qhead && (G < 2 || G > 8)) return false;  // (one head a group: the keys are shared anyway)
+  return plain && G >= 1 && G <= 8 && (D == 64 || D == 128) && N <= 16 * TG_NB && topk <= 32;
 }
 
 template <int GMAX, int KS, bool BIAS, bool PERQ, bool HALF>
@@ -689,7 +689,9 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
                            int G, int D, int topk, int block_size, int window_size, int causal, int q_offset,
                            float sm_scale, int lse_bf16, int per_qhead, void* stream) {
   hipStream_t st = (hipStream_t)stream;
-  const int GM = (G == 1) ? 1 : 4;
+  // rows of a tile: queries x 1, 2 or 4 heads (three heads, and two with a key per query head, whose
+  // wavefronts are one per head of four: padding rows)
+  const int GM = (G == 1) ? 1 : ((G == 2 && !per_qhead) ? 2 : 4);
   const bool halves = G > 4;  // two wavefronts per four queries
   const int QGROUPS = halves ? (per_qhead ? 4 : 1) : (per_qhead ? 4 : TG_WAVES);  // wavefronts (pairs) of a workgroup with queries of their own
   const int NQ = 16 / GM;
@@ -724,6 +726,7 @@ int hils_topk_group_launch(const void* q, const void* lmk_packed, const float* l
     if (bias) TG_RANGE_B(G_, KS_, true, P_, H_); else TG_RANGE_B(G_, KS_, false, P_, H_);             \
   } while (0)
     if (GM == 1) { if (D == 64) TG_RANGE(1, 2, false, false); else TG_RANGE(1, 4, false, false); }
+    else if (GM == 2) { if (D == 64) TG_RANGE(2, 2, false, false); else TG_RANGE(2, 4, false, false); }
     else if (halves && per_qhead) { if (D == 64) TG_RANGE(4, 2, true, true); else TG_RANGE(4, 4, true, true); }
     else if (halves) { if (D == 64) TG_RANGE(4, 2, false, true); else TG_RANGE(4, 4, false, true); }
     else if (per_qhead) { if (D == 64) TG_RANGE(4, 2, true, false); else TG_RANGE(4, 4, true, false); }

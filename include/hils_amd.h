@@ -117,7 +117,7 @@ int hils_topk_fwd_weights(const void* q, const void* lmks, const float* lse_swa,
 /* hils_topk_fwd_weights for lse_swa in bf16, the dtype the reference's layer hands it over in
  * (lse_sum.to(hidden_states.dtype), models/FlashHiLS/hils_attention.py:547; its kernels read it in
  * that dtype, ops/topk_head_softmax.py:1291-1367): saves the conversion pass.  Only the shapes
- * hils_topk_lse16_covers accepts (many queries, shared chunk keys, G = 1 or 3..8, N <= 512, topk <= 32,
+ * hils_topk_lse16_covers accepts (many queries, shared chunk keys, G <= 8, N <= 512, topk <= 32,
  * no noise / drop mask: the one-pass prefill kernel), with the workspace of
  * hils_topk_fwd_workspace; other shapes are rejected and take hils_topk_fwd_weights with fp32.
  * bias / prior_b as in hils_topk_fwd_weights (NULL for none). */

@@ -20,7 +20,8 @@ def _oracle_step(orc, q, lmk, lse, pb, k, v, K, S, W, off, idx, scores_bf16):
 
 @pytest.mark.parametrize("L,N,HQ,H,D,K,off", [(4096, 64, 8, 2, 128, 16, 0), (9000, 300, 3, 1, 64, 32, 300 * 64 - 9000),
                                              (2048, 32, 4, 4, 64, 8, 0), (6000, 500, 4, 1, 128, 32, 500 * 64 - 6000),
-                                             (5000, 400, 16, 2, 64, 32, 400 * 64 - 5000), (3000, 47, 5, 1, 128, 16, 8)])
+                                             (5000, 400, 16, 2, 64, 32, 400 * 64 - 5000), (3000, 47, 5, 1, 128, 16, 8),
+                                             (5000, 400, 4, 2, 128, 32, 400 * 64 - 5000)])
 def test_prefill_selection_with_prior_bias(pkg, orc, dev, L, N, HQ, H, D, K, off):
     """topk_chunk_weights(prior_b=) at prefill sizes: the one-pass selection kernel adds the bias to
     its logits, the softmax kernel gathers it.  Checked against the exporting variant of the operator
@@ -67,7 +68,7 @@ def test_prefill_selection_with_prior_bias(pkg, orc, dev, L, N, HQ, H, D, K, off
 
 @pytest.mark.parametrize("L,N,HQ,H,D,K", [(3000, 47, 8, 2, 128, 16), (5000, 400, 4, 1, 64, 32),
                                           (5000, 400, 16, 2, 64, 32), (3000, 47, 7, 1, 128, 16),
-                                          (9000, 300, 12, 2, 128, 32)])
+                                          (9000, 300, 12, 2, 128, 32), (5000, 400, 4, 2, 64, 32)])
 def test_prefill_selection_with_a_key_per_query_head(pkg, orc, dev, L, N, HQ, H, D, K):
     """The layer's default pooling (attention-pooled chunk keys, one per query head, with their prior
     bias; models/FlashHiLS/hils_attention.py:391-416, 568-602) through topk_chunk_weights: same

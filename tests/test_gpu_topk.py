@@ -396,6 +396,8 @@ def test_topk_split_and_fused_paths_agree(pkg, dev):
     # five to eight query heads per KV head: two wavefronts per four queries trade their heads' scores
     (8192, 128, 2, 8, 64, 32, False), (5000, 79, 1, 5, 128, 16, True), (4096, 64, 2, 7, 64, 5, True),
     (16384, 256, 1, 8, 128, 32, True),
+    # two query heads per KV head: two queries a lane
+    (8192, 128, 2, 2, 128, 32, True), (5000, 79, 3, 2, 64, 7, False), (32768, 512, 1, 2, 64, 32, False),
 ])
 def test_topk_one_pass_prefill_kernel(pkg, orc, dev, L, N, h_kv, G, D, topk, dup):
     """The one-pass prefill kernel (chunk keys repacked into the workspace, up to 512 chunks and 32
@@ -414,7 +416,8 @@ def test_topk_one_pass_prefill_kernel(pkg, orc, dev, L, N, h_kv, G, D, topk, dup
     (4, 128, 6000, 125, 16, 1, 48, 1),    # chunk sizes that are no power of two (visibility by division)
     (1, 64, 5000, 50, 7, 30, 100, 2),
     (8, 64, 32000, 500, 32, 1, 64, 1),    # eight heads per KV head, all four launches
-    (6, 128, 20000, 313, 16, 1, 64, 2), (5, 64, 7000, 140, 9, 64, 48, 1)])
+    (6, 128, 20000, 313, 16, 1, 64, 2), (5, 64, 7000, 140, 9, 64, 48, 1),
+    (2, 128, 32000, 500, 32, 1, 64, 2), (2, 64, 9000, 250, 5, 30, 100, 1)])  # two heads per KV head
 def test_topk_one_pass_kernel_launches_match_export_variant(pkg, dev, G, D, L, N, topk, W, S, h_kv):
     """The one-pass prefill kernel as inference launches it (one instantiation per range of visible
     chunk counts, no logit export) against its exporting instantiation, which the cases above check
