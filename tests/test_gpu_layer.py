@@ -44,10 +44,13 @@ def test_chunk_weights_kernel(pkg, orc, dev):
     torch.manual_seed(3)
     for K in (16, 32, 12):
         _chunk_weights_case(pkg, orc, dev, K)
+    # long rows of queries: the backward's workgroups walk several tiles and add the bias gradients in LDS
+    _chunk_weights_case(pkg, orc, dev, 32, dims=(3, 5000, 16, 2, 79))
+    _chunk_weights_case(pkg, orc, dev, 8, dims=(1, 9001, 6, 3, 141))
 
 
-def _chunk_weights_case(pkg, orc, dev, K):
-    B, L, HQ, H, N = 2, 301, 8, 2, 40
+def _chunk_weights_case(pkg, orc, dev, K, dims=(2, 301, 8, 2, 40)):
+    B, L, HQ, H, N = dims
     scores = torch.randn(B, L, HQ, K).bfloat16()
     scores[:, :5, :, 7:] = float("-inf")
     lse = torch.randn(B, L, HQ).bfloat16()
