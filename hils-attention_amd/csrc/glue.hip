@@ -239,11 +239,14 @@ chunk_weights_bwd_kernel(const bf16_t* __restrict__ scores, const void* __restri
 // (K+1(+1))-wide d_weights rows of a wavefront are contiguous in memory but not 16-byte aligned:
 // they are loaded coalesced into LDS and read from there.
 // TAB (with d_prior_b): a workgroup walks a run of consecutive rows of one batch element and adds the bias
-// gradients into a table (N x HQ floats) in LDS, which it adds to d_prior_b once at the end.  One global
+// gradients into a table (N x HQ) in LDS, which it adds to d_prior_b once at the end.  One global
 // atomic per element has every query of a batch element adding into the same N x HQ words: 33 M adds into
-// 16 K words took 0.51 ms at B8 L8192 h16 K32.
+// 16 K words took 0.51 ms at B8 L8192 h16 K32.  The table is 64-bit fixed point (2^-40): integer LDS adds
+// run at several times the rate of float ones, and a run's sum does not depend on the order of its adds.
+// (TAB: 16 wavefronts a workgroup, two workgroups a compute unit: the rows of a run are walked one tile after
+// the other, and with four wavefronts a workgroup too few loads were in flight)
 template <int LPR, bool TAB>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(TAB ? 1024 : 256)
 chunk_weights_bwd_rows_kernel(const bf16_t* __restrict__ scores, const void* __restrict__ lse_swa,
                               int lse_bf16, const float* __restrict__ prior_b,
                               const int32_t* __restrict__ indices, const bf16_t* __restrict__ d_weights,
@@ -251,24 +254,26 @@ chunk_weights_bwd_rows_kernel(const bf16_t* __restrict__ scores, const void* __r
                               float* __restrict__ d_prior_b, long rows, int L, int HQ, int H, int N,
                               int softmax1, int tiles_per_wg) {
   constexpr int K = LPR * 8, RPW = 64 / LPR;
-  __shared__ bf16_t stage[4][RPW * (K + 2)];
-  extern __shared__ float cwb_tab[];  // TAB: N x HQ
+  constexpr int NWV = TAB ? 16 : 4;  // wavefronts of a workgroup
+  __shared__ bf16_t stage[NWV][RPW * (K + 2)];
+  extern __shared__ unsigned long long cwb_tab[];  // TAB: N x HQ, two's complement fixed point
+  constexpr float TAB_SCALE = 1099511627776.f;  // 2^40: |sums| below 2^23, steps far below an fp32 gradient's own
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPR, rl = lane / LPR;
   const int NW = K + 1 + (softmax1 ? 1 : 0);
   // rows of this workgroup: [first, last); TAB: a run inside batch element blockIdx.y
-  long first = (long)blockIdx.x * 4 * RPW, last = rows;
+  long first = (long)blockIdx.x * NWV * RPW, last = rows;
   int ntile = 1;
   if (TAB) {
     const long per_b = (long)L * HQ;
-    first = blockIdx.y * per_b + (long)blockIdx.x * tiles_per_wg * 4 * RPW;
+    first = blockIdx.y * per_b + (long)blockIdx.x * tiles_per_wg * NWV * RPW;
     last = (blockIdx.y + 1) * per_b;
     ntile = tiles_per_wg;
-    for (int i = threadIdx.x; i < N * HQ; i += 256) cwb_tab[i] = 0.f;
+    for (int i = threadIdx.x; i < N * HQ; i += NWV * 64) cwb_tab[i] = 0ull;
     __syncthreads();
   }
   for (int tile = 0; tile < ntile; ++tile) {
-    const long row0 = first + ((long)tile * 4 + wave) * RPW;
+    const long row0 = first + ((long)tile * NWV + wave) * RPW;
     const long row = row0 + rl;
     long nrow = last - row0;
     if (nrow > RPW) nrow = RPW;
@@ -350,7 +355,7 @@ chunk_weights_bwd_rows_kernel(const bf16_t* __restrict__ scores, const void* __r
 #pragma unroll
         for (int e = 0; e < 8; ++e)
           if (dl[e] != 0.f) {
-            if (TAB) atomicAdd(&cwb_tab[cidx[e] * HQ + hq], dl[e]);
+            if (TAB) atomicAdd(&cwb_tab[cidx[e] * HQ + hq], (unsigned long long)(long long)(dl[e] * TAB_SCALE));
             else atomicAdd(d_prior_b + (b * N + cidx[e]) * (long)HQ + hq, dl[e]);
           }
       }
@@ -360,9 +365,9 @@ chunk_weights_bwd_rows_kernel(const bf16_t* __restrict__ scores, const void* __r
   if (TAB) {
     __syncthreads();
     float* dst = d_prior_b + (long)blockIdx.y * N * HQ;
-    for (int i = threadIdx.x; i < N * HQ; i += 256) {
-      const float t = cwb_tab[i];
-      if (t != 0.f) atomicAdd(dst + i, t);
+    for (int i = threadIdx.x; i < N * HQ; i += NWV * 64) {
+      const long long t = (long long)cwb_tab[i];
+      if (t != 0) atomicAdd(dst + i, (float)((double)t * (1.0 / 1099511627776.0)));
     }
   }
 }
@@ -385,9 +390,9 @@ extern "C" int hils_chunk_weights_bwd(const void* scores, const void* lse_swa, i
     HILS_REQUIRE(nb <= 2147483647L, "hils_chunk_weights_bwd: grid too large");
     // with a bias gradient whose table fits the LDS: runs of rows per workgroup, about two workgroups a
     // compute unit, each run long enough that its adds outnumber the table it flushes
-    const size_t tab_b = (size_t)N * HQ * sizeof(float);
+    const size_t tab_b = (size_t)N * HQ * sizeof(unsigned long long);
     if (d_prior_b && tab_b <= 48 * 1024) {
-      const long tiles_b = ((long)L * HQ + 4 * rpw - 1) / (4 * rpw);  // 4-wavefront tiles of a batch element
+      const long tiles_b = ((long)L * HQ + 16 * rpw - 1) / (16 * rpw);  // 16-wavefront tiles of a batch element
       long segs = 2L * hils_device_cus() / B;
       if (segs < 1) segs = 1;
       if (segs > tiles_b) segs = tiles_b;
@@ -395,7 +400,7 @@ extern "C" int hils_chunk_weights_bwd(const void* scores, const void* lse_swa, i
       const dim3 grid((unsigned)((tiles_b + tiles_per_wg - 1) / tiles_per_wg), (unsigned)B);
       HILS_REQUIRE(B <= 65535, "hils_chunk_weights_bwd: batch too large for the grid");
 #define GL_CALL_T(LPR_)                                                                                \
-  hipLaunchKernelGGL((chunk_weights_bwd_rows_kernel<LPR_, true>), grid, dim3(256), tab_b,              \
+  hipLaunchKernelGGL((chunk_weights_bwd_rows_kernel<LPR_, true>), grid, dim3(1024), tab_b,             \
                      (hipStream_t)stream, (const bf16_t*)scores, lse_swa, lse_bf16, prior_b, indices,  \
                      (const bf16_t*)d_weights, (bf16_t*)d_scores, d_lse, d_prior_b, rows, L, HQ, H, N, \
                      softmax1, tiles_per_wg)
