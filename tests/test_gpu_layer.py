@@ -241,3 +241,52 @@ def test_decode_step_on_a_mostly_empty_cache(pkg, orc, dev, q_pos):
     assert_close_bf16(o1, ref, "decode_step output")
     if nvis == 0:  # nothing remote to attend to: all the weight on the local branch
         assert torch.count_nonzero(o1).item() == 0 and torch.all(w1[..., K].float() == 1.0)
+
+
+@pytest.mark.parametrize("L,HQ,H,D,K,W", [(4096, 16, 2, 64, 16, 512), (2500, 32, 4, 128, 8, 512), (3000, 8, 4, 64, 8, 200)])
+def test_default_mode_layer_forward_at_the_reference_head_counts(pkg, orc, dev, L, HQ, H, D, K, W):
+    """The layer in the reference's default mode (models/FlashHiLS/hils_attention.py:361-416, 540-623: sliding
+    window 512, attention-pooled chunk keys per query head, their entropy as prior bias of the selection and
+    of the inter-chunk softmax, the local branch merged by its weight) at the head counts of its
+    configurations (configs/hils_attention: 16 query / 2 KV heads of 64), every stage on the GPU, against the
+    oracle's stages on the same inputs and on the kernel's own selection."""
+    note(f"default-mode layer forward L{L} HQ{HQ} H{H} D{D} K{K} W{W}")
+    B, S = 1, 64
+    G, N = HQ // H, L // S
+    gen = torch.Generator().manual_seed(1010)
+    q = torch.randn(B, L, HQ, D, generator=gen).bfloat16()
+    k = torch.randn(B, L, H, D, generator=gen).bfloat16()
+    v = torch.randn(B, L, H, D, generator=gen).bfloat16()
+    mu = torch.randn(B, N, HQ, D, generator=gen).bfloat16()  # the chunks' prior queries
+    qd, kd, vd, mud = q.to(dev), k.to(dev), v.to(dev), mu.to(dev)
+    # the GPU pipeline
+    swa_o, lse_swa = pkg.flex_attn_tl(qd, kd, vd, W, S, training=False)
+    lmk_k, lmk_b = pkg.chunk_attn_pool(mud, kd[:, : N * S].reshape(B, N, S, H, D))
+    lse_h = lse_swa.bfloat16()  # the layer hands it over in its hidden dtype
+    idx, sc, w = pkg.topk_chunk_weights(qd, lmk_k, lse_h, K, S, W, prior_b=lmk_b, num_kv_heads=H)
+    o = pkg.HiLS_block_M_head(qd, kd, vd, w, idx, block_size=S, is_training=False, swa_o=swa_o)
+    torch.cuda.synchronize()
+    # the oracle's stages
+    r_swa_o, r_lse = orc.swa(q, k, v, window_size=W, chunk_size=S, mask_lmk=True)
+    assert_close_bf16(swa_o, r_swa_o, "local branch")
+    fin = torch.isfinite(r_lse)
+    assert torch.equal(torch.isfinite(lse_swa).cpu(), fin)
+    assert (lse_swa.cpu() - r_lse)[fin].abs().max().item() <= 1e-3
+    r_k, r_b, _ = orc.chunk_attn_pool(mu, k[:, : N * S].reshape(B, N, S, H, D).repeat_interleave(G, dim=3))
+    assert_close_bf16(lmk_k, r_k, "attention-pooled chunk keys")
+    assert (lmk_b.cpu() - r_b).abs().max().item() <= 1e-4
+    # selection on the GPU's own chunk keys / bias / lse: agreement with the oracle's, exactness from the logits
+    ridx, _, aux = orc.online_softmax_topk_head(q.view(B, L, H, G, D), lmk_k.cpu(), lse_h.float().cpu(), K, S, W,
+                                                bias=lmk_b.cpu(), return_aux=True)
+    assert (idx.cpu() == ridx).float().mean().item() >= 0.99
+    dbg = {}
+    idx_e, sc_e = pkg.online_softmax_topk_head(qd, lmk_k, lse_h.float(), K, S, W, is_training=False, bias=lmk_b, G=G,
+                                               _debug=dbg)
+    assert torch.equal(idx_e, idx) and torch.equal(sc_e.view(torch.int16), sc.view(torch.int16))
+    lim = orc.causal_chunk_limit(L, 0, W, S)
+    assert torch.equal(idx.cpu(), orc.topk_select(dbg["sel_logits"].cpu(), dbg["lse_total"].cpu(), lim, K))
+    w_ref = orc.inter_chunk_softmax(sc.float().cpu(), lse_h.float().cpu(), lmk_b.cpu().bfloat16().float(), idx.cpu(),
+                                    bf16_sum=True)
+    assert_close_bf16(w, w_ref, "inter-chunk weights with the prior bias", max_abs=8e-3)
+    o_ref = orc.sparse_attn(q, k, v, w.cpu(), idx.cpu(), chunk_size=S) + swa_o.float().cpu() * w[..., K].float().cpu().unsqueeze(-1)
+    assert_close_bf16(o, o_ref, "layer output")
