@@ -29,6 +29,7 @@ def _paged_copy(k, v, lmk, dev, seed, spare=5):
 
 @pytest.mark.parametrize("B,Lq,Lkv,HQ,H,D,K", [(32, 1, 32768, 32, 8, 128, 32), (16, 1, 16384, 8, 8, 64, 16),
                                                (50, 2, 20480, 4, 1, 128, 8),
+                                               (64, 1, 32768, 16, 2, 64, 32), (20, 1, 32768, 40, 8, 128, 16),  # eight / five heads per KV head
                                                # short caches: the token-major call runs on other kernels
                                                (5, 1, 4096, 8, 2, 128, 16), (3, 2, 2048, 4, 4, 64, 8)])
 def test_paged_decode_matches_contiguous(pkg, orc, dev, B, Lq, Lkv, HQ, H, D, K):
