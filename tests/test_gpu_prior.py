@@ -265,7 +265,7 @@ def test_paged_decode_with_prior_bias(pkg, orc, dev):
     assert_close_bf16(o3, o4.float(), "paged two-call path vs dense two-call path")
 
 
-@pytest.mark.parametrize("G,chunk_pooling", [(4, True), (1, False), (2, False), (4, False)])
+@pytest.mark.parametrize("G,chunk_pooling", [(4, True), (1, False), (2, False), (4, False), (8, False), (8, True)])
 def test_cache_layers_keep_and_use_the_prior(pkg, orc, dev, G, chunk_pooling):
     """HiLSDynamicLayer / HiLSPagedLayer filled incrementally with the chunks' prior queries: the
     entropy bias (and, without chunk pooling, the attention-pooled keys) match the oracle's attention
