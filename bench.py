@@ -263,6 +263,23 @@ def bench_decode(pkg, dev, steps, warmup):
             "attn_gbs": kv_bytes / (per["attn"] * 1e-3) / 1e9}
     del kc, vc
     torch.cuda.empty_cache()
+    # the same step at the head counts of the reference's own configurations (16 query / 2 KV heads of 64,
+    # eight query heads per KV head; 256 rows, 128K context): shared chunk keys, and the layer's default mode
+    HQ2, H2, D2 = 16, 2, 64
+    B2 = 256 // H2
+    q2 = gpu_randn((B2, 1, HQ2, D2), gen, dev)
+    k2 = gpu_randn((B2, Lkv, H2, D2), gen, dev)
+    v2 = gpu_randn((B2, Lkv, H2, D2), gen, dev)
+    lse2 = torch.randn(B2, 1, HQ2, device=dev, generator=gen) * 5 + 10
+    lmk2 = pkg.head_major_chunk_keys(pkg.chunk_mean_pool(k2, S))
+    lmk2_q = gpu_randn((B2, HQ2, N, D2), gen, dev)
+    prior2 = torch.randn(B2, H2, N, HQ2 // H2, device=dev, generator=gen)
+    per["hq16_hkv2_d64_step"] = time_steps(lambda: pkg.decode_step(
+        q2, lmk2, k2, v2, lse2, K, S, W, q_offset=Lkv - 1, lmk_head_major=True), steps, warmup) * 1e3
+    per["hq16_hkv2_d64_key_per_query_head_prior_bias_step"] = time_steps(lambda: pkg.decode_step(
+        q2, lmk2_q, k2, v2, lse2, K, S, W, q_offset=Lkv - 1, prior_b=prior2, lmk_head_major=True), steps, warmup) * 1e3
+    del q2, k2, v2, lmk2, lmk2_q, prior2
+    torch.cuda.empty_cache()
     return sec, per, roof
 
 
