@@ -182,8 +182,9 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   // the bias of this (batch, KV head): [chunk][head, padded to 4] fp32, a copy per wavefront (they never
   // synchronise); read back 16 bytes per lane right where a block's logits are formed, instead of
   // global loads whose latency the compiler covers with registers this kernel does not have.
-  // (PERQ with HALF: the wavefronts meet at barriers anyway, one copy per half of the heads.)
-  __shared__ __align__(16) float bias_w[BIAS ? (OVER ? 2 : TGW) : 1][BIAS ? NB * 16 : 1][4];
+  // (PERQ: the wavefronts meet at barriers anyway: one copy per workgroup, filled together; with HALF one
+  // per half of the heads.)
+  __shared__ __align__(16) float bias_w[BIAS ? (OVER ? 2 : (PERQ ? 1 : TGW)) : 1][BIAS ? NB * 16 : 1][4];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int half = HALF ? (wave & 1) : 0;   // this wavefront's heads are 4 * half ..
@@ -268,7 +269,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   };
   // bias (B, N, h_kv, G) fp32: the G values of a (chunk, KV head) are contiguous; accumulator row
   // 4j+i is head (4j+i) % GMAX
-  float (*bias_s)[4] = bias_w[BIAS ? (OVER ? half : wave) : 0];
+  float (*bias_s)[4] = bias_w[BIAS ? (OVER ? half : (PERQ ? 0 : wave)) : 0];
   if constexpr (BIAS) {
     const float* bias_u = bias + (b * N * (long)h_kv + hk) * G;
     if constexpr (HALF) {
@@ -286,7 +287,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
       }
     } else {
 #pragma unroll
-    for (int c = lane; c < NB * 16; c += 64) {
+    for (int c = PERQ ? wave * 64 + lane : lane; c < NB * 16; c += PERQ ? 64 * TGW : 64) {
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);  // chunks past N (never visible) and heads past G: 0
       if (c < N) {
         const float* bp = bias_u + (long)c * h_kv * G;
@@ -297,6 +298,7 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
       }
       *(float4*)bias_s[c] = v;
     }
+    if constexpr (PERQ) __syncthreads();  // the wavefronts add the bias to their accumulators before the first exchange
     }
   }
   auto bias_of = [&](int c, float (&bv)[4]) {  // c < 16 * NB
