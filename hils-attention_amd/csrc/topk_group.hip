@@ -182,9 +182,9 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   // the bias of this (batch, KV head): [chunk][head, padded to 4] fp32, a copy per wavefront (they never
   // synchronise); read back 16 bytes per lane right where a block's logits are formed, instead of
   // global loads whose latency the compiler covers with registers this kernel does not have.
-  // (PERQ: the wavefronts meet at barriers anyway: one copy per workgroup, filled together; with HALF one
-  // per half of the heads.)
-  __shared__ __align__(16) float bias_w[BIAS ? (OVER ? 2 : (PERQ ? 1 : TGW)) : 1][BIAS ? NB * 16 : 1][4];
+  // (One copy per workgroup, filled by its wavefronts together before they part; with HALF one per half of
+  // the heads.)
+  __shared__ __align__(16) float bias_w[BIAS ? (HALF ? (PERQ ? 2 : TGW) : 1) : 1][BIAS ? NB * 16 : 1][4];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int half = HALF ? (wave & 1) : 0;   // this wavefront's heads are 4 * half ..
@@ -199,10 +199,45 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   const int lane = threadIdx.x & 63, col = lane & 15, j = lane >> 4;
   const int t0 = t_base + (blockIdx.x * QGROUPS + pw) * NQ;
   const int t_wg = t_base + blockIdx.x * QGROUPS * NQ;  // PERQ: the workgroup's 16 queries
-  if ((PERQ ? t_wg : t0) >= t_end) return;          // (PERQ: the wavefronts meet at barriers until the logits are in)
+  // (with a bias and shared keys the wavefronts of a workgroup first stage the bias together, below)
+  const bool gone = (PERQ ? t_wg : t0) >= t_end;    // (PERQ: the wavefronts meet at barriers until the logits are in)
+  if (!(BIAS && !PERQ && !HALF) && gone) return;
   const int t_safe = PERQ ? t_wg : t0;              // a query of this launch, for the addresses of rows that have none
   const int hk = blockIdx.y;
   const long b = blockIdx.z;
+  float (*bias_s)[4] = bias_w[BIAS ? (OVER ? half : (HALF ? wave : 0)) : 0];
+  if constexpr (BIAS) {
+    const float* bias_u = bias + (b * N * (long)h_kv + hk) * G;
+    if constexpr (HALF) {
+      // this half's heads; PERQ: the four wavefronts of a half fill its copy together (the first
+      // barrier of the logits comes before anybody reads it)
+      for (int c = OVER ? pw * 64 + lane : lane; c < NB * 16; c += OVER ? 64 * QGROUPS : 64) {
+        float e4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (c < N) {
+          const float* bp = bias_u + (long)c * h_kv * G + gofs;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (gofs + e < G) e4[e] = bp[e];
+        }
+        *(float4*)bias_s[c] = make_float4(e4[0], e4[1], e4[2], e4[3]);
+      }
+    } else {
+#pragma unroll
+    for (int c = wave * 64 + lane; c < NB * 16; c += 64 * TGW) {  // the workgroup's wavefronts together
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);  // chunks past N (never visible) and heads past G: 0
+      if (c < N) {
+        const float* bp = bias_u + (long)c * h_kv * G;
+        v.x = bp[0];
+        if (GMAX > 1 && G > 1) v.y = bp[1];
+        if (GMAX > 2 && G > 2) v.z = bp[2];
+        if (GMAX > 2 && G > 3) v.w = bp[3];
+      }
+      *(float4*)bias_s[c] = v;
+    }
+    __syncthreads();  // (with a key per query head the bias is added before the first exchange)
+    }
+  }
+  if (BIAS && !PERQ && !HALF && gone) return;
 
   // chunks a query sees (visible_limit of common.h; bs_shift >= 0: the chunk size is 1 << bs_shift and
   // the division is an arithmetic shift, which rounds towards minus infinity as floordiv does)
@@ -269,38 +304,6 @@ topk_fwd_group_kernel(const bf16_t* __restrict__ q, const uint4* __restrict__ lm
   };
   // bias (B, N, h_kv, G) fp32: the G values of a (chunk, KV head) are contiguous; accumulator row
   // 4j+i is head (4j+i) % GMAX
-  float (*bias_s)[4] = bias_w[BIAS ? (OVER ? half : (PERQ ? 0 : wave)) : 0];
-  if constexpr (BIAS) {
-    const float* bias_u = bias + (b * N * (long)h_kv + hk) * G;
-    if constexpr (HALF) {
-      // this half's heads; PERQ: the four wavefronts of a half fill its copy together (the first
-      // barrier of the logits comes before anybody reads it)
-      for (int c = OVER ? pw * 64 + lane : lane; c < NB * 16; c += OVER ? 64 * QGROUPS : 64) {
-        float e4[4] = {0.f, 0.f, 0.f, 0.f};
-        if (c < N) {
-          const float* bp = bias_u + (long)c * h_kv * G + gofs;
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (gofs + e < G) e4[e] = bp[e];
-        }
-        *(float4*)bias_s[c] = make_float4(e4[0], e4[1], e4[2], e4[3]);
-      }
-    } else {
-#pragma unroll
-    for (int c = PERQ ? wave * 64 + lane : lane; c < NB * 16; c += PERQ ? 64 * TGW : 64) {
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);  // chunks past N (never visible) and heads past G: 0
-      if (c < N) {
-        const float* bp = bias_u + (long)c * h_kv * G;
-        v.x = bp[0];
-        if (GMAX > 1 && G > 1) v.y = bp[1];
-        if (GMAX > 2 && G > 2) v.z = bp[2];
-        if (GMAX > 2 && G > 3) v.w = bp[3];
-      }
-      *(float4*)bias_s[c] = v;
-    }
-    if constexpr (PERQ) __syncthreads();  // the wavefronts add the bias to their accumulators before the first exchange
-    }
-  }
   auto bias_of = [&](int c, float (&bv)[4]) {  // c < 16 * NB
     const float4 v = *(const float4*)bias_s[c];
     const float e[4] = {v.x, v.y, v.z, v.w};
